@@ -1,0 +1,190 @@
+"""ctypes front end of the CPU oracle (``sdpa_oracle.c``) plus tiny fp64 brute-force twins.
+
+TEST INFRASTRUCTURE ONLY: importable from ``tests/``, ``__graft_entry__.smoke()`` and the
+``cpu_baseline`` leg of ``bench.py``; never from the product package.
+
+bf16 tensors are numpy ``uint16`` arrays holding the raw bit patterns, contiguous ``[B,H,S,D]``.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "_build", "liboracle.so")
+_lib = None
+
+
+def build(force: bool = False) -> str:
+    """Compile ``sdpa_oracle.c`` with gcc (``make -C oracle``)."""
+    if force:
+        subprocess.check_call(["make", "-C", _HERE, "clean"], stdout=subprocess.DEVNULL)
+    subprocess.check_call(["make", "-C", _HERE], stdout=subprocess.DEVNULL)
+    return _LIB_PATH
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        _lib = ctypes.CDLL(_LIB_PATH)
+        _lib.oracle_num_threads.restype = ctypes.c_int
+    return _lib
+
+
+def _p(a):
+    return None if a is None else a.ctypes.data_as(ctypes.c_void_p)
+
+
+def num_threads() -> int:
+    return int(lib().oracle_num_threads())
+
+
+def set_num_threads(n: int) -> None:
+    lib().oracle_set_num_threads(ctypes.c_int(n))
+
+
+# ---------------------------------------------------------------- bf16 helpers (numpy)
+def f32_to_bf16(x: np.ndarray) -> np.ndarray:
+    """fp32 -> bf16 bit patterns (uint16), round-to-nearest-even."""
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+    nan = (u & 0x7FFFFFFF) > 0x7F800000
+    r = (u + (0x7FFF + ((u >> 16) & 1))) >> 16
+    r = np.where(nan, (u >> 16) | 0x40, r)
+    return r.astype(np.uint16)
+
+
+def bf16_to_f32(h: np.ndarray) -> np.ndarray:
+    return (np.ascontiguousarray(h, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+# ---------------------------------------------------------------- C oracle wrappers
+def _mask_args(mask, B, H, Sq, Sk):
+    """mask: uint8 array broadcastable to [B,H,Sq,Sk] (4-D, dims of size 1 broadcast)."""
+    if mask is None:
+        return None, (0, 0, 0, 0), None
+    m = np.ascontiguousarray(mask, dtype=np.uint8)
+    assert m.ndim == 4, "mask must be 4-D"
+    full = (B, H, Sq, Sk)
+    st = []
+    for ax in range(4):
+        assert m.shape[ax] in (1, full[ax]), f"mask dim {ax} not broadcastable"
+        st.append(0 if m.shape[ax] == 1 and full[ax] != 1 else m.strides[ax])
+    return m, tuple(st), m
+
+
+def sdpa_fwd(q, k, v, scale, causal=False, kv_len=None, mask=None, heads=None, want_f32=False):
+    """Naive fp32 forward. Returns (O bf16-bits, LSE fp32[, O fp32])."""
+    B, H, Sq, D = q.shape
+    Sk = k.shape[2]
+    q, k, v = (np.ascontiguousarray(t, dtype=np.uint16) for t in (q, k, v))
+    O = np.zeros((B, H, Sq, D), np.uint16)
+    LSE = np.zeros((B, H, Sq), np.float32)
+    O32 = np.zeros((B, H, Sq, D), np.float32) if want_f32 else None
+    kvl = None if kv_len is None else np.ascontiguousarray(kv_len, dtype=np.int32)
+    m, st, _keep = _mask_args(mask, B, H, Sq, Sk)
+    hb, he = (0, B * H) if heads is None else heads
+    rc = lib().oracle_sdpa_fwd(
+        _p(q), _p(k), _p(v), B, H, Sq, Sk, D, ctypes.c_float(scale), int(bool(causal)),
+        _p(kvl), _p(m), *(ctypes.c_int64(s) for s in st), hb, he, _p(O), _p(LSE), _p(O32))
+    if rc != 0:
+        raise RuntimeError(f"oracle_sdpa_fwd failed: {rc}")
+    return (O, LSE, O32) if want_f32 else (O, LSE)
+
+
+def sdpa_bwd(q, k, v, o, do, scale, causal=False, kv_len=None, mask=None, heads=None, want_f32=False):
+    """Naive fp32 backward. Returns (dQ, dK, dV) bf16 bits [+ fp32 copies]."""
+    B, H, Sq, D = q.shape
+    Sk = k.shape[2]
+    q, k, v, o, do = (np.ascontiguousarray(t, dtype=np.uint16) for t in (q, k, v, o, do))
+    dQ = np.zeros((B, H, Sq, D), np.uint16)
+    dK = np.zeros((B, H, Sk, D), np.uint16)
+    dV = np.zeros((B, H, Sk, D), np.uint16)
+    f = [np.zeros(t.shape, np.float32) for t in (dQ, dK, dV)] if want_f32 else [None] * 3
+    kvl = None if kv_len is None else np.ascontiguousarray(kv_len, dtype=np.int32)
+    m, st, _keep = _mask_args(mask, B, H, Sq, Sk)
+    hb, he = (0, B * H) if heads is None else heads
+    rc = lib().oracle_sdpa_bwd(
+        _p(q), _p(k), _p(v), _p(o), _p(do), B, H, Sq, Sk, D, ctypes.c_float(scale),
+        int(bool(causal)), _p(kvl), _p(m), *(ctypes.c_int64(s) for s in st), hb, he,
+        _p(dQ), _p(dK), _p(dV), _p(f[0]), _p(f[1]), _p(f[2]))
+    if rc != 0:
+        raise RuntimeError(f"oracle_sdpa_bwd failed: {rc}")
+    return (dQ, dK, dV, *f) if want_f32 else (dQ, dK, dV)
+
+
+def sage_quant(q, k, qblk=128, kblk=64, smooth_k=True):
+    """Returns dict(kmean, ks, qi8, ki8, sq, sk)."""
+    B, H, Sq, D = q.shape
+    Sk = k.shape[2]
+    q, k = (np.ascontiguousarray(t, dtype=np.uint16) for t in (q, k))
+    nqb, nkb = -(-Sq // qblk), -(-Sk // kblk)
+    out = dict(
+        kmean=np.zeros((B, H, D), np.float32), ks=np.zeros((B, H, Sk, D), np.uint16),
+        qi8=np.zeros((B, H, Sq, D), np.int8), ki8=np.zeros((B, H, Sk, D), np.int8),
+        sq=np.zeros((B, H, nqb), np.float32), sk=np.zeros((B, H, nkb), np.float32))
+    rc = lib().oracle_sage_quant(
+        _p(q), _p(k), B, H, Sq, Sk, D, qblk, kblk, int(bool(smooth_k)),
+        _p(out["kmean"]), _p(out["ks"]), _p(out["qi8"]), _p(out["ki8"]), _p(out["sq"]), _p(out["sk"]))
+    if rc != 0:
+        raise RuntimeError(f"oracle_sage_quant failed: {rc}")
+    return out
+
+
+def sage_fwd(qi8, ki8, sq, sk, v, scale, qblk=128, kblk=64, causal=False, heads=None):
+    B, H, Sq, D = qi8.shape
+    Sk = ki8.shape[2]
+    qi8, ki8 = (np.ascontiguousarray(t, dtype=np.int8) for t in (qi8, ki8))
+    sq, sk = (np.ascontiguousarray(t, dtype=np.float32) for t in (sq, sk))
+    v = np.ascontiguousarray(v, dtype=np.uint16)
+    O = np.zeros((B, H, Sq, D), np.uint16)
+    LSE = np.zeros((B, H, Sq), np.float32)
+    hb, he = (0, B * H) if heads is None else heads
+    rc = lib().oracle_sage_fwd(_p(qi8), _p(ki8), _p(sq), _p(sk), _p(v), B, H, Sq, Sk, D, qblk, kblk,
+                               ctypes.c_float(scale), int(bool(causal)), hb, he, _p(O), _p(LSE))
+    if rc != 0:
+        raise RuntimeError(f"oracle_sage_fwd failed: {rc}")
+    return O, LSE
+
+
+# ---------------------------------------------------------------- fp64 brute force (checker of the checker)
+def brute_sdpa_f64(q, k, v, scale, keep=None):
+    """Pure numpy fp64 attention on float arrays [.., Sq, D]; keep: bool [.., Sq, Sk] or None.
+
+    Returns (O, LSE, P), all fp64.  Written from the textbook definition, not from the C file.
+    """
+    q, k, v = (np.asarray(t, np.float64) for t in (q, k, v))
+    s = np.einsum("...id,...jd->...ij", q, k) * float(scale)
+    if keep is not None:
+        s = np.where(keep, s, -np.inf)
+    m = s.max(axis=-1, keepdims=True)
+    msafe = np.where(np.isfinite(m), m, 0.0)
+    e = np.exp(s - msafe)
+    l = e.sum(axis=-1, keepdims=True)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        p = np.where(l > 0, e / np.where(l > 0, l, 1.0), 0.0)
+        lse = np.where(l[..., 0] > 0, msafe[..., 0] + np.log(np.where(l[..., 0] > 0, l[..., 0], 1.0)), -np.inf)
+    return p @ v, lse, p
+
+
+# ---------------------------------------------------------------- error metrics used by every parity test
+def max_abs(a, b) -> float:
+    return float(np.max(np.abs(np.asarray(a, np.float64) - np.asarray(b, np.float64)))) if np.size(a) else 0.0
+
+
+def rel_l2(a, b) -> float:
+    a = np.asarray(a, np.float64).ravel()
+    b = np.asarray(b, np.float64).ravel()
+    den = np.linalg.norm(b)
+    return float(np.linalg.norm(a - b) / den) if den > 0 else float(np.linalg.norm(a - b))
+
+
+def cosine(a, b) -> float:
+    a = np.asarray(a, np.float64).ravel()
+    b = np.asarray(b, np.float64).ravel()
+    den = np.linalg.norm(a) * np.linalg.norm(b)
+    return float(a @ b / den) if den > 0 else 1.0

@@ -1,0 +1,417 @@
+/*
+ * CPU oracle for the activation-memory-saving attention path.
+ *
+ * TEST INFRASTRUCTURE ONLY.  Nothing in the shipped library may link, load or
+ * call this file; it exists so that the HIP kernels can be checked against a
+ * plain restatement of the reference's naive, materialised, fp32-accumulated
+ * scaled-dot-product attention, and so that the benchmark can time that naive
+ * algorithm on the host cores as a reported baseline.
+ *
+ * Reference algorithm followed (paths relative to the reference tree):
+ *   forward   tests/fa2_parity_naive.rs:90-140      (upcast, QK^T, scale, max/exp/sum/div, PV, bf16)
+ *   backward  tests/cudnn_sdpa_bwd_parity.rs:31-98  (dV=P^T dO, dP=dO V^T, D=rowsum(dO*O),
+ *                                                    dS=P*(dP-D), dQ=dS K scale, dK=dS^T Q scale)
+ *   keep-mask src/sdpa.rs:458-470, src/tests/attention_tests.rs:61-108 (mask < 0.5 => excluded)
+ *   causal    kernels/sdpa_kernels.cu:129-135       (absolute k > q is excluded)
+ *   LSE       third_party/cudnn_frontend/include/cudnn_frontend/node/softmax.h:139-213
+ *             (Stats = max + ln(sum exp(s - max)), natural log of the scaled logits)
+ *   int8 quantisation closed form  src/sage_attention.rs:524-541
+ *             (scale = absmax/127, q = clamp(round_half_even(x/scale), -128, 127))
+ *
+ * Deviations that are deliberate and stated:
+ *   - excluded positions are treated as exactly -inf (weight 0), where the
+ *     reference adds a large negative constant (-1e9 / -1e30): the results
+ *     agree unless a whole row is excluded; such a row here gives O = 0,
+ *     LSE = -inf and zero gradients.
+ *   - the backward forms D from the bf16-rounded O (what a kernel that reads
+ *     the saved O sees), the reference test uses its un-rounded fp32 O.
+ *
+ * Pinning status (see tests/test_oracle_*.py):
+ *   forward O        pinned: reference 2x2 known-answer test, fp64 brute force, torch CPU SDPA, invariants
+ *   LSE              pinned by the closed form and sum_j exp(s_ij - LSE_i) = 1 only;
+ *                    no reference test asserts Stats values ("parity unpinned" by the reference itself)
+ *   dQ, dK, dV       pinned: fp64 central finite differences, torch CPU autograd
+ *   int8 quantiser   pinned: brute force in Python integers/fp64, tie and absmax unit vectors
+ *   K-mean smoothing, per-block (128/64) granularity, int8-QK forward: new behaviour with no
+ *                    counterpart in the reference ("parity unpinned"); pinned only by softmax
+ *                    shift-invariance and cosine against the bf16 result.
+ *
+ * Layout: every tensor is contiguous [B,H,S,D]; bf16 is carried as uint16_t.
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+static inline float bf16_to_f32(uint16_t h) {
+    uint32_t u = (uint32_t)h << 16;
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+/* round-to-nearest-even, NaN kept quiet */
+static inline uint16_t f32_to_bf16(float f) {
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+void oracle_bf16_to_f32(const uint16_t* src, float* dst, int64_t n) {
+    for (int64_t i = 0; i < n; ++i) dst[i] = bf16_to_f32(src[i]);
+}
+void oracle_f32_to_bf16(const float* src, uint16_t* dst, int64_t n) {
+    for (int64_t i = 0; i < n; ++i) dst[i] = f32_to_bf16(src[i]);
+}
+
+int oracle_num_threads(void) {
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}
+void oracle_set_num_threads(int n) {
+#ifdef _OPENMP
+    if (n > 0) omp_set_num_threads(n);
+#else
+    (void)n;
+#endif
+}
+
+typedef struct {
+    int causal;
+    const int32_t* kv_len;   /* [B] or NULL: keys >= kv_len[b] are excluded          */
+    const uint8_t* mask;     /* keep-mask (non-zero = attend) or NULL                 */
+    int64_t msb, msh, msq, msk; /* element strides of mask over (b,h,q,k); 0 = broadcast */
+} mask_spec;
+
+static inline int excluded(const mask_spec* ms, int b, int h, int i, int j) {
+    if (ms->causal && j > i) return 1;
+    if (ms->kv_len && j >= ms->kv_len[b]) return 1;
+    if (ms->mask && ms->mask[b * ms->msb + h * ms->msh + i * ms->msq + j * ms->msk] == 0) return 1;
+    return 0;
+}
+
+/* P (fp32, Sq x Sk) for one head; also row LSE.  kt = K^T in fp32 [D][Sk]. */
+static void head_probs(const float* q, const float* kt, int Sq, int Sk, int D, float scale,
+                       const mask_spec* ms, int b, int h, float* P, float* lse) {
+    for (int i = 0; i < Sq; ++i) {
+        float* row = P + (size_t)i * Sk;
+        for (int j = 0; j < Sk; ++j) row[j] = 0.f;
+        for (int d = 0; d < D; ++d) {
+            const float qv = q[(size_t)i * D + d];
+            const float* kr = kt + (size_t)d * Sk;
+            for (int j = 0; j < Sk; ++j) row[j] += qv * kr[j];
+        }
+        float m = -INFINITY;
+        for (int j = 0; j < Sk; ++j) {
+            float s = excluded(ms, b, h, i, j) ? -INFINITY : row[j] * scale;
+            row[j] = s;
+            if (s > m) m = s;
+        }
+        if (m == -INFINITY) { /* whole row excluded */
+            for (int j = 0; j < Sk; ++j) row[j] = 0.f;
+            lse[i] = -INFINITY;
+            continue;
+        }
+        float l = 0.f;
+        for (int j = 0; j < Sk; ++j) {
+            float e = expf(row[j] - m);
+            row[j] = e;
+            l += e;
+        }
+        const float inv = 1.0f / l;
+        for (int j = 0; j < Sk; ++j) row[j] *= inv;
+        lse[i] = m + logf(l);
+    }
+}
+
+static int check_dims(int B, int H, int Sq, int Sk, int D) {
+    return (B > 0 && H > 0 && Sq > 0 && Sk > 0 && D > 0) ? 0 : -1;
+}
+
+/*
+ * Forward.  O: bf16 [B,H,Sq,D]; LSE: fp32 [B,H,Sq]; O32 (optional): un-rounded fp32 O.
+ * heads_begin/heads_end restrict the work to flat (b*H+h) indices in [begin,end) so that
+ * long configurations can be checked on a head subset; pass 0 and B*H for everything.
+ */
+int oracle_sdpa_fwd(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
+                    int B, int H, int Sq, int Sk, int D, float scale, int causal,
+                    const int32_t* kv_len, const uint8_t* mask,
+                    int64_t msb, int64_t msh, int64_t msq, int64_t msk,
+                    int heads_begin, int heads_end,
+                    uint16_t* O, float* LSE, float* O32) {
+    if (check_dims(B, H, Sq, Sk, D)) return -1;
+    mask_spec ms = {causal, kv_len, mask, msb, msh, msq, msk};
+    int fail = 0;
+#pragma omp parallel for schedule(dynamic, 1)
+    for (int bh = heads_begin; bh < heads_end; ++bh) {
+        const int b = bh / H, h = bh % H;
+        float* q = (float*)malloc(sizeof(float) * (size_t)Sq * D);
+        float* kt = (float*)malloc(sizeof(float) * (size_t)Sk * D);
+        float* v = (float*)malloc(sizeof(float) * (size_t)Sk * D);
+        float* P = (float*)malloc(sizeof(float) * (size_t)Sq * Sk);
+        float* o = (float*)malloc(sizeof(float) * (size_t)D);
+        if (!q || !kt || !v || !P || !o) {
+            fail = 1;
+        } else {
+            const uint16_t* Qh = Q + (size_t)bh * Sq * D;
+            const uint16_t* Kh = K + (size_t)bh * Sk * D;
+            const uint16_t* Vh = V + (size_t)bh * Sk * D;
+            for (size_t t = 0; t < (size_t)Sq * D; ++t) q[t] = bf16_to_f32(Qh[t]);
+            for (int j = 0; j < Sk; ++j)
+                for (int d = 0; d < D; ++d) {
+                    kt[(size_t)d * Sk + j] = bf16_to_f32(Kh[(size_t)j * D + d]);
+                    v[(size_t)j * D + d] = bf16_to_f32(Vh[(size_t)j * D + d]);
+                }
+            head_probs(q, kt, Sq, Sk, D, scale, &ms, b, h, P, LSE + (size_t)bh * Sq);
+            for (int i = 0; i < Sq; ++i) {
+                for (int d = 0; d < D; ++d) o[d] = 0.f;
+                const float* row = P + (size_t)i * Sk;
+                for (int j = 0; j < Sk; ++j) {
+                    const float p = row[j];
+                    if (p == 0.f) continue;
+                    const float* vr = v + (size_t)j * D;
+                    for (int d = 0; d < D; ++d) o[d] += p * vr[d];
+                }
+                for (int d = 0; d < D; ++d) {
+                    const size_t idx = ((size_t)bh * Sq + i) * D + d;
+                    O[idx] = f32_to_bf16(o[d]);
+                    if (O32) O32[idx] = o[d];
+                }
+            }
+        }
+        free(q); free(kt); free(v); free(P); free(o);
+    }
+    return fail ? -2 : 0;
+}
+
+/*
+ * Backward.  Recomputes P from Q,K (it does not consume a saved LSE, so it is independent of the
+ * forward under test).  O is the bf16-rounded forward output.  Outputs bf16 dQ [B,H,Sq,D],
+ * dK,dV [B,H,Sk,D]; optional fp32 copies dQ32,dK32,dV32 (NULL to skip).
+ */
+int oracle_sdpa_bwd(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
+                    const uint16_t* O, const uint16_t* dO,
+                    int B, int H, int Sq, int Sk, int D, float scale, int causal,
+                    const int32_t* kv_len, const uint8_t* mask,
+                    int64_t msb, int64_t msh, int64_t msq, int64_t msk,
+                    int heads_begin, int heads_end,
+                    uint16_t* dQ, uint16_t* dK, uint16_t* dV,
+                    float* dQ32, float* dK32, float* dV32) {
+    if (check_dims(B, H, Sq, Sk, D)) return -1;
+    mask_spec ms = {causal, kv_len, mask, msb, msh, msq, msk};
+    int fail = 0;
+#pragma omp parallel for schedule(dynamic, 1)
+    for (int bh = heads_begin; bh < heads_end; ++bh) {
+        const int b = bh / H, h = bh % H;
+        const size_t nq = (size_t)Sq * D, nk = (size_t)Sk * D;
+        float* q = (float*)malloc(sizeof(float) * nq);
+        float* g = (float*)malloc(sizeof(float) * nq);   /* dO */
+        float* k = (float*)malloc(sizeof(float) * nk);
+        float* kt = (float*)malloc(sizeof(float) * nk);
+        float* vt = (float*)malloc(sizeof(float) * nk);
+        float* P = (float*)malloc(sizeof(float) * (size_t)Sq * Sk);
+        float* dp = (float*)malloc(sizeof(float) * (size_t)Sk);
+        float* lse = (float*)malloc(sizeof(float) * (size_t)Sq);
+        float* dq = (float*)calloc(nq, sizeof(float));
+        float* dk = (float*)calloc(nk, sizeof(float));
+        float* dv = (float*)calloc(nk, sizeof(float));
+        if (!q || !g || !k || !kt || !vt || !P || !dp || !lse || !dq || !dk || !dv) {
+            fail = 1;
+        } else {
+            const uint16_t* Qh = Q + (size_t)bh * nq;
+            const uint16_t* Gh = dO + (size_t)bh * nq;
+            const uint16_t* Oh = O + (size_t)bh * nq;
+            const uint16_t* Kh = K + (size_t)bh * nk;
+            const uint16_t* Vh = V + (size_t)bh * nk;
+            for (size_t t = 0; t < nq; ++t) { q[t] = bf16_to_f32(Qh[t]); g[t] = bf16_to_f32(Gh[t]); }
+            for (int j = 0; j < Sk; ++j)
+                for (int d = 0; d < D; ++d) {
+                    const float kv = bf16_to_f32(Kh[(size_t)j * D + d]);
+                    k[(size_t)j * D + d] = kv;
+                    kt[(size_t)d * Sk + j] = kv;
+                    vt[(size_t)d * Sk + j] = bf16_to_f32(Vh[(size_t)j * D + d]);
+                }
+            head_probs(q, kt, Sq, Sk, D, scale, &ms, b, h, P, lse);
+            for (int i = 0; i < Sq; ++i) {
+                const float* gi = g + (size_t)i * D;
+                const float* qi = q + (size_t)i * D;
+                float* row = P + (size_t)i * Sk;
+                float delta = 0.f;
+                for (int d = 0; d < D; ++d) delta += gi[d] * bf16_to_f32(Oh[(size_t)i * D + d]);
+                for (int j = 0; j < Sk; ++j) dp[j] = 0.f;
+                for (int d = 0; d < D; ++d) {
+                    const float gv = gi[d];
+                    const float* vr = vt + (size_t)d * Sk;
+                    for (int j = 0; j < Sk; ++j) dp[j] += gv * vr[j];
+                }
+                float* dqi = dq + (size_t)i * D;
+                for (int j = 0; j < Sk; ++j) {
+                    const float p = row[j];
+                    if (p == 0.f) continue;
+                    const float ds = p * (dp[j] - delta);
+                    float* dvj = dv + (size_t)j * D;
+                    float* dkj = dk + (size_t)j * D;
+                    const float* kj = k + (size_t)j * D;
+                    for (int d = 0; d < D; ++d) {
+                        dvj[d] += p * gi[d];
+                        dqi[d] += ds * kj[d];
+                        dkj[d] += ds * qi[d];
+                    }
+                }
+            }
+            for (size_t t = 0; t < nq; ++t) {
+                const float x = dq[t] * scale;
+                dQ[(size_t)bh * nq + t] = f32_to_bf16(x);
+                if (dQ32) dQ32[(size_t)bh * nq + t] = x;
+            }
+            for (size_t t = 0; t < nk; ++t) {
+                const float x = dk[t] * scale;
+                dK[(size_t)bh * nk + t] = f32_to_bf16(x);
+                dV[(size_t)bh * nk + t] = f32_to_bf16(dv[t]);
+                if (dK32) dK32[(size_t)bh * nk + t] = x;
+                if (dV32) dV32[(size_t)bh * nk + t] = dv[t];
+            }
+        }
+        free(q); free(g); free(k); free(kt); free(vt); free(P); free(dp); free(lse);
+        free(dq); free(dk); free(dv);
+    }
+    return fail ? -2 : 0;
+}
+
+/* ------------------------------------------------------------------------------------------
+ * SageAttention int8-QK inference variant.
+ *
+ * Spec (all fp32 unless stated):
+ *   kmean[b,h,c] = (float)( (double) sum_t K[b,h,t,c] / Sk )      sum carried in fp64, which is
+ *                  exact for bf16 addends of ordinary magnitude and so independent of order
+ *   Ks           = bf16_rne( (float)K - kmean )
+ *   sq[b,h,i]    = max |Q[b,h, i*qblk : (i+1)*qblk, :]| / 127     (IEEE fp32 division)
+ *   sk[b,h,j]    = max |Ks[b,h, j*kblk : (j+1)*kblk, :]| / 127
+ *   Qi8          = clamp(rintf((float)Q / sq), -128, 127)         (IEEE division, ties to even)
+ *   Ki8          = clamp(rintf((float)Ks / sk), -128, 127)
+ *   absmax == 0  => scale = 0 and every quantised value of the block = 0
+ * The last block of a sequence may be short.
+ * ------------------------------------------------------------------------------------------ */
+static inline int8_t quant1(float x, float s) {
+    if (s == 0.f) return 0;
+    float r = rintf(x / s);
+    if (r > 127.f) r = 127.f;
+    if (r < -128.f) r = -128.f;
+    return (int8_t)r;
+}
+
+int oracle_sage_quant(const uint16_t* Q, const uint16_t* K,
+                      int B, int H, int Sq, int Sk, int D, int qblk, int kblk, int smooth_k,
+                      float* kmean /*[B,H,D]*/, uint16_t* Ks /*[B,H,Sk,D] or NULL*/,
+                      int8_t* Qi8, int8_t* Ki8,
+                      float* sq /*[B,H,ceil(Sq/qblk)]*/, float* sk /*[B,H,ceil(Sk/kblk)]*/) {
+    if (check_dims(B, H, Sq, Sk, D) || qblk <= 0 || kblk <= 0) return -1;
+    const int nqb = (Sq + qblk - 1) / qblk, nkb = (Sk + kblk - 1) / kblk;
+    int fail = 0;
+#pragma omp parallel for schedule(dynamic, 1)
+    for (int bh = 0; bh < B * H; ++bh) {
+        const uint16_t* Qh = Q + (size_t)bh * Sq * D;
+        const uint16_t* Kh = K + (size_t)bh * Sk * D;
+        float* mu = kmean + (size_t)bh * D;
+        float* ks = (float*)malloc(sizeof(float) * (size_t)Sk * D);
+        if (!ks) { fail = 1; continue; }
+        for (int c = 0; c < D; ++c) {
+            double acc = 0.0;
+            if (smooth_k)
+                for (int t = 0; t < Sk; ++t) acc += (double)bf16_to_f32(Kh[(size_t)t * D + c]);
+            mu[c] = smooth_k ? (float)(acc / (double)Sk) : 0.f;
+        }
+        for (int t = 0; t < Sk; ++t)
+            for (int c = 0; c < D; ++c) {
+                const uint16_t r = f32_to_bf16(bf16_to_f32(Kh[(size_t)t * D + c]) - mu[c]);
+                ks[(size_t)t * D + c] = bf16_to_f32(r);
+                if (Ks) Ks[((size_t)bh * Sk + t) * D + c] = r;
+            }
+        for (int ib = 0; ib < nqb; ++ib) {
+            const int r0 = ib * qblk, r1 = (r0 + qblk < Sq) ? r0 + qblk : Sq;
+            float amax = 0.f;
+            for (size_t t = (size_t)r0 * D; t < (size_t)r1 * D; ++t) {
+                const float a = fabsf(bf16_to_f32(Qh[t]));
+                if (a > amax) amax = a;
+            }
+            const float s = amax / 127.0f;
+            sq[(size_t)bh * nqb + ib] = s;
+            for (size_t t = (size_t)r0 * D; t < (size_t)r1 * D; ++t)
+                Qi8[(size_t)bh * Sq * D + t] = quant1(bf16_to_f32(Qh[t]), s);
+        }
+        for (int jb = 0; jb < nkb; ++jb) {
+            const int r0 = jb * kblk, r1 = (r0 + kblk < Sk) ? r0 + kblk : Sk;
+            float amax = 0.f;
+            for (size_t t = (size_t)r0 * D; t < (size_t)r1 * D; ++t) {
+                const float a = fabsf(ks[t]);
+                if (a > amax) amax = a;
+            }
+            const float s = amax / 127.0f;
+            sk[(size_t)bh * nkb + jb] = s;
+            for (size_t t = (size_t)r0 * D; t < (size_t)r1 * D; ++t)
+                Ki8[(size_t)bh * Sk * D + t] = quant1(ks[t], s);
+        }
+        free(ks);
+    }
+    return fail ? -2 : 0;
+}
+
+/*
+ * Sage forward from quantised operands:
+ *   S_ij = (float)(int32 sum_d Qi8_id Ki8_jd) * sq[i/qblk] * sk[j/kblk] * scale
+ *   P = softmax(S) in fp32 (naive, materialised); O = P V -> bf16.
+ */
+int oracle_sage_fwd(const int8_t* Qi8, const int8_t* Ki8, const float* sq, const float* sk,
+                    const uint16_t* V, int B, int H, int Sq, int Sk, int D, int qblk, int kblk,
+                    float scale, int causal, int heads_begin, int heads_end,
+                    uint16_t* O, float* LSE) {
+    if (check_dims(B, H, Sq, Sk, D) || qblk <= 0 || kblk <= 0) return -1;
+    const int nqb = (Sq + qblk - 1) / qblk, nkb = (Sk + kblk - 1) / kblk;
+    int fail = 0;
+#pragma omp parallel for schedule(dynamic, 1)
+    for (int bh = heads_begin; bh < heads_end; ++bh) {
+        float* v = (float*)malloc(sizeof(float) * (size_t)Sk * D);
+        float* row = (float*)malloc(sizeof(float) * (size_t)Sk);
+        float* o = (float*)malloc(sizeof(float) * (size_t)D);
+        if (!v || !row || !o) {
+            fail = 1;
+        } else {
+            const int8_t* Qh = Qi8 + (size_t)bh * Sq * D;
+            const int8_t* Kh = Ki8 + (size_t)bh * Sk * D;
+            const uint16_t* Vh = V + (size_t)bh * Sk * D;
+            for (size_t t = 0; t < (size_t)Sk * D; ++t) v[t] = bf16_to_f32(Vh[t]);
+            for (int i = 0; i < Sq; ++i) {
+                const float sqi = sq[(size_t)bh * nqb + i / qblk];
+                float m = -INFINITY;
+                for (int j = 0; j < Sk; ++j) {
+                    int32_t acc = 0;
+                    for (int d = 0; d < D; ++d)
+                        acc += (int32_t)Qh[(size_t)i * D + d] * (int32_t)Kh[(size_t)j * D + d];
+                    float s = (float)acc * (sqi * sk[(size_t)bh * nkb + j / kblk] * scale);
+                    if (causal && j > i) s = -INFINITY;
+                    row[j] = s;
+                    if (s > m) m = s;
+                }
+                float l = 0.f;
+                for (int j = 0; j < Sk; ++j) { row[j] = expf(row[j] - m); l += row[j]; }
+                for (int d = 0; d < D; ++d) o[d] = 0.f;
+                for (int j = 0; j < Sk; ++j) {
+                    const float p = row[j] / l;
+                    for (int d = 0; d < D; ++d) o[d] += p * v[(size_t)j * D + d];
+                }
+                for (int d = 0; d < D; ++d) O[((size_t)bh * Sq + i) * D + d] = f32_to_bf16(o[d]);
+                if (LSE) LSE[(size_t)bh * Sq + i] = m + logf(l);
+            }
+        }
+        free(v); free(row); free(o);
+    }
+    return fail ? -2 : 0;
+}
