@@ -1,0 +1,40 @@
+"""Compiles the HIP sources of the attention library for gfx950 into ``flame_amd/lib``.
+
+``python -m flame_amd.build`` (or ``build_lib()``) cross-compiles with hipcc; no GPU is needed.
+"""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB_DIR = os.path.join(HERE, "lib")
+LIB_PATH = os.path.join(LIB_DIR, "libflame_attn_hip.so")
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",   # keep packed fp32 VALU ops off
+    "-Wall", "-Wno-unused-function",
+]
+
+
+def build_lib(verbose: bool = False, extra=()) -> str:
+    os.makedirs(LIB_DIR, exist_ok=True)
+    src = os.path.join(CSRC, "flame_attn.hip")
+    cmd = [HIPCC, *FLAGS, *extra, src, "-o", LIB_PATH]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in res.stdout.splitlines() if "packed-fp32-ops" not in l)
+    if res.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + out)
+    if verbose and out.strip():
+        print(out)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    print(build_lib(verbose=True, extra=sys.argv[1:]))

@@ -1,0 +1,76 @@
+"""ctypes binding of ``libflame_attn_hip.so`` (the C ABI declared in ``include/flame_attn.h``).
+
+Tensors are torch CUDA(HIP) tensors used purely as device-memory handles: the library receives raw
+pointers, element strides and the current HIP stream.  There is no CPU path: if the shared library
+is missing or a call fails, an exception is raised.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libflame_attn_hip.so")
+_lib = None
+
+OK, ERR_INVALID, ERR_UNSUPPORTED = 0, -1, -2
+
+
+class FlameAttnError(RuntimeError):
+    def __init__(self, fn: str, code: int):
+        self.code = code
+        kind = {ERR_INVALID: "invalid argument", ERR_UNSUPPORTED: "unsupported"}.get(code, "HIP error")
+        super().__init__(f"{fn} failed: {kind} ({code})")
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise FileNotFoundError(
+                f"{LIB_PATH} is missing: build it with `python -m flame_amd.build` (hipcc, gfx950)")
+        _lib = ctypes.CDLL(LIB_PATH)
+    return _lib
+
+
+def _i64x4(vals):
+    return (ctypes.c_int64 * 4)(*[int(v) for v in vals])
+
+
+def _ptr(t):
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _mask_strides(mask, B, H, Sq, Sk):
+    if mask is None:
+        return None
+    assert mask.dtype == torch.uint8 and mask.dim() == 4
+    full = (B, H, Sq, Sk)
+    st = []
+    for ax in range(4):
+        assert mask.shape[ax] in (1, full[ax]), "mask is not broadcastable to [B,H,Sq,Sk]"
+        st.append(0 if (mask.shape[ax] == 1 and full[ax] != 1) else mask.stride(ax))
+    return _i64x4(st)
+
+
+def attn_fwd(q, k, v, scale, causal=False, kv_len=None, mask=None, want_lse=True, out=None):
+    """O, LSE = flame_attn_fwd_bf16(...).  q [B,H,Sq,D], k/v [B,H,Sk,D] bf16, D stride 1."""
+    B, H, Sq, D = q.shape
+    Sk = k.shape[2]
+    o = torch.empty((B, H, Sq, D), dtype=torch.bfloat16, device=q.device) if out is None else out
+    lse = torch.empty((B * H, Sq), dtype=torch.float32, device=q.device) if want_lse else None
+    ms = _mask_strides(mask, B, H, Sq, Sk)
+    rc = lib().flame_attn_fwd_bf16(
+        _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), B, H, Sq, Sk, D, ctypes.c_float(scale),
+        _i64x4(q.stride()), _i64x4(k.stride()), _i64x4(v.stride()), _i64x4(o.stride()),
+        *(ctypes.c_int64(0) for _ in range(5)),
+        int(bool(causal)), _ptr(kv_len), _ptr(mask), ms, _stream())
+    if rc != 0:
+        raise FlameAttnError("flame_attn_fwd_bf16", rc)
+    return o, lse

@@ -1,0 +1,97 @@
+// Shared device helpers for the gfx950 (CDNA4) attention kernels: 64-lane wavefronts,
+// v_mfma_f32_32x32x16_bf16 fragments, bf16 packing.  Compiled for gfx950 only.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace fattn {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kWave = 64;
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+// ---------------------------------------------------------------------------------------------
+// v_mfma_f32_32x32x16_bf16:  D[32x32] += A[32x16] * B[16x32]
+//   lane l, half h = l/32, n = l%32
+//   A operand: 8 bf16 = A[n][8h .. 8h+7]        (row n, eight consecutive k)
+//   B operand: 8 bf16 = B[8h .. 8h+7][n]        (column n, eight consecutive k)
+//   C/D      : 16 f32, register r holds D[8*(r/4) + 4h + (r%4)][n]
+// Because the k positions of A and B only have to agree with each other, any fixed permutation of
+// the contraction index may be applied to both operands.
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+
+// row index inside a 32x32 accumulator block for register r of a lane in half h
+__device__ __forceinline__ constexpr int acc_row(int r, int h) { return 8 * (r >> 2) + 4 * h + (r & 3); }
+
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+    f32x2 v = {lo, hi};
+    bf16x2 b = __builtin_convertvector(v, bf16x2);   // v_cvt_pk_bf16_f32, round-to-nearest-even
+    return __builtin_bit_cast(uint32_t, b);
+}
+
+__device__ __forceinline__ bf16x8 pack8(float a0, float a1, float a2, float a3, float a4, float a5, float a6,
+                                        float a7) {
+    u32x4 u = {pack_bf16(a0, a1), pack_bf16(a2, a3), pack_bf16(a4, a5), pack_bf16(a6, a7)};
+    return __builtin_bit_cast(bf16x8, u);
+}
+
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return __builtin_bit_cast(float, w & 0xffff0000u); }
+
+__device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }   // v_exp_f32
+__device__ __forceinline__ float log2_fast(float x) { return __builtin_amdgcn_logf(x); }    // v_log_f32
+
+// exchange with the lane 32 positions away (the other half of the wave)
+__device__ __forceinline__ float xhalf(float x) { return __shfl_xor(x, 32, 64); }
+
+// 16-byte global load of 8 bf16, zero when the predicate is false
+__device__ __forceinline__ u32x4 ldg16(const uint16_t* p, bool ok) {
+    u32x4 z = {0u, 0u, 0u, 0u};
+    return ok ? *reinterpret_cast<const u32x4*>(p) : z;
+}
+
+// Transposes a 4 (rows) x 8 (cols) block of bf16 held as four 16-byte row vectors into eight
+// 8-byte column vectors: out[c] = {r0[c], r1[c], r2[c], r3[c]}.
+__device__ __forceinline__ void transpose4x8(const u32x4 r[4], u32x2 out[8]) {
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+        const uint32_t a = r[0][m], b = r[1][m], c = r[2][m], d = r[3][m];
+        out[2 * m][0] = (a & 0xffffu) | (b << 16);
+        out[2 * m][1] = (c & 0xffffu) | (d << 16);
+        out[2 * m + 1][0] = (a >> 16) | (b & 0xffff0000u);
+        out[2 * m + 1][1] = (c >> 16) | (d & 0xffff0000u);
+    }
+}
+
+// Position of the 4-row group g (rows 4g..4g+3 of a tile) inside a transposed LDS row, chosen so
+// that the eight contraction slots one lane feeds to an MFMA are 16 contiguous bytes:
+// an accumulator lane in half h holds rows {16c+4h+t} and {16c+8+4h+t}, t=0..3, of chunk c, i.e.
+// groups 4c+h and 4c+2+h; they are stored at slots 4c+2h and 4c+2h+1.
+__device__ __forceinline__ constexpr int tslot(int g) { return (g & ~3) | ((g & 1) << 1) | ((g >> 1) & 1); }
+
+struct Strides {
+    int64_t b, h, n;   // element strides of a [B,H,N,D] bf16 view; the D stride is 1
+};
+
+struct MaskArgs {
+    const int32_t* kv_len;   // [B] or null
+    const uint8_t* mask;     // keep-mask (non-zero = attend) or null
+    int64_t sb, sh, sq, sk;  // element strides over (b,h,q,k); 0 broadcasts
+    int causal;              // key j > query i is excluded
+};
+
+}  // namespace fattn

@@ -1,0 +1,94 @@
+// C ABI of the gfx950 attention library: argument validation and kernel launches.
+// No allocation, no host synchronisation, no global state: every call only enqueues kernels on the
+// caller's stream, so calls may be captured into a HIP graph.
+#include "../../include/flame_attn.h"
+
+#include <hip/hip_runtime.h>
+#include <math.h>
+#include <stdio.h>
+
+#include "attn_fwd.hpp"
+
+using namespace fattn;
+
+namespace {
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// [B,H,N,D] element strides: D stride must be 1, the others multiples of 8 (16-byte rows)
+int check_view(const void* base, const int64_t* st, int64_t off) {
+    if (!base || !st) return FLAME_ATTN_ERR_INVALID;
+    if (st[3] != 1) return FLAME_ATTN_ERR_UNSUPPORTED;
+    if ((st[0] | st[1] | st[2] | off) & 7) return FLAME_ATTN_ERR_UNSUPPORTED;
+    if (st[0] < 0 || st[1] < 0 || st[2] < 0) return FLAME_ATTN_ERR_UNSUPPORTED;
+    if (!aligned16(static_cast<const uint16_t*>(base) + off)) return FLAME_ATTN_ERR_UNSUPPORTED;
+    return FLAME_ATTN_OK;
+}
+
+Strides mk(const int64_t* st) { return Strides{st[0], st[1], st[2]}; }
+
+template <int D, int NWQ>
+int launch_fwd(const FwdParams& p, hipStream_t s) {
+    using T = FwdTile<D>;
+    constexpr int BM = 128 * NWQ;
+    static bool attr_done = false;   // idempotent, so a benign race at worst repeats the call
+    auto kern = fwd_kernel<D, NWQ>;
+    if (!attr_done) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS_BYTES);
+        if (e != hipSuccess) return (int)e;
+        attr_done = true;
+    }
+    const int64_t n_qt = (p.Sq + BM - 1) / BM;
+    const int64_t grid = n_qt * p.B * p.H;
+    if (grid > 0x7fffffff) return FLAME_ATTN_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), T::LDS_BYTES, s, p);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? FLAME_ATTN_OK : (int)e;
+}
+
+}  // namespace
+
+extern "C" {
+
+int flame_attn_fwd_bf16(const void* Q, const void* K, const void* V, void* O, void* LSE,
+                        int B, int H, int N_q, int N_kv, int D, float scale,
+                        const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                        const int64_t* o_strides,
+                        int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off, int64_t lse_off,
+                        int causal, const int32_t* kv_len,
+                        const uint8_t* keep_mask, const int64_t* mask_strides,
+                        void* stream) {
+    if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0) return FLAME_ATTN_ERR_INVALID;
+    if (!(scale > 0.f) || !isfinite(scale)) return FLAME_ATTN_ERR_INVALID;
+    if (D != 64 && D != 128) return FLAME_ATTN_ERR_UNSUPPORTED;
+    int rc;
+    if ((rc = check_view(Q, q_strides, q_off))) return rc;
+    if ((rc = check_view(K, k_strides, k_off))) return rc;
+    if ((rc = check_view(V, v_strides, v_off))) return rc;
+    if ((rc = check_view(O, o_strides, o_off))) return rc;
+    if (keep_mask && !mask_strides) return FLAME_ATTN_ERR_INVALID;
+
+    FwdParams p;
+    p.q = static_cast<const uint16_t*>(Q) + q_off;
+    p.k = static_cast<const uint16_t*>(K) + k_off;
+    p.v = static_cast<const uint16_t*>(V) + v_off;
+    p.o = static_cast<uint16_t*>(O) + o_off;
+    p.lse = LSE ? static_cast<float*>(LSE) + lse_off : nullptr;
+    p.qs = mk(q_strides); p.ks = mk(k_strides); p.vs = mk(v_strides); p.os = mk(o_strides);
+    p.B = B; p.H = H; p.Sq = N_q; p.Sk = N_kv;
+    p.scale = scale;
+    p.m.kv_len = kv_len;
+    p.m.mask = keep_mask;
+    p.m.sb = keep_mask ? mask_strides[0] : 0;
+    p.m.sh = keep_mask ? mask_strides[1] : 0;
+    p.m.sq = keep_mask ? mask_strides[2] : 0;
+    p.m.sk = keep_mask ? mask_strides[3] : 0;
+    p.m.causal = causal ? 1 : 0;
+
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (D == 128) return launch_fwd<128, 1>(p, s);
+    return launch_fwd<64, 1>(p, s);
+}
+
+}  // extern "C"
