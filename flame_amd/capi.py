@@ -74,3 +74,37 @@ def attn_fwd(q, k, v, scale, causal=False, kv_len=None, mask=None, want_lse=True
     if rc != 0:
         raise FlameAttnError("flame_attn_fwd_bf16", rc)
     return o, lse
+
+
+def bwd_workspace_bytes(B, H, Sq, D) -> int:
+    f = lib().flame_attn_bwd_workspace_bytes
+    f.restype = ctypes.c_size_t
+    return int(f(B, H, Sq, D))
+
+
+def attn_bwd(q, k, v, o, do, lse, scale, causal=False, kv_len=None, mask=None, workspace=None, grads=None):
+    """dQ, dK, dV = flame_attn_bwd_bf16(...).  `workspace`: uint8 device tensor of at least
+    bwd_workspace_bytes(...) bytes (allocated here when omitted)."""
+    B, H, Sq, D = q.shape
+    Sk = k.shape[2]
+    need = bwd_workspace_bytes(B, H, Sq, D)
+    if workspace is None:
+        workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
+    if grads is None:
+        dq = torch.empty((B, H, Sq, D), dtype=torch.bfloat16, device=q.device)
+        dk = torch.empty((B, H, Sk, D), dtype=torch.bfloat16, device=q.device)
+        dv = torch.empty((B, H, Sk, D), dtype=torch.bfloat16, device=q.device)
+    else:
+        dq, dk, dv = grads
+    ms = _mask_strides(mask, B, H, Sq, Sk)
+    rc = lib().flame_attn_bwd_bf16(
+        _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(do), _ptr(lse), _ptr(dq), _ptr(dk), _ptr(dv),
+        B, H, Sq, Sk, D, ctypes.c_float(scale),
+        _i64x4(q.stride()), _i64x4(k.stride()), _i64x4(v.stride()), _i64x4(o.stride()),
+        _i64x4(do.stride()), _i64x4(dq.stride()), _i64x4(dk.stride()), _i64x4(dv.stride()),
+        *(ctypes.c_int64(0) for _ in range(9)),
+        int(bool(causal)), _ptr(kv_len), _ptr(mask), ms,
+        _ptr(workspace), ctypes.c_size_t(workspace.numel()), _stream())
+    if rc != 0:
+        raise FlameAttnError("flame_attn_bwd_bf16", rc)
+    return dq, dk, dv

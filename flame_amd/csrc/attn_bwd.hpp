@@ -1,0 +1,362 @@
+// Backward of the tiled attention for gfx950: recomputes P tile by tile from Q, K and the saved
+// log-sum-exp, never materialising the Sq x Sk matrix.
+//
+//   prep     delta_i = sum_d dO_id * O_id   (fp32), and clears the fp32 dQ accumulator
+//   main     one workgroup owns 128 keys (32 per wavefront) of one (batch, head) and walks over the
+//            query tiles (64 rows): S = Q K^T, dP = dO V^T, P = exp2(S*c - LSE*log2e),
+//            dS = P * (dP - delta); dV^T += dO^T P and dK^T += Q^T dS stay in registers for the
+//            whole walk (P and dS are used as MFMA operands straight from the accumulators);
+//            dS goes through LDS once to be re-read with keys as the contraction index for
+//            dQ += dS K, which is added to an fp32 accumulator in HBM with hardware atomics
+//   convert  dQ = bf16(scale * accumulator)
+//
+// Q and dO tiles are staged row-major; their transposed MFMA operands (Q^T, dO^T) and the dS
+// operand come from transposing LDS reads, so no tile is stored twice.
+#pragma once
+#include "attn_common.hpp"
+
+namespace fattn {
+
+struct BwdParams {
+    const uint16_t* q;
+    const uint16_t* k;
+    const uint16_t* v;
+    const uint16_t* o;
+    const uint16_t* dout;
+    const float* lse;     // contiguous [B*H, Sq]
+    uint16_t* dq;
+    uint16_t* dk;
+    uint16_t* dv;
+    float* delta;         // workspace, [B*H, Sq]
+    float* dq_acc;        // workspace, [B*H, Sq, D] fp32
+    Strides qs, ks, vs, os, dos, dqs, dks, dvs;
+    int B, H, Sq, Sk;
+    float scale;
+    MaskArgs m;
+};
+
+// ------------------------------------------------------------------------------------------ prep
+template <int D>
+__global__ __launch_bounds__(256) void bwd_prep_kernel(const BwdParams p) {
+    constexpr int TPR = D / 8;            // threads per row
+    constexpr int RPB = 256 / TPR;        // rows per block
+    const int tid = threadIdx.x;
+    const int64_t row_flat = (int64_t)blockIdx.x * RPB + tid / TPR;   // over B*H*Sq
+    const int chunk = tid % TPR;
+    const int64_t total = (int64_t)p.B * p.H * p.Sq;
+    float acc = 0.f;
+    const bool ok = row_flat < total;
+    if (ok) {
+        const int row = (int)(row_flat % p.Sq);
+        const int bh = (int)(row_flat / p.Sq);
+        const int b = bh / p.H, hh = bh % p.H;
+        const u32x4 a = *reinterpret_cast<const u32x4*>(p.dout + b * p.dos.b + hh * p.dos.h + (int64_t)row * p.dos.n + chunk * 8);
+        const u32x4 c = *reinterpret_cast<const u32x4*>(p.o + b * p.os.b + hh * p.os.h + (int64_t)row * p.os.n + chunk * 8);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc += bf16_lo(a[i]) * bf16_lo(c[i]) + bf16_hi(a[i]) * bf16_hi(c[i]);
+        f32x4 z = {0.f, 0.f, 0.f, 0.f};
+        f32x4* dst = reinterpret_cast<f32x4*>(p.dq_acc + row_flat * D + chunk * 8);
+        dst[0] = z;
+        dst[1] = z;
+    }
+#pragma unroll
+    for (int off = TPR / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+    if (ok && chunk == 0) p.delta[row_flat] = acc;
+}
+
+// --------------------------------------------------------------------------------------- convert
+template <int D>
+__global__ __launch_bounds__(256) void bwd_dq_convert_kernel(const BwdParams p) {
+    constexpr int TPR = D / 8;
+    constexpr int RPB = 256 / TPR;
+    const int tid = threadIdx.x;
+    const int64_t row_flat = (int64_t)blockIdx.x * RPB + tid / TPR;
+    const int chunk = tid % TPR;
+    if (row_flat >= (int64_t)p.B * p.H * p.Sq) return;
+    const int row = (int)(row_flat % p.Sq);
+    const int bh = (int)(row_flat / p.Sq);
+    const int b = bh / p.H, hh = bh % p.H;
+    const f32x4* src = reinterpret_cast<const f32x4*>(p.dq_acc + row_flat * D + chunk * 8);
+    const f32x4 x = src[0], y = src[1];
+    const float s = p.scale;
+    u32x4 w = {pack_bf16(x[0] * s, x[1] * s), pack_bf16(x[2] * s, x[3] * s), pack_bf16(y[0] * s, y[1] * s),
+               pack_bf16(y[2] * s, y[3] * s)};
+    *reinterpret_cast<u32x4*>(p.dq + b * p.dqs.b + hh * p.dqs.h + (int64_t)row * p.dqs.n + chunk * 8) = w;
+}
+
+// ------------------------------------------------------------------------------------------ main
+template <int D>
+struct BwdTile {
+    static constexpr int BM = 64;              // query rows per step
+    static constexpr int BN = 128;             // keys per workgroup
+    static constexpr int QS = D + 8;           // LDS row stride of the Q / dO / K / V tiles
+    static constexpr int DSS = BM + 8;         // LDS row stride of dS^T [key][query]
+    static constexpr int Q_ELEMS = BM * QS;
+    static constexpr int DS_ELEMS = BN * DSS;
+    static constexpr int LDS_BYTES = (2 * Q_ELEMS + DS_ELEMS) * 2 + 2 * BM * 4;
+    static constexpr int NC = BM * (D / 8) / 256;    // 16-byte chunks per thread per 64-row tile
+};
+
+template <int D>
+__global__ __launch_bounds__(256) void bwd_kernel(const BwdParams p) {
+    using T = BwdTile<D>;
+    constexpr int BM = T::BM, BN = T::BN, QS = T::QS, DSS = T::DSS, NC = T::NC;
+    constexpr int DC = D / 16;     // contraction chunks over the head dim
+    constexpr int DB = D / 32;     // 32-row blocks of dK^T / dV^T
+    constexpr int NSL = D / 32;    // 32-column slices of dQ
+    constexpr int QB_PER = 2 / (4 / NSL);   // query blocks per wave in the dQ step
+
+    extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
+    uint16_t* Qs = lds;                       // [BM][QS]
+    uint16_t* dOs = lds + T::Q_ELEMS;         // [BM][QS]   (Qs and dOs together also hold a [BN][QS] tile in the prologue)
+    uint16_t* dSt = lds + 2 * T::Q_ELEMS;     // [BN][DSS]
+    float* lse_s = reinterpret_cast<float*>(lds + 2 * T::Q_ELEMS + T::DS_ELEMS);   // [BM], pre-multiplied by log2(e)
+    float* delta_s = lse_s + BM;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int n = lane & 31, h = lane >> 5;
+
+    const int n_kt = (p.Sk + BN - 1) / BN;
+    const int kt = blockIdx.x % n_kt;
+    const int bh = blockIdx.x / n_kt;
+    const int b = bh / p.H, hh = bh % p.H;
+    const int k0 = kt * BN;
+    const int kw0 = k0 + 32 * wave;
+
+    const uint16_t* qbase = p.q + b * p.qs.b + hh * p.qs.h;
+    const uint16_t* kbase = p.k + b * p.ks.b + hh * p.ks.h;
+    const uint16_t* vbase = p.v + b * p.vs.b + hh * p.vs.h;
+    const uint16_t* dobase = p.dout + b * p.dos.b + hh * p.dos.h;
+    const float* lsebase = p.lse + (int64_t)bh * p.Sq;
+    const float* deltabase = p.delta + (int64_t)bh * p.Sq;
+    float* dqacc_base = p.dq_acc + (int64_t)bh * p.Sq * D;
+
+    int klimit = p.Sk;
+    if (p.m.kv_len) klimit = min(klimit, max(p.m.kv_len[b], 0));
+    const uint8_t* mbase = p.m.mask ? p.m.mask + b * p.m.sb + hh * p.m.sh : nullptr;
+
+    const int n_qt = (p.Sq + BM - 1) / BM;
+    int qt_begin = p.m.causal ? (k0 / BM) : 0;
+    if (k0 >= klimit) qt_begin = n_qt;        // nothing attends to these keys: dK = dV = 0
+
+    // ---- prologue: K and V fragments of this wavefront's 32 keys, held in registers for the walk
+    bf16x8 kf[DC], vf[DC], ktf[BN / 16];
+    {
+        constexpr int NCK = BN * (D / 8) / 256;
+#pragma unroll
+        for (int pass = 0; pass < 2; ++pass) {
+            const uint16_t* src = pass == 0 ? kbase : vbase;
+            const Strides st = pass == 0 ? p.ks : p.vs;
+            const int lim = pass == 0 ? p.Sk : klimit;
+#pragma unroll
+            for (int i = 0; i < NCK; ++i) {
+                const int c = tid + 256 * i;
+                const int row = c / (D / 8), col = c % (D / 8);
+                const int key = k0 + row;
+                *reinterpret_cast<u32x4*>(lds + row * QS + col * 8) = ldg16(src + (int64_t)key * st.n + col * 8, key < lim);
+            }
+            __syncthreads();
+#pragma unroll
+            for (int dc = 0; dc < DC; ++dc) {
+                const bf16x8 f = *reinterpret_cast<const bf16x8*>(lds + (32 * wave + n) * QS + 16 * dc + 8 * h);
+                if (pass == 0) kf[dc] = f; else vf[dc] = f;
+            }
+            if (pass == 0) {
+#pragma unroll
+                for (int kc = 0; kc < BN / 16; ++kc) ktf[kc] = lds_tr_frag(lds, QS, 16 * kc, 32 * (wave % NSL), lane);
+            }
+            __syncthreads();
+        }
+    }
+
+    // ---- staging of the 64-row Q / dO tiles
+    u32x4 qreg[NC], doreg[NC];
+    float lse_reg = 0.f, delta_reg = 0.f;
+    auto load_q_tile = [&](int qt) {
+        const int q0 = qt * BM;
+#pragma unroll
+        for (int i = 0; i < NC; ++i) {
+            const int c = tid + 256 * i;
+            const int row = c / (D / 8), col = c % (D / 8);
+            const int qi = q0 + row;
+            qreg[i] = ldg16(qbase + (int64_t)qi * p.qs.n + col * 8, qi < p.Sq);
+            doreg[i] = ldg16(dobase + (int64_t)qi * p.dos.n + col * 8, qi < p.Sq);
+        }
+        if (tid < BM) {
+            const int qi = q0 + tid;
+            float l = INFINITY;
+            float dl = 0.f;
+            if (qi < p.Sq) {
+                const float x = lsebase[qi];
+                l = (x == -INFINITY) ? INFINITY : x * kLog2e;    // +inf makes exp2(s*c - l) = 0
+                dl = deltabase[qi];
+            }
+            lse_reg = l;
+            delta_reg = dl;
+        }
+    };
+    auto store_q_tile = [&]() {
+#pragma unroll
+        for (int i = 0; i < NC; ++i) {
+            const int c = tid + 256 * i;
+            const int row = c / (D / 8), col = c % (D / 8);
+            *reinterpret_cast<u32x4*>(Qs + row * QS + col * 8) = qreg[i];
+            *reinterpret_cast<u32x4*>(dOs + row * QS + col * 8) = doreg[i];
+        }
+        if (tid < BM) {
+            lse_s[tid] = lse_reg;
+            delta_s[tid] = delta_reg;
+        }
+    };
+
+    f32x16 dkacc[DB], dvacc[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            dkacc[db][r] = 0.f;
+            dvacc[db][r] = 0.f;
+        }
+
+    const float c_log2 = p.scale * kLog2e;
+    const int dslice = wave % NSL;
+    const int qb_first = (wave / NSL) * QB_PER;
+
+    if (qt_begin < n_qt) {
+        load_q_tile(qt_begin);
+        store_q_tile();
+    }
+    __syncthreads();
+
+    for (int qt = qt_begin; qt < n_qt; ++qt) {
+        const int q0 = qt * BM;
+        const bool more = (qt + 1) < n_qt;
+        if (more) load_q_tile(qt + 1);
+
+        // ---- S = Q K^T and dP = dO V^T : rows = queries (two blocks of 32), columns = this wave's keys
+        f32x16 sacc[2], dpacc[2];
+#pragma unroll
+        for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                sacc[qb][r] = 0.f;
+                dpacc[qb][r] = 0.f;
+            }
+#pragma unroll
+        for (int dc = 0; dc < DC; ++dc) {
+#pragma unroll
+            for (int qb = 0; qb < 2; ++qb) {
+                const bf16x8 aq = *reinterpret_cast<const bf16x8*>(Qs + (32 * qb + n) * QS + 16 * dc + 8 * h);
+                sacc[qb] = mfma32(aq, kf[dc], sacc[qb]);
+                const bf16x8 ad = *reinterpret_cast<const bf16x8*>(dOs + (32 * qb + n) * QS + 16 * dc + 8 * h);
+                dpacc[qb] = mfma32(ad, vf[dc], dpacc[qb]);
+            }
+        }
+
+        // ---- P and dS; lane = key column kw0+n, registers = queries
+        const int key = kw0 + n;
+        const bool need_mask = (k0 + BN > klimit) || (p.m.causal && (k0 + BN - 1 > q0)) || mbase;
+        bf16x8 pf[2][2], dsf[2][2];
+#pragma unroll
+        for (int qb = 0; qb < 2; ++qb) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const f32x4 l4 = *reinterpret_cast<const f32x4*>(lse_s + 32 * qb + 8 * g + 4 * h);
+                const f32x4 d4 = *reinterpret_cast<const f32x4*>(delta_s + 32 * qb + 8 * g + 4 * h);
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const int r = 4 * g + t;
+                    float pr = exp2_fast(fmaf(sacc[qb][r], c_log2, -l4[t]));
+                    if (need_mask) {
+                        const int qi = q0 + 32 * qb + 8 * g + 4 * h + t;
+                        bool drop = key >= klimit;
+                        if (p.m.causal) drop = drop || key > qi;
+                        if (mbase && !drop && qi < p.Sq)
+                            drop = mbase[(int64_t)qi * p.m.sq + (int64_t)key * p.m.sk] == 0;
+                        if (drop) pr = 0.f;
+                    }
+                    sacc[qb][r] = pr;
+                    dpacc[qb][r] = pr * (dpacc[qb][r] - d4[t]);
+                }
+            }
+#pragma unroll
+            for (int c = 0; c < 2; ++c) {
+                const f32x16& s = sacc[qb];
+                const f32x16& d = dpacc[qb];
+                const int o8 = 8 * c;
+                pf[qb][c] = pack8(s[o8], s[o8 + 1], s[o8 + 2], s[o8 + 3], s[o8 + 4], s[o8 + 5], s[o8 + 6], s[o8 + 7]);
+                dsf[qb][c] = pack8(d[o8], d[o8 + 1], d[o8 + 2], d[o8 + 3], d[o8 + 4], d[o8 + 5], d[o8 + 6], d[o8 + 7]);
+            }
+            // dS^T[key][query]: four consecutive queries per 8-byte store
+            const u32x4 dsu0 = __builtin_bit_cast(u32x4, dsf[qb][0]);
+            const u32x4 dsu1 = __builtin_bit_cast(u32x4, dsf[qb][1]);
+            uint16_t* drow = dSt + (32 * wave + n) * DSS + 32 * qb + 4 * h;
+            u32x2 w0 = {dsu0[0], dsu0[1]}, w1 = {dsu0[2], dsu0[3]}, w2 = {dsu1[0], dsu1[1]}, w3 = {dsu1[2], dsu1[3]};
+            *reinterpret_cast<u32x2*>(drow + 0) = w0;
+            *reinterpret_cast<u32x2*>(drow + 8) = w1;
+            *reinterpret_cast<u32x2*>(drow + 16) = w2;
+            *reinterpret_cast<u32x2*>(drow + 24) = w3;
+        }
+
+        // ---- dV^T += dO^T P,  dK^T += Q^T dS : rows = d, columns = keys, contraction over the 64 queries
+#pragma unroll
+        for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+            for (int c = 0; c < 2; ++c) {
+                const int cc = 2 * qb + c;
+#pragma unroll
+                for (int db = 0; db < DB; ++db) {
+                    const bf16x8 a_do = lds_tr_frag(dOs, QS, 16 * cc, 32 * db, lane);
+                    dvacc[db] = mfma32(a_do, pf[qb][c], dvacc[db]);
+                    const bf16x8 a_q = lds_tr_frag(Qs, QS, 16 * cc, 32 * db, lane);
+                    dkacc[db] = mfma32(a_q, dsf[qb][c], dkacc[db]);
+                }
+            }
+
+        __syncthreads();   // dS^T complete; every wave is done with this step's Q / dO tiles
+        if (more) store_q_tile();
+
+        // ---- dQ[query][d slice] += dS K : contraction over the 128 keys of the workgroup
+#pragma unroll
+        for (int i = 0; i < QB_PER; ++i) {
+            const int qb = qb_first + i;
+            f32x16 dq;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) dq[r] = 0.f;
+#pragma unroll
+            for (int kc = 0; kc < BN / 16; ++kc) {
+                const bf16x8 a = lds_tr_frag(dSt, DSS, 16 * kc, 32 * qb, lane);
+                dq = mfma32(a, ktf[kc], dq);
+            }
+            float* dst = dqacc_base + (int64_t)(q0 + 32 * qb) * D + 32 * dslice + n;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int ql = acc_row(r, h);
+                if (q0 + 32 * qb + ql < p.Sq) unsafeAtomicAdd(dst + (int64_t)ql * D, dq[r]);
+            }
+        }
+        __syncthreads();   // next tile staged; dS^T free again
+    }
+
+    // ---- epilogue: dK^T / dV^T accumulators -> dK, dV rows of this wavefront's keys
+    const int krow = kw0 + n;
+    if (krow < p.Sk) {
+        uint16_t* dkrow = p.dk + b * p.dks.b + hh * p.dks.h + (int64_t)krow * p.dks.n;
+        uint16_t* dvrow = p.dv + b * p.dvs.b + hh * p.dvs.h + (int64_t)krow * p.dvs.n;
+        const float s = p.scale;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const f32x16& a = dkacc[db];
+                const f32x16& c = dvacc[db];
+                u32x2 wk = {pack_bf16(a[4 * g] * s, a[4 * g + 1] * s), pack_bf16(a[4 * g + 2] * s, a[4 * g + 3] * s)};
+                u32x2 wv = {pack_bf16(c[4 * g], c[4 * g + 1]), pack_bf16(c[4 * g + 2], c[4 * g + 3])};
+                *reinterpret_cast<u32x2*>(dkrow + 32 * db + 8 * g + 4 * h) = wk;
+                *reinterpret_cast<u32x2*>(dvrow + 32 * db + 8 * g + 4 * h) = wv;
+            }
+    }
+}
+
+}  // namespace fattn

@@ -64,6 +64,32 @@ __device__ __forceinline__ u32x4 ldg16(const uint16_t* p, bool ok) {
     return ok ? *reinterpret_cast<const u32x4*>(p) : z;
 }
 
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+
+// ds_read_b64_tr_b16: within each group of 16 lanes, lane i receives element (i%4) of the four
+// 8-byte rows addressed by lanes i/4, i/4+4, i/4+8, i/4+12 of the group.  When lane r of a group
+// points at &X[k0 + r/4][c0 + 4*(r%4)] of a row-major tile X, lane i therefore receives
+// X[k0+0..3][c0+i]: the group transposes a 4(k) x 16(column) block so that every lane ends up with
+// four consecutive contraction elements of its own column.
+__device__ __forceinline__ u32x2 lds_read_tr16(const uint16_t* p) {
+    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+    s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p));
+    return __builtin_bit_cast(u32x2, v);
+}
+
+// MFMA 32x32x16 operand (8 contraction elements for column n = lane%32) gathered from a row-major
+// LDS tile X[k][col]: elements 0..3 = X[k0 + 4h + 0..3][c0 + n], elements 4..7 = X[k0 + 8 + 4h + 0..3][c0 + n].
+// This k order matches a 32x32 accumulator lane (rows 8g + 4h + t), so accumulator values converted
+// to bf16 pair with it directly.
+__device__ __forceinline__ bf16x8 lds_tr_frag(const uint16_t* tile, int stride, int k0, int c0, int lane) {
+    const int r = lane & 15, g16 = (lane >> 4) & 1, h = lane >> 5;
+    const uint16_t* p = tile + (k0 + 4 * h + (r >> 2)) * stride + c0 + 16 * g16 + 4 * (r & 3);
+    const u32x2 lo = lds_read_tr16(p);
+    const u32x2 hi = lds_read_tr16(p + 8 * stride);
+    u32x4 u = {lo[0], lo[1], hi[0], hi[1]};
+    return __builtin_bit_cast(bf16x8, u);
+}
+
 // Transposes a 4 (rows) x 8 (cols) block of bf16 held as four 16-byte row vectors into eight
 // 8-byte column vectors: out[c] = {r0[c], r1[c], r2[c], r3[c]}.
 __device__ __forceinline__ void transpose4x8(const u32x4 r[4], u32x2 out[8]) {

@@ -3,10 +3,11 @@
 //
 // One workgroup = 4 wavefronts = 128*NWQ query rows of one (batch, head); each wavefront owns
 // 32*NWQ rows whose Q fragments stay in registers.  K/V tiles of 64 keys are staged through LDS
-// (double buffered, register prefetch).  The logits are produced transposed, S^T = K Q^T, so that
+// (double buffered, register prefetch), both row-major.  The logits are produced transposed, S^T = K Q^T, so that
 // every lane holds values of a single query: row max / row sum are in-lane reductions plus one
 // exchange between the wave halves, the bf16 P^T values are already in the B-operand layout of the
-// second MFMA (O^T = V^T P^T), and the running rescale of O is a per-lane scalar.
+// second MFMA (O^T = V^T P^T), and the running rescale of O is a per-lane scalar.  The V^T operand
+// of that MFMA is gathered from the row-major V tile with the transposing LDS read.
 #pragma once
 #include "attn_common.hpp"
 
@@ -28,12 +29,12 @@ template <int D>
 struct FwdTile {
     static constexpr int BN = 64;            // keys per tile
     static constexpr int KS = D + 8;         // LDS row stride of the K tile, elements
-    static constexpr int VS = BN + 8;        // LDS row stride of the transposed V tile, elements
+    static constexpr int VS = D + 8;         // LDS row stride of the V tile, elements
     static constexpr int K_ELEMS = BN * KS;
-    static constexpr int V_ELEMS = D * VS;
+    static constexpr int V_ELEMS = BN * VS;
     static constexpr int STAGE_ELEMS = K_ELEMS + V_ELEMS;
     static constexpr int LDS_BYTES = 2 * STAGE_ELEMS * 2;
-    static constexpr int NKC = BN * (D / 8) / 256;   // 16-byte K chunks per thread
+    static constexpr int NKC = BN * (D / 8) / 256;   // 16-byte chunks per thread and tensor
 };
 
 template <int D, int NWQ>
@@ -82,10 +83,7 @@ __global__ __launch_bounds__(256) void fwd_kernel(const FwdParams p) {
 
     // ---- staging assignment
     u32x4 kreg[T::NKC];
-    u32x4 vreg[4];
-    const int vs_chunk = wave * 4 + (lane >> 4);   // 8-wide d chunk handled by this lane
-    const int vg = lane & 15;                      // 4-key group handled by this lane
-    const bool v_active = vs_chunk < D / 8;
+    u32x4 vreg[T::NKC];
 
     auto load_tile = [&](int t) {
         const int key0 = t * BN;
@@ -95,31 +93,18 @@ __global__ __launch_bounds__(256) void fwd_kernel(const FwdParams p) {
             const int row = c / (D / 8), col = c % (D / 8);
             const int key = key0 + row;
             kreg[i] = ldg16(kbase + (int64_t)key * p.ks.n + col * 8, key < p.Sk);
-        }
-        if (v_active) {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int key = key0 + 4 * vg + j;
-                vreg[j] = ldg16(vbase + (int64_t)key * p.vs.n + vs_chunk * 8, key < klimit);
-            }
+            vreg[i] = ldg16(vbase + (int64_t)key * p.vs.n + col * 8, key < klimit);
         }
     };
     auto store_tile = [&](int buf) {
         uint16_t* ks = lds + buf * T::STAGE_ELEMS;
-        uint16_t* vt = ks + T::K_ELEMS;
+        uint16_t* vs = ks + T::K_ELEMS;
 #pragma unroll
         for (int i = 0; i < T::NKC; ++i) {
             const int c = tid + 256 * i;
             const int row = c / (D / 8), col = c % (D / 8);
             *reinterpret_cast<u32x4*>(ks + row * KS + col * 8) = kreg[i];
-        }
-        if (v_active) {
-            u32x2 tr[8];
-            transpose4x8(vreg, tr);
-            const int slot = tslot(vg);
-#pragma unroll
-            for (int c = 0; c < 8; ++c)
-                *reinterpret_cast<u32x2*>(vt + (vs_chunk * 8 + c) * VS + slot * 4) = tr[c];
+            *reinterpret_cast<u32x4*>(vs + row * VS + col * 8) = vreg[i];
         }
     };
 
@@ -149,7 +134,7 @@ __global__ __launch_bounds__(256) void fwd_kernel(const FwdParams p) {
         if (more) load_tile(t + 1);
 
         const uint16_t* ks = lds + buf * T::STAGE_ELEMS;
-        const uint16_t* vt = ks + T::K_ELEMS;
+        const uint16_t* vs = ks + T::K_ELEMS;
         const int key0 = t * BN;
 
         // ---- S^T = K Q^T : rows = keys (two blocks of 32), columns = queries
@@ -234,7 +219,7 @@ __global__ __launch_bounds__(256) void fwd_kernel(const FwdParams p) {
         for (int cc = 0; cc < 4; ++cc) {
 #pragma unroll
             for (int db = 0; db < DB; ++db) {
-                const bf16x8 va = *reinterpret_cast<const bf16x8*>(vt + (32 * db + n) * VS + (4 * cc + 2 * h) * 4);
+                const bf16x8 va = lds_tr_frag(vs, VS, 16 * cc, 32 * db, lane);
 #pragma unroll
                 for (int qb = 0; qb < NWQ; ++qb) oacc[qb][db] = mfma32(va, pf[qb][cc], oacc[qb][db]);
             }

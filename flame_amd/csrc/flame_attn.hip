@@ -7,6 +7,7 @@
 #include <math.h>
 #include <stdio.h>
 
+#include "attn_bwd.hpp"
 #include "attn_fwd.hpp"
 
 using namespace fattn;
@@ -47,9 +48,98 @@ int launch_fwd(const FwdParams& p, hipStream_t s) {
     return e == hipSuccess ? FLAME_ATTN_OK : (int)e;
 }
 
+size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+template <int D>
+int launch_bwd(const BwdParams& p, hipStream_t s) {
+    using T = BwdTile<D>;
+    static bool attr_done = false;
+    auto kern = bwd_kernel<D>;
+    if (!attr_done) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS_BYTES);
+        if (e != hipSuccess) return (int)e;
+        attr_done = true;
+    }
+    constexpr int RPB = 256 / (D / 8);
+    const int64_t rows = (int64_t)p.B * p.H * p.Sq;
+    const int64_t row_blocks = (rows + RPB - 1) / RPB;
+    const int64_t n_kt = (p.Sk + T::BN - 1) / T::BN;
+    const int64_t grid = n_kt * p.B * p.H;
+    if (row_blocks > 0x7fffffff || grid > 0x7fffffff) return FLAME_ATTN_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(bwd_prep_kernel<D>, dim3((unsigned)row_blocks), dim3(256), 0, s, p);
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), T::LDS_BYTES, s, p);
+    hipLaunchKernelGGL(bwd_dq_convert_kernel<D>, dim3((unsigned)row_blocks), dim3(256), 0, s, p);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? FLAME_ATTN_OK : (int)e;
+}
+
 }  // namespace
 
 extern "C" {
+
+size_t flame_attn_bwd_workspace_bytes(int B, int H, int N_q, int D) {
+    if (B <= 0 || H <= 0 || N_q <= 0 || D <= 0) return 0;
+    const size_t rows = (size_t)B * H * N_q;
+    return align_up(rows * sizeof(float), 256) + rows * (size_t)D * sizeof(float);
+}
+
+int flame_attn_bwd_bf16(const void* Q, const void* K, const void* V, const void* O, const void* dO,
+                        const void* LSE, void* dQ, void* dK, void* dV,
+                        int B, int H, int N_q, int N_kv, int D, float scale,
+                        const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                        const int64_t* o_strides, const int64_t* do_strides, const int64_t* dq_strides,
+                        const int64_t* dk_strides, const int64_t* dv_strides,
+                        int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off, int64_t do_off,
+                        int64_t lse_off, int64_t dq_off, int64_t dk_off, int64_t dv_off,
+                        int causal, const int32_t* kv_len,
+                        const uint8_t* keep_mask, const int64_t* mask_strides,
+                        void* workspace, size_t workspace_bytes, void* stream) {
+    if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0) return FLAME_ATTN_ERR_INVALID;
+    if (!(scale > 0.f) || !isfinite(scale)) return FLAME_ATTN_ERR_INVALID;
+    if (!LSE || !workspace) return FLAME_ATTN_ERR_INVALID;
+    if (D != 64 && D != 128) return FLAME_ATTN_ERR_UNSUPPORTED;
+    if (workspace_bytes < flame_attn_bwd_workspace_bytes(B, H, N_q, D)) return FLAME_ATTN_ERR_INVALID;
+    if (!aligned16(workspace)) return FLAME_ATTN_ERR_UNSUPPORTED;
+    int rc;
+    if ((rc = check_view(Q, q_strides, q_off))) return rc;
+    if ((rc = check_view(K, k_strides, k_off))) return rc;
+    if ((rc = check_view(V, v_strides, v_off))) return rc;
+    if ((rc = check_view(O, o_strides, o_off))) return rc;
+    if ((rc = check_view(dO, do_strides, do_off))) return rc;
+    if ((rc = check_view(dQ, dq_strides, dq_off))) return rc;
+    if ((rc = check_view(dK, dk_strides, dk_off))) return rc;
+    if ((rc = check_view(dV, dv_strides, dv_off))) return rc;
+    if (keep_mask && !mask_strides) return FLAME_ATTN_ERR_INVALID;
+
+    BwdParams p;
+    p.q = static_cast<const uint16_t*>(Q) + q_off;
+    p.k = static_cast<const uint16_t*>(K) + k_off;
+    p.v = static_cast<const uint16_t*>(V) + v_off;
+    p.o = static_cast<const uint16_t*>(O) + o_off;
+    p.dout = static_cast<const uint16_t*>(dO) + do_off;
+    p.lse = static_cast<const float*>(LSE) + lse_off;
+    p.dq = static_cast<uint16_t*>(dQ) + dq_off;
+    p.dk = static_cast<uint16_t*>(dK) + dk_off;
+    p.dv = static_cast<uint16_t*>(dV) + dv_off;
+    const size_t rows = (size_t)B * H * N_q;
+    p.delta = static_cast<float*>(workspace);
+    p.dq_acc = reinterpret_cast<float*>(static_cast<char*>(workspace) + align_up(rows * sizeof(float), 256));
+    p.qs = mk(q_strides); p.ks = mk(k_strides); p.vs = mk(v_strides); p.os = mk(o_strides);
+    p.dos = mk(do_strides); p.dqs = mk(dq_strides); p.dks = mk(dk_strides); p.dvs = mk(dv_strides);
+    p.B = B; p.H = H; p.Sq = N_q; p.Sk = N_kv;
+    p.scale = scale;
+    p.m.kv_len = kv_len;
+    p.m.mask = keep_mask;
+    p.m.sb = keep_mask ? mask_strides[0] : 0;
+    p.m.sh = keep_mask ? mask_strides[1] : 0;
+    p.m.sq = keep_mask ? mask_strides[2] : 0;
+    p.m.sk = keep_mask ? mask_strides[3] : 0;
+    p.m.causal = causal ? 1 : 0;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (D == 128) return launch_bwd<128>(p, s);
+    return launch_bwd<64>(p, s);
+}
 
 int flame_attn_fwd_bf16(const void* Q, const void* K, const void* V, void* O, void* LSE,
                         int B, int H, int N_q, int N_kv, int D, float scale,

@@ -1,6 +1,7 @@
 /* placeholder while the kernels come up; replaced by the full header */
 #ifndef FLAME_ATTN_H
 #define FLAME_ATTN_H
+#include <stddef.h>
 #include <stdint.h>
 #ifdef __cplusplus
 extern "C" {
@@ -16,6 +17,18 @@ int flame_attn_fwd_bf16(const void* Q, const void* K, const void* V, void* O, vo
                         int causal, const int32_t* kv_len,
                         const uint8_t* keep_mask, const int64_t* mask_strides,
                         void* stream);
+size_t flame_attn_bwd_workspace_bytes(int B, int H, int N_q, int D);
+int flame_attn_bwd_bf16(const void* Q, const void* K, const void* V, const void* O, const void* dO,
+                        const void* LSE, void* dQ, void* dK, void* dV,
+                        int B, int H, int N_q, int N_kv, int D, float scale,
+                        const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                        const int64_t* o_strides, const int64_t* do_strides, const int64_t* dq_strides,
+                        const int64_t* dk_strides, const int64_t* dv_strides,
+                        int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off, int64_t do_off,
+                        int64_t lse_off, int64_t dq_off, int64_t dk_off, int64_t dv_off,
+                        int causal, const int32_t* kv_len,
+                        const uint8_t* keep_mask, const int64_t* mask_strides,
+                        void* workspace, size_t workspace_bytes, void* stream);
 #ifdef __cplusplus
 }
 #endif

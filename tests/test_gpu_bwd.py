@@ -1,0 +1,113 @@
+"""GPU parity of the tile-recompute backward (dQ, dK, dV) against the CPU oracle, through the C ABI."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from flame_amd import workloads as W
+from tests.gpu_util import assert_close_bf16, to_dev, to_f32
+
+pytestmark = pytest.mark.gpu
+
+
+def _check_bwd(oracle, w, heads=None, tag=""):
+    from flame_amd import capi
+    print(f"[bwd] {w.name} {tag} shape={w.shape} causal={w.causal}", flush=True)
+    q, k, v, do = (to_dev(t) for t in (w.q, w.k, w.v, w.do))
+    kvl = None if w.kv_len is None else torch.from_numpy(w.kv_len).cuda()
+    mask = None if w.mask is None else torch.from_numpy(w.mask).cuda()
+    o, lse = capi.attn_fwd(q, k, v, w.scale, causal=w.causal, kv_len=kvl, mask=mask)
+    dq, dk, dv = capi.attn_bwd(q, k, v, o, do, lse, w.scale, causal=w.causal, kv_len=kvl, mask=mask)
+    torch.cuda.synchronize()
+    B, H, Sq, Sk, D = w.shape
+    # the oracle backward is fed the oracle's own bf16 O, not the kernel's
+    ro, _ = oracle.sdpa_fwd(w.q, w.k, w.v, w.scale, causal=w.causal, kv_len=w.kv_len, mask=w.mask, heads=heads)
+    ref = oracle.sdpa_bwd(w.q, w.k, w.v, ro, w.do, w.scale, causal=w.causal, kv_len=w.kv_len, mask=w.mask,
+                          heads=heads, want_f32=True)
+    hb, he = (0, B * H) if heads is None else heads
+    for i, (name, got, S) in enumerate((("dQ", dq, Sq), ("dK", dk, Sk), ("dV", dv, Sk))):
+        g = to_f32(got).reshape(B * H, S, D)[hb:he]
+        assert_close_bf16(oracle, name, g, ref[i].reshape(B * H, S, D)[hb:he], ref[i + 3].reshape(B * H, S, D)[hb:he])
+    return dq, dk, dv
+
+
+def test_cfg1_small_noncausal(oracle):
+    _check_bwd(oracle, W.config1())
+
+
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("Sq,Sk", [(1, 1), (37, 91), (64, 128), (129, 193), (300, 257)])
+def test_partial_tiles(oracle, D, Sq, Sk):
+    seed = 2000 + Sq * 7 + Sk
+    B, H = 2, 2
+    t = [W.f32_to_bf16_bits(W.normal_f32(seed, s, B * H * n * D).reshape(B, H, n, D))
+         for s, n in enumerate((Sq, Sk, Sk, Sq))]
+    _check_bwd(oracle, W.Workload(f"partial_{Sq}x{Sk}_d{D}", t[0], t[1], t[2], t[3], 1.0 / math.sqrt(D)))
+
+
+@pytest.mark.parametrize("D", [64, 128])
+def test_causal(oracle, D):
+    _check_bwd(oracle, W.config4(H=2, S=320, D=D))
+
+
+def test_causal_rectangular(oracle):
+    for Sq, Sk in ((100, 260), (260, 100)):
+        t = [W.f32_to_bf16_bits(W.normal_f32(15 + Sq, s, 2 * n * 64).reshape(1, 2, n, 64))
+             for s, n in enumerate((Sq, Sk, Sk, Sq))]
+        _check_bwd(oracle, W.Workload(f"causal_rect_{Sq}x{Sk}", t[0], t[1], t[2], t[3], 0.125, causal=True))
+
+
+def test_cfg3_ragged_key_lengths(oracle):
+    w = W.config3(H=2, Sq=192)
+    dq, dk, dv = _check_bwd(oracle, w)
+    # gradients of padded keys are exactly zero
+    for b, L in enumerate(w.kv_len):
+        assert torch.all(dk[b, :, int(L):] == 0) and torch.all(dv[b, :, int(L):] == 0)
+
+
+def test_general_keep_mask_and_fully_masked_rows(oracle):
+    B, H, Sq, Sk, D = 2, 2, 70, 150, 64
+    t = [W.f32_to_bf16_bits(W.normal_f32(87, s, B * H * n * D).reshape(B, H, n, D))
+         for s, n in enumerate((Sq, Sk, Sk, Sq))]
+    mask = (W.normal_f32(88, 0, B * H * Sq * Sk).reshape(B, H, Sq, Sk) > 0.3).astype(np.uint8)
+    mask[0, 1, 5, :] = 0
+    mask[:, :, :, 149] = 0          # a key nobody attends to: dK = dV = 0 there
+    w = W.Workload("general_mask", t[0], t[1], t[2], t[3], 0.2, mask=mask)
+    dq, dk, dv = _check_bwd(oracle, w)
+    assert torch.all(dq[0, 1, 5] == 0)
+    assert torch.all(dk[:, :, 149] == 0) and torch.all(dv[:, :, 149] == 0)
+
+
+def test_strided_views_match_contiguous(oracle):
+    from flame_amd import capi
+    w = W.config2(H=3, n_text=40, grid=12, D=128)
+    q, k, v, do = (to_dev(t) for t in (w.q, w.k, w.v, w.do))
+    o, lse = capi.attn_fwd(q, k, v, w.scale)
+    ref = capi.attn_bwd(q, k, v, o, do, lse, w.scale)
+
+    def bnhd(t):   # same values, memory laid out [B,N,H,D]
+        return t.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
+
+    grads = tuple(bnhd(torch.empty_like(t)) for t in (q, k, v))
+    got = capi.attn_bwd(bnhd(q), bnhd(k), bnhd(v), bnhd(o), bnhd(do), lse, w.scale, grads=grads)
+    for a, b_ in zip(got[1:], ref[1:]):
+        assert torch.equal(a, b_)            # dK, dV: no atomics, bit-identical
+    assert oracle.max_abs(to_f32(got[0]), to_f32(ref[0])) < 1e-2   # dQ: fp32 atomic order may differ
+    _check_bwd(oracle, w)
+
+
+def test_cfg2_production_shape_head_subset(oracle):
+    w = W.config2()
+    _check_bwd(oracle, w, heads=(0, 1), tag="head 0")
+    _check_bwd(oracle, w, heads=(23, 24), tag="head 23")
+
+
+def test_workspace_too_small_is_rejected():
+    from flame_amd import capi
+    q = torch.zeros(1, 1, 64, 64, dtype=torch.bfloat16, device="cuda")
+    o, lse = capi.attn_fwd(q, q, q, 0.125)
+    ws = torch.empty(capi.bwd_workspace_bytes(1, 1, 64, 64) - 1, dtype=torch.uint8, device="cuda")
+    with pytest.raises(capi.FlameAttnError) as e:
+        capi.attn_bwd(q, q, q, o, q, lse, 0.125, workspace=ws)
+    assert e.value.code == capi.ERR_INVALID
