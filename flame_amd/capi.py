@@ -108,3 +108,63 @@ def attn_bwd(q, k, v, o, do, lse, scale, causal=False, kv_len=None, mask=None, w
     if rc != 0:
         raise FlameAttnError("flame_attn_bwd_bf16", rc)
     return dq, dk, dv
+
+
+KERNEL_KINDS = ("fwd", "bwd_prep", "bwd_main", "bwd_dq_convert", "sage_kmean", "sage_quant", "sage_fwd", "reserved")
+
+
+class _KernelTimes(ctypes.Structure):
+    _fields_ = [("total_ms", ctypes.c_double * 8), ("launches", ctypes.c_int * 8)]
+
+
+def profiling_enable(on: bool) -> None:
+    """Bracket every kernel launch with HIP events on the launch stream (clears earlier samples)."""
+    rc = lib().flame_attn_profiling_enable(int(bool(on)))
+    if rc != 0:
+        raise FlameAttnError("flame_attn_profiling_enable", rc)
+
+
+def profiling_read() -> dict:
+    """{kernel: (total_ms, launches)} since the last read; waits for the recorded events."""
+    kt = _KernelTimes()
+    rc = lib().flame_attn_profiling_read(ctypes.byref(kt))
+    if rc != 0:
+        raise FlameAttnError("flame_attn_profiling_read", rc)
+    return {name: (kt.total_ms[i], kt.launches[i]) for i, name in enumerate(KERNEL_KINDS)}
+
+
+def sage_quant(q, k, smooth_k=True):
+    """Per-block int8 quantisation of Q (128 rows) and mean-smoothed K (64 rows).
+
+    Returns dict(qi8, ki8, sq, sk, kmean): int8 [B,H,S,D], fp32 [B,H,nblk], fp32 [B,H,D]."""
+    B, H, Sq, D = q.shape
+    Sk = k.shape[2]
+    dev = q.device
+    out = dict(
+        qi8=torch.empty((B, H, Sq, D), dtype=torch.int8, device=dev),
+        ki8=torch.empty((B, H, Sk, D), dtype=torch.int8, device=dev),
+        sq=torch.empty((B, H, -(-Sq // 128)), dtype=torch.float32, device=dev),
+        sk=torch.empty((B, H, -(-Sk // 64)), dtype=torch.float32, device=dev),
+        kmean=torch.empty((B, H, D), dtype=torch.float32, device=dev))
+    rc = lib().flame_sage_quant_qk_int8(
+        _ptr(q), _ptr(k), B, H, Sq, Sk, D, _i64x4(q.stride()), _i64x4(k.stride()),
+        ctypes.c_int64(0), ctypes.c_int64(0), int(bool(smooth_k)),
+        _ptr(out["qi8"]), _ptr(out["ki8"]), _ptr(out["sq"]), _ptr(out["sk"]), _ptr(out["kmean"]), _stream())
+    if rc != 0:
+        raise FlameAttnError("flame_sage_quant_qk_int8", rc)
+    return out
+
+
+def sage_fwd(qz, v, scale, causal=False, kv_len=None, want_lse=False, out=None):
+    """O (and LSE) from quantised operands `qz` (the dict returned by sage_quant) and bf16 V."""
+    B, H, Sq, D = qz["qi8"].shape
+    Sk = qz["ki8"].shape[2]
+    o = torch.empty((B, H, Sq, D), dtype=torch.bfloat16, device=v.device) if out is None else out
+    lse = torch.empty((B * H, Sq), dtype=torch.float32, device=v.device) if want_lse else None
+    rc = lib().flame_sage_attn_fwd_int8(
+        _ptr(qz["qi8"]), _ptr(qz["ki8"]), _ptr(qz["sq"]), _ptr(qz["sk"]), _ptr(v), _ptr(o), _ptr(lse),
+        B, H, Sq, Sk, D, ctypes.c_float(scale), _i64x4(v.stride()), _i64x4(o.stride()),
+        ctypes.c_int64(0), ctypes.c_int64(0), int(bool(causal)), _ptr(kv_len), _stream())
+    if rc != 0:
+        raise FlameAttnError("flame_sage_attn_fwd_int8", rc)
+    return (o, lse) if want_lse else o

@@ -7,8 +7,12 @@
 #include <math.h>
 #include <stdio.h>
 
+#include <mutex>
+#include <vector>
+
 #include "attn_bwd.hpp"
 #include "attn_fwd.hpp"
+#include "sage.hpp"
 
 using namespace fattn;
 
@@ -28,6 +32,47 @@ int check_view(const void* base, const int64_t* st, int64_t off) {
 
 Strides mk(const int64_t* st) { return Strides{st[0], st[1], st[2]}; }
 
+// Optional per-kernel timing with HIP events on the caller's stream (off by default; when off the
+// launch path touches none of this).  Event pairs are created on demand and summed on read.
+struct Profiler {
+    static constexpr int kKinds = FLAME_ATTN_N_KERNEL_KINDS;
+    static constexpr size_t kMaxPairs = 8192;
+    std::mutex mu;
+    bool enabled = false;
+    std::vector<hipEvent_t> start[kKinds], stop[kKinds];
+    size_t used[kKinds] = {};
+
+    hipEvent_t begin(int kind, hipStream_t s, size_t* slot) {
+        std::lock_guard<std::mutex> g(mu);
+        if (!enabled || used[kind] >= kMaxPairs) return nullptr;
+        if (used[kind] == start[kind].size()) {
+            hipEvent_t a, b;
+            if (hipEventCreate(&a) != hipSuccess) return nullptr;
+            if (hipEventCreate(&b) != hipSuccess) { (void)hipEventDestroy(a); return nullptr; }
+            start[kind].push_back(a);
+            stop[kind].push_back(b);
+        }
+        *slot = used[kind]++;
+        (void)hipEventRecord(start[kind][*slot], s);
+        return stop[kind][*slot];
+    }
+};
+Profiler g_prof;
+
+struct ScopedKernelTimer {
+    hipEvent_t stop_ev = nullptr;
+    hipStream_t s;
+    ScopedKernelTimer(int kind, hipStream_t stream) : s(stream) {
+        if (g_prof.enabled) {
+            size_t slot;
+            stop_ev = g_prof.begin(kind, stream, &slot);
+        }
+    }
+    ~ScopedKernelTimer() {
+        if (stop_ev) (void)hipEventRecord(stop_ev, s);
+    }
+};
+
 template <int D, int NWQ>
 int launch_fwd(const FwdParams& p, hipStream_t s) {
     using T = FwdTile<D>;
@@ -43,7 +88,10 @@ int launch_fwd(const FwdParams& p, hipStream_t s) {
     const int64_t n_qt = (p.Sq + BM - 1) / BM;
     const int64_t grid = n_qt * p.B * p.H;
     if (grid > 0x7fffffff) return FLAME_ATTN_ERR_UNSUPPORTED;
-    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), T::LDS_BYTES, s, p);
+    {
+        ScopedKernelTimer t(FLAME_ATTN_KERNEL_FWD, s);
+        hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), T::LDS_BYTES, s, p);
+    }
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? FLAME_ATTN_OK : (int)e;
 }
@@ -67,9 +115,18 @@ int launch_bwd(const BwdParams& p, hipStream_t s) {
     const int64_t n_kt = (p.Sk + T::BN - 1) / T::BN;
     const int64_t grid = n_kt * p.B * p.H;
     if (row_blocks > 0x7fffffff || grid > 0x7fffffff) return FLAME_ATTN_ERR_UNSUPPORTED;
-    hipLaunchKernelGGL(bwd_prep_kernel<D>, dim3((unsigned)row_blocks), dim3(256), 0, s, p);
-    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), T::LDS_BYTES, s, p);
-    hipLaunchKernelGGL(bwd_dq_convert_kernel<D>, dim3((unsigned)row_blocks), dim3(256), 0, s, p);
+    {
+        ScopedKernelTimer t(FLAME_ATTN_KERNEL_BWD_PREP, s);
+        hipLaunchKernelGGL(bwd_prep_kernel<D>, dim3((unsigned)row_blocks), dim3(256), 0, s, p);
+    }
+    {
+        ScopedKernelTimer t(FLAME_ATTN_KERNEL_BWD_MAIN, s);
+        hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), T::LDS_BYTES, s, p);
+    }
+    {
+        ScopedKernelTimer t(FLAME_ATTN_KERNEL_BWD_DQ_CONVERT, s);
+        hipLaunchKernelGGL(bwd_dq_convert_kernel<D>, dim3((unsigned)row_blocks), dim3(256), 0, s, p);
+    }
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? FLAME_ATTN_OK : (int)e;
 }
@@ -77,6 +134,33 @@ int launch_bwd(const BwdParams& p, hipStream_t s) {
 }  // namespace
 
 extern "C" {
+
+int flame_attn_profiling_enable(int on) {
+    std::lock_guard<std::mutex> g(g_prof.mu);
+    g_prof.enabled = on != 0;
+    for (int k = 0; k < Profiler::kKinds; ++k) g_prof.used[k] = 0;
+    return FLAME_ATTN_OK;
+}
+
+int flame_attn_profiling_read(FlameAttnKernelTimes* out) {
+    if (!out) return FLAME_ATTN_ERR_INVALID;
+    std::lock_guard<std::mutex> g(g_prof.mu);
+    for (int k = 0; k < Profiler::kKinds; ++k) {
+        double total = 0.0;
+        for (size_t i = 0; i < g_prof.used[k]; ++i) {
+            hipError_t e = hipEventSynchronize(g_prof.stop[k][i]);
+            if (e != hipSuccess) return (int)e;
+            float ms = 0.f;
+            e = hipEventElapsedTime(&ms, g_prof.start[k][i], g_prof.stop[k][i]);
+            if (e != hipSuccess) return (int)e;
+            total += ms;
+        }
+        out->total_ms[k] = total;
+        out->launches[k] = (int)g_prof.used[k];
+        g_prof.used[k] = 0;
+    }
+    return FLAME_ATTN_OK;
+}
 
 size_t flame_attn_bwd_workspace_bytes(int B, int H, int N_q, int D) {
     if (B <= 0 || H <= 0 || N_q <= 0 || D <= 0) return 0;
@@ -139,6 +223,101 @@ int flame_attn_bwd_bf16(const void* Q, const void* K, const void* V, const void*
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (D == 128) return launch_bwd<128>(p, s);
     return launch_bwd<64>(p, s);
+}
+
+int flame_sage_quant_qk_int8(const void* Q, const void* K, int B, int H, int N_q, int N_kv, int D,
+                             const int64_t* q_strides, const int64_t* k_strides, int64_t q_off, int64_t k_off,
+                             int smooth_k, void* Qi8, void* Ki8, void* q_scales, void* k_scales, void* k_mean,
+                             void* stream) {
+    if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0) return FLAME_ATTN_ERR_INVALID;
+    if (!Qi8 || !Ki8 || !q_scales || !k_scales || !k_mean) return FLAME_ATTN_ERR_INVALID;
+    if (D != 64 && D != 128) return FLAME_ATTN_ERR_UNSUPPORTED;
+    int rc;
+    if ((rc = check_view(Q, q_strides, q_off))) return rc;
+    if ((rc = check_view(K, k_strides, k_off))) return rc;
+    if (!aligned16(Qi8) || !aligned16(Ki8) || !aligned16(k_mean)) return FLAME_ATTN_ERR_UNSUPPORTED;
+    SageQuantParams p;
+    p.q = static_cast<const uint16_t*>(Q) + q_off;
+    p.k = static_cast<const uint16_t*>(K) + k_off;
+    p.qs = mk(q_strides); p.ks = mk(k_strides);
+    p.B = B; p.H = H; p.Sq = N_q; p.Sk = N_kv;
+    p.smooth_k = smooth_k ? 1 : 0;
+    p.kmean = static_cast<float*>(k_mean);
+    p.qi8 = static_cast<int8_t*>(Qi8);
+    p.ki8 = static_cast<int8_t*>(Ki8);
+    p.sq = static_cast<float*>(q_scales);
+    p.sk = static_cast<float*>(k_scales);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int64_t bh = (int64_t)B * H;
+    const int64_t nblk = (N_q + kSageQBlk - 1) / kSageQBlk + (N_kv + kSageKBlk - 1) / kSageKBlk;
+    if (bh * nblk > 0x7fffffff) return FLAME_ATTN_ERR_UNSUPPORTED;
+    {
+        ScopedKernelTimer t(FLAME_ATTN_KERNEL_SAGE_KMEAN, s);
+        if (D == 128) hipLaunchKernelGGL(sage_kmean_kernel<128>, dim3((unsigned)bh), dim3(512), 0, s, p);
+        else hipLaunchKernelGGL(sage_kmean_kernel<64>, dim3((unsigned)bh), dim3(512), 0, s, p);
+    }
+    {
+        ScopedKernelTimer t(FLAME_ATTN_KERNEL_SAGE_QUANT, s);
+        if (D == 128) hipLaunchKernelGGL(sage_quant_kernel<128>, dim3((unsigned)(bh * nblk)), dim3(256), 0, s, p);
+        else hipLaunchKernelGGL(sage_quant_kernel<64>, dim3((unsigned)(bh * nblk)), dim3(256), 0, s, p);
+    }
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? FLAME_ATTN_OK : (int)e;
+}
+
+}  // extern "C"
+
+template <int D>
+static int launch_sage_fwd(const SageFwdParams& p, hipStream_t s) {
+    using T = SageTile<D>;
+    static bool attr_done = false;
+    auto kern = sage_fwd_kernel<D>;
+    if (!attr_done) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS_BYTES);
+        if (e != hipSuccess) return (int)e;
+        attr_done = true;
+    }
+    const int64_t grid = (int64_t)((p.Sq + T::BM - 1) / T::BM) * p.B * p.H;
+    if (grid > 0x7fffffff) return FLAME_ATTN_ERR_UNSUPPORTED;
+    {
+        ScopedKernelTimer t(FLAME_ATTN_KERNEL_SAGE_FWD, s);
+        hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), T::LDS_BYTES, s, p);
+    }
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? FLAME_ATTN_OK : (int)e;
+}
+
+extern "C" {
+
+int flame_sage_attn_fwd_int8(const void* Qi8, const void* Ki8, const void* q_scales, const void* k_scales,
+                             const void* V, void* O, void* LSE, int B, int H, int N_q, int N_kv, int D,
+                             float scale, const int64_t* v_strides, const int64_t* o_strides,
+                             int64_t v_off, int64_t o_off, int causal, const int32_t* kv_len, void* stream) {
+    if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0) return FLAME_ATTN_ERR_INVALID;
+    if (!(scale > 0.f) || !isfinite(scale)) return FLAME_ATTN_ERR_INVALID;
+    if (!Qi8 || !Ki8 || !q_scales || !k_scales) return FLAME_ATTN_ERR_INVALID;
+    if (D != 64 && D != 128) return FLAME_ATTN_ERR_UNSUPPORTED;
+    if (!aligned16(Qi8) || !aligned16(Ki8)) return FLAME_ATTN_ERR_UNSUPPORTED;
+    int rc;
+    if ((rc = check_view(V, v_strides, v_off))) return rc;
+    if ((rc = check_view(O, o_strides, o_off))) return rc;
+    SageFwdParams p;
+    p.qi8 = static_cast<const int8_t*>(Qi8);
+    p.ki8 = static_cast<const int8_t*>(Ki8);
+    p.sq = static_cast<const float*>(q_scales);
+    p.sk = static_cast<const float*>(k_scales);
+    p.v = static_cast<const uint16_t*>(V) + v_off;
+    p.o = static_cast<uint16_t*>(O) + o_off;
+    p.lse = static_cast<float*>(LSE);
+    p.vs = mk(v_strides); p.os = mk(o_strides);
+    p.B = B; p.H = H; p.Sq = N_q; p.Sk = N_kv;
+    p.scale = scale;
+    p.kv_len = kv_len;
+    p.causal = causal ? 1 : 0;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (D == 128) return launch_sage_fwd<128>(p, s);
+    return launch_sage_fwd<64>(p, s);
 }
 
 int flame_attn_fwd_bf16(const void* Q, const void* K, const void* V, void* O, void* LSE,
