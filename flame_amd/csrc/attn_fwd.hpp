@@ -2,12 +2,14 @@
 // per-row log-sum-exp of the scaled logits; the Sq x Sk score matrix never leaves registers.
 //
 // One workgroup = 4 wavefronts = 128*NWQ query rows of one (batch, head); each wavefront owns
-// 32*NWQ rows whose Q fragments stay in registers.  K/V tiles of 64 keys are staged through LDS
-// (double buffered, register prefetch), both row-major.  The logits are produced transposed, S^T = K Q^T, so that
+// 32*NWQ rows whose Q fragments stay in registers.  K/V tiles of 64 keys are copied global -> LDS
+// by the asynchronous LDS-DMA loads (no staging registers), double buffered, row-major with an XOR
+// swizzle of the 16-byte granules so that both the row reads of K and the transposing reads of V are
+// free of bank conflicts without padding.  The logits are produced transposed, S^T = K Q^T, so that
 // every lane holds values of a single query: row max / row sum are in-lane reductions plus one
 // exchange between the wave halves, the bf16 P^T values are already in the B-operand layout of the
-// second MFMA (O^T = V^T P^T), and the running rescale of O is a per-lane scalar.  The V^T operand
-// of that MFMA is gathered from the row-major V tile with the transposing LDS read.
+// second MFMA (O^T = V^T P^T), and the running rescale of O is a per-lane scalar that is skipped
+// while the running maximum stays within 2^8 of the reference maximum in use.
 #pragma once
 #include "attn_common.hpp"
 
@@ -25,27 +27,44 @@ struct FwdParams {
     MaskArgs m;
 };
 
+// 16-byte-granule XOR swizzle of a row-major bf16 tile whose rows are D*2 bytes (no padding).
+// 16 consecutive rows get distinct bank groups for the same logical granule, and 4 consecutive rows
+// land in 4 disjoint 64-byte bank groups: both access patterns used by the kernels (16-byte row
+// reads, transposing 8-byte reads of a 4-row x 64-byte block) are conflict-free on the 64-bank LDS.
+template <int D>
+__device__ __forceinline__ constexpr int swz(int row) {
+    return D == 128 ? (((row & 3) << 2) | ((row >> 2) & 3)) : ((((row >> 1) & 1) << 2) | ((row >> 2) & 3));
+}
+
 template <int D>
 struct FwdTile {
-    static constexpr int BN = 64;            // keys per tile
-    static constexpr int KS = D + 8;         // LDS row stride of the K tile, elements
-    static constexpr int VS = D + 8;         // LDS row stride of the V tile, elements
-    static constexpr int K_ELEMS = BN * KS;
-    static constexpr int V_ELEMS = BN * VS;
-    static constexpr int STAGE_ELEMS = K_ELEMS + V_ELEMS;
+    static constexpr int BN = 64;                   // keys per tile
+    static constexpr int RS = D;                    // LDS row stride, elements
+    static constexpr int TILE_ELEMS = BN * D;       // one K or V tile
+    static constexpr int STAGE_ELEMS = 2 * TILE_ELEMS;
     static constexpr int LDS_BYTES = 2 * STAGE_ELEMS * 2;
-    static constexpr int NKC = BN * (D / 8) / 256;   // 16-byte chunks per thread and tensor
+    static constexpr int ROWS_PER_DMA = 1024 / (D * 2);          // rows covered by one 64-lane x 16-byte copy
+    static constexpr int DMA_PER_WAVE = BN / ROWS_PER_DMA / 4;   // copies per wave and tensor
 };
 
-template <int D, int NWQ>
+// One wave-wide asynchronous copy of 1 KiB global -> LDS: lane l delivers 16 bytes to lds_dst + 16*l.
+__device__ __forceinline__ void dma16(const uint16_t* gsrc, uint16_t* lds_dst_wave_uniform) {
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gsrc,
+                                     (__attribute__((address_space(3))) void*)lds_dst_wave_uniform, 16, 0, 0);
+}
+
+__device__ __forceinline__ void wait_vm0() { __builtin_amdgcn_s_waitcnt(0x0F70); }   // vmcnt(0) only
+
+template <int D, int NWQ, bool HASMASK>
 __global__ __launch_bounds__(256) void fwd_kernel(const FwdParams p) {
     using T = FwdTile<D>;
-    constexpr int BN = T::BN, KS = T::KS, VS = T::VS;
+    constexpr int BN = T::BN, RS = T::RS;
     constexpr int BM = 128 * NWQ;
     constexpr int DC = D / 16;   // contraction chunks of QK^T
     constexpr int DB = D / 32;   // 32-row blocks of O^T
+    constexpr int GPR = D / 8;   // 16-byte granules per row
 
-    extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
+    extern __shared__ __attribute__((aligned(1024))) uint16_t lds[];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -68,7 +87,7 @@ __global__ __launch_bounds__(256) void fwd_kernel(const FwdParams p) {
     int kend = klimit;
     if (p.m.causal) kend = min(kend, q0 + BM);
     const int n_tiles = (kend + BN - 1) / BN;
-    const uint8_t* mbase = p.m.mask ? p.m.mask + b * p.m.sb + hh * p.m.sh : nullptr;
+    const uint8_t* mbase = HASMASK ? p.m.mask + b * p.m.sb + hh * p.m.sh : nullptr;
 
     // ---- Q fragments (B operand of S^T = K Q^T): column = query, 8 consecutive d
     bf16x8 qf[NWQ][DC];
@@ -81,35 +100,40 @@ __global__ __launch_bounds__(256) void fwd_kernel(const FwdParams p) {
         for (int dc = 0; dc < DC; ++dc) qf[qb][dc] = __builtin_bit_cast(bf16x8, ldg16(rp + 16 * dc, ok));
     }
 
-    // ---- staging assignment
-    u32x4 kreg[T::NKC];
-    u32x4 vreg[T::NKC];
+    // ---- asynchronous tile copies: this lane's source offsets (rows clamped into the attended range)
+    const int dma_row_in = lane / GPR;                       // row inside one 1 KiB copy
+    const int dma_gran = lane % GPR;                         // physical granule written by this lane
+    auto issue_tile = [&](int t, int buf) {
+        uint16_t* kdst = lds + buf * T::STAGE_ELEMS;
+        uint16_t* vdst = kdst + T::TILE_ELEMS;
+#pragma unroll
+        for (int i = 0; i < T::DMA_PER_WAVE; ++i) {
+            const int ji = wave * T::DMA_PER_WAVE + i;
+            const int row = ji * T::ROWS_PER_DMA + dma_row_in;
+            const int key = min(t * BN + row, klimit - 1);   // tail rows re-read the last attended key
+            const int c = dma_gran ^ swz<D>(row);
+            dma16(kbase + (int64_t)key * p.ks.n + c * 8, kdst + ji * 512);
+            dma16(vbase + (int64_t)key * p.vs.n + c * 8, vdst + ji * 512);
+        }
+    };
 
-    auto load_tile = [&](int t) {
-        const int key0 = t * BN;
+    // ---- per-lane LDS read offsets (elements), constant over the key loop
+    int koff[DC];          // K fragment: row 32*kb + n, logical granule 2*dc + h
 #pragma unroll
-        for (int i = 0; i < T::NKC; ++i) {
-            const int c = tid + 256 * i;
-            const int row = c / (D / 8), col = c % (D / 8);
-            const int key = key0 + row;
-            kreg[i] = ldg16(kbase + (int64_t)key * p.ks.n + col * 8, key < p.Sk);
-            vreg[i] = ldg16(vbase + (int64_t)key * p.vs.n + col * 8, key < klimit);
-        }
-    };
-    auto store_tile = [&](int buf) {
-        uint16_t* ks = lds + buf * T::STAGE_ELEMS;
-        uint16_t* vs = ks + T::K_ELEMS;
+    for (int dc = 0; dc < DC; ++dc) koff[dc] = n * RS + (((2 * dc + h) ^ swz<D>(n)) << 3);
+    const int tr_r = lane & 15, tr_g16 = (lane >> 4) & 1;
+    int voff[2][DB];       // V^T fragment halves: rows 4h + r/4 (+8), logical granule 4*db + 2*g16 + (r&3)/2
 #pragma unroll
-        for (int i = 0; i < T::NKC; ++i) {
-            const int c = tid + 256 * i;
-            const int row = c / (D / 8), col = c % (D / 8);
-            *reinterpret_cast<u32x4*>(ks + row * KS + col * 8) = kreg[i];
-            *reinterpret_cast<u32x4*>(vs + row * VS + col * 8) = vreg[i];
-        }
-    };
+    for (int half = 0; half < 2; ++half) {
+        const int row = 4 * h + (tr_r >> 2) + 8 * half;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+            voff[half][db] = row * RS + (((4 * db + 2 * tr_g16 + ((tr_r & 3) >> 1)) ^ swz<D>(row)) << 3) + 4 * (tr_r & 1);
+    }
 
     // ---- running state; each lane serves query column n of every block qb
     const float c_log2 = p.scale * kLog2e;
+    const float stale_ok = 8.0f / c_log2;     // the reference maximum may lag the true one by 2^8
     float m_run[NWQ], l_run[NWQ];
     f32x16 oacc[NWQ][DB];
 #pragma unroll
@@ -122,19 +146,16 @@ __global__ __launch_bounds__(256) void fwd_kernel(const FwdParams p) {
             for (int r = 0; r < 16; ++r) oacc[qb][db][r] = 0.f;
     }
 
-    if (n_tiles > 0) {
-        load_tile(0);
-        store_tile(0);
-    }
+    if (n_tiles > 0) issue_tile(0, 0);
+    wait_vm0();
     __syncthreads();
 
     for (int t = 0; t < n_tiles; ++t) {
         const int buf = t & 1;
-        const bool more = (t + 1) < n_tiles;
-        if (more) load_tile(t + 1);
+        if (t + 1 < n_tiles) issue_tile(t + 1, buf ^ 1);
 
         const uint16_t* ks = lds + buf * T::STAGE_ELEMS;
-        const uint16_t* vs = ks + T::K_ELEMS;
+        const uint16_t* vs = ks + T::TILE_ELEMS;
         const int key0 = t * BN;
 
         // ---- S^T = K Q^T : rows = keys (two blocks of 32), columns = queries
@@ -149,7 +170,7 @@ __global__ __launch_bounds__(256) void fwd_kernel(const FwdParams p) {
         for (int dc = 0; dc < DC; ++dc) {
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb) {
-                const bf16x8 ka = *reinterpret_cast<const bf16x8*>(ks + (32 * kb + n) * KS + 16 * dc + 8 * h);
+                const bf16x8 ka = *reinterpret_cast<const bf16x8*>(ks + koff[dc] + 32 * kb * RS);
 #pragma unroll
                 for (int qb = 0; qb < NWQ; ++qb) sacc[qb][kb] = mfma32(ka, qf[qb][dc], sacc[qb][kb]);
             }
@@ -158,7 +179,7 @@ __global__ __launch_bounds__(256) void fwd_kernel(const FwdParams p) {
         // ---- exclusions: ragged tail / key length, causal, explicit keep-mask
         const bool tail = key0 + BN > klimit;
         const bool diag = p.m.causal && (key0 + BN - 1 > qw0);
-        if (tail || diag || mbase) {
+        if (tail || diag || HASMASK) {
 #pragma unroll
             for (int qb = 0; qb < NWQ; ++qb) {
                 const int qi = qw0 + 32 * qb + n;
@@ -169,8 +190,9 @@ __global__ __launch_bounds__(256) void fwd_kernel(const FwdParams p) {
                         const int key = key0 + 32 * kb + acc_row(r, h);
                         bool drop = key >= klimit;
                         if (p.m.causal) drop = drop || key > qi;
-                        if (mbase && !drop && qi < p.Sq)
-                            drop = mbase[(int64_t)qi * p.m.sq + (int64_t)key * p.m.sk] == 0;
+                        if (HASMASK) {
+                            if (!drop && qi < p.Sq) drop = mbase[(int64_t)qi * p.m.sq + (int64_t)key * p.m.sk] == 0;
+                        }
                         if (drop) sacc[qb][kb][r] = -INFINITY;
                     }
             }
@@ -186,10 +208,21 @@ __global__ __launch_bounds__(256) void fwd_kernel(const FwdParams p) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, sacc[qb][kb][r]);
             tmax = fmaxf(tmax, xhalf(tmax));
-            const float m_new = fmaxf(m_run[qb], tmax);
-            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-            const float alpha = exp2_fast((m_run[qb] - m_use) * c_log2);
-            m_run[qb] = m_new;
+            // move the reference maximum (and rescale the running sums) only when some lane's tile
+            // maximum exceeds it by more than 2^8 in the exponent domain; wave-uniform branch
+            if (__any(tmax > m_run[qb] + stale_ok)) {
+                const float m_old = m_run[qb];
+                const float m_new = fmaxf(m_old, tmax);
+                const float m_to = (m_new == -INFINITY) ? 0.f : m_new;
+                const float alpha = exp2_fast((m_old - m_to) * c_log2);
+                m_run[qb] = m_new;
+                l_run[qb] *= alpha;
+#pragma unroll
+                for (int db = 0; db < DB; ++db)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) oacc[qb][db][r] *= alpha;
+            }
+            const float m_use = (m_run[qb] == -INFINITY) ? 0.f : m_run[qb];
             const float msc = m_use * c_log2;
             float rsum = 0.f;
 #pragma unroll
@@ -200,11 +233,7 @@ __global__ __launch_bounds__(256) void fwd_kernel(const FwdParams p) {
                     sacc[qb][kb][r] = e;
                     rsum += e;
                 }
-            l_run[qb] = l_run[qb] * alpha + rsum;
-#pragma unroll
-            for (int db = 0; db < DB; ++db)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) oacc[qb][db][r] *= alpha;
+            l_run[qb] += rsum;
 #pragma unroll
             for (int cc = 0; cc < 4; ++cc) {
                 const int kb = cc >> 1, o8 = 8 * (cc & 1);
@@ -219,14 +248,17 @@ __global__ __launch_bounds__(256) void fwd_kernel(const FwdParams p) {
         for (int cc = 0; cc < 4; ++cc) {
 #pragma unroll
             for (int db = 0; db < DB; ++db) {
-                const bf16x8 va = lds_tr_frag(vs, VS, 16 * cc, 32 * db, lane);
+                const u32x2 lo = lds_read_tr16(vs + voff[0][db] + 16 * cc * RS);
+                const u32x2 hi = lds_read_tr16(vs + voff[1][db] + 16 * cc * RS);
+                const u32x4 u = {lo[0], lo[1], hi[0], hi[1]};
+                const bf16x8 va = __builtin_bit_cast(bf16x8, u);
 #pragma unroll
                 for (int qb = 0; qb < NWQ; ++qb) oacc[qb][db] = mfma32(va, pf[qb][cc], oacc[qb][db]);
             }
         }
 
-        if (more) store_tile(buf ^ 1);
-        __syncthreads();
+        wait_vm0();          // next tile has landed in the other buffer
+        __syncthreads();     // ... for every wave, and everyone is done reading this one
     }
 
     // ---- epilogue

@@ -173,7 +173,7 @@ template <int D>
 struct SageTile {
     static constexpr int BM = 128, BN = 64;
     static constexpr int KSB = D + 16;            // bytes per row of the int8 K tile
-    static constexpr int VS = D + 8;              // elements per row of the bf16 V tile
+    static constexpr int VS = D + 32;             // elements per row of the bf16 V tile (transposing reads)
     static constexpr int K_BYTES = BN * KSB;
     static constexpr int V_BYTES = BN * VS * 2;
     static constexpr int STAGE_BYTES = K_BYTES + V_BYTES;
