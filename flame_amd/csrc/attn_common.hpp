@@ -34,6 +34,27 @@ __device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
 }
 
+// acc *= alpha for an accumulator that lives in the accumulation register file, done with explicit
+// reads/writes of that file so that the (rare) rescale does not pull the accumulator into the
+// architectural registers for the whole loop.  The leading no-ops cover the MFMA-write -> accvgpr-read
+// wait states that the assembler-level hazard recogniser cannot see inside an asm block.
+__device__ __forceinline__ void scale_acc_agpr(f32x16& acc, float alpha) {
+    float t0, t1, t2, t3;
+    asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 3" ::: "memory");
+#define FATTN_SCALE4(i)                                                                                   \
+    asm volatile("v_accvgpr_read_b32 %1, %0\n\t"                                                          \
+                 "v_mul_f32 %1, %1, %2\n\t"                                                               \
+                 "s_nop 1\n\t"                                                                            \
+                 "v_accvgpr_write_b32 %0, %1"                                                              \
+                 : "+a"(acc[i]), "=&v"(t0)                                                                 \
+                 : "v"(alpha));
+    FATTN_SCALE4(0) FATTN_SCALE4(1) FATTN_SCALE4(2) FATTN_SCALE4(3) FATTN_SCALE4(4) FATTN_SCALE4(5)
+    FATTN_SCALE4(6) FATTN_SCALE4(7) FATTN_SCALE4(8) FATTN_SCALE4(9) FATTN_SCALE4(10) FATTN_SCALE4(11)
+    FATTN_SCALE4(12) FATTN_SCALE4(13) FATTN_SCALE4(14) FATTN_SCALE4(15)
+#undef FATTN_SCALE4
+    (void)t1; (void)t2; (void)t3;
+}
+
 // row index inside a 32x32 accumulator block for register r of a lane in half h
 __device__ __forceinline__ constexpr int acc_row(int r, int h) { return 8 * (r >> 2) + 4 * h + (r & 3); }
 

@@ -56,7 +56,7 @@ __device__ __forceinline__ void dma16(const uint16_t* gsrc, uint16_t* lds_dst_wa
 __device__ __forceinline__ void wait_vm0() { __builtin_amdgcn_s_waitcnt(0x0F70); }   // vmcnt(0) only
 
 template <int D, int NWQ, bool HASMASK>
-__global__ __launch_bounds__(256) void fwd_kernel(const FwdParams p) {
+__global__ __launch_bounds__(256, (NWQ == 1 ? 2 : 1)) void fwd_kernel(const FwdParams p) {
     using T = FwdTile<D>;
     constexpr int BN = T::BN, RS = T::RS;
     constexpr int BM = 128 * NWQ;
@@ -217,10 +217,15 @@ __global__ __launch_bounds__(256) void fwd_kernel(const FwdParams p) {
                 const float alpha = exp2_fast((m_old - m_to) * c_log2);
                 m_run[qb] = m_new;
                 l_run[qb] *= alpha;
+                if constexpr (NWQ > 1) {
 #pragma unroll
-                for (int db = 0; db < DB; ++db)
+                    for (int db = 0; db < DB; ++db) scale_acc_agpr(oacc[qb][db], alpha);
+                } else {
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) oacc[qb][db][r] *= alpha;
+                    for (int db = 0; db < DB; ++db)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) oacc[qb][db][r] *= alpha;
+                }
             }
             const float m_use = (m_run[qb] == -INFINITY) ? 0.f : m_run[qb];
             const float msc = m_use * c_log2;
