@@ -1,7 +1,7 @@
 // Backward of the tiled attention for gfx950: recomputes P tile by tile from Q, K and the saved
 // log-sum-exp, never materialising the Sq x Sk matrix.
 //
-//   prep     delta_i = sum_d dO_id * O_id   (fp32), and clears the fp32 dQ accumulator
+//   prep     delta_i = sum_d dO_id * O_id   (fp32), LSE_i * log2(e), and clears the fp32 dQ accumulator
 //   main     one workgroup owns 128 keys (32 per wavefront) of one (batch, head) and walks over the
 //            query tiles (64 rows): S = Q K^T, dP = dO V^T, P = exp2(S*c - LSE*log2e),
 //            dS = P * (dP - delta); dV^T += dO^T P and dK^T += Q^T dS stay in registers for the
@@ -10,8 +10,10 @@
 //            dQ += dS K, which is added to an fp32 accumulator in HBM with hardware atomics
 //   convert  dQ = bf16(scale * accumulator)
 //
-// Q and dO tiles are staged row-major; their transposed MFMA operands (Q^T, dO^T) and the dS
-// operand come from transposing LDS reads, so no tile is stored twice.
+// Q and dO tiles are copied global -> LDS by asynchronous LDS-DMA loads, double buffered, row-major
+// with an XOR swizzle of the 16-byte granules; their transposed MFMA operands (Q^T, dO^T) and the dS
+// operand come from transposing LDS reads, so no tile is stored twice and no access pattern has
+// bank conflicts.  One workgroup barrier per step.
 #pragma once
 #include "attn_common.hpp"
 
@@ -28,6 +30,7 @@ struct BwdParams {
     uint16_t* dk;
     uint16_t* dv;
     float* delta;         // workspace, [B*H, Sq]
+    float* lse2;          // workspace, [B*H, Sq]: LSE * log2(e), +inf where LSE = -inf
     float* dq_acc;        // workspace, [B*H, Sq, D] fp32
     Strides qs, ks, vs, os, dos, dqs, dks, dvs;
     int B, H, Sq, Sk;
@@ -61,7 +64,11 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(const BwdParams p) {
     }
 #pragma unroll
     for (int off = TPR / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
-    if (ok && chunk == 0) p.delta[row_flat] = acc;
+    if (ok && chunk == 0) {
+        p.delta[row_flat] = acc;
+        const float l = p.lse[row_flat];
+        p.lse2[row_flat] = (l == -INFINITY) ? INFINITY : l * kLog2e;   // exp2(s*c - inf) = 0 for excluded rows
+    }
 }
 
 // --------------------------------------------------------------------------------------- convert
@@ -87,31 +94,34 @@ __global__ __launch_bounds__(256) void bwd_dq_convert_kernel(const BwdParams p) 
 // ------------------------------------------------------------------------------------------ main
 template <int D>
 struct BwdTile {
-    static constexpr int BM = 64;              // query rows per step
-    static constexpr int BN = 128;             // keys per workgroup
-    static constexpr int QS = D + 8;           // LDS row stride of the Q / dO / K / V tiles
-    static constexpr int DSS = BM + 8;         // LDS row stride of dS^T [key][query]
-    static constexpr int Q_ELEMS = BM * QS;
+    static constexpr int BM = 64;                   // query rows per step
+    static constexpr int BN = 128;                  // keys per workgroup
+    static constexpr int RS = D;                    // LDS row stride of the Q / dO / K / V tiles (swizzled, unpadded)
+    static constexpr int DSS = BM;                  // LDS row stride of dS^T [key][query] (swizzled, unpadded)
+    static constexpr int Q_ELEMS = BM * RS;
+    static constexpr int STAGE_ELEMS = 2 * Q_ELEMS;               // Q tile + dO tile
     static constexpr int DS_ELEMS = BN * DSS;
-    static constexpr int LDS_BYTES = (2 * Q_ELEMS + DS_ELEMS) * 2 + 2 * BM * 4;
-    static constexpr int NC = BM * (D / 8) / 256;    // 16-byte chunks per thread per 64-row tile
+    static constexpr int ROW_FLOATS = 2 * BM;                     // lse2 + delta of one step
+    // [2 stages of Q,dO][2 dS^T buffers][2 x (lse2, delta)]
+    static constexpr int LDS_BYTES = (2 * STAGE_ELEMS + 2 * DS_ELEMS) * 2 + 2 * ROW_FLOATS * 4;
+    static constexpr int ROWS_PER_DMA = 1024 / (D * 2);
+    static constexpr int DMA_PER_WAVE = BM / ROWS_PER_DMA / 4;    // 1 KiB copies per wave and tensor
 };
 
-template <int D>
+template <int D, bool HASMASK>
 __global__ __launch_bounds__(256) void bwd_kernel(const BwdParams p) {
     using T = BwdTile<D>;
-    constexpr int BM = T::BM, BN = T::BN, QS = T::QS, DSS = T::DSS, NC = T::NC;
+    constexpr int BM = T::BM, BN = T::BN, RS = T::RS, DSS = T::DSS;
     constexpr int DC = D / 16;     // contraction chunks over the head dim
     constexpr int DB = D / 32;     // 32-row blocks of dK^T / dV^T
     constexpr int NSL = D / 32;    // 32-column slices of dQ
     constexpr int QB_PER = 2 / (4 / NSL);   // query blocks per wave in the dQ step
+    constexpr int GPR = D / 8;     // 16-byte granules per row
 
-    extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
-    uint16_t* Qs = lds;                       // [BM][QS]
-    uint16_t* dOs = lds + T::Q_ELEMS;         // [BM][QS]   (Qs and dOs together also hold a [BN][QS] tile in the prologue)
-    uint16_t* dSt = lds + 2 * T::Q_ELEMS;     // [BN][DSS]
-    float* lse_s = reinterpret_cast<float*>(lds + 2 * T::Q_ELEMS + T::DS_ELEMS);   // [BM], pre-multiplied by log2(e)
-    float* delta_s = lse_s + BM;
+    extern __shared__ __attribute__((aligned(1024))) uint16_t lds[];
+    uint16_t* stage0 = lds;                                        // [2][Q tile | dO tile]
+    uint16_t* dst0 = lds + 2 * T::STAGE_ELEMS;                     // [2][BN][DSS]
+    float* rows0 = reinterpret_cast<float*>(lds + 2 * T::STAGE_ELEMS + 2 * T::DS_ELEMS);   // [2][lse2 | delta]
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -128,85 +138,87 @@ __global__ __launch_bounds__(256) void bwd_kernel(const BwdParams p) {
     const uint16_t* kbase = p.k + b * p.ks.b + hh * p.ks.h;
     const uint16_t* vbase = p.v + b * p.vs.b + hh * p.vs.h;
     const uint16_t* dobase = p.dout + b * p.dos.b + hh * p.dos.h;
-    const float* lsebase = p.lse + (int64_t)bh * p.Sq;
+    const float* lsebase = p.lse2 + (int64_t)bh * p.Sq;
     const float* deltabase = p.delta + (int64_t)bh * p.Sq;
     float* dqacc_base = p.dq_acc + (int64_t)bh * p.Sq * D;
 
     int klimit = p.Sk;
     if (p.m.kv_len) klimit = min(klimit, max(p.m.kv_len[b], 0));
-    const uint8_t* mbase = p.m.mask ? p.m.mask + b * p.m.sb + hh * p.m.sh : nullptr;
+    const uint8_t* mbase = HASMASK ? p.m.mask + b * p.m.sb + hh * p.m.sh : nullptr;
 
     const int n_qt = (p.Sq + BM - 1) / BM;
     int qt_begin = p.m.causal ? (k0 / BM) : 0;
     if (k0 >= klimit) qt_begin = n_qt;        // nothing attends to these keys: dK = dV = 0
 
+    // ---- per-lane LDS offsets (elements), constant over the walk
+    int roff[DC];          // 16-byte row reads: row (32*blk + n), logical granule 2*dc + h
+#pragma unroll
+    for (int dc = 0; dc < DC; ++dc) roff[dc] = n * RS + (((2 * dc + h) ^ swz<D>(n)) << 3);
+    const int tr_r = lane & 15, tr_g16 = (lane >> 4) & 1;
+    int toff[2][DB];       // transposing reads of a D-wide tile: rows 4h + r/4 (+8), granule 4*db + 2*g16 + (r&3)/2
+    int soff[2][2];        // transposing reads of dS^T (64 wide): granule 4*qb + 2*g16 + (r&3)/2
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+        const int row = 4 * h + (tr_r >> 2) + 8 * half;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+            toff[half][db] = row * RS + (((4 * db + 2 * tr_g16 + ((tr_r & 3) >> 1)) ^ swz<D>(row)) << 3) + 4 * (tr_r & 1);
+#pragma unroll
+        for (int qb = 0; qb < 2; ++qb)
+            soff[half][qb] = row * DSS + (((4 * qb + 2 * tr_g16 + ((tr_r & 3) >> 1)) ^ swz<64>(row)) << 3) + 4 * (tr_r & 1);
+    }
+    auto tr_frag = [&](const uint16_t* tile, int o0, int o1) {
+        const u32x2 lo = lds_read_tr16(tile + o0);
+        const u32x2 hi = lds_read_tr16(tile + o1);
+        const u32x4 u = {lo[0], lo[1], hi[0], hi[1]};
+        return __builtin_bit_cast(bf16x8, u);
+    };
+
     // ---- prologue: K and V fragments of this wavefront's 32 keys, held in registers for the walk
     bf16x8 kf[DC], vf[DC], ktf[BN / 16];
     {
-        constexpr int NCK = BN * (D / 8) / 256;
+        const int dma_row_in = lane / GPR, dma_gran = lane % GPR;
+        constexpr int NDMA = BN / T::ROWS_PER_DMA / 4;     // 1 KiB copies per wave for a 128-row tile
 #pragma unroll
-        for (int pass = 0; pass < 2; ++pass) {
-            const uint16_t* src = pass == 0 ? kbase : vbase;
-            const Strides st = pass == 0 ? p.ks : p.vs;
-            const int lim = pass == 0 ? p.Sk : klimit;
-#pragma unroll
-            for (int i = 0; i < NCK; ++i) {
-                const int c = tid + 256 * i;
-                const int row = c / (D / 8), col = c % (D / 8);
-                const int key = k0 + row;
-                *reinterpret_cast<u32x4*>(lds + row * QS + col * 8) = ldg16(src + (int64_t)key * st.n + col * 8, key < lim);
-            }
-            __syncthreads();
-#pragma unroll
-            for (int dc = 0; dc < DC; ++dc) {
-                const bf16x8 f = *reinterpret_cast<const bf16x8*>(lds + (32 * wave + n) * QS + 16 * dc + 8 * h);
-                if (pass == 0) kf[dc] = f; else vf[dc] = f;
-            }
-            if (pass == 0) {
-#pragma unroll
-                for (int kc = 0; kc < BN / 16; ++kc) ktf[kc] = lds_tr_frag(lds, QS, 16 * kc, 32 * (wave % NSL), lane);
-            }
-            __syncthreads();
+        for (int i = 0; i < NDMA; ++i) {
+            const int ji = wave * NDMA + i;
+            const int row = ji * T::ROWS_PER_DMA + dma_row_in;
+            const int key = max(min(k0 + row, klimit - 1), 0);   // rows past the attended range re-read a valid row
+            const int c = dma_gran ^ swz<D>(row);
+            dma16(kbase + (int64_t)key * p.ks.n + c * 8, lds + ji * 512);
+            dma16(vbase + (int64_t)key * p.vs.n + c * 8, lds + BN * RS + ji * 512);
         }
+        wait_vm0();
+        __syncthreads();
+#pragma unroll
+        for (int dc = 0; dc < DC; ++dc) {
+            kf[dc] = *reinterpret_cast<const bf16x8*>(lds + roff[dc] + 32 * wave * RS);
+            vf[dc] = *reinterpret_cast<const bf16x8*>(lds + BN * RS + roff[dc] + 32 * wave * RS);
+        }
+#pragma unroll
+        for (int kc = 0; kc < BN / 16; ++kc)
+            ktf[kc] = tr_frag(lds, toff[0][wave % NSL] + 16 * kc * RS, toff[1][wave % NSL] + 16 * kc * RS);
+        __syncthreads();
     }
 
-    // ---- staging of the 64-row Q / dO tiles
-    u32x4 qreg[NC], doreg[NC];
-    float lse_reg = 0.f, delta_reg = 0.f;
-    auto load_q_tile = [&](int qt) {
+    // ---- asynchronous staging of the 64-row Q / dO tiles and their lse2 / delta rows
+    const int dma_row_in = lane / GPR, dma_gran = lane % GPR;
+    auto issue_q_tile = [&](int qt, int buf) {
+        uint16_t* qdst = stage0 + buf * T::STAGE_ELEMS;
+        uint16_t* ddst = qdst + T::Q_ELEMS;
         const int q0 = qt * BM;
 #pragma unroll
-        for (int i = 0; i < NC; ++i) {
-            const int c = tid + 256 * i;
-            const int row = c / (D / 8), col = c % (D / 8);
-            const int qi = q0 + row;
-            qreg[i] = ldg16(qbase + (int64_t)qi * p.qs.n + col * 8, qi < p.Sq);
-            doreg[i] = ldg16(dobase + (int64_t)qi * p.dos.n + col * 8, qi < p.Sq);
+        for (int i = 0; i < T::DMA_PER_WAVE; ++i) {
+            const int ji = wave * T::DMA_PER_WAVE + i;
+            const int row = ji * T::ROWS_PER_DMA + dma_row_in;
+            const int qi = min(q0 + row, p.Sq - 1);
+            const int c = dma_gran ^ swz<D>(row);
+            dma16(qbase + (int64_t)qi * p.qs.n + c * 8, qdst + ji * 512);
+            dma16(dobase + (int64_t)qi * p.dos.n + c * 8, ddst + ji * 512);
         }
-        if (tid < BM) {
-            const int qi = q0 + tid;
-            float l = INFINITY;
-            float dl = 0.f;
-            if (qi < p.Sq) {
-                const float x = lsebase[qi];
-                l = (x == -INFINITY) ? INFINITY : x * kLog2e;    // +inf makes exp2(s*c - l) = 0
-                dl = deltabase[qi];
-            }
-            lse_reg = l;
-            delta_reg = dl;
-        }
-    };
-    auto store_q_tile = [&]() {
-#pragma unroll
-        for (int i = 0; i < NC; ++i) {
-            const int c = tid + 256 * i;
-            const int row = c / (D / 8), col = c % (D / 8);
-            *reinterpret_cast<u32x4*>(Qs + row * QS + col * 8) = qreg[i];
-            *reinterpret_cast<u32x4*>(dOs + row * QS + col * 8) = doreg[i];
-        }
-        if (tid < BM) {
-            lse_s[tid] = lse_reg;
-            delta_s[tid] = delta_reg;
+        if (wave < 2) {
+            const int qi = min(q0 + lane, p.Sq - 1);
+            dma4((wave == 0 ? lsebase : deltabase) + qi, rows0 + buf * T::ROW_FLOATS + wave * BM);
         }
     };
 
@@ -222,17 +234,23 @@ __global__ __launch_bounds__(256) void bwd_kernel(const BwdParams p) {
     const float c_log2 = p.scale * kLog2e;
     const int dslice = wave % NSL;
     const int qb_first = (wave / NSL) * QB_PER;
+    const int key = kw0 + n;
 
-    if (qt_begin < n_qt) {
-        load_q_tile(qt_begin);
-        store_q_tile();
-    }
+    if (qt_begin < n_qt) issue_q_tile(qt_begin, 0);
+    wait_vm0();
     __syncthreads();
 
     for (int qt = qt_begin; qt < n_qt; ++qt) {
+        const int it = qt - qt_begin;
+        const int buf = it & 1;
         const int q0 = qt * BM;
-        const bool more = (qt + 1) < n_qt;
-        if (more) load_q_tile(qt + 1);
+        if (qt + 1 < n_qt) issue_q_tile(qt + 1, buf ^ 1);
+
+        const uint16_t* Qs = stage0 + buf * T::STAGE_ELEMS;
+        const uint16_t* dOs = Qs + T::Q_ELEMS;
+        uint16_t* dSt = dst0 + buf * T::DS_ELEMS;
+        const float* lse_s = rows0 + buf * T::ROW_FLOATS;
+        const float* delta_s = lse_s + BM;
 
         // ---- S = Q K^T and dP = dO V^T : rows = queries (two blocks of 32), columns = this wave's keys
         f32x16 sacc[2], dpacc[2];
@@ -247,16 +265,15 @@ __global__ __launch_bounds__(256) void bwd_kernel(const BwdParams p) {
         for (int dc = 0; dc < DC; ++dc) {
 #pragma unroll
             for (int qb = 0; qb < 2; ++qb) {
-                const bf16x8 aq = *reinterpret_cast<const bf16x8*>(Qs + (32 * qb + n) * QS + 16 * dc + 8 * h);
+                const bf16x8 aq = *reinterpret_cast<const bf16x8*>(Qs + roff[dc] + 32 * qb * RS);
                 sacc[qb] = mfma32(aq, kf[dc], sacc[qb]);
-                const bf16x8 ad = *reinterpret_cast<const bf16x8*>(dOs + (32 * qb + n) * QS + 16 * dc + 8 * h);
+                const bf16x8 ad = *reinterpret_cast<const bf16x8*>(dOs + roff[dc] + 32 * qb * RS);
                 dpacc[qb] = mfma32(ad, vf[dc], dpacc[qb]);
             }
         }
 
         // ---- P and dS; lane = key column kw0+n, registers = queries
-        const int key = kw0 + n;
-        const bool need_mask = (k0 + BN > klimit) || (p.m.causal && (k0 + BN - 1 > q0)) || mbase;
+        const bool need_mask = HASMASK || (k0 + BN > klimit) || (q0 + BM > p.Sq) || (p.m.causal && (k0 + BN - 1 > q0));
         bf16x8 pf[2][2], dsf[2][2];
 #pragma unroll
         for (int qb = 0; qb < 2; ++qb) {
@@ -270,10 +287,11 @@ __global__ __launch_bounds__(256) void bwd_kernel(const BwdParams p) {
                     float pr = exp2_fast(fmaf(sacc[qb][r], c_log2, -l4[t]));
                     if (need_mask) {
                         const int qi = q0 + 32 * qb + 8 * g + 4 * h + t;
-                        bool drop = key >= klimit;
+                        bool drop = key >= klimit || qi >= p.Sq;
                         if (p.m.causal) drop = drop || key > qi;
-                        if (mbase && !drop && qi < p.Sq)
-                            drop = mbase[(int64_t)qi * p.m.sq + (int64_t)key * p.m.sk] == 0;
+                        if (HASMASK) {
+                            if (!drop) drop = mbase[(int64_t)qi * p.m.sq + (int64_t)key * p.m.sk] == 0;
+                        }
                         if (drop) pr = 0.f;
                     }
                     sacc[qb][r] = pr;
@@ -288,15 +306,17 @@ __global__ __launch_bounds__(256) void bwd_kernel(const BwdParams p) {
                 pf[qb][c] = pack8(s[o8], s[o8 + 1], s[o8 + 2], s[o8 + 3], s[o8 + 4], s[o8 + 5], s[o8 + 6], s[o8 + 7]);
                 dsf[qb][c] = pack8(d[o8], d[o8 + 1], d[o8 + 2], d[o8 + 3], d[o8 + 4], d[o8 + 5], d[o8 + 6], d[o8 + 7]);
             }
-            // dS^T[key][query]: four consecutive queries per 8-byte store
+            // dS^T[key][query]: four consecutive queries per 8-byte store, granule 4*qb + j, half h
             const u32x4 dsu0 = __builtin_bit_cast(u32x4, dsf[qb][0]);
             const u32x4 dsu1 = __builtin_bit_cast(u32x4, dsf[qb][1]);
-            uint16_t* drow = dSt + (32 * wave + n) * DSS + 32 * qb + 4 * h;
+            const int krow = 32 * wave + n;
+            uint16_t* drow = dSt + krow * DSS + 4 * h;
+            const int f = swz<64>(krow);
             u32x2 w0 = {dsu0[0], dsu0[1]}, w1 = {dsu0[2], dsu0[3]}, w2 = {dsu1[0], dsu1[1]}, w3 = {dsu1[2], dsu1[3]};
-            *reinterpret_cast<u32x2*>(drow + 0) = w0;
-            *reinterpret_cast<u32x2*>(drow + 8) = w1;
-            *reinterpret_cast<u32x2*>(drow + 16) = w2;
-            *reinterpret_cast<u32x2*>(drow + 24) = w3;
+            *reinterpret_cast<u32x2*>(drow + (((4 * qb + 0) ^ f) << 3)) = w0;
+            *reinterpret_cast<u32x2*>(drow + (((4 * qb + 1) ^ f) << 3)) = w1;
+            *reinterpret_cast<u32x2*>(drow + (((4 * qb + 2) ^ f) << 3)) = w2;
+            *reinterpret_cast<u32x2*>(drow + (((4 * qb + 3) ^ f) << 3)) = w3;
         }
 
         // ---- dV^T += dO^T P,  dK^T += Q^T dS : rows = d, columns = keys, contraction over the 64 queries
@@ -307,15 +327,15 @@ __global__ __launch_bounds__(256) void bwd_kernel(const BwdParams p) {
                 const int cc = 2 * qb + c;
 #pragma unroll
                 for (int db = 0; db < DB; ++db) {
-                    const bf16x8 a_do = lds_tr_frag(dOs, QS, 16 * cc, 32 * db, lane);
+                    const bf16x8 a_do = tr_frag(dOs, toff[0][db] + 16 * cc * RS, toff[1][db] + 16 * cc * RS);
                     dvacc[db] = mfma32(a_do, pf[qb][c], dvacc[db]);
-                    const bf16x8 a_q = lds_tr_frag(Qs, QS, 16 * cc, 32 * db, lane);
+                    const bf16x8 a_q = tr_frag(Qs, toff[0][db] + 16 * cc * RS, toff[1][db] + 16 * cc * RS);
                     dkacc[db] = mfma32(a_q, dsf[qb][c], dkacc[db]);
                 }
             }
 
-        __syncthreads();   // dS^T complete; every wave is done with this step's Q / dO tiles
-        if (more) store_q_tile();
+        wait_vm0();        // next Q / dO tile has landed in the other stage
+        __syncthreads();   // dS^T of this step complete; every wave is done with this step's Q / dO stage
 
         // ---- dQ[query][d slice] += dS K : contraction over the 128 keys of the workgroup
 #pragma unroll
@@ -326,7 +346,7 @@ __global__ __launch_bounds__(256) void bwd_kernel(const BwdParams p) {
             for (int r = 0; r < 16; ++r) dq[r] = 0.f;
 #pragma unroll
             for (int kc = 0; kc < BN / 16; ++kc) {
-                const bf16x8 a = lds_tr_frag(dSt, DSS, 16 * kc, 32 * qb, lane);
+                const bf16x8 a = tr_frag(dSt, soff[0][qb] + 16 * kc * DSS, soff[1][qb] + 16 * kc * DSS);
                 dq = mfma32(a, ktf[kc], dq);
             }
             float* dst = dqacc_base + (int64_t)(q0 + 32 * qb) * D + 32 * dslice + n;
@@ -336,7 +356,6 @@ __global__ __launch_bounds__(256) void bwd_kernel(const BwdParams p) {
                 if (q0 + 32 * qb + ql < p.Sq) unsafeAtomicAdd(dst + (int64_t)ql * D, dq[r]);
             }
         }
-        __syncthreads();   // next tile staged; dS^T free again
     }
 
     // ---- epilogue: dK^T / dV^T accumulators -> dK, dV rows of this wavefront's keys

@@ -130,6 +130,27 @@ __device__ __forceinline__ void transpose4x8(const u32x4 r[4], u32x2 out[8]) {
 // groups 4c+h and 4c+2+h; they are stored at slots 4c+2h and 4c+2h+1.
 __device__ __forceinline__ constexpr int tslot(int g) { return (g & ~3) | ((g & 1) << 1) | ((g >> 1) & 1); }
 
+// 16-byte-granule XOR swizzle of a row-major bf16 tile whose rows are D*2 bytes (no padding).
+// 16 consecutive rows get distinct bank groups for the same logical granule, and 4 consecutive rows
+// land in 4 disjoint 64-byte bank groups: both access patterns used by the kernels (16-byte row
+// reads, transposing 8-byte reads of a 4-row x 64-byte block) are conflict-free on the 64-bank LDS.
+template <int D>
+__device__ __forceinline__ constexpr int swz(int row) {
+    return D == 128 ? (((row & 3) << 2) | ((row >> 2) & 3)) : ((((row >> 1) & 1) << 2) | ((row >> 2) & 3));
+}
+
+// One wave-wide asynchronous copy global -> LDS: lane l delivers 16 (or 4) bytes to lds_dst + 16*l (4*l).
+// The destination must be wave-uniform.  Completion is tracked by vmcnt.
+__device__ __forceinline__ void dma16(const void* gsrc, void* lds_dst_wave_uniform) {
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gsrc,
+                                     (__attribute__((address_space(3))) void*)lds_dst_wave_uniform, 16, 0, 0);
+}
+__device__ __forceinline__ void dma4(const void* gsrc, void* lds_dst_wave_uniform) {
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gsrc,
+                                     (__attribute__((address_space(3))) void*)lds_dst_wave_uniform, 4, 0, 0);
+}
+__device__ __forceinline__ void wait_vm0() { __builtin_amdgcn_s_waitcnt(0x0F70); }   // vmcnt(0) only
+
 struct Strides {
     int64_t b, h, n;   // element strides of a [B,H,N,D] bf16 view; the D stride is 1
 };

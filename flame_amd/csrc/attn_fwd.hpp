@@ -27,15 +27,6 @@ struct FwdParams {
     MaskArgs m;
 };
 
-// 16-byte-granule XOR swizzle of a row-major bf16 tile whose rows are D*2 bytes (no padding).
-// 16 consecutive rows get distinct bank groups for the same logical granule, and 4 consecutive rows
-// land in 4 disjoint 64-byte bank groups: both access patterns used by the kernels (16-byte row
-// reads, transposing 8-byte reads of a 4-row x 64-byte block) are conflict-free on the 64-bank LDS.
-template <int D>
-__device__ __forceinline__ constexpr int swz(int row) {
-    return D == 128 ? (((row & 3) << 2) | ((row >> 2) & 3)) : ((((row >> 1) & 1) << 2) | ((row >> 2) & 3));
-}
-
 template <int D>
 struct FwdTile {
     static constexpr int BN = 64;                   // keys per tile
@@ -46,14 +37,6 @@ struct FwdTile {
     static constexpr int ROWS_PER_DMA = 1024 / (D * 2);          // rows covered by one 64-lane x 16-byte copy
     static constexpr int DMA_PER_WAVE = BN / ROWS_PER_DMA / 4;   // copies per wave and tensor
 };
-
-// One wave-wide asynchronous copy of 1 KiB global -> LDS: lane l delivers 16 bytes to lds_dst + 16*l.
-__device__ __forceinline__ void dma16(const uint16_t* gsrc, uint16_t* lds_dst_wave_uniform) {
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gsrc,
-                                     (__attribute__((address_space(3))) void*)lds_dst_wave_uniform, 16, 0, 0);
-}
-
-__device__ __forceinline__ void wait_vm0() { __builtin_amdgcn_s_waitcnt(0x0F70); }   // vmcnt(0) only
 
 template <int D, int NWQ, bool HASMASK>
 __global__ __launch_bounds__(256, (NWQ == 1 ? 2 : 1)) void fwd_kernel(const FwdParams p) {

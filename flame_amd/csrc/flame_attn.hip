@@ -105,11 +105,11 @@ int launch_fwd(const FwdParams& p, hipStream_t s) {
 
 size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
-template <int D>
+template <int D, bool HASMASK>
 int launch_bwd(const BwdParams& p, hipStream_t s) {
     using T = BwdTile<D>;
     static bool attr_done = false;
-    auto kern = bwd_kernel<D>;
+    auto kern = bwd_kernel<D, HASMASK>;
     if (!attr_done) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS_BYTES);
@@ -172,7 +172,7 @@ int flame_attn_profiling_read(FlameAttnKernelTimes* out) {
 size_t flame_attn_bwd_workspace_bytes(int B, int H, int N_q, int D) {
     if (B <= 0 || H <= 0 || N_q <= 0 || D <= 0) return 0;
     const size_t rows = (size_t)B * H * N_q;
-    return align_up(rows * sizeof(float), 256) + rows * (size_t)D * sizeof(float);
+    return 2 * align_up(rows * sizeof(float), 256) + rows * (size_t)D * sizeof(float);
 }
 
 int flame_attn_bwd_bf16(const void* Q, const void* K, const void* V, const void* O, const void* dO,
@@ -215,7 +215,8 @@ int flame_attn_bwd_bf16(const void* Q, const void* K, const void* V, const void*
     p.dv = static_cast<uint16_t*>(dV) + dv_off;
     const size_t rows = (size_t)B * H * N_q;
     p.delta = static_cast<float*>(workspace);
-    p.dq_acc = reinterpret_cast<float*>(static_cast<char*>(workspace) + align_up(rows * sizeof(float), 256));
+    p.lse2 = reinterpret_cast<float*>(static_cast<char*>(workspace) + align_up(rows * sizeof(float), 256));
+    p.dq_acc = reinterpret_cast<float*>(static_cast<char*>(workspace) + 2 * align_up(rows * sizeof(float), 256));
     p.qs = mk(q_strides); p.ks = mk(k_strides); p.vs = mk(v_strides); p.os = mk(o_strides);
     p.dos = mk(do_strides); p.dqs = mk(dq_strides); p.dks = mk(dk_strides); p.dvs = mk(dv_strides);
     p.B = B; p.H = H; p.Sq = N_q; p.Sk = N_kv;
@@ -228,8 +229,8 @@ int flame_attn_bwd_bf16(const void* Q, const void* K, const void* V, const void*
     p.m.sk = keep_mask ? mask_strides[3] : 0;
     p.m.causal = causal ? 1 : 0;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (D == 128) return launch_bwd<128>(p, s);
-    return launch_bwd<64>(p, s);
+    if (D == 128) return keep_mask ? launch_bwd<128, true>(p, s) : launch_bwd<128, false>(p, s);
+    return keep_mask ? launch_bwd<64, true>(p, s) : launch_bwd<64, false>(p, s);
 }
 
 int flame_sage_quant_qk_int8(const void* Q, const void* K, int B, int H, int N_q, int N_kv, int D,
