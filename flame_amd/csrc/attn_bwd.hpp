@@ -15,6 +15,8 @@
 // operand come from transposing LDS reads, so no tile is stored twice and no access pattern has
 // bank conflicts.  One workgroup barrier per step.
 #pragma once
+#include <type_traits>
+
 #include "attn_common.hpp"
 
 namespace fattn {
@@ -36,6 +38,7 @@ struct BwdParams {
     int B, H, Sq, Sk;
     float scale;
     MaskArgs m;
+    unsigned long long* phase_cycles;   // profiling aid: per-phase cycle sums of wave 0 of every workgroup, or null
 };
 
 // ------------------------------------------------------------------------------------------ prep
@@ -99,16 +102,17 @@ struct BwdTile {
     static constexpr int RS = D;                    // LDS row stride of the Q / dO / K / V tiles (swizzled, unpadded)
     static constexpr int DSS = BM;                  // LDS row stride of dS^T [key][query] (swizzled, unpadded)
     static constexpr int Q_ELEMS = BM * RS;
-    static constexpr int STAGE_ELEMS = 2 * Q_ELEMS;               // Q tile + dO tile
+    static constexpr int STAGE_ELEMS = 2 * Q_ELEMS;               // Q tile + dO tile (also one 128-row tile)
     static constexpr int DS_ELEMS = BN * DSS;
+    static constexpr int K_ELEMS = BN * RS;                       // resident K tile
     static constexpr int ROW_FLOATS = 2 * BM;                     // lse2 + delta of one step
-    // [2 stages of Q,dO][2 dS^T buffers][2 x (lse2, delta)]
-    static constexpr int LDS_BYTES = (2 * STAGE_ELEMS + 2 * DS_ELEMS) * 2 + 2 * ROW_FLOATS * 4;
+    // [2 stages of Q,dO][2 dS^T buffers][resident K][2 x (lse2, delta)]
+    static constexpr int LDS_BYTES = (2 * STAGE_ELEMS + 2 * DS_ELEMS + K_ELEMS) * 2 + 2 * ROW_FLOATS * 4;
     static constexpr int ROWS_PER_DMA = 1024 / (D * 2);
     static constexpr int DMA_PER_WAVE = BM / ROWS_PER_DMA / 4;    // 1 KiB copies per wave and tensor
 };
 
-template <int D, bool HASMASK>
+template <int D, bool HASMASK, bool TIMING>
 __global__ __launch_bounds__(256) void bwd_kernel(const BwdParams p) {
     using T = BwdTile<D>;
     constexpr int BM = T::BM, BN = T::BN, RS = T::RS, DSS = T::DSS;
@@ -117,19 +121,22 @@ __global__ __launch_bounds__(256) void bwd_kernel(const BwdParams p) {
     constexpr int NSL = D / 32;    // 32-column slices of dQ
     constexpr int QB_PER = 2 / (4 / NSL);   // query blocks per wave in the dQ step
     constexpr int GPR = D / 8;     // 16-byte granules per row
+    constexpr int RPD = T::ROWS_PER_DMA, NDQ = T::DMA_PER_WAVE;
 
     extern __shared__ __attribute__((aligned(1024))) uint16_t lds[];
     uint16_t* stage0 = lds;                                        // [2][Q tile | dO tile]
     uint16_t* dst0 = lds + 2 * T::STAGE_ELEMS;                     // [2][BN][DSS]
-    float* rows0 = reinterpret_cast<float*>(lds + 2 * T::STAGE_ELEMS + 2 * T::DS_ELEMS);   // [2][lse2 | delta]
+    uint16_t* Kres = dst0 + 2 * T::DS_ELEMS;                       // [BN][RS]
+    float* rows0 = reinterpret_cast<float*>(Kres + T::K_ELEMS);    // [2][lse2 | delta]
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int n = lane & 31, h = lane >> 5;
 
     const int n_kt = (p.Sk + BN - 1) / BN;
-    const int kt = blockIdx.x % n_kt;
-    const int bh = blockIdx.x / n_kt;
+    const int wg = xcd_remap(blockIdx.x, gridDim.x);
+    const int kt = wg % n_kt;
+    const int bh = wg / n_kt;
     const int b = bh / p.H, hh = bh % p.H;
     const int k0 = kt * BN;
     const int kw0 = k0 + 32 * wave;
@@ -149,6 +156,12 @@ __global__ __launch_bounds__(256) void bwd_kernel(const BwdParams p) {
     const int n_qt = (p.Sq + BM - 1) / BM;
     int qt_begin = p.m.causal ? (k0 / BM) : 0;
     if (k0 >= klimit) qt_begin = n_qt;        // nothing attends to these keys: dK = dV = 0
+    const int n_it = n_qt - qt_begin;
+    // Workgroups of one head start their walk at different query tiles (and wrap around), so that at
+    // any moment they add into different rows of the dQ accumulator instead of contending for the
+    // same cache lines in L2.
+    const int rot = n_it > 0 ? (int)(((int64_t)kt * n_it) / n_kt) : 0;
+    auto tile_of = [&](int it) { int r = it + rot; if (r >= n_it) r -= n_it; return qt_begin + r; };
 
     // ---- per-lane LDS offsets (elements), constant over the walk
     int roff[DC];          // 16-byte row reads: row (32*blk + n), logical granule 2*dc + h
@@ -174,51 +187,70 @@ __global__ __launch_bounds__(256) void bwd_kernel(const BwdParams p) {
         return __builtin_bit_cast(bf16x8, u);
     };
 
-    // ---- prologue: K and V fragments of this wavefront's 32 keys, held in registers for the walk
-    bf16x8 kf[DC], vf[DC], ktf[BN / 16];
+    const int dma_row_in = lane / GPR, dma_gran = lane % GPR;
+
+    // ---- prologue: K tile stays resident in LDS (B operand of the dQ step); the K and V fragments
+    //      of this wavefront's 32 keys are held in registers for the whole walk
+    bf16x8 kf[DC], vf[DC];
     {
-        const int dma_row_in = lane / GPR, dma_gran = lane % GPR;
-        constexpr int NDMA = BN / T::ROWS_PER_DMA / 4;     // 1 KiB copies per wave for a 128-row tile
+        constexpr int NDMA = BN / RPD / 4;     // 1 KiB copies per wave for a 128-row tile
 #pragma unroll
         for (int i = 0; i < NDMA; ++i) {
             const int ji = wave * NDMA + i;
-            const int row = ji * T::ROWS_PER_DMA + dma_row_in;
+            const int row = ji * RPD + dma_row_in;
             const int key = max(min(k0 + row, klimit - 1), 0);   // rows past the attended range re-read a valid row
             const int c = dma_gran ^ swz<D>(row);
-            dma16(kbase + (int64_t)key * p.ks.n + c * 8, lds + ji * 512);
-            dma16(vbase + (int64_t)key * p.vs.n + c * 8, lds + BN * RS + ji * 512);
+            dma16(kbase + (int64_t)key * p.ks.n + c * 8, Kres + ji * 512);
+            dma16(vbase + (int64_t)key * p.vs.n + c * 8, stage0 + ji * 512);
         }
         wait_vm0();
         __syncthreads();
 #pragma unroll
         for (int dc = 0; dc < DC; ++dc) {
-            kf[dc] = *reinterpret_cast<const bf16x8*>(lds + roff[dc] + 32 * wave * RS);
-            vf[dc] = *reinterpret_cast<const bf16x8*>(lds + BN * RS + roff[dc] + 32 * wave * RS);
+            kf[dc] = *reinterpret_cast<const bf16x8*>(Kres + roff[dc] + 32 * wave * RS);
+            vf[dc] = *reinterpret_cast<const bf16x8*>(stage0 + roff[dc] + 32 * wave * RS);
         }
-#pragma unroll
-        for (int kc = 0; kc < BN / 16; ++kc)
-            ktf[kc] = tr_frag(lds, toff[0][wave % NSL] + 16 * kc * RS, toff[1][wave % NSL] + 16 * kc * RS);
         __syncthreads();
     }
 
-    // ---- asynchronous staging of the 64-row Q / dO tiles and their lse2 / delta rows
-    const int dma_row_in = lane / GPR, dma_gran = lane % GPR;
+    // ---- asynchronous staging of the 64-row Q / dO tiles and their lse2 / delta rows.
+    //      Address = uniform tile base + a per-lane 32-bit offset that never changes.
+    int q_lane_off[NDQ], do_lane_off[NDQ];
+#pragma unroll
+    for (int i = 0; i < NDQ; ++i) {
+        const int row = (wave * NDQ + i) * RPD + dma_row_in;
+        const int c = dma_gran ^ swz<D>(row);
+        q_lane_off[i] = row * (int)p.qs.n + c * 8;
+        do_lane_off[i] = row * (int)p.dos.n + c * 8;
+    }
     auto issue_q_tile = [&](int qt, int buf) {
         uint16_t* qdst = stage0 + buf * T::STAGE_ELEMS;
         uint16_t* ddst = qdst + T::Q_ELEMS;
         const int q0 = qt * BM;
+        if (q0 + BM <= p.Sq) {
+            const uint16_t* qt_base = qbase + (int64_t)q0 * p.qs.n;
+            const uint16_t* dot_base = dobase + (int64_t)q0 * p.dos.n;
 #pragma unroll
-        for (int i = 0; i < T::DMA_PER_WAVE; ++i) {
-            const int ji = wave * T::DMA_PER_WAVE + i;
-            const int row = ji * T::ROWS_PER_DMA + dma_row_in;
-            const int qi = min(q0 + row, p.Sq - 1);
-            const int c = dma_gran ^ swz<D>(row);
-            dma16(qbase + (int64_t)qi * p.qs.n + c * 8, qdst + ji * 512);
-            dma16(dobase + (int64_t)qi * p.dos.n + c * 8, ddst + ji * 512);
-        }
-        if (wave < 2) {
-            const int qi = min(q0 + lane, p.Sq - 1);
-            dma4((wave == 0 ? lsebase : deltabase) + qi, rows0 + buf * T::ROW_FLOATS + wave * BM);
+            for (int i = 0; i < NDQ; ++i) {
+                const int ji = wave * NDQ + i;
+                dma16(qt_base + q_lane_off[i], qdst + ji * 512);
+                dma16(dot_base + do_lane_off[i], ddst + ji * 512);
+            }
+            if (wave < 2) dma4((wave == 0 ? lsebase : deltabase) + q0 + lane, rows0 + buf * T::ROW_FLOATS + wave * BM);
+        } else {   // last, partial tile: rows past the end re-read the last valid row
+#pragma unroll
+            for (int i = 0; i < NDQ; ++i) {
+                const int ji = wave * NDQ + i;
+                const int row = ji * RPD + dma_row_in;
+                const int qi = min(q0 + row, p.Sq - 1);
+                const int c = dma_gran ^ swz<D>(row);
+                dma16(qbase + (int64_t)qi * p.qs.n + c * 8, qdst + ji * 512);
+                dma16(dobase + (int64_t)qi * p.dos.n + c * 8, ddst + ji * 512);
+            }
+            if (wave < 2) {
+                const int qi = min(q0 + lane, p.Sq - 1);
+                dma4((wave == 0 ? lsebase : deltabase) + qi, rows0 + buf * T::ROW_FLOATS + wave * BM);
+            }
         }
     };
 
@@ -235,16 +267,29 @@ __global__ __launch_bounds__(256) void bwd_kernel(const BwdParams p) {
     const int dslice = wave % NSL;
     const int qb_first = (wave / NSL) * QB_PER;
     const int key = kw0 + n;
+    // dQ accumulator offsets of this lane (floats): d column 32*dslice + n, query rows 8g + 4h + t
+    int dq_lane_off[4];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) dq_lane_off[g] = (8 * g + 4 * h) * D + 32 * dslice + n;
 
-    if (qt_begin < n_qt) issue_q_tile(qt_begin, 0);
+    unsigned long long ph[6] = {0, 0, 0, 0, 0, 0};
+    unsigned long long tprev = TIMING ? __builtin_readcyclecounter() : 0ull;
+#define FATTN_PHASE(i)                                                  \
+    if (TIMING) {                                                       \
+        const unsigned long long tnow = __builtin_readcyclecounter();   \
+        ph[i] += tnow - tprev;                                          \
+        tprev = tnow;                                                   \
+    }
+
+    if (n_it > 0) issue_q_tile(tile_of(0), 0);
+    if (n_it > 1) issue_q_tile(tile_of(1), 1);
     wait_vm0();
     __syncthreads();
 
-    for (int qt = qt_begin; qt < n_qt; ++qt) {
-        const int it = qt - qt_begin;
+    for (int it = 0; it < n_it; ++it) {
+        const int qt = tile_of(it);
         const int buf = it & 1;
         const int q0 = qt * BM;
-        if (qt + 1 < n_qt) issue_q_tile(qt + 1, buf ^ 1);
 
         const uint16_t* Qs = stage0 + buf * T::STAGE_ELEMS;
         const uint16_t* dOs = Qs + T::Q_ELEMS;
@@ -261,102 +306,173 @@ __global__ __launch_bounds__(256) void bwd_kernel(const BwdParams p) {
                 sacc[qb][r] = 0.f;
                 dpacc[qb][r] = 0.f;
             }
+        {
+            // LDS reads run PD fragments ahead of the MFMAs that consume them; the scheduling barriers
+            // keep the compiler from sinking the reads back next to their uses (one wave per SIMD:
+            // nothing else hides the LDS latency).
+            constexpr int NF = 4 * DC, PD = 4;
+            bf16x8 fb[PD];
+            auto rd = [&](int i) {
+                const int dc = i >> 2, qb = (i >> 1) & 1;
+                return *reinterpret_cast<const bf16x8*>(((i & 1) ? dOs : Qs) + roff[dc] + 32 * qb * RS);
+            };
 #pragma unroll
-        for (int dc = 0; dc < DC; ++dc) {
+            for (int i = 0; i < PD; ++i) fb[i] = rd(i);
 #pragma unroll
-            for (int qb = 0; qb < 2; ++qb) {
-                const bf16x8 aq = *reinterpret_cast<const bf16x8*>(Qs + roff[dc] + 32 * qb * RS);
-                sacc[qb] = mfma32(aq, kf[dc], sacc[qb]);
-                const bf16x8 ad = *reinterpret_cast<const bf16x8*>(dOs + roff[dc] + 32 * qb * RS);
-                dpacc[qb] = mfma32(ad, vf[dc], dpacc[qb]);
+            for (int i = 0; i < NF; ++i) {
+                const int dc = i >> 2, qb = (i >> 1) & 1;
+                if (i & 1) dpacc[qb] = mfma32(fb[i % PD], vf[dc], dpacc[qb]);
+                else sacc[qb] = mfma32(fb[i % PD], kf[dc], sacc[qb]);
+                if (i + PD < NF) fb[i % PD] = rd(i + PD);
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
 
+        FATTN_PHASE(0)
         // ---- P and dS; lane = key column kw0+n, registers = queries
         const bool need_mask = HASMASK || (k0 + BN > klimit) || (q0 + BM > p.Sq) || (p.m.causal && (k0 + BN - 1 > q0));
         bf16x8 pf[2][2], dsf[2][2];
+        auto elementwise = [&](auto masked_tag) {
+            constexpr bool MASKED = decltype(masked_tag)::value;
 #pragma unroll
-        for (int qb = 0; qb < 2; ++qb) {
+            for (int qb = 0; qb < 2; ++qb) {
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const f32x4 l4 = *reinterpret_cast<const f32x4*>(lse_s + 32 * qb + 8 * g + 4 * h);
-                const f32x4 d4 = *reinterpret_cast<const f32x4*>(delta_s + 32 * qb + 8 * g + 4 * h);
+                for (int g = 0; g < 4; ++g) {
+                    const f32x4 l4 = *reinterpret_cast<const f32x4*>(lse_s + 32 * qb + 8 * g + 4 * h);
+                    const f32x4 d4 = *reinterpret_cast<const f32x4*>(delta_s + 32 * qb + 8 * g + 4 * h);
 #pragma unroll
-                for (int t = 0; t < 4; ++t) {
-                    const int r = 4 * g + t;
-                    float pr = exp2_fast(fmaf(sacc[qb][r], c_log2, -l4[t]));
-                    if (need_mask) {
-                        const int qi = q0 + 32 * qb + 8 * g + 4 * h + t;
-                        bool drop = key >= klimit || qi >= p.Sq;
-                        if (p.m.causal) drop = drop || key > qi;
-                        if (HASMASK) {
-                            if (!drop) drop = mbase[(int64_t)qi * p.m.sq + (int64_t)key * p.m.sk] == 0;
+                    for (int t = 0; t < 4; ++t) {
+                        const int r = 4 * g + t;
+                        float pr = exp2_fast(fmaf(sacc[qb][r], c_log2, -l4[t]));
+                        if (MASKED) {
+                            const int qi = q0 + 32 * qb + 8 * g + 4 * h + t;
+                            bool drop = key >= klimit || qi >= p.Sq;
+                            if (p.m.causal) drop = drop || key > qi;
+                            if (HASMASK) {
+                                if (!drop) drop = mbase[(int64_t)qi * p.m.sq + (int64_t)key * p.m.sk] == 0;
+                            }
+                            pr = drop ? 0.f : pr;
                         }
-                        if (drop) pr = 0.f;
+                        sacc[qb][r] = pr;
+                        dpacc[qb][r] = pr * (dpacc[qb][r] - d4[t]);
                     }
-                    sacc[qb][r] = pr;
-                    dpacc[qb][r] = pr * (dpacc[qb][r] - d4[t]);
+                }
+#pragma unroll
+                for (int c = 0; c < 2; ++c) {
+                    const f32x16& s = sacc[qb];
+                    const f32x16& d = dpacc[qb];
+                    const int o8 = 8 * c;
+                    pf[qb][c] = pack8(s[o8], s[o8 + 1], s[o8 + 2], s[o8 + 3], s[o8 + 4], s[o8 + 5], s[o8 + 6], s[o8 + 7]);
+                    dsf[qb][c] = pack8(d[o8], d[o8 + 1], d[o8 + 2], d[o8 + 3], d[o8 + 4], d[o8 + 5], d[o8 + 6], d[o8 + 7]);
                 }
             }
-#pragma unroll
-            for (int c = 0; c < 2; ++c) {
-                const f32x16& s = sacc[qb];
-                const f32x16& d = dpacc[qb];
-                const int o8 = 8 * c;
-                pf[qb][c] = pack8(s[o8], s[o8 + 1], s[o8 + 2], s[o8 + 3], s[o8 + 4], s[o8 + 5], s[o8 + 6], s[o8 + 7]);
-                dsf[qb][c] = pack8(d[o8], d[o8 + 1], d[o8 + 2], d[o8 + 3], d[o8 + 4], d[o8 + 5], d[o8 + 6], d[o8 + 7]);
-            }
-            // dS^T[key][query]: four consecutive queries per 8-byte store, granule 4*qb + j, half h
-            const u32x4 dsu0 = __builtin_bit_cast(u32x4, dsf[qb][0]);
-            const u32x4 dsu1 = __builtin_bit_cast(u32x4, dsf[qb][1]);
+        };
+        if (need_mask) elementwise(std::true_type{});
+        else elementwise(std::false_type{});
+
+        // dS^T[key][query]: four consecutive queries per 8-byte store, granule 4*qb + j, half h
+        {
             const int krow = 32 * wave + n;
             uint16_t* drow = dSt + krow * DSS + 4 * h;
             const int f = swz<64>(krow);
-            u32x2 w0 = {dsu0[0], dsu0[1]}, w1 = {dsu0[2], dsu0[3]}, w2 = {dsu1[0], dsu1[1]}, w3 = {dsu1[2], dsu1[3]};
-            *reinterpret_cast<u32x2*>(drow + (((4 * qb + 0) ^ f) << 3)) = w0;
-            *reinterpret_cast<u32x2*>(drow + (((4 * qb + 1) ^ f) << 3)) = w1;
-            *reinterpret_cast<u32x2*>(drow + (((4 * qb + 2) ^ f) << 3)) = w2;
-            *reinterpret_cast<u32x2*>(drow + (((4 * qb + 3) ^ f) << 3)) = w3;
+#pragma unroll
+            for (int qb = 0; qb < 2; ++qb) {
+                const u32x4 dsu0 = __builtin_bit_cast(u32x4, dsf[qb][0]);
+                const u32x4 dsu1 = __builtin_bit_cast(u32x4, dsf[qb][1]);
+                u32x2 w0 = {dsu0[0], dsu0[1]}, w1 = {dsu0[2], dsu0[3]}, w2 = {dsu1[0], dsu1[1]}, w3 = {dsu1[2], dsu1[3]};
+                *reinterpret_cast<u32x2*>(drow + (((4 * qb + 0) ^ f) << 3)) = w0;
+                *reinterpret_cast<u32x2*>(drow + (((4 * qb + 1) ^ f) << 3)) = w1;
+                *reinterpret_cast<u32x2*>(drow + (((4 * qb + 2) ^ f) << 3)) = w2;
+                *reinterpret_cast<u32x2*>(drow + (((4 * qb + 3) ^ f) << 3)) = w3;
+            }
         }
 
+        FATTN_PHASE(1)
         // ---- dV^T += dO^T P,  dK^T += Q^T dS : rows = d, columns = keys, contraction over the 64 queries
+        {
+            constexpr int NF = 8 * DB, PD = 3;
+            bf16x8 fb[PD];
+            auto rd = [&](int i) {
+                const int db = (i >> 1) % DB, cc = i / (2 * DB);
+                return tr_frag((i & 1) ? Qs : dOs, toff[0][db] + 16 * cc * RS, toff[1][db] + 16 * cc * RS);
+            };
 #pragma unroll
-        for (int qb = 0; qb < 2; ++qb)
+            for (int i = 0; i < PD; ++i) fb[i] = rd(i);
 #pragma unroll
-            for (int c = 0; c < 2; ++c) {
-                const int cc = 2 * qb + c;
-#pragma unroll
-                for (int db = 0; db < DB; ++db) {
-                    const bf16x8 a_do = tr_frag(dOs, toff[0][db] + 16 * cc * RS, toff[1][db] + 16 * cc * RS);
-                    dvacc[db] = mfma32(a_do, pf[qb][c], dvacc[db]);
-                    const bf16x8 a_q = tr_frag(Qs, toff[0][db] + 16 * cc * RS, toff[1][db] + 16 * cc * RS);
-                    dkacc[db] = mfma32(a_q, dsf[qb][c], dkacc[db]);
-                }
+            for (int i = 0; i < NF; ++i) {
+                const int db = (i >> 1) % DB, cc = i / (2 * DB);
+                const int qb = cc >> 1, c = cc & 1;
+                if (i & 1) dkacc[db] = mfma32(fb[i % PD], dsf[qb][c], dkacc[db]);
+                else dvacc[db] = mfma32(fb[i % PD], pf[qb][c], dvacc[db]);
+                if (i + PD < NF) fb[i % PD] = rd(i + PD);
+                __builtin_amdgcn_sched_barrier(0);
             }
+        }
 
-        wait_vm0();        // next Q / dO tile has landed in the other stage
-        __syncthreads();   // dS^T of this step complete; every wave is done with this step's Q / dO stage
+        FATTN_PHASE(2)
+        wait_vm0();        // the other stage (copy issued one step ago) has landed; older dQ atomics are done
+        FATTN_PHASE(3)
+        __syncthreads();   // dS^T of this step complete; every wave is done reading this step's stage
+        FATTN_PHASE(4)
 
         // ---- dQ[query][d slice] += dS K : contraction over the 128 keys of the workgroup
+        {
+            f32x16 dq[QB_PER];
 #pragma unroll
-        for (int i = 0; i < QB_PER; ++i) {
-            const int qb = qb_first + i;
-            f32x16 dq;
+            for (int i = 0; i < QB_PER; ++i)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) dq[r] = 0.f;
+                for (int r = 0; r < 16; ++r) dq[i][r] = 0.f;
+            constexpr int NK = BN / 16;
+            // fragment stream per key chunk: K^T slice, then dS of each query block
+            constexpr int PER = 1 + QB_PER, NF = NK * PER, PD = 3;
+            bf16x8 fb[PD];
+            auto rd = [&](int i) {
+                const int kc = i / PER, j = i % PER;
+                if (j == 0) return tr_frag(Kres, toff[0][dslice] + 16 * kc * RS, toff[1][dslice] + 16 * kc * RS);
+                const int qb = qb_first + j - 1;
+                return tr_frag(dSt, soff[0][qb] + 16 * kc * DSS, soff[1][qb] + 16 * kc * DSS);
+            };
+            // query blocks are selected per wave at run time only through qb_first (0 or QB_PER)
+            bf16x8 kfrag;
 #pragma unroll
-            for (int kc = 0; kc < BN / 16; ++kc) {
-                const bf16x8 a = tr_frag(dSt, soff[0][qb] + 16 * kc * DSS, soff[1][qb] + 16 * kc * DSS);
-                dq = mfma32(a, ktf[kc], dq);
+            for (int i = 0; i < PD; ++i) fb[i] = rd(i);
+#pragma unroll
+            for (int i = 0; i < NF; ++i) {
+                const int j = i % PER;
+                if (j == 0) kfrag = fb[i % PD];
+                else dq[j - 1] = mfma32(fb[i % PD], kfrag, dq[j - 1]);
+                if (i + PD < NF) fb[i % PD] = rd(i + PD);
+                __builtin_amdgcn_sched_barrier(0);
             }
-            float* dst = dqacc_base + (int64_t)(q0 + 32 * qb) * D + 32 * dslice + n;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int ql = acc_row(r, h);
-                if (q0 + 32 * qb + ql < p.Sq) unsafeAtomicAdd(dst + (int64_t)ql * D, dq[r]);
+            for (int i = 0; i < QB_PER; ++i) {
+                const int qb = qb_first + i;
+                float* dst = dqacc_base + (int64_t)(q0 + 32 * qb) * D;     // uniform
+                if (q0 + BM <= p.Sq) {
+#pragma unroll
+                    for (int g = 0; g < 4; ++g)
+#pragma unroll
+                        for (int t = 0; t < 4; ++t) unsafeAtomicAdd(dst + dq_lane_off[g] + t * D, dq[i][4 * g + t]);
+                } else {
+#pragma unroll
+                    for (int g = 0; g < 4; ++g)
+#pragma unroll
+                        for (int t = 0; t < 4; ++t)
+                            if (q0 + 32 * qb + 8 * g + 4 * h + t < p.Sq)
+                                unsafeAtomicAdd(dst + dq_lane_off[g] + t * D, dq[i][4 * g + t]);
+                }
             }
         }
+        // this step's stage is free (everyone passed the barrier): refill it two steps ahead
+        if (it + 2 < n_it) issue_q_tile(tile_of(it + 2), buf);
+        FATTN_PHASE(5)
     }
+
+    if (TIMING && p.phase_cycles && tid == 0) {
+#pragma unroll
+        for (int i = 0; i < 6; ++i) p.phase_cycles[(size_t)blockIdx.x * 6 + i] = ph[i];
+    }
+#undef FATTN_PHASE
 
     // ---- epilogue: dK^T / dV^T accumulators -> dK, dV rows of this wavefront's keys
     const int krow = kw0 + n;

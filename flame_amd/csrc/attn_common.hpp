@@ -151,6 +151,14 @@ __device__ __forceinline__ void dma4(const void* gsrc, void* lds_dst_wave_unifor
 }
 __device__ __forceinline__ void wait_vm0() { __builtin_amdgcn_s_waitcnt(0x0F70); }   // vmcnt(0) only
 
+// Workgroups are dealt to the 8 XCDs (each with its own L2) round-robin by linear id.  Remap the id
+// so that XCD x works on the contiguous range [x*total/8, (x+1)*total/8) of tiles: all tiles of one
+// (batch, head) then share one L2 and its K/V (forward) or Q/dO (backward) stay resident there.
+__device__ __forceinline__ int xcd_remap(int linear, int total) {
+    constexpr int kXcd = 8;
+    return (total % kXcd == 0) ? (linear % kXcd) * (total / kXcd) + linear / kXcd : linear;
+}
+
 struct Strides {
     int64_t b, h, n;   // element strides of a [B,H,N,D] bf16 view; the D stride is 1
 };

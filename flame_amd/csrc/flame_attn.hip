@@ -26,12 +26,20 @@ int check_view(const void* base, const int64_t* st, int64_t off) {
     if (!base || !st) return FLAME_ATTN_ERR_INVALID;
     if (st[3] != 1) return FLAME_ATTN_ERR_UNSUPPORTED;
     if ((st[0] | st[1] | st[2] | off) & 7) return FLAME_ATTN_ERR_UNSUPPORTED;
+    if (st[2] >= (int64_t(1) << 24)) return FLAME_ATTN_ERR_UNSUPPORTED;   // row offsets inside a tile are kept in 32 bits
     if (st[0] < 0 || st[1] < 0 || st[2] < 0) return FLAME_ATTN_ERR_UNSUPPORTED;
     if (!aligned16(static_cast<const uint16_t*>(base) + off)) return FLAME_ATTN_ERR_UNSUPPORTED;
     return FLAME_ATTN_OK;
 }
 
 Strides mk(const int64_t* st) { return Strides{st[0], st[1], st[2]}; }
+
+// Tile-shape override for profiling sweeps: FLAME_ATTN_FWD_VARIANT = 0 (default) | 1 | 2 ...
+int env_int(const char* name, int dflt) {
+    const char* v = getenv(name);
+    return v ? atoi(v) : dflt;
+}
+
 
 // Optional per-kernel timing with HIP events on the caller's stream (off by default; when off the
 // launch path touches none of this).  Event pairs are created on demand and summed on read.
@@ -59,6 +67,7 @@ struct Profiler {
     }
 };
 Profiler g_prof;
+unsigned long long* g_phase_cycles = nullptr;   // device buffer set by flame_attn_debug_set_phase_buffer
 
 struct ScopedKernelTimer {
     hipEvent_t stop_ev = nullptr;
@@ -73,12 +82,6 @@ struct ScopedKernelTimer {
         if (stop_ev) (void)hipEventRecord(stop_ev, s);
     }
 };
-
-// Tile-shape override for profiling sweeps: FLAME_ATTN_FWD_VARIANT = 0 (default) | 1 | 2 ...
-int env_int(const char* name, int dflt) {
-    const char* v = getenv(name);
-    return v ? atoi(v) : dflt;
-}
 
 template <int D, int NWQ, bool HASMASK>
 int launch_fwd(const FwdParams& p, hipStream_t s) {
@@ -105,11 +108,11 @@ int launch_fwd(const FwdParams& p, hipStream_t s) {
 
 size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
-template <int D, bool HASMASK>
+template <int D, bool HASMASK, bool TIMING = false>
 int launch_bwd(const BwdParams& p, hipStream_t s) {
     using T = BwdTile<D>;
     static bool attr_done = false;
-    auto kern = bwd_kernel<D, HASMASK>;
+    auto kern = bwd_kernel<D, HASMASK, TIMING>;
     if (!attr_done) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS_BYTES);
@@ -141,6 +144,11 @@ int launch_bwd(const BwdParams& p, hipStream_t s) {
 }  // namespace
 
 extern "C" {
+
+int flame_attn_debug_set_phase_buffer(void* device_buffer) {
+    g_phase_cycles = static_cast<unsigned long long*>(device_buffer);
+    return FLAME_ATTN_OK;
+}
 
 int flame_attn_profiling_enable(int on) {
     std::lock_guard<std::mutex> g(g_prof.mu);
@@ -228,7 +236,9 @@ int flame_attn_bwd_bf16(const void* Q, const void* K, const void* V, const void*
     p.m.sq = keep_mask ? mask_strides[2] : 0;
     p.m.sk = keep_mask ? mask_strides[3] : 0;
     p.m.causal = causal ? 1 : 0;
+    p.phase_cycles = g_phase_cycles;
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (D == 128 && !keep_mask && g_phase_cycles) return launch_bwd<128, false, true>(p, s);   // phase-timing build
     if (D == 128) return keep_mask ? launch_bwd<128, true>(p, s) : launch_bwd<128, false>(p, s);
     return keep_mask ? launch_bwd<64, true>(p, s) : launch_bwd<64, false>(p, s);
 }

@@ -196,8 +196,9 @@ __global__ __launch_bounds__(256) void sage_fwd_kernel(const SageFwdParams p) {
     const int n = lane & 31, h = lane >> 5;
 
     const int n_qt = (p.Sq + BM - 1) / BM;
-    const int qt = blockIdx.x % n_qt;
-    const int bh = blockIdx.x / n_qt;
+    const int wg = xcd_remap(blockIdx.x, gridDim.x);
+    const int qt = wg % n_qt;
+    const int bh = wg / n_qt;
     const int b = bh / p.H, hh = bh % p.H;
     const int q0 = qt * BM;
     const int qw0 = q0 + wave * 32;
