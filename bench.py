@@ -96,7 +96,7 @@ def main():
     tflops = (flops_fwd + flops_bwd) / (ms * 1e-3) / 1e12
     per_kernel = {kname: tot / n for kname, (tot, n) in times.items() if n}
     # dominant kernel: the backward main kernel carries the five backward GEMMs (10*B*H*Sq*Sk*D flops)
-    dom = "bwd_main"
+    dom = "bwd_dkdv"
     dom_ms = per_kernel[dom]
     achieved = flops_bwd / (dom_ms * 1e-3) / 1e12
     fwd_tflops = flops_fwd / (per_kernel["fwd"] * 1e-3) / 1e12

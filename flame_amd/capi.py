@@ -110,7 +110,7 @@ def attn_bwd(q, k, v, o, do, lse, scale, causal=False, kv_len=None, mask=None, w
     return dq, dk, dv
 
 
-KERNEL_KINDS = ("fwd", "bwd_prep", "bwd_main", "bwd_dq_convert", "sage_kmean", "sage_quant", "sage_fwd", "reserved")
+KERNEL_KINDS = ("fwd", "bwd_prep", "bwd_dkdv", "bwd_dq", "sage_kmean", "sage_quant", "sage_fwd", "reserved")
 
 
 class _KernelTimes(ctypes.Structure):

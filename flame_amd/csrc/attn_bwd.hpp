@@ -1,14 +1,18 @@
 // Backward of the tiled attention for gfx950: recomputes P tile by tile from Q, K and the saved
 // log-sum-exp, never materialising the Sq x Sk matrix.
 //
-//   prep     delta_i = sum_d dO_id * O_id   (fp32), LSE_i * log2(e), and clears the fp32 dQ accumulator
-//   main     one workgroup owns 128 keys (32 per wavefront) of one (batch, head) and walks over the
+//   prep     delta_i = sum_d dO_id * O_id  and  LSE_i * log2(e)   (fp32, one value per query row)
+//   dkdv     one workgroup owns 128 keys (32 per wavefront) of one (batch, head) and walks over the
 //            query tiles (64 rows): S = Q K^T, dP = dO V^T, P = exp2(S*c - LSE*log2e),
-//            dS = P * (dP - delta); dV^T += dO^T P and dK^T += Q^T dS stay in registers for the
-//            whole walk (P and dS are used as MFMA operands straight from the accumulators);
-//            dS goes through LDS once to be re-read with keys as the contraction index for
-//            dQ += dS K, which is added to an fp32 accumulator in HBM with hardware atomics
-//   convert  dQ = bf16(scale * accumulator)
+//            dS = P * (dP - delta); dV^T += dO^T P and dK^T += Q^T dS stay in fp32 registers for the
+//            whole walk (P and dS are used as MFMA operands straight from the accumulators)
+//   dq       one workgroup owns 128 queries (32 per wavefront) and walks over the key tiles (64 keys),
+//            with the logits transposed (lane = query): S^T = K Q^T, dP^T = V dO^T,
+//            dS^T = P^T (dP^T - delta) and dQ^T += K^T dS^T accumulated in fp32 registers for the whole
+//            walk, dS^T going into the last MFMA straight from the accumulators.
+// Accumulating dQ from the dkdv walk with fp32 atomics was measured at about one lane-atomic per
+// clock per CU, more than the whole MFMA time of the backward; recomputing S and dP in a second,
+// query-major kernel costs 2 extra GEMMs out of 7 and no atomics, no fp32 scratch and no convert pass.
 //
 // Q and dO tiles are copied global -> LDS by asynchronous LDS-DMA loads, double buffered, row-major
 // with an XOR swizzle of the 16-byte granules; their transposed MFMA operands (Q^T, dO^T) and the dS
@@ -33,7 +37,6 @@ struct BwdParams {
     uint16_t* dv;
     float* delta;         // workspace, [B*H, Sq]
     float* lse2;          // workspace, [B*H, Sq]: LSE * log2(e), +inf where LSE = -inf
-    float* dq_acc;        // workspace, [B*H, Sq, D] fp32
     Strides qs, ks, vs, os, dos, dqs, dks, dvs;
     int B, H, Sq, Sk;
     float scale;
@@ -60,10 +63,6 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(const BwdParams p) {
         const u32x4 c = *reinterpret_cast<const u32x4*>(p.o + b * p.os.b + hh * p.os.h + (int64_t)row * p.os.n + chunk * 8);
 #pragma unroll
         for (int i = 0; i < 4; ++i) acc += bf16_lo(a[i]) * bf16_lo(c[i]) + bf16_hi(a[i]) * bf16_hi(c[i]);
-        f32x4 z = {0.f, 0.f, 0.f, 0.f};
-        f32x4* dst = reinterpret_cast<f32x4*>(p.dq_acc + row_flat * D + chunk * 8);
-        dst[0] = z;
-        dst[1] = z;
     }
 #pragma unroll
     for (int off = TPR / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
@@ -74,60 +73,33 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(const BwdParams p) {
     }
 }
 
-// --------------------------------------------------------------------------------------- convert
-template <int D>
-__global__ __launch_bounds__(256) void bwd_dq_convert_kernel(const BwdParams p) {
-    constexpr int TPR = D / 8;
-    constexpr int RPB = 256 / TPR;
-    const int tid = threadIdx.x;
-    const int64_t row_flat = (int64_t)blockIdx.x * RPB + tid / TPR;
-    const int chunk = tid % TPR;
-    if (row_flat >= (int64_t)p.B * p.H * p.Sq) return;
-    const int row = (int)(row_flat % p.Sq);
-    const int bh = (int)(row_flat / p.Sq);
-    const int b = bh / p.H, hh = bh % p.H;
-    const f32x4* src = reinterpret_cast<const f32x4*>(p.dq_acc + row_flat * D + chunk * 8);
-    const f32x4 x = src[0], y = src[1];
-    const float s = p.scale;
-    u32x4 w = {pack_bf16(x[0] * s, x[1] * s), pack_bf16(x[2] * s, x[3] * s), pack_bf16(y[0] * s, y[1] * s),
-               pack_bf16(y[2] * s, y[3] * s)};
-    *reinterpret_cast<u32x4*>(p.dq + b * p.dqs.b + hh * p.dqs.h + (int64_t)row * p.dqs.n + chunk * 8) = w;
-}
-
-// ------------------------------------------------------------------------------------------ main
+// ------------------------------------------------------------------------------------------ dkdv
 template <int D>
 struct BwdTile {
     static constexpr int BM = 64;                   // query rows per step
     static constexpr int BN = 128;                  // keys per workgroup
     static constexpr int RS = D;                    // LDS row stride of the Q / dO / K / V tiles (swizzled, unpadded)
-    static constexpr int DSS = BM;                  // LDS row stride of dS^T [key][query] (swizzled, unpadded)
     static constexpr int Q_ELEMS = BM * RS;
     static constexpr int STAGE_ELEMS = 2 * Q_ELEMS;               // Q tile + dO tile (also one 128-row tile)
-    static constexpr int DS_ELEMS = BN * DSS;
-    static constexpr int K_ELEMS = BN * RS;                       // resident K tile
     static constexpr int ROW_FLOATS = 2 * BM;                     // lse2 + delta of one step
-    // [2 stages of Q,dO][2 dS^T buffers][resident K][2 x (lse2, delta)]
-    static constexpr int LDS_BYTES = (2 * STAGE_ELEMS + 2 * DS_ELEMS + K_ELEMS) * 2 + 2 * ROW_FLOATS * 4;
+    // [2 stages of Q,dO][2 x (lse2, delta)]
+    static constexpr int LDS_BYTES = 2 * STAGE_ELEMS * 2 + 2 * ROW_FLOATS * 4;
     static constexpr int ROWS_PER_DMA = 1024 / (D * 2);
     static constexpr int DMA_PER_WAVE = BM / ROWS_PER_DMA / 4;    // 1 KiB copies per wave and tensor
 };
 
 template <int D, bool HASMASK, bool TIMING>
-__global__ __launch_bounds__(256) void bwd_kernel(const BwdParams p) {
+__global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
     using T = BwdTile<D>;
-    constexpr int BM = T::BM, BN = T::BN, RS = T::RS, DSS = T::DSS;
+    constexpr int BM = T::BM, BN = T::BN, RS = T::RS;
     constexpr int DC = D / 16;     // contraction chunks over the head dim
     constexpr int DB = D / 32;     // 32-row blocks of dK^T / dV^T
-    constexpr int NSL = D / 32;    // 32-column slices of dQ
-    constexpr int QB_PER = 2 / (4 / NSL);   // query blocks per wave in the dQ step
     constexpr int GPR = D / 8;     // 16-byte granules per row
     constexpr int RPD = T::ROWS_PER_DMA, NDQ = T::DMA_PER_WAVE;
 
     extern __shared__ __attribute__((aligned(1024))) uint16_t lds[];
     uint16_t* stage0 = lds;                                        // [2][Q tile | dO tile]
-    uint16_t* dst0 = lds + 2 * T::STAGE_ELEMS;                     // [2][BN][DSS]
-    uint16_t* Kres = dst0 + 2 * T::DS_ELEMS;                       // [BN][RS]
-    float* rows0 = reinterpret_cast<float*>(Kres + T::K_ELEMS);    // [2][lse2 | delta]
+    float* rows0 = reinterpret_cast<float*>(lds + 2 * T::STAGE_ELEMS);   // [2][lse2 | delta]
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -147,7 +119,6 @@ __global__ __launch_bounds__(256) void bwd_kernel(const BwdParams p) {
     const uint16_t* dobase = p.dout + b * p.dos.b + hh * p.dos.h;
     const float* lsebase = p.lse2 + (int64_t)bh * p.Sq;
     const float* deltabase = p.delta + (int64_t)bh * p.Sq;
-    float* dqacc_base = p.dq_acc + (int64_t)bh * p.Sq * D;
 
     int klimit = p.Sk;
     if (p.m.kv_len) klimit = min(klimit, max(p.m.kv_len[b], 0));
@@ -169,16 +140,12 @@ __global__ __launch_bounds__(256) void bwd_kernel(const BwdParams p) {
     for (int dc = 0; dc < DC; ++dc) roff[dc] = n * RS + (((2 * dc + h) ^ swz<D>(n)) << 3);
     const int tr_r = lane & 15, tr_g16 = (lane >> 4) & 1;
     int toff[2][DB];       // transposing reads of a D-wide tile: rows 4h + r/4 (+8), granule 4*db + 2*g16 + (r&3)/2
-    int soff[2][2];        // transposing reads of dS^T (64 wide): granule 4*qb + 2*g16 + (r&3)/2
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
         const int row = 4 * h + (tr_r >> 2) + 8 * half;
 #pragma unroll
         for (int db = 0; db < DB; ++db)
             toff[half][db] = row * RS + (((4 * db + 2 * tr_g16 + ((tr_r & 3) >> 1)) ^ swz<D>(row)) << 3) + 4 * (tr_r & 1);
-#pragma unroll
-        for (int qb = 0; qb < 2; ++qb)
-            soff[half][qb] = row * DSS + (((4 * qb + 2 * tr_g16 + ((tr_r & 3) >> 1)) ^ swz<64>(row)) << 3) + 4 * (tr_r & 1);
     }
     auto tr_frag = [&](const uint16_t* tile, int o0, int o1) {
         const u32x2 lo = lds_read_tr16(tile + o0);
@@ -189,8 +156,7 @@ __global__ __launch_bounds__(256) void bwd_kernel(const BwdParams p) {
 
     const int dma_row_in = lane / GPR, dma_gran = lane % GPR;
 
-    // ---- prologue: K tile stays resident in LDS (B operand of the dQ step); the K and V fragments
-    //      of this wavefront's 32 keys are held in registers for the whole walk
+    // ---- prologue: the K and V fragments of this wavefront's 32 keys are held in registers for the whole walk
     bf16x8 kf[DC], vf[DC];
     {
         constexpr int NDMA = BN / RPD / 4;     // 1 KiB copies per wave for a 128-row tile
@@ -200,14 +166,14 @@ __global__ __launch_bounds__(256) void bwd_kernel(const BwdParams p) {
             const int row = ji * RPD + dma_row_in;
             const int key = max(min(k0 + row, klimit - 1), 0);   // rows past the attended range re-read a valid row
             const int c = dma_gran ^ swz<D>(row);
-            dma16(kbase + (int64_t)key * p.ks.n + c * 8, Kres + ji * 512);
+            dma16(kbase + (int64_t)key * p.ks.n + c * 8, stage0 + T::STAGE_ELEMS + ji * 512);
             dma16(vbase + (int64_t)key * p.vs.n + c * 8, stage0 + ji * 512);
         }
         wait_vm0();
         __syncthreads();
 #pragma unroll
         for (int dc = 0; dc < DC; ++dc) {
-            kf[dc] = *reinterpret_cast<const bf16x8*>(Kres + roff[dc] + 32 * wave * RS);
+            kf[dc] = *reinterpret_cast<const bf16x8*>(stage0 + T::STAGE_ELEMS + roff[dc] + 32 * wave * RS);
             vf[dc] = *reinterpret_cast<const bf16x8*>(stage0 + roff[dc] + 32 * wave * RS);
         }
         __syncthreads();
@@ -264,13 +230,7 @@ __global__ __launch_bounds__(256) void bwd_kernel(const BwdParams p) {
         }
 
     const float c_log2 = p.scale * kLog2e;
-    const int dslice = wave % NSL;
-    const int qb_first = (wave / NSL) * QB_PER;
     const int key = kw0 + n;
-    // dQ accumulator offsets of this lane (floats): d column 32*dslice + n, query rows 8g + 4h + t
-    int dq_lane_off[4];
-#pragma unroll
-    for (int g = 0; g < 4; ++g) dq_lane_off[g] = (8 * g + 4 * h) * D + 32 * dslice + n;
 
     unsigned long long ph[6] = {0, 0, 0, 0, 0, 0};
     unsigned long long tprev = TIMING ? __builtin_readcyclecounter() : 0ull;
@@ -293,7 +253,6 @@ __global__ __launch_bounds__(256) void bwd_kernel(const BwdParams p) {
 
         const uint16_t* Qs = stage0 + buf * T::STAGE_ELEMS;
         const uint16_t* dOs = Qs + T::Q_ELEMS;
-        uint16_t* dSt = dst0 + buf * T::DS_ELEMS;
         const float* lse_s = rows0 + buf * T::ROW_FLOATS;
         const float* delta_s = lse_s + BM;
 
@@ -370,23 +329,6 @@ __global__ __launch_bounds__(256) void bwd_kernel(const BwdParams p) {
         if (need_mask) elementwise(std::true_type{});
         else elementwise(std::false_type{});
 
-        // dS^T[key][query]: four consecutive queries per 8-byte store, granule 4*qb + j, half h
-        {
-            const int krow = 32 * wave + n;
-            uint16_t* drow = dSt + krow * DSS + 4 * h;
-            const int f = swz<64>(krow);
-#pragma unroll
-            for (int qb = 0; qb < 2; ++qb) {
-                const u32x4 dsu0 = __builtin_bit_cast(u32x4, dsf[qb][0]);
-                const u32x4 dsu1 = __builtin_bit_cast(u32x4, dsf[qb][1]);
-                u32x2 w0 = {dsu0[0], dsu0[1]}, w1 = {dsu0[2], dsu0[3]}, w2 = {dsu1[0], dsu1[1]}, w3 = {dsu1[2], dsu1[3]};
-                *reinterpret_cast<u32x2*>(drow + (((4 * qb + 0) ^ f) << 3)) = w0;
-                *reinterpret_cast<u32x2*>(drow + (((4 * qb + 1) ^ f) << 3)) = w1;
-                *reinterpret_cast<u32x2*>(drow + (((4 * qb + 2) ^ f) << 3)) = w2;
-                *reinterpret_cast<u32x2*>(drow + (((4 * qb + 3) ^ f) << 3)) = w3;
-            }
-        }
-
         FATTN_PHASE(1)
         // ---- dV^T += dO^T P,  dK^T += Q^T dS : rows = d, columns = keys, contraction over the 64 queries
         {
@@ -410,59 +352,10 @@ __global__ __launch_bounds__(256) void bwd_kernel(const BwdParams p) {
         }
 
         FATTN_PHASE(2)
-        wait_vm0();        // the other stage (copy issued one step ago) has landed; older dQ atomics are done
+        wait_vm0();        // the other stage (copy issued one step ago) has landed
         FATTN_PHASE(3)
-        __syncthreads();   // dS^T of this step complete; every wave is done reading this step's stage
+        __syncthreads();   // ... for every wave, and every wave is done reading this step's stage
         FATTN_PHASE(4)
-
-        // ---- dQ[query][d slice] += dS K : contraction over the 128 keys of the workgroup
-        {
-            f32x16 dq[QB_PER];
-#pragma unroll
-            for (int i = 0; i < QB_PER; ++i)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) dq[i][r] = 0.f;
-            constexpr int NK = BN / 16;
-            // fragment stream per key chunk: K^T slice, then dS of each query block
-            constexpr int PER = 1 + QB_PER, NF = NK * PER, PD = 3;
-            bf16x8 fb[PD];
-            auto rd = [&](int i) {
-                const int kc = i / PER, j = i % PER;
-                if (j == 0) return tr_frag(Kres, toff[0][dslice] + 16 * kc * RS, toff[1][dslice] + 16 * kc * RS);
-                const int qb = qb_first + j - 1;
-                return tr_frag(dSt, soff[0][qb] + 16 * kc * DSS, soff[1][qb] + 16 * kc * DSS);
-            };
-            // query blocks are selected per wave at run time only through qb_first (0 or QB_PER)
-            bf16x8 kfrag;
-#pragma unroll
-            for (int i = 0; i < PD; ++i) fb[i] = rd(i);
-#pragma unroll
-            for (int i = 0; i < NF; ++i) {
-                const int j = i % PER;
-                if (j == 0) kfrag = fb[i % PD];
-                else dq[j - 1] = mfma32(fb[i % PD], kfrag, dq[j - 1]);
-                if (i + PD < NF) fb[i % PD] = rd(i + PD);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-#pragma unroll
-            for (int i = 0; i < QB_PER; ++i) {
-                const int qb = qb_first + i;
-                float* dst = dqacc_base + (int64_t)(q0 + 32 * qb) * D;     // uniform
-                if (q0 + BM <= p.Sq) {
-#pragma unroll
-                    for (int g = 0; g < 4; ++g)
-#pragma unroll
-                        for (int t = 0; t < 4; ++t) unsafeAtomicAdd(dst + dq_lane_off[g] + t * D, dq[i][4 * g + t]);
-                } else {
-#pragma unroll
-                    for (int g = 0; g < 4; ++g)
-#pragma unroll
-                        for (int t = 0; t < 4; ++t)
-                            if (q0 + 32 * qb + 8 * g + 4 * h + t < p.Sq)
-                                unsafeAtomicAdd(dst + dq_lane_off[g] + t * D, dq[i][4 * g + t]);
-                }
-            }
-        }
         // this step's stage is free (everyone passed the barrier): refill it two steps ahead
         if (it + 2 < n_it) issue_q_tile(tile_of(it + 2), buf);
         FATTN_PHASE(5)
@@ -490,6 +383,185 @@ __global__ __launch_bounds__(256) void bwd_kernel(const BwdParams p) {
                 u32x2 wv = {pack_bf16(c[4 * g], c[4 * g + 1]), pack_bf16(c[4 * g + 2], c[4 * g + 3])};
                 *reinterpret_cast<u32x2*>(dkrow + 32 * db + 8 * g + 4 * h) = wk;
                 *reinterpret_cast<u32x2*>(dvrow + 32 * db + 8 * g + 4 * h) = wv;
+            }
+    }
+}
+
+// -------------------------------------------------------------------------------------------- dq
+template <int D>
+struct BwdDqTile {
+    static constexpr int BM = 128;                  // query rows per workgroup (32 per wavefront)
+    static constexpr int BN = 64;                   // keys per tile
+    static constexpr int RS = D;
+    static constexpr int TILE_ELEMS = BN * D;
+    static constexpr int STAGE_ELEMS = 2 * TILE_ELEMS;            // K tile + V tile
+    static constexpr int LDS_BYTES = 2 * STAGE_ELEMS * 2;
+    static constexpr int ROWS_PER_DMA = 1024 / (D * 2);
+    static constexpr int DMA_PER_WAVE = BN / ROWS_PER_DMA / 4;
+};
+
+template <int D, bool HASMASK>
+__global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams p) {
+    using T = BwdDqTile<D>;
+    constexpr int BM = T::BM, BN = T::BN, RS = T::RS;
+    constexpr int DC = D / 16;
+    constexpr int DB = D / 32;
+    constexpr int GPR = D / 8;
+
+    extern __shared__ __attribute__((aligned(1024))) uint16_t lds[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int n = lane & 31, h = lane >> 5;
+
+    const int n_qt = (p.Sq + BM - 1) / BM;
+    const int wg = xcd_remap(blockIdx.x, gridDim.x);
+    const int qt = wg % n_qt;
+    const int bh = wg / n_qt;
+    const int b = bh / p.H, hh = bh % p.H;
+    const int q0 = qt * BM;
+    const int qw0 = q0 + wave * 32;
+
+    const uint16_t* qbase = p.q + b * p.qs.b + hh * p.qs.h;
+    const uint16_t* kbase = p.k + b * p.ks.b + hh * p.ks.h;
+    const uint16_t* vbase = p.v + b * p.vs.b + hh * p.vs.h;
+    const uint16_t* dobase = p.dout + b * p.dos.b + hh * p.dos.h;
+
+    int klimit = p.Sk;
+    if (p.m.kv_len) klimit = min(klimit, max(p.m.kv_len[b], 0));
+    int kend = klimit;
+    if (p.m.causal) kend = min(kend, q0 + BM);
+    const int n_tiles = (kend + BN - 1) / BN;
+    const uint8_t* mbase = HASMASK ? p.m.mask + b * p.m.sb + hh * p.m.sh : nullptr;
+
+    // ---- Q and dO fragments (B operands: column = query, 8 consecutive d), per-query scalars
+    const int qrow = qw0 + n;
+    const bool qok = qrow < p.Sq;
+    bf16x8 qf[DC], dof[DC];
+    {
+        const uint16_t* rq = qbase + (int64_t)qrow * p.qs.n + 8 * h;
+        const uint16_t* rd = dobase + (int64_t)qrow * p.dos.n + 8 * h;
+#pragma unroll
+        for (int dc = 0; dc < DC; ++dc) {
+            qf[dc] = __builtin_bit_cast(bf16x8, ldg16(rq + 16 * dc, qok));
+            dof[dc] = __builtin_bit_cast(bf16x8, ldg16(rd + 16 * dc, qok));
+        }
+    }
+    // rows past the end behave like fully excluded rows: lse2 = +inf gives P = 0
+    const float lse2 = qok ? p.lse2[(int64_t)bh * p.Sq + qrow] : INFINITY;
+    const float delta = qok ? p.delta[(int64_t)bh * p.Sq + qrow] : 0.f;
+
+    const int dma_row_in = lane / GPR, dma_gran = lane % GPR;
+    auto issue_tile = [&](int t, int buf) {
+        uint16_t* kdst = lds + buf * T::STAGE_ELEMS;
+        uint16_t* vdst = kdst + T::TILE_ELEMS;
+#pragma unroll
+        for (int i = 0; i < T::DMA_PER_WAVE; ++i) {
+            const int ji = wave * T::DMA_PER_WAVE + i;
+            const int row = ji * T::ROWS_PER_DMA + dma_row_in;
+            const int key = min(t * BN + row, klimit - 1);   // tail rows re-read the last attended key
+            const int c = dma_gran ^ swz<D>(row);
+            dma16(kbase + (int64_t)key * p.ks.n + c * 8, kdst + ji * 512);
+            dma16(vbase + (int64_t)key * p.vs.n + c * 8, vdst + ji * 512);
+        }
+    };
+
+    int koff[DC];          // 16-byte row reads of K / V: row 32*kb + n, logical granule 2*dc + h
+#pragma unroll
+    for (int dc = 0; dc < DC; ++dc) koff[dc] = n * RS + (((2 * dc + h) ^ swz<D>(n)) << 3);
+    const int tr_r = lane & 15, tr_g16 = (lane >> 4) & 1;
+    int toff[2][DB];       // transposing reads of K: rows 4h + r/4 (+8), logical granule 4*db + 2*g16 + (r&3)/2
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+        const int row = 4 * h + (tr_r >> 2) + 8 * half;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+            toff[half][db] = row * RS + (((4 * db + 2 * tr_g16 + ((tr_r & 3) >> 1)) ^ swz<D>(row)) << 3) + 4 * (tr_r & 1);
+    }
+
+    const float c_log2 = p.scale * kLog2e;
+    f32x16 dqacc[DB];      // dQ^T: rows = d, column = this lane's query
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dqacc[db][r] = 0.f;
+
+    if (n_tiles > 0) issue_tile(0, 0);
+    wait_vm0();
+    __syncthreads();
+
+    for (int t = 0; t < n_tiles; ++t) {
+        const int buf = t & 1;
+        if (t + 1 < n_tiles) issue_tile(t + 1, buf ^ 1);
+        const uint16_t* ks = lds + buf * T::STAGE_ELEMS;
+        const uint16_t* vs = ks + T::TILE_ELEMS;
+        const int key0 = t * BN;
+
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {       // two blocks of 32 keys per tile
+            // ---- S^T = K Q^T and dP^T = V dO^T : rows = keys, columns = queries
+            f32x16 sacc, dpacc;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                sacc[r] = 0.f;
+                dpacc[r] = 0.f;
+            }
+#pragma unroll
+            for (int dc = 0; dc < DC; ++dc) {
+                const bf16x8 ka = *reinterpret_cast<const bf16x8*>(ks + koff[dc] + 32 * kb * RS);
+                sacc = mfma32(ka, qf[dc], sacc);
+                const bf16x8 va = *reinterpret_cast<const bf16x8*>(vs + koff[dc] + 32 * kb * RS);
+                dpacc = mfma32(va, dof[dc], dpacc);
+            }
+            // ---- P^T and dS^T: one query per lane, so LSE and delta are per-lane scalars
+            const int kblk0 = key0 + 32 * kb;
+            const bool tail = kblk0 + 32 > klimit;
+            const bool diag = p.m.causal && (kblk0 + 31 > qw0);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                float pr = exp2_fast(fmaf(sacc[r], c_log2, -lse2));
+                if (tail || diag || HASMASK) {
+                    const int key = kblk0 + acc_row(r, h);
+                    bool drop = key >= klimit;
+                    if (p.m.causal) drop = drop || key > qrow;
+                    if (HASMASK) {
+                        if (!drop && qok) drop = mbase[(int64_t)qrow * p.m.sq + (int64_t)key * p.m.sk] == 0;
+                    }
+                    pr = drop ? 0.f : pr;
+                }
+                dpacc[r] = pr * (dpacc[r] - delta);
+            }
+            const bf16x8 ds0 = pack8(dpacc[0], dpacc[1], dpacc[2], dpacc[3], dpacc[4], dpacc[5], dpacc[6], dpacc[7]);
+            const bf16x8 ds1 = pack8(dpacc[8], dpacc[9], dpacc[10], dpacc[11], dpacc[12], dpacc[13], dpacc[14], dpacc[15]);
+            // ---- dQ^T += K^T dS^T : rows = d, columns = queries, contraction over the 32 keys
+#pragma unroll
+            for (int c = 0; c < 2; ++c) {
+                const int cc = 2 * kb + c;
+#pragma unroll
+                for (int db = 0; db < DB; ++db) {
+                    const u32x2 lo = lds_read_tr16(ks + toff[0][db] + 16 * cc * RS);
+                    const u32x2 hi = lds_read_tr16(ks + toff[1][db] + 16 * cc * RS);
+                    const u32x4 u = {lo[0], lo[1], hi[0], hi[1]};
+                    dqacc[db] = mfma32(__builtin_bit_cast(bf16x8, u), c == 0 ? ds0 : ds1, dqacc[db]);
+                }
+            }
+        }
+
+        wait_vm0();
+        __syncthreads();
+    }
+
+    // ---- epilogue: dQ = scale * dQ^T, bf16
+    if (qok) {
+        uint16_t* dqrow = p.dq + b * p.dqs.b + hh * p.dqs.h + (int64_t)qrow * p.dqs.n;
+        const float s = p.scale;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const f32x16& a = dqacc[db];
+                u32x2 w = {pack_bf16(a[4 * g] * s, a[4 * g + 1] * s), pack_bf16(a[4 * g + 2] * s, a[4 * g + 3] * s)};
+                *reinterpret_cast<u32x2*>(dqrow + 32 * db + 8 * g + 4 * h) = w;
             }
     }
 }

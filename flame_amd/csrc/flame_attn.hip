@@ -111,11 +111,16 @@ size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 template <int D, bool HASMASK, bool TIMING = false>
 int launch_bwd(const BwdParams& p, hipStream_t s) {
     using T = BwdTile<D>;
+    using TQ = BwdDqTile<D>;
     static bool attr_done = false;
-    auto kern = bwd_kernel<D, HASMASK, TIMING>;
+    auto kern = bwd_dkdv_kernel<D, HASMASK, TIMING>;
+    auto kern_dq = bwd_dq_kernel<D, HASMASK>;
     if (!attr_done) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS_BYTES);
+        if (e != hipSuccess) return (int)e;
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern_dq),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, TQ::LDS_BYTES);
         if (e != hipSuccess) return (int)e;
         attr_done = true;
     }
@@ -124,18 +129,20 @@ int launch_bwd(const BwdParams& p, hipStream_t s) {
     const int64_t row_blocks = (rows + RPB - 1) / RPB;
     const int64_t n_kt = (p.Sk + T::BN - 1) / T::BN;
     const int64_t grid = n_kt * p.B * p.H;
-    if (row_blocks > 0x7fffffff || grid > 0x7fffffff) return FLAME_ATTN_ERR_UNSUPPORTED;
+    const int64_t n_qt = (p.Sq + TQ::BM - 1) / TQ::BM;
+    const int64_t grid_dq = n_qt * p.B * p.H;
+    if (row_blocks > 0x7fffffff || grid > 0x7fffffff || grid_dq > 0x7fffffff) return FLAME_ATTN_ERR_UNSUPPORTED;
     {
         ScopedKernelTimer t(FLAME_ATTN_KERNEL_BWD_PREP, s);
         hipLaunchKernelGGL(bwd_prep_kernel<D>, dim3((unsigned)row_blocks), dim3(256), 0, s, p);
     }
     {
-        ScopedKernelTimer t(FLAME_ATTN_KERNEL_BWD_MAIN, s);
+        ScopedKernelTimer t(FLAME_ATTN_KERNEL_BWD_DKDV, s);
         hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), T::LDS_BYTES, s, p);
     }
     {
-        ScopedKernelTimer t(FLAME_ATTN_KERNEL_BWD_DQ_CONVERT, s);
-        hipLaunchKernelGGL(bwd_dq_convert_kernel<D>, dim3((unsigned)row_blocks), dim3(256), 0, s, p);
+        ScopedKernelTimer t(FLAME_ATTN_KERNEL_BWD_DQ, s);
+        hipLaunchKernelGGL(kern_dq, dim3((unsigned)grid_dq), dim3(256), TQ::LDS_BYTES, s, p);
     }
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? FLAME_ATTN_OK : (int)e;
@@ -180,7 +187,8 @@ int flame_attn_profiling_read(FlameAttnKernelTimes* out) {
 size_t flame_attn_bwd_workspace_bytes(int B, int H, int N_q, int D) {
     if (B <= 0 || H <= 0 || N_q <= 0 || D <= 0) return 0;
     const size_t rows = (size_t)B * H * N_q;
-    return 2 * align_up(rows * sizeof(float), 256) + rows * (size_t)D * sizeof(float);
+    (void)D;
+    return 2 * align_up(rows * sizeof(float), 256);
 }
 
 int flame_attn_bwd_bf16(const void* Q, const void* K, const void* V, const void* O, const void* dO,
@@ -224,7 +232,6 @@ int flame_attn_bwd_bf16(const void* Q, const void* K, const void* V, const void*
     const size_t rows = (size_t)B * H * N_q;
     p.delta = static_cast<float*>(workspace);
     p.lse2 = reinterpret_cast<float*>(static_cast<char*>(workspace) + align_up(rows * sizeof(float), 256));
-    p.dq_acc = reinterpret_cast<float*>(static_cast<char*>(workspace) + 2 * align_up(rows * sizeof(float), 256));
     p.qs = mk(q_strides); p.ks = mk(k_strides); p.vs = mk(v_strides); p.os = mk(o_strides);
     p.dos = mk(do_strides); p.dqs = mk(dq_strides); p.dks = mk(dk_strides); p.dvs = mk(dv_strides);
     p.B = B; p.H = H; p.Sq = N_q; p.Sk = N_kv;

@@ -9,8 +9,8 @@ extern "C" {
 #define FLAME_ATTN_OK 0
 #define FLAME_ATTN_ERR_INVALID (-1)
 #define FLAME_ATTN_ERR_UNSUPPORTED (-2)
-enum { FLAME_ATTN_KERNEL_FWD = 0, FLAME_ATTN_KERNEL_BWD_PREP = 1, FLAME_ATTN_KERNEL_BWD_MAIN = 2,
-       FLAME_ATTN_KERNEL_BWD_DQ_CONVERT = 3, FLAME_ATTN_KERNEL_SAGE_KMEAN = 4, FLAME_ATTN_KERNEL_SAGE_QUANT = 5,
+enum { FLAME_ATTN_KERNEL_FWD = 0, FLAME_ATTN_KERNEL_BWD_PREP = 1, FLAME_ATTN_KERNEL_BWD_DKDV = 2,
+       FLAME_ATTN_KERNEL_BWD_DQ = 3, FLAME_ATTN_KERNEL_SAGE_KMEAN = 4, FLAME_ATTN_KERNEL_SAGE_QUANT = 5,
        FLAME_ATTN_KERNEL_SAGE_FWD = 6, FLAME_ATTN_N_KERNEL_KINDS = 8 };
 typedef struct { double total_ms[FLAME_ATTN_N_KERNEL_KINDS]; int launches[FLAME_ATTN_N_KERNEL_KINDS]; } FlameAttnKernelTimes;
 int flame_attn_profiling_enable(int on);
