@@ -12,7 +12,7 @@ import os
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libflame_attn_hip.so")
+LIB_PATH = os.environ.get("FLAME_ATTN_LIB") or os.path.join(_HERE, "lib", "libflame_attn_hip.so")
 _lib = None
 
 OK, ERR_INVALID, ERR_UNSUPPORTED = 0, -1, -2

@@ -128,12 +128,24 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
     int qt_begin = p.m.causal ? (k0 / BM) : 0;
     if (k0 >= klimit) qt_begin = n_qt;        // nothing attends to these keys: dK = dV = 0
     const int n_it = n_qt - qt_begin;
-    // Workgroups of one head start their walk at different query tiles (and wrap around), so that at
-    // any moment they add into different rows of the dQ accumulator instead of contending for the
-    // same cache lines in L2.
-    const int rot = n_it > 0 ? (int)(((int64_t)kt * n_it) / n_kt) : 0;
-    auto tile_of = [&](int it) { int r = it + rot; if (r >= n_it) r -= n_it; return qt_begin + r; };
-
+    // The walk visits the query tiles that need per-element exclusions first (all of them when the key
+    // tile is ragged or an explicit mask is given, else the causal diagonal tiles and a partial last
+    // tile) and the fully attended ones afterwards, so that each of the two loops runs one
+    // specialised, branch-free body.  The order of the tiles does not matter to the sums.
+    const bool all_masked = HASMASK || (k0 + BN > klimit);
+    int lead_end = qt_begin;
+    if (n_it > 0) {
+        if (all_masked) lead_end = n_qt;
+        else if (p.m.causal) lead_end = max(qt_begin, min(n_qt, (k0 + BN - 2) / BM + 1));
+    }
+    const int n_lead = lead_end - qt_begin;
+    const int tail_extra = (n_it > 0 && !all_masked && (p.Sq % BM) != 0 && lead_end < n_qt) ? 1 : 0;
+    const int n_masked = n_lead + tail_extra;
+    auto tile_of = [&](int it) {
+        if (it < n_lead) return qt_begin + it;
+        if (it < n_masked) return n_qt - 1;
+        return lead_end + (it - n_masked);
+    };
     // ---- per-lane LDS offsets (elements), constant over the walk
     int roff[DC];          // 16-byte row reads: row (32*blk + n), logical granule 2*dc + h
 #pragma unroll
@@ -242,124 +254,186 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
     }
 
     if (n_it > 0) issue_q_tile(tile_of(0), 0);
-    if (n_it > 1) issue_q_tile(tile_of(1), 1);
     wait_vm0();
     __syncthreads();
 
-    for (int it = 0; it < n_it; ++it) {
+    // One step of the walk, written as an explicit software pipeline for a single wavefront per SIMD:
+    // the MFMA pipe and the vector ALU run side by side only when their instructions alternate in the
+    // instruction stream, so the per-element softmax / dS arithmetic of one 32-query block is
+    // threaded between the MFMAs of the neighbouring block, one accumulator register per MFMA:
+    //   A0: S,dP(block 0)                      | issue of the next tile's copies
+    //   A1: S,dP(block 1)                      | P,dS(block 0)
+    //   B0: dV,dK += (block 0)                 | P,dS(block 1)
+    //   B1: dV,dK += (block 1)
+    // LDS reads run PD fragments ahead of the MFMAs that consume them; the scheduling barriers keep the
+    // compiler from undoing either interleave.
+    // COPY: 0 = this is the last step, 1 = the next tile is a full one (straight-line copies),
+    //       2 = decide at run time (used by the few steps that need exclusions)
+    auto step = [&](auto masked_tag, auto copy_tag, int it) {
+        constexpr bool MASKED = decltype(masked_tag)::value;
+        constexpr int COPY = decltype(copy_tag)::value;
+        static_assert((2 * DC) % 4 == 0 && (4 * DB) % 4 == 0, "read-ahead depth must divide the fragment count");
         const int qt = tile_of(it);
         const int buf = it & 1;
         const int q0 = qt * BM;
+        const bool have_next = COPY == 1 || (COPY == 2 && it + 1 < n_it);
+        const int qt_next = have_next ? tile_of(it + 1) : qt;
 
         const uint16_t* Qs = stage0 + buf * T::STAGE_ELEMS;
         const uint16_t* dOs = Qs + T::Q_ELEMS;
         const float* lse_s = rows0 + buf * T::ROW_FLOATS;
         const float* delta_s = lse_s + BM;
 
-        // ---- S = Q K^T and dP = dO V^T : rows = queries (two blocks of 32), columns = this wave's keys
         f32x16 sacc[2], dpacc[2];
-#pragma unroll
-        for (int qb = 0; qb < 2; ++qb)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                sacc[qb][r] = 0.f;
-                dpacc[qb][r] = 0.f;
+        bf16x8 pf[2][2], dsf[2][2];
+        f32x4 l4, d4, l4n, d4n;
+        // the per-query rows are read one group of four queries ahead of their use, so that waiting
+        // for them never drains the fragment reads that were issued in between
+        auto rows_ahead = [&](int qb, int g) {
+            l4n = *reinterpret_cast<const f32x4*>(lse_s + 32 * qb + 8 * g + 4 * h);
+            d4n = *reinterpret_cast<const f32x4*>(delta_s + 32 * qb + 8 * g + 4 * h);
+        };
+
+        // element r of block qb: P = exp2(S*c - lse2), dS = P*(dP - delta); pack after 8 and 16
+        auto elem = [&](int qb, int r) {
+            const int g = r >> 2, t = r & 3;
+            if (t == 0) {
+                l4 = l4n;
+                d4 = d4n;
+                if (g < 3) rows_ahead(qb, g + 1);
+                else if (qb == 0) rows_ahead(1, 0);
             }
+            float pr = exp2_fast(fmaf(sacc[qb][r], c_log2, -l4[t]));
+            if (MASKED) {
+                const int qi = q0 + 32 * qb + 8 * g + 4 * h + t;
+                bool drop = key >= klimit || qi >= p.Sq;
+                if (p.m.causal) drop = drop || key > qi;
+                if (HASMASK) {
+                    if (!drop) drop = mbase[(int64_t)qi * p.m.sq + (int64_t)key * p.m.sk] == 0;
+                }
+                pr = drop ? 0.f : pr;
+            }
+            sacc[qb][r] = pr;
+            dpacc[qb][r] = pr * (dpacc[qb][r] - d4[t]);
+            if ((r & 7) == 7) {
+                const int c = r >> 3, o8 = 8 * c;
+                const f32x16& s = sacc[qb];
+                const f32x16& d = dpacc[qb];
+                pf[qb][c] = pack8(s[o8], s[o8 + 1], s[o8 + 2], s[o8 + 3], s[o8 + 4], s[o8 + 5], s[o8 + 6], s[o8 + 7]);
+                dsf[qb][c] = pack8(d[o8], d[o8 + 1], d[o8 + 2], d[o8 + 3], d[o8 + 4], d[o8 + 5], d[o8 + 6], d[o8 + 7]);
+            }
+        };
+
+        // copies of the next tile, one instruction at a time (full tiles: uniform base + lane offset)
+        const bool next_full = COPY == 1 || (qt_next * BM + BM) <= p.Sq;
+        const uint16_t* nq_base = qbase + (int64_t)qt_next * BM * p.qs.n;
+        const uint16_t* ndo_base = dobase + (int64_t)qt_next * BM * p.dos.n;
+        uint16_t* nq_dst = stage0 + (buf ^ 1) * T::STAGE_ELEMS;
+        auto copy_slice = [&](int j) {     // j in [0, 2*NDQ]
+            if (COPY == 0) return;
+            if (COPY == 2 && (!have_next || !next_full)) return;
+            if (j < 2 * NDQ) {
+                const int i = j >> 1, ji = wave * NDQ + i;
+                if (j & 1) dma16(ndo_base + do_lane_off[i], nq_dst + T::Q_ELEMS + ji * 512);
+                else dma16(nq_base + q_lane_off[i], nq_dst + ji * 512);
+            } else if (wave < 2) {
+                dma4((wave == 0 ? lsebase : deltabase) + qt_next * BM + lane,
+                     rows0 + (buf ^ 1) * T::ROW_FLOATS + wave * BM);
+            }
+        };
+        if (COPY == 2 && have_next && !next_full) issue_q_tile(qt_next, buf ^ 1);   // partial tile: slow path, all at once
+
+        // ---- phase A: S = Q K^T and dP = dO V^T, rows = queries of block qb, columns = this wave's keys
+        constexpr int NA = 2 * DC, PDA = 4;      // fragments per block: (dc, Q|dO); PDA divides NA
         {
-            // LDS reads run PD fragments ahead of the MFMAs that consume them; the scheduling barriers
-            // keep the compiler from sinking the reads back next to their uses (one wave per SIMD:
-            // nothing else hides the LDS latency).
-            constexpr int NF = 4 * DC, PD = 4;
-            bf16x8 fb[PD];
-            auto rd = [&](int i) {
-                const int dc = i >> 2, qb = (i >> 1) & 1;
+            bf16x8 fb[PDA];
+            auto rd = [&](int qb, int i) {
+                const int dc = i >> 1;
                 return *reinterpret_cast<const bf16x8*>(((i & 1) ? dOs : Qs) + roff[dc] + 32 * qb * RS);
             };
 #pragma unroll
-            for (int i = 0; i < PD; ++i) fb[i] = rd(i);
-#pragma unroll
-            for (int i = 0; i < NF; ++i) {
-                const int dc = i >> 2, qb = (i >> 1) & 1;
-                if (i & 1) dpacc[qb] = mfma32(fb[i % PD], vf[dc], dpacc[qb]);
-                else sacc[qb] = mfma32(fb[i % PD], kf[dc], sacc[qb]);
-                if (i + PD < NF) fb[i % PD] = rd(i + PD);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        }
-
-        FATTN_PHASE(0)
-        // ---- P and dS; lane = key column kw0+n, registers = queries
-        const bool need_mask = HASMASK || (k0 + BN > klimit) || (q0 + BM > p.Sq) || (p.m.causal && (k0 + BN - 1 > q0));
-        bf16x8 pf[2][2], dsf[2][2];
-        auto elementwise = [&](auto masked_tag) {
-            constexpr bool MASKED = decltype(masked_tag)::value;
-#pragma unroll
             for (int qb = 0; qb < 2; ++qb) {
 #pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const f32x4 l4 = *reinterpret_cast<const f32x4*>(lse_s + 32 * qb + 8 * g + 4 * h);
-                    const f32x4 d4 = *reinterpret_cast<const f32x4*>(delta_s + 32 * qb + 8 * g + 4 * h);
+                for (int r = 0; r < 16; ++r) {
+                    sacc[qb][r] = 0.f;
+                    dpacc[qb][r] = 0.f;
+                }
+                if (qb == 0) {
 #pragma unroll
-                    for (int t = 0; t < 4; ++t) {
-                        const int r = 4 * g + t;
-                        float pr = exp2_fast(fmaf(sacc[qb][r], c_log2, -l4[t]));
-                        if (MASKED) {
-                            const int qi = q0 + 32 * qb + 8 * g + 4 * h + t;
-                            bool drop = key >= klimit || qi >= p.Sq;
-                            if (p.m.causal) drop = drop || key > qi;
-                            if (HASMASK) {
-                                if (!drop) drop = mbase[(int64_t)qi * p.m.sq + (int64_t)key * p.m.sk] == 0;
-                            }
-                            pr = drop ? 0.f : pr;
-                        }
-                        sacc[qb][r] = pr;
-                        dpacc[qb][r] = pr * (dpacc[qb][r] - d4[t]);
+                    for (int i = 0; i < PDA; ++i) {
+                        fb[i] = rd(0, i);
+                        __builtin_amdgcn_sched_barrier(0);
                     }
+                    rows_ahead(0, 0);
                 }
 #pragma unroll
-                for (int c = 0; c < 2; ++c) {
-                    const f32x16& s = sacc[qb];
-                    const f32x16& d = dpacc[qb];
-                    const int o8 = 8 * c;
-                    pf[qb][c] = pack8(s[o8], s[o8 + 1], s[o8 + 2], s[o8 + 3], s[o8 + 4], s[o8 + 5], s[o8 + 6], s[o8 + 7]);
-                    dsf[qb][c] = pack8(d[o8], d[o8 + 1], d[o8 + 2], d[o8 + 3], d[o8 + 4], d[o8 + 5], d[o8 + 6], d[o8 + 7]);
+                for (int i = 0; i < NA; ++i) {
+                    const int dc = i >> 1;
+                    if (i & 1) dpacc[qb] = mfma32(fb[i % PDA], vf[dc], dpacc[qb]);
+                    else sacc[qb] = mfma32(fb[i % PDA], kf[dc], sacc[qb]);
+                    // refill: continue into the next block's fragments
+                    const int nxt = i + PDA;
+                    if (nxt < NA) fb[i % PDA] = rd(qb, nxt);
+                    else if (qb == 0) fb[i % PDA] = rd(1, nxt - NA);
+                    if (qb == 0) {
+                        if (i <= 2 * NDQ) copy_slice(i);
+                    } else {
+                        if (NA == 16) elem(0, i);
+                        else { elem(0, 2 * i); elem(0, 2 * i + 1); }
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
                 }
             }
-        };
-        if (need_mask) elementwise(std::true_type{});
-        else elementwise(std::false_type{});
+        }
+        FATTN_PHASE(0)
 
-        FATTN_PHASE(1)
-        // ---- dV^T += dO^T P,  dK^T += Q^T dS : rows = d, columns = keys, contraction over the 64 queries
+        // ---- phase B: dV^T += dO^T P, dK^T += Q^T dS, rows = d, columns = keys, contraction over queries
+        constexpr int NB = 4 * DB, PDB = 4;      // fragments per block: (16-query chunk, db, dO^T|Q^T); PDB divides NB
         {
-            constexpr int NF = 8 * DB, PD = 3;
-            bf16x8 fb[PD];
-            auto rd = [&](int i) {
-                const int db = (i >> 1) % DB, cc = i / (2 * DB);
+            bf16x8 fb[PDB];
+            auto rd = [&](int qb, int i) {
+                const int c = i / (2 * DB), db = (i >> 1) % DB, cc = 2 * qb + c;
                 return tr_frag((i & 1) ? Qs : dOs, toff[0][db] + 16 * cc * RS, toff[1][db] + 16 * cc * RS);
             };
 #pragma unroll
-            for (int i = 0; i < PD; ++i) fb[i] = rd(i);
+            for (int qb = 0; qb < 2; ++qb) {
+                if (qb == 0) {
 #pragma unroll
-            for (int i = 0; i < NF; ++i) {
-                const int db = (i >> 1) % DB, cc = i / (2 * DB);
-                const int qb = cc >> 1, c = cc & 1;
-                if (i & 1) dkacc[db] = mfma32(fb[i % PD], dsf[qb][c], dkacc[db]);
-                else dvacc[db] = mfma32(fb[i % PD], pf[qb][c], dvacc[db]);
-                if (i + PD < NF) fb[i % PD] = rd(i + PD);
-                __builtin_amdgcn_sched_barrier(0);
+                    for (int i = 0; i < PDB; ++i) {
+                        fb[i] = rd(0, i);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+#pragma unroll
+                for (int i = 0; i < NB; ++i) {
+                    const int c = i / (2 * DB), db = (i >> 1) % DB;
+                    if (i & 1) dkacc[db] = mfma32(fb[i % PDB], dsf[qb][c], dkacc[db]);
+                    else dvacc[db] = mfma32(fb[i % PDB], pf[qb][c], dvacc[db]);
+                    const int nxt = i + PDB;
+                    if (nxt < NB) fb[i % PDB] = rd(qb, nxt);
+                    else if (qb == 0) fb[i % PDB] = rd(1, nxt - NB);
+                    if (qb == 0) {
+                        if (NB == 16) elem(1, i);
+                        else { elem(1, 2 * i); elem(1, 2 * i + 1); }
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
         }
-
         FATTN_PHASE(2)
-        wait_vm0();        // the other stage (copy issued one step ago) has landed
+        wait_vm0();        // the other stage has landed
         FATTN_PHASE(3)
         __syncthreads();   // ... for every wave, and every wave is done reading this step's stage
         FATTN_PHASE(4)
-        // this step's stage is free (everyone passed the barrier): refill it two steps ahead
-        if (it + 2 < n_it) issue_q_tile(tile_of(it + 2), buf);
-        FATTN_PHASE(5)
-    }
+    };
+
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    using I2 = std::integral_constant<int, 2>;
+    for (int it = 0; it < n_masked; ++it) step(std::true_type{}, I2{}, it);
+    // every tile after the first n_masked is a full, fully attended one
+    for (int it = n_masked; it < n_it - 1; ++it) step(std::false_type{}, I1{}, it);
+    if (n_it > n_masked) step(std::false_type{}, I0{}, n_it - 1);
 
     if (TIMING && p.phase_cycles && tid == 0) {
 #pragma unroll
