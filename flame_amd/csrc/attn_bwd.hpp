@@ -526,6 +526,14 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams p) {
     const float delta = qok ? p.delta[(int64_t)bh * p.Sq + qrow] : 0.f;
 
     const int dma_row_in = lane / GPR, dma_gran = lane % GPR;
+    int k_lane_off[T::DMA_PER_WAVE], v_lane_off[T::DMA_PER_WAVE];
+#pragma unroll
+    for (int i = 0; i < T::DMA_PER_WAVE; ++i) {
+        const int row = (wave * T::DMA_PER_WAVE + i) * T::ROWS_PER_DMA + dma_row_in;
+        const int c = dma_gran ^ swz<D>(row);
+        k_lane_off[i] = row * (int)p.ks.n + c * 8;
+        v_lane_off[i] = row * (int)p.vs.n + c * 8;
+    }
     auto issue_tile = [&](int t, int buf) {
         uint16_t* kdst = lds + buf * T::STAGE_ELEMS;
         uint16_t* vdst = kdst + T::TILE_ELEMS;
@@ -537,6 +545,18 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams p) {
             const int c = dma_gran ^ swz<D>(row);
             dma16(kbase + (int64_t)key * p.ks.n + c * 8, kdst + ji * 512);
             dma16(vbase + (int64_t)key * p.vs.n + c * 8, vdst + ji * 512);
+        }
+    };
+    auto issue_full_tile = [&](int t, int buf) {
+        uint16_t* kdst = lds + buf * T::STAGE_ELEMS;
+        uint16_t* vdst = kdst + T::TILE_ELEMS;
+        const uint16_t* kt = kbase + (int64_t)t * BN * p.ks.n;
+        const uint16_t* vt = vbase + (int64_t)t * BN * p.vs.n;
+#pragma unroll
+        for (int i = 0; i < T::DMA_PER_WAVE; ++i) {
+            const int ji = wave * T::DMA_PER_WAVE + i;
+            dma16(kt + k_lane_off[i], kdst + ji * 512);
+            dma16(vt + v_lane_off[i], vdst + ji * 512);
         }
     };
 
@@ -564,9 +584,12 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams p) {
     wait_vm0();
     __syncthreads();
 
-    for (int t = 0; t < n_tiles; ++t) {
+    auto tile_step = [&](auto masked_tag, auto copy_tag, int t) {
+        constexpr bool MASKED = decltype(masked_tag)::value;
+        constexpr int COPY = decltype(copy_tag)::value;
         const int buf = t & 1;
-        if (t + 1 < n_tiles) issue_tile(t + 1, buf ^ 1);
+        if (COPY == 1) issue_full_tile(t + 1, buf ^ 1);
+        else if (t + 1 < n_tiles) issue_tile(t + 1, buf ^ 1);
         const uint16_t* ks = lds + buf * T::STAGE_ELEMS;
         const uint16_t* vs = ks + T::TILE_ELEMS;
         const int key0 = t * BN;
@@ -580,21 +603,32 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams p) {
                 sacc[r] = 0.f;
                 dpacc[r] = 0.f;
             }
+            {
+                constexpr int NF = 2 * DC, PD = 4;
+                bf16x8 fb[PD];
+                auto rd = [&](int i) {
+                    return *reinterpret_cast<const bf16x8*>(((i & 1) ? vs : ks) + koff[i >> 1] + 32 * kb * RS);
+                };
 #pragma unroll
-            for (int dc = 0; dc < DC; ++dc) {
-                const bf16x8 ka = *reinterpret_cast<const bf16x8*>(ks + koff[dc] + 32 * kb * RS);
-                sacc = mfma32(ka, qf[dc], sacc);
-                const bf16x8 va = *reinterpret_cast<const bf16x8*>(vs + koff[dc] + 32 * kb * RS);
-                dpacc = mfma32(va, dof[dc], dpacc);
+                for (int i = 0; i < PD; ++i) {
+                    fb[i] = rd(i);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+#pragma unroll
+                for (int i = 0; i < NF; ++i) {
+                    const int dc = i >> 1;
+                    if (i & 1) dpacc = mfma32(fb[i % PD], dof[dc], dpacc);
+                    else sacc = mfma32(fb[i % PD], qf[dc], sacc);
+                    if (i + PD < NF) fb[i % PD] = rd(i + PD);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
             // ---- P^T and dS^T: one query per lane, so LSE and delta are per-lane scalars
             const int kblk0 = key0 + 32 * kb;
-            const bool tail = kblk0 + 32 > klimit;
-            const bool diag = p.m.causal && (kblk0 + 31 > qw0);
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 float pr = exp2_fast(fmaf(sacc[r], c_log2, -lse2));
-                if (tail || diag || HASMASK) {
+                if (MASKED) {
                     const int key = kblk0 + acc_row(r, h);
                     bool drop = key >= klimit;
                     if (p.m.causal) drop = drop || key > qrow;
@@ -608,22 +642,43 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams p) {
             const bf16x8 ds0 = pack8(dpacc[0], dpacc[1], dpacc[2], dpacc[3], dpacc[4], dpacc[5], dpacc[6], dpacc[7]);
             const bf16x8 ds1 = pack8(dpacc[8], dpacc[9], dpacc[10], dpacc[11], dpacc[12], dpacc[13], dpacc[14], dpacc[15]);
             // ---- dQ^T += K^T dS^T : rows = d, columns = queries, contraction over the 32 keys
-#pragma unroll
-            for (int c = 0; c < 2; ++c) {
-                const int cc = 2 * kb + c;
-#pragma unroll
-                for (int db = 0; db < DB; ++db) {
+            {
+                constexpr int NF = 2 * DB, PD = 4;
+                bf16x8 fb[PD];
+                auto rd = [&](int i) {
+                    const int c = i / DB, db = i % DB, cc = 2 * kb + c;
                     const u32x2 lo = lds_read_tr16(ks + toff[0][db] + 16 * cc * RS);
                     const u32x2 hi = lds_read_tr16(ks + toff[1][db] + 16 * cc * RS);
                     const u32x4 u = {lo[0], lo[1], hi[0], hi[1]};
-                    dqacc[db] = mfma32(__builtin_bit_cast(bf16x8, u), c == 0 ? ds0 : ds1, dqacc[db]);
+                    return __builtin_bit_cast(bf16x8, u);
+                };
+#pragma unroll
+                for (int i = 0; i < PD && i < NF; ++i) {
+                    fb[i] = rd(i);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+#pragma unroll
+                for (int i = 0; i < NF; ++i) {
+                    const int c = i / DB, db = i % DB;
+                    dqacc[db] = mfma32(fb[i % PD], c == 0 ? ds0 : ds1, dqacc[db]);
+                    if (i + PD < NF) fb[i % PD] = rd(i + PD);
+                    __builtin_amdgcn_sched_barrier(0);
                 }
             }
         }
 
         wait_vm0();
         __syncthreads();
-    }
+    };
+
+    int n_full = HASMASK ? 0 : klimit / BN;
+    if (p.m.causal) n_full = min(n_full, (q0 + 1) / BN);
+    n_full = min(n_full, n_tiles);
+    using I1 = std::integral_constant<int, 1>;
+    using I2 = std::integral_constant<int, 2>;
+    for (int t = 0; t < n_full - 1; ++t) tile_step(std::false_type{}, I1{}, t);
+    if (n_full > 0) tile_step(std::false_type{}, I2{}, n_full - 1);
+    for (int t = n_full; t < n_tiles; ++t) tile_step(std::true_type{}, I2{}, t);
 
     // ---- epilogue: dQ = scale * dQ^T, bf16
     if (qok) {

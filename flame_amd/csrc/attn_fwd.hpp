@@ -11,6 +11,8 @@
 // second MFMA (O^T = V^T P^T), and the running rescale of O is a per-lane scalar that is skipped
 // while the running maximum stays within 2^8 of the reference maximum in use.
 #pragma once
+#include <type_traits>
+
 #include "attn_common.hpp"
 
 namespace fattn {
@@ -84,9 +86,18 @@ __global__ __launch_bounds__(256, (NWQ == 1 ? 2 : 1)) void fwd_kernel(const FwdP
         for (int dc = 0; dc < DC; ++dc) qf[qb][dc] = __builtin_bit_cast(bf16x8, ldg16(rp + 16 * dc, ok));
     }
 
-    // ---- asynchronous tile copies: this lane's source offsets (rows clamped into the attended range)
+    // ---- asynchronous tile copies.  Full tiles: uniform tile base + a per-lane 32-bit offset that
+    //      never changes; the ragged last tile clamps its rows into the attended range.
     const int dma_row_in = lane / GPR;                       // row inside one 1 KiB copy
     const int dma_gran = lane % GPR;                         // physical granule written by this lane
+    int k_lane_off[T::DMA_PER_WAVE], v_lane_off[T::DMA_PER_WAVE];
+#pragma unroll
+    for (int i = 0; i < T::DMA_PER_WAVE; ++i) {
+        const int row = (wave * T::DMA_PER_WAVE + i) * T::ROWS_PER_DMA + dma_row_in;
+        const int c = dma_gran ^ swz<D>(row);
+        k_lane_off[i] = row * (int)p.ks.n + c * 8;
+        v_lane_off[i] = row * (int)p.vs.n + c * 8;
+    }
     auto issue_tile = [&](int t, int buf) {
         uint16_t* kdst = lds + buf * T::STAGE_ELEMS;
         uint16_t* vdst = kdst + T::TILE_ELEMS;
@@ -98,6 +109,18 @@ __global__ __launch_bounds__(256, (NWQ == 1 ? 2 : 1)) void fwd_kernel(const FwdP
             const int c = dma_gran ^ swz<D>(row);
             dma16(kbase + (int64_t)key * p.ks.n + c * 8, kdst + ji * 512);
             dma16(vbase + (int64_t)key * p.vs.n + c * 8, vdst + ji * 512);
+        }
+    };
+    auto issue_full_tile = [&](int t, int buf) {
+        uint16_t* kdst = lds + buf * T::STAGE_ELEMS;
+        uint16_t* vdst = kdst + T::TILE_ELEMS;
+        const uint16_t* kt = kbase + (int64_t)t * BN * p.ks.n;
+        const uint16_t* vt = vbase + (int64_t)t * BN * p.vs.n;
+#pragma unroll
+        for (int i = 0; i < T::DMA_PER_WAVE; ++i) {
+            const int ji = wave * T::DMA_PER_WAVE + i;
+            dma16(kt + k_lane_off[i], kdst + ji * 512);
+            dma16(vt + v_lane_off[i], vdst + ji * 512);
         }
     };
 
@@ -134,15 +157,21 @@ __global__ __launch_bounds__(256, (NWQ == 1 ? 2 : 1)) void fwd_kernel(const FwdP
     wait_vm0();
     __syncthreads();
 
-    for (int t = 0; t < n_tiles; ++t) {
+    // One key tile.  MASKED: the tile needs per-element exclusions (ragged tail, causal diagonal,
+    // explicit mask).  COPY: 1 = the next tile is a full one (straight-line copies), 2 = decide at run time.
+    auto tile_step = [&](auto masked_tag, auto copy_tag, int t) {
+        constexpr bool MASKED = decltype(masked_tag)::value;
+        constexpr int COPY = decltype(copy_tag)::value;
         const int buf = t & 1;
-        if (t + 1 < n_tiles) issue_tile(t + 1, buf ^ 1);
+        if (COPY == 1) issue_full_tile(t + 1, buf ^ 1);
+        else if (t + 1 < n_tiles) issue_tile(t + 1, buf ^ 1);
 
         const uint16_t* ks = lds + buf * T::STAGE_ELEMS;
         const uint16_t* vs = ks + T::TILE_ELEMS;
         const int key0 = t * BN;
 
-        // ---- S^T = K Q^T : rows = keys (two blocks of 32), columns = queries
+        // ---- S^T = K Q^T : rows = keys (two blocks of 32), columns = queries.  K fragments are read
+        //      PD ahead of the MFMAs that consume them.
         f32x16 sacc[NWQ][2];
 #pragma unroll
         for (int qb = 0; qb < NWQ; ++qb)
@@ -150,20 +179,27 @@ __global__ __launch_bounds__(256, (NWQ == 1 ? 2 : 1)) void fwd_kernel(const FwdP
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) sacc[qb][kb][r] = 0.f;
+        {
+            constexpr int NF = 2 * DC, PD = 4;
+            bf16x8 fb[PD];
+            auto rd = [&](int i) { return *reinterpret_cast<const bf16x8*>(ks + koff[i >> 1] + 32 * (i & 1) * RS); };
 #pragma unroll
-        for (int dc = 0; dc < DC; ++dc) {
+            for (int i = 0; i < PD; ++i) {
+                fb[i] = rd(i);
+                __builtin_amdgcn_sched_barrier(0);
+            }
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
-                const bf16x8 ka = *reinterpret_cast<const bf16x8*>(ks + koff[dc] + 32 * kb * RS);
+            for (int i = 0; i < NF; ++i) {
+                const int dc = i >> 1, kb = i & 1;
 #pragma unroll
-                for (int qb = 0; qb < NWQ; ++qb) sacc[qb][kb] = mfma32(ka, qf[qb][dc], sacc[qb][kb]);
+                for (int qb = 0; qb < NWQ; ++qb) sacc[qb][kb] = mfma32(fb[i % PD], qf[qb][dc], sacc[qb][kb]);
+                if (i + PD < NF) fb[i % PD] = rd(i + PD);
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
 
         // ---- exclusions: ragged tail / key length, causal, explicit keep-mask
-        const bool tail = key0 + BN > klimit;
-        const bool diag = p.m.causal && (key0 + BN - 1 > qw0);
-        if (tail || diag || HASMASK) {
+        if (MASKED) {
 #pragma unroll
             for (int qb = 0; qb < NWQ; ++qb) {
                 const int qi = qw0 + 32 * qb + n;
@@ -177,7 +213,7 @@ __global__ __launch_bounds__(256, (NWQ == 1 ? 2 : 1)) void fwd_kernel(const FwdP
                         if (HASMASK) {
                             if (!drop && qi < p.Sq) drop = mbase[(int64_t)qi * p.m.sq + (int64_t)key * p.m.sk] == 0;
                         }
-                        if (drop) sacc[qb][kb][r] = -INFINITY;
+                        sacc[qb][kb][r] = drop ? -INFINITY : sacc[qb][kb][r];   // select, not a divergent store
                     }
             }
         }
@@ -233,22 +269,45 @@ __global__ __launch_bounds__(256, (NWQ == 1 ? 2 : 1)) void fwd_kernel(const FwdP
         }
 
         // ---- O^T += V^T P^T : rows = d, columns = queries, contraction over the 64 keys
-#pragma unroll
-        for (int cc = 0; cc < 4; ++cc) {
-#pragma unroll
-            for (int db = 0; db < DB; ++db) {
+        {
+            constexpr int NF = 4 * DB, PD = 4;
+            bf16x8 fb[PD];
+            auto rd = [&](int i) {
+                const int cc = i / DB, db = i % DB;
                 const u32x2 lo = lds_read_tr16(vs + voff[0][db] + 16 * cc * RS);
                 const u32x2 hi = lds_read_tr16(vs + voff[1][db] + 16 * cc * RS);
                 const u32x4 u = {lo[0], lo[1], hi[0], hi[1]};
-                const bf16x8 va = __builtin_bit_cast(bf16x8, u);
+                return __builtin_bit_cast(bf16x8, u);
+            };
 #pragma unroll
-                for (int qb = 0; qb < NWQ; ++qb) oacc[qb][db] = mfma32(va, pf[qb][cc], oacc[qb][db]);
+            for (int i = 0; i < PD; ++i) {
+                fb[i] = rd(i);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int i = 0; i < NF; ++i) {
+                const int cc = i / DB, db = i % DB;
+#pragma unroll
+                for (int qb = 0; qb < NWQ; ++qb) oacc[qb][db] = mfma32(fb[i % PD], pf[qb][cc], oacc[qb][db]);
+                if (i + PD < NF) fb[i % PD] = rd(i + PD);
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
 
         wait_vm0();          // next tile has landed in the other buffer
         __syncthreads();     // ... for every wave, and everyone is done reading this one
-    }
+    };
+
+    // Tiles [0, n_full) need no exclusions for any query of the workgroup; the rest (ragged tail, causal
+    // diagonal, or everything under an explicit mask) run the specialised masked body.
+    int n_full = HASMASK ? 0 : klimit / BN;
+    if (p.m.causal) n_full = min(n_full, (q0 + 1) / BN);
+    n_full = min(n_full, n_tiles);
+    using I1 = std::integral_constant<int, 1>;
+    using I2 = std::integral_constant<int, 2>;
+    for (int t = 0; t < n_full - 1; ++t) tile_step(std::false_type{}, I1{}, t);
+    if (n_full > 0) tile_step(std::false_type{}, I2{}, n_full - 1);
+    for (int t = n_full; t < n_tiles; ++t) tile_step(std::true_type{}, I2{}, t);
 
     // ---- epilogue
 #pragma unroll

@@ -314,7 +314,8 @@ __global__ __launch_bounds__(256) void sage_fwd_kernel(const SageFwdParams p) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int key = key0 + 32 * kb + acc_row(r, h);
-                    if (key >= klimit || (p.causal && key > qi)) sacc[kb][r] = -INFINITY;
+                    const bool drop = key >= klimit || (p.causal && key > qi);
+                    sacc[kb][r] = drop ? -INFINITY : sacc[kb][r];
                 }
         }
 
