@@ -393,4 +393,184 @@ int flame_attn_fwd_bf16(const void* Q, const void* K, const void* V, void* O, vo
     return launch_fwd<64, 1, false>(p, s);
 }
 
+
+// ------------------------------------------------------------------------------------------------
+// Entry points with the names and argument lists of the reference's FFI for this path.  They are
+// thin shims onto flame_attn_fwd_bf16 / flame_attn_bwd_bf16.
+// ------------------------------------------------------------------------------------------------
+
+int flame_cudnn_sdpa_bf16(const void* Q, const void* K, const void* V, void* O,
+                          int B, int H, int N_q, int N_kv, int D, float scale,
+                          const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                          const int64_t* o_strides,
+                          int64_t q_offset_elems, int64_t k_offset_elems, int64_t v_offset_elems,
+                          int64_t o_offset_elems, void* stream) {
+    return flame_attn_fwd_bf16(Q, K, V, O, nullptr, B, H, N_q, N_kv, D, scale, q_strides, k_strides, v_strides,
+                               o_strides, q_offset_elems, k_offset_elems, v_offset_elems, o_offset_elems, 0,
+                               0, nullptr, nullptr, nullptr, stream);
+}
+
+int flame_cudnn_sdpa_bf16_train_fwd(const void* Q, const void* K, const void* V, void* O, void* Stats,
+                                    int B, int H, int N_q, int N_kv, int D, float scale,
+                                    const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                                    const int64_t* o_strides,
+                                    int64_t q_offset_elems, int64_t k_offset_elems, int64_t v_offset_elems,
+                                    int64_t o_offset_elems, int64_t stats_offset_elems, void* stream) {
+    if (!Stats) return FLAME_ATTN_ERR_INVALID;
+    return flame_attn_fwd_bf16(Q, K, V, O, Stats, B, H, N_q, N_kv, D, scale, q_strides, k_strides, v_strides,
+                               o_strides, q_offset_elems, k_offset_elems, v_offset_elems, o_offset_elems,
+                               stats_offset_elems, 0, nullptr, nullptr, nullptr, stream);
+}
+
+}  // extern "C"
+
+namespace {
+// Scratch for the reference-signature backward, which has no workspace argument: one lazily grown
+// buffer per device (the reference's shim likewise keeps a workspace it allocated once per shape).
+// Calls that overlap on one device share it and therefore race; callers that need concurrency or
+// graph capture from the first call use flame_attn_bwd_bf16 with their own workspace.
+struct BwdScratch {
+    std::mutex mu;
+    void* ptr[64] = {};
+    size_t bytes[64] = {};
+};
+BwdScratch g_bwd_scratch;
+
+int bwd_scratch_get(size_t need, void** out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= 64) return FLAME_ATTN_ERR_UNSUPPORTED;
+    std::lock_guard<std::mutex> g(g_bwd_scratch.mu);
+    if (g_bwd_scratch.bytes[dev] < need) {
+        if (g_bwd_scratch.ptr[dev]) {
+            e = hipFree(g_bwd_scratch.ptr[dev]);      // synchronises: earlier users are done
+            if (e != hipSuccess) return (int)e;
+            g_bwd_scratch.ptr[dev] = nullptr;
+            g_bwd_scratch.bytes[dev] = 0;
+        }
+        e = hipMalloc(&g_bwd_scratch.ptr[dev], need);
+        if (e != hipSuccess) return (int)e;
+        g_bwd_scratch.bytes[dev] = need;
+    }
+    *out = g_bwd_scratch.ptr[dev];
+    return FLAME_ATTN_OK;
+}
+
+// bf16 keep-mask (>= 0.5 attends) -> uint8 keep-mask, contiguous
+__global__ void mask_bf16_to_u8_kernel(const uint16_t* src, uint8_t* dst, int64_t n, int invert) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const bool ge_half = __builtin_bit_cast(float, (uint32_t)src[i] << 16) >= 0.5f;
+    dst[i] = (ge_half != (invert != 0)) ? 1 : 0;
+}
+}  // namespace
+
+extern "C" {
+
+int flame_cudnn_sdpa_bwd_bf16(const void* Q, const void* K, const void* V, const void* O, const void* dO,
+                              const void* Stats, void* dQ, void* dK, void* dV,
+                              int B, int H, int N_q, int N_kv, int D, float scale,
+                              const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                              const int64_t* o_strides, const int64_t* do_strides, const int64_t* dq_strides,
+                              const int64_t* dk_strides, const int64_t* dv_strides,
+                              int64_t q_offset_elems, int64_t k_offset_elems, int64_t v_offset_elems,
+                              int64_t o_offset_elems, int64_t do_offset_elems, int64_t stats_offset_elems,
+                              int64_t dq_offset_elems, int64_t dk_offset_elems, int64_t dv_offset_elems,
+                              void* stream) {
+    const size_t need = flame_attn_bwd_workspace_bytes(B, H, N_q, D);
+    if (need == 0) return FLAME_ATTN_ERR_INVALID;
+    void* ws = nullptr;
+    int rc = bwd_scratch_get(need, &ws);
+    if (rc) return rc;
+    return flame_attn_bwd_bf16(Q, K, V, O, dO, Stats, dQ, dK, dV, B, H, N_q, N_kv, D, scale, q_strides, k_strides,
+                               v_strides, o_strides, do_strides, dq_strides, dk_strides, dv_strides, q_offset_elems,
+                               k_offset_elems, v_offset_elems, o_offset_elems, do_offset_elems, stats_offset_elems,
+                               dq_offset_elems, dk_offset_elems, dv_offset_elems, 0, nullptr, nullptr, nullptr, ws,
+                               need, stream);
+}
+
+int flame_flash_attention_bf16(const void* Q, const void* K, const void* V, void* O, float* LSE,
+                               int batch_heads, int seq_len_q, int seq_len_kv, int head_dim, void* stream) {
+    if (batch_heads <= 0 || seq_len_q <= 0 || seq_len_kv <= 0 || head_dim <= 0) return FLAME_ATTN_ERR_INVALID;
+    const int64_t qs[4] = {(int64_t)seq_len_q * head_dim, (int64_t)seq_len_q * head_dim, head_dim, 1};
+    const int64_t ks[4] = {(int64_t)seq_len_kv * head_dim, (int64_t)seq_len_kv * head_dim, head_dim, 1};
+    return flame_attn_fwd_bf16(Q, K, V, O, LSE, batch_heads, 1, seq_len_q, seq_len_kv, head_dim,
+                               1.0f / sqrtf((float)head_dim), qs, ks, ks, qs, 0, 0, 0, 0, 0, 0, nullptr, nullptr,
+                               nullptr, stream);
+}
+
+static FlameAttnStatus to_status(int rc) {
+    if (rc == FLAME_ATTN_OK) return FLAME_ATTN_STATUS_OK;
+    if (rc == FLAME_ATTN_ERR_INVALID) return FLAME_ATTN_STATUS_ERR_INVALID;
+    if (rc == FLAME_ATTN_ERR_UNSUPPORTED) return FLAME_ATTN_STATUS_ERR_UNSUPPORTED;
+    return FLAME_ATTN_STATUS_ERR_HIP;
+}
+
+FlameAttnStatus flame_sdpa_chunked_bf16(const void* q, const void* k, const void* v, int B, int H, int Q, int K,
+                                        int Dh, int Dv, float scale, int chunk, int causal, int mask_heads,
+                                        const void* mask, void* out, void* workspace, uint64_t workspace_bytes,
+                                        void* stream) {
+    if (!q || !k || !v || !out) return FLAME_ATTN_STATUS_ERR_INVALID;
+    if (B <= 0 || H <= 0 || Q < 0 || K < 0 || Dh <= 0 || Dv <= 0) return FLAME_ATTN_STATUS_ERR_INVALID;
+    if (Q == 0 || K == 0) return FLAME_ATTN_STATUS_OK;
+    if (chunk <= 0) return FLAME_ATTN_STATUS_ERR_INVALID;
+    if (Dv != Dh) return FLAME_ATTN_STATUS_ERR_UNSUPPORTED;
+    const int64_t qs[4] = {(int64_t)H * Q * Dh, (int64_t)Q * Dh, Dh, 1};
+    const int64_t ks[4] = {(int64_t)H * K * Dh, (int64_t)K * Dh, Dh, 1};
+    const uint8_t* m8 = nullptr;
+    int64_t ms[4] = {0, 0, 0, 0};
+    if (mask) {
+        if (mask_heads != 1 && mask_heads != H) return FLAME_ATTN_STATUS_ERR_INVALID;
+        const int64_t n = (int64_t)B * mask_heads * Q * K;
+        if (!workspace || workspace_bytes < (uint64_t)n) return FLAME_ATTN_STATUS_ERR_UNSUPPORTED;
+        hipLaunchKernelGGL(mask_bf16_to_u8_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
+                           static_cast<hipStream_t>(stream), static_cast<const uint16_t*>(mask),
+                           static_cast<uint8_t*>(workspace), n, 0);
+        m8 = static_cast<const uint8_t*>(workspace);
+        ms[0] = (int64_t)mask_heads * Q * K;
+        ms[1] = mask_heads == 1 ? 0 : (int64_t)Q * K;
+        ms[2] = K;
+        ms[3] = 1;
+    }
+    return to_status(flame_attn_fwd_bf16(q, k, v, out, nullptr, B, H, Q, K, Dh, scale, qs, ks, ks, qs, 0, 0, 0, 0, 0,
+                                         causal, nullptr, m8, m8 ? ms : nullptr, stream));
+}
+
+int streaming_attn_bf16_fp32_launch(const void* Q, const void* K, const void* V, int B, int H, int S, int Dh, int Dv,
+                                    long qB, long qH, long qS, long qD, long kB, long kH, long kS, long kD,
+                                    long vB, long vH, long vS, long vD, void* O, long oB, long oH, long oS, long oD,
+                                    float scale, int chunk_size, int causal, const uint8_t* k_pad_mask,
+                                    void* stream) {
+    if (chunk_size <= 0) return FLAME_ATTN_ERR_INVALID;
+    if (Dv != Dh) return FLAME_ATTN_ERR_UNSUPPORTED;
+    const int64_t qs[4] = {qB, qH, qS, qD}, ks[4] = {kB, kH, kS, kD}, vs[4] = {vB, vH, vS, vD}, os[4] = {oB, oH, oS, oD};
+    const int64_t ms[4] = {(int64_t)H * S, S, 0, 1};     // [B,H,S] key-padding mask, 0 = excluded
+    return flame_attn_fwd_bf16(Q, K, V, O, nullptr, B, H, S, S, Dh, scale, qs, ks, vs, os, 0, 0, 0, 0, 0, causal,
+                               nullptr, k_pad_mask, k_pad_mask ? ms : nullptr, stream);
+}
+
+bool sdpa_stream_bf16_launch(const void* dQ, const void* dK, const void* dV, void* dO, int B, int H, int Q_len,
+                             int K_len, int d, float scale, const void* attn_mask, int64_t mask_stride_ek,
+                             int64_t mask_stride_eq, int64_t mask_stride_eh, int64_t mask_stride_eb, int head_tile,
+                             int q_tile, int max_q_tile, void* stream, char* unsupported_reason, int reason_buflen) {
+    auto fail = [&](const char* why) {
+        if (unsupported_reason && reason_buflen > 0) snprintf(unsupported_reason, (size_t)reason_buflen, "%s", why);
+        return false;
+    };
+    (void)mask_stride_ek; (void)mask_stride_eq; (void)mask_stride_eh; (void)mask_stride_eb; (void)head_tile;
+    if (q_tile > max_q_tile) return fail("q_tile exceeds max_q_tile");
+    if (attn_mask) return fail("bf16 masks are not taken here: pass a uint8 keep-mask to flame_attn_fwd_bf16");
+    if (d != 64 && d != 128) return fail("head dim must be 64 or 128");
+    const int64_t qs[4] = {(int64_t)H * Q_len * d, (int64_t)Q_len * d, d, 1};
+    const int64_t ks[4] = {(int64_t)H * K_len * d, (int64_t)K_len * d, d, 1};
+    const int rc = flame_attn_fwd_bf16(dQ, dK, dV, dO, nullptr, B, H, Q_len, K_len, d, scale, qs, ks, ks, qs, 0, 0, 0,
+                                       0, 0, 0, nullptr, nullptr, nullptr, stream);
+    if (rc != FLAME_ATTN_OK) return fail(rc == FLAME_ATTN_ERR_INVALID ? "invalid argument" : "unsupported shape or HIP error");
+    if (unsupported_reason && reason_buflen > 0) unsupported_reason[0] = 0;
+    return true;
+}
+
+const char* flame_attn_version(void) { return "flame-attn-gfx950 0.1"; }
+
 }  // extern "C"

@@ -1,20 +1,66 @@
-/* placeholder while the kernels come up; replaced by the full header */
+/*
+ * flame_attn.h -- C ABI of libflame_attn_hip.so, the gfx950 (MI355X) implementation of the
+ * activation-memory-saving attention path of flame-core.
+ *
+ * What the library is: tiled QK^T -> online softmax -> PV forward that writes O and the per-row
+ * log-sum-exp (never the Sq x Sk matrix), a backward that recomputes P tile by tile to form
+ * dQ, dK, dV, and a SageAttention int8-QK inference forward.  Hand-written HIP for gfx950 only.
+ *
+ * Conventions shared by every entry point
+ *   - tensors are device pointers owned by the caller; nothing is retained or freed by the callee
+ *   - bf16 tensors are 4-D [B, H, N, D]; `*_strides` are four ELEMENT strides in (B, H, N, D) order,
+ *     `*_off` / `*_offset_elems` are element offsets added to the base pointer.  The D stride must
+ *     be 1, the other strides and the offsets multiples of 8 (16-byte rows), N strides below 2^24.
+ *     This admits the DiT view reshape([B,N,H,D]).permute(0,2,1,3) without a copy
+ *     (reference: src/sdpa.rs:607-621, :646-651).
+ *   - D is 64 or 128; anything else returns FLAME_ATTN_ERR_UNSUPPORTED.
+ *   - LSE / Stats: fp32, contiguous [B*H, N_q] (== [B,H,N_q,1] with strides [H*N_q, N_q, 1, 1]),
+ *     value = max_j s_ij + ln(sum_j exp(s_ij - max)), s = scale * Q K^T, natural log
+ *     (reference: src/cuda/cudnn_sdpa.cpp:271-279, src/sdpa.rs:715-722).  A row with no attended
+ *     key has LSE = -inf, O = 0 and zero gradients.
+ *   - exclusions: `causal` excludes key j > query i (absolute indices, reference
+ *     kernels/sdpa_kernels.cu:129-135); `kv_len` (int32 [B] on the device, may be null) excludes keys
+ *     j >= kv_len[b]; `keep_mask` (uint8 on the device, may be null, non-zero = attend, reference
+ *     src/sdpa.rs:458-470) is addressed with four element strides over (b, h, q, k), 0 = broadcast.
+ *   - `stream` is a hipStream_t passed as void*; null = the default stream.  Every call only
+ *     enqueues kernels: no host synchronisation, and no allocation except where stated.
+ *   - return value: 0 on success, FLAME_ATTN_ERR_INVALID (-1) for null pointers / non-positive
+ *     sizes / non-positive scale (reference: src/cuda/cudnn_sdpa.cpp:326-328),
+ *     FLAME_ATTN_ERR_UNSUPPORTED (-2) for layouts or head sizes that are not built, otherwise the
+ *     positive hipError_t of a failed launch.  Nothing is printed and nothing is thrown.
+ */
 #ifndef FLAME_ATTN_H
 #define FLAME_ATTN_H
+
+#include <stdbool.h>
 #include <stddef.h>
 #include <stdint.h>
+
 #ifdef __cplusplus
 extern "C" {
 #endif
+
 #define FLAME_ATTN_OK 0
 #define FLAME_ATTN_ERR_INVALID (-1)
 #define FLAME_ATTN_ERR_UNSUPPORTED (-2)
-enum { FLAME_ATTN_KERNEL_FWD = 0, FLAME_ATTN_KERNEL_BWD_PREP = 1, FLAME_ATTN_KERNEL_BWD_DKDV = 2,
-       FLAME_ATTN_KERNEL_BWD_DQ = 3, FLAME_ATTN_KERNEL_SAGE_KMEAN = 4, FLAME_ATTN_KERNEL_SAGE_QUANT = 5,
-       FLAME_ATTN_KERNEL_SAGE_FWD = 6, FLAME_ATTN_N_KERNEL_KINDS = 8 };
-typedef struct { double total_ms[FLAME_ATTN_N_KERNEL_KINDS]; int launches[FLAME_ATTN_N_KERNEL_KINDS]; } FlameAttnKernelTimes;
-int flame_attn_profiling_enable(int on);
-int flame_attn_profiling_read(FlameAttnKernelTimes* out);
+
+/* Status enum of the reference's flame_* / fc_* family (cuda/include/flame_cuda_status.h:7-12). */
+typedef enum {
+    FLAME_ATTN_STATUS_OK = 0,
+    FLAME_ATTN_STATUS_ERR_INVALID = 1,
+    FLAME_ATTN_STATUS_ERR_UNSUPPORTED = 2,
+    FLAME_ATTN_STATUS_ERR_HIP = 3
+} FlameAttnStatus;
+
+/* ------------------------------------------------------------------------------------------------
+ * Primary entry points (extensions of the reference trio: causal flag, key lengths, keep-mask,
+ * caller-provided workspace).
+ * ---------------------------------------------------------------------------------------------- */
+
+/* Forward.  LSE may be null (inference).  Replaces flame_cudnn_sdpa_bf16 /
+ * flame_cudnn_sdpa_bf16_train_fwd (src/cuda/ffi.rs:609-666), flame_flash_attention_bf16
+ * (src/cuda/ffi.rs:584-595) and the streaming / chunked fallbacks (src/cuda_ops_ffi.rs:199-221,
+ * src/ffi/cuda_ffi.h:98-115, cuda/streaming_attn_bf16.h:7-17). */
 int flame_attn_fwd_bf16(const void* Q, const void* K, const void* V, void* O, void* LSE,
                         int B, int H, int N_q, int N_kv, int D, float scale,
                         const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
@@ -23,15 +69,16 @@ int flame_attn_fwd_bf16(const void* Q, const void* K, const void* V, void* O, vo
                         int causal, const int32_t* kv_len,
                         const uint8_t* keep_mask, const int64_t* mask_strides,
                         void* stream);
-int flame_sage_quant_qk_int8(const void* Q, const void* K, int B, int H, int N_q, int N_kv, int D,
-                             const int64_t* q_strides, const int64_t* k_strides, int64_t q_off, int64_t k_off,
-                             int smooth_k, void* Qi8, void* Ki8, void* q_scales, void* k_scales, void* k_mean,
-                             void* stream);
-int flame_sage_attn_fwd_int8(const void* Qi8, const void* Ki8, const void* q_scales, const void* k_scales,
-                             const void* V, void* O, void* LSE, int B, int H, int N_q, int N_kv, int D,
-                             float scale, const int64_t* v_strides, const int64_t* o_strides,
-                             int64_t v_off, int64_t o_off, int causal, const int32_t* kv_len, void* stream);
+
+/* Bytes of device scratch the backward needs (two fp32 values per query row). */
 size_t flame_attn_bwd_workspace_bytes(int B, int H, int N_q, int D);
+
+/* Backward from Q, K, V, the saved O and LSE, and the upstream gradient dO (bf16).  Writes bf16
+ * dQ [B,H,N_q,D], dK, dV [B,H,N_kv,D] through their own strides.  `workspace` is 16-byte aligned
+ * device memory of at least flame_attn_bwd_workspace_bytes(...) bytes, used only during the call.
+ * Replaces flame_cudnn_sdpa_bwd_bf16 (src/cuda/ffi.rs:682-716) and the materialising recompute
+ * attention_backward_recompute (src/autograd.rs:801-848); follows the arithmetic of
+ * tests/cudnn_sdpa_bwd_parity.rs:31-98 with D_i = rowsum(dO * O). */
 int flame_attn_bwd_bf16(const void* Q, const void* K, const void* V, const void* O, const void* dO,
                         const void* LSE, void* dQ, void* dK, void* dV,
                         int B, int H, int N_q, int N_kv, int D, float scale,
@@ -43,7 +90,120 @@ int flame_attn_bwd_bf16(const void* Q, const void* K, const void* V, const void*
                         int causal, const int32_t* kv_len,
                         const uint8_t* keep_mask, const int64_t* mask_strides,
                         void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * SageAttention int8-QK inference variant (API shape: src/sage_attention.rs:21-65; quantiser closed
+ * form: src/sage_attention.rs:524-541; block granularity, K mean smoothing and int8 MFMA are new).
+ * ---------------------------------------------------------------------------------------------- */
+
+/* k_mean[b,h,c] = float(fp64 sum_t K[b,h,t,c] / N_kv) (0 when smooth_k == 0);
+ * Ks = bf16(float(K) - k_mean);  per 128-row block of Q and per 64-row block of Ks:
+ * scale = absmax / 127 (IEEE fp32 division), code = clamp(rint(x / scale), -128, 127), scale 0 -> 0.
+ * Outputs are contiguous: Qi8 [B,H,N_q,D], Ki8 [B,H,N_kv,D] int8; q_scales [B,H,ceil(N_q/128)],
+ * k_scales [B,H,ceil(N_kv/64)], k_mean [B,H,D] fp32. */
+int flame_sage_quant_qk_int8(const void* Q, const void* K, int B, int H, int N_q, int N_kv, int D,
+                             const int64_t* q_strides, const int64_t* k_strides, int64_t q_off, int64_t k_off,
+                             int smooth_k, void* Qi8, void* Ki8, void* q_scales, void* k_scales, void* k_mean,
+                             void* stream);
+
+/* S = float(int32 Q^ K^^T) * sq * sk * scale on int8 MFMA, online softmax fp32, P bf16, O = P V
+ * on bf16 MFMA.  LSE may be null. */
+int flame_sage_attn_fwd_int8(const void* Qi8, const void* Ki8, const void* q_scales, const void* k_scales,
+                             const void* V, void* O, void* LSE, int B, int H, int N_q, int N_kv, int D,
+                             float scale, const int64_t* v_strides, const int64_t* o_strides,
+                             int64_t v_off, int64_t o_off, int causal, const int32_t* kv_len, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Entry points with the reference's own names and argument lists: drop-in symbols for the
+ * declarations in src/cuda/ffi.rs, src/cuda_ops_ffi.rs, src/ffi/cuda_ffi.h and
+ * cuda/streaming_attn_bf16.h.  All are shims onto the primary entry points above.
+ * ---------------------------------------------------------------------------------------------- */
+
+/* src/cuda/ffi.rs:609-629 (implementation replaced: src/cuda/cudnn_sdpa.cpp:314-395). */
+int flame_cudnn_sdpa_bf16(const void* Q, const void* K, const void* V, void* O,
+                          int B, int H, int N_q, int N_kv, int D, float scale,
+                          const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                          const int64_t* o_strides,
+                          int64_t q_offset_elems, int64_t k_offset_elems, int64_t v_offset_elems,
+                          int64_t o_offset_elems, void* stream);
+
+/* src/cuda/ffi.rs:644-666 (src/cuda/cudnn_sdpa.cpp:405-484). */
+int flame_cudnn_sdpa_bf16_train_fwd(const void* Q, const void* K, const void* V, void* O, void* Stats,
+                                    int B, int H, int N_q, int N_kv, int D, float scale,
+                                    const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                                    const int64_t* o_strides,
+                                    int64_t q_offset_elems, int64_t k_offset_elems, int64_t v_offset_elems,
+                                    int64_t o_offset_elems, int64_t stats_offset_elems, void* stream);
+
+/* src/cuda/ffi.rs:682-716 (src/cuda/cudnn_sdpa_bwd.cpp:265-361).  The reference signature has no
+ * workspace argument: this shim keeps one lazily grown scratch buffer per device (hipMalloc on first
+ * use or growth, as the reference's shim does at src/cuda/cudnn_sdpa.cpp:204-212), so overlapping
+ * calls on one device race and the first call cannot be captured into a graph.  Use
+ * flame_attn_bwd_bf16 when either matters. */
+int flame_cudnn_sdpa_bwd_bf16(const void* Q, const void* K, const void* V, const void* O, const void* dO,
+                              const void* Stats, void* dQ, void* dK, void* dV,
+                              int B, int H, int N_q, int N_kv, int D, float scale,
+                              const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                              const int64_t* o_strides, const int64_t* do_strides, const int64_t* dq_strides,
+                              const int64_t* dk_strides, const int64_t* dv_strides,
+                              int64_t q_offset_elems, int64_t k_offset_elems, int64_t v_offset_elems,
+                              int64_t o_offset_elems, int64_t do_offset_elems, int64_t stats_offset_elems,
+                              int64_t dq_offset_elems, int64_t dk_offset_elems, int64_t dv_offset_elems,
+                              void* stream);
+
+/* src/cuda/ffi.rs:584-595 (src/cuda/flash_attention_fwd.cu:352-366): contiguous [BH,N,HD],
+ * scale = 1/sqrt(HD); LSE (may be null) is filled here, the reference left it unused. */
+int flame_flash_attention_bf16(const void* Q, const void* K, const void* V, void* O, float* LSE,
+                               int batch_heads, int seq_len_q, int seq_len_kv, int head_dim, void* stream);
+
+/* src/ffi/cuda_ffi.h:98-115 (cuda/src/flame_sdpa_stub.cu:869-1379): contiguous tensors, optional bf16
+ * keep-mask [B, mask_heads, Q, K] (< 0.5 excluded, flame_sdpa_stub.cu:793-802) which is converted to
+ * uint8 inside `workspace` (needs B*mask_heads*Q*K bytes there); Dv must equal Dh. */
+FlameAttnStatus flame_sdpa_chunked_bf16(const void* q, const void* k, const void* v, int B, int H, int Q, int K,
+                                        int Dh, int Dv, float scale, int chunk, int causal, int mask_heads,
+                                        const void* mask, void* out, void* workspace, uint64_t workspace_bytes,
+                                        void* stream);
+
+/* cuda/streaming_attn_bf16.h:7-17 (cuda/streaming_attn_bf16.cu:305-432): strided Q,K,V,O, causal,
+ * key-padding mask uint8 [B,H,S] with 0 = excluded (streaming_attn_bf16.cu:164-170). */
+int streaming_attn_bf16_fp32_launch(const void* Q, const void* K, const void* V, int B, int H, int S, int Dh, int Dv,
+                                    long qB, long qH, long qS, long qD, long kB, long kH, long kS, long kD,
+                                    long vB, long vH, long vS, long vD, void* O, long oB, long oH, long oS, long oD,
+                                    float scale, int chunk_size, int causal, const uint8_t* k_pad_mask,
+                                    void* stream);
+
+/* src/cuda_ops_ffi.rs:199-221 (cuda/sdpa_stream_bf16.cu:180-413): contiguous, d in {64,128}.  A bf16
+ * mask (where >= 0.5 means EXCLUDED in that one entry point, cuda/include/sdpa_stream_bf16.h:30-33)
+ * is reported as unsupported with a reason, which is the documented way for the caller to take its
+ * other path (src/cuda_ops_bf16.rs:1955-2059). */
+bool sdpa_stream_bf16_launch(const void* dQ, const void* dK, const void* dV, void* dO, int B, int H, int Q_len,
+                             int K_len, int d, float scale, const void* attn_mask, int64_t mask_stride_ek,
+                             int64_t mask_stride_eq, int64_t mask_stride_eh, int64_t mask_stride_eb, int head_tile,
+                             int q_tile, int max_q_tile, void* stream, char* unsupported_reason, int reason_buflen);
+
+/* ------------------------------------------------------------------------------------------------
+ * Profiling aids (the counterpart of the reference's SdpaStats / SdpaHooks timing fields,
+ * src/autograd_v4/ops/sdpa.rs:55-79).  No counterpart in the FFI of the reference.
+ * ---------------------------------------------------------------------------------------------- */
+enum { FLAME_ATTN_KERNEL_FWD = 0, FLAME_ATTN_KERNEL_BWD_PREP = 1, FLAME_ATTN_KERNEL_BWD_DKDV = 2,
+       FLAME_ATTN_KERNEL_BWD_DQ = 3, FLAME_ATTN_KERNEL_SAGE_KMEAN = 4, FLAME_ATTN_KERNEL_SAGE_QUANT = 5,
+       FLAME_ATTN_KERNEL_SAGE_FWD = 6, FLAME_ATTN_N_KERNEL_KINDS = 8 };
+typedef struct {
+    double total_ms[FLAME_ATTN_N_KERNEL_KINDS];
+    int launches[FLAME_ATTN_N_KERNEL_KINDS];
+} FlameAttnKernelTimes;
+/* When on, every kernel launch is bracketed by HIP events on the launch stream (events are created
+ * on demand: this mode allocates).  Turning it on or off clears the samples. */
+int flame_attn_profiling_enable(int on);
+/* Waits for the recorded events and returns per-kernel sums since the last read. */
+int flame_attn_profiling_read(FlameAttnKernelTimes* out);
+/* Device buffer of 6 uint64 per workgroup that the dK/dV kernel fills with per-phase cycle counts
+ * (null switches the timing build of the kernel off again). */
+int flame_attn_debug_set_phase_buffer(void* device_buffer);
+
+const char* flame_attn_version(void);
+
 #ifdef __cplusplus
 }
 #endif
-#endif
+#endif /* FLAME_ATTN_H */

@@ -1,0 +1,158 @@
+"""The entry points that keep the reference's own names and argument lists, called through ctypes the
+way the reference's FFI declarations bind them, checked against the primary entry points / the oracle."""
+import ctypes
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from flame_amd import workloads as W
+from tests.gpu_util import assert_close_bf16, to_dev, to_f32
+
+pytestmark = pytest.mark.gpu
+
+
+def _i64x4(v):
+    return (ctypes.c_int64 * 4)(*[int(x) for x in v])
+
+
+def _p(t):
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _z(n):
+    return [ctypes.c_int64(0)] * n
+
+
+def test_cudnn_named_trio_matches_reference_test_logic(oracle):
+    """Shapes and seeds of tests/cudnn_sdpa_bwd_parity.rs:311-320: (1,4,128,64) and (1,4,256,128);
+    train-forward O equals inference-forward O (ibid :250-308); grads against the fp32 recompute."""
+    from flame_amd import capi
+    lib = capi.lib()
+    for (B, H, N, D) in ((1, 4, 128, 64), (1, 4, 256, 128)):
+        t = [W.f32_to_bf16_bits(W.normal_f32(sd, 0, B * H * N * D).reshape(B, H, N, D)) for sd in (11, 22, 33, 44)]
+        q, k, v, do = (to_dev(x) for x in t)
+        scale = 1.0 / math.sqrt(D)
+        st = _i64x4(q.stride())
+        o_inf = torch.empty_like(q)
+        o_trn = torch.empty_like(q)
+        stats = torch.empty(B * H, N, dtype=torch.float32, device="cuda")
+        assert lib.flame_cudnn_sdpa_bf16(_p(q), _p(k), _p(v), _p(o_inf), B, H, N, N, D, ctypes.c_float(scale),
+                                         st, st, st, st, *_z(4), _stream()) == 0
+        assert lib.flame_cudnn_sdpa_bf16_train_fwd(_p(q), _p(k), _p(v), _p(o_trn), _p(stats), B, H, N, N, D,
+                                                   ctypes.c_float(scale), st, st, st, st, *_z(5), _stream()) == 0
+        assert torch.equal(o_inf, o_trn)
+        dq, dk, dv = (torch.empty_like(q) for _ in range(3))
+        assert lib.flame_cudnn_sdpa_bwd_bf16(_p(q), _p(k), _p(v), _p(o_trn), _p(do), _p(stats), _p(dq), _p(dk), _p(dv),
+                                             B, H, N, N, D, ctypes.c_float(scale), *([st] * 8), *_z(9), _stream()) == 0
+        torch.cuda.synchronize()
+        ro, rlse, ro32 = oracle.sdpa_fwd(t[0], t[1], t[2], scale, want_f32=True)
+        ref = oracle.sdpa_bwd(t[0], t[1], t[2], ro, t[3], scale, want_f32=True)
+        assert_close_bf16(oracle, "O", to_f32(o_trn), ro, ro32)
+        assert oracle.max_abs(stats.cpu().numpy().reshape(rlse.shape), rlse) <= 1e-3
+        for i, (name, g) in enumerate((("dQ", dq), ("dK", dk), ("dV", dv))):
+            assert_close_bf16(oracle, name, to_f32(g), ref[i], ref[i + 3])
+            # the reference's own gate (ibid :136-138): cosine >= 0.9999
+            assert oracle.cosine(to_f32(g), ref[i + 3]) >= 0.9999
+
+
+def test_flash_attention_symbol_fills_lse(oracle):
+    """Shapes of tests/fa2_parity_naive.rs:374-376 (N in {512}, HD in {64,128}, 8 heads)."""
+    from flame_amd import capi
+    lib = capi.lib()
+    for HD in (64, 128):
+        BH, N = 8, 512
+        t = [W.f32_to_bf16_bits(W.normal_f32(0xFA2 + HD, s, BH * N * HD).reshape(1, BH, N, HD)) for s in range(3)]
+        q, k, v = (to_dev(x) for x in t)
+        o = torch.empty_like(q)
+        lse = torch.empty(BH, N, dtype=torch.float32, device="cuda")
+        assert lib.flame_flash_attention_bf16(_p(q), _p(k), _p(v), _p(o), _p(lse), BH, N, N, HD, _stream()) == 0
+        torch.cuda.synchronize()
+        ro, rlse, ro32 = oracle.sdpa_fwd(t[0], t[1], t[2], 1.0 / math.sqrt(HD), want_f32=True)
+        ma, _ = assert_close_bf16(oracle, "O", to_f32(o), ro, ro32)
+        assert ma <= 1e-2 and oracle.cosine(to_f32(o), ro32) >= 0.9999        # the reference's gate (:369-370)
+        assert oracle.max_abs(lse.cpu().numpy().reshape(rlse.shape), rlse) <= 1e-3
+
+
+def test_chunked_symbol_with_bf16_keep_mask_and_causal(oracle):
+    from flame_amd import capi
+    lib = capi.lib()
+    lib.flame_sdpa_chunked_bf16.restype = ctypes.c_int
+    B, H, Q, K, D = 2, 3, 40, 100, 64
+    t = [W.f32_to_bf16_bits(W.normal_f32(321, s, B * H * n * D).reshape(B, H, n, D)) for s, n in enumerate((Q, K, K))]
+    q, k, v = (to_dev(x) for x in t)
+    keep = (W.normal_f32(322, 0, B * Q * K).reshape(B, 1, Q, K) > -0.2).astype(np.uint8)
+    keep[..., 0] = 1
+    mask_bf16 = torch.from_numpy(keep.astype(np.float32)).to(torch.bfloat16).cuda()
+    out = torch.empty_like(q)
+    ws = torch.empty(B * Q * K, dtype=torch.uint8, device="cuda")
+    rc = lib.flame_sdpa_chunked_bf16(_p(q), _p(k), _p(v), B, H, Q, K, D, D, ctypes.c_float(0.125), 64, 0, 1,
+                                     _p(mask_bf16), _p(out), _p(ws), ctypes.c_uint64(ws.numel()), _stream())
+    assert rc == 0
+    torch.cuda.synchronize()
+    ro, _, ro32 = oracle.sdpa_fwd(t[0], t[1], t[2], 0.125, mask=keep, want_f32=True)
+    assert_close_bf16(oracle, "O", to_f32(out), ro, ro32)
+    # causal, no mask
+    rc = lib.flame_sdpa_chunked_bf16(_p(q), _p(k), _p(v), B, H, Q, K, D, D, ctypes.c_float(0.125), 64, 1, 1,
+                                     None, _p(out), None, ctypes.c_uint64(0), _stream())
+    assert rc == 0
+    torch.cuda.synchronize()
+    ro, _, ro32 = oracle.sdpa_fwd(t[0], t[1], t[2], 0.125, causal=True, want_f32=True)
+    assert_close_bf16(oracle, "O", to_f32(out), ro, ro32)
+    # Dv != Dh -> unsupported (2), bad chunk -> invalid (1): status enum of cuda/include/flame_cuda_status.h
+    assert lib.flame_sdpa_chunked_bf16(_p(q), _p(k), _p(v), B, H, Q, K, D, 32, ctypes.c_float(0.125), 64, 0, 1,
+                                       None, _p(out), None, ctypes.c_uint64(0), _stream()) == 2
+    assert lib.flame_sdpa_chunked_bf16(_p(q), _p(k), _p(v), B, H, Q, K, D, D, ctypes.c_float(0.125), 0, 0, 1,
+                                       None, _p(out), None, ctypes.c_uint64(0), _stream()) == 1
+
+
+def test_streaming_symbol_causal_and_key_padding(oracle):
+    """Mirrors tests/streaming_attn.rs: small-sequence, causal, explicit key-padding mask."""
+    from flame_amd import capi
+    lib = capi.lib()
+    B, H, S, D = 2, 2, 150, 64
+    t = [W.f32_to_bf16_bits(W.normal_f32(555, s, B * H * S * D).reshape(B, H, S, D)) for s in range(3)]
+    q, k, v = (to_dev(x) for x in t)
+    o = torch.empty_like(q)
+    st = [ctypes.c_long(x) for x in q.stride()]
+    pad = (W.normal_f32(556, 0, B * H * S).reshape(B, H, S) > -0.5).astype(np.uint8)
+    pad[..., 0] = 1
+    padd = torch.from_numpy(pad).cuda()
+    for causal, mask in ((0, None), (1, None), (0, padd), (1, padd)):
+        rc = lib.streaming_attn_bf16_fp32_launch(_p(q), _p(k), _p(v), B, H, S, D, D, *st, *st, *st, _p(o), *st,
+                                                 ctypes.c_float(0.125), 128, causal, _p(mask), _stream())
+        assert rc == 0
+        torch.cuda.synchronize()
+        m4 = None if mask is None else pad.reshape(B, H, 1, S)
+        ro, _, ro32 = oracle.sdpa_fwd(t[0], t[1], t[2], 0.125, causal=bool(causal), mask=m4, want_f32=True)
+        assert_close_bf16(oracle, f"O causal={causal} mask={mask is not None}", to_f32(o), ro, ro32)
+    assert lib.streaming_attn_bf16_fp32_launch(_p(q), _p(k), _p(v), B, H, S, D, D, *st, *st, *st, _p(o), *st,
+                                               ctypes.c_float(0.125), 0, 0, None, _stream()) != 0
+
+
+def test_stream_symbol_reports_reason_when_unsupported(oracle):
+    from flame_amd import capi
+    lib = capi.lib()
+    lib.sdpa_stream_bf16_launch.restype = ctypes.c_bool
+    B, H, Q, K, D = 1, 2, 96, 200, 64
+    t = [W.f32_to_bf16_bits(W.normal_f32(777, s, B * H * n * D).reshape(B, H, n, D)) for s, n in enumerate((Q, K, K))]
+    q, k, v = (to_dev(x) for x in t)
+    o = torch.empty_like(q)
+    reason = ctypes.create_string_buffer(256)
+    ok = lib.sdpa_stream_bf16_launch(_p(q), _p(k), _p(v), _p(o), B, H, Q, K, D, ctypes.c_float(0.125), None,
+                                     *_z(4), 12, 96, 96, _stream(), reason, 256)
+    assert ok and reason.value == b""
+    torch.cuda.synchronize()
+    ro, _, ro32 = oracle.sdpa_fwd(t[0], t[1], t[2], 0.125, want_f32=True)
+    assert_close_bf16(oracle, "O", to_f32(o), ro, ro32)
+    ok = lib.sdpa_stream_bf16_launch(_p(q), _p(k), _p(v), _p(o), B, H, Q, K, D, ctypes.c_float(0.125), _p(q),
+                                     *_z(4), 12, 96, 96, _stream(), reason, 256)
+    assert not ok and b"mask" in reason.value
+    ok = lib.sdpa_stream_bf16_launch(_p(q), _p(k), _p(v), _p(o), B, H, Q, K, D, ctypes.c_float(0.125), None,
+                                     *_z(4), 12, 128, 96, _stream(), reason, 256)
+    assert not ok and b"q_tile" in reason.value
