@@ -36,5 +36,23 @@ def build_lib(verbose: bool = False, extra=()) -> str:
     return LIB_PATH
 
 
+
+
+def build_host_test(verbose: bool = False) -> str:
+    """Compiles the C++ host-layer test driver (tests/host/host_api_test.cpp) against the library."""
+    root = os.path.dirname(HERE)
+    src = os.path.join(root, "tests", "host", "host_api_test.cpp")
+    out = os.path.join(root, "tests", "host", "host_api_test")
+    cmd = [HIPCC, "--offload-arch=gfx950", "-O2", "-std=c++17", "-x", "hip", src, "-o", out,
+           "-L" + LIB_DIR, "-lflame_attn_hip", "-Wl,-rpath,$ORIGIN/../../flame_amd/lib"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + res.stdout)
+    return out
+
+
 if __name__ == "__main__":
     print(build_lib(verbose=True, extra=sys.argv[1:]))
+    print(build_host_test(verbose=True))

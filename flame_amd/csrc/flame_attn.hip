@@ -464,6 +464,14 @@ __global__ void mask_bf16_to_u8_kernel(const uint16_t* src, uint8_t* dst, int64_
     const bool ge_half = __builtin_bit_cast(float, (uint32_t)src[i] << 16) >= 0.5f;
     dst[i] = (ge_half != (invert != 0)) ? 1 : 0;
 }
+__global__ void mask_f32_to_u8_kernel(const float* src, uint8_t* dst, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) dst[i] = src[i] >= 0.5f ? 1 : 0;
+}
+__global__ void cast_f32_to_bf16_kernel(const float* src, uint16_t* dst, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) dst[i] = (uint16_t)(pack_bf16(src[i], 0.f) & 0xffffu);
+}
 }  // namespace
 
 extern "C" {
@@ -569,6 +577,33 @@ bool sdpa_stream_bf16_launch(const void* dQ, const void* dK, const void* dV, voi
     if (rc != FLAME_ATTN_OK) return fail(rc == FLAME_ATTN_ERR_INVALID ? "invalid argument" : "unsupported shape or HIP error");
     if (unsupported_reason && reason_buflen > 0) unsupported_reason[0] = 0;
     return true;
+}
+
+int flame_attn_convert_keep_mask(const void* src, int src_dtype, void* dst_u8, int64_t n, void* stream) {
+    if (!src || !dst_u8 || n <= 0) return FLAME_ATTN_ERR_INVALID;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const unsigned grid = (unsigned)((n + 255) / 256);
+    if (n > (int64_t)0x7fffffff * 256) return FLAME_ATTN_ERR_UNSUPPORTED;
+    if (src_dtype == FLAME_ATTN_DTYPE_BF16)
+        hipLaunchKernelGGL(mask_bf16_to_u8_kernel, dim3(grid), dim3(256), 0, s, static_cast<const uint16_t*>(src),
+                           static_cast<uint8_t*>(dst_u8), n, 0);
+    else if (src_dtype == FLAME_ATTN_DTYPE_F32)
+        hipLaunchKernelGGL(mask_f32_to_u8_kernel, dim3(grid), dim3(256), 0, s, static_cast<const float*>(src),
+                           static_cast<uint8_t*>(dst_u8), n);
+    else
+        return FLAME_ATTN_ERR_UNSUPPORTED;
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? FLAME_ATTN_OK : (int)e;
+}
+
+int flame_attn_cast_f32_to_bf16(const void* src_f32, void* dst_bf16, int64_t n, void* stream) {
+    if (!src_f32 || !dst_bf16 || n <= 0) return FLAME_ATTN_ERR_INVALID;
+    if (n > (int64_t)0x7fffffff * 256) return FLAME_ATTN_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(cast_f32_to_bf16_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), static_cast<const float*>(src_f32),
+                       static_cast<uint16_t*>(dst_bf16), n);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? FLAME_ATTN_OK : (int)e;
 }
 
 const char* flame_attn_version(void) { return "flame-attn-gfx950 0.1"; }

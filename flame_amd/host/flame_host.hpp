@@ -1,0 +1,534 @@
+// Host side of the attention path above the C ABI, in C++ (the reference's host side is Rust, for
+// which this environment has no toolchain).  It mirrors the reference's operator interface for this
+// path -- same names, argument meaning and error behaviour -- so that a Rust shim is a line-by-line
+// transliteration:
+//
+//   flame::sdpa::forward / forward_train            src/sdpa.rs:85-207
+//   flame::attention::sdpa / attend / attention_impl / build_causal_mask
+//                                                   src/attention/sdpa.rs:521-558, :395-458, :11-34
+//   flame::autograd::{AutogradContext, Op::FlashAttention node, flash_attention_backward}
+//                                                   src/autograd.rs:289-296, :672-795, :3824-3916
+//   flame::autograd_v4::{SdpaConfig, SdpaSave, SdpaCtx, sdpa_forward, sdpa_backward}
+//                                                   src/autograd_v4/ops/sdpa.rs:21-96, :98-326, :826-1009
+//   flame::SageAttention                            src/sage_attention.rs:21-171
+//
+// Only what the path needs of the tensor type is here: a reference-counted device buffer with a
+// shape, element strides, an offset and a dtype (the reference's Tensor supplies exactly these to
+// the FFI: src/tensor.rs:558, :2637, :2657).  Header-only; link against libflame_attn_hip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdint>
+#include <cstring>
+#include <memory>
+#include <mutex>
+#include <optional>
+#include <string>
+#include <tuple>
+#include <utility>
+#include <vector>
+
+#include "../../include/flame_attn.h"
+
+namespace flame {
+
+// ------------------------------------------------------------------------------------ errors
+// The reference's `Error` enum, reduced to the variants this path raises (src/error.rs).
+struct Error {
+    enum Kind { InvalidInput, Unsupported, Cuda } kind;
+    std::string message;
+};
+
+template <class T>
+class Result {
+   public:
+    Result(T v) : value_(std::move(v)) {}
+    Result(Error e) : error_(std::move(e)) {}
+    bool ok() const { return value_.has_value(); }
+    const T& value() const { return *value_; }
+    T& value() { return *value_; }
+    const Error& error() const { return *error_; }
+
+   private:
+    std::optional<T> value_;
+    std::optional<Error> error_;
+};
+
+inline Error invalid(std::string m) { return Error{Error::InvalidInput, std::move(m)}; }
+inline Error unsupported(std::string m) { return Error{Error::Unsupported, std::move(m)}; }
+inline Error cuda_error(const std::string& what, int code) {
+    return Error{Error::Cuda, what + " HIP error: " + std::to_string(code)};   // src/sdpa.rs:680-682
+}
+
+// ------------------------------------------------------------------------------------ tensor
+enum class DType { BF16, F32, U8, I8, I32 };
+inline size_t dtype_size(DType d) { return d == DType::BF16 ? 2 : (d == DType::U8 || d == DType::I8) ? 1 : 4; }
+
+class Tensor {
+   public:
+    Tensor() = default;
+
+    static Result<Tensor> empty(std::vector<int64_t> shape, DType dtype) {
+        int64_t n = 1;
+        for (auto d : shape) {
+            if (d <= 0) return invalid("empty: non-positive dimension");
+            n *= d;
+        }
+        void* p = nullptr;
+        hipError_t e = hipMalloc(&p, (size_t)n * dtype_size(dtype));
+        if (e != hipSuccess) return cuda_error("hipMalloc", (int)e);
+        Tensor t;
+        t.storage_ = std::shared_ptr<void>(p, [](void* q) { (void)hipFree(q); });
+        t.shape_ = std::move(shape);
+        t.strides_ = contiguous_strides(t.shape_);
+        t.dtype_ = dtype;
+        return t;
+    }
+    static Result<Tensor> from_host(const void* src, std::vector<int64_t> shape, DType dtype) {
+        auto r = empty(std::move(shape), dtype);
+        if (!r.ok()) return r;
+        hipError_t e = hipMemcpy(r.value().data(), src, (size_t)r.value().numel() * dtype_size(dtype), hipMemcpyHostToDevice);
+        if (e != hipSuccess) return cuda_error("hipMemcpy", (int)e);
+        return r;
+    }
+    // contiguous tensors only
+    Result<bool> to_host(void* dst) const {
+        if (!is_contiguous()) return unsupported("to_host: tensor is a strided view");
+        hipError_t e = hipMemcpy(dst, data(), (size_t)numel() * dtype_size(dtype_), hipMemcpyDeviceToHost);
+        if (e != hipSuccess) return cuda_error("hipMemcpy", (int)e);
+        return true;
+    }
+
+    const std::vector<int64_t>& shape() const { return shape_; }
+    const std::vector<int64_t>& strides() const { return strides_; }
+    int64_t offset() const { return offset_; }
+    DType dtype() const { return dtype_; }
+    int64_t numel() const {
+        int64_t n = 1;
+        for (auto d : shape_) n *= d;
+        return n;
+    }
+    void* base() const { return storage_.get(); }
+    void* data() const { return static_cast<char*>(storage_.get()) + offset_ * (int64_t)dtype_size(dtype_); }
+    bool defined() const { return storage_ != nullptr; }
+    uint64_t id() const { return (uint64_t)(uintptr_t)storage_.get() ^ ((uint64_t)offset_ << 1); }
+    bool requires_grad = false;
+
+    bool is_contiguous() const { return strides_ == contiguous_strides(shape_); }
+    // view with permuted dimensions (no copy), e.g. [B,N,H,D] -> [B,H,N,D] with {0,2,1,3}
+    Tensor permute(const std::vector<int>& order) const {
+        Tensor t = *this;
+        for (size_t i = 0; i < order.size(); ++i) {
+            t.shape_[i] = shape_[order[i]];
+            t.strides_[i] = strides_[order[i]];
+        }
+        return t;
+    }
+    Tensor reshape_contiguous(std::vector<int64_t> shape) const {
+        Tensor t = *this;
+        t.shape_ = std::move(shape);
+        t.strides_ = contiguous_strides(t.shape_);
+        return t;
+    }
+
+    static std::vector<int64_t> contiguous_strides(const std::vector<int64_t>& shape) {
+        std::vector<int64_t> st(shape.size(), 1);
+        for (int i = (int)shape.size() - 2; i >= 0; --i) st[i] = st[i + 1] * shape[i + 1];
+        return st;
+    }
+
+   private:
+    std::shared_ptr<void> storage_;
+    std::vector<int64_t> shape_, strides_;
+    int64_t offset_ = 0;
+    DType dtype_ = DType::BF16;
+};
+
+namespace detail {
+
+// trap_is_bf16 of the reference (src/tensor/contracts.rs:22-33): non-bf16 -> InvalidInput
+inline std::optional<Error> trap_is_bf16(const char* what, const Tensor& t) {
+    if (t.dtype() != DType::BF16) return invalid(std::string(what) + ": expected BF16 tensor");
+    return std::nullopt;
+}
+
+struct Dims {
+    int B, H, Sq, Sk, D;
+};
+
+// shape / mask validation of forward_inner (src/sdpa.rs:330-374), same messages' meaning
+inline Result<Dims> validate(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor* mask) {
+    for (const Tensor* t : {&q, &k, &v})
+        if (t->shape().size() != 4) return invalid("expected 4D tensor [B,H,S,D]");
+    const auto &qs = q.shape(), &ks = k.shape(), &vs = v.shape();
+    if (!(qs[0] == ks[0] && qs[0] == vs[0] && qs[1] == ks[1] && qs[1] == vs[1])) return invalid("batch/head mismatch");
+    if (!(qs[3] == ks[3] && qs[3] == vs[3])) return invalid("embed mismatch");
+    if (ks[2] != vs[2]) return invalid("sequence mismatch: k_len != v_len");
+    if (mask) {
+        const auto& ms = mask->shape();
+        if (ms.size() != 4) return invalid("mask must be 4D [B,H,Q,K]");
+        if (!(ms[0] == qs[0] || ms[0] == 1) || !(ms[1] == qs[1] || ms[1] == 1) || ms[2] != qs[2] || ms[3] != ks[2])
+            return invalid("mask dims not broadcastable to [B,H,Q,K]");
+    }
+    if (auto e = trap_is_bf16("sdpa.forward q", q)) return *e;
+    if (auto e = trap_is_bf16("sdpa.forward k", k)) return *e;
+    if (auto e = trap_is_bf16("sdpa.forward v", v)) return *e;
+    return Dims{(int)qs[0], (int)qs[1], (int)qs[2], (int)ks[2], (int)qs[3]};
+}
+
+inline bool abi_friendly(const Tensor& t) {
+    const auto& st = t.strides();
+    return st[3] == 1 && ((st[0] | st[1] | st[2] | t.offset()) & 7) == 0;
+}
+
+// binary keep-mask of any supported dtype -> contiguous uint8 keep-mask + broadcast strides
+inline Result<std::pair<Tensor, std::vector<int64_t>>> prepare_mask(const Tensor& mask, const Dims& d) {
+    Tensor m8 = mask;
+    if (mask.dtype() != DType::U8) {
+        if (!mask.is_contiguous()) return unsupported("non-contiguous non-uint8 mask");
+        if (mask.dtype() != DType::BF16 && mask.dtype() != DType::F32) return invalid("mask dtype must be U8, BF16 or F32");
+        auto r = Tensor::empty(mask.shape(), DType::U8);
+        if (!r.ok()) return r.error();
+        const int rc = flame_attn_convert_keep_mask(mask.data(), mask.dtype() == DType::BF16 ? FLAME_ATTN_DTYPE_BF16 : FLAME_ATTN_DTYPE_F32,
+                                                    r.value().data(), mask.numel(), nullptr);
+        if (rc != 0) return cuda_error("flame_attn_convert_keep_mask", rc);
+        m8 = r.value();
+    }
+    std::vector<int64_t> st(4);
+    const int64_t full[4] = {d.B, d.H, d.Sq, d.Sk};
+    for (int i = 0; i < 4; ++i) st[i] = (m8.shape()[i] == 1 && full[i] != 1) ? 0 : m8.strides()[i];
+    return std::make_pair(m8, st);
+}
+
+struct FwdOut {
+    Tensor o, stats;
+};
+
+inline Result<FwdOut> run_forward(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor* mask, bool causal,
+                                  std::optional<float> scale, bool want_stats) {
+    auto dv = validate(q, k, v, mask);
+    if (!dv.ok()) return dv.error();
+    const Dims d = dv.value();
+    for (const Tensor* t : {&q, &k, &v})
+        if (!abi_friendly(*t)) return unsupported("tensor view needs D stride 1 and 16-byte aligned rows; make it contiguous first");
+    auto o = Tensor::empty({d.B, d.H, d.Sq, d.D}, DType::BF16);      // O = q.shape, contiguous (src/sdpa.rs:631)
+    if (!o.ok()) return o.error();
+    Tensor stats;
+    if (want_stats) {
+        auto s = Tensor::empty({(int64_t)d.B * d.H, d.Sq}, DType::F32);   // [B*H, Sq] fp32 (src/sdpa.rs:712-722)
+        if (!s.ok()) return s.error();
+        stats = s.value();
+    }
+    Tensor m8;
+    std::vector<int64_t> mst;
+    if (mask) {
+        auto pm = prepare_mask(*mask, d);
+        if (!pm.ok()) return pm.error();
+        m8 = pm.value().first;
+        mst = pm.value().second;
+    }
+    const float sc = scale.value_or(1.0f / std::sqrt((float)d.D));
+    const int rc = flame_attn_fwd_bf16(q.base(), k.base(), v.base(), o.value().base(), want_stats ? stats.base() : nullptr,
+                                       d.B, d.H, d.Sq, d.Sk, d.D, sc, q.strides().data(), k.strides().data(),
+                                       v.strides().data(), o.value().strides().data(), q.offset(), k.offset(), v.offset(), 0, 0,
+                                       causal ? 1 : 0, nullptr, mask ? static_cast<const uint8_t*>(m8.data()) : nullptr,
+                                       mask ? mst.data() : nullptr, nullptr /* default stream, as the reference */);
+    if (rc == FLAME_ATTN_ERR_UNSUPPORTED) return unsupported("flame_attn_fwd_bf16: head dim or layout not built");
+    if (rc != 0) return cuda_error("flame_attn_fwd_bf16", rc);
+    return FwdOut{o.value(), stats};
+}
+
+}  // namespace detail
+
+// ------------------------------------------------------------------------------------ autograd (default engine)
+namespace autograd {
+
+// Op::FlashAttention and its saved set {Q, K, V, O, Stats(, mask)} (src/autograd.rs:289-296, src/sdpa.rs:170-201)
+struct FlashAttentionNode {
+    uint64_t output_id = 0;
+    Tensor query, key, value, output, stats;
+    std::optional<Tensor> mask;
+    float scale = 0.f;
+    bool causal = false;
+};
+
+class AutogradContext {
+   public:
+    static bool is_recording() { return state().recording; }
+    static void set_recording(bool on) { state().recording = on; }
+    static void record_op(FlashAttentionNode node) {
+        std::lock_guard<std::mutex> g(state().mu);
+        state().tape.push_back(std::move(node));
+    }
+    static std::optional<FlashAttentionNode> find(const Tensor& output) {
+        std::lock_guard<std::mutex> g(state().mu);
+        for (auto it = state().tape.rbegin(); it != state().tape.rend(); ++it)
+            if (it->output_id == output.id()) return *it;
+        return std::nullopt;
+    }
+    static void clear() {
+        std::lock_guard<std::mutex> g(state().mu);
+        state().tape.clear();
+    }
+    // bytes this node keeps alive between forward and backward that a materialised softmax would not
+    static size_t saved_activation_bytes(const FlashAttentionNode& n) {
+        return (size_t)n.output.numel() * 2 + (size_t)n.stats.numel() * 4;
+    }
+
+   private:
+    struct State {
+        bool recording = false;
+        std::mutex mu;
+        std::vector<FlashAttentionNode> tape;
+    };
+    static State& state() {
+        static State s;
+        return s;
+    }
+};
+
+struct AttentionGrads {
+    Tensor dq, dk, dv;
+};
+
+// The Op::FlashAttention backward arm (src/autograd.rs:3824-3916) with try_cudnn_sdpa_backward
+// (:672-795): contiguous bf16 dQ/dK/dV; an fp32 upstream gradient is cast to bf16 instead of
+// falling back to the materialising recompute (the reference bails out at :702-705).
+inline Result<AttentionGrads> flash_attention_backward(const FlashAttentionNode& n, const Tensor& grad_out) {
+    const auto& qs = n.query.shape();
+    const auto& ks = n.key.shape();
+    const int B = (int)qs[0], H = (int)qs[1], Sq = (int)qs[2], D = (int)qs[3], Sk = (int)ks[2];
+    if (grad_out.shape() != n.output.shape()) return invalid("grad_out shape does not match the attention output");
+    if (n.stats.dtype() != DType::F32 || n.stats.numel() != (int64_t)B * H * Sq)
+        return invalid("saved Stats must be fp32 [B*H, Sq]");       // found by dtype + shape, :3877-3885
+    Tensor g = grad_out;
+    if (g.dtype() == DType::F32) {
+        if (!g.is_contiguous()) return unsupported("strided fp32 grad_out");
+        auto c = Tensor::empty(g.shape(), DType::BF16);
+        if (!c.ok()) return c.error();
+        const int rc = flame_attn_cast_f32_to_bf16(g.data(), c.value().data(), g.numel(), nullptr);
+        if (rc != 0) return cuda_error("flame_attn_cast_f32_to_bf16", rc);
+        g = c.value();
+    } else if (g.dtype() != DType::BF16) {
+        return invalid("grad_out must be BF16 or F32");
+    }
+    auto dq = Tensor::empty(n.query.shape(), DType::BF16);
+    auto dk = Tensor::empty(n.key.shape(), DType::BF16);
+    auto dv = Tensor::empty(n.value.shape(), DType::BF16);
+    const size_t wsb = flame_attn_bwd_workspace_bytes(B, H, Sq, D);
+    auto ws = Tensor::empty({(int64_t)wsb}, DType::U8);
+    if (!dq.ok() || !dk.ok() || !dv.ok() || !ws.ok()) return cuda_error("hipMalloc", -1);
+    Tensor m8;
+    std::vector<int64_t> mst;
+    if (n.mask) {
+        auto pm = detail::prepare_mask(*n.mask, detail::Dims{B, H, Sq, Sk, D});
+        if (!pm.ok()) return pm.error();
+        m8 = pm.value().first;
+        mst = pm.value().second;
+    }
+    const int rc = flame_attn_bwd_bf16(
+        n.query.base(), n.key.base(), n.value.base(), n.output.base(), g.base(), n.stats.base(), dq.value().base(),
+        dk.value().base(), dv.value().base(), B, H, Sq, Sk, D, n.scale, n.query.strides().data(), n.key.strides().data(),
+        n.value.strides().data(), n.output.strides().data(), g.strides().data(), dq.value().strides().data(),
+        dk.value().strides().data(), dv.value().strides().data(), n.query.offset(), n.key.offset(), n.value.offset(),
+        n.output.offset(), g.offset(), 0, 0, 0, 0, n.causal ? 1 : 0, nullptr,
+        n.mask ? static_cast<const uint8_t*>(m8.data()) : nullptr, n.mask ? mst.data() : nullptr, ws.value().data(), wsb,
+        nullptr);
+    if (rc == FLAME_ATTN_ERR_UNSUPPORTED) return unsupported("flame_attn_bwd_bf16: head dim or layout not built");
+    if (rc != 0) return cuda_error("flame_attn_bwd_bf16", rc);
+    return AttentionGrads{dq.value(), dk.value(), dv.value()};
+}
+
+inline Result<AttentionGrads> backward(const Tensor& attention_output, const Tensor& grad_out) {
+    auto n = AutogradContext::find(attention_output);
+    if (!n) return invalid("no FlashAttention node recorded for this tensor");
+    return flash_attention_backward(*n, grad_out);
+}
+
+}  // namespace autograd
+
+// ------------------------------------------------------------------------------------ sdpa
+namespace sdpa {
+
+inline Result<Tensor> forward_train(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor* mask);
+
+// sdpa::forward(q, k, v, mask) (src/sdpa.rs:85-102): routes to forward_train while taping
+inline Result<Tensor> forward(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor* mask = nullptr) {
+    if (autograd::AutogradContext::is_recording() && (q.requires_grad || k.requires_grad || v.requires_grad))
+        return forward_train(q, k, v, mask);
+    auto r = detail::run_forward(q, k, v, mask, false, std::nullopt, false);
+    if (!r.ok()) return r.error();
+    return r.value().o;
+}
+
+// sdpa::forward_train (src/sdpa.rs:109-207): forward with Stats, then one Op::FlashAttention node;
+// scale = 1/sqrt(D), causal = false.  Unlike the reference a mask keeps the O(S*D) path (the
+// reference skips Stats for masked calls, :148-163).
+inline Result<Tensor> forward_train(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor* mask = nullptr) {
+    auto r = detail::run_forward(q, k, v, mask, false, std::nullopt, true);
+    if (!r.ok()) return r.error();
+    Tensor o = r.value().o;
+    o.requires_grad = true;
+    autograd::FlashAttentionNode n;
+    n.output_id = o.id();
+    n.query = q; n.key = k; n.value = v; n.output = o; n.stats = r.value().stats;
+    if (mask) n.mask = *mask;
+    n.scale = 1.0f / std::sqrt((float)q.shape()[3]);
+    n.causal = false;
+    autograd::AutogradContext::record_op(std::move(n));
+    return o;
+}
+
+// sdpa::forward_v4 (src/sdpa.rs:398-440): causal flag, optional scale, chunk sizes accepted and ignored
+// (the fused kernel has no chunking knob)
+inline Result<Tensor> forward_v4(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor* mask, bool causal,
+                                 std::optional<float> scale, std::optional<std::pair<size_t, size_t>> /*chunk*/ = std::nullopt) {
+    auto r = detail::run_forward(q, k, v, mask, causal, scale, false);
+    if (!r.ok()) return r.error();
+    return r.value().o;
+}
+
+}  // namespace sdpa
+
+// ------------------------------------------------------------------------------------ attention
+namespace attention {
+
+// lower-triangular keep-mask [1,1,Sq,Sk] (src/attention/sdpa.rs:11-34); the fused path does not need
+// it (pass causal = true instead), it exists for callers that want the tensor
+inline Result<Tensor> build_causal_mask(int64_t q_len, int64_t k_len) {
+    std::vector<uint8_t> h((size_t)q_len * k_len);
+    for (int64_t i = 0; i < q_len; ++i)
+        for (int64_t j = 0; j < k_len; ++j) h[(size_t)i * k_len + j] = j <= i ? 1 : 0;
+    return Tensor::from_host(h.data(), {1, 1, q_len, k_len}, DType::U8);
+}
+
+inline Result<Tensor> sdpa(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor* mask = nullptr) {
+    return flame::sdpa::forward(q, k, v, mask);
+}
+inline Result<Tensor> attend(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor* mask = nullptr) {
+    return flame::sdpa::forward(q, k, v, mask);
+}
+// attention_impl(q, k, v, mask, causal, scale) (src/attention/sdpa.rs:395-458).  The reference
+// rejects mask + causal together (:437-442); both are honoured here.
+inline Result<Tensor> attention_impl(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor* mask, bool causal,
+                                     std::optional<float> scale) {
+    return flame::sdpa::forward_v4(q, k, v, mask, causal, scale);
+}
+
+}  // namespace attention
+
+// ------------------------------------------------------------------------------------ autograd_v4
+namespace autograd_v4 {
+
+enum class SdpaSave { SaveProbs, SaveLSE, Recompute };
+
+struct SdpaConfig {                       // src/autograd_v4/ops/sdpa.rs:21-47
+    bool causal = false;
+    std::optional<float> scale;
+    float dropout_p = 0.f;
+    std::optional<uint64_t> dropout_seed;
+    bool upcast_compute = true;
+    std::optional<size_t> chunk_q, chunk_kv;
+    SdpaSave save = SdpaSave::SaveLSE;
+};
+
+struct SdpaStats {                        // :56-65
+    float fwd_ms = 0.f, bwd_ms = 0.f;
+    uint64_t bytes_alloc = 0, bytes_saved = 0;
+    uint32_t nan_inf_hits = 0, syncs = 0, recompute_blocks = 0;
+};
+
+struct SdpaCtx {                          // :80-96
+    Tensor q, k, v, o;
+    std::optional<Tensor> attn_mask;
+    float scale = 0.f;
+    SdpaSave save = SdpaSave::SaveLSE;
+    bool causal = false;
+    Tensor lse;                           // fp32 [B*H, Q]
+    std::tuple<size_t, size_t, size_t, size_t> shapes;   // (B,H,Q,K)
+    SdpaStats stats;
+};
+
+// sdpa_forward(q,k,v,mask,&cfg) -> (output, ctx) (:98-326).  SaveProbs would materialise the
+// [B,H,Q,K] matrix and dropout is not built: both are refused rather than emulated.
+inline Result<std::pair<Tensor, SdpaCtx>> sdpa_forward(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor* mask,
+                                                       const SdpaConfig& cfg) {
+    if (cfg.dropout_p != 0.f) return unsupported("dropout is not built into the fused kernels");
+    if (cfg.save == SdpaSave::SaveProbs) return unsupported("SaveProbs materialises [B,H,Q,K]; use SaveLSE");
+    auto r = detail::run_forward(q, k, v, mask, cfg.causal, cfg.scale, true);
+    if (!r.ok()) return r.error();
+    SdpaCtx ctx;
+    ctx.q = q; ctx.k = k; ctx.v = v; ctx.o = r.value().o;
+    if (mask) ctx.attn_mask = *mask;
+    ctx.scale = cfg.scale.value_or(1.0f / std::sqrt((float)q.shape()[3]));
+    ctx.save = cfg.save;
+    ctx.causal = cfg.causal;
+    ctx.lse = r.value().stats;
+    ctx.shapes = {(size_t)q.shape()[0], (size_t)q.shape()[1], (size_t)q.shape()[2], (size_t)k.shape()[2]};
+    ctx.stats.bytes_saved = (uint64_t)ctx.o.numel() * 2 + (uint64_t)ctx.lse.numel() * 4;
+    return std::make_pair(r.value().o, ctx);
+}
+
+// sdpa_backward(&ctx, &grad_out) -> (dq, dk, dv) (:826-1009).  Gradients are bf16 here (the
+// reference returns fp32 tensors from its fp32 tensor-op implementation).
+inline Result<std::tuple<Tensor, Tensor, Tensor>> sdpa_backward(const SdpaCtx& ctx, const Tensor& grad_out) {
+    autograd::FlashAttentionNode n;
+    n.query = ctx.q; n.key = ctx.k; n.value = ctx.v; n.output = ctx.o; n.stats = ctx.lse;
+    n.mask = ctx.attn_mask;
+    n.scale = ctx.scale;
+    n.causal = ctx.causal;
+    auto g = autograd::flash_attention_backward(n, grad_out);
+    if (!g.ok()) return g.error();
+    return std::make_tuple(g.value().dq, g.value().dk, g.value().dv);
+}
+
+}  // namespace autograd_v4
+
+// ------------------------------------------------------------------------------------ SageAttention
+// Builder-style API of the reference (src/sage_attention.rs:21-65).  `scale` is the softmax scale
+// (default 1/sqrt(D)); the reference's field of the same name is a divisor defaulting to sqrt(D)
+// (:108, :588), i.e. the same default arithmetic.  Inference only: int8 Q/K per block, mean-smoothed K.
+class SageAttention {
+   public:
+    SageAttention() = default;
+    SageAttention with_scale(float softmax_scale) const { auto s = *this; s.scale_ = softmax_scale; return s; }
+    SageAttention with_causal(bool causal) const { auto s = *this; s.causal_ = causal; return s; }
+    SageAttention with_smoothing(bool on) const { auto s = *this; s.smooth_k_ = on; return s; }
+
+    Result<Tensor> forward(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor* attention_mask = nullptr) const {
+        if (attention_mask) return unsupported("SageAttention: explicit masks are not built (causal and key lengths are)");
+        auto dv = detail::validate(q, k, v, nullptr);
+        if (!dv.ok()) return dv.error();
+        const detail::Dims d = dv.value();
+        for (const Tensor* t : {&q, &k, &v})
+            if (!detail::abi_friendly(*t)) return unsupported("tensor view needs D stride 1 and 16-byte aligned rows");
+        const int64_t nqb = (d.Sq + 127) / 128, nkb = (d.Sk + 63) / 64;
+        auto qi8 = Tensor::empty({d.B, d.H, d.Sq, d.D}, DType::I8);
+        auto ki8 = Tensor::empty({d.B, d.H, d.Sk, d.D}, DType::I8);
+        auto sq = Tensor::empty({d.B, d.H, nqb}, DType::F32);
+        auto sk = Tensor::empty({d.B, d.H, nkb}, DType::F32);
+        auto km = Tensor::empty({d.B, d.H, d.D}, DType::F32);
+        auto o = Tensor::empty({d.B, d.H, d.Sq, d.D}, DType::BF16);
+        if (!qi8.ok() || !ki8.ok() || !sq.ok() || !sk.ok() || !km.ok() || !o.ok()) return cuda_error("hipMalloc", -1);
+        int rc = flame_sage_quant_qk_int8(q.base(), k.base(), d.B, d.H, d.Sq, d.Sk, d.D, q.strides().data(), k.strides().data(),
+                                          q.offset(), k.offset(), smooth_k_ ? 1 : 0, qi8.value().data(), ki8.value().data(),
+                                          sq.value().data(), sk.value().data(), km.value().data(), nullptr);
+        if (rc == FLAME_ATTN_ERR_UNSUPPORTED) return unsupported("flame_sage_quant_qk_int8: head dim or layout not built");
+        if (rc != 0) return cuda_error("flame_sage_quant_qk_int8", rc);
+        const float sc = scale_.value_or(1.0f / std::sqrt((float)d.D));
+        rc = flame_sage_attn_fwd_int8(qi8.value().data(), ki8.value().data(), sq.value().data(), sk.value().data(), v.base(),
+                                      o.value().base(), nullptr, d.B, d.H, d.Sq, d.Sk, d.D, sc, v.strides().data(),
+                                      o.value().strides().data(), v.offset(), 0, causal_ ? 1 : 0, nullptr, nullptr);
+        if (rc != 0) return cuda_error("flame_sage_attn_fwd_int8", rc);
+        return o.value();
+    }
+
+   private:
+    std::optional<float> scale_;
+    bool causal_ = false;
+    bool smooth_k_ = true;
+};
+
+}  // namespace flame

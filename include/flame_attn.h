@@ -201,6 +201,18 @@ int flame_attn_profiling_read(FlameAttnKernelTimes* out);
  * (null switches the timing build of the kernel off again). */
 int flame_attn_debug_set_phase_buffer(void* device_buffer);
 
+/* ------------------------------------------------------------------------------------------------
+ * Small conversions the host layer needs at the boundary.
+ * ---------------------------------------------------------------------------------------------- */
+enum { FLAME_ATTN_DTYPE_BF16 = 0, FLAME_ATTN_DTYPE_F32 = 1 };
+/* Binary keep-mask in bf16 / fp32 (>= 0.5 attends; the public mask convention of the reference,
+ * src/sdpa.rs:458-470) -> contiguous uint8 keep-mask of n elements. */
+int flame_attn_convert_keep_mask(const void* src, int src_dtype, void* dst_u8, int64_t n, void* stream);
+/* fp32 -> bf16, round to nearest even, n contiguous elements.  Lets the autograd shim hand an fp32
+ * upstream gradient to the bf16 backward instead of falling back to the materialising recompute as
+ * the reference does (src/autograd.rs:702-705). */
+int flame_attn_cast_f32_to_bf16(const void* src_f32, void* dst_bf16, int64_t n, void* stream);
+
 const char* flame_attn_version(void);
 
 #ifdef __cplusplus

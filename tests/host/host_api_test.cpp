@@ -1,0 +1,310 @@
+// GPU test driver for the C++ host layer (flame_amd/host/flame_host.hpp).  Written the way the
+// reference's own integration tests are: inputs from a seeded generator, a naive fp32 materialised
+// reference computed inside the test (cf. tests/fa2_parity_naive.rs:84-140,
+// tests/cudnn_sdpa_bwd_parity.rs:31-98, src/tests/attention_tests.rs:61-155), tolerances asserted.
+// Exit status 0 = every check passed.
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <vector>
+
+#include "../../flame_amd/host/flame_host.hpp"
+
+using namespace flame;
+
+static int g_fail = 0;
+#define CHECK(cond, ...)                                                          \
+    do {                                                                          \
+        if (!(cond)) {                                                            \
+            ++g_fail;                                                             \
+            std::printf("FAIL %s:%d: %s : ", __FILE__, __LINE__, #cond);          \
+            std::printf(__VA_ARGS__);                                             \
+            std::printf("\n");                                                    \
+        }                                                                         \
+    } while (0)
+
+static uint16_t f2bf(float f) {
+    uint32_t u;
+    std::memcpy(&u, &f, 4);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+static float bf2f(uint16_t h) {
+    uint32_t u = (uint32_t)h << 16;
+    float f;
+    std::memcpy(&f, &u, 4);
+    return f;
+}
+static uint64_t g_rng = 0x9E3779B97F4A7C15ull;
+static float gauss() {   // Box-Muller on a 64-bit LCG, good enough for test inputs
+    auto next = [] {
+        g_rng = g_rng * 6364136223846793005ull + 1442695040888963407ull;
+        return (double)((g_rng >> 11) + 1) / 9007199254740993.0;
+    };
+    const double u1 = next(), u2 = next();
+    return (float)(std::sqrt(-2.0 * std::log(u1)) * std::cos(6.283185307179586 * u2));
+}
+static std::vector<uint16_t> randn_bf16(size_t n) {
+    std::vector<uint16_t> v(n);
+    for (auto& x : v) x = f2bf(gauss());
+    return v;
+}
+static Tensor dev_bf16(const std::vector<uint16_t>& h, std::vector<int64_t> shape) {
+    return Tensor::from_host(h.data(), std::move(shape), DType::BF16).value();
+}
+static std::vector<float> host_f32_of_bf16(const Tensor& t) {
+    std::vector<uint16_t> h((size_t)t.numel());
+    t.to_host(h.data());
+    std::vector<float> f(h.size());
+    for (size_t i = 0; i < h.size(); ++i) f[i] = bf2f(h[i]);
+    return f;
+}
+
+// naive fp32 materialised attention for one (b,h): O, and grads from dO (D = rowsum(dO*O))
+struct Naive {
+    std::vector<float> o, dq, dk, dv;
+};
+static Naive naive_head(const uint16_t* q, const uint16_t* k, const uint16_t* v, const uint16_t* d_o, int Sq, int Sk, int D,
+                        float scale, bool causal, const uint8_t* keep /*[Sq,Sk] or null*/) {
+    Naive r;
+    r.o.assign((size_t)Sq * D, 0.f);
+    r.dq.assign((size_t)Sq * D, 0.f);
+    r.dk.assign((size_t)Sk * D, 0.f);
+    r.dv.assign((size_t)Sk * D, 0.f);
+    std::vector<float> p(Sk), dp(Sk);
+    for (int i = 0; i < Sq; ++i) {
+        float m = -INFINITY;
+        for (int j = 0; j < Sk; ++j) {
+            float s = 0.f;
+            for (int d = 0; d < D; ++d) s += bf2f(q[i * D + d]) * bf2f(k[j * D + d]);
+            s *= scale;
+            if ((causal && j > i) || (keep && !keep[(size_t)i * Sk + j])) s = -INFINITY;
+            p[j] = s;
+            m = std::fmax(m, s);
+        }
+        if (m == -INFINITY) continue;
+        float l = 0.f;
+        for (int j = 0; j < Sk; ++j) { p[j] = std::exp(p[j] - m); l += p[j]; }
+        for (int j = 0; j < Sk; ++j) p[j] /= l;
+        for (int j = 0; j < Sk; ++j)
+            for (int d = 0; d < D; ++d) r.o[(size_t)i * D + d] += p[j] * bf2f(v[j * D + d]);
+        if (!d_o) continue;
+        float delta = 0.f;
+        for (int d = 0; d < D; ++d) delta += bf2f(d_o[i * D + d]) * bf2f(f2bf(r.o[(size_t)i * D + d]));
+        for (int j = 0; j < Sk; ++j) {
+            float a = 0.f;
+            for (int d = 0; d < D; ++d) a += bf2f(d_o[i * D + d]) * bf2f(v[j * D + d]);
+            dp[j] = a;
+        }
+        for (int j = 0; j < Sk; ++j) {
+            const float ds = p[j] * (dp[j] - delta);
+            for (int d = 0; d < D; ++d) {
+                r.dv[(size_t)j * D + d] += p[j] * bf2f(d_o[i * D + d]);
+                r.dq[(size_t)i * D + d] += ds * bf2f(k[j * D + d]) * scale;
+                r.dk[(size_t)j * D + d] += ds * bf2f(q[i * D + d]) * scale;
+            }
+        }
+    }
+    return r;
+}
+static void compare(const char* name, const std::vector<float>& got, const std::vector<float>& ref) {
+    double ma = 0, dot = 0, ng = 0, nr = 0;
+    for (size_t i = 0; i < ref.size(); ++i) {
+        ma = std::fmax(ma, std::fabs((double)got[i] - ref[i]));
+        dot += (double)got[i] * ref[i];
+        ng += (double)got[i] * got[i];
+        nr += (double)ref[i] * ref[i];
+    }
+    const double cosv = (ng > 0 && nr > 0) ? dot / std::sqrt(ng * nr) : 1.0;
+    std::printf("  %-28s max_abs=%.3e cos=%.6f\n", name, ma, cosv);
+    CHECK(ma <= 2e-2, "%s max_abs %.3e", name, ma);
+    CHECK(cosv >= 0.9999, "%s cosine %.6f", name, cosv);     // the reference's gate
+}
+
+int main() {
+    int ndev = 0;
+    if (hipGetDeviceCount(&ndev) != hipSuccess || ndev == 0) {
+        std::printf("no GPU\n");
+        return 2;
+    }
+
+    // ---- 1. known-answer test of the reference (src/tests/attention_tests.rs:110-155), head dim 2 padded to 64
+    {
+        std::printf("[kat 2x2 masked]\n");
+        const float qv[4] = {0.2f, -0.4f, 0.5f, 0.1f}, kv[4] = {0.3f, 0.7f, -0.2f, 0.4f}, vv[4] = {0.1f, -0.3f, 0.6f, 0.2f};
+        const float mask[4] = {1.f, 0.f, 1.f, 1.f};
+        auto pad = [](const float* x) {
+            std::vector<uint16_t> h(2 * 64, 0);
+            for (int i = 0; i < 2; ++i)
+                for (int d = 0; d < 2; ++d) h[i * 64 + d] = f2bf(x[i * 2 + d]);
+            return dev_bf16(h, {1, 1, 2, 64});
+        };
+        Tensor q = pad(qv), k = pad(kv), v = pad(vv);
+        Tensor m = Tensor::from_host(mask, {1, 1, 2, 2}, DType::F32).value();
+        auto out = attention::attention_impl(q, k, v, &m, false, 1.0f / std::sqrt(2.0f));
+        CHECK(out.ok(), "attention_impl failed");
+        if (out.ok()) {
+            auto o = host_f32_of_bf16(out.value());
+            const float want[4] = {0.1f, -0.3f, 0.325332f, -0.074668f};
+            for (int i = 0; i < 2; ++i)
+                for (int d = 0; d < 2; ++d) CHECK(std::fabs(o[i * 64 + d] - want[i * 2 + d]) < 2e-3, "kat[%d][%d] = %f", i, d, o[i * 64 + d]);
+        }
+    }
+
+    // ---- 2. validation errors (src/sdpa.rs:335-374, src/tensor/contracts.rs:22-33)
+    {
+        std::printf("[validation]\n");
+        Tensor a = Tensor::empty({1, 2, 8, 64}, DType::BF16).value();
+        Tensor r3 = Tensor::empty({2, 8, 64}, DType::BF16).value();
+        Tensor hb = Tensor::empty({1, 3, 8, 64}, DType::BF16).value();
+        Tensor dd = Tensor::empty({1, 2, 8, 128}, DType::BF16).value();
+        Tensor ln = Tensor::empty({1, 2, 16, 64}, DType::BF16).value();
+        Tensor f32 = Tensor::empty({1, 2, 8, 64}, DType::F32).value();
+        Tensor d96 = Tensor::empty({1, 2, 8, 96}, DType::BF16).value();
+        Tensor badm = Tensor::empty({1, 2, 8, 9}, DType::U8).value();
+        auto kind = [](const Result<Tensor>& r) { return r.ok() ? -1 : (int)r.error().kind; };
+        CHECK(kind(sdpa::forward(r3, r3, r3)) == Error::InvalidInput, "rank 3");
+        CHECK(kind(sdpa::forward(a, hb, hb)) == Error::InvalidInput, "head mismatch");
+        CHECK(kind(sdpa::forward(a, dd, dd)) == Error::InvalidInput, "embed mismatch");
+        CHECK(kind(sdpa::forward(a, a, ln)) == Error::InvalidInput, "k_len != v_len");
+        CHECK(kind(sdpa::forward(a, a, a, &badm)) == Error::InvalidInput, "mask not broadcastable");
+        CHECK(kind(sdpa::forward(f32, f32, f32)) == Error::InvalidInput, "non-bf16");
+        CHECK(kind(sdpa::forward(d96, d96, d96)) == Error::Unsupported, "head dim 96");
+    }
+
+    // ---- 3. forward == forward_train, taped backward vs the naive recompute; shapes of
+    //         tests/cudnn_sdpa_bwd_parity.rs:311-320
+    for (int D : {64, 128}) {
+        const int B = 1, H = 4, N = D == 64 ? 128 : 256;
+        std::printf("[train fwd/bwd  B=%d H=%d N=%d D=%d]\n", B, H, N, D);
+        auto hq = randn_bf16((size_t)B * H * N * D), hk = randn_bf16(hq.size()), hv = randn_bf16(hq.size()), hdo = randn_bf16(hq.size());
+        Tensor q = dev_bf16(hq, {B, H, N, D}), k = dev_bf16(hk, {B, H, N, D}), v = dev_bf16(hv, {B, H, N, D});
+        Tensor d_o = dev_bf16(hdo, {B, H, N, D});
+        q.requires_grad = true;
+        auto o_inf = sdpa::forward(q, k, v);
+        autograd::AutogradContext::set_recording(true);
+        auto o_trn = sdpa::forward(q, k, v);                 // routed to forward_train
+        autograd::AutogradContext::set_recording(false);
+        CHECK(o_inf.ok() && o_trn.ok(), "forward failed");
+        if (!o_inf.ok() || !o_trn.ok()) continue;
+        auto a = host_f32_of_bf16(o_inf.value()), b2 = host_f32_of_bf16(o_trn.value());
+        CHECK(a == b2, "train-forward O differs from inference-forward O");
+        auto node = autograd::AutogradContext::find(o_trn.value());
+        CHECK(node.has_value(), "no FlashAttention node recorded");
+        if (node) CHECK(autograd::AutogradContext::saved_activation_bytes(*node) == (size_t)B * H * N * D * 2 + (size_t)B * H * N * 4,
+                        "saved set is not O + LSE");
+        auto g = autograd::backward(o_trn.value(), d_o);
+        CHECK(g.ok(), "backward failed");
+        if (!g.ok()) continue;
+        // fp32 upstream gradient takes the same kernel after a cast
+        std::vector<float> hdo32(hdo.size());
+        for (size_t i = 0; i < hdo.size(); ++i) hdo32[i] = bf2f(hdo[i]);
+        Tensor d_o32 = Tensor::from_host(hdo32.data(), {B, H, N, D}, DType::F32).value();
+        auto g32 = autograd::backward(o_trn.value(), d_o32);
+        CHECK(g32.ok() && host_f32_of_bf16(g32.value().dk) == host_f32_of_bf16(g.value().dk), "fp32 dO path differs");
+        std::vector<float> ro, rdq, rdk, rdv;
+        for (int bh = 0; bh < B * H; ++bh) {
+            const size_t off = (size_t)bh * N * D;
+            Naive nv = naive_head(&hq[off], &hk[off], &hv[off], &hdo[off], N, N, D, 1.0f / std::sqrt((float)D), false, nullptr);
+            ro.insert(ro.end(), nv.o.begin(), nv.o.end());
+            rdq.insert(rdq.end(), nv.dq.begin(), nv.dq.end());
+            rdk.insert(rdk.end(), nv.dk.begin(), nv.dk.end());
+            rdv.insert(rdv.end(), nv.dv.begin(), nv.dv.end());
+        }
+        compare("O", a, ro);
+        compare("dQ", host_f32_of_bf16(g.value().dq), rdq);
+        compare("dK", host_f32_of_bf16(g.value().dk), rdk);
+        compare("dV", host_f32_of_bf16(g.value().dv), rdv);
+        autograd::AutogradContext::clear();
+    }
+
+    // ---- 4. the DiT view reshape([B,N,H,D]).permute(0,2,1,3) runs without a copy (src/sdpa.rs:607-621)
+    {
+        std::printf("[permuted view]\n");
+        const int B = 1, H = 3, N = 96, D = 128;
+        auto hq = randn_bf16((size_t)B * N * H * D), hk = randn_bf16(hq.size()), hv = randn_bf16(hq.size());
+        Tensor qn = dev_bf16(hq, {B, N, H, D}), kn = dev_bf16(hk, {B, N, H, D}), vn = dev_bf16(hv, {B, N, H, D});
+        auto o = sdpa::forward(qn.permute({0, 2, 1, 3}), kn.permute({0, 2, 1, 3}), vn.permute({0, 2, 1, 3}));
+        CHECK(o.ok(), "strided forward failed");
+        if (o.ok()) {
+            auto got = host_f32_of_bf16(o.value());
+            std::vector<float> ref((size_t)B * H * N * D);
+            for (int h = 0; h < H; ++h) {
+                std::vector<uint16_t> q1((size_t)N * D), k1(q1.size()), v1(q1.size());
+                for (int i = 0; i < N; ++i)
+                    for (int d = 0; d < D; ++d) {
+                        q1[i * D + d] = hq[((size_t)i * H + h) * D + d];
+                        k1[i * D + d] = hk[((size_t)i * H + h) * D + d];
+                        v1[i * D + d] = hv[((size_t)i * H + h) * D + d];
+                    }
+                Naive nv = naive_head(q1.data(), k1.data(), v1.data(), nullptr, N, N, D, 1.0f / std::sqrt((float)D), false, nullptr);
+                std::copy(nv.o.begin(), nv.o.end(), ref.begin() + (size_t)h * N * D);
+            }
+            compare("O (strided inputs)", got, ref);
+        }
+    }
+
+    // ---- 5. autograd_v4 surface: causal SaveLSE forward + backward; refused options
+    {
+        std::printf("[autograd_v4 causal]\n");
+        const int B = 1, H = 2, N = 160, D = 64;
+        auto hq = randn_bf16((size_t)B * H * N * D), hk = randn_bf16(hq.size()), hv = randn_bf16(hq.size()), hdo = randn_bf16(hq.size());
+        Tensor q = dev_bf16(hq, {B, H, N, D}), k = dev_bf16(hk, {B, H, N, D}), v = dev_bf16(hv, {B, H, N, D}), d_o = dev_bf16(hdo, {B, H, N, D});
+        autograd_v4::SdpaConfig cfg;
+        cfg.causal = true;
+        cfg.chunk_q = 3; cfg.chunk_kv = 4;          // accepted, ignored
+        auto f = autograd_v4::sdpa_forward(q, k, v, nullptr, cfg);
+        CHECK(f.ok(), "sdpa_forward failed");
+        if (f.ok()) {
+            CHECK(f.value().second.stats.bytes_saved == (uint64_t)B * H * N * D * 2 + (uint64_t)B * H * N * 4, "bytes_saved");
+            auto g = autograd_v4::sdpa_backward(f.value().second, d_o);
+            CHECK(g.ok(), "sdpa_backward failed");
+            std::vector<float> ro, rdq, rdk, rdv;
+            for (int bh = 0; bh < B * H; ++bh) {
+                const size_t off = (size_t)bh * N * D;
+                Naive nv = naive_head(&hq[off], &hk[off], &hv[off], &hdo[off], N, N, D, 1.0f / std::sqrt((float)D), true, nullptr);
+                ro.insert(ro.end(), nv.o.begin(), nv.o.end());
+                rdq.insert(rdq.end(), nv.dq.begin(), nv.dq.end());
+                rdk.insert(rdk.end(), nv.dk.begin(), nv.dk.end());
+                rdv.insert(rdv.end(), nv.dv.begin(), nv.dv.end());
+            }
+            compare("O causal", host_f32_of_bf16(f.value().first), ro);
+            if (g.ok()) {
+                compare("dQ causal", host_f32_of_bf16(std::get<0>(g.value())), rdq);
+                compare("dK causal", host_f32_of_bf16(std::get<1>(g.value())), rdk);
+                compare("dV causal", host_f32_of_bf16(std::get<2>(g.value())), rdv);
+            }
+        }
+        cfg.dropout_p = 0.1f;
+        CHECK(!autograd_v4::sdpa_forward(q, k, v, nullptr, cfg).ok(), "dropout must be refused");
+        cfg.dropout_p = 0.f;
+        cfg.save = autograd_v4::SdpaSave::SaveProbs;
+        CHECK(!autograd_v4::sdpa_forward(q, k, v, nullptr, cfg).ok(), "SaveProbs must be refused");
+    }
+
+    // ---- 6. SageAttention vs the bf16 path: cosine >= 0.999
+    {
+        std::printf("[sage]\n");
+        const int B = 1, H = 2, N = 384, D = 128;
+        auto hq = randn_bf16((size_t)B * H * N * D), hk = randn_bf16(hq.size()), hv = randn_bf16(hq.size());
+        for (size_t i = 7; i < hk.size(); i += D) hk[i] = f2bf(bf2f(hk[i]) * 3.0f + 1.5f);     // outlier channel
+        Tensor q = dev_bf16(hq, {B, H, N, D}), k = dev_bf16(hk, {B, H, N, D}), v = dev_bf16(hv, {B, H, N, D});
+        auto o1 = SageAttention().forward(q, k, v);
+        auto o2 = sdpa::forward(q, k, v);
+        CHECK(o1.ok() && o2.ok(), "sage/bf16 forward failed");
+        if (o1.ok() && o2.ok()) {
+            auto a = host_f32_of_bf16(o1.value()), b2 = host_f32_of_bf16(o2.value());
+            double dot = 0, na = 0, nb = 0;
+            for (size_t i = 0; i < a.size(); ++i) { dot += (double)a[i] * b2[i]; na += (double)a[i] * a[i]; nb += (double)b2[i] * b2[i]; }
+            const double c = dot / std::sqrt(na * nb);
+            std::printf("  cosine sage vs bf16 = %.6f\n", c);
+            CHECK(c >= 0.999, "sage cosine %.6f", c);
+        }
+        Tensor m = Tensor::empty({1, 1, N, N}, DType::U8).value();
+        CHECK(!SageAttention().forward(q, k, v, &m).ok(), "sage + mask must be refused");
+    }
+
+    if (hipDeviceSynchronize() != hipSuccess) ++g_fail;
+    std::printf(g_fail ? "HOST API TEST: %d FAILURES\n" : "HOST API TEST: all checks passed\n", g_fail);
+    return g_fail ? 1 : 0;
+}
