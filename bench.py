@@ -48,6 +48,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--config", type=int, default=2, help="workload configuration (2 = the headline shape)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--traffic-calibration", action="store_true",
+                    help="also run one plain 256 MiB device copy, so that FETCH_SIZE / WRITE_SIZE read under "
+                         "rocprofv3 --pmc can be scaled by what the same counters report for a known size")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (heads shard without communication; "
@@ -79,6 +82,9 @@ def main():
         _, lse = capi.attn_fwd(q, k, v, w.scale, causal=w.causal, kv_len=kvl, out=o)
         capi.attn_bwd(q, k, v, o, do, lse, w.scale, causal=w.causal, kv_len=kvl, workspace=ws, grads=grads)
 
+    if args.traffic_calibration:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+        torch.empty_like(src).copy_(src)          # one elementwise copy kernel: reads 256 MiB, writes 256 MiB
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()

@@ -17,7 +17,7 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",   # keep packed fp32 VALU ops off
-    "-Wall", "-Wno-unused-function",
+    "-Wall", "-Wno-unused-function", "-Wno-inline-asm",   # m0 is clobbered on purpose by the LDS-DMA helpers
 ]
 
 

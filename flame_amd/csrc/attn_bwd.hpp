@@ -211,8 +211,8 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
 #pragma unroll
             for (int i = 0; i < NDQ; ++i) {
                 const int ji = wave * NDQ + i;
-                dma16(qt_base + q_lane_off[i], qdst + ji * 512);
-                dma16(dot_base + do_lane_off[i], ddst + ji * 512);
+                dma16u(qt_base, 2u * q_lane_off[i], qdst + ji * 512);
+                dma16u(dot_base, 2u * do_lane_off[i], ddst + ji * 512);
             }
             if (wave < 2) dma4((wave == 0 ? lsebase : deltabase) + q0 + lane, rows0 + buf * T::ROW_FLOATS + wave * BM);
         } else {   // last, partial tile: rows past the end re-read the last valid row
@@ -334,8 +334,8 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
             if (COPY == 2 && (!have_next || !next_full)) return;
             if (j < 2 * NDQ) {
                 const int i = j >> 1, ji = wave * NDQ + i;
-                if (j & 1) dma16(ndo_base + do_lane_off[i], nq_dst + T::Q_ELEMS + ji * 512);
-                else dma16(nq_base + q_lane_off[i], nq_dst + ji * 512);
+                if (j & 1) dma16u(ndo_base, 2u * do_lane_off[i], nq_dst + T::Q_ELEMS + ji * 512);
+                else dma16u(nq_base, 2u * q_lane_off[i], nq_dst + ji * 512);
             } else if (wave < 2) {
                 dma4((wave == 0 ? lsebase : deltabase) + qt_next * BM + lane,
                      rows0 + (buf ^ 1) * T::ROW_FLOATS + wave * BM);
@@ -555,8 +555,8 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams p) {
 #pragma unroll
         for (int i = 0; i < T::DMA_PER_WAVE; ++i) {
             const int ji = wave * T::DMA_PER_WAVE + i;
-            dma16(kt + k_lane_off[i], kdst + ji * 512);
-            dma16(vt + v_lane_off[i], vdst + ji * 512);
+            dma16u(kt, 2u * k_lane_off[i], kdst + ji * 512);
+            dma16u(vt, 2u * v_lane_off[i], vdst + ji * 512);
         }
     };
 

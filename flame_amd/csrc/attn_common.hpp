@@ -140,14 +140,28 @@ __device__ __forceinline__ constexpr int swz(int row) {
 }
 
 // One wave-wide asynchronous copy global -> LDS: lane l delivers 16 (or 4) bytes to lds_dst + 16*l (4*l).
-// The destination must be wave-uniform.  Completion is tracked by vmcnt.
+// The destination must be wave-uniform (it travels in M0).  Completion is tracked by vmcnt only, and
+// the caller waits explicitly (wait_vm0 + barrier) before anyone reads the destination.
+// The instruction is emitted by hand: when the compiler knows of a pending LDS-DMA it turns every
+// following LDS-read wait into a full drain (lgkmcnt(0)), which defeats the read-ahead pipelines of
+// the kernels.  Hidden from its wait-count bookkeeping, LDS reads of *other* buffers keep their exact
+// counts.  Compiler-issued vmcnt waits stay correct: extra outstanding operations only make a
+// counted wait stricter.
+__device__ __forceinline__ uint32_t lds_addr(const void* p) {
+    return __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(const __attribute__((address_space(3))) char*)p);
+}
 __device__ __forceinline__ void dma16(const void* gsrc, void* lds_dst_wave_uniform) {
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gsrc,
-                                     (__attribute__((address_space(3))) void*)lds_dst_wave_uniform, 16, 0, 0);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                 :: "s"(lds_addr(lds_dst_wave_uniform)), "v"(gsrc) : "m0", "memory");
 }
 __device__ __forceinline__ void dma4(const void* gsrc, void* lds_dst_wave_uniform) {
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gsrc,
-                                     (__attribute__((address_space(3))) void*)lds_dst_wave_uniform, 4, 0, 0);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off"
+                 :: "s"(lds_addr(lds_dst_wave_uniform)), "v"(gsrc) : "m0", "memory");
+}
+// Same, with the address split into a wave-uniform base and a non-negative per-lane byte offset.
+__device__ __forceinline__ void dma16u(const void* gbase_wave_uniform, uint32_t lane_byte_off, void* lds_dst_wave_uniform) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :: "s"(lds_addr(lds_dst_wave_uniform)), "v"(lane_byte_off), "s"(gbase_wave_uniform) : "m0", "memory");
 }
 __device__ __forceinline__ void wait_vm0() { __builtin_amdgcn_s_waitcnt(0x0F70); }   // vmcnt(0) only
 

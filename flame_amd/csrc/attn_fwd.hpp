@@ -119,8 +119,8 @@ __global__ __launch_bounds__(256, (NWQ == 1 ? 2 : 1)) void fwd_kernel(const FwdP
 #pragma unroll
         for (int i = 0; i < T::DMA_PER_WAVE; ++i) {
             const int ji = wave * T::DMA_PER_WAVE + i;
-            dma16(kt + k_lane_off[i], kdst + ji * 512);
-            dma16(vt + v_lane_off[i], vdst + ji * 512);
+            dma16u(kt, 2u * k_lane_off[i], kdst + ji * 512);
+            dma16u(vt, 2u * v_lane_off[i], vdst + ji * 512);
         }
     };
 
