@@ -150,18 +150,23 @@ __device__ __forceinline__ constexpr int swz(int row) {
 __device__ __forceinline__ uint32_t lds_addr(const void* p) {
     return __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(const __attribute__((address_space(3))) char*)p);
 }
-__device__ __forceinline__ void dma16(const void* gsrc, void* lds_dst_wave_uniform) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
-                 :: "s"(lds_addr(lds_dst_wave_uniform)), "v"(gsrc) : "m0", "memory");
+// destination given as a wave-uniform LDS byte address
+__device__ __forceinline__ void dma16(const void* gsrc, uint32_t lds_byte_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(lds_byte_addr), "v"(gsrc) : "m0", "memory");
 }
-__device__ __forceinline__ void dma4(const void* gsrc, void* lds_dst_wave_uniform) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off"
-                 :: "s"(lds_addr(lds_dst_wave_uniform)), "v"(gsrc) : "m0", "memory");
+__device__ __forceinline__ void dma4(const void* gsrc, uint32_t lds_byte_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, off" :: "s"(lds_byte_addr), "v"(gsrc) : "m0", "memory");
 }
-// Same, with the address split into a wave-uniform base and a non-negative per-lane byte offset.
-__device__ __forceinline__ void dma16u(const void* gbase_wave_uniform, uint32_t lane_byte_off, void* lds_dst_wave_uniform) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                 :: "s"(lds_addr(lds_dst_wave_uniform)), "v"(lane_byte_off), "s"(gbase_wave_uniform) : "m0", "memory");
+// ... and the source split into a wave-uniform base and a non-negative per-lane byte offset
+__device__ __forceinline__ void dma16u(const void* gbase_wave_uniform, uint32_t lane_byte_off, uint32_t lds_byte_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :: "s"(lds_byte_addr), "v"(lane_byte_off), "s"(gbase_wave_uniform) : "m0", "memory");
+}
+// destination given as a pointer into LDS (wave-uniform)
+__device__ __forceinline__ void dma16(const void* gsrc, void* lds_dst) { dma16(gsrc, lds_addr(lds_dst)); }
+__device__ __forceinline__ void dma4(const void* gsrc, void* lds_dst) { dma4(gsrc, lds_addr(lds_dst)); }
+__device__ __forceinline__ void dma16u(const void* gbase_wave_uniform, uint32_t lane_byte_off, void* lds_dst) {
+    dma16u(gbase_wave_uniform, lane_byte_off, lds_addr(lds_dst));
 }
 __device__ __forceinline__ void wait_vm0() { __builtin_amdgcn_s_waitcnt(0x0F70); }   // vmcnt(0) only
 

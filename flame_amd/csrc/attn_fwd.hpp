@@ -1,8 +1,8 @@
 // Tiled QK^T -> online softmax -> PV forward for gfx950.  Writes O (bf16) and, when asked, the
 // per-row log-sum-exp of the scaled logits; the Sq x Sk score matrix never leaves registers.
 //
-// One workgroup = 4 wavefronts = 128*NWQ query rows of one (batch, head); each wavefront owns
-// 32*NWQ rows whose Q fragments stay in registers.  K/V tiles of 64 keys are copied global -> LDS
+// One workgroup = 4 wavefronts = 128 query rows of one (batch, head); each wavefront owns
+// 32 rows whose Q fragments stay in registers.  K/V tiles of 64 keys are copied global -> LDS
 // by the asynchronous LDS-DMA loads (no staging registers), double buffered, row-major with an XOR
 // swizzle of the 16-byte granules so that both the row reads of K and the transposing reads of V are
 // free of bank conflicts without padding.  The logits are produced transposed, S^T = K Q^T, so that
@@ -10,6 +10,12 @@
 // exchange between the wave halves, the bf16 P^T values are already in the B-operand layout of the
 // second MFMA (O^T = V^T P^T), and the running rescale of O is a per-lane scalar that is skipped
 // while the running maximum stays within 2^8 of the reference maximum in use.
+//
+// The key loop is software-pipelined inside each wavefront: a wavefront issues at most one
+// instruction every four cycles, and the matrix pipe and the vector ALU only run side by side when
+// their instructions alternate in that stream.  Step t therefore threads the exponentials of tile t
+// between the MFMAs that produce the logits of tile t+1, and the row-maximum scan of tile t+1 between
+// the MFMAs of O += P(t) V(t).  The K tile in LDS runs one tile ahead of the V tile.
 #pragma once
 #include <type_traits>
 
@@ -40,19 +46,24 @@ struct FwdTile {
     static constexpr int DMA_PER_WAVE = BN / ROWS_PER_DMA / 4;   // copies per wave and tensor
 };
 
-template <int D, int NWQ, bool HASMASK>
-__global__ __launch_bounds__(256, (NWQ == 1 ? 2 : 1)) void fwd_kernel(const FwdParams p) {
+template <int D, bool HASMASK>
+__global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
     using T = FwdTile<D>;
     constexpr int BN = T::BN, RS = T::RS;
-    constexpr int BM = 128 * NWQ;
+    constexpr int BM = 128;
     constexpr int DC = D / 16;   // contraction chunks of QK^T
     constexpr int DB = D / 32;   // 32-row blocks of O^T
     constexpr int GPR = D / 8;   // 16-byte granules per row
+    constexpr int NDMA = T::DMA_PER_WAVE;
+    constexpr int PD = 4;        // LDS read-ahead depth, in fragments
+    static_assert((2 * DC) % PD == 0 && (4 * DB) % PD == 0, "read-ahead depth must divide the fragment counts");
+    static_assert(2 * DC == 16 || 2 * DC == 8, "softmax slicing assumes 16 or 8 logit MFMAs per tile");
 
     extern __shared__ __attribute__((aligned(1024))) uint16_t lds[];
 
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 31, h = lane >> 5;
 
     const int n_qt = (p.Sq + BM - 1) / BM;
@@ -61,7 +72,7 @@ __global__ __launch_bounds__(256, (NWQ == 1 ? 2 : 1)) void fwd_kernel(const FwdP
     const int bh = wg / n_qt;
     const int b = bh / p.H, hh = bh % p.H;
     const int q0 = qt * BM;
-    const int qw0 = q0 + wave * 32 * NWQ;
+    const int qw0 = q0 + wave * 32;
 
     const uint16_t* qbase = p.q + b * p.qs.b + hh * p.qs.h;
     const uint16_t* kbase = p.k + b * p.ks.b + hh * p.ks.h;
@@ -76,51 +87,50 @@ __global__ __launch_bounds__(256, (NWQ == 1 ? 2 : 1)) void fwd_kernel(const FwdP
     const uint8_t* mbase = HASMASK ? p.m.mask + b * p.m.sb + hh * p.m.sh : nullptr;
 
     // ---- Q fragments (B operand of S^T = K Q^T): column = query, 8 consecutive d
-    bf16x8 qf[NWQ][DC];
-#pragma unroll
-    for (int qb = 0; qb < NWQ; ++qb) {
-        const int row = qw0 + 32 * qb + n;
+    bf16x8 qf[DC];
+    {
+        const int row = qw0 + n;
         const bool ok = row < p.Sq;
         const uint16_t* rp = qbase + (int64_t)row * p.qs.n + 8 * h;
 #pragma unroll
-        for (int dc = 0; dc < DC; ++dc) qf[qb][dc] = __builtin_bit_cast(bf16x8, ldg16(rp + 16 * dc, ok));
+        for (int dc = 0; dc < DC; ++dc) qf[dc] = __builtin_bit_cast(bf16x8, ldg16(rp + 16 * dc, ok));
     }
 
-    // ---- asynchronous tile copies.  Full tiles: uniform tile base + a per-lane 32-bit offset that
-    //      never changes; the ragged last tile clamps its rows into the attended range.
+    // ---- asynchronous tile copies.  K(t) and V(t) live in stage t&1.  Full tiles: uniform tile base
+    //      + a per-lane 32-bit byte offset that never changes; ragged tiles clamp their rows into the
+    //      attended range.
+    const uint32_t lds0 = lds_addr(lds);
     const int dma_row_in = lane / GPR;                       // row inside one 1 KiB copy
     const int dma_gran = lane % GPR;                         // physical granule written by this lane
-    int k_lane_off[T::DMA_PER_WAVE], v_lane_off[T::DMA_PER_WAVE];
+    uint32_t k_lane_off[NDMA], v_lane_off[NDMA];
 #pragma unroll
-    for (int i = 0; i < T::DMA_PER_WAVE; ++i) {
-        const int row = (wave * T::DMA_PER_WAVE + i) * T::ROWS_PER_DMA + dma_row_in;
+    for (int i = 0; i < NDMA; ++i) {
+        const int row = (wave * NDMA + i) * T::ROWS_PER_DMA + dma_row_in;
         const int c = dma_gran ^ swz<D>(row);
-        k_lane_off[i] = row * (int)p.ks.n + c * 8;
-        v_lane_off[i] = row * (int)p.vs.n + c * 8;
+        k_lane_off[i] = 2u * (uint32_t)(row * (int)p.ks.n + c * 8);
+        v_lane_off[i] = 2u * (uint32_t)(row * (int)p.vs.n + c * 8);
     }
-    auto issue_tile = [&](int t, int buf) {
-        uint16_t* kdst = lds + buf * T::STAGE_ELEMS;
-        uint16_t* vdst = kdst + T::TILE_ELEMS;
+    auto dst_of = [&](int t, int which, int i) {             // LDS byte address of copy i of this wave
+        return lds0 + 2u * (uint32_t)((t & 1) * T::STAGE_ELEMS + which * T::TILE_ELEMS + (wave * NDMA + i) * 512);
+    };
+    auto issue_ragged = [&](const uint16_t* base, int64_t row_stride, int t, int which) {
 #pragma unroll
-        for (int i = 0; i < T::DMA_PER_WAVE; ++i) {
-            const int ji = wave * T::DMA_PER_WAVE + i;
-            const int row = ji * T::ROWS_PER_DMA + dma_row_in;
+        for (int i = 0; i < NDMA; ++i) {
+            const int row = (wave * NDMA + i) * T::ROWS_PER_DMA + dma_row_in;
             const int key = min(t * BN + row, klimit - 1);   // tail rows re-read the last attended key
             const int c = dma_gran ^ swz<D>(row);
-            dma16(kbase + (int64_t)key * p.ks.n + c * 8, kdst + ji * 512);
-            dma16(vbase + (int64_t)key * p.vs.n + c * 8, vdst + ji * 512);
+            dma16(base + (int64_t)key * row_stride + c * 8, dst_of(t, which, i));
         }
     };
-    auto issue_full_tile = [&](int t, int buf) {
-        uint16_t* kdst = lds + buf * T::STAGE_ELEMS;
-        uint16_t* vdst = kdst + T::TILE_ELEMS;
-        const uint16_t* kt = kbase + (int64_t)t * BN * p.ks.n;
-        const uint16_t* vt = vbase + (int64_t)t * BN * p.vs.n;
+    auto issue_k = [&](int t) { issue_ragged(kbase, p.ks.n, t, 0); };
+    auto issue_v = [&](int t) { issue_ragged(vbase, p.vs.n, t, 1); };
+    auto issue_full_kv = [&](int tk, int tv) {               // K tile tk and V tile tv, both full
+        const uint16_t* kt = kbase + (int64_t)tk * BN * p.ks.n;
+        const uint16_t* vt = vbase + (int64_t)tv * BN * p.vs.n;
 #pragma unroll
-        for (int i = 0; i < T::DMA_PER_WAVE; ++i) {
-            const int ji = wave * T::DMA_PER_WAVE + i;
-            dma16u(kt, 2u * k_lane_off[i], kdst + ji * 512);
-            dma16u(vt, 2u * v_lane_off[i], vdst + ji * 512);
+        for (int i = 0; i < NDMA; ++i) {
+            dma16u(kt, k_lane_off[i], dst_of(tk, 0, i));
+            dma16u(vt, v_lane_off[i], dst_of(tv, 1, i));
         }
     };
 
@@ -137,183 +147,227 @@ __global__ __launch_bounds__(256, (NWQ == 1 ? 2 : 1)) void fwd_kernel(const FwdP
         for (int db = 0; db < DB; ++db)
             voff[half][db] = row * RS + (((4 * db + 2 * tr_g16 + ((tr_r & 3) >> 1)) ^ swz<D>(row)) << 3) + 4 * (tr_r & 1);
     }
+    auto k_frag = [&](int t, int i) {       // fragment i = (dc, kb) of K(t)
+        const uint16_t* ks = lds + (t & 1) * T::STAGE_ELEMS;
+        return *reinterpret_cast<const bf16x8*>(ks + koff[i >> 1] + 32 * (i & 1) * RS);
+    };
+    auto v_frag = [&](int t, int i) {       // fragment i = (cc, db) of V(t)^T
+        const uint16_t* vs = lds + (t & 1) * T::STAGE_ELEMS + T::TILE_ELEMS;
+        const int cc = i / DB, db = i % DB;
+        const u32x2 lo = lds_read_tr16(vs + voff[0][db] + 16 * cc * RS);
+        const u32x2 hi = lds_read_tr16(vs + voff[1][db] + 16 * cc * RS);
+        const u32x4 u = {lo[0], lo[1], hi[0], hi[1]};
+        return __builtin_bit_cast(bf16x8, u);
+    };
 
-    // ---- running state; each lane serves query column n of every block qb
+    // ---- running state; each lane serves query column n
     const float c_log2 = p.scale * kLog2e;
     const float stale_ok = 8.0f / c_log2;     // the reference maximum may lag the true one by 2^8
-    float m_run[NWQ], l_run[NWQ];
-    f32x16 oacc[NWQ][DB];
+    float m_run = -INFINITY, l_run = 0.f;
+    f32x16 oacc[DB];
 #pragma unroll
-    for (int qb = 0; qb < NWQ; ++qb) {
-        m_run[qb] = -INFINITY;
-        l_run[qb] = 0.f;
+    for (int db = 0; db < DB; ++db)
 #pragma unroll
-        for (int db = 0; db < DB; ++db)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) oacc[qb][db][r] = 0.f;
-    }
+        for (int r = 0; r < 16; ++r) oacc[db][r] = 0.f;
 
-    if (n_tiles > 0) issue_tile(0, 0);
-    wait_vm0();
-    __syncthreads();
+    constexpr int NS = 2 * DC;     // logit MFMAs per tile
+    constexpr int NP = 4 * DB;     // PV MFMAs per tile
+    constexpr int EPS = 32 / NS;   // logits handled per softmax slice
 
-    // One key tile.  MASKED: the tile needs per-element exclusions (ragged tail, causal diagonal,
-    // explicit mask).  COPY: 1 = the next tile is a full one (straight-line copies), 2 = decide at run time.
-    auto tile_step = [&](auto masked_tag, auto copy_tag, int t) {
-        constexpr bool MASKED = decltype(masked_tag)::value;
-        constexpr int COPY = decltype(copy_tag)::value;
-        const int buf = t & 1;
-        if (COPY == 1) issue_full_tile(t + 1, buf ^ 1);
-        else if (t + 1 < n_tiles) issue_tile(t + 1, buf ^ 1);
+    // exclusions of tile t: ragged tail / key length, causal, explicit keep-mask
+    auto apply_mask = [&](f32x16 (&s)[2], int t) {
+        const int qi = qw0 + n;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int key = t * BN + 32 * kb + acc_row(r, h);
+                bool drop = key >= klimit;
+                if (p.m.causal) drop = drop || key > qi;
+                if (HASMASK) {
+                    if (!drop && qi < p.Sq) drop = mbase[(int64_t)qi * p.m.sq + (int64_t)key * p.m.sk] == 0;
+                }
+                s[kb][r] = drop ? -INFINITY : s[kb][r];   // select, not a divergent store
+            }
+    };
+    // Fold the maximum of a freshly computed tile into the running state.  The reference maximum
+    // moves (and the running sums are rescaled) only when some lane's tile maximum exceeds it by more
+    // than 2^8 in the exponent domain; the branch is wave-uniform.
+    auto fold_max = [&](float tmax) {
+        tmax = fmaxf(tmax, xhalf(tmax));
+        if (__any(tmax > m_run + stale_ok)) {
+            const float m_old = m_run;
+            const float m_new = fmaxf(m_old, tmax);
+            const float m_to = (m_new == -INFINITY) ? 0.f : m_new;
+            const float alpha = exp2_fast((m_old - m_to) * c_log2);
+            m_run = m_new;
+            l_run *= alpha;
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
+        }
+    };
+    auto zero_tile = [&](f32x16 (&s)[2]) {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s[kb][r] = 0.f;
+    };
 
-        const uint16_t* ks = lds + buf * T::STAGE_ELEMS;
-        const uint16_t* vs = ks + T::TILE_ELEMS;
-        const int key0 = t * BN;
+    // One step: P(t) from the logits in `cur`, logits of tile t+1 into `nxt`, O += P(t) V(t).
+    // FAST: tile t+1 needs no exclusions and K(t+2), V(t+1) are full tiles (straight-line copies and the
+    // interleaved instruction stream).  Otherwise every decision is taken at run time and the phases
+    // run one after the other.
+    auto step = [&](auto fast_tag, f32x16 (&cur)[2], f32x16 (&nxt)[2], int t) {
+        constexpr bool FAST = decltype(fast_tag)::value;
+        const bool has_next = FAST || t + 1 < n_tiles;
+        if (FAST) {
+            issue_full_kv(t + 2, t + 1);
+        } else {
+            if (t + 2 < n_tiles) issue_k(t + 2);
+            if (has_next) issue_v(t + 1);
+        }
+        const float m_use = (m_run == -INFINITY) ? 0.f : m_run;
+        const float msc = m_use * c_log2;
+        float rsum0 = 0.f, rsum1 = 0.f;
+        bf16x8 pf[4];
+        bf16x8 fb[PD];
+        // P(t): slice j covers logits [EPS*j, EPS*j + EPS) of the tile in (kb, r) order
+        auto exp_slice = [&](int j) {
+#pragma unroll
+            for (int e = 0; e < EPS; ++e) {
+                const int idx = EPS * j + e, kb = idx >> 4, r = idx & 15;
+                const float v = exp2_fast(fmaf(cur[kb][r], c_log2, -msc));
+                cur[kb][r] = v;
+                if (e & 1) rsum1 += v;
+                else rsum0 += v;
+                if ((idx & 7) == 7) {
+                    const int o8 = r - 7;
+                    const f32x16& s = cur[kb];
+                    pf[idx >> 3] = pack8(s[o8 + 0], s[o8 + 1], s[o8 + 2], s[o8 + 3], s[o8 + 4], s[o8 + 5], s[o8 + 6], s[o8 + 7]);
+                }
+            }
+        };
 
-        // ---- S^T = K Q^T : rows = keys (two blocks of 32), columns = queries.  K fragments are read
-        //      PD ahead of the MFMAs that consume them.
-        f32x16 sacc[NWQ][2];
-#pragma unroll
-        for (int qb = 0; qb < NWQ; ++qb)
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) sacc[qb][kb][r] = 0.f;
-        {
-            constexpr int NF = 2 * DC, PD = 4;
-            bf16x8 fb[PD];
-            auto rd = [&](int i) { return *reinterpret_cast<const bf16x8*>(ks + koff[i >> 1] + 32 * (i & 1) * RS); };
+        if (FAST) {
+            // ---- S(t+1)^T = K(t+1) Q^T between the exponentials of tile t
+            zero_tile(nxt);
 #pragma unroll
             for (int i = 0; i < PD; ++i) {
-                fb[i] = rd(i);
+                fb[i] = k_frag(t + 1, i);
                 __builtin_amdgcn_sched_barrier(0);
             }
 #pragma unroll
-            for (int i = 0; i < NF; ++i) {
-                const int dc = i >> 1, kb = i & 1;
-#pragma unroll
-                for (int qb = 0; qb < NWQ; ++qb) sacc[qb][kb] = mfma32(fb[i % PD], qf[qb][dc], sacc[qb][kb]);
-                if (i + PD < NF) fb[i % PD] = rd(i + PD);
+            for (int i = 0; i < NS; ++i) {
+                nxt[i & 1] = mfma32(fb[i % PD], qf[i >> 1], nxt[i & 1]);
+                if (i + PD < NS) fb[i % PD] = k_frag(t + 1, i + PD);
+                else fb[i % PD] = v_frag(t, i + PD - NS);          // run on into the V fragments
+                exp_slice(i);
                 __builtin_amdgcn_sched_barrier(0);
             }
-        }
-
-        // ---- exclusions: ragged tail / key length, causal, explicit keep-mask
-        if (MASKED) {
+            l_run += rsum0 + rsum1;
+            // ---- O^T += V(t)^T P(t)^T between the row-maximum scan of tile t+1
+            float tmax = nxt[0][0];
 #pragma unroll
-            for (int qb = 0; qb < NWQ; ++qb) {
-                const int qi = qw0 + 32 * qb + n;
+            for (int i = 0; i < NP; ++i) {
+                oacc[i % DB] = mfma32(fb[i % PD], pf[i / DB], oacc[i % DB]);
+                if (i + PD < NP) fb[i % PD] = v_frag(t, i + PD);
+                constexpr int MPS = 32 / NP;
+#pragma unroll
+                for (int e = 0; e < MPS; e += 2) {
+                    const int idx = MPS * i + e;
+                    tmax = fmaxf(fmaxf(tmax, nxt[idx >> 4][idx & 15]), nxt[(idx + 1) >> 4][(idx + 1) & 15]);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            fold_max(tmax);
+        } else {
+            if (has_next) {
+                zero_tile(nxt);
+#pragma unroll
+                for (int i = 0; i < PD; ++i) {
+                    fb[i] = k_frag(t + 1, i);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+#pragma unroll
+                for (int i = 0; i < NS; ++i) {
+                    nxt[i & 1] = mfma32(fb[i % PD], qf[i >> 1], nxt[i & 1]);
+                    if (i + PD < NS) fb[i % PD] = k_frag(t + 1, i + PD);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                apply_mask(nxt, t + 1);
+            }
+#pragma unroll
+            for (int j = 0; j < NS; ++j) exp_slice(j);
+            l_run += rsum0 + rsum1;
+#pragma unroll
+            for (int i = 0; i < PD; ++i) {
+                fb[i] = v_frag(t, i);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int i = 0; i < NP; ++i) {
+                oacc[i % DB] = mfma32(fb[i % PD], pf[i / DB], oacc[i % DB]);
+                if (i + PD < NP) fb[i % PD] = v_frag(t, i + PD);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (has_next) {
+                float tmax = nxt[0][0];
 #pragma unroll
                 for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        const int key = key0 + 32 * kb + acc_row(r, h);
-                        bool drop = key >= klimit;
-                        if (p.m.causal) drop = drop || key > qi;
-                        if (HASMASK) {
-                            if (!drop && qi < p.Sq) drop = mbase[(int64_t)qi * p.m.sq + (int64_t)key * p.m.sk] == 0;
-                        }
-                        sacc[qb][kb][r] = drop ? -INFINITY : sacc[qb][kb][r];   // select, not a divergent store
-                    }
+                    for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, nxt[kb][r]);
+                fold_max(tmax);
             }
         }
-
-        // ---- online softmax, one query per lane
-        bf16x8 pf[NWQ][4];
-#pragma unroll
-        for (int qb = 0; qb < NWQ; ++qb) {
-            float tmax = sacc[qb][0][0];
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, sacc[qb][kb][r]);
-            tmax = fmaxf(tmax, xhalf(tmax));
-            // move the reference maximum (and rescale the running sums) only when some lane's tile
-            // maximum exceeds it by more than 2^8 in the exponent domain; wave-uniform branch
-            if (__any(tmax > m_run[qb] + stale_ok)) {
-                const float m_old = m_run[qb];
-                const float m_new = fmaxf(m_old, tmax);
-                const float m_to = (m_new == -INFINITY) ? 0.f : m_new;
-                const float alpha = exp2_fast((m_old - m_to) * c_log2);
-                m_run[qb] = m_new;
-                l_run[qb] *= alpha;
-                if constexpr (NWQ > 1) {
-#pragma unroll
-                    for (int db = 0; db < DB; ++db) scale_acc_agpr(oacc[qb][db], alpha);
-                } else {
-#pragma unroll
-                    for (int db = 0; db < DB; ++db)
-#pragma unroll
-                        for (int r = 0; r < 16; ++r) oacc[qb][db][r] *= alpha;
-                }
-            }
-            const float m_use = (m_run[qb] == -INFINITY) ? 0.f : m_run[qb];
-            const float msc = m_use * c_log2;
-            float rsum = 0.f;
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const float e = exp2_fast(fmaf(sacc[qb][kb][r], c_log2, -msc));
-                    sacc[qb][kb][r] = e;
-                    rsum += e;
-                }
-            l_run[qb] += rsum;
-#pragma unroll
-            for (int cc = 0; cc < 4; ++cc) {
-                const int kb = cc >> 1, o8 = 8 * (cc & 1);
-                const f32x16& s = sacc[qb][kb];
-                pf[qb][cc] = pack8(s[o8 + 0], s[o8 + 1], s[o8 + 2], s[o8 + 3], s[o8 + 4], s[o8 + 5], s[o8 + 6],
-                                   s[o8 + 7]);
-            }
-        }
-
-        // ---- O^T += V^T P^T : rows = d, columns = queries, contraction over the 64 keys
-        {
-            constexpr int NF = 4 * DB, PD = 4;
-            bf16x8 fb[PD];
-            auto rd = [&](int i) {
-                const int cc = i / DB, db = i % DB;
-                const u32x2 lo = lds_read_tr16(vs + voff[0][db] + 16 * cc * RS);
-                const u32x2 hi = lds_read_tr16(vs + voff[1][db] + 16 * cc * RS);
-                const u32x4 u = {lo[0], lo[1], hi[0], hi[1]};
-                return __builtin_bit_cast(bf16x8, u);
-            };
-#pragma unroll
-            for (int i = 0; i < PD; ++i) {
-                fb[i] = rd(i);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-#pragma unroll
-            for (int i = 0; i < NF; ++i) {
-                const int cc = i / DB, db = i % DB;
-#pragma unroll
-                for (int qb = 0; qb < NWQ; ++qb) oacc[qb][db] = mfma32(fb[i % PD], pf[qb][cc], oacc[qb][db]);
-                if (i + PD < NF) fb[i % PD] = rd(i + PD);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        }
-
-        wait_vm0();          // next tile has landed in the other buffer
-        __syncthreads();     // ... for every wave, and everyone is done reading this one
+        wait_vm0();          // the copies issued by this step have landed
+        __syncthreads();     // ... for every wave, and everyone is done reading this step's tiles
     };
 
     // Tiles [0, n_full) need no exclusions for any query of the workgroup; the rest (ragged tail, causal
-    // diagonal, or everything under an explicit mask) run the specialised masked body.
+    // diagonal, or everything under an explicit mask) carry per-element exclusions.
     int n_full = HASMASK ? 0 : klimit / BN;
     if (p.m.causal) n_full = min(n_full, (q0 + 1) / BN);
     n_full = min(n_full, n_tiles);
-    using I1 = std::integral_constant<int, 1>;
-    using I2 = std::integral_constant<int, 2>;
-    for (int t = 0; t < n_full - 1; ++t) tile_step(std::false_type{}, I1{}, t);
-    if (n_full > 0) tile_step(std::false_type{}, I2{}, n_full - 1);
-    for (int t = n_full; t < n_tiles; ++t) tile_step(std::true_type{}, I2{}, t);
+
+    f32x16 sa[2], sb[2];
+    if (n_tiles > 0) {
+        // prologue: K(0), V(0), K(1) land; logits and maximum of tile 0
+        issue_k(0);
+        issue_v(0);
+        if (n_tiles > 1) issue_k(1);
+        wait_vm0();
+        __syncthreads();
+        zero_tile(sa);
+#pragma unroll
+        for (int i = 0; i < NS; ++i) sa[i & 1] = mfma32(k_frag(0, i), qf[i >> 1], sa[i & 1]);
+        if (n_full < 1) apply_mask(sa, 0);
+        float tmax = sa[0][0];
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, sa[kb][r]);
+        fold_max(tmax);
+        __syncthreads();     // every wave has read K(0) before step 0 starts overwriting it
+
+        // step t is FAST when t + 2 < n_full; an even number of them keeps `sa` the current tile
+        const int n_fast = max(0, n_full - 2) & ~1;
+        int t = 0;
+        for (; t < n_fast; t += 2) {
+            step(std::true_type{}, sa, sb, t);
+            step(std::true_type{}, sb, sa, t + 1);
+        }
+        for (; t < n_tiles; t += 2) {
+            step(std::false_type{}, sa, sb, t);
+            if (t + 1 < n_tiles) step(std::false_type{}, sb, sa, t + 1);
+        }
+    }
 
     // ---- epilogue
-#pragma unroll
-    for (int qb = 0; qb < NWQ; ++qb) {
-        const int row = qw0 + 32 * qb + n;
-        const float l = l_run[qb] + xhalf(l_run[qb]);
+    {
+        const int row = qw0 + n;
+        const float l = l_run + xhalf(l_run);
         const float inv = l > 0.f ? 1.0f / l : 0.f;
         if (row < p.Sq) {
             uint16_t* orow = obase + (int64_t)row * p.os.n;
@@ -321,13 +375,13 @@ __global__ __launch_bounds__(256, (NWQ == 1 ? 2 : 1)) void fwd_kernel(const FwdP
             for (int db = 0; db < DB; ++db)
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
-                    const f32x16& a = oacc[qb][db];
+                    const f32x16& a = oacc[db];
                     u32x2 w = {pack_bf16(a[4 * g] * inv, a[4 * g + 1] * inv),
                                pack_bf16(a[4 * g + 2] * inv, a[4 * g + 3] * inv)};
                     *reinterpret_cast<u32x2*>(orow + 32 * db + 8 * g + 4 * h) = w;
                 }
             if (p.lse && h == 0) {
-                const float v = l > 0.f ? (m_run[qb] * c_log2 + log2_fast(l)) * kLn2 : -INFINITY;
+                const float v = l > 0.f ? (m_run * c_log2 + log2_fast(l)) * kLn2 : -INFINITY;
                 p.lse[(int64_t)bh * p.Sq + row] = v;
             }
         }

@@ -34,7 +34,6 @@ int check_view(const void* base, const int64_t* st, int64_t off) {
 
 Strides mk(const int64_t* st) { return Strides{st[0], st[1], st[2]}; }
 
-// Tile-shape override for profiling sweeps: FLAME_ATTN_FWD_VARIANT = 0 (default) | 1 | 2 ...
 int env_int(const char* name, int dflt) {
     const char* v = getenv(name);
     return v ? atoi(v) : dflt;
@@ -83,12 +82,12 @@ struct ScopedKernelTimer {
     }
 };
 
-template <int D, int NWQ, bool HASMASK>
+template <int D, bool HASMASK>
 int launch_fwd(const FwdParams& p, hipStream_t s) {
     using T = FwdTile<D>;
-    constexpr int BM = 128 * NWQ;
+    constexpr int BM = 128;
     static bool attr_done = false;   // idempotent, so a benign race at worst repeats the call
-    auto kern = fwd_kernel<D, NWQ, HASMASK>;
+    auto kern = fwd_kernel<D, HASMASK>;
     if (!attr_done) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS_BYTES);
@@ -381,16 +380,9 @@ int flame_attn_fwd_bf16(const void* Q, const void* K, const void* V, void* O, vo
     p.m.causal = causal ? 1 : 0;
 
     hipStream_t s = static_cast<hipStream_t>(stream);
-    static const int variant = env_int("FLAME_ATTN_FWD_VARIANT", 0);
     const bool hm = keep_mask != nullptr;
-    if (D == 128) {
-        if (hm) return launch_fwd<128, 1, true>(p, s);
-        if (variant == 2) return launch_fwd<128, 2, false>(p, s);
-        return launch_fwd<128, 1, false>(p, s);
-    }
-    if (hm) return launch_fwd<64, 1, true>(p, s);
-    if (variant == 2) return launch_fwd<64, 2, false>(p, s);
-    return launch_fwd<64, 1, false>(p, s);
+    if (D == 128) return hm ? launch_fwd<128, true>(p, s) : launch_fwd<128, false>(p, s);
+    return hm ? launch_fwd<64, true>(p, s) : launch_fwd<64, false>(p, s);
 }
 
 
