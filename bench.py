@@ -17,6 +17,11 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0      # MI355X dense bf16 MFMA, published
+# HBM bytes per launch of the dominant kernel (bwd_dkdv_kernel) at the headline configuration, from two
+# rocprofv3 --pmc passes (FETCH_SIZE, WRITE_SIZE; KiB per dispatch), each scaled by what the same
+# counter reads for a plain 256 MiB device copy (FETCH_SIZE under-reads by 2.0, WRITE_SIZE is exact):
+# 83 940 KiB x 2.0 fetched + 55 426 KiB written.  Counters cannot be read from inside this script.
+DKDV_TRAFFIC_BYTES_CFG2 = int((83940 * 2.0 + 55426 * 1.0) * 1024)
 METRIC = "fwd+bwd attn TFLOP/s & % MFMA peak, S=4608 D=128 bf16; saved-activation bytes"
 
 
@@ -124,7 +129,8 @@ def main():
                    "step": "forward (O+LSE) + recompute backward (dQ,dK,dV)"},
         "frac_of_bf16_mfma_peak": tflops / PEAK_BF16_TFLOPS,
         "roofline": {"bound": "mfma", "kernel": "bwd_dkdv_kernel", "achieved": achieved, "peak": PEAK_BF16_TFLOPS,
-                     "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None,
+                     "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS,
+                     "traffic": DKDV_TRAFFIC_BYTES_CFG2 if args.config == 2 else None,
                      "avg_launch_ms": per_kernel[dom], "flops_per_launch": 8 * pairs_d},
         "kernels": kernels,
         "kernels_ms": per_kernel,
