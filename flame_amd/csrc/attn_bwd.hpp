@@ -102,7 +102,8 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
     float* rows0 = reinterpret_cast<float*>(lds + 2 * T::STAGE_ELEMS);   // [2][lse2 | delta]
 
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 31, h = lane >> 5;
 
     const int n_kt = (p.Sk + BN - 1) / BN;
@@ -167,6 +168,8 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
     };
 
     const int dma_row_in = lane / GPR, dma_gran = lane % GPR;
+    const uint32_t lds0 = lds_addr(lds);
+    const uint32_t rows_lds0 = lds0 + 2u * 2u * T::STAGE_ELEMS;   // byte address of rows0
 
     // ---- prologue: the K and V fragments of this wavefront's 32 keys are held in registers for the whole walk
     bf16x8 kf[DC], vf[DC];
@@ -178,8 +181,8 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
             const int row = ji * RPD + dma_row_in;
             const int key = max(min(k0 + row, klimit - 1), 0);   // rows past the attended range re-read a valid row
             const int c = dma_gran ^ swz<D>(row);
-            dma16(kbase + (int64_t)key * p.ks.n + c * 8, stage0 + T::STAGE_ELEMS + ji * 512);
-            dma16(vbase + (int64_t)key * p.vs.n + c * 8, stage0 + ji * 512);
+            dma16(kbase + (int64_t)key * p.ks.n + c * 8, lds0 + 2u * (T::STAGE_ELEMS + ji * 512));
+            dma16(vbase + (int64_t)key * p.vs.n + c * 8, lds0 + 2u * (ji * 512));
         }
         wait_vm0();
         __syncthreads();
@@ -193,28 +196,29 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
 
     // ---- asynchronous staging of the 64-row Q / dO tiles and their lse2 / delta rows.
     //      Address = uniform tile base + a per-lane 32-bit offset that never changes.
-    int q_lane_off[NDQ], do_lane_off[NDQ];
+    uint32_t q_lane_off[NDQ], do_lane_off[NDQ];     // bytes
 #pragma unroll
     for (int i = 0; i < NDQ; ++i) {
         const int row = (wave * NDQ + i) * RPD + dma_row_in;
         const int c = dma_gran ^ swz<D>(row);
-        q_lane_off[i] = row * (int)p.qs.n + c * 8;
-        do_lane_off[i] = row * (int)p.dos.n + c * 8;
+        q_lane_off[i] = 2u * (uint32_t)(row * (int)p.qs.n + c * 8);
+        do_lane_off[i] = 2u * (uint32_t)(row * (int)p.dos.n + c * 8);
     }
+    auto q_dst = [&](int buf, int which, int i) {    // LDS byte address of copy i of this wave (which: 0 = Q, 1 = dO)
+        return lds0 + 2u * (uint32_t)(buf * T::STAGE_ELEMS + which * T::Q_ELEMS + (wave * NDQ + i) * 512);
+    };
+    auto rows_dst = [&](int buf) { return rows_lds0 + 4u * (uint32_t)(buf * T::ROW_FLOATS + wave * BM); };
     auto issue_q_tile = [&](int qt, int buf) {
-        uint16_t* qdst = stage0 + buf * T::STAGE_ELEMS;
-        uint16_t* ddst = qdst + T::Q_ELEMS;
         const int q0 = qt * BM;
         if (q0 + BM <= p.Sq) {
             const uint16_t* qt_base = qbase + (int64_t)q0 * p.qs.n;
             const uint16_t* dot_base = dobase + (int64_t)q0 * p.dos.n;
 #pragma unroll
             for (int i = 0; i < NDQ; ++i) {
-                const int ji = wave * NDQ + i;
-                dma16u(qt_base, 2u * q_lane_off[i], qdst + ji * 512);
-                dma16u(dot_base, 2u * do_lane_off[i], ddst + ji * 512);
+                dma16u(qt_base, q_lane_off[i], q_dst(buf, 0, i));
+                dma16u(dot_base, do_lane_off[i], q_dst(buf, 1, i));
             }
-            if (wave < 2) dma4((wave == 0 ? lsebase : deltabase) + q0 + lane, rows0 + buf * T::ROW_FLOATS + wave * BM);
+            if (wave < 2) dma4((wave == 0 ? lsebase : deltabase) + q0 + lane, rows_dst(buf));
         } else {   // last, partial tile: rows past the end re-read the last valid row
 #pragma unroll
             for (int i = 0; i < NDQ; ++i) {
@@ -222,12 +226,12 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
                 const int row = ji * RPD + dma_row_in;
                 const int qi = min(q0 + row, p.Sq - 1);
                 const int c = dma_gran ^ swz<D>(row);
-                dma16(qbase + (int64_t)qi * p.qs.n + c * 8, qdst + ji * 512);
-                dma16(dobase + (int64_t)qi * p.dos.n + c * 8, ddst + ji * 512);
+                dma16(qbase + (int64_t)qi * p.qs.n + c * 8, q_dst(buf, 0, i));
+                dma16(dobase + (int64_t)qi * p.dos.n + c * 8, q_dst(buf, 1, i));
             }
             if (wave < 2) {
                 const int qi = min(q0 + lane, p.Sq - 1);
-                dma4((wave == 0 ? lsebase : deltabase) + qi, rows0 + buf * T::ROW_FLOATS + wave * BM);
+                dma4((wave == 0 ? lsebase : deltabase) + qi, rows_dst(buf));
             }
         }
     };
@@ -269,15 +273,15 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
     // compiler from undoing either interleave.
     // COPY: 0 = this is the last step, 1 = the next tile is a full one (straight-line copies),
     //       2 = decide at run time (used by the few steps that need exclusions)
-    auto step = [&](auto masked_tag, auto copy_tag, int it) {
+    // BUF: stage that holds this step's tile (0 / 1), or -1 to take it from the parity of `it`.
+    auto step = [&](auto masked_tag, auto copy_tag, auto buf_tag, int it, int qt, int qt_next) {
         constexpr bool MASKED = decltype(masked_tag)::value;
         constexpr int COPY = decltype(copy_tag)::value;
+        constexpr int BUF = decltype(buf_tag)::value;
         static_assert((2 * DC) % 4 == 0 && (4 * DB) % 4 == 0, "read-ahead depth must divide the fragment count");
-        const int qt = tile_of(it);
-        const int buf = it & 1;
+        const int buf = BUF >= 0 ? BUF : (it & 1);
         const int q0 = qt * BM;
         const bool have_next = COPY == 1 || (COPY == 2 && it + 1 < n_it);
-        const int qt_next = have_next ? tile_of(it + 1) : qt;
 
         const uint16_t* Qs = stage0 + buf * T::STAGE_ELEMS;
         const uint16_t* dOs = Qs + T::Q_ELEMS;
@@ -328,17 +332,15 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
         const bool next_full = COPY == 1 || (qt_next * BM + BM) <= p.Sq;
         const uint16_t* nq_base = qbase + (int64_t)qt_next * BM * p.qs.n;
         const uint16_t* ndo_base = dobase + (int64_t)qt_next * BM * p.dos.n;
-        uint16_t* nq_dst = stage0 + (buf ^ 1) * T::STAGE_ELEMS;
         auto copy_slice = [&](int j) {     // j in [0, 2*NDQ]
             if (COPY == 0) return;
             if (COPY == 2 && (!have_next || !next_full)) return;
             if (j < 2 * NDQ) {
-                const int i = j >> 1, ji = wave * NDQ + i;
-                if (j & 1) dma16u(ndo_base, 2u * do_lane_off[i], nq_dst + T::Q_ELEMS + ji * 512);
-                else dma16u(nq_base, 2u * q_lane_off[i], nq_dst + ji * 512);
+                const int i = j >> 1;
+                if (j & 1) dma16u(ndo_base, do_lane_off[i], q_dst(buf ^ 1, 1, i));
+                else dma16u(nq_base, q_lane_off[i], q_dst(buf ^ 1, 0, i));
             } else if (wave < 2) {
-                dma4((wave == 0 ? lsebase : deltabase) + qt_next * BM + lane,
-                     rows0 + (buf ^ 1) * T::ROW_FLOATS + wave * BM);
+                dma4((wave == 0 ? lsebase : deltabase) + qt_next * BM + lane, rows_dst(buf ^ 1));
             }
         };
         if (COPY == 2 && have_next && !next_full) issue_q_tile(qt_next, buf ^ 1);   // partial tile: slow path, all at once
@@ -427,13 +429,30 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
         FATTN_PHASE(4)
     };
 
+    using IM = std::integral_constant<int, -1>;
     using I0 = std::integral_constant<int, 0>;
     using I1 = std::integral_constant<int, 1>;
     using I2 = std::integral_constant<int, 2>;
-    for (int it = 0; it < n_masked; ++it) step(std::true_type{}, I2{}, it);
-    // every tile after the first n_masked is a full, fully attended one
-    for (int it = n_masked; it < n_it - 1; ++it) step(std::false_type{}, I1{}, it);
-    if (n_it > n_masked) step(std::false_type{}, I0{}, n_it - 1);
+    for (int it = 0; it < n_masked; ++it)
+        step(std::true_type{}, I2{}, IM{}, it, tile_of(it), it + 1 < n_it ? tile_of(it + 1) : 0);
+    // every tile after the first n_masked is a full, fully attended one, and they are consecutive
+    {
+        int it = n_masked;
+        int qt = lead_end;
+        if ((it & 1) && it < n_it - 1) {
+            step(std::false_type{}, I1{}, I1{}, it, qt, qt + 1);
+            ++it, ++qt;
+        }
+        for (; it + 1 < n_it - 1; it += 2, qt += 2) {
+            step(std::false_type{}, I1{}, I0{}, it, qt, qt + 1);
+            step(std::false_type{}, I1{}, I1{}, it + 1, qt + 1, qt + 2);
+        }
+        if (it < n_it - 1) {
+            step(std::false_type{}, I1{}, IM{}, it, qt, qt + 1);
+            ++it, ++qt;
+        }
+        if (it < n_it) step(std::false_type{}, I0{}, IM{}, it, qt, qt);
+    }
 
     if (TIMING && p.phase_cycles && tid == 0) {
 #pragma unroll
