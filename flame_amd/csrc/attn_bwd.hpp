@@ -504,7 +504,8 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams p) {
     extern __shared__ __attribute__((aligned(1024))) uint16_t lds[];
 
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 31, h = lane >> 5;
 
     const int n_qt = (p.Sq + BM - 1) / BM;
@@ -545,37 +546,36 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams p) {
     const float delta = qok ? p.delta[(int64_t)bh * p.Sq + qrow] : 0.f;
 
     const int dma_row_in = lane / GPR, dma_gran = lane % GPR;
-    int k_lane_off[T::DMA_PER_WAVE], v_lane_off[T::DMA_PER_WAVE];
+    constexpr int NDMA = T::DMA_PER_WAVE;
+    const uint32_t lds0 = lds_addr(lds);
+    uint32_t k_lane_off[NDMA], v_lane_off[NDMA];     // bytes
 #pragma unroll
-    for (int i = 0; i < T::DMA_PER_WAVE; ++i) {
-        const int row = (wave * T::DMA_PER_WAVE + i) * T::ROWS_PER_DMA + dma_row_in;
+    for (int i = 0; i < NDMA; ++i) {
+        const int row = (wave * NDMA + i) * T::ROWS_PER_DMA + dma_row_in;
         const int c = dma_gran ^ swz<D>(row);
-        k_lane_off[i] = row * (int)p.ks.n + c * 8;
-        v_lane_off[i] = row * (int)p.vs.n + c * 8;
+        k_lane_off[i] = 2u * (uint32_t)(row * (int)p.ks.n + c * 8);
+        v_lane_off[i] = 2u * (uint32_t)(row * (int)p.vs.n + c * 8);
     }
+    auto dst_of = [&](int buf, int which, int i) {    // LDS byte address of copy i of this wave (which: 0 = K, 1 = V)
+        return lds0 + 2u * (uint32_t)(buf * T::STAGE_ELEMS + which * T::TILE_ELEMS + (wave * NDMA + i) * 512);
+    };
     auto issue_tile = [&](int t, int buf) {
-        uint16_t* kdst = lds + buf * T::STAGE_ELEMS;
-        uint16_t* vdst = kdst + T::TILE_ELEMS;
 #pragma unroll
-        for (int i = 0; i < T::DMA_PER_WAVE; ++i) {
-            const int ji = wave * T::DMA_PER_WAVE + i;
-            const int row = ji * T::ROWS_PER_DMA + dma_row_in;
+        for (int i = 0; i < NDMA; ++i) {
+            const int row = (wave * NDMA + i) * T::ROWS_PER_DMA + dma_row_in;
             const int key = min(t * BN + row, klimit - 1);   // tail rows re-read the last attended key
             const int c = dma_gran ^ swz<D>(row);
-            dma16(kbase + (int64_t)key * p.ks.n + c * 8, kdst + ji * 512);
-            dma16(vbase + (int64_t)key * p.vs.n + c * 8, vdst + ji * 512);
+            dma16(kbase + (int64_t)key * p.ks.n + c * 8, dst_of(buf, 0, i));
+            dma16(vbase + (int64_t)key * p.vs.n + c * 8, dst_of(buf, 1, i));
         }
     };
     auto issue_full_tile = [&](int t, int buf) {
-        uint16_t* kdst = lds + buf * T::STAGE_ELEMS;
-        uint16_t* vdst = kdst + T::TILE_ELEMS;
         const uint16_t* kt = kbase + (int64_t)t * BN * p.ks.n;
         const uint16_t* vt = vbase + (int64_t)t * BN * p.vs.n;
 #pragma unroll
-        for (int i = 0; i < T::DMA_PER_WAVE; ++i) {
-            const int ji = wave * T::DMA_PER_WAVE + i;
-            dma16u(kt, 2u * k_lane_off[i], kdst + ji * 512);
-            dma16u(vt, 2u * v_lane_off[i], vdst + ji * 512);
+        for (int i = 0; i < NDMA; ++i) {
+            dma16u(kt, k_lane_off[i], dst_of(buf, 0, i));
+            dma16u(vt, v_lane_off[i], dst_of(buf, 1, i));
         }
     };
 
@@ -603,88 +603,116 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams p) {
     wait_vm0();
     __syncthreads();
 
-    auto tile_step = [&](auto masked_tag, auto copy_tag, int t) {
+    // One tile of 64 keys = two blocks of 32.  The phases of the two blocks are staggered so that the
+    // element-wise work of one phase is threaded between the MFMAs of the next, two logits per MFMA:
+    //   S(0) | dP(0) + P(0) | S(1) + dS(0) | dP(1) + P(1) | dQ(0) + dS(1) | dQ(1)
+    // with one ring of LDS fragments, read PD ahead, running through all 48 operand fetches.
+    // BUF: stage that holds this tile (0 / 1), or -1 to take it from the parity of t.
+    auto tile_step = [&](auto masked_tag, auto copy_tag, auto buf_tag, int t) {
         constexpr bool MASKED = decltype(masked_tag)::value;
         constexpr int COPY = decltype(copy_tag)::value;
-        const int buf = t & 1;
+        constexpr int BUF = decltype(buf_tag)::value;
+        constexpr int PD = 4;
+        static_assert(DC % PD == 0 && (2 * DB) % PD == 0, "read-ahead depth must divide the fragment counts");
+        const int buf = BUF >= 0 ? BUF : (t & 1);
         if (COPY == 1) issue_full_tile(t + 1, buf ^ 1);
         else if (t + 1 < n_tiles) issue_tile(t + 1, buf ^ 1);
         const uint16_t* ks = lds + buf * T::STAGE_ELEMS;
         const uint16_t* vs = ks + T::TILE_ELEMS;
         const int key0 = t * BN;
 
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {       // two blocks of 32 keys per tile
-            // ---- S^T = K Q^T and dP^T = V dO^T : rows = keys, columns = queries
-            f32x16 sacc, dpacc;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                sacc[r] = 0.f;
-                dpacc[r] = 0.f;
+        // operand fetch f of the tile, in consumption order
+        constexpr int NROW = 4 * DC;                // row-read fragments: S(0), dP(0), S(1), dP(1)
+        constexpr int NALL = NROW + 4 * DB;         // + the transposed K fragments of dQ(0), dQ(1)
+        auto fetch = [&](int f) {
+            if (f < NROW) {
+                const int phase = f / DC, dc = f % DC;            // phase: 0 S(0), 1 dP(0), 2 S(1), 3 dP(1)
+                return *reinterpret_cast<const bf16x8*>(((phase & 1) ? vs : ks) + koff[dc] + 32 * (phase >> 1) * RS);
             }
-            {
-                constexpr int NF = 2 * DC, PD = 4;
-                bf16x8 fb[PD];
-                auto rd = [&](int i) {
-                    return *reinterpret_cast<const bf16x8*>(((i & 1) ? vs : ks) + koff[i >> 1] + 32 * kb * RS);
-                };
+            const int g = f - NROW, cc = g / DB, db = g % DB;      // cc = 16-key chunk of the tile
+            const u32x2 lo = lds_read_tr16(ks + toff[0][db] + 16 * cc * RS);
+            const u32x2 hi = lds_read_tr16(ks + toff[1][db] + 16 * cc * RS);
+            const u32x4 u = {lo[0], lo[1], hi[0], hi[1]};
+            return __builtin_bit_cast(bf16x8, u);
+        };
+        bf16x8 fb[PD];
 #pragma unroll
-                for (int i = 0; i < PD; ++i) {
-                    fb[i] = rd(i);
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-#pragma unroll
-                for (int i = 0; i < NF; ++i) {
-                    const int dc = i >> 1;
-                    if (i & 1) dpacc = mfma32(fb[i % PD], dof[dc], dpacc);
-                    else sacc = mfma32(fb[i % PD], qf[dc], sacc);
-                    if (i + PD < NF) fb[i % PD] = rd(i + PD);
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-            }
-            // ---- P^T and dS^T: one query per lane, so LSE and delta are per-lane scalars
-            const int kblk0 = key0 + 32 * kb;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                float pr = exp2_fast(fmaf(sacc[r], c_log2, -lse2));
-                if (MASKED) {
-                    const int key = kblk0 + acc_row(r, h);
-                    bool drop = key >= klimit;
-                    if (p.m.causal) drop = drop || key > qrow;
-                    if (HASMASK) {
-                        if (!drop && qok) drop = mbase[(int64_t)qrow * p.m.sq + (int64_t)key * p.m.sk] == 0;
-                    }
-                    pr = drop ? 0.f : pr;
-                }
-                dpacc[r] = pr * (dpacc[r] - delta);
-            }
-            const bf16x8 ds0 = pack8(dpacc[0], dpacc[1], dpacc[2], dpacc[3], dpacc[4], dpacc[5], dpacc[6], dpacc[7]);
-            const bf16x8 ds1 = pack8(dpacc[8], dpacc[9], dpacc[10], dpacc[11], dpacc[12], dpacc[13], dpacc[14], dpacc[15]);
-            // ---- dQ^T += K^T dS^T : rows = d, columns = queries, contraction over the 32 keys
-            {
-                constexpr int NF = 2 * DB, PD = 4;
-                bf16x8 fb[PD];
-                auto rd = [&](int i) {
-                    const int c = i / DB, db = i % DB, cc = 2 * kb + c;
-                    const u32x2 lo = lds_read_tr16(ks + toff[0][db] + 16 * cc * RS);
-                    const u32x2 hi = lds_read_tr16(ks + toff[1][db] + 16 * cc * RS);
-                    const u32x4 u = {lo[0], lo[1], hi[0], hi[1]};
-                    return __builtin_bit_cast(bf16x8, u);
-                };
-#pragma unroll
-                for (int i = 0; i < PD && i < NF; ++i) {
-                    fb[i] = rd(i);
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-#pragma unroll
-                for (int i = 0; i < NF; ++i) {
-                    const int c = i / DB, db = i % DB;
-                    dqacc[db] = mfma32(fb[i % PD], c == 0 ? ds0 : ds1, dqacc[db]);
-                    if (i + PD < NF) fb[i % PD] = rd(i + PD);
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-            }
+        for (int i = 0; i < PD; ++i) {
+            fb[i] = fetch(i);
+            __builtin_amdgcn_sched_barrier(0);
         }
+
+        f32x16 sacc[2], dpacc[2];
+        bf16x8 dsf[2][2];
+        auto p_elem = [&](int kb, int r) {          // P^T: one query per lane, so LSE is a per-lane scalar
+            float pr = exp2_fast(fmaf(sacc[kb][r], c_log2, -lse2));
+            if (MASKED) {
+                const int key = key0 + 32 * kb + acc_row(r, h);
+                bool drop = key >= klimit;
+                if (p.m.causal) drop = drop || key > qrow;
+                if (HASMASK) {
+                    if (!drop && qok) drop = mbase[(int64_t)qrow * p.m.sq + (int64_t)key * p.m.sk] == 0;
+                }
+                pr = drop ? 0.f : pr;
+            }
+            sacc[kb][r] = pr;
+        };
+        auto ds_elem = [&](int kb, int r) {         // dS^T = P^T (dP^T - delta), packed after 8 and 16
+            dpacc[kb][r] = sacc[kb][r] * (dpacc[kb][r] - delta);
+            if ((r & 7) == 7) {
+                const int o8 = r - 7;
+                const f32x16& d = dpacc[kb];
+                dsf[kb][r >> 3] = pack8(d[o8], d[o8 + 1], d[o8 + 2], d[o8 + 3], d[o8 + 4], d[o8 + 5], d[o8 + 6], d[o8 + 7]);
+            }
+        };
+        constexpr int EPM = 16 / DC;                // logits per MFMA slot in the row phases
+        constexpr int EPQ = 16 / (2 * DB);          // ... and in the dQ phases
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                sacc[kb][r] = 0.f;
+                dpacc[kb][r] = 0.f;
+            }
+        auto row_phase = [&](auto phase_tag) {
+            constexpr int PH = decltype(phase_tag)::value, KB = PH >> 1;
+#pragma unroll
+            for (int dc = 0; dc < DC; ++dc) {
+                constexpr int F0 = PH * DC;
+                const int f = F0 + dc;
+                if (PH & 1) dpacc[KB] = mfma32(fb[f % PD], dof[dc], dpacc[KB]);
+                else sacc[KB] = mfma32(fb[f % PD], qf[dc], sacc[KB]);
+                fb[f % PD] = fetch(f + PD);
+#pragma unroll
+                for (int e = 0; e < EPM; ++e) {
+                    const int r = EPM * dc + e;
+                    if (PH == 1) p_elem(0, r);
+                    if (PH == 2) ds_elem(0, r);
+                    if (PH == 3) p_elem(1, r);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        };
+        auto dq_phase = [&](auto kb_tag) {
+            constexpr int KB = decltype(kb_tag)::value;
+#pragma unroll
+            for (int g = 0; g < 2 * DB; ++g) {
+                const int f = NROW + 2 * DB * KB + g, c = g / DB, db = g % DB;
+                dqacc[db] = mfma32(fb[f % PD], dsf[KB][c], dqacc[db]);
+                if (f + PD < NALL) fb[f % PD] = fetch(f + PD);
+                if (KB == 0) {
+#pragma unroll
+                    for (int e = 0; e < EPQ; ++e) ds_elem(1, EPQ * g + e);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        };
+        row_phase(std::integral_constant<int, 0>{});
+        row_phase(std::integral_constant<int, 1>{});
+        row_phase(std::integral_constant<int, 2>{});
+        row_phase(std::integral_constant<int, 3>{});
+        dq_phase(std::integral_constant<int, 0>{});
+        dq_phase(std::integral_constant<int, 1>{});
 
         wait_vm0();
         __syncthreads();
@@ -693,11 +721,19 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams p) {
     int n_full = HASMASK ? 0 : klimit / BN;
     if (p.m.causal) n_full = min(n_full, (q0 + 1) / BN);
     n_full = min(n_full, n_tiles);
+    using IM = std::integral_constant<int, -1>;
+    using I0 = std::integral_constant<int, 0>;
     using I1 = std::integral_constant<int, 1>;
     using I2 = std::integral_constant<int, 2>;
-    for (int t = 0; t < n_full - 1; ++t) tile_step(std::false_type{}, I1{}, t);
-    if (n_full > 0) tile_step(std::false_type{}, I2{}, n_full - 1);
-    for (int t = n_full; t < n_tiles; ++t) tile_step(std::true_type{}, I2{}, t);
+    {
+        int t = 0;
+        for (; t + 2 < n_full; t += 2) {      // tiles t+1 and t+2 are full: straight-line copies, fixed stages
+            tile_step(std::false_type{}, I1{}, I0{}, t);
+            tile_step(std::false_type{}, I1{}, I1{}, t + 1);
+        }
+        for (; t < n_full; ++t) tile_step(std::false_type{}, I2{}, IM{}, t);
+        for (; t < n_tiles; ++t) tile_step(std::true_type{}, I2{}, IM{}, t);
+    }
 
     // ---- epilogue: dQ = scale * dQ^T, bf16
     if (qok) {
