@@ -46,6 +46,30 @@ def cpu_baseline(w, max_seconds_hint=30.0):
             "seconds": dt}
 
 
+def input_prep_rate(capi, W, torch, B, H, N, D, dev, iters=20):
+    """Fused RMS-norm + RoPE + layout change of one [B,N,H,D] projection output (the caller of the hot
+    path on the input side), outside the timed step: HBM-bound, reported against 8 TB/s."""
+    x = torch.randn((B, N, H, D), device=dev, dtype=torch.float32).to(torch.bfloat16)
+    wgt = torch.ones((D,), device=dev, dtype=torch.bfloat16)
+    side = int(round((N - 512) ** 0.5))
+    cos, sin = W.axial_rope_tables(N - side * side, side, side, D)
+    cos, sin = torch.from_numpy(cos).to(dev), torch.from_numpy(sin).to(dev)
+    y = torch.empty((B, H, N, D), device=dev, dtype=torch.bfloat16)
+    for _ in range(3):
+        capi.prep_rmsnorm_rope(x, wgt, cos, sin, out=y)
+    torch.cuda.synchronize()
+    capi.profiling_enable(True)
+    for _ in range(iters):
+        capi.prep_rmsnorm_rope(x, wgt, cos, sin, out=y)
+    torch.cuda.synchronize()
+    tot, n = capi.profiling_read()["input_prep"]
+    capi.profiling_enable(False)
+    ms = tot / max(n, 1)
+    nbytes = 2 * x.numel() * 2 + 2 * cos.numel() * 4 + D * 2       # read x, write y, read both tables and the scale
+    return {"kernel": "prep_qk_kernel", "ms_per_tensor": ms, "algorithmic_bytes": nbytes,
+            "GB_per_s": nbytes / (ms * 1e-3) / 1e9, "frac_of_hbm_peak": nbytes / (ms * 1e-3) / 8e12}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -136,6 +160,8 @@ def main():
         "kernels_ms": per_kernel,
         "saved_activations": w.saved_activation_bytes(),
     }
+    if args.config == 2:
+        out["input_prep"] = input_prep_rate(capi, W, torch, B, H, Sq, D, dev)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(w)
     print(json.dumps(out))

@@ -110,7 +110,7 @@ def attn_bwd(q, k, v, o, do, lse, scale, causal=False, kv_len=None, mask=None, w
     return dq, dk, dv
 
 
-KERNEL_KINDS = ("fwd", "bwd_prep", "bwd_dkdv", "bwd_dq", "sage_kmean", "sage_quant", "sage_fwd", "reserved")
+KERNEL_KINDS = ("fwd", "bwd_prep", "bwd_dkdv", "bwd_dq", "sage_kmean", "sage_quant", "sage_fwd", "input_prep")
 
 
 class _KernelTimes(ctypes.Structure):
@@ -168,3 +168,29 @@ def sage_fwd(qz, v, scale, causal=False, kv_len=None, want_lse=False, out=None):
     if rc != 0:
         raise FlameAttnError("flame_sage_attn_fwd_int8", rc)
     return (o, lse) if want_lse else o
+
+
+def prep_rmsnorm_rope(x_bnhd, weight=None, cos=None, sin=None, eps=1e-6, apply_norm=True, out=None):
+    """Fused RMS-norm over the head dim + interleaved RoPE + [B,N,H,D] -> [B,H,N,D].
+
+    x_bnhd: bf16 [B,N,H,D] (any B/N/H strides); weight: bf16 [D] or None; cos/sin: [N,D/2] fp32 or
+    bf16, or None.  Returns a contiguous bf16 [B,H,N,D] tensor."""
+    B, N, H, D = x_bnhd.shape
+    xv = x_bnhd.permute(0, 2, 1, 3)                       # logical [B,H,N,D] view of the same memory
+    if out is None:
+        out = torch.empty((B, H, N, D), dtype=torch.bfloat16, device=x_bnhd.device)
+    tdt = 0
+    if cos is not None:
+        if cos.dtype != sin.dtype or cos.shape != sin.shape or tuple(cos.shape) != (N, D // 2):
+            raise ValueError("cos/sin must both be [N, D/2] of one dtype")
+        if not (cos.is_contiguous() and sin.is_contiguous()):
+            raise ValueError("cos/sin must be contiguous")
+        tdt = 1 if cos.dtype == torch.float32 else 0
+    rc = lib().flame_attn_prep_rmsnorm_rope_bf16(
+        _ptr(xv), _ptr(weight) if weight is not None else None,
+        _ptr(cos) if cos is not None else None, _ptr(sin) if sin is not None else None, tdt,
+        _ptr(out), B, H, N, D, ctypes.c_float(eps), int(bool(apply_norm)),
+        _i64x4(xv.stride()), _i64x4(out.stride()), ctypes.c_int64(0), ctypes.c_int64(0), _stream())
+    if rc != 0:
+        raise FlameAttnError("flame_attn_prep_rmsnorm_rope_bf16", rc)
+    return out

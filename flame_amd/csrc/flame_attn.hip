@@ -13,6 +13,7 @@
 
 #include "attn_bwd.hpp"
 #include "attn_fwd.hpp"
+#include "prep.hpp"
 #include "sage.hpp"
 
 using namespace fattn;
@@ -594,6 +595,46 @@ int flame_attn_cast_f32_to_bf16(const void* src_f32, void* dst_bf16, int64_t n, 
     hipLaunchKernelGGL(cast_f32_to_bf16_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
                        static_cast<hipStream_t>(stream), static_cast<const float*>(src_f32),
                        static_cast<uint16_t*>(dst_bf16), n);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? FLAME_ATTN_OK : (int)e;
+}
+
+int flame_attn_prep_rmsnorm_rope_bf16(const void* X, const void* weight, const void* cos, const void* sin,
+                                      int table_dtype, void* Y, int B, int H, int N, int D, float eps,
+                                      int apply_norm, const int64_t* x_strides, const int64_t* y_strides,
+                                      int64_t x_off, int64_t y_off, void* stream) {
+    if (!X || !Y || !x_strides || !y_strides || B <= 0 || H <= 0 || N <= 0) return FLAME_ATTN_ERR_INVALID;
+    if ((cos == nullptr) != (sin == nullptr)) return FLAME_ATTN_ERR_INVALID;
+    if (D != 64 && D != 128) return FLAME_ATTN_ERR_UNSUPPORTED;
+    if (table_dtype != FLAME_ATTN_DTYPE_BF16 && table_dtype != FLAME_ATTN_DTYPE_F32) return FLAME_ATTN_ERR_INVALID;
+    if (int rc = check_view(X, x_strides, x_off)) return rc;
+    if (int rc = check_view(Y, y_strides, y_off)) return rc;
+    if (weight && !aligned16(weight)) return FLAME_ATTN_ERR_UNSUPPORTED;
+    if (cos && (!aligned16(cos) || !aligned16(sin))) return FLAME_ATTN_ERR_UNSUPPORTED;
+    PrepParams p{};
+    p.x = static_cast<const uint16_t*>(X) + x_off;
+    p.y = static_cast<uint16_t*>(Y) + y_off;
+    p.w = static_cast<const uint16_t*>(weight);
+    p.cos_t = cos;
+    p.sin_t = sin;
+    p.xs = mk(x_strides);
+    p.ys = mk(y_strides);
+    p.B = B;
+    p.H = H;
+    p.N = N;
+    p.eps = eps;
+    p.norm = apply_norm ? 1 : 0;
+    p.table_f32 = table_dtype == FLAME_ATTN_DTYPE_F32;
+    const int64_t rows = (int64_t)B * H * N;
+    const int rpb = 256 / (D / 8);
+    const int64_t grid = (rows + rpb - 1) / rpb;
+    if (grid > 0x7fffffff) return FLAME_ATTN_ERR_UNSUPPORTED;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    {
+        ScopedKernelTimer t(FLAME_ATTN_KERNEL_INPUT_PREP, s);
+        if (D == 128) hipLaunchKernelGGL(prep_qk_kernel<128>, dim3((unsigned)grid), dim3(256), 0, s, p);
+        else hipLaunchKernelGGL(prep_qk_kernel<64>, dim3((unsigned)grid), dim3(256), 0, s, p);
+    }
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? FLAME_ATTN_OK : (int)e;
 }

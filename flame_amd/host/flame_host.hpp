@@ -486,6 +486,68 @@ inline Result<std::tuple<Tensor, Tensor, Tensor>> sdpa_backward(const SdpaCtx& c
 
 }  // namespace autograd_v4
 
+// ------------------------------------------------------------------------------------ input preparation
+// Counterparts of the reference's rope_fused_bf16 / rope_fused_bf16_f32pe (src/bf16_ops.rs:476-582,
+// x [B,H,N,D], tables [1,1,N,D/2]) and of its per-head RMSNorm (src/norm.rs:1090-1092,
+// x * weight / sqrt(mean(x^2) + eps) over the last dim), plus the fused form that reads the
+// projection output [B,N,H,D] and returns the normalised, rotated [B,H,N,D] tensor in one pass.
+namespace bf16_ops {
+namespace detail_prep {
+inline Result<Tensor> run(const Tensor& x_bhnd, const Tensor* weight, const Tensor* cos, const Tensor* sin, float eps,
+                          bool apply_norm, const char* who) {
+    if (x_bhnd.shape().size() != 4) return invalid(std::string(who) + ": expected 4D [B,H,N,D]");
+    if (x_bhnd.dtype() != DType::BF16) return invalid(std::string(who) + ": expects BF16");
+    const auto& sh = x_bhnd.shape();
+    const int64_t B = sh[0], H = sh[1], N = sh[2], D = sh[3];
+    int tdt = FLAME_ATTN_DTYPE_BF16;
+    if ((cos == nullptr) != (sin == nullptr)) return invalid(std::string(who) + ": cos and sin go together");
+    if (cos) {
+        if (cos->dtype() != sin->dtype() || (cos->dtype() != DType::BF16 && cos->dtype() != DType::F32))
+            return invalid(std::string(who) + ": cos/sin must both be BF16 or both F32");
+        if (cos->numel() != N * (D / 2) || sin->numel() != N * (D / 2) || !cos->is_contiguous() || !sin->is_contiguous())
+            return invalid(std::string(who) + ": cos/sin must be contiguous [1,1,N,D/2]");
+        tdt = cos->dtype() == DType::F32 ? FLAME_ATTN_DTYPE_F32 : FLAME_ATTN_DTYPE_BF16;
+    }
+    if (weight && (weight->dtype() != DType::BF16 || weight->numel() != D)) return invalid(std::string(who) + ": weight must be BF16 [D]");
+    auto y = Tensor::empty({B, H, N, D}, DType::BF16);
+    if (!y.ok()) return y.error();
+    const int rc = flame_attn_prep_rmsnorm_rope_bf16(x_bhnd.base(), weight ? weight->data() : nullptr, cos ? cos->data() : nullptr,
+                                                     sin ? sin->data() : nullptr, tdt, y.value().base(), (int)B, (int)H, (int)N,
+                                                     (int)D, eps, apply_norm ? 1 : 0, x_bhnd.strides().data(),
+                                                     y.value().strides().data(), x_bhnd.offset(), 0, nullptr);
+    if (rc == FLAME_ATTN_ERR_UNSUPPORTED) return unsupported(std::string(who) + ": head dim or layout not built");
+    if (rc == FLAME_ATTN_ERR_INVALID) return invalid(std::string(who) + ": bad arguments");
+    if (rc != 0) return cuda_error(who, rc);
+    return y.value();
+}
+}  // namespace detail_prep
+
+inline Result<Tensor> rope_fused_bf16(const Tensor& x, const Tensor& cos, const Tensor& sin) {
+    if (cos.dtype() != DType::BF16 || sin.dtype() != DType::BF16) return invalid("rope_fused_bf16: cos/sin must be BF16");
+    return detail_prep::run(x, nullptr, &cos, &sin, 0.f, false, "rope_fused_bf16");
+}
+inline Result<Tensor> rope_fused_bf16_f32pe(const Tensor& x, const Tensor& cos, const Tensor& sin) {
+    if (cos.dtype() != DType::F32 || sin.dtype() != DType::F32) return invalid("rope_fused_bf16_f32pe: cos/sin must be F32");
+    return detail_prep::run(x, nullptr, &cos, &sin, 0.f, false, "rope_fused_bf16_f32pe");
+}
+}  // namespace bf16_ops
+
+namespace norm {
+// RMSNorm over the last (head) dim of a 4-D tensor.
+inline Result<Tensor> rms_norm(const Tensor& x, const Tensor* weight, float eps) {
+    return bf16_ops::detail_prep::run(x, weight, nullptr, nullptr, eps, true, "rms_norm");
+}
+}  // namespace norm
+
+namespace attention {
+// x: projection output [B,N,H,D] (any strides over B, N, H).  Returns rope(rms_norm(x) * weight) as
+// contiguous [B,H,N,D]; weight and the tables are optional.
+inline Result<Tensor> prep_qk(const Tensor& x_bnhd, const Tensor* weight, const Tensor* cos, const Tensor* sin, float eps = 1e-6f) {
+    if (x_bnhd.shape().size() != 4) return invalid("prep_qk: expected 4D [B,N,H,D]");
+    return bf16_ops::detail_prep::run(x_bnhd.permute({0, 2, 1, 3}), weight, cos, sin, eps, true, "prep_qk");
+}
+}  // namespace attention
+
 // ------------------------------------------------------------------------------------ SageAttention
 // Builder-style API of the reference (src/sage_attention.rs:21-65).  `scale` is the softmax scale
 // (default 1/sqrt(D)); the reference's field of the same name is a divisor defaulting to sqrt(D)

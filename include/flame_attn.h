@@ -187,7 +187,7 @@ bool sdpa_stream_bf16_launch(const void* dQ, const void* dK, const void* dV, voi
  * ---------------------------------------------------------------------------------------------- */
 enum { FLAME_ATTN_KERNEL_FWD = 0, FLAME_ATTN_KERNEL_BWD_PREP = 1, FLAME_ATTN_KERNEL_BWD_DKDV = 2,
        FLAME_ATTN_KERNEL_BWD_DQ = 3, FLAME_ATTN_KERNEL_SAGE_KMEAN = 4, FLAME_ATTN_KERNEL_SAGE_QUANT = 5,
-       FLAME_ATTN_KERNEL_SAGE_FWD = 6, FLAME_ATTN_N_KERNEL_KINDS = 8 };
+       FLAME_ATTN_KERNEL_SAGE_FWD = 6, FLAME_ATTN_KERNEL_INPUT_PREP = 7, FLAME_ATTN_N_KERNEL_KINDS = 8 };
 typedef struct {
     double total_ms[FLAME_ATTN_N_KERNEL_KINDS];
     int launches[FLAME_ATTN_N_KERNEL_KINDS];
@@ -212,6 +212,24 @@ int flame_attn_convert_keep_mask(const void* src, int src_dtype, void* dst_u8, i
  * upstream gradient to the bf16 backward instead of falling back to the materialising recompute as
  * the reference does (src/autograd.rs:702-705). */
 int flame_attn_cast_f32_to_bf16(const void* src_f32, void* dst_bf16, int64_t n, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Fused input preparation for joint attention: RMS normalisation over the head dim, interleaved-
+ * pair rotary embedding and the [B,N,H,D] -> [B,H,N,D] layout change in one pass.  Replaces, run
+ * back to back and with the same bf16 rounding between them,
+ *   flame_fused_rms_norm_bf16   src/cuda/fused_rms_norm.cu:89-111  (src/norm.rs:686-732)
+ *   rope_fused_bf16 / rope_fused_bf16_f32pe   src/bf16_ops.rs:361-394, :476-582 (tables [1,1,N,D/2])
+ *   the permute that makes [B,H,N,D] contiguous   cuda/permute0213.cu
+ * X is read through element strides given in (B,H,N,D) order (D stride must be 1, the others and the
+ * offsets multiples of 8), so a [B,N,H,D] buffer is passed as strides (N*H*D, D, H*D, 1).
+ * weight: [D] bf16 or null; eps as in the reference's RMSNorm; apply_norm = 0 skips the normalisation.
+ * cos, sin: contiguous [N, D/2], bf16 (table_dtype = FLAME_ATTN_DTYPE_BF16) or fp32; null skips the
+ * rotation.  D in {64, 128}.
+ * ---------------------------------------------------------------------------------------------- */
+int flame_attn_prep_rmsnorm_rope_bf16(const void* X, const void* weight, const void* cos, const void* sin,
+                                      int table_dtype, void* Y, int B, int H, int N, int D, float eps,
+                                      int apply_norm, const int64_t* x_strides, const int64_t* y_strides,
+                                      int64_t x_off, int64_t y_off, void* stream);
 
 const char* flame_attn_version(void);
 

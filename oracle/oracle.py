@@ -188,3 +188,36 @@ def cosine(a, b) -> float:
     b = np.asarray(b, np.float64).ravel()
     den = np.linalg.norm(a) * np.linalg.norm(b)
     return float(a @ b / den) if den > 0 else 1.0
+
+
+def prep_rmsnorm_rope(x_bnhd, weight=None, cos=None, sin=None, eps=1e-6, apply_norm=True):
+    """Input preparation of joint attention, restated from the reference's two kernels run back to back.
+
+    x_bnhd: uint16 bf16 bits [B,N,H,D]; weight: bf16 bits [D] or None; cos/sin: fp32 [N,D/2] (pass
+    bf16 tables already widened to fp32).  Returns bf16 bits [B,H,N,D].
+
+      fused_rms_norm.cu:26-86   v = bf16(x * rsqrt(mean(x^2) + eps) * w), fp32 arithmetic
+      bf16_ops.rs:361-394       y[2p] = bf16(v[2p] c - v[2p+1] s), y[2p+1] = bf16(v[2p] s + v[2p+1] c)
+
+    Plain IEEE fp32 without contraction; the mean of squares is accumulated in fp64 and rounded once
+    (the reference's summation order is a property of its launch shape, not of the algorithm).
+    Pinned by the reference's RoPE known-answer test and by closed forms (see tests)."""
+    x = bf16_to_f32(np.asarray(x_bnhd))
+    if apply_norm:
+        ms = np.mean(x.astype(np.float64) ** 2, axis=-1, keepdims=True).astype(np.float32)
+        with np.errstate(divide="ignore", invalid="ignore"):       # eps = 0 on an all-zero row
+            rs = (np.float32(1.0) / np.sqrt(ms + np.float32(eps), dtype=np.float32)).astype(np.float32)
+            v = (x * rs).astype(np.float32)
+        if weight is not None:
+            v = (v * bf16_to_f32(np.asarray(weight))).astype(np.float32)
+        x = bf16_to_f32(f32_to_bf16(v))
+    x = np.ascontiguousarray(np.transpose(x, (0, 2, 1, 3)))          # [B,H,N,D]
+    if cos is not None:
+        c = np.asarray(cos, np.float32)[None, None]
+        s_ = np.asarray(sin, np.float32)[None, None]
+        e, o = x[..., 0::2], x[..., 1::2]
+        y = np.empty_like(x)
+        y[..., 0::2] = (e * c).astype(np.float32) - (o * s_).astype(np.float32)
+        y[..., 1::2] = (e * s_).astype(np.float32) + (o * c).astype(np.float32)
+        x = y
+    return f32_to_bf16(x)

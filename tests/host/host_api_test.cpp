@@ -304,6 +304,48 @@ int main() {
         CHECK(!SageAttention().forward(q, k, v, &m).ok(), "sage + mask must be refused");
     }
 
+    // ---- 7. input preparation: fused RMS-norm + RoPE + [B,N,H,D]->[B,H,N,D] equals the three separate calls,
+    //         and the rotation matches the scalar formula of the reference test (src/tests/attention_tests.rs:8-34)
+    {
+        std::printf("[input prep]\n");
+        const int B = 1, N = 40, H = 3, D = 128;
+        auto hx = randn_bf16((size_t)B * N * H * D);
+        Tensor x_bnhd = dev_bf16(hx, {B, N, H, D});
+        std::vector<float> hc((size_t)N * D / 2), hs(hc.size());
+        for (int n = 0; n < N; ++n)
+            for (int p2 = 0; p2 < D / 2; ++p2) {
+                const double ang = n * std::pow(10000.0, -2.0 * p2 / D);
+                hc[(size_t)n * (D / 2) + p2] = (float)std::cos(ang);
+                hs[(size_t)n * (D / 2) + p2] = (float)std::sin(ang);
+            }
+        Tensor cos = Tensor::from_host(hc.data(), {1, 1, N, D / 2}, DType::F32).value();
+        Tensor sin = Tensor::from_host(hs.data(), {1, 1, N, D / 2}, DType::F32).value();
+        auto fused = attention::prep_qk(x_bnhd, nullptr, &cos, &sin, 1e-6f);
+        auto normed = norm::rms_norm(x_bnhd.permute({0, 2, 1, 3}), nullptr, 1e-6f);
+        CHECK(fused.ok() && normed.ok(), "prep calls failed");
+        if (fused.ok() && normed.ok()) {
+            auto roped = bf16_ops::rope_fused_bf16_f32pe(normed.value(), cos, sin);
+            CHECK(roped.ok(), "rope_fused_bf16_f32pe failed");
+            auto a = host_f32_of_bf16(fused.value()), b2 = host_f32_of_bf16(roped.value()), nv = host_f32_of_bf16(normed.value());
+            size_t diff = 0;
+            for (size_t i = 0; i < a.size(); ++i) diff += a[i] != b2[i];
+            CHECK(diff == 0, "fused != norm-then-rope in %zu elements", diff);
+            double worst = 0;
+            for (int h = 0; h < H; ++h)
+                for (int n = 0; n < N; ++n)
+                    for (int p2 = 0; p2 < D / 2; ++p2) {
+                        const size_t o = (((size_t)h * N + n) * D) + 2 * p2;
+                        const double c = hc[(size_t)n * (D / 2) + p2], s2 = hs[(size_t)n * (D / 2) + p2];
+                        worst = std::fmax(worst, std::fabs(nv[o] * c - nv[o + 1] * s2 - a[o]));
+                        worst = std::fmax(worst, std::fabs(nv[o] * s2 + nv[o + 1] * c - a[o + 1]));
+                    }
+            std::printf("  rotation vs scalar formula: max_abs=%.3e\n", worst);
+            CHECK(worst <= 2e-2, "rotation max_abs %.3e", worst);
+        }
+        Tensor bad = Tensor::empty({1, 1, N, D / 2}, DType::BF16).value();
+        CHECK(!bf16_ops::rope_fused_bf16_f32pe(normed.value(), bad, bad).ok(), "f32pe must refuse bf16 tables");
+    }
+
     if (hipDeviceSynchronize() != hipSuccess) ++g_fail;
     std::printf(g_fail ? "HOST API TEST: %d FAILURES\n" : "HOST API TEST: all checks passed\n", g_fail);
     return g_fail ? 1 : 0;
