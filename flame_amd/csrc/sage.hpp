@@ -6,11 +6,15 @@
 //   sage_quant_kernel   Ks = bf16(float(K) - kmean); per 128-row Q block and per 64-row Ks block:
 //                       scale = absmax/127 (IEEE division), code = clamp(rint(x/scale), -128, 127)
 //   sage_fwd_kernel     S^T = K^ Q^^T on v_mfma_i32_32x32x32_i8 (int32 accumulate), dequantised with
-//                       sq*sk*scale, online softmax in fp32, P -> bf16, O^T = V^T P^T on bf16 MFMA
+//                       sq*sk*scale, online softmax in fp32, P -> bf16, O^T = V^T P^T on bf16 MFMA;
+//                       same tile walk, LDS-DMA staging and in-wave software pipeline as the bf16
+//                       forward kernel (the int8 K tile is half the size, the logit MFMAs half as many)
 //
 // Quantisation closed form follows the reference's sage_quantize_tensor
 // (src/sage_attention.rs:524-541); block granularity, mean smoothing and the int8 MFMA are new.
 #pragma once
+#include <type_traits>
+
 #include "attn_common.hpp"
 
 namespace fattn {
@@ -172,27 +176,44 @@ struct SageFwdParams {
 template <int D>
 struct SageTile {
     static constexpr int BM = 128, BN = 64;
-    static constexpr int KSB = D + 16;            // bytes per row of the int8 K tile
-    static constexpr int VS = D + 32;             // elements per row of the bf16 V tile (transposing reads)
-    static constexpr int K_BYTES = BN * KSB;
-    static constexpr int V_BYTES = BN * VS * 2;
+    static constexpr int K_BYTES = BN * D;             // int8 K tile, row-major, swizzled, no padding
+    static constexpr int V_BYTES = BN * D * 2;         // bf16 V tile, likewise
     static constexpr int STAGE_BYTES = K_BYTES + V_BYTES;
     static constexpr int LDS_BYTES = 2 * STAGE_BYTES;
-    static constexpr int NKC = BN * (D / 16) / 256;   // 16-byte int8 chunks per thread (D=128: 2, D=64: 1)
-    static constexpr int NVC = BN * (D / 8) / 256;    // 16-byte bf16 chunks per thread
+    static constexpr int K_DMA_PER_WAVE = K_BYTES / 1024 / 4;
+    static constexpr int V_DMA_PER_WAVE = V_BYTES / 1024 / 4;
 };
 
+// granule swizzle of the int8 K tile (rows of D bytes): 16-byte row reads by 16 adjacent rows hit 16
+// distinct bank groups
 template <int D>
-__global__ __launch_bounds__(256) void sage_fwd_kernel(const SageFwdParams p) {
-    using T = SageTile<D>;
-    constexpr int BM = T::BM, BN = T::BN, KSB = T::KSB, VS = T::VS;
-    constexpr int DC = D / 32;   // int8 contraction chunks (32 per MFMA)
-    constexpr int DB = D / 32;
+__device__ __forceinline__ constexpr int swz_i8(int row) {
+    return D == 128 ? swz<64>(row) : ((row >> 2) & 3);
+}
 
-    extern __shared__ __attribute__((aligned(16))) uint8_t lds8[];
+template <int D>
+__global__ __launch_bounds__(256, 2) void sage_fwd_kernel(const SageFwdParams p) {
+    using T = SageTile<D>;
+    constexpr int BM = T::BM, BN = T::BN;
+    constexpr int KC = D / 32;   // int8 contraction chunks (32 per MFMA)
+    constexpr int DB = D / 32;   // 32-row blocks of O^T
+    constexpr int RS = D;        // V row stride, elements
+    constexpr int GPK = D / 16;  // 16-byte granules per K^ row
+    constexpr int GPV = D / 8;   // ... per V row
+    constexpr int NKD = T::K_DMA_PER_WAVE, NVD = T::V_DMA_PER_WAVE;
+    constexpr int PD = 4;
+    constexpr int NS = 2 * KC;   // logit MFMAs per tile
+    constexpr int NP = 4 * DB;   // PV MFMAs per tile
+    static_assert(NS % PD == 0 && NP % PD == 0, "read-ahead depth must divide the fragment counts");
+    constexpr int EPS = 32 / NS; // logits per softmax slice
+    constexpr int MPS = 32 / NP; // logits per maximum-scan slice
+    static_assert(MPS % 2 == 0, "maximum scan takes logits in pairs");
+
+    extern __shared__ __attribute__((aligned(1024))) uint8_t lds8[];
 
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 31, h = lane >> 5;
 
     const int n_qt = (p.Sq + BM - 1) / BM;
@@ -217,147 +238,280 @@ __global__ __launch_bounds__(256) void sage_fwd_kernel(const SageFwdParams p) {
     const int n_tiles = (kend + BN - 1) / BN;
 
     // Q^ fragments: column = query, 16 consecutive int8 of the contraction per lane
-    i32x4 qf[DC];
+    i32x4 qf[KC];
     {
         const int row = qw0 + n;
         const i32x4 z = {0, 0, 0, 0};
 #pragma unroll
-        for (int dc = 0; dc < DC; ++dc)
-            qf[dc] = row < p.Sq ? *reinterpret_cast<const i32x4*>(qbase + (int64_t)row * D + 32 * dc + 16 * h) : z;
+        for (int kc = 0; kc < KC; ++kc)
+            qf[kc] = row < p.Sq ? *reinterpret_cast<const i32x4*>(qbase + (int64_t)row * D + 32 * kc + 16 * h) : z;
     }
     // one quantisation block of Q per workgroup (BM == 128); fold softmax scale and log2(e)
     const float qfac = p.sq[(int64_t)bh * n_qt + qt] * p.scale * kLog2e;
 
-    u32x4 kreg[T::NKC], vreg[T::NVC];
-    auto load_tile = [&](int t) {
-        const int key0 = t * BN;
+    // ---- asynchronous tile copies: K^(t) and V(t) live in stage t&1
+    const uint32_t lds0 = lds_addr(lds8);
+    const int k_row_in = lane / GPK, k_gran = lane % GPK;
+    const int v_row_in = lane / GPV, v_gran = lane % GPV;
+    constexpr int RPK = 1024 / D, RPV = 1024 / (2 * D);      // rows per 1 KiB copy
+    uint32_t k_lane_off[NKD], v_lane_off[NVD];               // bytes
 #pragma unroll
-        for (int i = 0; i < T::NKC; ++i) {
-            const int c = tid + 256 * i;
-            const int row = c / (D / 16), col = c % (D / 16);
-            const int key = key0 + row;
-            const u32x4 z = {0u, 0u, 0u, 0u};
-            kreg[i] = key < p.Sk ? *reinterpret_cast<const u32x4*>(kbase + (int64_t)key * D + col * 16) : z;
-        }
+    for (int i = 0; i < NKD; ++i) {
+        const int row = (wave * NKD + i) * RPK + k_row_in;
+        k_lane_off[i] = (uint32_t)(row * D + ((k_gran ^ swz_i8<D>(row)) << 4));
+    }
 #pragma unroll
-        for (int i = 0; i < T::NVC; ++i) {
-            const int c = tid + 256 * i;
-            const int row = c / (D / 8), col = c % (D / 8);
-            const int key = key0 + row;
-            vreg[i] = ldg16(vbase + (int64_t)key * p.vs.n + col * 8, key < klimit);
+    for (int i = 0; i < NVD; ++i) {
+        const int row = (wave * NVD + i) * RPV + v_row_in;
+        v_lane_off[i] = 2u * (uint32_t)(row * (int)p.vs.n + ((v_gran ^ swz<D>(row)) << 3));
+    }
+    auto k_dst = [&](int t, int i) { return lds0 + (uint32_t)((t & 1) * T::STAGE_BYTES + (wave * NKD + i) * 1024); };
+    auto v_dst = [&](int t, int i) { return lds0 + (uint32_t)((t & 1) * T::STAGE_BYTES + T::K_BYTES + (wave * NVD + i) * 1024); };
+    auto issue_k = [&](int t) {                              // ragged: rows clamped into the attended range
+#pragma unroll
+        for (int i = 0; i < NKD; ++i) {
+            const int row = (wave * NKD + i) * RPK + k_row_in;
+            const int key = min(t * BN + row, klimit - 1);
+            dma16(kbase + (int64_t)key * D + ((k_gran ^ swz_i8<D>(row)) << 4), k_dst(t, i));
         }
     };
-    auto store_tile = [&](int buf) {
-        uint8_t* ks = lds8 + buf * T::STAGE_BYTES;
-        uint16_t* vs = reinterpret_cast<uint16_t*>(ks + T::K_BYTES);
+    auto issue_v = [&](int t) {
 #pragma unroll
-        for (int i = 0; i < T::NKC; ++i) {
-            const int c = tid + 256 * i;
-            const int row = c / (D / 16), col = c % (D / 16);
-            *reinterpret_cast<u32x4*>(ks + row * KSB + col * 16) = kreg[i];
+        for (int i = 0; i < NVD; ++i) {
+            const int row = (wave * NVD + i) * RPV + v_row_in;
+            const int key = min(t * BN + row, klimit - 1);
+            dma16(vbase + (int64_t)key * p.vs.n + ((v_gran ^ swz<D>(row)) << 3), v_dst(t, i));
         }
+    };
+    auto issue_full_kv = [&](int tk, int tv) {               // K^ tile tk and V tile tv, both full
+        const int8_t* kt = kbase + (int64_t)tk * BN * D;
+        const uint16_t* vt = vbase + (int64_t)tv * BN * p.vs.n;
 #pragma unroll
-        for (int i = 0; i < T::NVC; ++i) {
-            const int c = tid + 256 * i;
-            const int row = c / (D / 8), col = c % (D / 8);
-            *reinterpret_cast<u32x4*>(vs + row * VS + col * 8) = vreg[i];
-        }
+        for (int i = 0; i < NKD; ++i) dma16u(kt, k_lane_off[i], k_dst(tk, i));
+#pragma unroll
+        for (int i = 0; i < NVD; ++i) dma16u(vt, v_lane_off[i], v_dst(tv, i));
     };
 
-    float m_run = -INFINITY, l_run = 0.f;    // m_run in log2 units of the dequantised, scaled logits
+    // ---- per-lane LDS read offsets
+    int koff[KC];          // bytes: K^ fragment of row n, logical granule 2*kc + h
+#pragma unroll
+    for (int kc = 0; kc < KC; ++kc) koff[kc] = n * D + (((2 * kc + h) ^ swz_i8<D>(n)) << 4);
+    const int tr_r = lane & 15, tr_g16 = (lane >> 4) & 1;
+    int voff[2][DB];       // elements: V^T fragment halves, rows 4h + r/4 (+8)
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+        const int row = 4 * h + (tr_r >> 2) + 8 * half;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+            voff[half][db] = row * RS + (((4 * db + 2 * tr_g16 + ((tr_r & 3) >> 1)) ^ swz<D>(row)) << 3) + 4 * (tr_r & 1);
+    }
+    auto k_frag = [&](int t, int i) {       // fragment i = (kc, kb) of K^(t); rows 32*kb + n share the swizzle of row n
+        const uint8_t* ks = lds8 + (t & 1) * T::STAGE_BYTES;
+        return *reinterpret_cast<const u32x4*>(ks + koff[i >> 1] + 32 * (i & 1) * D);
+    };
+    auto v_frag = [&](int t, int i) {       // fragment i = (cc, db) of V(t)^T
+        const uint16_t* vs = reinterpret_cast<const uint16_t*>(lds8 + (t & 1) * T::STAGE_BYTES + T::K_BYTES);
+        const int cc = i / DB, db = i % DB;
+        const u32x2 lo = lds_read_tr16(vs + voff[0][db] + 16 * cc * RS);
+        const u32x2 hi = lds_read_tr16(vs + voff[1][db] + 16 * cc * RS);
+        const u32x4 u = {lo[0], lo[1], hi[0], hi[1]};
+        return u;
+    };
+
+    // ---- running state; m_run is in log2 units of the dequantised, scaled logits
+    float m_run = -INFINITY, l_run = 0.f;
     f32x16 oacc[DB];
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
         for (int r = 0; r < 16; ++r) oacc[db][r] = 0.f;
 
-    if (n_tiles > 0) {
-        load_tile(0);
-        store_tile(0);
-    }
-    __syncthreads();
-
-    for (int t = 0; t < n_tiles; ++t) {
-        const int buf = t & 1;
-        const bool more = (t + 1) < n_tiles;
-        if (more) load_tile(t + 1);
-        const uint8_t* ks = lds8 + buf * T::STAGE_BYTES;
-        const uint16_t* vs = reinterpret_cast<const uint16_t*>(ks + T::K_BYTES);
-        const int key0 = t * BN;
-
-        i32x16 iacc[2];
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) iacc[kb][r] = 0;
-#pragma unroll
-        for (int dc = 0; dc < DC; ++dc)
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
-                const i32x4 ka = *reinterpret_cast<const i32x4*>(ks + (32 * kb + n) * KSB + 32 * dc + 16 * h);
-                iacc[kb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ka, qf[dc], iacc[kb], 0, 0, 0);
-            }
-
-        const float f = qfac * skb[t];       // one K quantisation block per 64-key tile
-        f32x16 sacc[2];
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) sacc[kb][r] = (float)iacc[kb][r] * f;
-
-        const bool tail = key0 + BN > klimit;
-        const bool diag = p.causal && (key0 + BN - 1 > qw0);
-        if (tail || diag) {
-            const int qi = qw0 + n;
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int key = key0 + 32 * kb + acc_row(r, h);
-                    const bool drop = key >= klimit || (p.causal && key > qi);
-                    sacc[kb][r] = drop ? -INFINITY : sacc[kb][r];
-                }
-        }
-
-        float tmax = sacc[0][0];
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, sacc[kb][r]);
+    auto fold_max = [&](float tmax) {        // tmax in log2 units
         tmax = fmaxf(tmax, xhalf(tmax));
-        const float m_new = fmaxf(m_run, tmax);
-        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = exp2_fast(m_run - m_use);
-        m_run = m_new;
-        float rsum = 0.f;
+        if (__any(tmax > m_run + 8.0f)) {    // the reference maximum may lag the true one by 2^8
+            const float m_old = m_run;
+            const float m_new = fmaxf(m_old, tmax);
+            const float m_to = (m_new == -INFINITY) ? 0.f : m_new;
+            const float alpha = exp2_fast(m_old - m_to);
+            m_run = m_new;
+            l_run *= alpha;
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
+        }
+    };
+    auto zero_tile = [&](i32x16 (&s)[2]) {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s[kb][r] = 0;
+    };
+    // int32 accumulators -> dequantised, scaled, masked logits (log2 units), in place; returns their maximum
+    auto finish_masked = [&](i32x16 (&s)[2], int t) {
+        const float f = qfac * skb[t];
+        const int qi = qw0 + n;
+        float tmax = -INFINITY;
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const float e = exp2_fast(sacc[kb][r] - m_use);
-                sacc[kb][r] = e;
-                rsum += e;
+                const int key = t * BN + 32 * kb + acc_row(r, h);
+                const bool drop = key >= klimit || (p.causal && key > qi);
+                const float v = drop ? -INFINITY : (float)s[kb][r] * f;
+                tmax = fmaxf(tmax, v);
+                s[kb][r] = __float_as_int(v);
             }
-        l_run = l_run * alpha + rsum;
-#pragma unroll
-        for (int db = 0; db < DB; ++db)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
+        return tmax;
+    };
 
+    // The logits of the current tile are kept as floats in the accumulator registers: either the plain
+    // converted int32 sums, to be multiplied by cur_fac inside the exponential's fused multiply-add
+    // (tiles without exclusions), or already scaled and masked values with cur_fac = 1.
+    float cur_fac = 1.0f;
+
+    auto step = [&](auto fast_tag, i32x16 (&cur)[2], i32x16 (&nxt)[2], int t) {
+        constexpr bool FAST = decltype(fast_tag)::value;
+        const bool has_next = FAST || t + 1 < n_tiles;
+        if (FAST) {
+            issue_full_kv(t + 2, t + 1);
+        } else {
+            if (t + 2 < n_tiles) issue_k(t + 2);
+            if (has_next) issue_v(t + 1);
+        }
+        const float m_use = (m_run == -INFINITY) ? 0.f : m_run;
+        const float fac = cur_fac;
+        float rsum0 = 0.f, rsum1 = 0.f;
+        bf16x8 pf[4];
+        u32x4 fb[PD];
+        auto exp_slice = [&](int j) {
 #pragma unroll
-        for (int cc = 0; cc < 4; ++cc) {
-            const int kb = cc >> 1, o8 = 8 * (cc & 1);
-            const f32x16& s = sacc[kb];
-            const bf16x8 pf = pack8(s[o8], s[o8 + 1], s[o8 + 2], s[o8 + 3], s[o8 + 4], s[o8 + 5], s[o8 + 6], s[o8 + 7]);
+            for (int e = 0; e < EPS; ++e) {
+                const int idx = EPS * j + e, kb = idx >> 4, r = idx & 15;
+                const float v = exp2_fast(fmaf(__int_as_float(cur[kb][r]), fac, -m_use));
+                cur[kb][r] = __float_as_int(v);
+                if (e & 1) rsum1 += v;
+                else rsum0 += v;
+                if ((idx & 7) == 7) {
+                    const int o8 = r - 7;
+                    const i32x16& s = cur[kb];
+                    pf[idx >> 3] = pack8(__int_as_float(s[o8 + 0]), __int_as_float(s[o8 + 1]), __int_as_float(s[o8 + 2]),
+                                         __int_as_float(s[o8 + 3]), __int_as_float(s[o8 + 4]), __int_as_float(s[o8 + 5]),
+                                         __int_as_float(s[o8 + 6]), __int_as_float(s[o8 + 7]));
+                }
+            }
+        };
+        auto s_mfma = [&](int i) {
+            nxt[i & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, fb[i % PD]), qf[i >> 1], nxt[i & 1], 0, 0, 0);
+        };
+        auto pv_mfma = [&](int i) {
+            oacc[i % DB] = mfma32(__builtin_bit_cast(bf16x8, fb[i % PD]), pf[i / DB], oacc[i % DB]);
+        };
+
+        if (FAST) {
+            const float f_next = qfac * skb[t + 1];
+            zero_tile(nxt);
 #pragma unroll
-            for (int db = 0; db < DB; ++db) {
-                const bf16x8 va = lds_tr_frag(vs, VS, 16 * cc, 32 * db, lane);
-                oacc[db] = mfma32(va, pf, oacc[db]);
+            for (int i = 0; i < PD; ++i) {
+                fb[i] = k_frag(t + 1, i);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int i = 0; i < NS; ++i) {
+                s_mfma(i);
+                if (i + PD < NS) fb[i % PD] = k_frag(t + 1, i + PD);
+                else fb[i % PD] = v_frag(t, i + PD - NS);          // run on into the V fragments
+                exp_slice(i);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            l_run += rsum0 + rsum1;
+            // O^T += V(t)^T P(t)^T between the int32 -> float conversion and maximum scan of tile t+1
+            float tmax = -INFINITY;
+#pragma unroll
+            for (int i = 0; i < NP; ++i) {
+                pv_mfma(i);
+                if (i + PD < NP) fb[i % PD] = v_frag(t, i + PD);
+#pragma unroll
+                for (int e = 0; e < MPS; e += 2) {
+                    const int i0 = MPS * i + e, i1 = i0 + 1;
+                    const float a = (float)nxt[i0 >> 4][i0 & 15], c = (float)nxt[i1 >> 4][i1 & 15];
+                    nxt[i0 >> 4][i0 & 15] = __float_as_int(a);
+                    nxt[i1 >> 4][i1 & 15] = __float_as_int(c);
+                    tmax = fmaxf(fmaxf(tmax, a), c);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            cur_fac = f_next;
+            fold_max(tmax * f_next);         // f_next >= 0 and the sums are finite
+        } else {
+            if (has_next) {
+                zero_tile(nxt);
+#pragma unroll
+                for (int i = 0; i < PD; ++i) {
+                    fb[i] = k_frag(t + 1, i);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+#pragma unroll
+                for (int i = 0; i < NS; ++i) {
+                    s_mfma(i);
+                    if (i + PD < NS) fb[i % PD] = k_frag(t + 1, i + PD);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < NS; ++j) exp_slice(j);
+            l_run += rsum0 + rsum1;
+#pragma unroll
+            for (int i = 0; i < PD; ++i) {
+                fb[i] = v_frag(t, i);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int i = 0; i < NP; ++i) {
+                pv_mfma(i);
+                if (i + PD < NP) fb[i % PD] = v_frag(t, i + PD);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (has_next) {
+                const float tmax = finish_masked(nxt, t + 1);
+                cur_fac = 1.0f;
+                fold_max(tmax);
             }
         }
+        wait_vm0();          // the copies issued by this step have landed
+        __syncthreads();     // ... for every wave, and everyone is done reading this step's tiles
+    };
 
-        if (more) store_tile(buf ^ 1);
+    // tiles [0, n_full) need no exclusions for any query of the workgroup
+    int n_full = klimit / BN;
+    if (p.causal) n_full = min(n_full, (q0 + 1) / BN);
+    n_full = min(n_full, n_tiles);
+
+    i32x16 sa[2], sb[2];
+    if (n_tiles > 0) {
+        issue_k(0);
+        issue_v(0);
+        if (n_tiles > 1) issue_k(1);
+        wait_vm0();
         __syncthreads();
+        zero_tile(sa);
+#pragma unroll
+        for (int i = 0; i < NS; ++i)
+            sa[i & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, k_frag(0, i)), qf[i >> 1], sa[i & 1], 0, 0, 0);
+        fold_max(finish_masked(sa, 0));
+        cur_fac = 1.0f;
+        __syncthreads();     // every wave has read K^(0) before step 0 starts overwriting it
+
+        const int n_fast = max(0, n_full - 2) & ~1;      // step t is FAST when t + 2 < n_full
+        int t = 0;
+        for (; t < n_fast; t += 2) {
+            step(std::true_type{}, sa, sb, t);
+            step(std::true_type{}, sb, sa, t + 1);
+        }
+        for (; t < n_tiles; t += 2) {
+            step(std::false_type{}, sa, sb, t);
+            if (t + 1 < n_tiles) step(std::false_type{}, sb, sa, t + 1);
+        }
     }
 
     const int row = qw0 + n;

@@ -24,12 +24,13 @@ def test_rope_only_matches_reference_known_answer(oracle):
     kat = json.load(open(os.path.join(GOLD, "kat_rope_1x2x3x4.json")))
     B, H, S, D = kat["B"], kat["H"], kat["S"], kat["D"]
     x = (np.arange(B * H * S * D, dtype=np.float32) * np.float32(0.01)).reshape(B, H, S, D)
+    xr = _f32(_bits(x))           # the bf16 values the kernel sees
     want = np.zeros_like(x)
     for h in range(H):            # scalar loop from the reference test: pair p, freq = theta^(-2p/D), angle = s*freq
         for s in range(S):
             for p in range(D // 2):
                 ang = s * (1.0 / kat["theta"] ** (2.0 * p / D))
-                x0, x1 = float(_f32(_bits(x[0, h, s, 2 * p]))), float(_f32(_bits(x[0, h, s, 2 * p + 1])))
+                x0, x1 = float(xr[0, h, s, 2 * p]), float(xr[0, h, s, 2 * p + 1])
                 want[0, h, s, 2 * p] = x0 * math.cos(ang) - x1 * math.sin(ang)
                 want[0, h, s, 2 * p + 1] = x0 * math.sin(ang) + x1 * math.cos(ang)
     pos = np.arange(S, dtype=np.float64)[:, None]
