@@ -110,11 +110,12 @@ def attn_bwd(q, k, v, o, do, lse, scale, causal=False, kv_len=None, mask=None, w
     return dq, dk, dv
 
 
-KERNEL_KINDS = ("fwd", "bwd_prep", "bwd_dkdv", "bwd_dq", "sage_kmean", "sage_quant", "sage_fwd", "input_prep")
+KERNEL_KINDS = ("fwd", "unused1", "bwd_dkdv", "bwd_dq", "sage_kmean", "sage_quant", "sage_fwd", "input_prep",
+                "bwd_merge", "reserved9", "reserved10", "reserved11")
 
 
 class _KernelTimes(ctypes.Structure):
-    _fields_ = [("total_ms", ctypes.c_double * 8), ("launches", ctypes.c_int * 8)]
+    _fields_ = [("total_ms", ctypes.c_double * 12), ("launches", ctypes.c_int * 12)]
 
 
 def profiling_enable(on: bool) -> None:

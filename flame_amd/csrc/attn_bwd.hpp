@@ -1,15 +1,18 @@
 // Backward of the tiled attention for gfx950: recomputes P tile by tile from Q, K and the saved
 // log-sum-exp, never materialising the Sq x Sk matrix.
 //
-//   prep     delta_i = sum_d dO_id * O_id  and  LSE_i * log2(e)   (fp32, one value per query row)
-//   dkdv     one workgroup owns 128 keys (32 per wavefront) of one (batch, head) and walks over the
-//            query tiles (64 rows): S = Q K^T, dP = dO V^T, P = exp2(S*c - LSE*log2e),
-//            dS = P * (dP - delta); dV^T += dO^T P and dK^T += Q^T dS stay in fp32 registers for the
-//            whole walk (P and dS are used as MFMA operands straight from the accumulators)
 //   dq       one workgroup owns 128 queries (32 per wavefront) and walks over the key tiles (64 keys),
 //            with the logits transposed (lane = query): S^T = K Q^T, dP^T = V dO^T,
 //            dS^T = P^T (dP^T - delta) and dQ^T += K^T dS^T accumulated in fp32 registers for the whole
-//            walk, dS^T going into the last MFMA straight from the accumulators.
+//            walk, dS^T going into the last MFMA straight from the accumulators.  Runs first and also
+//            leaves delta_i = sum_d dO_id * O_id and LSE_i * log2(e) (fp32, one value per query row)
+//            in the workspace for the next kernel.
+//   dkdv     one workgroup owns 128 keys (32 per wavefront) of one (batch, head) and walks over the
+//            query tiles (64 rows): S = Q K^T, dP = dO V^T, P = exp2(S*c - LSE*log2e),
+//            dS = P * (dP - delta); dV^T += dO^T P and dK^T += Q^T dS stay in fp32 registers for the
+//            whole walk (P and dS are used as MFMA operands straight from the accumulators).  When the
+//            key blocks do not fill the last scheduling round, the blocks of that round are split
+//            along the walk and their fp32 partial sums are combined by the merge kernel.
 // Accumulating dQ from the dkdv walk with fp32 atomics was measured at about one lane-atomic per
 // clock per CU, more than the whole MFMA time of the backward; recomputing S and dP in a second,
 // query-major kernel costs 2 extra GEMMs out of 7 and no atomics, no fp32 scratch and no convert pass.
@@ -26,6 +29,13 @@
 namespace fattn {
 
 struct BwdParams {
+    // dK/dV grid: workgroups [0, n_whole) walk every query tile of one key block; the remaining key
+    // blocks are served by split_parts workgroups each, every one walking a slice of the query tiles
+    // and leaving fp32 partial sums in split_ws for bwd_dkdv_merge_kernel.  n_whole < 0: no splitting.
+    int n_whole = -1;
+    int split_parts = 1;
+    float* split_ws = nullptr;
+    size_t split_ws_bytes = 0;     // host side only
     const uint16_t* q;
     const uint16_t* k;
     const uint16_t* v;
@@ -44,35 +54,6 @@ struct BwdParams {
     unsigned long long* phase_cycles;   // profiling aid: per-phase cycle sums of wave 0 of every workgroup, or null
 };
 
-// ------------------------------------------------------------------------------------------ prep
-template <int D>
-__global__ __launch_bounds__(256) void bwd_prep_kernel(const BwdParams p) {
-    constexpr int TPR = D / 8;            // threads per row
-    constexpr int RPB = 256 / TPR;        // rows per block
-    const int tid = threadIdx.x;
-    const int64_t row_flat = (int64_t)blockIdx.x * RPB + tid / TPR;   // over B*H*Sq
-    const int chunk = tid % TPR;
-    const int64_t total = (int64_t)p.B * p.H * p.Sq;
-    float acc = 0.f;
-    const bool ok = row_flat < total;
-    if (ok) {
-        const int row = (int)(row_flat % p.Sq);
-        const int bh = (int)(row_flat / p.Sq);
-        const int b = bh / p.H, hh = bh % p.H;
-        const u32x4 a = *reinterpret_cast<const u32x4*>(p.dout + b * p.dos.b + hh * p.dos.h + (int64_t)row * p.dos.n + chunk * 8);
-        const u32x4 c = *reinterpret_cast<const u32x4*>(p.o + b * p.os.b + hh * p.os.h + (int64_t)row * p.os.n + chunk * 8);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) acc += bf16_lo(a[i]) * bf16_lo(c[i]) + bf16_hi(a[i]) * bf16_hi(c[i]);
-    }
-#pragma unroll
-    for (int off = TPR / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
-    if (ok && chunk == 0) {
-        p.delta[row_flat] = acc;
-        const float l = p.lse[row_flat];
-        p.lse2[row_flat] = (l == -INFINITY) ? INFINITY : l * kLog2e;   // exp2(s*c - inf) = 0 for excluded rows
-    }
-}
-
 // ------------------------------------------------------------------------------------------ dkdv
 template <int D>
 struct BwdTile {
@@ -87,6 +68,10 @@ struct BwdTile {
     static constexpr int ROWS_PER_DMA = 1024 / (D * 2);
     static constexpr int DMA_PER_WAVE = BM / ROWS_PER_DMA / 4;    // 1 KiB copies per wave and tensor
 };
+
+template <int D>
+__device__ __forceinline__ void dkdv_store(const BwdParams& p, const f32x16 (&dkacc)[D / 32], const f32x16 (&dvacc)[D / 32],
+                                           int b, int hh, int krow, int h);
 
 template <int D, bool HASMASK, bool TIMING>
 __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
@@ -107,7 +92,17 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
     const int n = lane & 31, h = lane >> 5;
 
     const int n_kt = (p.Sk + BN - 1) / BN;
-    const int wg = xcd_remap(blockIdx.x, gridDim.x);
+    int wg, part = 0, nparts = 1;
+    if (p.n_whole < 0) {
+        wg = xcd_remap(blockIdx.x, gridDim.x);
+    } else if ((int)blockIdx.x < p.n_whole) {
+        wg = xcd_remap(blockIdx.x, p.n_whole);
+    } else {          // the split key blocks come last in dispatch order and fill the final, partial round
+        const int e = (int)blockIdx.x - p.n_whole;
+        nparts = p.split_parts;
+        wg = p.n_whole + e / nparts;
+        part = e % nparts;
+    }
     const int kt = wg % n_kt;
     const int bh = wg / n_kt;
     const int b = bh / p.H, hh = bh % p.H;
@@ -257,7 +252,10 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
         tprev = tnow;                                                   \
     }
 
-    if (n_it > 0) issue_q_tile(tile_of(0), 0);
+    // this workgroup's slice [it_lo, it_hi) of the walk
+    const int it_lo = (int)((int64_t)part * n_it / nparts);
+    const int it_hi = (int)((int64_t)(part + 1) * n_it / nparts);
+    if (it_hi > it_lo) issue_q_tile(tile_of(it_lo), it_lo & 1);
     wait_vm0();
     __syncthreads();
 
@@ -281,7 +279,7 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
         static_assert((2 * DC) % 4 == 0 && (4 * DB) % 4 == 0, "read-ahead depth must divide the fragment count");
         const int buf = BUF >= 0 ? BUF : (it & 1);
         const int q0 = qt * BM;
-        const bool have_next = COPY == 1 || (COPY == 2 && it + 1 < n_it);
+        const bool have_next = COPY == 1 || (COPY == 2 && it + 1 < it_hi);
 
         const uint16_t* Qs = stage0 + buf * T::STAGE_ELEMS;
         const uint16_t* dOs = Qs + T::Q_ELEMS;
@@ -433,25 +431,25 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
     using I0 = std::integral_constant<int, 0>;
     using I1 = std::integral_constant<int, 1>;
     using I2 = std::integral_constant<int, 2>;
-    for (int it = 0; it < n_masked; ++it)
-        step(std::true_type{}, I2{}, IM{}, it, tile_of(it), it + 1 < n_it ? tile_of(it + 1) : 0);
+    for (int it = it_lo; it < min(n_masked, it_hi); ++it)
+        step(std::true_type{}, I2{}, IM{}, it, tile_of(it), it + 1 < it_hi ? tile_of(it + 1) : 0);
     // every tile after the first n_masked is a full, fully attended one, and they are consecutive
     {
-        int it = n_masked;
-        int qt = lead_end;
-        if ((it & 1) && it < n_it - 1) {
+        int it = max(n_masked, it_lo);
+        int qt = lead_end + (it - n_masked);
+        if ((it & 1) && it < it_hi - 1) {
             step(std::false_type{}, I1{}, I1{}, it, qt, qt + 1);
             ++it, ++qt;
         }
-        for (; it + 1 < n_it - 1; it += 2, qt += 2) {
+        for (; it + 1 < it_hi - 1; it += 2, qt += 2) {
             step(std::false_type{}, I1{}, I0{}, it, qt, qt + 1);
             step(std::false_type{}, I1{}, I1{}, it + 1, qt + 1, qt + 2);
         }
-        if (it < n_it - 1) {
+        if (it < it_hi - 1) {
             step(std::false_type{}, I1{}, IM{}, it, qt, qt + 1);
             ++it, ++qt;
         }
-        if (it < n_it) step(std::false_type{}, I0{}, IM{}, it, qt, qt);
+        if (it < it_hi) step(std::false_type{}, I0{}, IM{}, it, qt, qt);
     }
 
     if (TIMING && p.phase_cycles && tid == 0) {
@@ -460,8 +458,31 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
     }
 #undef FATTN_PHASE
 
-    // ---- epilogue: dK^T / dV^T accumulators -> dK, dV rows of this wavefront's keys
-    const int krow = kw0 + n;
+    // ---- epilogue
+    if (nparts > 1) {
+        // fp32 partial sums of this slice, in accumulator order: [tensor][thread][db][16]
+        float* dst = p.split_ws + ((size_t)(wg - p.n_whole) * nparts + part) * (size_t)(2 * BN * D);
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const f32x16& a = dkacc[db];
+                const f32x16& c = dvacc[db];
+                const f32x4 wk = {a[4 * g], a[4 * g + 1], a[4 * g + 2], a[4 * g + 3]};
+                const f32x4 wv = {c[4 * g], c[4 * g + 1], c[4 * g + 2], c[4 * g + 3]};
+                *reinterpret_cast<f32x4*>(dst + ((size_t)tid * DB + db) * 16 + 4 * g) = wk;
+                *reinterpret_cast<f32x4*>(dst + (size_t)BN * D + ((size_t)tid * DB + db) * 16 + 4 * g) = wv;
+            }
+        return;
+    }
+    dkdv_store<D>(p, dkacc, dvacc, b, hh, kw0 + n, h);
+}
+
+// dK^T / dV^T accumulators (rows = d, column = this lane's key) -> bf16 rows of dK (scaled) and dV
+template <int D>
+__device__ __forceinline__ void dkdv_store(const BwdParams& p, const f32x16 (&dkacc)[D / 32], const f32x16 (&dvacc)[D / 32],
+                                           int b, int hh, int krow, int h) {
+    constexpr int DB = D / 32;
     if (krow < p.Sk) {
         uint16_t* dkrow = p.dk + b * p.dks.b + hh * p.dks.h + (int64_t)krow * p.dks.n;
         uint16_t* dvrow = p.dv + b * p.dvs.b + hh * p.dvs.h + (int64_t)krow * p.dvs.n;
@@ -477,6 +498,49 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
                 *reinterpret_cast<u32x2*>(dkrow + 32 * db + 8 * g + 4 * h) = wk;
                 *reinterpret_cast<u32x2*>(dvrow + 32 * db + 8 * g + 4 * h) = wv;
             }
+    }
+}
+
+// Sums the fp32 partials that the split workgroups of one key block left behind and writes dK, dV.
+// One workgroup per (split key block, 32-wide block of d); the thread layout mirrors the accumulators.
+template <int D>
+__global__ __launch_bounds__(256) void bwd_dkdv_merge_kernel(const BwdParams p) {
+    constexpr int BN = BwdTile<D>::BN, DB = D / 32;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int n = lane & 31, h = lane >> 5;
+    const int n_kt = (p.Sk + BN - 1) / BN;
+    const int sb = (int)blockIdx.x / DB, db = (int)blockIdx.x % DB;
+    const int wg = p.n_whole + sb;
+    const int kt = wg % n_kt;
+    const int bh = wg / n_kt;
+    const int b = bh / p.H, hh = bh % p.H;
+    f32x4 ak[4], av[4];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        ak[g] = f32x4{0.f, 0.f, 0.f, 0.f};
+        av[g] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    for (int part = 0; part < p.split_parts; ++part) {
+        const float* src = p.split_ws + ((size_t)sb * p.split_parts + part) * (size_t)(2 * BN * D) + ((size_t)tid * DB + db) * 16;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            ak[g] += *reinterpret_cast<const f32x4*>(src + 4 * g);
+            av[g] += *reinterpret_cast<const f32x4*>(src + (size_t)BN * D + 4 * g);
+        }
+    }
+    const int krow = kt * BN + 32 * wave + n;
+    if (krow < p.Sk) {
+        uint16_t* dkrow = p.dk + b * p.dks.b + hh * p.dks.h + (int64_t)krow * p.dks.n;
+        uint16_t* dvrow = p.dv + b * p.dvs.b + hh * p.dvs.h + (int64_t)krow * p.dvs.n;
+        const float s = p.scale;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            u32x2 wk = {pack_bf16(ak[g][0] * s, ak[g][1] * s), pack_bf16(ak[g][2] * s, ak[g][3] * s)};
+            u32x2 wv = {pack_bf16(av[g][0], av[g][1]), pack_bf16(av[g][2], av[g][3])};
+            *reinterpret_cast<u32x2*>(dkrow + 32 * db + 8 * g + 4 * h) = wk;
+            *reinterpret_cast<u32x2*>(dvrow + 32 * db + 8 * g + 4 * h) = wv;
+        }
     }
 }
 
@@ -541,9 +605,31 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams p) {
             dof[dc] = __builtin_bit_cast(bf16x8, ldg16(rd + 16 * dc, qok));
         }
     }
-    // rows past the end behave like fully excluded rows: lse2 = +inf gives P = 0
-    const float lse2 = qok ? p.lse2[(int64_t)bh * p.Sq + qrow] : INFINITY;
-    const float delta = qok ? p.delta[(int64_t)bh * p.Sq + qrow] : 0.f;
+    // Per-query scalars, formed here and also left in the workspace for the dK/dV kernel that runs next:
+    //   delta = rowsum(dO * O)   (the bf16 O that the forward saved)
+    //   lse2  = LSE * log2(e), +inf for fully excluded rows and rows past the end (P = exp2(s - inf) = 0)
+    float lse2 = INFINITY, delta = 0.f;
+    {
+        const uint16_t* ro = p.o + b * p.os.b + hh * p.os.h + (int64_t)qrow * p.os.n + 8 * h;
+        float part = 0.f;
+#pragma unroll
+        for (int dc = 0; dc < DC; ++dc) {
+            const u32x4 ov = ldg16(ro + 16 * dc, qok);
+            const u32x4 dv = __builtin_bit_cast(u32x4, dof[dc]);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) part += bf16_lo(dv[i]) * bf16_lo(ov[i]) + bf16_hi(dv[i]) * bf16_hi(ov[i]);
+        }
+        part += xhalf(part);
+        if (qok) {
+            const float l = p.lse[(int64_t)bh * p.Sq + qrow];
+            lse2 = (l == -INFINITY) ? INFINITY : l * kLog2e;
+            delta = part;
+            if (h == 0) {
+                p.delta[(int64_t)bh * p.Sq + qrow] = delta;
+                p.lse2[(int64_t)bh * p.Sq + qrow] = lse2;
+            }
+        }
+    }
 
     const int dma_row_in = lane / GPR, dma_gran = lane % GPR;
     constexpr int NDMA = T::DMA_PER_WAVE;

@@ -3,6 +3,8 @@
 // caller's stream, so calls may be captured into a HIP graph.
 #include "../../include/flame_attn.h"
 
+#include <algorithm>
+
 #include <hip/hip_runtime.h>
 #include <math.h>
 #include <stdio.h>
@@ -108,6 +110,24 @@ int launch_fwd(const FwdParams& p, hipStream_t s) {
 
 size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
+// compute units of the current device (cached; 256 when the query fails)
+int device_cu_count() {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) == hipSuccess &&
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+            cus = n;
+        else
+            cus = 256;
+    }
+    return cus;
+}
+
+// backward workspace: [delta rows][lse2 rows][fp32 partials of the split dK/dV workgroups]
+size_t bwd_rows_bytes(int B, int H, int N_q) { return 2 * align_up((size_t)B * H * N_q * sizeof(float), 256); }
+size_t bwd_split_slot_bytes(int D) { return (size_t)2 * 128 * D * sizeof(float); }   // dK^T and dV^T of one 128-key block
+
 template <int D, bool HASMASK, bool TIMING = false>
 int launch_bwd(const BwdParams& p, hipStream_t s) {
     using T = BwdTile<D>;
@@ -124,25 +144,48 @@ int launch_bwd(const BwdParams& p, hipStream_t s) {
         if (e != hipSuccess) return (int)e;
         attr_done = true;
     }
-    constexpr int RPB = 256 / (D / 8);
-    const int64_t rows = (int64_t)p.B * p.H * p.Sq;
-    const int64_t row_blocks = (rows + RPB - 1) / RPB;
     const int64_t n_kt = (p.Sk + T::BN - 1) / T::BN;
     const int64_t grid = n_kt * p.B * p.H;
     const int64_t n_qt = (p.Sq + TQ::BM - 1) / TQ::BM;
     const int64_t grid_dq = n_qt * p.B * p.H;
-    if (row_blocks > 0x7fffffff || grid > 0x7fffffff || grid_dq > 0x7fffffff) return FLAME_ATTN_ERR_UNSUPPORTED;
-    {
-        ScopedKernelTimer t(FLAME_ATTN_KERNEL_BWD_PREP, s);
-        hipLaunchKernelGGL(bwd_prep_kernel<D>, dim3((unsigned)row_blocks), dim3(256), 0, s, p);
-    }
-    {
-        ScopedKernelTimer t(FLAME_ATTN_KERNEL_BWD_DKDV, s);
-        hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), T::LDS_BYTES, s, p);
-    }
+    if (grid > 0x7fffffff || grid_dq > 0x7fffffff) return FLAME_ATTN_ERR_UNSUPPORTED;
+    // dQ first: besides dQ it leaves delta = rowsum(dO * O) and the rescaled LSE of every query row in the
+    // workspace, which the dK/dV kernel stages per query tile.
     {
         ScopedKernelTimer t(FLAME_ATTN_KERNEL_BWD_DQ, s);
         hipLaunchKernelGGL(kern_dq, dim3((unsigned)grid_dq), dim3(256), TQ::LDS_BYTES, s, p);
+    }
+    // The dK/dV kernel keeps one workgroup per compute unit.  When the key blocks do not fill the last
+    // round of that schedule, the blocks of the last round are split over the idle units along the query
+    // walk (fp32 partial sums, merged by a small second kernel).  Needs equally long walks (no causal,
+    // key-length or explicit mask) and room in the workspace.
+    BwdParams pk = p;
+    int64_t grid_kv = grid;
+    int n_split = 0;
+    {
+        const int cus = device_cu_count();
+        const int64_t rem = grid % cus;
+        const int64_t n_qtiles = (p.Sq + T::BM - 1) / T::BM;
+        const bool uniform = !HASMASK && !p.m.causal && !p.m.kv_len;
+        if (uniform && grid > cus && rem > 0 && 2 * rem <= cus && n_qtiles >= 16 && p.split_ws) {
+            int parts = (int)std::min<int64_t>(cus / rem, 4);
+            const size_t room = p.split_ws_bytes / bwd_split_slot_bytes(D);
+            while (parts > 1 && (size_t)(rem * parts) > room) --parts;
+            if (parts > 1) {
+                pk.n_whole = (int)(grid - rem);
+                pk.split_parts = parts;
+                n_split = (int)rem;
+                grid_kv = pk.n_whole + rem * parts;
+            }
+        }
+    }
+    {
+        ScopedKernelTimer t(FLAME_ATTN_KERNEL_BWD_DKDV, s);
+        hipLaunchKernelGGL(kern, dim3((unsigned)grid_kv), dim3(256), T::LDS_BYTES, s, pk);
+    }
+    if (n_split > 0) {
+        ScopedKernelTimer t(FLAME_ATTN_KERNEL_BWD_MERGE, s);
+        hipLaunchKernelGGL(bwd_dkdv_merge_kernel<D>, dim3((unsigned)(n_split * (D / 32))), dim3(256), 0, s, pk);
     }
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? FLAME_ATTN_OK : (int)e;
@@ -186,9 +229,7 @@ int flame_attn_profiling_read(FlameAttnKernelTimes* out) {
 
 size_t flame_attn_bwd_workspace_bytes(int B, int H, int N_q, int D) {
     if (B <= 0 || H <= 0 || N_q <= 0 || D <= 0) return 0;
-    const size_t rows = (size_t)B * H * N_q;
-    (void)D;
-    return 2 * align_up(rows * sizeof(float), 256);
+    return bwd_rows_bytes(B, H, N_q) + (size_t)device_cu_count() * bwd_split_slot_bytes(D);
 }
 
 int flame_attn_bwd_bf16(const void* Q, const void* K, const void* V, const void* O, const void* dO,
@@ -206,7 +247,7 @@ int flame_attn_bwd_bf16(const void* Q, const void* K, const void* V, const void*
     if (!(scale > 0.f) || !isfinite(scale)) return FLAME_ATTN_ERR_INVALID;
     if (!LSE || !workspace) return FLAME_ATTN_ERR_INVALID;
     if (D != 64 && D != 128) return FLAME_ATTN_ERR_UNSUPPORTED;
-    if (workspace_bytes < flame_attn_bwd_workspace_bytes(B, H, N_q, D)) return FLAME_ATTN_ERR_INVALID;
+    if (workspace_bytes < bwd_rows_bytes(B, H, N_q)) return FLAME_ATTN_ERR_INVALID;
     if (!aligned16(workspace)) return FLAME_ATTN_ERR_UNSUPPORTED;
     int rc;
     if ((rc = check_view(Q, q_strides, q_off))) return rc;
@@ -232,6 +273,8 @@ int flame_attn_bwd_bf16(const void* Q, const void* K, const void* V, const void*
     const size_t rows = (size_t)B * H * N_q;
     p.delta = static_cast<float*>(workspace);
     p.lse2 = reinterpret_cast<float*>(static_cast<char*>(workspace) + align_up(rows * sizeof(float), 256));
+    p.split_ws = reinterpret_cast<float*>(static_cast<char*>(workspace) + bwd_rows_bytes(B, H, N_q));
+    p.split_ws_bytes = workspace_bytes - bwd_rows_bytes(B, H, N_q);
     p.qs = mk(q_strides); p.ks = mk(k_strides); p.vs = mk(v_strides); p.os = mk(o_strides);
     p.dos = mk(do_strides); p.dqs = mk(dq_strides); p.dks = mk(dk_strides); p.dvs = mk(dv_strides);
     p.B = B; p.H = H; p.Sq = N_q; p.Sk = N_kv;

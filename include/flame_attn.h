@@ -70,12 +70,15 @@ int flame_attn_fwd_bf16(const void* Q, const void* K, const void* V, void* O, vo
                         const uint8_t* keep_mask, const int64_t* mask_strides,
                         void* stream);
 
-/* Bytes of device scratch the backward needs (two fp32 values per query row). */
+/* Recommended bytes of device scratch for the backward: two fp32 values per query row (required),
+ * plus one 128-key block of fp32 dK/dV partial sums per compute unit of the current device
+ * (optional: lets the dK/dV kernel split the key blocks of its last, partly filled scheduling round
+ * over the idle compute units).  A workspace that only covers the row part is accepted. */
 size_t flame_attn_bwd_workspace_bytes(int B, int H, int N_q, int D);
 
 /* Backward from Q, K, V, the saved O and LSE, and the upstream gradient dO (bf16).  Writes bf16
  * dQ [B,H,N_q,D], dK, dV [B,H,N_kv,D] through their own strides.  `workspace` is 16-byte aligned
- * device memory of at least flame_attn_bwd_workspace_bytes(...) bytes, used only during the call.
+ * device memory, ideally of flame_attn_bwd_workspace_bytes(...) bytes, used only during the call.
  * Replaces flame_cudnn_sdpa_bwd_bf16 (src/cuda/ffi.rs:682-716) and the materialising recompute
  * attention_backward_recompute (src/autograd.rs:801-848); follows the arithmetic of
  * tests/cudnn_sdpa_bwd_parity.rs:31-98 with D_i = rowsum(dO * O). */
@@ -185,9 +188,10 @@ bool sdpa_stream_bf16_launch(const void* dQ, const void* dK, const void* dV, voi
  * Profiling aids (the counterpart of the reference's SdpaStats / SdpaHooks timing fields,
  * src/autograd_v4/ops/sdpa.rs:55-79).  No counterpart in the FFI of the reference.
  * ---------------------------------------------------------------------------------------------- */
-enum { FLAME_ATTN_KERNEL_FWD = 0, FLAME_ATTN_KERNEL_BWD_PREP = 1, FLAME_ATTN_KERNEL_BWD_DKDV = 2,
+enum { FLAME_ATTN_KERNEL_FWD = 0, FLAME_ATTN_KERNEL_UNUSED_1 = 1, FLAME_ATTN_KERNEL_BWD_DKDV = 2,
        FLAME_ATTN_KERNEL_BWD_DQ = 3, FLAME_ATTN_KERNEL_SAGE_KMEAN = 4, FLAME_ATTN_KERNEL_SAGE_QUANT = 5,
-       FLAME_ATTN_KERNEL_SAGE_FWD = 6, FLAME_ATTN_KERNEL_INPUT_PREP = 7, FLAME_ATTN_N_KERNEL_KINDS = 8 };
+       FLAME_ATTN_KERNEL_SAGE_FWD = 6, FLAME_ATTN_KERNEL_INPUT_PREP = 7, FLAME_ATTN_KERNEL_BWD_MERGE = 8,
+       FLAME_ATTN_N_KERNEL_KINDS = 12 };
 typedef struct {
     double total_ms[FLAME_ATTN_N_KERNEL_KINDS];
     int launches[FLAME_ATTN_N_KERNEL_KINDS];

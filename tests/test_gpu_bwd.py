@@ -107,7 +107,31 @@ def test_workspace_too_small_is_rejected():
     from flame_amd import capi
     q = torch.zeros(1, 1, 64, 64, dtype=torch.bfloat16, device="cuda")
     o, lse = capi.attn_fwd(q, q, q, 0.125)
-    ws = torch.empty(capi.bwd_workspace_bytes(1, 1, 64, 64) - 1, dtype=torch.uint8, device="cuda")
+    ws = torch.empty(2 * 256 - 1, dtype=torch.uint8, device="cuda")     # the two fp32 rows per query need 2 x 256 B
     with pytest.raises(capi.FlameAttnError) as e:
         capi.attn_bwd(q, q, q, o, q, lse, 0.125, workspace=ws)
     assert e.value.code == capi.ERR_INVALID
+
+
+def test_split_last_round_matches_unsplit_walk():
+    """With the recommended workspace the key blocks of the last, partly filled scheduling round are
+    split along the query walk and merged from fp32 partials; with the minimal workspace every block is
+    walked by one workgroup.  Both orders of summation must agree to bf16 rounding, on every head."""
+    from flame_amd import capi
+    w = W.config2()
+    B, H, Sq, Sk, D = w.shape
+    q, k, v, do = (to_dev(t) for t in (w.q, w.k, w.v, w.do))
+    o, lse = capi.attn_fwd(q, k, v, w.scale)
+    rows_only = 2 * (-(-(B * H * Sq * 4) // 256) * 256)
+    assert capi.bwd_workspace_bytes(B, H, Sq, D) > rows_only
+    a = capi.attn_bwd(q, k, v, o, do, lse, w.scale)      # default workspace: split path for the last 96 key blocks
+    b = capi.attn_bwd(q, k, v, o, do, lse, w.scale, workspace=torch.empty(rows_only, dtype=torch.uint8, device="cuda"))
+    torch.cuda.synchronize()
+    assert torch.equal(a[0], b[0])                       # dQ does not depend on the dK/dV schedule
+    for name, x, y in (("dK", a[1], b[1]), ("dV", a[2], b[2])):
+        xf, yf = x.float(), y.float()
+        diff = (xf - yf).abs()
+        ulp = torch.pow(2.0, torch.floor(torch.log2(yf.abs().clamp_min(2.0 ** -126))) - 7)
+        assert bool((diff <= ulp + 1e-3).all()), (name, float(diff.max()))     # 1e-3: cancellation near zero
+        whole = slice(0, 20)                             # heads whose key blocks all sit in the unsplit range
+        assert torch.equal(x[:, whole], y[:, whole]), name
