@@ -73,8 +73,8 @@ def input_prep_rate(capi, W, torch, B, H, N, D, dev, iters=20):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--config", type=int, default=2, help="workload configuration (2 = the headline shape)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--traffic-calibration", action="store_true",
