@@ -321,8 +321,20 @@ int flame_sage_quant_qk_int8(const void* Q, const void* K, int B, int H, int N_q
     if (bh * nblk > 0x7fffffff) return FLAME_ATTN_ERR_UNSUPPORTED;
     {
         ScopedKernelTimer t(FLAME_ATTN_KERNEL_SAGE_KMEAN, s);
-        if (D == 128) hipLaunchKernelGGL(sage_kmean_kernel<128>, dim3((unsigned)bh), dim3(512), 0, s, p);
-        else hipLaunchKernelGGL(sage_kmean_kernel<64>, dim3((unsigned)bh), dim3(512), 0, s, p);
+        // the partial sums of a head (n_chunks * D doubles) must fit in that head's int8 K output
+        const int n_chunks = (int)std::max<int64_t>(1, std::min<int64_t>(32, N_kv / 256));
+        const int rows_per_chunk = (N_kv + n_chunks - 1) / n_chunks;
+        if (N_kv < 256) {       // short: one workgroup per head sums all rows
+            if (D == 128) hipLaunchKernelGGL(sage_kmean_kernel<128>, dim3((unsigned)bh), dim3(512), 0, s, p);
+            else hipLaunchKernelGGL(sage_kmean_kernel<64>, dim3((unsigned)bh), dim3(512), 0, s, p);
+        } else {
+        if (smooth_k) {
+            if (D == 128) hipLaunchKernelGGL(sage_kmean_partial_kernel<128>, dim3((unsigned)(bh * n_chunks)), dim3(512), 0, s, p, n_chunks, rows_per_chunk);
+            else hipLaunchKernelGGL(sage_kmean_partial_kernel<64>, dim3((unsigned)(bh * n_chunks)), dim3(512), 0, s, p, n_chunks, rows_per_chunk);
+        }
+        if (D == 128) hipLaunchKernelGGL(sage_kmean_final_kernel<128>, dim3((unsigned)bh), dim3(128), 0, s, p, n_chunks);
+        else hipLaunchKernelGGL(sage_kmean_final_kernel<64>, dim3((unsigned)bh), dim3(64), 0, s, p, n_chunks);
+        }
     }
     {
         ScopedKernelTimer t(FLAME_ATTN_KERNEL_SAGE_QUANT, s);

@@ -35,7 +35,7 @@ struct SageQuantParams {
     float* sk;       // [B*H, ceil(Sk/64)]
 };
 
-// one workgroup of 512 threads per (batch, head)
+// Channel mean of K, short sequences: one workgroup of 512 threads per (batch, head)
 template <int D>
 __global__ __launch_bounds__(512) void sage_kmean_kernel(const SageQuantParams p) {
     constexpr int CPR = D / 8;            // 16-byte chunks per row
@@ -67,6 +67,55 @@ __global__ __launch_bounds__(512) void sage_kmean_kernel(const SageQuantParams p
         for (int g = 0; g < RG; ++g) s += part[g][tid];
         p.kmean[(int64_t)bh * D + tid] = p.smooth_k ? (float)(s / (double)p.Sk) : 0.f;
     }
+}
+
+// Long sequences: channel mean of K in two steps so that the whole device takes part: workgroup (bh, c) sums the rows
+// of chunk c in fp64 and parks its D partial sums in the first bytes of that head's int8 K output
+// (overwritten by the quantisation that follows); sage_kmean_final_kernel adds the chunks in order.
+// fp64 sums of bf16 values are exact at these lengths, so the result does not depend on the chunking.
+template <int D>
+__global__ __launch_bounds__(512) void sage_kmean_partial_kernel(const SageQuantParams p, int n_chunks, int rows_per_chunk) {
+    constexpr int CPR = D / 8;            // 16-byte chunks per row
+    constexpr int RG = 512 / CPR;         // row groups
+    __shared__ double part[RG][D + 1];
+    const int tid = threadIdx.x;
+    const int chunk = tid % CPR, rg = tid / CPR;
+    const int bh = blockIdx.x / n_chunks, c = blockIdx.x % n_chunks;
+    const int b = bh / p.H, hh = bh % p.H;
+    const uint16_t* kb = p.k + b * p.ks.b + hh * p.ks.h + chunk * 8;
+    const int r_end = min(p.Sk, (c + 1) * rows_per_chunk);
+    double acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = 0.0;
+    for (int row = c * rows_per_chunk + rg; row < r_end; row += RG) {
+        const u32x4 w = *reinterpret_cast<const u32x4*>(kb + (int64_t)row * p.ks.n);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            acc[2 * i] += (double)bf16_lo(w[i]);
+            acc[2 * i + 1] += (double)bf16_hi(w[i]);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) part[rg][chunk * 8 + i] = acc[i];
+    __syncthreads();
+    if (tid < D) {
+        double s = 0.0;
+        for (int g = 0; g < RG; ++g) s += part[g][tid];
+        reinterpret_cast<double*>(p.ki8 + (int64_t)bh * p.Sk * D)[c * D + tid] = s;
+    }
+}
+
+template <int D>
+__global__ __launch_bounds__(D) void sage_kmean_final_kernel(const SageQuantParams p, int n_chunks) {
+    const int bh = blockIdx.x, tid = threadIdx.x;
+    float m = 0.f;
+    if (p.smooth_k) {
+        const double* scr = reinterpret_cast<const double*>(p.ki8 + (int64_t)bh * p.Sk * D);
+        double s = 0.0;
+        for (int c = 0; c < n_chunks; ++c) s += scr[c * D + tid];
+        m = (float)(s / (double)p.Sk);
+    }
+    p.kmean[(int64_t)bh * D + tid] = m;
 }
 
 __device__ __forceinline__ int quant_code(float x, float s) {
