@@ -76,6 +76,29 @@ def attn_fwd(q, k, v, scale, causal=False, kv_len=None, mask=None, want_lse=True
     return o, lse
 
 
+def attn_fwd_bias(q, k, v, scale, bias, mask=None, want_lse=True):
+    """softmax(scale * Q K^T + bias) V.  bias: fp32 or bf16 [B|1, H|1, Sq, Sk] (inference only)."""
+    B, H, Sq, D = q.shape
+    Sk = k.shape[2]
+    assert bias.dim() == 4 and bias.dtype in (torch.float32, torch.bfloat16)
+    full = (B, H, Sq, Sk)
+    bst = []
+    for ax in range(4):
+        assert bias.shape[ax] in (1, full[ax]), "bias is not broadcastable to [B,H,Sq,Sk]"
+        bst.append(0 if (bias.shape[ax] == 1 and full[ax] != 1) else bias.stride(ax))
+    o = torch.empty((B, H, Sq, D), dtype=torch.bfloat16, device=q.device)
+    lse = torch.empty((B * H, Sq), dtype=torch.float32, device=q.device) if want_lse else None
+    rc = lib().flame_attn_fwd_bias_bf16(
+        _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), B, H, Sq, Sk, D, ctypes.c_float(scale),
+        _i64x4(q.stride()), _i64x4(k.stride()), _i64x4(v.stride()), _i64x4(o.stride()),
+        *(ctypes.c_int64(0) for _ in range(5)),
+        _ptr(bias), 1 if bias.dtype == torch.float32 else 0, _i64x4(bst),
+        _ptr(mask), _mask_strides(mask, B, H, Sq, Sk), _stream())
+    if rc != 0:
+        raise FlameAttnError("flame_attn_fwd_bias_bf16", rc)
+    return o, lse
+
+
 def bwd_workspace_bytes(B, H, Sq, D) -> int:
     f = lib().flame_attn_bwd_workspace_bytes
     f.restype = ctypes.c_size_t

@@ -187,6 +187,11 @@ struct MaskArgs {
     const uint8_t* mask;     // keep-mask (non-zero = attend) or null
     int64_t sb, sh, sq, sk;  // element strides over (b,h,q,k); 0 broadcasts
     int causal;              // key j > query i is excluded
+    // additive bias on the scaled logits (forward only), fp32 or bf16, or null
+    const void* bias = nullptr;
+    int64_t bb = 0, bh = 0, bq = 0, bk = 0;   // element strides over (b,h,q,k); 0 broadcasts
+    int bias_f32 = 1;
+    float inv_scale = 1.f;   // 1 / softmax scale: the bias is folded into the raw scores as bias / scale
 };
 
 }  // namespace fattn

@@ -84,7 +84,10 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
     int kend = klimit;
     if (p.m.causal) kend = min(kend, q0 + BM);
     const int n_tiles = (kend + BN - 1) / BN;
-    const uint8_t* mbase = HASMASK ? p.m.mask + b * p.m.sb + hh * p.m.sh : nullptr;
+    const uint8_t* mbase = (HASMASK && p.m.mask) ? p.m.mask + b * p.m.sb + hh * p.m.sh : nullptr;
+    const char* bbase = (HASMASK && p.m.bias)
+                            ? static_cast<const char*>(p.m.bias) + (b * p.m.bb + hh * p.m.bh) * (p.m.bias_f32 ? 4 : 2)
+                            : nullptr;
 
     // ---- Q fragments (B operand of S^T = K Q^T): column = query, 8 consecutive d
     bf16x8 qf[DC];
@@ -184,10 +187,20 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
                 const int key = t * BN + 32 * kb + acc_row(r, h);
                 bool drop = key >= klimit;
                 if (p.m.causal) drop = drop || key > qi;
+                float val = s[kb][r];
                 if (HASMASK) {
-                    if (!drop && qi < p.Sq) drop = mbase[(int64_t)qi * p.m.sq + (int64_t)key * p.m.sk] == 0;
+                    if (mbase && !drop && qi < p.Sq) drop = mbase[(int64_t)qi * p.m.sq + (int64_t)key * p.m.sk] == 0;
+                    if (bbase) {      // scale * (s + bias / scale) = scale * s + bias
+                        float bv = 0.f;
+                        if (!drop && qi < p.Sq) {
+                            const int64_t e = (int64_t)qi * p.m.bq + (int64_t)key * p.m.bk;
+                            bv = p.m.bias_f32 ? reinterpret_cast<const float*>(bbase)[e]
+                                              : __uint_as_float((uint32_t)reinterpret_cast<const uint16_t*>(bbase)[e] << 16);
+                        }
+                        val = fmaf(bv, p.m.inv_scale, val);
+                    }
                 }
-                s[kb][r] = drop ? -INFINITY : s[kb][r];   // select, not a divergent store
+                s[kb][r] = drop ? -INFINITY : val;   // select, not a divergent store
             }
     };
     // Fold the maximum of a freshly computed tile into the running state.  The reference maximum

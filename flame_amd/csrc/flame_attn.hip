@@ -400,13 +400,16 @@ int flame_sage_attn_fwd_int8(const void* Qi8, const void* Ki8, const void* q_sca
     return launch_sage_fwd<64>(p, s);
 }
 
-int flame_attn_fwd_bf16(const void* Q, const void* K, const void* V, void* O, void* LSE,
+}  // extern "C"
+
+static int attn_fwd_impl(const void* Q, const void* K, const void* V, void* O, void* LSE,
                         int B, int H, int N_q, int N_kv, int D, float scale,
                         const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
                         const int64_t* o_strides,
                         int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off, int64_t lse_off,
                         int causal, const int32_t* kv_len,
                         const uint8_t* keep_mask, const int64_t* mask_strides,
+                        const void* bias, int bias_dtype, const int64_t* bias_strides,
                         void* stream) {
     if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0) return FLAME_ATTN_ERR_INVALID;
     if (!(scale > 0.f) || !isfinite(scale)) return FLAME_ATTN_ERR_INVALID;
@@ -417,6 +420,8 @@ int flame_attn_fwd_bf16(const void* Q, const void* K, const void* V, void* O, vo
     if ((rc = check_view(V, v_strides, v_off))) return rc;
     if ((rc = check_view(O, o_strides, o_off))) return rc;
     if (keep_mask && !mask_strides) return FLAME_ATTN_ERR_INVALID;
+    if (bias && !bias_strides) return FLAME_ATTN_ERR_INVALID;
+    if (bias && bias_dtype != FLAME_ATTN_DTYPE_BF16 && bias_dtype != FLAME_ATTN_DTYPE_F32) return FLAME_ATTN_ERR_INVALID;
 
     FwdParams p;
     p.q = static_cast<const uint16_t*>(Q) + q_off;
@@ -434,13 +439,48 @@ int flame_attn_fwd_bf16(const void* Q, const void* K, const void* V, void* O, vo
     p.m.sq = keep_mask ? mask_strides[2] : 0;
     p.m.sk = keep_mask ? mask_strides[3] : 0;
     p.m.causal = causal ? 1 : 0;
+    p.m.bias = bias;
+    if (bias) {
+        p.m.bb = bias_strides[0]; p.m.bh = bias_strides[1]; p.m.bq = bias_strides[2]; p.m.bk = bias_strides[3];
+        p.m.bias_f32 = bias_dtype == FLAME_ATTN_DTYPE_F32;
+        p.m.inv_scale = 1.0f / scale;
+    }
 
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const bool hm = keep_mask != nullptr;
+    const bool hm = keep_mask != nullptr || bias != nullptr;
     if (D == 128) return hm ? launch_fwd<128, true>(p, s) : launch_fwd<128, false>(p, s);
     return hm ? launch_fwd<64, true>(p, s) : launch_fwd<64, false>(p, s);
 }
 
+
+extern "C" {
+
+int flame_attn_fwd_bf16(const void* Q, const void* K, const void* V, void* O, void* LSE,
+                        int B, int H, int N_q, int N_kv, int D, float scale,
+                        const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                        const int64_t* o_strides,
+                        int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off, int64_t lse_off,
+                        int causal, const int32_t* kv_len,
+                        const uint8_t* keep_mask, const int64_t* mask_strides,
+                        void* stream) {
+    return attn_fwd_impl(Q, K, V, O, LSE, B, H, N_q, N_kv, D, scale, q_strides, k_strides, v_strides, o_strides,
+                         q_off, k_off, v_off, o_off, lse_off, causal, kv_len, keep_mask, mask_strides,
+                         nullptr, FLAME_ATTN_DTYPE_F32, nullptr, stream);
+}
+
+int flame_attn_fwd_bias_bf16(const void* Q, const void* K, const void* V, void* O, void* LSE,
+                             int B, int H, int N_q, int N_kv, int D, float scale,
+                             const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                             const int64_t* o_strides,
+                             int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off, int64_t lse_off,
+                             const void* bias, int bias_dtype, const int64_t* bias_strides,
+                             const uint8_t* keep_mask, const int64_t* mask_strides,
+                             void* stream) {
+    if (!bias) return FLAME_ATTN_ERR_INVALID;
+    return attn_fwd_impl(Q, K, V, O, LSE, B, H, N_q, N_kv, D, scale, q_strides, k_strides, v_strides, o_strides,
+                         q_off, k_off, v_off, o_off, lse_off, 0, nullptr, keep_mask, mask_strides,
+                         bias, bias_dtype, bias_strides, stream);
+}
 
 // ------------------------------------------------------------------------------------------------
 // Entry points with the names and argument lists of the reference's FFI for this path.  They are
@@ -519,6 +559,22 @@ __global__ void mask_f32_to_u8_kernel(const float* src, uint8_t* dst, int64_t n)
 __global__ void cast_f32_to_bf16_kernel(const float* src, uint16_t* dst, int64_t n) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) dst[i] = (uint16_t)(pack_bf16(src[i], 0.f) & 0xffffu);
+}
+// gradient accumulation of the host layer: acc += float(g) with g bf16 or fp32; fill with a constant
+__global__ void accumulate_f32_kernel(float* acc, const void* g, int g_is_f32, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) {
+        const float v = g_is_f32 ? static_cast<const float*>(g)[i]
+                                 : __uint_as_float((uint32_t)static_cast<const uint16_t*>(g)[i] << 16);
+        acc[i] += v;
+    }
+}
+__global__ void fill_kernel(void* dst, float value, int is_f32, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) {
+        if (is_f32) static_cast<float*>(dst)[i] = value;
+        else static_cast<uint16_t*>(dst)[i] = (uint16_t)(pack_bf16(value, 0.f) & 0xffffu);
+    }
 }
 }  // namespace
 
@@ -650,6 +706,27 @@ int flame_attn_cast_f32_to_bf16(const void* src_f32, void* dst_bf16, int64_t n, 
     hipLaunchKernelGGL(cast_f32_to_bf16_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
                        static_cast<hipStream_t>(stream), static_cast<const float*>(src_f32),
                        static_cast<uint16_t*>(dst_bf16), n);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? FLAME_ATTN_OK : (int)e;
+}
+
+int flame_attn_accumulate_f32(void* acc_f32, const void* grad, int grad_dtype, int64_t n, void* stream) {
+    if (!acc_f32 || !grad || n <= 0) return FLAME_ATTN_ERR_INVALID;
+    if (grad_dtype != FLAME_ATTN_DTYPE_BF16 && grad_dtype != FLAME_ATTN_DTYPE_F32) return FLAME_ATTN_ERR_INVALID;
+    if (n > (int64_t)0x7fffffff * 256) return FLAME_ATTN_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(accumulate_f32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), static_cast<float*>(acc_f32), grad,
+                       grad_dtype == FLAME_ATTN_DTYPE_F32 ? 1 : 0, n);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? FLAME_ATTN_OK : (int)e;
+}
+
+int flame_attn_fill(void* dst, int dtype, float value, int64_t n, void* stream) {
+    if (!dst || n <= 0) return FLAME_ATTN_ERR_INVALID;
+    if (dtype != FLAME_ATTN_DTYPE_BF16 && dtype != FLAME_ATTN_DTYPE_F32) return FLAME_ATTN_ERR_INVALID;
+    if (n > (int64_t)0x7fffffff * 256) return FLAME_ATTN_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(fill_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       dst, value, dtype == FLAME_ATTN_DTYPE_F32 ? 1 : 0, n);
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? FLAME_ATTN_OK : (int)e;
 }

@@ -19,6 +19,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cmath>
 #include <cstdint>
 #include <cstring>
@@ -27,6 +28,7 @@
 #include <optional>
 #include <string>
 #include <tuple>
+#include <unordered_map>
 #include <utility>
 #include <vector>
 
@@ -390,6 +392,39 @@ inline Result<Tensor> forward_v4(const Tensor& q, const Tensor& k, const Tensor&
     return r.value().o;
 }
 
+// sdpa::forward_with_bias(q, k, v, bias, scale) (src/sdpa.rs:232-328): additive float bias on the
+// logits (T5-style relative position bias), softmax in fp32.  scale = None -> 1/sqrt(D); Some(s) ->
+// multiply the scores by s.  bias: optional [B|1, H|1, Q, K], F32 or BF16.  Forward only, as in the
+// reference; runs the fused kernel instead of materialising the fp32 score matrix.
+inline Result<Tensor> forward_with_bias(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor* bias,
+                                        std::optional<float> scale) {
+    auto dv = detail::validate(q, k, v, nullptr);
+    if (!dv.ok()) return dv.error();
+    const detail::Dims d = dv.value();
+    if (!bias) return forward_v4(q, k, v, nullptr, false, scale);
+    const auto& bs = bias->shape();
+    if (bs.size() != 4) return invalid("bias must be 4D [B|1, H|1, Q, K]");
+    if (!(bs[0] == d.B || bs[0] == 1) || !(bs[1] == d.H || bs[1] == 1) || bs[2] != d.Sq || bs[3] != d.Sk)
+        return invalid("bias dims not broadcastable to [B,H,Q,K]");
+    if (bias->dtype() != DType::F32 && bias->dtype() != DType::BF16) return invalid("bias must be F32 or BF16");
+    for (const Tensor* t : {&q, &k, &v})
+        if (!detail::abi_friendly(*t)) return unsupported("tensor view needs D stride 1 and 16-byte aligned rows; make it contiguous first");
+    auto o = Tensor::empty({d.B, d.H, d.Sq, d.D}, DType::BF16);
+    if (!o.ok()) return o.error();
+    std::vector<int64_t> bst(4);
+    const int64_t full[4] = {d.B, d.H, d.Sq, d.Sk};
+    for (int i = 0; i < 4; ++i) bst[i] = (bs[i] == 1 && full[i] != 1) ? 0 : bias->strides()[i];
+    const float sc = scale.value_or(1.0f / std::sqrt((float)d.D));
+    const int rc = flame_attn_fwd_bias_bf16(q.base(), k.base(), v.base(), o.value().base(), nullptr, d.B, d.H, d.Sq, d.Sk, d.D, sc,
+                                            q.strides().data(), k.strides().data(), v.strides().data(), o.value().strides().data(),
+                                            q.offset(), k.offset(), v.offset(), 0, 0, bias->data(),
+                                            bias->dtype() == DType::F32 ? FLAME_ATTN_DTYPE_F32 : FLAME_ATTN_DTYPE_BF16, bst.data(),
+                                            nullptr, nullptr, nullptr);
+    if (rc == FLAME_ATTN_ERR_UNSUPPORTED) return unsupported("flame_attn_fwd_bias_bf16: head dim or layout not built");
+    if (rc != 0) return cuda_error("flame_attn_fwd_bias_bf16", rc);
+    return o.value();
+}
+
 }  // namespace sdpa
 
 // ------------------------------------------------------------------------------------ attention
@@ -409,6 +444,11 @@ inline Result<Tensor> sdpa(const Tensor& q, const Tensor& k, const Tensor& v, co
 }
 inline Result<Tensor> attend(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor* mask = nullptr) {
     return flame::sdpa::forward(q, k, v, mask);
+}
+// attention::sdpa_with_bias(q, k, v, bias, scale) (src/attention/sdpa.rs:542-558)
+inline Result<Tensor> sdpa_with_bias(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor* bias,
+                                     std::optional<float> scale) {
+    return flame::sdpa::forward_with_bias(q, k, v, bias, scale);
 }
 // attention_impl(q, k, v, mask, causal, scale) (src/attention/sdpa.rs:395-458).  The reference
 // rejects mask + causal together (:437-442); both are honoured here.
@@ -451,6 +491,88 @@ struct SdpaCtx {                          // :80-96
     SdpaStats stats;
 };
 
+// ---- tape of the v4 engine (src/autograd_v4/graph.rs:12-94): nodes keyed by the output tensor's id,
+//      in recording order; thread local.
+struct Op {                               // the only variant on this path: Op::Sdpa
+    std::shared_ptr<SdpaCtx> ctx;
+    uint64_t q_id = 0, k_id = 0, v_id = 0;
+};
+struct GradNode {
+    uint64_t id = 0;
+    std::vector<uint64_t> parents;
+    Op op;
+};
+struct Tape {
+    std::unordered_map<uint64_t, std::shared_ptr<GradNode>> nodes;
+    std::vector<uint64_t> order;
+};
+inline Tape& tape() {
+    thread_local Tape t;
+    return t;
+}
+// attach_backward_node / clear_tape (src/autograd_v4/ops/mod.rs:17-25)
+inline void attach_backward_node(std::shared_ptr<GradNode> node) {
+    tape().order.push_back(node->id);
+    tape().nodes[node->id] = std::move(node);
+}
+inline void clear_tape() {
+    tape().nodes.clear();
+    tape().order.clear();
+}
+
+// Gradients (src/autograd_v4/gradients.rs:7-100): id -> fp32 gradient, accumulated on insert
+class Gradients {
+   public:
+    Result<bool> accumulate(uint64_t id, const Tensor& grad) {
+        if (grad.dtype() != DType::BF16 && grad.dtype() != DType::F32) return invalid("Gradients: gradient must be BF16 or F32");
+        if (!grad.is_contiguous()) return unsupported("Gradients: gradient must be contiguous");
+        auto it = map_.find(id);
+        if (it == map_.end()) {
+            auto acc = Tensor::empty(grad.shape(), DType::F32);
+            if (!acc.ok()) return acc.error();
+            int rc = flame_attn_fill(acc.value().data(), FLAME_ATTN_DTYPE_F32, 0.f, acc.value().numel(), nullptr);
+            if (rc != 0) return cuda_error("flame_attn_fill", rc);
+            it = map_.emplace(id, acc.value()).first;
+        } else if (it->second.numel() != grad.numel()) {
+            return invalid("Gradients: shape mismatch on accumulate");
+        }
+        const int rc = flame_attn_accumulate_f32(it->second.data(), grad.data(),
+                                                 grad.dtype() == DType::F32 ? FLAME_ATTN_DTYPE_F32 : FLAME_ATTN_DTYPE_BF16,
+                                                 grad.numel(), nullptr);
+        if (rc != 0) return cuda_error("flame_attn_accumulate_f32", rc);
+        return true;
+    }
+    const Tensor* get(uint64_t id) const {
+        auto it = map_.find(id);
+        return it == map_.end() ? nullptr : &it->second;
+    }
+    std::optional<Tensor> take(uint64_t id) {
+        auto it = map_.find(id);
+        if (it == map_.end()) return std::nullopt;
+        Tensor t = it->second;
+        map_.erase(it);
+        return t;
+    }
+    void register_name(uint64_t id, std::string name) { names_[id] = std::move(name); }
+    const std::string* name_for(uint64_t id) const {
+        auto it = names_.find(id);
+        return it == names_.end() ? nullptr : &it->second;
+    }
+    Result<bool> merge(const Gradients& other) {
+        for (const auto& kv : other.map_) {
+            auto r = accumulate(kv.first, kv.second);
+            if (!r.ok()) return r.error();
+        }
+        for (const auto& kv : other.names_) names_.emplace(kv.first, kv.second);
+        return true;
+    }
+    size_t size() const { return map_.size(); }
+
+   private:
+    std::unordered_map<uint64_t, Tensor> map_;
+    std::unordered_map<uint64_t, std::string> names_;
+};
+
 // sdpa_forward(q,k,v,mask,&cfg) -> (output, ctx) (:98-326).  SaveProbs would materialise the
 // [B,H,Q,K] matrix and dropout is not built: both are refused rather than emulated.
 inline Result<std::pair<Tensor, SdpaCtx>> sdpa_forward(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor* mask,
@@ -468,7 +590,18 @@ inline Result<std::pair<Tensor, SdpaCtx>> sdpa_forward(const Tensor& q, const Te
     ctx.lse = r.value().stats;
     ctx.shapes = {(size_t)q.shape()[0], (size_t)q.shape()[1], (size_t)q.shape()[2], (size_t)k.shape()[2]};
     ctx.stats.bytes_saved = (uint64_t)ctx.o.numel() * 2 + (uint64_t)ctx.lse.numel() * 4;
-    return std::make_pair(r.value().o, ctx);
+    Tensor out = r.value().o;
+    if (q.requires_grad || k.requires_grad || v.requires_grad) {     // record one Op::Sdpa node (:300-324)
+        out.requires_grad = true;
+        auto node = std::make_shared<GradNode>();
+        node->id = out.id();
+        node->op.ctx = std::make_shared<SdpaCtx>(ctx);
+        node->op.q_id = q.id(); node->op.k_id = k.id(); node->op.v_id = v.id();
+        for (const Tensor* t : {&q, &k, &v})
+            if (t->requires_grad) node->parents.push_back(t->id());
+        attach_backward_node(std::move(node));
+    }
+    return std::make_pair(out, ctx);
 }
 
 // sdpa_backward(&ctx, &grad_out) -> (dq, dk, dv) (:826-1009).  Gradients are bf16 here (the
@@ -484,7 +617,67 @@ inline Result<std::tuple<Tensor, Tensor, Tensor>> sdpa_backward(const SdpaCtx& c
     return std::make_tuple(g.value().dq, g.value().dk, g.value().dv);
 }
 
+// backward_v4(loss) (src/autograd_v4/ops/mod.rs:27-74): seed ones at the loss, walk the tape in reverse
+// recording order, accumulate fp32 gradients for the parents that require them, clear the tape.  On this
+// path the "loss" is an attention output itself (no other ops are taped), i.e. the seed is dL/dO = 1.
+inline Result<Gradients> backward_v4(const Tensor& loss) {
+    if (!loss.requires_grad) return Error{Error::InvalidInput, "backward_v4 called on tensor that does not require gradients"};
+    Gradients grads;
+    auto seed = Tensor::empty(loss.shape(), DType::F32);
+    if (!seed.ok()) return seed.error();
+    int rc = flame_attn_fill(seed.value().data(), FLAME_ATTN_DTYPE_F32, 1.0f, seed.value().numel(), nullptr);
+    if (rc != 0) return cuda_error("flame_attn_fill", rc);
+    auto acc = grads.accumulate(loss.id(), seed.value());
+    if (!acc.ok()) return acc.error();
+    const std::vector<uint64_t> order = tape().order;
+    for (auto it = order.rbegin(); it != order.rend(); ++it) {
+        auto nit = tape().nodes.find(*it);
+        if (nit == tape().nodes.end()) continue;
+        const std::shared_ptr<GradNode> node = nit->second;
+        auto grad_out = grads.take(node->id);
+        if (!grad_out) continue;                       // not reachable from the loss
+        auto g = sdpa_backward(*node->op.ctx, *grad_out);
+        if (!g.ok()) return g.error();
+        const auto has = [&](uint64_t id) { return std::find(node->parents.begin(), node->parents.end(), id) != node->parents.end(); };
+        if (has(node->op.q_id)) { auto r = grads.accumulate(node->op.q_id, std::get<0>(g.value())); if (!r.ok()) return r.error(); }
+        if (has(node->op.k_id)) { auto r = grads.accumulate(node->op.k_id, std::get<1>(g.value())); if (!r.ok()) return r.error(); }
+        if (has(node->op.v_id)) { auto r = grads.accumulate(node->op.v_id, std::get<2>(g.value())); if (!r.ok()) return r.error(); }
+    }
+    clear_tape();
+    return grads;
+}
+
 }  // namespace autograd_v4
+
+// ------------------------------------------------------------------------------------ streaming wrappers
+// cuda_ops_bf16::sdpa_stream_bf16(q, k, v, mask, chunk, causal, scale) (src/cuda_ops_bf16.rs:1674-1684)
+// and ops::attn::streaming_attn_bf16_fp32(q, k, v, StreamingAttnCfg) (src/ops/attn.rs:7-25, :327-598):
+// the reference's host-looped / per-row streaming kernels.  Same arguments and checks; the chunk size is
+// validated and otherwise ignored, the fused kernel streams K/V tiles by itself.
+namespace cuda_ops_bf16 {
+inline Result<Tensor> sdpa_stream_bf16(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor* mask, size_t chunk,
+                                       bool causal, std::optional<float> scale) {
+    if (chunk == 0) return invalid("sdpa_stream_bf16: chunk must be > 0");
+    return flame::sdpa::forward_v4(q, k, v, mask, causal, scale);
+}
+}  // namespace cuda_ops_bf16
+
+namespace ops {
+namespace attn {
+struct StreamingAttnCfg {
+    float scale = 1.0f;
+    size_t chunk_size = 2048;
+    bool causal = false;
+    const Tensor* mask = nullptr;
+};
+inline Result<Tensor> streaming_attn_bf16_fp32(const Tensor& q, const Tensor& k, const Tensor& v, const StreamingAttnCfg& cfg) {
+    if (cfg.chunk_size == 0) return invalid("streaming attention chunk_size must be > 0");
+    if (q.dtype() != DType::BF16 || k.dtype() != DType::BF16 || v.dtype() != DType::BF16)
+        return invalid("streaming attention expects BF16 tensors");
+    return flame::sdpa::forward_v4(q, k, v, cfg.mask, cfg.causal, cfg.scale);
+}
+}  // namespace attn
+}  // namespace ops
 
 // ------------------------------------------------------------------------------------ input preparation
 // Counterparts of the reference's rope_fused_bf16 / rope_fused_bf16_f32pe (src/bf16_ops.rs:476-582,

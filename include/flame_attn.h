@@ -70,6 +70,21 @@ int flame_attn_fwd_bf16(const void* Q, const void* K, const void* V, void* O, vo
                         const uint8_t* keep_mask, const int64_t* mask_strides,
                         void* stream);
 
+/* Forward with an additive bias on the scaled logits: softmax(scale * Q K^T + bias) V, fp32 softmax.
+ * bias: fp32 (FLAME_ATTN_DTYPE_F32) or bf16 device tensor read through four element strides over
+ * (B,H,N_q,N_kv); a stride of 0 broadcasts that dimension ([1,H,Q,K] relative-position biases).
+ * keep_mask may be given as well.  Inference only: there is no backward for the bias.
+ * Replaces sdpa::forward_with_bias / attention::sdpa_with_bias (src/sdpa.rs:232-328,
+ * src/attention/sdpa.rs:542-558), which materialise the fp32 score matrix. */
+int flame_attn_fwd_bias_bf16(const void* Q, const void* K, const void* V, void* O, void* LSE,
+                             int B, int H, int N_q, int N_kv, int D, float scale,
+                             const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                             const int64_t* o_strides,
+                             int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off, int64_t lse_off,
+                             const void* bias, int bias_dtype, const int64_t* bias_strides,
+                             const uint8_t* keep_mask, const int64_t* mask_strides,
+                             void* stream);
+
 /* Recommended bytes of device scratch for the backward: two fp32 values per query row (required),
  * plus one 128-key block of fp32 dK/dV partial sums per compute unit of the current device
  * (optional: lets the dK/dV kernel split the key blocks of its last, partly filled scheduling round
@@ -216,6 +231,13 @@ int flame_attn_convert_keep_mask(const void* src, int src_dtype, void* dst_u8, i
  * upstream gradient to the bf16 backward instead of falling back to the materialising recompute as
  * the reference does (src/autograd.rs:702-705). */
 int flame_attn_cast_f32_to_bf16(const void* src_f32, void* dst_bf16, int64_t n, void* stream);
+/* acc_f32[i] += float(grad[i]), grad bf16 or fp32, n contiguous elements: what Gradients::accumulate
+ * of the reference's v4 engine does with tensor ops (src/autograd_v4/gradients.rs:20-32, gradients are
+ * kept in fp32). */
+int flame_attn_accumulate_f32(void* acc_f32, const void* grad, int grad_dtype, int64_t n, void* stream);
+/* dst[i] = value (bf16 or fp32), n contiguous elements: the ones-seed of backward_v4
+ * (src/autograd_v4/ops/mod.rs:37-38) and zero-initialised accumulators. */
+int flame_attn_fill(void* dst, int dtype, float value, int64_t n, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
  * Fused input preparation for joint attention: RMS normalisation over the head dim, interleaved-

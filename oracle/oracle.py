@@ -96,6 +96,25 @@ def sdpa_fwd(q, k, v, scale, causal=False, kv_len=None, mask=None, heads=None, w
     return (O, LSE, O32) if want_f32 else (O, LSE)
 
 
+def sdpa_fwd_bias(q, k, v, scale, bias, want_f32=False):
+    """Naive fp32 forward with an additive fp32 bias [B|1, H|1, Sq, Sk] on the scaled logits."""
+    B, H, Sq, D = q.shape
+    Sk = k.shape[2]
+    q, k, v = (np.ascontiguousarray(t, dtype=np.uint16) for t in (q, k, v))
+    bias = np.ascontiguousarray(bias, dtype=np.float32)
+    assert bias.ndim == 4 and bias.shape[2:] == (Sq, Sk) and bias.shape[0] in (1, B) and bias.shape[1] in (1, H)
+    st = [0 if bias.shape[i] == 1 and i < 2 else bias.strides[i] // 4 for i in range(4)]
+    O = np.zeros((B, H, Sq, D), np.uint16)
+    LSE = np.zeros((B, H, Sq), np.float32)
+    O32 = np.zeros((B, H, Sq, D), np.float32) if want_f32 else None
+    rc = lib().oracle_sdpa_fwd_bias(
+        _p(q), _p(k), _p(v), B, H, Sq, Sk, D, ctypes.c_float(scale), _p(bias),
+        *(ctypes.c_int64(s_) for s_ in st), _p(O), _p(LSE), _p(O32))
+    if rc != 0:
+        raise RuntimeError(f"oracle_sdpa_fwd_bias failed: {rc}")
+    return (O, LSE, O32) if want_f32 else (O, LSE)
+
+
 def sdpa_bwd(q, k, v, o, do, scale, causal=False, kv_len=None, mask=None, heads=None, want_f32=False):
     """Naive fp32 backward. Returns (dQ, dK, dV) bf16 bits [+ fp32 copies]."""
     B, H, Sq, D = q.shape

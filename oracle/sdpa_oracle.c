@@ -11,6 +11,7 @@
  *   forward   tests/fa2_parity_naive.rs:90-140      (upcast, QK^T, scale, max/exp/sum/div, PV, bf16)
  *   backward  tests/cudnn_sdpa_bwd_parity.rs:31-98  (dV=P^T dO, dP=dO V^T, D=rowsum(dO*O),
  *                                                    dS=P*(dP-D), dQ=dS K scale, dK=dS^T Q scale)
+ *   bias      src/sdpa.rs:232-328                   (additive fp32 bias on the scaled logits, forward only)
  *   keep-mask src/sdpa.rs:458-470, src/tests/attention_tests.rs:61-108 (mask < 0.5 => excluded)
  *   causal    kernels/sdpa_kernels.cu:129-135       (absolute k > q is excluded)
  *   LSE       third_party/cudnn_frontend/include/cudnn_frontend/node/softmax.h:139-213
@@ -28,6 +29,8 @@
  *
  * Pinning status (see tests/test_oracle_*.py):
  *   forward O        pinned: reference 2x2 known-answer test, fp64 brute force, torch CPU SDPA, invariants
+ *   additive bias    pinned: torch CPU SDPA with a float attn_mask, shift invariance (bias constant
+ *                    per row leaves O unchanged), bias = -inf-like values reproduce the keep-mask result
  *   LSE              pinned by the closed form and sum_j exp(s_ij - LSE_i) = 1 only;
  *                    no reference test asserts Stats values ("parity unpinned" by the reference itself)
  *   dQ, dK, dV       pinned: fp64 central finite differences, torch CPU autograd
@@ -89,6 +92,8 @@ typedef struct {
     const int32_t* kv_len;   /* [B] or NULL: keys >= kv_len[b] are excluded          */
     const uint8_t* mask;     /* keep-mask (non-zero = attend) or NULL                 */
     int64_t msb, msh, msq, msk; /* element strides of mask over (b,h,q,k); 0 = broadcast */
+    const float* bias;       /* additive fp32 bias on the scaled logits or NULL (src/sdpa.rs:288-305) */
+    int64_t bsb, bsh, bsq, bsk; /* its element strides over (b,h,q,k); 0 = broadcast     */
 } mask_spec;
 
 static inline int excluded(const mask_spec* ms, int b, int h, int i, int j) {
@@ -112,6 +117,7 @@ static void head_probs(const float* q, const float* kt, int Sq, int Sk, int D, f
         float m = -INFINITY;
         for (int j = 0; j < Sk; ++j) {
             float s = excluded(ms, b, h, i, j) ? -INFINITY : row[j] * scale;
+            if (ms->bias && s != -INFINITY) s += ms->bias[b * ms->bsb + h * ms->bsh + i * ms->bsq + j * ms->bsk];
             row[j] = s;
             if (s > m) m = s;
         }
@@ -141,14 +147,34 @@ static int check_dims(int B, int H, int Sq, int Sk, int D) {
  * heads_begin/heads_end restrict the work to flat (b*H+h) indices in [begin,end) so that
  * long configurations can be checked on a head subset; pass 0 and B*H for everything.
  */
+static int sdpa_fwd_impl(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
+                         int B, int H, int Sq, int Sk, int D, float scale, mask_spec ms,
+                         int heads_begin, int heads_end, uint16_t* O, float* LSE, float* O32);
+
 int oracle_sdpa_fwd(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
                     int B, int H, int Sq, int Sk, int D, float scale, int causal,
                     const int32_t* kv_len, const uint8_t* mask,
                     int64_t msb, int64_t msh, int64_t msq, int64_t msk,
                     int heads_begin, int heads_end,
                     uint16_t* O, float* LSE, float* O32) {
+    mask_spec ms = {causal, kv_len, mask, msb, msh, msq, msk, NULL, 0, 0, 0, 0};
+    return sdpa_fwd_impl(Q, K, V, B, H, Sq, Sk, D, scale, ms, heads_begin, heads_end, O, LSE, O32);
+}
+
+/* Forward with an additive fp32 bias on the scaled logits (T5-style relative position bias),
+ * following src/sdpa.rs:232-328: scores * scale, + bias, fp32 softmax, P V. */
+int oracle_sdpa_fwd_bias(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
+                         int B, int H, int Sq, int Sk, int D, float scale,
+                         const float* bias, int64_t bsb, int64_t bsh, int64_t bsq, int64_t bsk,
+                         uint16_t* O, float* LSE, float* O32) {
+    mask_spec ms = {0, NULL, NULL, 0, 0, 0, 0, bias, bsb, bsh, bsq, bsk};
+    return sdpa_fwd_impl(Q, K, V, B, H, Sq, Sk, D, scale, ms, 0, B * H, O, LSE, O32);
+}
+
+static int sdpa_fwd_impl(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
+                         int B, int H, int Sq, int Sk, int D, float scale, mask_spec ms,
+                         int heads_begin, int heads_end, uint16_t* O, float* LSE, float* O32) {
     if (check_dims(B, H, Sq, Sk, D)) return -1;
-    mask_spec ms = {causal, kv_len, mask, msb, msh, msq, msk};
     int fail = 0;
 #pragma omp parallel for schedule(dynamic, 1)
     for (int bh = heads_begin; bh < heads_end; ++bh) {
@@ -206,7 +232,7 @@ int oracle_sdpa_bwd(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
                     uint16_t* dQ, uint16_t* dK, uint16_t* dV,
                     float* dQ32, float* dK32, float* dV32) {
     if (check_dims(B, H, Sq, Sk, D)) return -1;
-    mask_spec ms = {causal, kv_len, mask, msb, msh, msq, msk};
+    mask_spec ms = {causal, kv_len, mask, msb, msh, msq, msk, NULL, 0, 0, 0, 0};
     int fail = 0;
 #pragma omp parallel for schedule(dynamic, 1)
     for (int bh = heads_begin; bh < heads_end; ++bh) {

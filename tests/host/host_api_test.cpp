@@ -346,6 +346,97 @@ int main() {
         CHECK(!bf16_ops::rope_fused_bf16_f32pe(normed.value(), bad, bad).ok(), "f32pe must refuse bf16 tables");
     }
 
+    // ---- 8. additive bias (sdpa::forward_with_bias): against a scalar softmax(scale*QK^T + bias) V on the host
+    {
+        std::printf("[forward_with_bias]\n");
+        const int B = 1, H = 2, Sq = 70, Sk = 90, D = 64;
+        auto hq = randn_bf16((size_t)B * H * Sq * D), hk = randn_bf16((size_t)B * H * Sk * D), hv = randn_bf16((size_t)B * H * Sk * D);
+        std::vector<float> hb((size_t)H * Sq * Sk);
+        for (auto& x : hb) x = 1.5f * gauss();
+        Tensor q = dev_bf16(hq, {B, H, Sq, D}), k = dev_bf16(hk, {B, H, Sk, D}), v = dev_bf16(hv, {B, H, Sk, D});
+        Tensor bias = Tensor::from_host(hb.data(), {1, H, Sq, Sk}, DType::F32).value();
+        auto o = sdpa::forward_with_bias(q, k, v, &bias, 0.2f);
+        CHECK(o.ok(), "forward_with_bias failed");
+        if (o.ok()) {
+            auto got = host_f32_of_bf16(o.value());
+            std::vector<float> ref(got.size());
+            std::vector<double> s(Sk);
+            for (int h = 0; h < H; ++h)
+                for (int i = 0; i < Sq; ++i) {
+                    double m = -1e300;
+                    for (int j = 0; j < Sk; ++j) {
+                        double acc = 0;
+                        for (int d = 0; d < D; ++d) acc += (double)bf2f(hq[((size_t)h * Sq + i) * D + d]) * bf2f(hk[((size_t)h * Sk + j) * D + d]);
+                        s[j] = acc * 0.2 + hb[((size_t)h * Sq + i) * Sk + j];
+                        m = std::fmax(m, s[j]);
+                    }
+                    double l = 0;
+                    for (int j = 0; j < Sk; ++j) { s[j] = std::exp(s[j] - m); l += s[j]; }
+                    for (int d = 0; d < D; ++d) {
+                        double acc = 0;
+                        for (int j = 0; j < Sk; ++j) acc += s[j] * bf2f(hv[((size_t)h * Sk + j) * D + d]);
+                        ref[((size_t)h * Sq + i) * D + d] = (float)(acc / l);
+                    }
+                }
+            compare("O (bias)", got, ref);
+        }
+        Tensor badb = Tensor::empty({1, H, Sq, Sk + 1}, DType::F32).value();
+        CHECK(!sdpa::forward_with_bias(q, k, v, &badb, std::nullopt).ok(), "bias with a wrong K extent must be refused");
+        ops::attn::StreamingAttnCfg cfg;
+        cfg.scale = 0.125f;
+        cfg.causal = true;
+        auto so = ops::attn::streaming_attn_bf16_fp32(q, k, v, cfg);
+        auto so2 = cuda_ops_bf16::sdpa_stream_bf16(q, k, v, nullptr, 1024, true, 0.125f);
+        CHECK(so.ok() && so2.ok(), "streaming wrappers failed");
+        if (so.ok() && so2.ok()) CHECK(host_f32_of_bf16(so.value()) == host_f32_of_bf16(so2.value()), "streaming wrappers disagree");
+        cfg.chunk_size = 0;
+        CHECK(!ops::attn::streaming_attn_bf16_fp32(q, k, v, cfg).ok(), "chunk_size 0 must be refused");
+    }
+
+    // ---- 9. v4 engine: tape, Gradients, backward_v4 (seed = ones at the attention output)
+    {
+        std::printf("[autograd_v4 tape]\n");
+        const int B = 1, H = 2, N = 96, D = 64;
+        auto hq = randn_bf16((size_t)B * H * N * D), hk = randn_bf16(hq.size()), hv = randn_bf16(hq.size());
+        Tensor q = dev_bf16(hq, {B, H, N, D}), k = dev_bf16(hk, {B, H, N, D}), v = dev_bf16(hv, {B, H, N, D});
+        q.requires_grad = true;
+        v.requires_grad = true;                    // k does not require a gradient
+        autograd_v4::clear_tape();
+        autograd_v4::SdpaConfig cfg;
+        cfg.causal = true;
+        auto f = autograd_v4::sdpa_forward(q, k, v, nullptr, cfg);
+        CHECK(f.ok(), "sdpa_forward failed");
+        if (f.ok()) {
+            CHECK(autograd_v4::tape().order.size() == 1, "one node expected on the tape");
+            auto grads = autograd_v4::backward_v4(f.value().first);
+            CHECK(grads.ok(), "backward_v4 failed");
+            CHECK(autograd_v4::tape().order.empty(), "backward_v4 must clear the tape");
+            if (grads.ok()) {
+                CHECK(grads.value().get(q.id()) && grads.value().get(v.id()) && !grads.value().get(k.id()), "gradients for q and v only");
+                std::vector<uint16_t> ones((size_t)B * H * N * D, f2bf(1.0f));
+                Tensor g1 = dev_bf16(ones, {B, H, N, D});
+                auto direct = autograd_v4::sdpa_backward(f.value().second, g1);
+                CHECK(direct.ok(), "sdpa_backward failed");
+                if (direct.ok() && grads.value().get(q.id())) {
+                    std::vector<float> gq((size_t)B * H * N * D);
+                    CHECK(grads.value().get(q.id())->dtype() == DType::F32, "accumulated gradients are fp32");
+                    CHECK(grads.value().get(q.id())->to_host(gq.data()).ok(), "to_host");
+                    CHECK(gq == host_f32_of_bf16(std::get<0>(direct.value())), "backward_v4 dQ != sdpa_backward dQ");
+                    // accumulate twice: the sum doubles
+                    autograd_v4::Gradients acc;
+                    CHECK(acc.accumulate(7, std::get<0>(direct.value())).ok() && acc.accumulate(7, std::get<0>(direct.value())).ok(), "accumulate");
+                    std::vector<float> twice(gq.size());
+                    CHECK(acc.get(7)->to_host(twice.data()).ok(), "to_host");
+                    bool dbl = true;
+                    for (size_t i = 0; i < gq.size(); ++i) dbl = dbl && twice[i] == 2.0f * gq[i];
+                    CHECK(dbl, "accumulating the same gradient twice must double it");
+                }
+            }
+        }
+        Tensor plain = dev_bf16(hq, {B, H, N, D});
+        CHECK(!autograd_v4::backward_v4(plain).ok(), "backward_v4 on a tensor without requires_grad must fail");
+    }
+
     if (hipDeviceSynchronize() != hipSuccess) ++g_fail;
     std::printf(g_fail ? "HOST API TEST: %d FAILURES\n" : "HOST API TEST: all checks passed\n", g_fail);
     return g_fail ? 1 : 0;

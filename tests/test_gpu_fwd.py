@@ -152,3 +152,35 @@ def test_invalid_arguments_are_rejected():
     with pytest.raises(capi.FlameAttnError) as e:
         capi.attn_fwd(q.transpose(2, 3), q, q, 0.1)         # D stride != 1
     assert e.value.code in (capi.ERR_UNSUPPORTED, capi.ERR_INVALID)
+
+
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("bias_dtype", ["f32", "bf16"])
+def test_additive_bias(oracle, D, bias_dtype):
+    """softmax(scale*QK^T + bias) V with a [1,H,Sq,Sk] relative-position style bias."""
+    from flame_amd import capi
+    B, H, Sq, Sk = 2, 3, 200, 333
+    print(f"[fwd bias] D={D} bias={bias_dtype}", flush=True)
+    q, k, v = (W.f32_to_bf16_bits(W.normal_f32(91, s, B * H * n * D).reshape(B, H, n, D))
+               for s, n in enumerate((Sq, Sk, Sk)))
+    bias = (W.normal_f32(91, 7, H * Sq * Sk).reshape(1, H, Sq, Sk) * np.float32(1.5)).astype(np.float32)
+    if bias_dtype == "bf16":
+        bias_bits = W.f32_to_bf16_bits(bias)
+        bias = W.bf16_bits_to_f32(bias_bits)
+        bd = to_dev(bias_bits)
+    else:
+        bd = torch.from_numpy(bias).cuda()
+    scale = 1.0 / math.sqrt(D)
+    o, lse = capi.attn_fwd_bias(to_dev(q), to_dev(k), to_dev(v), scale, bd)
+    torch.cuda.synchronize()
+    ro, rlse, rof = oracle.sdpa_fwd_bias(q, k, v, scale, bias, want_f32=True)
+    assert_close_bf16(oracle, "O", to_f32(o), ro, rof)
+    assert np.max(np.abs(lse.cpu().numpy().reshape(rlse.shape) - rlse)) <= TOL_LSE
+    # with a keep-mask on top
+    keep = (np.random.default_rng(5).random((B, 1, Sq, Sk)) < 0.5).astype(np.uint8)
+    keep[..., 0] = 1
+    o2, _ = capi.attn_fwd_bias(to_dev(q), to_dev(k), to_dev(v), scale, bd, mask=torch.from_numpy(keep).cuda())
+    torch.cuda.synchronize()
+    ro2, _, rof2 = oracle.sdpa_fwd_bias(q, k, v, scale, (bias + (1.0 - keep) * np.float32(-1e9)).astype(np.float32),
+                                        want_f32=True)
+    assert_close_bf16(oracle, "O masked", to_f32(o2), ro2, rof2)

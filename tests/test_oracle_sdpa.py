@@ -202,3 +202,33 @@ def test_ragged_tail_is_excluded_not_zero_filled(oracle):
         a, la = oracle.sdpa_fwd(q, k, v, 0.125, kv_len=np.array([L], np.int32))
         b, lb = oracle.sdpa_fwd(q, k[:, :, :L].copy(), v[:, :, :L].copy(), 0.125)
         assert np.array_equal(a, b) and np.array_equal(la, lb)
+
+
+def test_additive_bias_forward_against_torch_and_invariants(oracle):
+    """softmax(scale*QK^T + bias) V: torch's CPU SDPA with a float attn_mask is the library check; a
+    bias that is constant along each row must leave O unchanged; a bias of -1e9 where a keep-mask is 0
+    must reproduce the keep-mask result (the reference's own masking arithmetic, src/sdpa.rs:458-470)."""
+    import torch
+    import torch.nn.functional as F
+    B, H, Sq, Sk, D = 2, 3, 37, 53, 64
+    q, k, v = (W.f32_to_bf16_bits(W.normal_f32(77, s, B * H * n * D).reshape(B, H, n, D))
+               for s, n in enumerate((Sq, Sk, Sk)))
+    bias = (W.normal_f32(77, 9, H * Sq * Sk).reshape(1, H, Sq, Sk) * np.float32(2.0)).astype(np.float32)
+    scale = 0.3
+    o, lse, o32 = oracle.sdpa_fwd_bias(q, k, v, scale, bias, want_f32=True)
+    tq, tk, tv = (torch.from_numpy(W.bf16_bits_to_f32(t)) for t in (q, k, v))
+    ref = F.scaled_dot_product_attention(tq, tk, tv, attn_mask=torch.from_numpy(bias), scale=scale).numpy()
+    assert np.max(np.abs(o32 - ref)) < 2e-5
+    s = np.einsum("bhqd,bhkd->bhqk", tq.numpy().astype(np.float64), tk.numpy().astype(np.float64)) * scale + bias
+    assert np.max(np.abs(lse - np.log(np.exp(s - s.max(-1, keepdims=True)).sum(-1)) - s.max(-1))) < 1e-4
+    # row-constant bias: softmax is shift invariant
+    rowc = np.broadcast_to(W.normal_f32(78, 0, H * Sq).reshape(1, H, Sq, 1), (1, H, Sq, Sk)).copy()
+    o_c, _ = oracle.sdpa_fwd_bias(q, k, v, scale, rowc)
+    o_0, _ = oracle.sdpa_fwd(q, k, v, scale)
+    assert np.max(np.abs(W.bf16_bits_to_f32(o_c) - W.bf16_bits_to_f32(o_0))) <= 2 ** -7
+    # large negative bias == keep-mask
+    keep = (np.random.default_rng(3).random((B, 1, Sq, Sk)) < 0.7).astype(np.uint8)
+    keep[..., 0] = 1
+    o_m, _ = oracle.sdpa_fwd(q, k, v, scale, mask=keep)
+    o_b, _ = oracle.sdpa_fwd_bias(q, k, v, scale, ((1.0 - keep) * -1e9).astype(np.float32))
+    assert np.array_equal(o_m, o_b)
