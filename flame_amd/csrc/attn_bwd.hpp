@@ -557,10 +557,12 @@ struct BwdDqTile {
     static constexpr int DMA_PER_WAVE = BN / ROWS_PER_DMA / 4;
 };
 
-template <int D, bool HASMASK>
-__global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams p) {
+// NW wavefronts (4 or 8) of 32 queries each per workgroup; eight share every K/V tile among twice as
+// many queries.  Two wavefronts per SIMD either way.
+template <int D, bool HASMASK, int NW>
+__global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void bwd_dq_kernel(const BwdParams p) {
     using T = BwdDqTile<D>;
-    constexpr int BM = T::BM, BN = T::BN, RS = T::RS;
+    constexpr int BM = 32 * NW, BN = T::BN, RS = T::RS;
     constexpr int DC = D / 16;
     constexpr int DB = D / 32;
     constexpr int GPR = D / 8;
@@ -632,7 +634,7 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams p) {
     }
 
     const int dma_row_in = lane / GPR, dma_gran = lane % GPR;
-    constexpr int NDMA = T::DMA_PER_WAVE;
+    constexpr int NDMA = T::DMA_PER_WAVE * 4 / NW;
     const uint32_t lds0 = lds_addr(lds);
     uint32_t k_lane_off[NDMA], v_lane_off[NDMA];     // bytes
 #pragma unroll

@@ -1,8 +1,10 @@
 // Tiled QK^T -> online softmax -> PV forward for gfx950.  Writes O (bf16) and, when asked, the
 // per-row log-sum-exp of the scaled logits; the Sq x Sk score matrix never leaves registers.
 //
-// One workgroup = 4 wavefronts = 128 query rows of one (batch, head); each wavefront owns
-// 32 rows whose Q fragments stay in registers.  K/V tiles of 64 keys are copied global -> LDS
+// One workgroup = NW wavefronts (4 or 8) = 32*NW query rows of one (batch, head); each wavefront owns
+// 32 rows whose Q fragments stay in registers.  Eight wavefronts share each K/V tile among twice as
+// many queries (half the copy traffic per MFMA) and are used when the query count fills such
+// workgroups; either way two wavefronts are resident per SIMD.  K/V tiles of 64 keys are copied global -> LDS
 // by the asynchronous LDS-DMA loads (no staging registers), double buffered, row-major with an XOR
 // swizzle of the 16-byte granules so that both the row reads of K and the transposing reads of V are
 // free of bank conflicts without padding.  The logits are produced transposed, S^T = K Q^T, so that
@@ -46,16 +48,20 @@ struct FwdTile {
     static constexpr int DMA_PER_WAVE = BN / ROWS_PER_DMA / 4;   // copies per wave and tensor
 };
 
-template <int D, bool HASMASK>
-__global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
+template <int D, bool HASMASK, int NW>
+__global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void fwd_kernel(const FwdParams p) {
     using T = FwdTile<D>;
     constexpr int BN = T::BN, RS = T::RS;
-    constexpr int BM = 128;
+    constexpr int BM = 32 * NW;  // query rows per workgroup
     constexpr int DC = D / 16;   // contraction chunks of QK^T
     constexpr int DB = D / 32;   // 32-row blocks of O^T
     constexpr int GPR = D / 8;   // 16-byte granules per row
-    constexpr int NDMA = T::DMA_PER_WAVE;
+    constexpr int NDMA = T::DMA_PER_WAVE * 4 / NW;
     constexpr int PD = 4;        // LDS read-ahead depth, in fragments
+    // Tile t lives in stage t % 2; K runs 2 tiles and V 1 tile ahead of use, one barrier per step.
+    // (Measured: four stages with deeper prefetch, or a barrier only every second step, are slower.)
+    constexpr int NSTAGE = 2;
+    constexpr int KD = NSTAGE / 2 + 1, VD = NSTAGE / 2;      // prefetch distances, in tiles
     static_assert((2 * DC) % PD == 0 && (4 * DB) % PD == 0, "read-ahead depth must divide the fragment counts");
     static_assert(2 * DC == 16 || 2 * DC == 8, "softmax slicing assumes 16 or 8 logit MFMAs per tile");
 
@@ -114,7 +120,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
         v_lane_off[i] = 2u * (uint32_t)(row * (int)p.vs.n + c * 8);
     }
     auto dst_of = [&](int t, int which, int i) {             // LDS byte address of copy i of this wave
-        return lds0 + 2u * (uint32_t)((t & 1) * T::STAGE_ELEMS + which * T::TILE_ELEMS + (wave * NDMA + i) * 512);
+        return lds0 + 2u * (uint32_t)((t & (NSTAGE - 1)) * T::STAGE_ELEMS + which * T::TILE_ELEMS + (wave * NDMA + i) * 512);
     };
     auto issue_ragged = [&](const uint16_t* base, int64_t row_stride, int t, int which) {
 #pragma unroll
@@ -151,11 +157,11 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
             voff[half][db] = row * RS + (((4 * db + 2 * tr_g16 + ((tr_r & 3) >> 1)) ^ swz<D>(row)) << 3) + 4 * (tr_r & 1);
     }
     auto k_frag = [&](int t, int i) {       // fragment i = (dc, kb) of K(t)
-        const uint16_t* ks = lds + (t & 1) * T::STAGE_ELEMS;
+        const uint16_t* ks = lds + (t & (NSTAGE - 1)) * T::STAGE_ELEMS;
         return *reinterpret_cast<const bf16x8*>(ks + koff[i >> 1] + 32 * (i & 1) * RS);
     };
     auto v_frag = [&](int t, int i) {       // fragment i = (cc, db) of V(t)^T
-        const uint16_t* vs = lds + (t & 1) * T::STAGE_ELEMS + T::TILE_ELEMS;
+        const uint16_t* vs = lds + (t & (NSTAGE - 1)) * T::STAGE_ELEMS + T::TILE_ELEMS;
         const int cc = i / DB, db = i % DB;
         const u32x2 lo = lds_read_tr16(vs + voff[0][db] + 16 * cc * RS);
         const u32x2 hi = lds_read_tr16(vs + voff[1][db] + 16 * cc * RS);
@@ -229,17 +235,17 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
     };
 
     // One step: P(t) from the logits in `cur`, logits of tile t+1 into `nxt`, O += P(t) V(t).
-    // FAST: tile t+1 needs no exclusions and K(t+2), V(t+1) are full tiles (straight-line copies and the
-    // interleaved instruction stream).  Otherwise every decision is taken at run time and the phases
-    // run one after the other.
+    // FAST: tile t+1 needs no exclusions and K(t+KD), V(t+VD) are full tiles (straight-line copies and
+    // the interleaved instruction stream).  Otherwise every decision is taken at run time and the
+    // phases run one after the other.
     auto step = [&](auto fast_tag, f32x16 (&cur)[2], f32x16 (&nxt)[2], int t) {
         constexpr bool FAST = decltype(fast_tag)::value;
         const bool has_next = FAST || t + 1 < n_tiles;
         if (FAST) {
-            issue_full_kv(t + 2, t + 1);
+            issue_full_kv(t + KD, t + VD);
         } else {
-            if (t + 2 < n_tiles) issue_k(t + 2);
-            if (has_next) issue_v(t + 1);
+            if (t + KD < n_tiles) issue_k(t + KD);
+            if (t + VD < n_tiles) issue_v(t + VD);
         }
         const float m_use = (m_run == -INFINITY) ? 0.f : m_run;
         const float msc = m_use * c_log2;
@@ -346,10 +352,12 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
 
     f32x16 sa[2], sb[2];
     if (n_tiles > 0) {
-        // prologue: K(0), V(0), K(1) land; logits and maximum of tile 0
-        issue_k(0);
-        issue_v(0);
-        if (n_tiles > 1) issue_k(1);
+        // prologue: the first KD tiles of K and VD tiles of V land; logits and maximum of tile 0
+#pragma unroll
+        for (int i = 0; i < KD; ++i) {
+            if (i < n_tiles) issue_k(i);
+            if (i < VD && i < n_tiles) issue_v(i);
+        }
         wait_vm0();
         __syncthreads();
         zero_tile(sa);
@@ -364,8 +372,8 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
         fold_max(tmax);
         __syncthreads();     // every wave has read K(0) before step 0 starts overwriting it
 
-        // step t is FAST when t + 2 < n_full; an even number of them keeps `sa` the current tile
-        const int n_fast = max(0, n_full - 2) & ~1;
+        // step t is FAST when t + KD < n_full; an even number of them keeps `sa` the current tile
+        const int n_fast = max(0, n_full - KD) & ~1;
         int t = 0;
         for (; t < n_fast; t += 2) {
             step(std::true_type{}, sa, sb, t);

@@ -240,16 +240,18 @@ __device__ __forceinline__ constexpr int swz_i8(int row) {
     return D == 128 ? swz<64>(row) : ((row >> 2) & 3);
 }
 
-template <int D>
-__global__ __launch_bounds__(256, 2) void sage_fwd_kernel(const SageFwdParams p) {
+// NW wavefronts (4 or 8) of 32 queries each per workgroup, as in the bf16 forward kernel.
+template <int D, int NW>
+__global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sage_fwd_kernel(const SageFwdParams p) {
     using T = SageTile<D>;
-    constexpr int BM = T::BM, BN = T::BN;
+    constexpr int BM = 32 * NW, BN = T::BN;
     constexpr int KC = D / 32;   // int8 contraction chunks (32 per MFMA)
     constexpr int DB = D / 32;   // 32-row blocks of O^T
     constexpr int RS = D;        // V row stride, elements
     constexpr int GPK = D / 16;  // 16-byte granules per K^ row
     constexpr int GPV = D / 8;   // ... per V row
-    constexpr int NKD = T::K_DMA_PER_WAVE, NVD = T::V_DMA_PER_WAVE;
+    constexpr int NKD = T::K_DMA_PER_WAVE * 4 / NW, NVD = T::V_DMA_PER_WAVE * 4 / NW;
+    static_assert(NKD >= 1 && NVD >= 1, "too many wavefronts for this tile");
     constexpr int PD = 4;
     constexpr int NS = 2 * KC;   // logit MFMAs per tile
     constexpr int NP = 4 * DB;   // PV MFMAs per tile
@@ -295,8 +297,9 @@ __global__ __launch_bounds__(256, 2) void sage_fwd_kernel(const SageFwdParams p)
         for (int kc = 0; kc < KC; ++kc)
             qf[kc] = row < p.Sq ? *reinterpret_cast<const i32x4*>(qbase + (int64_t)row * D + 32 * kc + 16 * h) : z;
     }
-    // one quantisation block of Q per workgroup (BM == 128); fold softmax scale and log2(e)
-    const float qfac = p.sq[(int64_t)bh * n_qt + qt] * p.scale * kLog2e;
+    // the 32 queries of a wavefront lie in one quantisation block of Q (128 rows); fold softmax scale and log2(e)
+    const int nqb = (p.Sq + kSageQBlk - 1) / kSageQBlk;
+    const float qfac = p.sq[(int64_t)bh * nqb + min(qw0 / kSageQBlk, nqb - 1)] * p.scale * kLog2e;
 
     // ---- asynchronous tile copies: K^(t) and V(t) live in stage t&1
     const uint32_t lds0 = lds_addr(lds8);
