@@ -135,3 +135,15 @@ def test_split_last_round_matches_unsplit_walk():
         assert bool((diff <= ulp + 1e-3).all()), (name, float(diff.max()))     # 1e-3: cancellation near zero
         whole = slice(0, 20)                             # heads whose key blocks all sit in the unsplit range
         assert torch.equal(x[:, whole], y[:, whole]), name
+
+
+@pytest.mark.parametrize("mode", ["causal", "kvlen"])
+def test_wide_workgroups_with_exclusions(oracle, mode):
+    """Enough query tiles that the forward and dQ kernels pick their 256-query (8-wavefront)
+    workgroups, combined with a causal diagonal or ragged key lengths; oracle parity on a head subset."""
+    B, H, S, D = 2, 16, 2048, 128
+    t = [W.f32_to_bf16_bits(W.normal_f32(4242, s, B * H * S * D).reshape(B, H, S, D) * np.float32(0.7071)) for s in range(4)]
+    w = W.Workload(f"wide_{mode}", t[0], t[1], t[2], t[3], 1.0 / math.sqrt(D), causal=(mode == "causal"),
+                   kv_len=np.array([S, 777], np.int32) if mode == "kvlen" else None)
+    _check_bwd(oracle, w, heads=(0, 1), tag="first head")
+    _check_bwd(oracle, w, heads=(B * H - 1, B * H), tag="last head")
