@@ -34,27 +34,6 @@ __device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
 }
 
-// acc *= alpha for an accumulator that lives in the accumulation register file, done with explicit
-// reads/writes of that file so that the (rare) rescale does not pull the accumulator into the
-// architectural registers for the whole loop.  The leading no-ops cover the MFMA-write -> accvgpr-read
-// wait states that the assembler-level hazard recogniser cannot see inside an asm block.
-__device__ __forceinline__ void scale_acc_agpr(f32x16& acc, float alpha) {
-    float t0, t1, t2, t3;
-    asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 3" ::: "memory");
-#define FATTN_SCALE4(i)                                                                                   \
-    asm volatile("v_accvgpr_read_b32 %1, %0\n\t"                                                          \
-                 "v_mul_f32 %1, %1, %2\n\t"                                                               \
-                 "s_nop 1\n\t"                                                                            \
-                 "v_accvgpr_write_b32 %0, %1"                                                              \
-                 : "+a"(acc[i]), "=&v"(t0)                                                                 \
-                 : "v"(alpha));
-    FATTN_SCALE4(0) FATTN_SCALE4(1) FATTN_SCALE4(2) FATTN_SCALE4(3) FATTN_SCALE4(4) FATTN_SCALE4(5)
-    FATTN_SCALE4(6) FATTN_SCALE4(7) FATTN_SCALE4(8) FATTN_SCALE4(9) FATTN_SCALE4(10) FATTN_SCALE4(11)
-    FATTN_SCALE4(12) FATTN_SCALE4(13) FATTN_SCALE4(14) FATTN_SCALE4(15)
-#undef FATTN_SCALE4
-    (void)t1; (void)t2; (void)t3;
-}
-
 // row index inside a 32x32 accumulator block for register r of a lane in half h
 __device__ __forceinline__ constexpr int acc_row(int r, int h) { return 8 * (r >> 2) + 4 * h + (r & 3); }
 
@@ -97,38 +76,6 @@ __device__ __forceinline__ u32x2 lds_read_tr16(const uint16_t* p) {
     s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p));
     return __builtin_bit_cast(u32x2, v);
 }
-
-// MFMA 32x32x16 operand (8 contraction elements for column n = lane%32) gathered from a row-major
-// LDS tile X[k][col]: elements 0..3 = X[k0 + 4h + 0..3][c0 + n], elements 4..7 = X[k0 + 8 + 4h + 0..3][c0 + n].
-// This k order matches a 32x32 accumulator lane (rows 8g + 4h + t), so accumulator values converted
-// to bf16 pair with it directly.
-__device__ __forceinline__ bf16x8 lds_tr_frag(const uint16_t* tile, int stride, int k0, int c0, int lane) {
-    const int r = lane & 15, g16 = (lane >> 4) & 1, h = lane >> 5;
-    const uint16_t* p = tile + (k0 + 4 * h + (r >> 2)) * stride + c0 + 16 * g16 + 4 * (r & 3);
-    const u32x2 lo = lds_read_tr16(p);
-    const u32x2 hi = lds_read_tr16(p + 8 * stride);
-    u32x4 u = {lo[0], lo[1], hi[0], hi[1]};
-    return __builtin_bit_cast(bf16x8, u);
-}
-
-// Transposes a 4 (rows) x 8 (cols) block of bf16 held as four 16-byte row vectors into eight
-// 8-byte column vectors: out[c] = {r0[c], r1[c], r2[c], r3[c]}.
-__device__ __forceinline__ void transpose4x8(const u32x4 r[4], u32x2 out[8]) {
-#pragma unroll
-    for (int m = 0; m < 4; ++m) {
-        const uint32_t a = r[0][m], b = r[1][m], c = r[2][m], d = r[3][m];
-        out[2 * m][0] = (a & 0xffffu) | (b << 16);
-        out[2 * m][1] = (c & 0xffffu) | (d << 16);
-        out[2 * m + 1][0] = (a >> 16) | (b & 0xffff0000u);
-        out[2 * m + 1][1] = (c >> 16) | (d & 0xffff0000u);
-    }
-}
-
-// Position of the 4-row group g (rows 4g..4g+3 of a tile) inside a transposed LDS row, chosen so
-// that the eight contraction slots one lane feeds to an MFMA are 16 contiguous bytes:
-// an accumulator lane in half h holds rows {16c+4h+t} and {16c+8+4h+t}, t=0..3, of chunk c, i.e.
-// groups 4c+h and 4c+2+h; they are stored at slots 4c+2h and 4c+2h+1.
-__device__ __forceinline__ constexpr int tslot(int g) { return (g & ~3) | ((g & 1) << 1) | ((g >> 1) & 1); }
 
 // 16-byte-granule XOR swizzle of a row-major bf16 tile whose rows are D*2 bytes (no padding).
 // 16 consecutive rows get distinct bank groups for the same logical granule, and 4 consecutive rows
