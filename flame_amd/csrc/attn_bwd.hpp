@@ -366,21 +366,30 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
                     }
                     rows_ahead(0, 0);
                 }
-#pragma unroll
-                for (int i = 0; i < NA; ++i) {
-                    const int dc = i >> 1;
-                    if (i & 1) dpacc[qb] = mfma32(fb[i % PDA], vf[dc], dpacc[qb]);
-                    else sacc[qb] = mfma32(fb[i % PDA], kf[dc], sacc[qb]);
-                    // refill: continue into the next block's fragments
+                // fragments are consumed in pairs, the younger read first: one s_waitcnt serves two MFMAs
+                auto refill = [&](int i) {
                     const int nxt = i + PDA;
-                    if (nxt < NA) fb[i % PDA] = rd(qb, nxt);
+                    if (nxt < NA) fb[i % PDA] = rd(qb, nxt);          // ... and on into the next block's fragments
                     else if (qb == 0) fb[i % PDA] = rd(1, nxt - NA);
+                };
+                auto side = [&](int i) {
                     if (qb == 0) {
                         if (i <= 2 * NDQ) copy_slice(i);
                     } else {
                         if (NA == 16) elem(0, i);
                         else { elem(0, 2 * i); elem(0, 2 * i + 1); }
                     }
+                };
+#pragma unroll
+                for (int i = 0; i < NA; i += 2) {
+                    const int dc = i >> 1;
+                    dpacc[qb] = mfma32(fb[(i + 1) % PDA], vf[dc], dpacc[qb]);
+                    side(i);
+                    __builtin_amdgcn_sched_barrier(0);
+                    sacc[qb] = mfma32(fb[i % PDA], kf[dc], sacc[qb]);
+                    side(i + 1);
+                    refill(i);
+                    refill(i + 1);
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
@@ -404,18 +413,27 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
                         __builtin_amdgcn_sched_barrier(0);
                     }
                 }
-#pragma unroll
-                for (int i = 0; i < NB; ++i) {
-                    const int c = i / (2 * DB), db = (i >> 1) % DB;
-                    if (i & 1) dkacc[db] = mfma32(fb[i % PDB], dsf[qb][c], dkacc[db]);
-                    else dvacc[db] = mfma32(fb[i % PDB], pf[qb][c], dvacc[db]);
+                auto refill = [&](int i) {
                     const int nxt = i + PDB;
                     if (nxt < NB) fb[i % PDB] = rd(qb, nxt);
                     else if (qb == 0) fb[i % PDB] = rd(1, nxt - NB);
+                };
+                auto side = [&](int i) {
                     if (qb == 0) {
                         if (NB == 16) elem(1, i);
                         else { elem(1, 2 * i); elem(1, 2 * i + 1); }
                     }
+                };
+#pragma unroll
+                for (int i = 0; i < NB; i += 2) {
+                    const int c = i / (2 * DB), db = (i >> 1) % DB;
+                    dkacc[db] = mfma32(fb[(i + 1) % PDB], dsf[qb][c], dkacc[db]);
+                    side(i);
+                    __builtin_amdgcn_sched_barrier(0);
+                    dvacc[db] = mfma32(fb[i % PDB], pf[qb][c], dvacc[db]);
+                    side(i + 1);
+                    refill(i);
+                    refill(i + 1);
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }

@@ -277,26 +277,42 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void fwd_kernel(const Fwd
                 fb[i] = k_frag(t + 1, i);
                 __builtin_amdgcn_sched_barrier(0);
             }
+            // Fragments are consumed in pairs, the younger read of a pair first: LDS returns in order, so
+            // the wait for it also covers its partner and one s_waitcnt serves two MFMAs.  The two reads
+            // that refill the ring are issued together at the end of the pair.
+            auto frag_of = [&](int f) { return f < NS ? k_frag(t + 1, f) : v_frag(t, f - NS); };   // f in [0, NS + NP)
 #pragma unroll
-            for (int i = 0; i < NS; ++i) {
-                nxt[i & 1] = mfma32(fb[i % PD], qf[i >> 1], nxt[i & 1]);
-                if (i + PD < NS) fb[i % PD] = k_frag(t + 1, i + PD);
-                else fb[i % PD] = v_frag(t, i + PD - NS);          // run on into the V fragments
+            for (int i = 0; i < NS; i += 2) {
+                nxt[1] = mfma32(fb[(i + 1) % PD], qf[i >> 1], nxt[1]);
                 exp_slice(i);
+                __builtin_amdgcn_sched_barrier(0);
+                nxt[0] = mfma32(fb[i % PD], qf[i >> 1], nxt[0]);
+                exp_slice(i + 1);
+                fb[i % PD] = frag_of(i + PD);
+                fb[(i + 1) % PD] = frag_of(i + 1 + PD);
                 __builtin_amdgcn_sched_barrier(0);
             }
             l_run += rsum0 + rsum1;
             // ---- O^T += V(t)^T P(t)^T between the row-maximum scan of tile t+1
             float tmax = nxt[0][0];
-#pragma unroll
-            for (int i = 0; i < NP; ++i) {
-                oacc[i % DB] = mfma32(fb[i % PD], pf[i / DB], oacc[i % DB]);
-                if (i + PD < NP) fb[i % PD] = v_frag(t, i + PD);
-                constexpr int MPS = 32 / NP;
+            constexpr int MPS = 32 / NP;
+            auto max_slice = [&](int i) {
 #pragma unroll
                 for (int e = 0; e < MPS; e += 2) {
                     const int idx = MPS * i + e;
                     tmax = fmaxf(fmaxf(tmax, nxt[idx >> 4][idx & 15]), nxt[(idx + 1) >> 4][(idx + 1) & 15]);
+                }
+            };
+#pragma unroll
+            for (int i = 0; i < NP; i += 2) {
+                oacc[(i + 1) % DB] = mfma32(fb[(i + 1) % PD], pf[(i + 1) / DB], oacc[(i + 1) % DB]);
+                max_slice(i);
+                __builtin_amdgcn_sched_barrier(0);
+                oacc[i % DB] = mfma32(fb[i % PD], pf[i / DB], oacc[i % DB]);
+                max_slice(i + 1);
+                if (i + PD < NP) {
+                    fb[i % PD] = frag_of(NS + i + PD);
+                    fb[(i + 1) % PD] = frag_of(NS + i + 1 + PD);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }

@@ -468,21 +468,23 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sage_fwd_kernel(cons
                 fb[i] = k_frag(t + 1, i);
                 __builtin_amdgcn_sched_barrier(0);
             }
+            // fragments are consumed in pairs, the younger read of a pair first: one s_waitcnt serves two MFMAs
+            auto frag_of = [&](int f) { return f < NS ? k_frag(t + 1, f) : v_frag(t, f - NS); };   // f in [0, NS + NP)
 #pragma unroll
-            for (int i = 0; i < NS; ++i) {
-                s_mfma(i);
-                if (i + PD < NS) fb[i % PD] = k_frag(t + 1, i + PD);
-                else fb[i % PD] = v_frag(t, i + PD - NS);          // run on into the V fragments
+            for (int i = 0; i < NS; i += 2) {
+                s_mfma(i + 1);
                 exp_slice(i);
+                __builtin_amdgcn_sched_barrier(0);
+                s_mfma(i);
+                exp_slice(i + 1);
+                fb[i % PD] = frag_of(i + PD);
+                fb[(i + 1) % PD] = frag_of(i + 1 + PD);
                 __builtin_amdgcn_sched_barrier(0);
             }
             l_run += rsum0 + rsum1;
             // O^T += V(t)^T P(t)^T between the int32 -> float conversion and maximum scan of tile t+1
             float tmax = -INFINITY;
-#pragma unroll
-            for (int i = 0; i < NP; ++i) {
-                pv_mfma(i);
-                if (i + PD < NP) fb[i % PD] = v_frag(t, i + PD);
+            auto scan_slice = [&](int i) {
 #pragma unroll
                 for (int e = 0; e < MPS; e += 2) {
                     const int i0 = MPS * i + e, i1 = i0 + 1;
@@ -490,6 +492,18 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sage_fwd_kernel(cons
                     nxt[i0 >> 4][i0 & 15] = __float_as_int(a);
                     nxt[i1 >> 4][i1 & 15] = __float_as_int(c);
                     tmax = fmaxf(fmaxf(tmax, a), c);
+                }
+            };
+#pragma unroll
+            for (int i = 0; i < NP; i += 2) {
+                pv_mfma(i + 1);
+                scan_slice(i);
+                __builtin_amdgcn_sched_barrier(0);
+                pv_mfma(i);
+                scan_slice(i + 1);
+                if (i + PD < NP) {
+                    fb[i % PD] = frag_of(NS + i + PD);
+                    fb[(i + 1) % PD] = frag_of(NS + i + 1 + PD);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
