@@ -68,3 +68,41 @@ def test_random_case(oracle, seed):
     if kv_len is not None:                            # keys past the length receive exactly zero gradient
         for b in range(B):
             assert not bool(dk[b, :, int(kv_len[b]):].any()) and not bool(dv[b, :, int(kv_len[b]):].any())
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_case_many_heads(oracle, seed):
+    """Larger grids: enough workgroups that the kernels choose their 256-query workgroups and the dK/dV
+    kernel splits its last scheduling round; oracle parity on the first and last (batch, head)."""
+    from flame_amd import capi
+    rng = np.random.default_rng(7000 + seed)
+    D = int(rng.choice([64, 128]))
+    B, H = int(rng.integers(1, 3)), int(rng.choice([12, 20, 33, 40]))
+    Sq = int(rng.choice([512, 768, 1000, 1280, 1536]))
+    Sk = int(rng.choice([512, 777, 1024, 1408]))
+    mode = ["none", "causal", "kvlen", "none"][seed % 4]
+    if mode == "causal":
+        Sk = Sq
+    print(f"[random many heads] seed={seed} B={B} H={H} Sq={Sq} Sk={Sk} D={D} mode={mode}", flush=True)
+    q, k, v, do = (W.f32_to_bf16_bits(W.normal_f32(9000 + seed, s, B * H * n * D).reshape(B, H, n, D))
+                   for s, n in enumerate((Sq, Sk, Sk, Sq)))
+    scale = 1.0 / math.sqrt(D)
+    causal = mode == "causal"
+    kv_len = None
+    if mode == "kvlen":
+        kv_len = rng.integers(1, Sk + 1, size=B).astype(np.int32)
+    kvl = None if kv_len is None else torch.from_numpy(kv_len).cuda()
+    qd, kd, vd, dod = (to_dev(t) for t in (q, k, v, do))
+    o, lse = capi.attn_fwd(qd, kd, vd, scale, causal=causal, kv_len=kvl)
+    dq, dk, dv = capi.attn_bwd(qd, kd, vd, o, dod, lse, scale, causal=causal, kv_len=kvl)
+    torch.cuda.synchronize()
+    for hb in (0, B * H - 1):
+        heads = (hb, hb + 1)
+        ro, rlse, rof = oracle.sdpa_fwd(q, k, v, scale, causal=causal, kv_len=kv_len, heads=heads, want_f32=True)
+        sel = lambda t, S: to_f32(t).reshape(B * H, S, D)[hb:hb + 1]
+        assert_close_bf16(oracle, f"O[{hb}]", sel(o, Sq), ro.reshape(B * H, Sq, D)[hb:hb + 1], rof.reshape(B * H, Sq, D)[hb:hb + 1])
+        assert np.max(np.abs(lse.cpu().numpy().reshape(B * H, Sq)[hb] - rlse.reshape(B * H, Sq)[hb])) <= TOL_LSE
+        ref = oracle.sdpa_bwd(q, k, v, ro, do, scale, causal=causal, kv_len=kv_len, heads=heads, want_f32=True)
+        for i, (name, got, S) in enumerate((("dQ", dq, Sq), ("dK", dk, Sk), ("dV", dv, Sk))):
+            assert_close_bf16(oracle, f"{name}[{hb}]", sel(got, S), ref[i].reshape(B * H, S, D)[hb:hb + 1],
+                              ref[i + 3].reshape(B * H, S, D)[hb:hb + 1])
