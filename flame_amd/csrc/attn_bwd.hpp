@@ -326,6 +326,14 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
             }
         };
 
+        // slice s (of 16 per block) of the element-wise work: one logit register for D = 128, two for D = 64
+        constexpr int LAG = 2;
+        static_assert(2 * DC == 4 * DB, "both phases must have the same number of MFMA slots per block");
+        auto elem_slot = [&](int qb, int s) {
+            if (2 * DC == 16) elem(qb, s);
+            else { elem(qb, 2 * s); elem(qb, 2 * s + 1); }
+        };
+
         // copies of the next tile, one instruction at a time (full tiles: uniform base + lane offset)
         const bool next_full = COPY == 1 || (qt_next * BM + BM) <= p.Sq;
         const uint16_t* nq_base = qbase + (int64_t)qt_next * BM * p.qs.n;
@@ -353,11 +361,6 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
             };
 #pragma unroll
             for (int qb = 0; qb < 2; ++qb) {
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    sacc[qb][r] = 0.f;
-                    dpacc[qb][r] = 0.f;
-                }
                 if (qb == 0) {
 #pragma unroll
                     for (int i = 0; i < PDA; ++i) {
@@ -372,21 +375,24 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
                     if (nxt < NA) fb[i % PDA] = rd(qb, nxt);          // ... and on into the next block's fragments
                     else if (qb == 0) fb[i % PDA] = rd(1, nxt - NA);
                 };
+                // the element-wise work of block 0 trails the MFMAs that produced its S and dP by two MFMA
+                    // slots (hand-emitted MFMAs: see mfma32_vgpr), so its last two slices run in phase B
                 auto side = [&](int i) {
                     if (qb == 0) {
                         if (i <= 2 * NDQ) copy_slice(i);
-                    } else {
-                        if (NA == 16) elem(0, i);
-                        else { elem(0, 2 * i); elem(0, 2 * i + 1); }
+                    } else if (i >= LAG) {
+                        elem_slot(0, i - LAG);
                     }
                 };
 #pragma unroll
                 for (int i = 0; i < NA; i += 2) {
                     const int dc = i >> 1;
-                    dpacc[qb] = mfma32(fb[(i + 1) % PDA], vf[dc], dpacc[qb]);
+                    if (i == 0) mfma32_vgpr_first(dpacc[qb], fb[(i + 1) % PDA], vf[dc]);
+                    else mfma32_vgpr(dpacc[qb], fb[(i + 1) % PDA], vf[dc]);
                     side(i);
                     __builtin_amdgcn_sched_barrier(0);
-                    sacc[qb] = mfma32(fb[i % PDA], kf[dc], sacc[qb]);
+                    if (i == 0) mfma32_vgpr_first(sacc[qb], fb[i % PDA], kf[dc]);
+                    else mfma32_vgpr(sacc[qb], fb[i % PDA], kf[dc]);
                     side(i + 1);
                     refill(i);
                     refill(i + 1);
@@ -418,11 +424,9 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
                     if (nxt < NB) fb[i % PDB] = rd(qb, nxt);
                     else if (qb == 0) fb[i % PDB] = rd(1, nxt - NB);
                 };
-                auto side = [&](int i) {
-                    if (qb == 0) {
-                        if (NB == 16) elem(1, i);
-                        else { elem(1, 2 * i); elem(1, 2 * i + 1); }
-                    }
+                auto side = [&](int i) {           // slices that trail their MFMAs by LAG slots (see phase A)
+                    if (i < LAG) elem_slot(qb, NB - LAG + i);
+                    else if (qb == 0) elem_slot(1, i - LAG);
                 };
 #pragma unroll
                 for (int i = 0; i < NB; i += 2) {

@@ -34,6 +34,19 @@ __device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
 }
 
+// The same MFMA with the accumulator pinned to the architectural VGPRs, for kernels that also keep
+// long-lived accumulators in the accumulation registers: the compiler picks one MFMA form per function,
+// and with the accumulation form every value the vector ALU wants to read costs a v_accvgpr_read.
+// Emitted by hand, so the compiler's hazard bookkeeping does not see it.  The caller must keep at
+// least two other MFMAs between the last of these writing an accumulator and the first vector-ALU
+// instruction that touches it (the result of an 8-pass MFMA is visible 11 issue cycles after issue).
+__device__ __forceinline__ void mfma32_vgpr_first(f32x16& acc, bf16x8 a, bf16x8 b) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(acc) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void mfma32_vgpr(f32x16& acc, bf16x8 a, bf16x8 b) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
+}
+
 // row index inside a 32x32 accumulator block for register r of a lane in half h
 __device__ __forceinline__ constexpr int acc_row(int r, int h) { return 8 * (r >> 2) + 4 * h + (r & 3); }
 
