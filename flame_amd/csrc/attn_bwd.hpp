@@ -5,22 +5,23 @@
 //            with the logits transposed (lane = query): S^T = K Q^T, dP^T = V dO^T,
 //            dS^T = P^T (dP^T - delta) and dQ^T += K^T dS^T accumulated in fp32 registers for the whole
 //            walk, dS^T going into the last MFMA straight from the accumulators.  Runs first and also
-//            leaves delta_i = sum_d dO_id * O_id and LSE_i * log2(e) (fp32, one value per query row)
+//            leaves -delta_i = -sum_d dO_id * O_id and LSE_i * log2(e) (fp32, one value per query row)
 //            in the workspace for the next kernel.
 //   dkdv     one workgroup owns 128 keys (32 per wavefront) of one (batch, head) and walks over the
 //            query tiles (64 rows): S = Q K^T, dP = dO V^T, P = exp2(S*c - LSE*log2e),
 //            dS = P * (dP - delta); dV^T += dO^T P and dK^T += Q^T dS stay in fp32 registers for the
-//            whole walk (P and dS are used as MFMA operands straight from the accumulators).  When the
+//            whole walk (P and dS are used as MFMA operands straight from the accumulators), and so do
+//            the wavefront's K and V fragments (in the accumulation registers).  When the
 //            key blocks do not fill the last scheduling round, the blocks of that round are split
 //            along the walk and their fp32 partial sums are combined by the merge kernel.
 // Accumulating dQ from the dkdv walk with fp32 atomics was measured at about one lane-atomic per
 // clock per CU, more than the whole MFMA time of the backward; recomputing S and dP in a second,
 // query-major kernel costs 2 extra GEMMs out of 7 and no atomics, no fp32 scratch and no convert pass.
 //
-// Q and dO tiles are copied global -> LDS by asynchronous LDS-DMA loads, double buffered, row-major
-// with an XOR swizzle of the 16-byte granules; their transposed MFMA operands (Q^T, dO^T) and the dS
-// operand come from transposing LDS reads, so no tile is stored twice and no access pattern has
-// bank conflicts.  One workgroup barrier per step.
+// Tiles are copied global -> LDS by asynchronous LDS-DMA loads (K / V tiles of dq double buffered,
+// Q / dO tiles of dkdv in three stages), row-major with an XOR swizzle of the 16-byte granules; their
+// transposed MFMA operands (Q^T, dO^T) and the dS operand come from transposing LDS reads, so no tile
+// is stored twice and no access pattern has bank conflicts.  One workgroup barrier per step.
 #pragma once
 #include <type_traits>
 
@@ -45,7 +46,7 @@ struct BwdParams {
     uint16_t* dq;
     uint16_t* dk;
     uint16_t* dv;
-    float* delta;         // workspace, [B*H, Sq]
+    float* ndelta;        // workspace, [B*H, Sq]: -rowsum(dO * O)
     float* lse2;          // workspace, [B*H, Sq]: LSE * log2(e), +inf where LSE = -inf
     Strides qs, ks, vs, os, dos, dqs, dks, dvs;
     int B, H, Sq, Sk;
@@ -62,9 +63,10 @@ struct BwdTile {
     static constexpr int RS = D;                    // LDS row stride of the Q / dO / K / V tiles (swizzled, unpadded)
     static constexpr int Q_ELEMS = BM * RS;
     static constexpr int STAGE_ELEMS = 2 * Q_ELEMS;               // Q tile + dO tile (also one 128-row tile)
-    static constexpr int ROW_FLOATS = 2 * BM;                     // lse2 + delta of one step
-    // [2 stages of Q,dO][2 x (lse2, delta)]
-    static constexpr int LDS_BYTES = 2 * STAGE_ELEMS * 2 + 2 * ROW_FLOATS * 4;
+    static constexpr int ROW_FLOATS = 2 * BM;                     // lse2 and -delta of one step
+    static constexpr int NSTAGE = 3;
+    // [3 stages of Q,dO][3 x (lse2, -delta)]
+    static constexpr int LDS_BYTES = NSTAGE * STAGE_ELEMS * 2 + NSTAGE * ROW_FLOATS * 4;
     static constexpr int ROWS_PER_DMA = 1024 / (D * 2);
     static constexpr int DMA_PER_WAVE = BM / ROWS_PER_DMA / 4;    // 1 KiB copies per wave and tensor
 };
@@ -83,8 +85,8 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
     constexpr int RPD = T::ROWS_PER_DMA, NDQ = T::DMA_PER_WAVE;
 
     extern __shared__ __attribute__((aligned(1024))) uint16_t lds[];
-    uint16_t* stage0 = lds;                                        // [2][Q tile | dO tile]
-    float* rows0 = reinterpret_cast<float*>(lds + 2 * T::STAGE_ELEMS);   // [2][lse2 | delta]
+    uint16_t* stage0 = lds;                                        // [3][Q tile | dO tile]
+    float* rows0 = reinterpret_cast<float*>(lds + T::NSTAGE * T::STAGE_ELEMS);   // [3][lse2 | -delta]
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -114,7 +116,7 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
     const uint16_t* vbase = p.v + b * p.vs.b + hh * p.vs.h;
     const uint16_t* dobase = p.dout + b * p.dos.b + hh * p.dos.h;
     const float* lsebase = p.lse2 + (int64_t)bh * p.Sq;
-    const float* deltabase = p.delta + (int64_t)bh * p.Sq;
+    const float* ndeltabase = p.ndelta + (int64_t)bh * p.Sq;
 
     int klimit = p.Sk;
     if (p.m.kv_len) klimit = min(klimit, max(p.m.kv_len[b], 0));
@@ -164,7 +166,7 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
 
     const int dma_row_in = lane / GPR, dma_gran = lane % GPR;
     const uint32_t lds0 = lds_addr(lds);
-    const uint32_t rows_lds0 = lds0 + 2u * 2u * T::STAGE_ELEMS;   // byte address of rows0
+    const uint32_t rows_lds0 = lds0 + 2u * T::NSTAGE * T::STAGE_ELEMS;   // byte address of rows0
 
     // ---- prologue: the K and V fragments of this wavefront's 32 keys are held in registers for the whole walk
     bf16x8 kf[DC], vf[DC];
@@ -189,7 +191,7 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
         __syncthreads();
     }
 
-    // ---- asynchronous staging of the 64-row Q / dO tiles and their lse2 / delta rows.
+    // ---- asynchronous staging of the 64-row Q / dO tiles and their lse2 / -delta rows, three stages.
     //      Address = uniform tile base + a per-lane 32-bit offset that never changes.
     uint32_t q_lane_off[NDQ], do_lane_off[NDQ];     // bytes
 #pragma unroll
@@ -199,21 +201,21 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
         q_lane_off[i] = 2u * (uint32_t)(row * (int)p.qs.n + c * 8);
         do_lane_off[i] = 2u * (uint32_t)(row * (int)p.dos.n + c * 8);
     }
-    auto q_dst = [&](int buf, int which, int i) {    // LDS byte address of copy i of this wave (which: 0 = Q, 1 = dO)
-        return lds0 + 2u * (uint32_t)(buf * T::STAGE_ELEMS + which * T::Q_ELEMS + (wave * NDQ + i) * 512);
+    auto q_dst = [&](int stg, int which, int i) {    // LDS byte address of copy i of this wave (which: 0 = Q, 1 = dO)
+        return lds0 + 2u * (uint32_t)(stg * T::STAGE_ELEMS + which * T::Q_ELEMS + (wave * NDQ + i) * 512);
     };
-    auto rows_dst = [&](int buf) { return rows_lds0 + 4u * (uint32_t)(buf * T::ROW_FLOATS + wave * BM); };
-    auto issue_q_tile = [&](int qt, int buf) {
+    auto rows_dst = [&](int stg) { return rows_lds0 + 4u * (uint32_t)(stg * T::ROW_FLOATS + wave * BM); };
+    auto issue_q_tile = [&](int qt, int stg) {
         const int q0 = qt * BM;
         if (q0 + BM <= p.Sq) {
             const uint16_t* qt_base = qbase + (int64_t)q0 * p.qs.n;
             const uint16_t* dot_base = dobase + (int64_t)q0 * p.dos.n;
 #pragma unroll
             for (int i = 0; i < NDQ; ++i) {
-                dma16u(qt_base, q_lane_off[i], q_dst(buf, 0, i));
-                dma16u(dot_base, do_lane_off[i], q_dst(buf, 1, i));
+                dma16u(qt_base, q_lane_off[i], q_dst(stg, 0, i));
+                dma16u(dot_base, do_lane_off[i], q_dst(stg, 1, i));
             }
-            if (wave < 2) dma4((wave == 0 ? lsebase : deltabase) + q0 + lane, rows_dst(buf));
+            if (wave < 2) dma4((wave == 0 ? lsebase : ndeltabase) + q0 + lane, rows_dst(stg));
         } else {   // last, partial tile: rows past the end re-read the last valid row
 #pragma unroll
             for (int i = 0; i < NDQ; ++i) {
@@ -221,12 +223,12 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
                 const int row = ji * RPD + dma_row_in;
                 const int qi = min(q0 + row, p.Sq - 1);
                 const int c = dma_gran ^ swz<D>(row);
-                dma16(qbase + (int64_t)qi * p.qs.n + c * 8, q_dst(buf, 0, i));
-                dma16(dobase + (int64_t)qi * p.dos.n + c * 8, q_dst(buf, 1, i));
+                dma16(qbase + (int64_t)qi * p.qs.n + c * 8, q_dst(stg, 0, i));
+                dma16(dobase + (int64_t)qi * p.dos.n + c * 8, q_dst(stg, 1, i));
             }
             if (wave < 2) {
                 const int qi = min(q0 + lane, p.Sq - 1);
-                dma4((wave == 0 ? lsebase : deltabase) + qi, rows_dst(buf));
+                dma4((wave == 0 ? lsebase : ndeltabase) + qi, rows_dst(stg));
             }
         }
     };
@@ -245,6 +247,7 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
 
     unsigned long long ph[6] = {0, 0, 0, 0, 0, 0};
     unsigned long long tprev = TIMING ? __builtin_readcyclecounter() : 0ull;
+    const unsigned long long wall0 = TIMING ? wall_clock64() : 0ull;
 #define FATTN_PHASE(i)                                                  \
     if (TIMING) {                                                       \
         const unsigned long long tnow = __builtin_readcyclecounter();   \
@@ -252,60 +255,113 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
         tprev = tnow;                                                   \
     }
 
+    // One step of the walk handles one 64-query tile as two 32-query blocks in four phases of NS MFMAs:
+    //   A0: S,dP(block 0)          | issue of the next tile's copies
+    //   A1: S,dP(block 1)          | P,dS(block 0)
+    //   B0: dV,dK += (block 0)     | P,dS(block 1)
+    //   B1: dV,dK += (block 1)
+    // written as an explicit software pipeline for a single wavefront per SIMD: the MFMA pipe and the
+    // vector ALU run side by side only when their instructions alternate in the instruction stream, so
+    // the per-element arithmetic of one block is threaded between the MFMAs of its neighbour, one
+    // accumulator register per MFMA.  The G = 4 NS operand fragments of a step come from LDS through one
+    // ring of PD registers that runs PD fragments ahead of the MFMAs, across the phases and on into the
+    // next step; the scheduling barriers keep the compiler from undoing either interleave.
+    //
+    // Three LDS stages, one workgroup barrier per step, placed just before the ring first reads the next
+    // stage: by then every wave's copies of the next tile have landed, and every wave has finished the
+    // previous step, whose stage the next step's copies overwrite.  No wave ever drains its pipeline.
+    //
+    // dP accumulates on top of -delta (loaded from LDS straight into the accumulator registers), so
+    // dS = P * dP' needs no subtraction.
+    constexpr int NS = 2 * DC;      // MFMAs per phase
+    constexpr int G = 4 * NS;       // MFMAs = operand fragments per step
+    constexpr int PD = 4;           // read-ahead depth of the fragment ring
+    static_assert(2 * DC == 4 * DB, "all phases must have the same number of MFMA slots");
+    static_assert(NS % PD == 0 && 4 * (2 * NDQ) + 1 < G - PD, "ring depth / copy slices do not fit");
+    f32x16 dpacc[2];
+    bf16x8 fb[PD];
+    // fragment g of a step: [0, 2 NS) 16-byte row reads (block, dc, Q | dO); [2 NS, 4 NS) transposing
+    // reads (block, 16-query chunk, db, dO^T | Q^T)
+    auto frag = [&](const uint16_t* Qs, int g) {
+        const uint16_t* dOs = Qs + T::Q_ELEMS;
+        const int qb = (g / NS) & 1, i = g % NS;
+        if (g < 2 * NS) {
+            const int dc = i >> 1;
+            return *reinterpret_cast<const bf16x8*>(((i & 1) ? dOs : Qs) + roff[dc] + 32 * qb * RS);
+        }
+        const int c = i / (2 * DB), db = (i >> 1) % DB, cc = 2 * qb + c;
+        return tr_frag((i & 1) ? Qs : dOs, toff[0][db] + 16 * cc * RS, toff[1][db] + 16 * cc * RS);
+    };
+    // -delta of queries 8*g4 + 4h .. +3 of block qb -> the dP accumulator registers of those rows
+    auto ndelta_rows = [&](const float* rows, int qb, int g4) {
+        const f32x4 v = *reinterpret_cast<const f32x4*>(rows + BM + 32 * qb + 8 * g4 + 4 * h);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) dpacc[qb][4 * g4 + t] = v[t];
+    };
+
     // this workgroup's slice [it_lo, it_hi) of the walk
     const int it_lo = (int)((int64_t)part * n_it / nparts);
     const int it_hi = (int)((int64_t)(part + 1) * n_it / nparts);
-    if (it_hi > it_lo) issue_q_tile(tile_of(it_lo), it_lo & 1);
-    wait_vm0();
-    __syncthreads();
+    // The stages are numbered so that the steps which need exclusions (they come first and take their
+    // stage from a run-time counter) leave the counter at 0 for the main loop, whose three unrolled
+    // steps have their stages fixed at compile time.
+    const int n_masked_here = max(min(n_masked, it_hi) - it_lo, 0);
+    int st = (3 - n_masked_here % 3) % 3;        // LDS stage of the step about to run
+    if (it_hi > it_lo) {
+        issue_q_tile(tile_of(it_lo), st);
+        wait_vm0();
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < PD; ++i) fb[i] = frag(stage0 + st * T::STAGE_ELEMS, i);
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) ndelta_rows(rows0 + st * T::ROW_FLOATS, 0, g4);
+    }
 
-    // One step of the walk, written as an explicit software pipeline for a single wavefront per SIMD:
-    // the MFMA pipe and the vector ALU run side by side only when their instructions alternate in the
-    // instruction stream, so the per-element softmax / dS arithmetic of one 32-query block is
-    // threaded between the MFMAs of the neighbouring block, one accumulator register per MFMA:
-    //   A0: S,dP(block 0)                      | issue of the next tile's copies
-    //   A1: S,dP(block 1)                      | P,dS(block 0)
-    //   B0: dV,dK += (block 0)                 | P,dS(block 1)
-    //   B1: dV,dK += (block 1)
-    // LDS reads run PD fragments ahead of the MFMAs that consume them; the scheduling barriers keep the
-    // compiler from undoing either interleave.
     // COPY: 0 = this is the last step, 1 = the next tile is a full one (straight-line copies),
     //       2 = decide at run time (used by the few steps that need exclusions)
-    // BUF: stage that holds this step's tile (0 / 1), or -1 to take it from the parity of `it`.
-    auto step = [&](auto masked_tag, auto copy_tag, auto buf_tag, int it, int qt, int qt_next) {
+    // STAGE: LDS stage that holds this step's tile (0 / 1 / 2), or -1 to take it from `st`.
+    auto step = [&](auto masked_tag, auto copy_tag, auto stage_tag, int st, int it, int qt, int qt_next,
+                    const uint16_t* nq_base, const uint16_t* ndo_base, const float* nrow_base) {
         constexpr bool MASKED = decltype(masked_tag)::value;
         constexpr int COPY = decltype(copy_tag)::value;
-        constexpr int BUF = decltype(buf_tag)::value;
-        static_assert((2 * DC) % 4 == 0 && (4 * DB) % 4 == 0, "read-ahead depth must divide the fragment count");
-        const int buf = BUF >= 0 ? BUF : (it & 1);
+        constexpr int STAGE = decltype(stage_tag)::value;
+        const int cur = STAGE >= 0 ? STAGE : st;
+        const int nxt = STAGE >= 0 ? (STAGE + 1) % 3 : (st == 2 ? 0 : st + 1);
         const int q0 = qt * BM;
         const bool have_next = COPY == 1 || (COPY == 2 && it + 1 < it_hi);
 
-        const uint16_t* Qs = stage0 + buf * T::STAGE_ELEMS;
-        const uint16_t* dOs = Qs + T::Q_ELEMS;
-        const float* lse_s = rows0 + buf * T::ROW_FLOATS;
-        const float* delta_s = lse_s + BM;
+        const uint16_t* Qs = stage0 + cur * T::STAGE_ELEMS;
+        const uint16_t* Qn = stage0 + nxt * T::STAGE_ELEMS;
+        const float* rows_c = rows0 + cur * T::ROW_FLOATS;      // [lse2 | -delta] of this step's queries
+        const float* rows_n = rows0 + nxt * T::ROW_FLOATS;
 
-        f32x16 sacc[2], dpacc[2];
+        f32x16 sacc[2];
         bf16x8 pf[2][2], dsf[2][2];
-        f32x4 l4, d4, l4n, d4n;
-        // the per-query rows are read one group of four queries ahead of their use, so that waiting
-        // for them never drains the fragment reads that were issued in between
-        auto rows_ahead = [&](int qb, int g) {
-            l4n = *reinterpret_cast<const f32x4*>(lse_s + 32 * qb + 8 * g + 4 * h);
-            d4n = *reinterpret_cast<const f32x4*>(delta_s + 32 * qb + 8 * g + 4 * h);
-        };
+        f32x4 l4, l4n;
+        // lse2 is read one group of four queries ahead of its use, so that waiting for it never drains
+        // the fragment reads that were issued in between
+        auto rows_ahead = [&](int qb, int g) { l4n = *reinterpret_cast<const f32x4*>(rows_c + 32 * qb + 8 * g + 4 * h); };
 
-        // element r of block qb: P = exp2(S*c - lse2), dS = P*(dP - delta); pack after 8 and 16
+        // element r of block qb: P = exp2(S*c - lse2), dS = P*(dP - delta); pack after 8 and 16.
+        // The product for element r is issued with the exponential of element r + 1, so that no
+        // instruction waits on the transcendental unit.
+        auto ds_mul = [&](int qb, int r) {
+            dpacc[qb][r] = sacc[qb][r] * dpacc[qb][r];
+            if ((r & 7) == 7) {
+                const int c = r >> 3, o8 = 8 * c;
+                const f32x16& d = dpacc[qb];
+                dsf[qb][c] = pack8(d[o8], d[o8 + 1], d[o8 + 2], d[o8 + 3], d[o8 + 4], d[o8 + 5], d[o8 + 6], d[o8 + 7]);
+            }
+        };
         auto elem = [&](int qb, int r) {
             const int g = r >> 2, t = r & 3;
             if (t == 0) {
                 l4 = l4n;
-                d4 = d4n;
                 if (g < 3) rows_ahead(qb, g + 1);
                 else if (qb == 0) rows_ahead(1, 0);
             }
             float pr = exp2_fast(fmaf(sacc[qb][r], c_log2, -l4[t]));
+            if (r > 0) ds_mul(qb, r - 1);
             if (MASKED) {
                 const int qi = q0 + 32 * qb + 8 * g + 4 * h + t;
                 bool drop = key >= klimit || qi >= p.Sq;
@@ -316,165 +372,164 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
                 pr = drop ? 0.f : pr;
             }
             sacc[qb][r] = pr;
-            dpacc[qb][r] = pr * (dpacc[qb][r] - d4[t]);
             if ((r & 7) == 7) {
                 const int c = r >> 3, o8 = 8 * c;
                 const f32x16& s = sacc[qb];
-                const f32x16& d = dpacc[qb];
                 pf[qb][c] = pack8(s[o8], s[o8 + 1], s[o8 + 2], s[o8 + 3], s[o8 + 4], s[o8 + 5], s[o8 + 6], s[o8 + 7]);
-                dsf[qb][c] = pack8(d[o8], d[o8 + 1], d[o8 + 2], d[o8 + 3], d[o8 + 4], d[o8 + 5], d[o8 + 6], d[o8 + 7]);
             }
         };
-
-        // slice s (of 16 per block) of the element-wise work: one logit register for D = 128, two for D = 64
-        constexpr int LAG = 2;
-        static_assert(2 * DC == 4 * DB, "both phases must have the same number of MFMA slots per block");
+        // slice s (of NS per block) of the element-wise work: one logit register for D = 128, two for D = 64;
+        // slice NS is the last product
         auto elem_slot = [&](int qb, int s) {
-            if (2 * DC == 16) elem(qb, s);
+            if (s == NS) ds_mul(qb, 15);
+            else if (NS == 16) elem(qb, s);
             else { elem(qb, 2 * s); elem(qb, 2 * s + 1); }
         };
 
-        // copies of the next tile, one instruction at a time (full tiles: uniform base + lane offset)
+        // copies of the next tile, one instruction at a time (full tiles: uniform base + lane offset), each
+        // in two halves around an MFMA: destination into M0, then the copy.  nq_base / ndo_base / nrow_base
+        // are the wave-uniform addresses of the next tile's Q rows, dO rows and lse2 (even waves) or
+        // -delta (odd waves) rows; waves 2 and 3 repeat the row copies of waves 0 and 1.
         const bool next_full = COPY == 1 || (qt_next * BM + BM) <= p.Sq;
-        const uint16_t* nq_base = qbase + (int64_t)qt_next * BM * p.qs.n;
-        const uint16_t* ndo_base = dobase + (int64_t)qt_next * BM * p.dos.n;
-        auto copy_slice = [&](int j) {     // j in [0, 2*NDQ]
-            if (COPY == 0) return;
-            if (COPY == 2 && (!have_next || !next_full)) return;
-            if (j < 2 * NDQ) {
-                const int i = j >> 1;
-                if (j & 1) dma16u(ndo_base, do_lane_off[i], q_dst(buf ^ 1, 1, i));
-                else dma16u(nq_base, q_lane_off[i], q_dst(buf ^ 1, 0, i));
-            } else if (wave < 2) {
-                dma4((wave == 0 ? lsebase : deltabase) + qt_next * BM + lane, rows_dst(buf ^ 1));
+        const bool copying = COPY == 1 || (COPY == 2 && have_next && next_full);
+        auto copy_dst_of = [&](int j) {
+            return j < 2 * NDQ ? q_dst(nxt, j & 1, j >> 1) : rows_lds0 + 4u * (uint32_t)(nxt * T::ROW_FLOATS + (wave & 1) * BM);
+        };
+        // Copy j goes with MFMA slot 4j + 1.  In straight-line steps, while that MFMA is a hand-emitted one
+        // (phases A0 and A1), the copy is split around it.
+        auto copy_dst = [&](int g) {
+            const int j = g / 4;
+            if (COPY == 1 && g % 4 == 1 && j <= 2 * NDQ && g < 2 * NS) dma_set_dst(copy_dst_of(j));
+        };
+        auto copy_issue = [&](int g) {
+            const int j = g / 4;
+            if (COPY == 0 || g % 4 != 1 || j > 2 * NDQ) return;
+            if (COPY == 1 && g < 2 * NS) {
+                if (j == 2 * NDQ) dma4u_issue(nrow_base, 4u * (uint32_t)lane);
+                else if (j & 1) dma16u_issue(ndo_base, do_lane_off[j >> 1]);
+                else dma16u_issue(nq_base, q_lane_off[j >> 1]);
+            } else if (copying) {          // destination and copy in one piece
+                if (j == 2 * NDQ) dma4(nrow_base + lane, copy_dst_of(j));
+                else if (j & 1) dma16u(ndo_base, do_lane_off[j >> 1], copy_dst_of(j));
+                else dma16u(nq_base, q_lane_off[j >> 1], copy_dst_of(j));
             }
         };
-        if (COPY == 2 && have_next && !next_full) issue_q_tile(qt_next, buf ^ 1);   // partial tile: slow path, all at once
+        if (COPY == 2 && have_next && !next_full) issue_q_tile(qt_next, nxt);   // partial tile: slow path, all at once
 
-        // ---- phase A: S = Q K^T and dP = dO V^T, rows = queries of block qb, columns = this wave's keys
-        constexpr int NA = 2 * DC, PDA = 4;      // fragments per block: (dc, Q|dO); PDA divides NA
-        {
-            bf16x8 fb[PDA];
-            auto rd = [&](int qb, int i) {
-                const int dc = i >> 1;
-                return *reinterpret_cast<const bf16x8*>(((i & 1) ? dOs : Qs) + roff[dc] + 32 * qb * RS);
-            };
-#pragma unroll
-            for (int qb = 0; qb < 2; ++qb) {
-                if (qb == 0) {
-#pragma unroll
-                    for (int i = 0; i < PDA; ++i) {
-                        fb[i] = rd(0, i);
-                        __builtin_amdgcn_sched_barrier(0);
-                    }
-                    rows_ahead(0, 0);
-                }
-                // fragments are consumed in pairs, the younger read first: one s_waitcnt serves two MFMAs
-                auto refill = [&](int i) {
-                    const int nxt = i + PDA;
-                    if (nxt < NA) fb[i % PDA] = rd(qb, nxt);          // ... and on into the next block's fragments
-                    else if (qb == 0) fb[i % PDA] = rd(1, nxt - NA);
-                };
-                // the element-wise work of block 0 trails the MFMAs that produced its S and dP by two MFMA
-                    // slots (hand-emitted MFMAs: see mfma32_vgpr), so its last two slices run in phase B
-                auto side = [&](int i) {
-                    if (qb == 0) {
-                        if (i <= 2 * NDQ) copy_slice(i);
-                    } else if (i >= LAG) {
-                        elem_slot(0, i - LAG);
-                    }
-                };
-#pragma unroll
-                for (int i = 0; i < NA; i += 2) {
-                    const int dc = i >> 1;
-                    if (i == 0) mfma32_vgpr_first(dpacc[qb], fb[(i + 1) % PDA], vf[dc]);
-                    else mfma32_vgpr(dpacc[qb], fb[(i + 1) % PDA], vf[dc]);
-                    side(i);
-                    __builtin_amdgcn_sched_barrier(0);
-                    if (i == 0) mfma32_vgpr_first(sacc[qb], fb[i % PDA], kf[dc]);
-                    else mfma32_vgpr(sacc[qb], fb[i % PDA], kf[dc]);
-                    side(i + 1);
-                    refill(i);
-                    refill(i + 1);
-                    __builtin_amdgcn_sched_barrier(0);
-                }
+        // The element-wise work of a block trails the hand-emitted MFMAs that produced its S and dP by
+        // LAG MFMA slots (see mfma32_vgpr), so its last LAG slices run at the start of the phase after.
+        constexpr int LAG = 2;
+        auto side = [&](int g) {
+            const int phase = g / NS, i = g % NS;
+            copy_issue(g);
+            if (phase == 0) {
+                if (i >= NS - 4) ndelta_rows(rows_c, 1, i - (NS - 4));
+                if (i == NS - 1) rows_ahead(0, 0);
+            } else if (phase == 1) {
+                if (i >= LAG) elem_slot(0, i - LAG);
+            } else if (phase == 2) {
+                if (i <= LAG) elem_slot(0, NS - LAG + i);
+                if (i >= LAG) elem_slot(1, i - LAG);
+            } else {
+                if (i <= LAG) elem_slot(1, NS - LAG + i);
             }
-        }
-        FATTN_PHASE(0)
+        };
+        auto refill = [&](int g) {
+            const int ng = g + PD;
+            if (ng < G) fb[g % PD] = frag(Qs, ng);
+            else if (COPY == 1 || (COPY == 2 && have_next)) fb[g % PD] = frag(Qn, ng - G);
+        };
 
-        // ---- phase B: dV^T += dO^T P, dK^T += Q^T dS, rows = d, columns = keys, contraction over queries
-        constexpr int NB = 4 * DB, PDB = 4;      // fragments per block: (16-query chunk, db, dO^T|Q^T); PDB divides NB
-        {
-            bf16x8 fb[PDB];
-            auto rd = [&](int qb, int i) {
-                const int c = i / (2 * DB), db = (i >> 1) % DB, cc = 2 * qb + c;
-                return tr_frag((i & 1) ? Qs : dOs, toff[0][db] + 16 * cc * RS, toff[1][db] + 16 * cc * RS);
-            };
+        // fragments are consumed in pairs, the younger read first: one s_waitcnt serves two MFMAs
+        auto run_phase = [&](auto phase_tag) {
+            constexpr int PHASE = decltype(phase_tag)::value;
 #pragma unroll
-            for (int qb = 0; qb < 2; ++qb) {
-                if (qb == 0) {
-#pragma unroll
-                    for (int i = 0; i < PDB; ++i) {
-                        fb[i] = rd(0, i);
+            for (int i = 0; i < NS; i += 2) {
+                const int g = PHASE * NS + i;
+                if constexpr (PHASE < 2) {      // S = Q K^T and dP = dO V^T - delta, rows = queries of block qb, columns = this wave's keys
+                    const int qb = PHASE, dc = i >> 1;
+                    mfma32_vgpr_bacc(dpacc[qb], fb[(g + 1) % PD], vf[dc]);
+                    side(g);
+                    __builtin_amdgcn_sched_barrier(0);
+                    copy_dst(g + 1);
+                    if (i == 0) mfma32_vgpr_first_bacc(sacc[qb], fb[g % PD], kf[dc]);
+                    else mfma32_vgpr_bacc(sacc[qb], fb[g % PD], kf[dc]);
+                    side(g + 1);
+                } else {              // dV^T += dO^T P, dK^T += Q^T dS: rows = d, columns = keys, contraction over queries
+                    const int qb = PHASE - 2, c = i / (2 * DB), db = (i >> 1) % DB;
+                    dkacc[db] = mfma32(fb[(g + 1) % PD], dsf[qb][c], dkacc[db]);
+                    side(g);
+                    __builtin_amdgcn_sched_barrier(0);
+                    dvacc[db] = mfma32(fb[g % PD], pf[qb][c], dvacc[db]);
+                    side(g + 1);
+                }
+                if (g == G - PD && COPY != 0) {
+                    if (COPY == 1 || have_next) {
                         __builtin_amdgcn_sched_barrier(0);
+                        FATTN_PHASE(3)
+                        wait_vm0();                          // this wave's copies of the next tile have landed
+                        __builtin_amdgcn_s_barrier();        // ... everyone's have, and everyone is past the previous step
+                        FATTN_PHASE(4)
+                        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                        for (int g4 = 0; g4 < 4; ++g4) ndelta_rows(rows_n, 0, g4);
                     }
                 }
-                auto refill = [&](int i) {
-                    const int nxt = i + PDB;
-                    if (nxt < NB) fb[i % PDB] = rd(qb, nxt);
-                    else if (qb == 0) fb[i % PDB] = rd(1, nxt - NB);
-                };
-                auto side = [&](int i) {           // slices that trail their MFMAs by LAG slots (see phase A)
-                    if (i < LAG) elem_slot(qb, NB - LAG + i);
-                    else if (qb == 0) elem_slot(1, i - LAG);
-                };
-#pragma unroll
-                for (int i = 0; i < NB; i += 2) {
-                    const int c = i / (2 * DB), db = (i >> 1) % DB;
-                    dkacc[db] = mfma32(fb[(i + 1) % PDB], dsf[qb][c], dkacc[db]);
-                    side(i);
-                    __builtin_amdgcn_sched_barrier(0);
-                    dvacc[db] = mfma32(fb[i % PDB], pf[qb][c], dvacc[db]);
-                    side(i + 1);
-                    refill(i);
-                    refill(i + 1);
-                    __builtin_amdgcn_sched_barrier(0);
-                }
+                refill(g);
+                refill(g + 1);
+                __builtin_amdgcn_sched_barrier(0);
             }
-        }
-        FATTN_PHASE(2)
-        wait_vm0();        // the other stage has landed
-        FATTN_PHASE(3)
-        __syncthreads();   // ... for every wave, and every wave is done reading this step's stage
-        FATTN_PHASE(4)
+            if (PHASE < 3) { FATTN_PHASE(PHASE) }
+        };
+        run_phase(std::integral_constant<int, 0>{});
+        run_phase(std::integral_constant<int, 1>{});
+        run_phase(std::integral_constant<int, 2>{});
+        run_phase(std::integral_constant<int, 3>{});
     };
 
     using IM = std::integral_constant<int, -1>;
     using I0 = std::integral_constant<int, 0>;
     using I1 = std::integral_constant<int, 1>;
     using I2 = std::integral_constant<int, 2>;
-    for (int it = it_lo; it < min(n_masked, it_hi); ++it)
-        step(std::true_type{}, I2{}, IM{}, it, tile_of(it), it + 1 < it_hi ? tile_of(it + 1) : 0);
-    // every tile after the first n_masked is a full, fully attended one, and they are consecutive
+    const int64_t q_tile_stride = (int64_t)BM * p.qs.n, do_tile_stride = (int64_t)BM * p.dos.n;
+    const float* rowbase = (wave & 1) ? ndeltabase : lsebase;
+    for (int it = it_lo; it < n_masked_here + it_lo; ++it) {
+        const int qn = it + 1 < it_hi ? tile_of(it + 1) : 0;
+        step(std::true_type{}, I2{}, IM{}, st, it, tile_of(it), qn, qbase + qn * q_tile_stride, dobase + qn * do_tile_stride,
+             rowbase + qn * BM);
+        st = st == 2 ? 0 : st + 1;
+    }
+    // every tile after the first n_masked is a full, fully attended one, and they are consecutive;
+    // the stage counter is 0 here
     {
         int it = max(n_masked, it_lo);
         int qt = lead_end + (it - n_masked);
-        if ((it & 1) && it < it_hi - 1) {
-            step(std::false_type{}, I1{}, I1{}, it, qt, qt + 1);
-            ++it, ++qt;
+        const uint16_t* nq = qbase + (qt + 1) * q_tile_stride;     // the tile after the current one
+        const uint16_t* ndo = dobase + (qt + 1) * do_tile_stride;
+        const float* nrow = rowbase + (qt + 1) * BM;
+        auto advance = [&]() {
+            nq += q_tile_stride;
+            ndo += do_tile_stride;
+            nrow += BM;
+        };
+        for (; it + 3 <= it_hi - 1; it += 3, qt += 3) {
+            step(std::false_type{}, I1{}, I0{}, 0, it, qt, qt + 1, nq, ndo, nrow);
+            advance();
+            step(std::false_type{}, I1{}, I1{}, 1, it + 1, qt + 1, qt + 2, nq, ndo, nrow);
+            advance();
+            step(std::false_type{}, I1{}, I2{}, 2, it + 2, qt + 2, qt + 3, nq, ndo, nrow);
+            advance();
         }
-        for (; it + 1 < it_hi - 1; it += 2, qt += 2) {
-            step(std::false_type{}, I1{}, I0{}, it, qt, qt + 1);
-            step(std::false_type{}, I1{}, I1{}, it + 1, qt + 1, qt + 2);
+        for (; it < it_hi - 1; ++it, ++qt) {
+            step(std::false_type{}, I1{}, IM{}, st, it, qt, qt + 1, nq, ndo, nrow);
+            advance();
+            st = st == 2 ? 0 : st + 1;
         }
-        if (it < it_hi - 1) {
-            step(std::false_type{}, I1{}, IM{}, it, qt, qt + 1);
-            ++it, ++qt;
-        }
-        if (it < it_hi) step(std::false_type{}, I0{}, IM{}, it, qt, qt);
+        if (it < it_hi) step(std::false_type{}, I0{}, IM{}, st, it, qt, qt, nq, ndo, nrow);
     }
 
     if (TIMING && p.phase_cycles && tid == 0) {
+        ph[5] = wall_clock64() - wall0;      // 100 MHz
 #pragma unroll
         for (int i = 0; i < 6; ++i) p.phase_cycles[(size_t)blockIdx.x * 6 + i] = ph[i];
     }
@@ -649,7 +704,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void bwd_dq_kernel(const 
             lse2 = (l == -INFINITY) ? INFINITY : l * kLog2e;
             delta = part;
             if (h == 0) {
-                p.delta[(int64_t)bh * p.Sq + qrow] = delta;
+                p.ndelta[(int64_t)bh * p.Sq + qrow] = -delta;
                 p.lse2[(int64_t)bh * p.Sq + qrow] = lse2;
             }
         }

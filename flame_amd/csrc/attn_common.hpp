@@ -46,6 +46,14 @@ __device__ __forceinline__ void mfma32_vgpr_first(f32x16& acc, bf16x8 a, bf16x8 
 __device__ __forceinline__ void mfma32_vgpr(f32x16& acc, bf16x8 a, bf16x8 b) {
     asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
 }
+// The same two with the B operand held in the accumulation registers: operands that live for a whole
+// kernel (a workgroup's own K / V fragments) then cost no architectural VGPRs.
+__device__ __forceinline__ void mfma32_vgpr_first_bacc(f32x16& acc, bf16x8 a, bf16x8 b) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(acc) : "v"(a), "a"(b));
+}
+__device__ __forceinline__ void mfma32_vgpr_bacc(f32x16& acc, bf16x8 a, bf16x8 b) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "a"(b));
+}
 
 // row index inside a 32x32 accumulator block for register r of a lane in half h
 __device__ __forceinline__ constexpr int acc_row(int r, int h) { return 8 * (r >> 2) + 4 * h + (r & 3); }
@@ -112,15 +120,27 @@ __device__ __forceinline__ uint32_t lds_addr(const void* p) {
 }
 // destination given as a wave-uniform LDS byte address
 __device__ __forceinline__ void dma16(const void* gsrc, uint32_t lds_byte_addr) {
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(lds_byte_addr), "v"(gsrc) : "m0", "memory");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(lds_byte_addr), "v"(gsrc) : "m0", "memory");
 }
 __device__ __forceinline__ void dma4(const void* gsrc, uint32_t lds_byte_addr) {
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, off" :: "s"(lds_byte_addr), "v"(gsrc) : "m0", "memory");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" :: "s"(lds_byte_addr), "v"(gsrc) : "m0", "memory");
 }
 // ... and the source split into a wave-uniform base and a non-negative per-lane byte offset
 __device__ __forceinline__ void dma16u(const void* gbase_wave_uniform, uint32_t lane_byte_off, uint32_t lds_byte_addr) {
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2"
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                  :: "s"(lds_byte_addr), "v"(lane_byte_off), "s"(gbase_wave_uniform) : "m0", "memory");
+}
+// The same copies in two halves, for software pipelines that place another instruction (an MFMA)
+// between them instead of the s_nop: writing M0 and reading it in an LDS-DMA need one wait state.
+// Nothing that writes M0 may come between the two halves.
+__device__ __forceinline__ void dma_set_dst(uint32_t lds_byte_addr) {
+    asm volatile("s_mov_b32 m0, %0" :: "s"(lds_byte_addr) : "m0");
+}
+__device__ __forceinline__ void dma16u_issue(const void* gbase_wave_uniform, uint32_t lane_byte_off) {
+    asm volatile("global_load_lds_dwordx4 %0, %1" :: "v"(lane_byte_off), "s"(gbase_wave_uniform) : "memory");
+}
+__device__ __forceinline__ void dma4u_issue(const void* gbase_wave_uniform, uint32_t lane_byte_off) {
+    asm volatile("global_load_lds_dword %0, %1" :: "v"(lane_byte_off), "s"(gbase_wave_uniform) : "memory");
 }
 // destination given as a pointer into LDS (wave-uniform)
 __device__ __forceinline__ void dma16(const void* gsrc, void* lds_dst) { dma16(gsrc, lds_addr(lds_dst)); }

@@ -124,7 +124,7 @@ int device_cu_count() {
     return cus;
 }
 
-// backward workspace: [delta rows][lse2 rows][fp32 partials of the split dK/dV workgroups]
+// backward workspace: [-delta rows][lse2 rows][fp32 partials of the split dK/dV workgroups]
 size_t bwd_rows_bytes(int B, int H, int N_q) { return 2 * align_up((size_t)B * H * N_q * sizeof(float), 256); }
 size_t bwd_split_slot_bytes(int D) { return (size_t)2 * 128 * D * sizeof(float); }   // dK^T and dV^T of one 128-key block
 
@@ -157,7 +157,7 @@ int launch_bwd(const BwdParams& p, hipStream_t s) {
     const int64_t n_qt = wide ? n256 : (p.Sq + TQ::BM - 1) / TQ::BM;
     const int64_t grid_dq = n_qt * p.B * p.H;
     if (grid > 0x7fffffff || grid_dq > 0x7fffffff) return FLAME_ATTN_ERR_UNSUPPORTED;
-    // dQ first: besides dQ it leaves delta = rowsum(dO * O) and the rescaled LSE of every query row in the
+    // dQ first: besides dQ it leaves -delta = -rowsum(dO * O) and the rescaled LSE of every query row in the
     // workspace, which the dK/dV kernel stages per query tile.
     {
         ScopedKernelTimer t(FLAME_ATTN_KERNEL_BWD_DQ, s);
@@ -280,7 +280,7 @@ int flame_attn_bwd_bf16(const void* Q, const void* K, const void* V, const void*
     p.dk = static_cast<uint16_t*>(dK) + dk_off;
     p.dv = static_cast<uint16_t*>(dV) + dv_off;
     const size_t rows = (size_t)B * H * N_q;
-    p.delta = static_cast<float*>(workspace);
+    p.ndelta = static_cast<float*>(workspace);
     p.lse2 = reinterpret_cast<float*>(static_cast<char*>(workspace) + align_up(rows * sizeof(float), 256));
     p.split_ws = reinterpret_cast<float*>(static_cast<char*>(workspace) + bwd_rows_bytes(B, H, N_q));
     p.split_ws_bytes = workspace_bytes - bwd_rows_bytes(B, H, N_q);

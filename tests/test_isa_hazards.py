@@ -1,9 +1,12 @@
-"""Static check of the one hazard the compiler cannot see.
+"""Static checks of the hazards the compiler cannot see, on the library compiled to assembly.
 
-The dK/dV kernel emits its S / dP MFMAs by hand (accumulators pinned to the architectural VGPRs), so
-the compiler's hazard recogniser does not insert the wait states an 8-pass MFMA needs before the
-vector ALU may touch its result.  The kernel is structured so that at least two further MFMAs are
-issued first; this test compiles the library to assembly and verifies that for every such MFMA."""
+1. The dK/dV kernel emits its S / dP MFMAs by hand (accumulators pinned to the architectural VGPRs),
+   so the compiler's hazard recogniser does not insert the wait states an 8-pass MFMA needs before
+   anything else may touch its result.  The kernel is structured so that at least two further MFMAs
+   are issued first.
+2. The LDS-DMA copies are emitted by hand as well and take their LDS destination from M0: every one of
+   them must find, in its own basic block, an s_mov_b32 to M0 with at least one instruction in between
+   (the wait state between a scalar write of M0 and an LDS-DMA that reads it)."""
 import os
 import re
 import shutil
@@ -25,14 +28,19 @@ def _regs(tok):
     return {int(m.group(1))} if m else set()
 
 
-@pytest.mark.skipif(shutil.which(fb.HIPCC) is None and not os.path.exists(fb.HIPCC), reason="hipcc not available")
-def test_hand_emitted_mfma_results_are_not_touched_too_early():
+@pytest.fixture(scope="module")
+def text():
+    if shutil.which(fb.HIPCC) is None and not os.path.exists(fb.HIPCC):
+        pytest.skip("hipcc not available")
     with tempfile.TemporaryDirectory() as tmp:
         out = os.path.join(tmp, "flame_attn.s")
         flags = [f for f in fb.FLAGS if f not in ("-shared", "-fPIC")]
         subprocess.run([fb.HIPCC, *flags, "-S", "--cuda-device-only", SRC, "-o", out], check=True,
                        stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
-        text = open(out).read()
+        return open(out).read()
+
+
+def test_hand_emitted_mfma_results_are_not_touched_too_early(text):
     kernels = re.findall(r"^(_ZN5fattn15bwd_dkdv_kernel\w+):.*?\.end_amdhsa_kernel", text, re.S | re.M)
     assert len(kernels) >= 4
     checked = 0
@@ -54,10 +62,38 @@ def test_hand_emitted_mfma_results_are_not_touched_too_early():
                     if later_mfma >= 2:
                         break
                     continue
-                if l2.startswith("s_") or l2.startswith("ds_read") or l2.startswith("global_load_lds"):
-                    continue                        # scalar, or vector registers used as addresses / LDS destinations only
+                if l2.startswith("s_") or l2.startswith("global_load_lds"):
+                    continue                        # scalar, or vector registers used as addresses only
+                toks = re.findall(r"v\[\d+:\d+\]|v\d+", l2)
+                if l2.startswith("ds_read"):
+                    toks = toks[:1]                 # the destination; the other register is an address
                 used = set()
-                for t in re.findall(r"v\[\d+:\d+\]|v\d+", l2):
+                for t in toks:
                     used |= _regs(t)
                 assert not (used & dst), f"{name}: `{l2}` touches the result of `{l}` before two more MFMAs"
     assert checked >= 4 * 96
+
+
+def test_every_lds_dma_finds_its_destination_in_m0(text):
+    kernels = re.findall(r"^(_ZN5fattn\w+):.*?\.end_amdhsa_kernel", text, re.S | re.M)
+    assert kernels
+    checked = 0
+    for name in kernels:
+        body = re.search(r"^%s:.*?\.end_amdhsa_kernel" % re.escape(name), text, re.S | re.M).group(0)
+        # instructions and labels, in order
+        ins = [l.strip() for l in body.split("\n") if re.match(r"^\s+[a-z]", l) or re.match(r"^\.LBB\S+:", l)]
+        for idx, l in enumerate(ins):
+            if not l.startswith("global_load_lds"):
+                continue
+            checked += 1
+            between = 0
+            for l2 in reversed(ins[:idx]):
+                assert not l2.startswith(".LBB"), f"{name}: `{l}` has no M0 write in its basic block"
+                if re.match(r"s_mov_b32\s+m0,", l2):
+                    break
+                assert "m0" not in l2.split(";")[0], f"{name}: `{l2}` uses M0 between its write and `{l}`"
+                between += 1
+            else:
+                raise AssertionError(f"{name}: `{l}` has no M0 write before it")
+            assert between >= 1, f"{name}: `{l}` follows its M0 write without a wait state"
+    assert checked >= 100
