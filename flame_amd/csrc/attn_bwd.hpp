@@ -915,4 +915,369 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void bwd_dq_kernel(const 
     }
 }
 
+// ---------------------------------------------------------------------------- dq, 256-query workgroups
+// The same computation as bwd_dq_kernel for workgroups of 256 queries, laid out for one wavefront per
+// SIMD: 4 wavefronts of 64 queries (two 32-query blocks) each.  Every K / V fragment read from LDS then
+// feeds two MFMAs (one per query block), which halves the LDS reads and waits per MFMA; the register
+// file of a lone wavefront holds dQ^T of both blocks and the Q / dO fragments in the accumulation
+// registers (Q / dO as MFMA B operands), and S^T / dP^T in architectural registers through hand-emitted
+// MFMAs (see mfma32_vgpr).  dP^T starts from -delta, so dS^T = P^T * dP'^T is one multiply.
+// Three LDS stages of K / V tiles, one barrier per tile, one ring of fragment reads that runs on into
+// the next tile, copies split around MFMAs and spread over the tile: as in bwd_dkdv_kernel.
+// No explicit keep-mask variant: such problems use bwd_dq_kernel.
+template <int D>
+struct BwdDqWideTile {
+    static constexpr int BM = 256;                  // query rows per workgroup (64 per wavefront)
+    static constexpr int BN = 64;                   // keys per tile
+    static constexpr int RS = D;
+    static constexpr int TILE_ELEMS = BN * D;
+    static constexpr int STAGE_ELEMS = 2 * TILE_ELEMS;            // K tile + V tile
+    static constexpr int NSTAGE = 3;
+    static constexpr int LDS_BYTES = NSTAGE * STAGE_ELEMS * 2;
+    static constexpr int ROWS_PER_DMA = 1024 / (D * 2);
+    static constexpr int DMA_PER_WAVE = BN / ROWS_PER_DMA / 4;    // 1 KiB copies per wave and tensor
+};
+
+template <int D>
+__global__ __launch_bounds__(256) void bwd_dq_wide_kernel(const BwdParams p) {
+    using T = BwdDqWideTile<D>;
+    constexpr int BM = T::BM, BN = T::BN, RS = T::RS;
+    constexpr int DC = D / 16;
+    constexpr int DB = D / 32;
+    constexpr int GPR = D / 8;
+    constexpr int NDMA = T::DMA_PER_WAVE;
+
+    extern __shared__ __attribute__((aligned(1024))) uint16_t lds[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 31, h = lane >> 5;
+
+    const int n_qt = (p.Sq + BM - 1) / BM;
+    const int wg = xcd_remap(blockIdx.x, gridDim.x);
+    const int qt = wg % n_qt;
+    const int bh = wg / n_qt;
+    const int b = bh / p.H, hh = bh % p.H;
+    const int q0 = qt * BM;
+    const int qw0 = q0 + wave * 64;
+
+    const uint16_t* qbase = p.q + b * p.qs.b + hh * p.qs.h;
+    const uint16_t* kbase = p.k + b * p.ks.b + hh * p.ks.h;
+    const uint16_t* vbase = p.v + b * p.vs.b + hh * p.vs.h;
+    const uint16_t* dobase = p.dout + b * p.dos.b + hh * p.dos.h;
+
+    int klimit = p.Sk;
+    if (p.m.kv_len) klimit = min(klimit, max(p.m.kv_len[b], 0));
+    int kend = klimit;
+    if (p.m.causal) kend = min(kend, q0 + BM);
+    const int n_tiles = (kend + BN - 1) / BN;
+
+    // ---- Q and dO fragments (B operands: column = query, 8 consecutive d) and the per-query scalars of
+    //      both query blocks; -delta and lse2 are also left in the workspace for the dK/dV kernel
+    bf16x8 qf[2][DC], dof[2][DC];          // pinned to accumulation registers: slots qb*DC + dc and 16 + qb*DC + dc
+    float lse2[2];
+    f32x16 ndelta16[2];
+    int qrow[2];
+    static_for<2>([&](auto qb_tag) {
+        constexpr int qb = decltype(qb_tag)::value;
+        qrow[qb] = qw0 + 32 * qb + n;
+        const bool qok = qrow[qb] < p.Sq;
+        const uint16_t* rq = qbase + (int64_t)qrow[qb] * p.qs.n + 8 * h;
+        const uint16_t* rd = dobase + (int64_t)qrow[qb] * p.dos.n + 8 * h;
+        const uint16_t* ro = p.o + b * p.os.b + hh * p.os.h + (int64_t)qrow[qb] * p.os.n + 8 * h;
+        float part = 0.f;
+        static_for<DC>([&](auto dc_tag) {
+            constexpr int dc = decltype(dc_tag)::value;
+            qf[qb][dc] = pin_b_fragment<qb * DC + dc>(ldg16(rq + 16 * dc, qok));
+            const u32x4 dv = ldg16(rd + 16 * dc, qok);
+            dof[qb][dc] = pin_b_fragment<16 + qb * DC + dc>(dv);
+            const u32x4 ov = ldg16(ro + 16 * dc, qok);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) part += bf16_lo(dv[i]) * bf16_lo(ov[i]) + bf16_hi(dv[i]) * bf16_hi(ov[i]);
+        });
+        part += xhalf(part);
+        lse2[qb] = INFINITY;
+        float nd = 0.f;
+        if (qok) {
+            const float l = p.lse[(int64_t)bh * p.Sq + qrow[qb]];
+            lse2[qb] = (l == -INFINITY) ? INFINITY : l * kLog2e;
+            nd = -part;
+            if (h == 0) {
+                p.ndelta[(int64_t)bh * p.Sq + qrow[qb]] = nd;
+                p.lse2[(int64_t)bh * p.Sq + qrow[qb]] = lse2[qb];
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) ndelta16[qb][r] = nd;
+    });
+
+    // ---- asynchronous staging of the K / V tiles
+    const int dma_row_in = lane / GPR, dma_gran = lane % GPR;
+    const uint32_t lds0 = lds_addr(lds);
+    uint32_t k_lane_off[NDMA], v_lane_off[NDMA];     // bytes
+#pragma unroll
+    for (int i = 0; i < NDMA; ++i) {
+        const int row = (wave * NDMA + i) * T::ROWS_PER_DMA + dma_row_in;
+        const int c = dma_gran ^ swz<D>(row);
+        k_lane_off[i] = 2u * (uint32_t)(row * (int)p.ks.n + c * 8);
+        v_lane_off[i] = 2u * (uint32_t)(row * (int)p.vs.n + c * 8);
+    }
+    auto dst_of = [&](int stg, int which, int i) {    // LDS byte address of copy i of this wave (which: 0 = K, 1 = V)
+        return lds0 + 2u * (uint32_t)(stg * T::STAGE_ELEMS + which * T::TILE_ELEMS + (wave * NDMA + i) * 512);
+    };
+    auto issue_tile = [&](int t, int stg) {          // any tile: rows past the attended range re-read the last attended key
+#pragma unroll
+        for (int i = 0; i < NDMA; ++i) {
+            const int row = (wave * NDMA + i) * T::ROWS_PER_DMA + dma_row_in;
+            const int key = max(min(t * BN + row, klimit - 1), 0);
+            const int c = dma_gran ^ swz<D>(row);
+            dma16(kbase + (int64_t)key * p.ks.n + c * 8, dst_of(stg, 0, i));
+            dma16(vbase + (int64_t)key * p.vs.n + c * 8, dst_of(stg, 1, i));
+        }
+    };
+
+    int koff[DC];          // 16-byte row reads of K / V: row 32*kb + n, logical granule 2*dc + h
+#pragma unroll
+    for (int dc = 0; dc < DC; ++dc) koff[dc] = n * RS + (((2 * dc + h) ^ swz<D>(n)) << 3);
+    const int tr_r = lane & 15, tr_g16 = (lane >> 4) & 1;
+    int toff[2][DB];       // transposing reads of K: rows 4h + r/4 (+8), logical granule 4*db + 2*g16 + (r&3)/2
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+        const int row = 4 * h + (tr_r >> 2) + 8 * half;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+            toff[half][db] = row * RS + (((4 * db + 2 * tr_g16 + ((tr_r & 3) >> 1)) ^ swz<D>(row)) << 3) + 4 * (tr_r & 1);
+    }
+
+    const float c_log2 = p.scale * kLog2e;
+    f32x16 dqacc[2][DB];      // dQ^T: rows = d, column = this lane's query of block qb
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) dqacc[qb][db][r] = 0.f;
+
+    // Operand fragments of a tile, in consumption order; each feeds two MFMAs (query blocks 0 and 1):
+    //   [0, DC) K rows of key block 0 (S), [DC, 2DC) V rows of block 0 (dP), then the same for block 1,
+    //   [4DC, 4DC + 2DB) K^T of key block 0 by (16-key chunk, db) (dQ), then of block 1
+    constexpr int NROW = 4 * DC, NF = NROW + 4 * DB;
+    constexpr int PD = 4;                            // read-ahead depth of the fragment ring
+    static_assert(DC % PD == 0 && (2 * DB) % PD == 0, "read-ahead depth must divide the fragment counts");
+    auto fetch = [&](const uint16_t* ks, int f) {
+        const uint16_t* vs = ks + T::TILE_ELEMS;
+        if (f < NROW) {
+            const int phase = f / DC, dc = f % DC;            // phase: 0 S(0), 1 dP(0), 2 S(1), 3 dP(1)
+            return *reinterpret_cast<const bf16x8*>(((phase & 1) ? vs : ks) + koff[dc] + 32 * (phase >> 1) * RS);
+        }
+        const int g = f - NROW, cc = g / DB, db = g % DB;      // cc = 16-key chunk of the tile
+        const u32x2 lo = lds_read_tr16(ks + toff[0][db] + 16 * cc * RS);
+        const u32x2 hi = lds_read_tr16(ks + toff[1][db] + 16 * cc * RS);
+        const u32x4 u = {lo[0], lo[1], hi[0], hi[1]};
+        return __builtin_bit_cast(bf16x8, u);
+    };
+    bf16x8 fb[PD];
+    if (n_tiles > 0) {
+        issue_tile(0, 0);
+        wait_vm0();
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < PD; ++i) fb[i] = fetch(lds, i);
+    }
+
+    // One tile of 64 keys = two key blocks of 32, six phases of 2 DC MFMAs (MFMA slot = 2 * fragment +
+    // query block).  The element-wise work of a phase is threaded between the MFMAs of the next one:
+    //   S(0) | dP(0) + P(0) | S(1) + dS(0) | dP(1) + P(1) | dQ(0) + dS(1) | dQ(1)
+    // Element e of query block 0 goes with slot e of its phase, that of query block 1 with slot e + 1
+    // (its S / dP are complete one MFMA later), the sixteenth spilling into the first slot of the
+    // next phase: every hand-emitted MFMA result is first touched two MFMAs after it was issued.
+    // COPY: 1 = the next tile is a full one (copies split around the MFMAs), 2 = decide at run time.
+    // STAGE: LDS stage that holds this tile (0 / 1 / 2), or -1 to take it from st.
+    auto tile_step = [&](auto masked_tag, auto copy_tag, auto stage_tag, int st, int t, const uint16_t* nk_base,
+                         const uint16_t* nv_base) {
+        constexpr bool MASKED = decltype(masked_tag)::value;
+        constexpr int COPY = decltype(copy_tag)::value;
+        constexpr int STAGE = decltype(stage_tag)::value;
+        const int cur = STAGE >= 0 ? STAGE : st;
+        const int nxt = STAGE >= 0 ? (STAGE + 1) % 3 : (st == 2 ? 0 : st + 1);
+        const bool have_next = COPY == 1 || t + 1 < n_tiles;
+        if (COPY == 2 && have_next) issue_tile(t + 1, nxt);
+        const uint16_t* ks = lds + cur * T::STAGE_ELEMS;
+        const uint16_t* kn = lds + nxt * T::STAGE_ELEMS;
+        const int key0 = t * BN;
+
+        f32x16 sacc[2][2], dpacc[2][2];             // [query block][key block]
+        u32x4 dsw[2][2][2];                         // dS^T operands: [query block][key block][16-key chunk]
+
+        auto p_elem = [&](int qb, int kb, int r) {  // P^T: one query per lane, so LSE is a per-lane scalar
+            float pr = exp2_fast(fmaf(sacc[qb][kb][r], c_log2, -lse2[qb]));
+            if (MASKED) {
+                const int key = key0 + 32 * kb + acc_row(r, h);
+                bool drop = key >= klimit;
+                if (p.m.causal) drop = drop || key > qrow[qb];
+                pr = drop ? 0.f : pr;
+            }
+            sacc[qb][kb][r] = pr;
+        };
+        auto ds_elem = [&](int qb, int kb, int r) { // dS^T = P^T * (dP^T - delta), packed in pairs
+            f32x16& d = dpacc[qb][kb];
+            d[r] = sacc[qb][kb][r] * d[r];
+            if (r & 1) dsw[qb][kb][r >> 3][(r & 7) >> 1] = pack_bf16(d[r - 1], d[r]);
+        };
+        // element-wise work that goes with MFMA slot i of phase ph
+        constexpr int NSL = 2 * DC;                 // MFMA slots per phase
+        static_assert(NSL == 16 || NSL == 8, "element schedule written for 16 or 8 slots per phase");
+        auto elems_of = [&](int ph, int i, auto fn) {      // fn(qb, e) for the elements scheduled at (ph, i)
+            // query block 0: elements [EL*i, EL*(i+1)) at slot i; query block 1: one slot later
+            constexpr int EL = 16 / NSL;            // 1 or 2 elements per slot and block
+#pragma unroll
+            for (int e = 0; e < EL; ++e) fn(0, EL * i + e);
+            if (i > 0) {
+#pragma unroll
+                for (int e = 0; e < EL; ++e) fn(1, EL * (i - 1) + e);
+            }
+        };
+        auto spill_of = [&](auto fn) {               // the last elements of query block 1, in slot 0 of the next phase
+            constexpr int EL = 16 / NSL;
+#pragma unroll
+            for (int e = 0; e < EL; ++e) fn(1, EL * (NSL - 1) + e);
+        };
+        // copies of the next tile: copy j goes with MFMA slot CS * j + 1 of the S / dP phases
+        constexpr int NCOPY = 2 * NDMA;
+        constexpr int CS = (4 * NSL - 2) / NCOPY;
+        static_assert(CS >= 2, "copies do not fit the S / dP phases");
+        auto copy_dst = [&](int g) {
+            const int j = (g - 1) / CS;
+            if (COPY == 1 && g >= 1 && (g - 1) % CS == 0 && j < NCOPY) dma_set_dst(dst_of(nxt, j & 1, j >> 1));
+        };
+        auto copy_issue = [&](int g) {
+            const int j = (g - 1) / CS;
+            if (COPY == 1 && g >= 1 && (g - 1) % CS == 0 && j < NCOPY) {
+                if (j & 1) dma16u_issue(nv_base, v_lane_off[j >> 1]);
+                else dma16u_issue(nk_base, k_lane_off[j >> 1]);
+            }
+        };
+        auto refill = [&](int f) {
+            const int nf = f + PD;
+            if (nf < NF) fb[f % PD] = fetch(ks, nf);
+            else if (have_next) fb[f % PD] = fetch(kn, nf - NF);
+        };
+        auto side = [&](int ph, int i) {
+            if (ph == 1) elems_of(ph, i, [&](int qb, int e) { p_elem(qb, 0, e); });
+            if (ph == 2) {
+                if (i == 0) spill_of([&](int qb, int e) { p_elem(qb, 0, e); });
+                elems_of(ph, i, [&](int qb, int e) { ds_elem(qb, 0, e); });
+            }
+            if (ph == 3) {
+                if (i == 0) spill_of([&](int qb, int e) { ds_elem(qb, 0, e); });
+                elems_of(ph, i, [&](int qb, int e) { p_elem(qb, 1, e); });
+            }
+            if (ph == 4) {
+                if (i == 0) spill_of([&](int qb, int e) { p_elem(qb, 1, e); });
+                elems_of(ph, i, [&](int qb, int e) { ds_elem(qb, 1, e); });
+            }
+            if (ph == 5 && i == 0) spill_of([&](int qb, int e) { ds_elem(qb, 1, e); });
+        };
+
+        auto row_phase = [&](auto phase_tag) {      // S^T(kb) = K Q^T or dP^T(kb) = V dO^T - delta
+            constexpr int PH = decltype(phase_tag)::value, KB = PH >> 1;
+            static_for<DC>([&](auto dc_tag) {
+                constexpr int dc = decltype(dc_tag)::value;
+                constexpr int f = PH * DC + dc;
+                static_for<2>([&](auto qb_tag) {
+                    constexpr int qb = decltype(qb_tag)::value;
+                    constexpr int i = 2 * dc + qb, g = PH * NSL + i;
+                    constexpr int SLOT = ((PH & 1) ? 16 : 0) + qb * DC + dc;      // Q fragments first, then dO
+                    copy_dst(g);
+                    if constexpr (PH & 1)
+                        mfma32_vgpr_bpinned<SLOT, dc == 0 ? 2 : 1>(dpacc[qb][KB], fb[f % PD], dof[qb][dc], ndelta16[qb]);
+                    else
+                        mfma32_vgpr_bpinned<SLOT, dc == 0 ? 0 : 1>(sacc[qb][KB], fb[f % PD], qf[qb][dc], ndelta16[qb]);
+                    __builtin_amdgcn_sched_barrier(0);      // the element-wise work below must not move above this MFMA
+                    copy_issue(g);
+                    side(PH, i);
+                    if (qb == 1) refill(f);
+                    __builtin_amdgcn_sched_barrier(0);
+                });
+            });
+        };
+        auto dq_phase = [&](auto kb_tag) {          // dQ^T += K^T(kb) dS^T(kb)
+            constexpr int KB = decltype(kb_tag)::value;
+#pragma unroll
+            for (int g = 0; g < 2 * DB; ++g) {
+                const int f = NROW + 2 * DB * KB + g, c = g / DB, db = g % DB;
+#pragma unroll
+                for (int qb = 0; qb < 2; ++qb) {
+                    dqacc[qb][db] = mfma32(fb[f % PD], __builtin_bit_cast(bf16x8, dsw[qb][KB][c]), dqacc[qb][db]);
+                    __builtin_amdgcn_sched_barrier(0);
+                    side(4 + KB, 2 * g + qb);
+                    if (qb == 1) {
+                        if (f == NF - PD && have_next) {
+                            __builtin_amdgcn_sched_barrier(0);
+                            wait_vm0();                          // this wave's copies of the next tile have landed
+                            __builtin_amdgcn_s_barrier();        // ... everyone's have, and everyone is past the previous tile
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
+                        refill(f);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        };
+        row_phase(std::integral_constant<int, 0>{});
+        row_phase(std::integral_constant<int, 1>{});
+        row_phase(std::integral_constant<int, 2>{});
+        row_phase(std::integral_constant<int, 3>{});
+        dq_phase(std::integral_constant<int, 0>{});
+        dq_phase(std::integral_constant<int, 1>{});
+    };
+
+    int n_full = klimit / BN;
+    if (p.m.causal) n_full = min(n_full, (q0 + 1) / BN);
+    n_full = min(n_full, n_tiles);
+    using IM = std::integral_constant<int, -1>;
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    using I2 = std::integral_constant<int, 2>;
+    {
+        const int64_t k_tile_stride = (int64_t)BN * p.ks.n, v_tile_stride = (int64_t)BN * p.vs.n;
+        const uint16_t* nk = kbase + k_tile_stride;      // the tile after the current one
+        const uint16_t* nv = vbase + v_tile_stride;
+        int t = 0, st = 0;
+        for (; t + 3 < n_full; t += 3) {      // tiles t+1 .. t+3 are full: straight-line copies, fixed stages
+            tile_step(std::false_type{}, I1{}, I0{}, 0, t, nk, nv);
+            nk += k_tile_stride, nv += v_tile_stride;
+            tile_step(std::false_type{}, I1{}, I1{}, 1, t + 1, nk, nv);
+            nk += k_tile_stride, nv += v_tile_stride;
+            tile_step(std::false_type{}, I1{}, I2{}, 2, t + 2, nk, nv);
+            nk += k_tile_stride, nv += v_tile_stride;
+        }
+        for (; t < n_full; ++t) {
+            tile_step(std::false_type{}, I2{}, IM{}, st, t, nk, nv);
+            st = st == 2 ? 0 : st + 1;
+        }
+        for (; t < n_tiles; ++t) {
+            tile_step(std::true_type{}, I2{}, IM{}, st, t, nk, nv);
+            st = st == 2 ? 0 : st + 1;
+        }
+    }
+
+    // ---- epilogue: dQ = scale * dQ^T, bf16
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb)
+        if (qrow[qb] < p.Sq) {
+            uint16_t* dqrow = p.dq + b * p.dqs.b + hh * p.dqs.h + (int64_t)qrow[qb] * p.dqs.n;
+            const float s = p.scale;
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const f32x16& a = dqacc[qb][db];
+                    u32x2 w = {pack_bf16(a[4 * g] * s, a[4 * g + 1] * s), pack_bf16(a[4 * g + 2] * s, a[4 * g + 3] * s)};
+                    *reinterpret_cast<u32x2*>(dqrow + 32 * db + 8 * g + 4 * h) = w;
+                }
+        }
+}
+
 }  // namespace fattn

@@ -1,6 +1,8 @@
 // Shared device helpers for the gfx950 (CDNA4) attention kernels: 64-lane wavefronts,
 // v_mfma_f32_32x32x16_bf16 fragments, bf16 packing.  Compiled for gfx950 only.
 #pragma once
+#include <type_traits>
+#include <utility>
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -53,6 +55,108 @@ __device__ __forceinline__ void mfma32_vgpr_first_bacc(f32x16& acc, bf16x8 a, bf
 }
 __device__ __forceinline__ void mfma32_vgpr_bacc(f32x16& acc, bf16x8 a, bf16x8 b) {
     asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "a"(b));
+}
+// The same three with the B operand pinned to accumulation registers a[128 + 4 SLOT : 131 + 4 SLOT], for a
+// kernel whose 32 resident B fragments must stay put there (left to itself the register allocator
+// homes some of them in architectural registers and copies them over before every use).
+// MODE 0: acc = a b; 1: acc += a b; 2: acc = c + a b.
+template <int SLOT, int MODE>
+__device__ __forceinline__ void mfma32_vgpr_bpinned(f32x16& acc, bf16x8 a, bf16x8 b, const f32x16& c) {
+    static_assert(SLOT >= 0 && SLOT < 32, "32 pinned fragments");
+#define FATTN_PIN(I, R)                                                                                                  \
+    if constexpr (SLOT == I) {                                                                                           \
+        if constexpr (MODE == 0) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(acc) : "v"(a), R(b));     \
+        if constexpr (MODE == 1) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), R(b));     \
+        if constexpr (MODE == 2) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %3" : "=&v"(acc) : "v"(a), R(b), "v"(c)); \
+    }
+    FATTN_PIN(0, "{a[128:131]}")
+    FATTN_PIN(1, "{a[132:135]}")
+    FATTN_PIN(2, "{a[136:139]}")
+    FATTN_PIN(3, "{a[140:143]}")
+    FATTN_PIN(4, "{a[144:147]}")
+    FATTN_PIN(5, "{a[148:151]}")
+    FATTN_PIN(6, "{a[152:155]}")
+    FATTN_PIN(7, "{a[156:159]}")
+    FATTN_PIN(8, "{a[160:163]}")
+    FATTN_PIN(9, "{a[164:167]}")
+    FATTN_PIN(10, "{a[168:171]}")
+    FATTN_PIN(11, "{a[172:175]}")
+    FATTN_PIN(12, "{a[176:179]}")
+    FATTN_PIN(13, "{a[180:183]}")
+    FATTN_PIN(14, "{a[184:187]}")
+    FATTN_PIN(15, "{a[188:191]}")
+    FATTN_PIN(16, "{a[192:195]}")
+    FATTN_PIN(17, "{a[196:199]}")
+    FATTN_PIN(18, "{a[200:203]}")
+    FATTN_PIN(19, "{a[204:207]}")
+    FATTN_PIN(20, "{a[208:211]}")
+    FATTN_PIN(21, "{a[212:215]}")
+    FATTN_PIN(22, "{a[216:219]}")
+    FATTN_PIN(23, "{a[220:223]}")
+    FATTN_PIN(24, "{a[224:227]}")
+    FATTN_PIN(25, "{a[228:231]}")
+    FATTN_PIN(26, "{a[232:235]}")
+    FATTN_PIN(27, "{a[236:239]}")
+    FATTN_PIN(28, "{a[240:243]}")
+    FATTN_PIN(29, "{a[244:247]}")
+    FATTN_PIN(30, "{a[248:251]}")
+    FATTN_PIN(31, "{a[252:255]}")
+#undef FATTN_PIN
+}
+
+// Moves a fragment into its pinned accumulation registers (the value the MFMAs above are given).
+template <int SLOT>
+__device__ __forceinline__ bf16x8 pin_b_fragment(u32x4 w) {
+    bf16x8 out;
+#define FATTN_PIN(I, C, R0, R1, R2, R3)                                                                        \
+    if constexpr (SLOT == I)                                                                                   \
+        asm volatile("v_accvgpr_write_b32 " R0 ", %1\n\tv_accvgpr_write_b32 " R1 ", %2\n\t"                    \
+                     "v_accvgpr_write_b32 " R2 ", %3\n\tv_accvgpr_write_b32 " R3 ", %4"                         \
+                     : C(out) : "v"(w[0]), "v"(w[1]), "v"(w[2]), "v"(w[3]));
+    FATTN_PIN(0, "={a[128:131]}", "a128", "a129", "a130", "a131")
+    FATTN_PIN(1, "={a[132:135]}", "a132", "a133", "a134", "a135")
+    FATTN_PIN(2, "={a[136:139]}", "a136", "a137", "a138", "a139")
+    FATTN_PIN(3, "={a[140:143]}", "a140", "a141", "a142", "a143")
+    FATTN_PIN(4, "={a[144:147]}", "a144", "a145", "a146", "a147")
+    FATTN_PIN(5, "={a[148:151]}", "a148", "a149", "a150", "a151")
+    FATTN_PIN(6, "={a[152:155]}", "a152", "a153", "a154", "a155")
+    FATTN_PIN(7, "={a[156:159]}", "a156", "a157", "a158", "a159")
+    FATTN_PIN(8, "={a[160:163]}", "a160", "a161", "a162", "a163")
+    FATTN_PIN(9, "={a[164:167]}", "a164", "a165", "a166", "a167")
+    FATTN_PIN(10, "={a[168:171]}", "a168", "a169", "a170", "a171")
+    FATTN_PIN(11, "={a[172:175]}", "a172", "a173", "a174", "a175")
+    FATTN_PIN(12, "={a[176:179]}", "a176", "a177", "a178", "a179")
+    FATTN_PIN(13, "={a[180:183]}", "a180", "a181", "a182", "a183")
+    FATTN_PIN(14, "={a[184:187]}", "a184", "a185", "a186", "a187")
+    FATTN_PIN(15, "={a[188:191]}", "a188", "a189", "a190", "a191")
+    FATTN_PIN(16, "={a[192:195]}", "a192", "a193", "a194", "a195")
+    FATTN_PIN(17, "={a[196:199]}", "a196", "a197", "a198", "a199")
+    FATTN_PIN(18, "={a[200:203]}", "a200", "a201", "a202", "a203")
+    FATTN_PIN(19, "={a[204:207]}", "a204", "a205", "a206", "a207")
+    FATTN_PIN(20, "={a[208:211]}", "a208", "a209", "a210", "a211")
+    FATTN_PIN(21, "={a[212:215]}", "a212", "a213", "a214", "a215")
+    FATTN_PIN(22, "={a[216:219]}", "a216", "a217", "a218", "a219")
+    FATTN_PIN(23, "={a[220:223]}", "a220", "a221", "a222", "a223")
+    FATTN_PIN(24, "={a[224:227]}", "a224", "a225", "a226", "a227")
+    FATTN_PIN(25, "={a[228:231]}", "a228", "a229", "a230", "a231")
+    FATTN_PIN(26, "={a[232:235]}", "a232", "a233", "a234", "a235")
+    FATTN_PIN(27, "={a[236:239]}", "a236", "a237", "a238", "a239")
+    FATTN_PIN(28, "={a[240:243]}", "a240", "a241", "a242", "a243")
+    FATTN_PIN(29, "={a[244:247]}", "a244", "a245", "a246", "a247")
+    FATTN_PIN(30, "={a[248:251]}", "a248", "a249", "a250", "a251")
+    FATTN_PIN(31, "={a[252:255]}", "a252", "a253", "a254", "a255")
+#undef FATTN_PIN
+    return out;
+}
+
+// compile-time loop: f(std::integral_constant<int, 0>{}) ... f(std::integral_constant<int, N - 1>{})
+template <class F, int... Is>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, Is...>) {
+    (f(std::integral_constant<int, Is>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+    static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
 
 // row index inside a 32x32 accumulator block for register r of a lane in half h

@@ -135,7 +135,8 @@ int launch_bwd(const BwdParams& p, hipStream_t s) {
     static bool attr_done = false;
     auto kern = bwd_dkdv_kernel<D, HASMASK, TIMING>;
     auto kern_dq = bwd_dq_kernel<D, HASMASK, 4>;
-    auto kern_dq8 = bwd_dq_kernel<D, HASMASK, HASMASK ? 4 : 8>;      // 256-query workgroups, unmasked builds only
+    using TW = BwdDqWideTile<D>;
+    auto kern_dqw = bwd_dq_wide_kernel<D>;                           // 256-query workgroups, builds without a keep-mask only
     if (!attr_done) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS_BYTES);
@@ -143,14 +144,14 @@ int launch_bwd(const BwdParams& p, hipStream_t s) {
         e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern_dq),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, TQ::LDS_BYTES);
         if (e != hipSuccess) return (int)e;
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern_dq8),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, TQ::LDS_BYTES);
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern_dqw),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, TW::LDS_BYTES);
         if (e != hipSuccess) return (int)e;
         attr_done = true;
     }
     const int64_t n_kt = (p.Sk + T::BN - 1) / T::BN;
     const int64_t grid = n_kt * p.B * p.H;
-    // 256-query workgroups (8 wavefronts) when they neither add padding rows nor leave compute units idle
+    // 256-query workgroups (4 wavefronts of 64 queries) when they neither add padding rows nor leave compute units idle
     const int64_t n256 = (p.Sq + 255) / 256;
     const bool wide = !HASMASK && n256 * 256 <= ((int64_t)(p.Sq + 127) / 128) * 128 && n256 * p.B * p.H >= device_cu_count() &&
                       env_int("FLAME_ATTN_WG_WAVES", 8) != 4;
@@ -161,7 +162,7 @@ int launch_bwd(const BwdParams& p, hipStream_t s) {
     // workspace, which the dK/dV kernel stages per query tile.
     {
         ScopedKernelTimer t(FLAME_ATTN_KERNEL_BWD_DQ, s);
-        if (wide) hipLaunchKernelGGL(kern_dq8, dim3((unsigned)grid_dq), dim3(512), TQ::LDS_BYTES, s, p);
+        if (wide) hipLaunchKernelGGL(kern_dqw, dim3((unsigned)grid_dq), dim3(256), TW::LDS_BYTES, s, p);
         else hipLaunchKernelGGL(kern_dq, dim3((unsigned)grid_dq), dim3(256), TQ::LDS_BYTES, s, p);
     }
     // The dK/dV kernel keeps one workgroup per compute unit.  When the key blocks do not fill the last

@@ -41,7 +41,7 @@ def text():
 
 
 def test_hand_emitted_mfma_results_are_not_touched_too_early(text):
-    kernels = re.findall(r"^(_ZN5fattn15bwd_dkdv_kernel\w+):.*?\.end_amdhsa_kernel", text, re.S | re.M)
+    kernels = re.findall(r"^(_ZN5fattn(?:15bwd_dkdv_kernel|18bwd_dq_wide_kernel)\w+):.*?\.end_amdhsa_kernel", text, re.S | re.M)
     assert len(kernels) >= 4
     checked = 0
     for name in kernels:
