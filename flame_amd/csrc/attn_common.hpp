@@ -149,6 +149,31 @@ __device__ __forceinline__ bf16x8 pin_b_fragment(u32x4 w) {
     return out;
 }
 
+// acc *= alpha for an accumulator tuple pinned to a[16 IDX : 16 IDX + 15], one register at a time through a
+// single architectural register: rescaling accumulators that live in the accumulation registers
+// through compiler-generated copies needs dozens of temporaries and ended in scratch spills.
+template <int IDX>
+__device__ __forceinline__ void rescale_pinned(f32x16& acc, float alpha) {
+    static_assert(IDX >= 0 && IDX < 8, "eight pinned accumulator tuples");
+    float tmp;
+    if constexpr (IDX == 0)
+        asm volatile("v_accvgpr_read_b32 %1, a0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a0, %1\n\tv_accvgpr_read_b32 %1, a1\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a1, %1\n\tv_accvgpr_read_b32 %1, a2\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a2, %1\n\tv_accvgpr_read_b32 %1, a3\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a3, %1\n\tv_accvgpr_read_b32 %1, a4\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a4, %1\n\tv_accvgpr_read_b32 %1, a5\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a5, %1\n\tv_accvgpr_read_b32 %1, a6\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a6, %1\n\tv_accvgpr_read_b32 %1, a7\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a7, %1\n\tv_accvgpr_read_b32 %1, a8\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a8, %1\n\tv_accvgpr_read_b32 %1, a9\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a9, %1\n\tv_accvgpr_read_b32 %1, a10\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a10, %1\n\tv_accvgpr_read_b32 %1, a11\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a11, %1\n\tv_accvgpr_read_b32 %1, a12\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a12, %1\n\tv_accvgpr_read_b32 %1, a13\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a13, %1\n\tv_accvgpr_read_b32 %1, a14\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a14, %1\n\tv_accvgpr_read_b32 %1, a15\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a15, %1" : "+{a[0:15]}"(acc), "=&v"(tmp) : "v"(alpha));
+    if constexpr (IDX == 1)
+        asm volatile("v_accvgpr_read_b32 %1, a16\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a16, %1\n\tv_accvgpr_read_b32 %1, a17\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a17, %1\n\tv_accvgpr_read_b32 %1, a18\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a18, %1\n\tv_accvgpr_read_b32 %1, a19\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a19, %1\n\tv_accvgpr_read_b32 %1, a20\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a20, %1\n\tv_accvgpr_read_b32 %1, a21\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a21, %1\n\tv_accvgpr_read_b32 %1, a22\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a22, %1\n\tv_accvgpr_read_b32 %1, a23\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a23, %1\n\tv_accvgpr_read_b32 %1, a24\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a24, %1\n\tv_accvgpr_read_b32 %1, a25\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a25, %1\n\tv_accvgpr_read_b32 %1, a26\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a26, %1\n\tv_accvgpr_read_b32 %1, a27\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a27, %1\n\tv_accvgpr_read_b32 %1, a28\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a28, %1\n\tv_accvgpr_read_b32 %1, a29\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a29, %1\n\tv_accvgpr_read_b32 %1, a30\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a30, %1\n\tv_accvgpr_read_b32 %1, a31\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a31, %1" : "+{a[16:31]}"(acc), "=&v"(tmp) : "v"(alpha));
+    if constexpr (IDX == 2)
+        asm volatile("v_accvgpr_read_b32 %1, a32\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a32, %1\n\tv_accvgpr_read_b32 %1, a33\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a33, %1\n\tv_accvgpr_read_b32 %1, a34\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a34, %1\n\tv_accvgpr_read_b32 %1, a35\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a35, %1\n\tv_accvgpr_read_b32 %1, a36\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a36, %1\n\tv_accvgpr_read_b32 %1, a37\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a37, %1\n\tv_accvgpr_read_b32 %1, a38\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a38, %1\n\tv_accvgpr_read_b32 %1, a39\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a39, %1\n\tv_accvgpr_read_b32 %1, a40\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a40, %1\n\tv_accvgpr_read_b32 %1, a41\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a41, %1\n\tv_accvgpr_read_b32 %1, a42\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a42, %1\n\tv_accvgpr_read_b32 %1, a43\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a43, %1\n\tv_accvgpr_read_b32 %1, a44\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a44, %1\n\tv_accvgpr_read_b32 %1, a45\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a45, %1\n\tv_accvgpr_read_b32 %1, a46\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a46, %1\n\tv_accvgpr_read_b32 %1, a47\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a47, %1" : "+{a[32:47]}"(acc), "=&v"(tmp) : "v"(alpha));
+    if constexpr (IDX == 3)
+        asm volatile("v_accvgpr_read_b32 %1, a48\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a48, %1\n\tv_accvgpr_read_b32 %1, a49\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a49, %1\n\tv_accvgpr_read_b32 %1, a50\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a50, %1\n\tv_accvgpr_read_b32 %1, a51\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a51, %1\n\tv_accvgpr_read_b32 %1, a52\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a52, %1\n\tv_accvgpr_read_b32 %1, a53\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a53, %1\n\tv_accvgpr_read_b32 %1, a54\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a54, %1\n\tv_accvgpr_read_b32 %1, a55\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a55, %1\n\tv_accvgpr_read_b32 %1, a56\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a56, %1\n\tv_accvgpr_read_b32 %1, a57\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a57, %1\n\tv_accvgpr_read_b32 %1, a58\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a58, %1\n\tv_accvgpr_read_b32 %1, a59\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a59, %1\n\tv_accvgpr_read_b32 %1, a60\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a60, %1\n\tv_accvgpr_read_b32 %1, a61\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a61, %1\n\tv_accvgpr_read_b32 %1, a62\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a62, %1\n\tv_accvgpr_read_b32 %1, a63\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a63, %1" : "+{a[48:63]}"(acc), "=&v"(tmp) : "v"(alpha));
+    if constexpr (IDX == 4)
+        asm volatile("v_accvgpr_read_b32 %1, a64\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a64, %1\n\tv_accvgpr_read_b32 %1, a65\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a65, %1\n\tv_accvgpr_read_b32 %1, a66\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a66, %1\n\tv_accvgpr_read_b32 %1, a67\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a67, %1\n\tv_accvgpr_read_b32 %1, a68\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a68, %1\n\tv_accvgpr_read_b32 %1, a69\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a69, %1\n\tv_accvgpr_read_b32 %1, a70\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a70, %1\n\tv_accvgpr_read_b32 %1, a71\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a71, %1\n\tv_accvgpr_read_b32 %1, a72\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a72, %1\n\tv_accvgpr_read_b32 %1, a73\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a73, %1\n\tv_accvgpr_read_b32 %1, a74\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a74, %1\n\tv_accvgpr_read_b32 %1, a75\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a75, %1\n\tv_accvgpr_read_b32 %1, a76\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a76, %1\n\tv_accvgpr_read_b32 %1, a77\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a77, %1\n\tv_accvgpr_read_b32 %1, a78\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a78, %1\n\tv_accvgpr_read_b32 %1, a79\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a79, %1" : "+{a[64:79]}"(acc), "=&v"(tmp) : "v"(alpha));
+    if constexpr (IDX == 5)
+        asm volatile("v_accvgpr_read_b32 %1, a80\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a80, %1\n\tv_accvgpr_read_b32 %1, a81\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a81, %1\n\tv_accvgpr_read_b32 %1, a82\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a82, %1\n\tv_accvgpr_read_b32 %1, a83\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a83, %1\n\tv_accvgpr_read_b32 %1, a84\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a84, %1\n\tv_accvgpr_read_b32 %1, a85\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a85, %1\n\tv_accvgpr_read_b32 %1, a86\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a86, %1\n\tv_accvgpr_read_b32 %1, a87\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a87, %1\n\tv_accvgpr_read_b32 %1, a88\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a88, %1\n\tv_accvgpr_read_b32 %1, a89\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a89, %1\n\tv_accvgpr_read_b32 %1, a90\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a90, %1\n\tv_accvgpr_read_b32 %1, a91\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a91, %1\n\tv_accvgpr_read_b32 %1, a92\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a92, %1\n\tv_accvgpr_read_b32 %1, a93\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a93, %1\n\tv_accvgpr_read_b32 %1, a94\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a94, %1\n\tv_accvgpr_read_b32 %1, a95\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a95, %1" : "+{a[80:95]}"(acc), "=&v"(tmp) : "v"(alpha));
+    if constexpr (IDX == 6)
+        asm volatile("v_accvgpr_read_b32 %1, a96\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a96, %1\n\tv_accvgpr_read_b32 %1, a97\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a97, %1\n\tv_accvgpr_read_b32 %1, a98\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a98, %1\n\tv_accvgpr_read_b32 %1, a99\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a99, %1\n\tv_accvgpr_read_b32 %1, a100\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a100, %1\n\tv_accvgpr_read_b32 %1, a101\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a101, %1\n\tv_accvgpr_read_b32 %1, a102\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a102, %1\n\tv_accvgpr_read_b32 %1, a103\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a103, %1\n\tv_accvgpr_read_b32 %1, a104\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a104, %1\n\tv_accvgpr_read_b32 %1, a105\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a105, %1\n\tv_accvgpr_read_b32 %1, a106\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a106, %1\n\tv_accvgpr_read_b32 %1, a107\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a107, %1\n\tv_accvgpr_read_b32 %1, a108\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a108, %1\n\tv_accvgpr_read_b32 %1, a109\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a109, %1\n\tv_accvgpr_read_b32 %1, a110\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a110, %1\n\tv_accvgpr_read_b32 %1, a111\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a111, %1" : "+{a[96:111]}"(acc), "=&v"(tmp) : "v"(alpha));
+    if constexpr (IDX == 7)
+        asm volatile("v_accvgpr_read_b32 %1, a112\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a112, %1\n\tv_accvgpr_read_b32 %1, a113\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a113, %1\n\tv_accvgpr_read_b32 %1, a114\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a114, %1\n\tv_accvgpr_read_b32 %1, a115\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a115, %1\n\tv_accvgpr_read_b32 %1, a116\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a116, %1\n\tv_accvgpr_read_b32 %1, a117\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a117, %1\n\tv_accvgpr_read_b32 %1, a118\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a118, %1\n\tv_accvgpr_read_b32 %1, a119\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a119, %1\n\tv_accvgpr_read_b32 %1, a120\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a120, %1\n\tv_accvgpr_read_b32 %1, a121\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a121, %1\n\tv_accvgpr_read_b32 %1, a122\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a122, %1\n\tv_accvgpr_read_b32 %1, a123\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a123, %1\n\tv_accvgpr_read_b32 %1, a124\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a124, %1\n\tv_accvgpr_read_b32 %1, a125\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a125, %1\n\tv_accvgpr_read_b32 %1, a126\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a126, %1\n\tv_accvgpr_read_b32 %1, a127\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a127, %1" : "+{a[112:127]}"(acc), "=&v"(tmp) : "v"(alpha));
+}
+
 // compile-time loop: f(std::integral_constant<int, 0>{}) ... f(std::integral_constant<int, N - 1>{})
 template <class F, int... Is>
 __device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, Is...>) {

@@ -425,4 +425,379 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void fwd_kernel(const Fwd
     }
 }
 
+// ------------------------------------------------------------------- forward, 256-query workgroups
+// The same computation as fwd_kernel for workgroups of 256 queries, laid out for one wavefront per
+// SIMD: 4 wavefronts of 64 queries (two 32-query blocks) each, so that every K / V fragment read from
+// LDS feeds two MFMAs and the LDS reads and waits per MFMA halve.  O^T of both blocks and the Q
+// fragments live in the accumulation registers (Q as pinned MFMA B operands), the logits in
+// architectural registers through hand-emitted MFMAs (see mfma32_vgpr): nothing may touch them until
+// two further MFMAs have been issued.  Four LDS stages, K(t) and V(t) in stage t % 4: step t reads
+// K(t+1) and V(t) and issues the copies of K(t+3) and V(t+2), each into a slot whose previous tile was
+// last read two barriers ago, and each with more than a full step to land; one workgroup barrier
+// per step, placed just before the fragment ring first reads K(t+2); the ring runs on across steps.
+// Every step is the pipelined one: the kernel serves problems without any exclusion (no causal
+// flag, key lengths, keep-mask or bias, Sk a multiple of 64); all others use fwd_kernel.  Copies past the
+// last tile re-read the last tile, and the logits "of the tile after the last" are never used.  A
+// kernel of this size must not spill: scratch memory per wavefront limits how many workgroups the
+// device keeps resident, which halved the throughput of a version with a general slow path.
+template <int D>
+struct FwdWideTile {
+    static constexpr int BM = 256;
+    static constexpr int BN = 64;
+    static constexpr int RS = D;
+    static constexpr int TILE_ELEMS = BN * D;
+    static constexpr int STAGE_ELEMS = 2 * TILE_ELEMS;
+    static constexpr int NSTAGE = 4;
+    static constexpr int LDS_BYTES = NSTAGE * STAGE_ELEMS * 2;
+    static constexpr int ROWS_PER_DMA = 1024 / (D * 2);
+    static constexpr int DMA_PER_WAVE = BN / ROWS_PER_DMA / 4;
+};
+
+template <int D>
+__global__ __launch_bounds__(256) void fwd_wide_kernel(const FwdParams p) {
+    using T = FwdWideTile<D>;
+    constexpr int BN = T::BN, RS = T::RS, BM = T::BM;
+    constexpr int DC = D / 16, DB = D / 32, GPR = D / 8;
+    constexpr int NDMA = T::DMA_PER_WAVE;
+    constexpr int PD = 4;
+    constexpr int NKF = 2 * DC;          // K fragments per tile (dc, kb); two logit MFMAs each
+    constexpr int NVF = 4 * DB;          // V^T fragments per tile (16-key chunk, db); two PV MFMAs each
+    static_assert(NKF % PD == 0 && NVF % PD == 0, "read-ahead depth must divide the fragment counts");
+    static_assert(NKF == 16 || NKF == 8, "softmax slicing assumes 16 or 8 K fragments per tile");
+    static_assert(DB <= 4, "O^T tuples are pinned four to a query block");
+
+    extern __shared__ __attribute__((aligned(1024))) uint16_t lds[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 31, h = lane >> 5;
+
+    const int n_qt = (p.Sq + BM - 1) / BM;
+    const int wg = xcd_remap(blockIdx.x, gridDim.x);
+    const int qt = wg % n_qt;
+    const int bh = wg / n_qt;
+    const int b = bh / p.H, hh = bh % p.H;
+    const int q0 = qt * BM;
+    const int qw0 = q0 + wave * 64;
+
+    const uint16_t* qbase = p.q + b * p.qs.b + hh * p.qs.h;
+    const uint16_t* kbase = p.k + b * p.ks.b + hh * p.ks.h;
+    const uint16_t* vbase = p.v + b * p.vs.b + hh * p.vs.h;
+    uint16_t* obase = p.o + b * p.os.b + hh * p.os.h;
+
+    const int n_tiles = p.Sk / BN;          // the launcher guarantees Sk % BN == 0 and no exclusions
+
+    // ---- Q fragments (B operand of S^T = K Q^T): column = query, 8 consecutive d; pinned slots qb*DC + dc
+    bf16x8 qf[2][DC];
+    int qrow[2];
+    static_for<2>([&](auto qb_tag) {
+        constexpr int qb = decltype(qb_tag)::value;
+        qrow[qb] = qw0 + 32 * qb + n;
+        const bool ok = qrow[qb] < p.Sq;
+        const uint16_t* rp = qbase + (int64_t)qrow[qb] * p.qs.n + 8 * h;
+        static_for<DC>([&](auto dc_tag) {
+            constexpr int dc = decltype(dc_tag)::value;
+            qf[qb][dc] = pin_b_fragment<qb * DC + dc>(ldg16(rp + 16 * dc, ok));
+        });
+    });
+
+    // ---- asynchronous tile copies: tile t (K and V) lives in stage t % 4
+    const uint32_t lds0 = lds_addr(lds);
+    const int dma_row_in = lane / GPR, dma_gran = lane % GPR;
+    uint32_t k_lane_off[NDMA], v_lane_off[NDMA];
+#pragma unroll
+    for (int i = 0; i < NDMA; ++i) {
+        const int row = (wave * NDMA + i) * T::ROWS_PER_DMA + dma_row_in;
+        const int c = dma_gran ^ swz<D>(row);
+        k_lane_off[i] = 2u * (uint32_t)(row * (int)p.ks.n + c * 8);
+        v_lane_off[i] = 2u * (uint32_t)(row * (int)p.vs.n + c * 8);
+    }
+    auto dst_of = [&](int stg, int which, int i) {
+        return lds0 + 2u * (uint32_t)(stg * T::STAGE_ELEMS + which * T::TILE_ELEMS + (wave * NDMA + i) * 512);
+    };
+    // whole tile t (clamped to the last one) of K or V into stage t % 4, all copies at once (prologue)
+    auto issue_whole = [&](const uint16_t* base, int64_t row_stride, const uint32_t (&lane_off)[NDMA], int t, int which) {
+        const uint16_t* tb = base + (int64_t)min(t, n_tiles - 1) * BN * row_stride;
+#pragma unroll
+        for (int i = 0; i < NDMA; ++i) dma16u(tb, lane_off[i], dst_of(t & 3, which, i));
+    };
+
+    // ---- per-lane LDS read offsets (elements), constant over the key loop
+    int koff[DC];
+#pragma unroll
+    for (int dc = 0; dc < DC; ++dc) koff[dc] = n * RS + (((2 * dc + h) ^ swz<D>(n)) << 3);
+    const int tr_r = lane & 15, tr_g16 = (lane >> 4) & 1;
+    int voff[2][DB];
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+        const int row = 4 * h + (tr_r >> 2) + 8 * half;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+            voff[half][db] = row * RS + (((4 * db + 2 * tr_g16 + ((tr_r & 3) >> 1)) ^ swz<D>(row)) << 3) + 4 * (tr_r & 1);
+    }
+    auto k_frag = [&](const uint16_t* stage, int i) {       // fragment i = (dc, kb)
+        return *reinterpret_cast<const bf16x8*>(stage + koff[i >> 1] + 32 * (i & 1) * RS);
+    };
+    auto v_frag = [&](const uint16_t* stage, int i) {       // fragment i = (cc, db) of V^T
+        const uint16_t* vs = stage + T::TILE_ELEMS;
+        const int cc = i / DB, db = i % DB;
+        const u32x2 lo = lds_read_tr16(vs + voff[0][db] + 16 * cc * RS);
+        const u32x2 hi = lds_read_tr16(vs + voff[1][db] + 16 * cc * RS);
+        const u32x4 u = {lo[0], lo[1], hi[0], hi[1]};
+        return __builtin_bit_cast(bf16x8, u);
+    };
+
+    // ---- running state; each lane serves query column n of both blocks
+    const float c_log2 = p.scale * kLog2e;
+    const float stale_ok = 8.0f / c_log2;
+    float m_run[2] = {-INFINITY, -INFINITY}, l_run[2] = {0.f, 0.f};
+    f32x16 oacc[2][DB];
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) oacc[qb][db][r] = 0.f;
+
+    // Fold the tile maximum of one query block into its running state (see fwd_kernel).  O^T of block
+    // qb is pinned to a[64 qb : 64 qb + 63] for the rescale.
+    auto fold_max = [&](auto qb_tag, float tmax) {
+        constexpr int qb = decltype(qb_tag)::value;
+        tmax = fmaxf(tmax, xhalf(tmax));
+        if (__any(tmax > m_run[qb] + stale_ok)) {
+            const float m_old = m_run[qb];
+            const float m_new = fmaxf(m_old, tmax);
+            const float m_to = (m_new == -INFINITY) ? 0.f : m_new;
+            const float alpha = exp2_fast((m_old - m_to) * c_log2);
+            m_run[qb] = m_new;
+            l_run[qb] *= alpha;
+            static_for<DB>([&](auto db_tag) {
+                constexpr int db = decltype(db_tag)::value;
+                rescale_pinned<4 * qb + db>(oacc[qb][db], alpha);
+            });
+        }
+    };
+    // the first tile: nothing accumulated yet
+    auto first_max = [&](int qb, float tmax) { m_run[qb] = fmaxf(tmax, xhalf(tmax)); };
+    // the hand-emitted MFMAs' results become visible 11 issue cycles after issue; the logits pass through
+    // the statement so that nothing that reads them can be scheduled ahead of it
+    auto settle = [&](f32x16 (&s)[2][2]) {
+        asm volatile("s_nop 7\n\ts_nop 7" : "+v"(s[0][0]), "+v"(s[0][1]), "+v"(s[1][0]), "+v"(s[1][1]));
+    };
+    // S(t)^T of both query blocks from the K tile in `stage`, no overlap (prologue and slow steps)
+    auto logits_plain = [&](f32x16 (&s)[2][2], const uint16_t* stage) {
+        static_for<NKF>([&](auto i_tag) {
+            constexpr int i = decltype(i_tag)::value;
+            const bf16x8 kfr = k_frag(stage, i);
+            static_for<2>([&](auto qb_tag) {
+                constexpr int qb = decltype(qb_tag)::value;
+                mfma32_vgpr_bpinned<qb * DC + (i >> 1), (i >> 1) == 0 ? 0 : 1>(s[qb][i & 1], kfr, qf[qb][i >> 1], s[qb][i & 1]);
+            });
+        });
+        settle(s);
+    };
+    auto tile_max = [&](const f32x16 (&s)[2]) {
+        float tmax = s[0][0];
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, s[kb][r]);
+        return tmax;
+    };
+
+    bf16x8 fb[PD];
+    // One step: P(t) from the logits in `cur`, logits of tile t+1 into `nxt`, O += P(t) V(t).  MFMA slot
+    // = 2 * fragment + query block.  The exponentials of tile t are threaded between the logit MFMAs of
+    // tile t+1, the row-maximum scan of tile t+1 between the MFMAs of O += P(t) V(t).
+    // STAGE: stage of tile t (0 .. 3).  k3_base / v2_base: tiles t+3 of K and t+2 of V (clamped).
+    auto step = [&](auto stage_tag, f32x16 (&cur)[2][2], f32x16 (&nxt)[2][2], const uint16_t* k3_base,
+                    const uint16_t* v2_base) {
+        constexpr int s0 = decltype(stage_tag)::value;
+        constexpr int s1 = (s0 + 1) & 3, s2 = (s0 + 2) & 3, s3 = (s0 + 3) & 3;
+        const uint16_t* stage_t = lds + s0 * T::STAGE_ELEMS;       // V(t)
+        const uint16_t* stage_t1 = lds + s1 * T::STAGE_ELEMS;      // K(t+1)
+        const uint16_t* stage_t2 = lds + s2 * T::STAGE_ELEMS;      // K(t+2), landed during this step at the latest
+        float msc[2], rsum0[2] = {0.f, 0.f}, rsum1[2] = {0.f, 0.f};
+#pragma unroll
+        for (int qb = 0; qb < 2; ++qb) msc[qb] = ((m_run[qb] == -INFINITY) ? 0.f : m_run[qb]) * c_log2;
+        u32x4 pw[2][4];                 // P^T operands: [query block][16-key chunk]
+        // exponentials of logits 2j, 2j + 1 (in (kb, r) order) of query block qb
+        auto exp_pair = [&](int qb, int j) {
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                const int idx = 2 * j + e, kb = idx >> 4, r = idx & 15;
+                cur[qb][kb][r] = exp2_fast(fmaf(cur[qb][kb][r], c_log2, -msc[qb]));
+            }
+        };
+        // sums and packs a pair one slot after its exponentials, so that nothing waits on the transcendental unit
+        auto pack_pair = [&](int qb, int j) {
+            const int idx = 2 * j, kb = idx >> 4, r = idx & 15;
+            rsum0[qb] += cur[qb][kb][r];
+            rsum1[qb] += cur[qb][kb][r + 1];
+            pw[qb][idx >> 3][(idx & 7) >> 1] = pack_bf16(cur[qb][kb][r], cur[qb][kb][r + 1]);
+        };
+
+        {
+            constexpr int NSL = 2 * NKF;             // MFMA slots of the logit phase
+            static_assert(NSL == 32 || NSL == 16, "slicing");
+            // copies of K(t+3) and V(t+2); copy j goes with slot CS*j + 1
+            constexpr int NCOPY = 2 * NDMA, CS = (NSL - 2) / NCOPY;
+            static_assert(CS >= 2, "copies do not fit the logit phase");
+            auto copy_dst = [&](int g) {
+                const int j = (g - 1) / CS;
+                if (g >= 1 && (g - 1) % CS == 0 && j < NCOPY) dma_set_dst(dst_of(j < NDMA ? s3 : s2, j / NDMA, j % NDMA));
+            };
+            auto copy_issue = [&](int g) {
+                const int j = (g - 1) / CS;
+                if (g >= 1 && (g - 1) % CS == 0 && j < NCOPY) {
+                    if (j < NDMA) dma16u_issue(k3_base, k_lane_off[j]);
+                    else dma16u_issue(v2_base, v_lane_off[j - NDMA]);
+                }
+            };
+            // ---- S(t+1)^T = K(t+1) Q^T between the exponentials of tile t
+            static_for<NKF>([&](auto i_tag) {
+                constexpr int i = decltype(i_tag)::value;
+                static_for<2>([&](auto qb_tag) {
+                    constexpr int qb = decltype(qb_tag)::value;
+                    constexpr int g = 2 * i + qb;
+                    copy_dst(g);
+                    mfma32_vgpr_bpinned<qb * DC + (i >> 1), (i >> 1) == 0 ? 0 : 1>(nxt[qb][i & 1], fb[i % PD], qf[qb][i >> 1], nxt[qb][i & 1]);
+                    __builtin_amdgcn_sched_barrier(0);
+                    copy_issue(g);
+                    // slot g: exponentials of pairs of query block qb, packing of the pairs of the slot before
+                    constexpr int PPS = 32 / NSL;        // pairs per slot and block: 1 or 2
+#pragma unroll
+                    for (int e = 0; e < PPS; ++e) exp_pair(qb, PPS * i + e);
+                    if (i > 0) {
+#pragma unroll
+                        for (int e = 0; e < PPS; ++e) pack_pair(qb, PPS * (i - 1) + e);
+                    }
+                    if (qb == 1) {
+                        if (i + PD < NKF) fb[i % PD] = k_frag(stage_t1, i + PD);
+                        else fb[i % PD] = v_frag(stage_t, i + PD - NKF);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                });
+            });
+#pragma unroll
+            for (int qb = 0; qb < 2; ++qb) {
+                constexpr int PPS = 32 / NSL;
+#pragma unroll
+                for (int e = 0; e < PPS; ++e) pack_pair(qb, PPS * (NKF - 1) + e);
+                l_run[qb] += rsum0[qb] + rsum1[qb];
+            }
+            // ---- O^T += V(t)^T P(t)^T between the row-maximum scan of tile t+1
+            float tmax[2];
+            constexpr int NPV = 2 * NVF;             // MFMA slots of this phase
+            static_for<NVF>([&](auto i_tag) {
+                constexpr int i = decltype(i_tag)::value;
+                constexpr int cc = i / DB, db = i % DB;
+                static_for<2>([&](auto qb_tag) {
+                    constexpr int qb = decltype(qb_tag)::value;
+                    constexpr int g = 2 * i + qb;
+                    oacc[qb][db] = mfma32(fb[i % PD], __builtin_bit_cast(bf16x8, pw[qb][cc]), oacc[qb][db]);
+                    __builtin_amdgcn_sched_barrier(0);
+                    // the logits of tile t+1 may be touched from slot 2 on
+                    if (g == 2 + qb) tmax[qb] = nxt[qb][0][0];
+                    if (g >= 2 + qb) {
+                        constexpr int MPS = (32 + (NPV - 2) / 2 - 1) / ((NPV - 2) / 2);     // logits per slot and block
+                        constexpr int k = (g - 2 - qb) / 2;
+#pragma unroll
+                        for (int e = 0; e < MPS; ++e) {
+                            const int idx = 1 + MPS * k + e;
+                            if (idx < 32) tmax[qb] = fmaxf(tmax[qb], nxt[qb][idx >> 4][idx & 15]);
+                        }
+                    }
+                    if (qb == 1) {
+                        if (i == NVF - PD) {
+                            __builtin_amdgcn_sched_barrier(0);
+                            // the copies of the step before (K(t+2), V(t+1)) have landed; this step's may be in flight ...
+                            __builtin_amdgcn_s_waitcnt(0x0F70 | ((2 * NDMA) & 15) | (((2 * NDMA) >> 4) << 14));
+                            __builtin_amdgcn_s_barrier();    // ... for every wave, and every wave is past tile t-1
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
+                        if (i + PD < NVF) fb[i % PD] = v_frag(stage_t, i + PD);
+                        else fb[i % PD] = k_frag(stage_t2, i + PD - NVF);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                });
+            });
+            // Both lanes of a query hold the same reference maximum, so each may test its own half; the
+            // exchange between the halves and the rescale stay inside the rarely taken branch.
+            if (__any(tmax[0] > m_run[0] + stale_ok || tmax[1] > m_run[1] + stale_ok)) {
+                fold_max(std::integral_constant<int, 0>{}, tmax[0]);
+                fold_max(std::integral_constant<int, 1>{}, tmax[1]);
+            }
+        }
+    };
+
+    f32x16 sa[2][2], sb[2][2];
+    if (n_tiles > 0) {
+        // prologue: K(0..2) and V(0..1) land; logits and maximum of tile 0; the ring starts on K(1)
+        issue_whole(kbase, p.ks.n, k_lane_off, 0, 0);
+        issue_whole(kbase, p.ks.n, k_lane_off, 1, 0);
+        issue_whole(kbase, p.ks.n, k_lane_off, 2, 0);
+        issue_whole(vbase, p.vs.n, v_lane_off, 0, 1);
+        issue_whole(vbase, p.vs.n, v_lane_off, 1, 1);
+        wait_vm0();
+        __syncthreads();
+        logits_plain(sa, lds);
+#pragma unroll
+        for (int qb = 0; qb < 2; ++qb) first_max(qb, tile_max(sa[qb]));
+#pragma unroll
+        for (int i = 0; i < PD; ++i) fb[i] = k_frag(lds + T::STAGE_ELEMS, i);
+
+        const int64_t k_tile_stride = (int64_t)BN * p.ks.n, v_tile_stride = (int64_t)BN * p.vs.n;
+        using I0 = std::integral_constant<int, 0>;
+        using I1 = std::integral_constant<int, 1>;
+        using I2 = std::integral_constant<int, 2>;
+        using I3 = std::integral_constant<int, 3>;
+        // Tile t sits in stage t % 4 and its logits in `sa` when t is even: four step bodies.
+        const uint16_t *k3, *v2;
+        auto bases = [&](int t) {      // copies past the last tile re-read the last tile
+            k3 = kbase + (int64_t)min(t + 3, n_tiles - 1) * k_tile_stride;
+            v2 = vbase + (int64_t)min(t + 2, n_tiles - 1) * v_tile_stride;
+        };
+        for (int t = 0; t < n_tiles; t += 4) {
+            bases(t);
+            step(I0{}, sa, sb, k3, v2);
+            if (t + 1 >= n_tiles) break;
+            bases(t + 1);
+            step(I1{}, sb, sa, k3, v2);
+            if (t + 2 >= n_tiles) break;
+            bases(t + 2);
+            step(I2{}, sa, sb, k3, v2);
+            if (t + 3 >= n_tiles) break;
+            bases(t + 3);
+            step(I3{}, sb, sa, k3, v2);
+        }
+        wait_vm0();          // no copy may land after the workgroup has gone
+    }
+
+    // ---- epilogue
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) {
+        const int row = qrow[qb];
+        const float l = l_run[qb] + xhalf(l_run[qb]);
+        const float inv = l > 0.f ? 1.0f / l : 0.f;
+        if (row < p.Sq) {
+            uint16_t* orow = obase + (int64_t)row * p.os.n;
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const f32x16& a = oacc[qb][db];
+                    u32x2 w = {pack_bf16(a[4 * g] * inv, a[4 * g + 1] * inv),
+                               pack_bf16(a[4 * g + 2] * inv, a[4 * g + 3] * inv)};
+                    *reinterpret_cast<u32x2*>(orow + 32 * db + 8 * g + 4 * h) = w;
+                }
+            if (p.lse && h == 0) {
+                const float v = l > 0.f ? (m_run[qb] * c_log2 + log2_fast(l)) * kLn2 : -INFINITY;
+                p.lse[(int64_t)bh * p.Sq + row] = v;
+            }
+        }
+    }
+}
+
 }  // namespace fattn

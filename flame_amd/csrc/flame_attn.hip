@@ -108,6 +108,29 @@ int launch_fwd(const FwdParams& p, hipStream_t s) {
     return e == hipSuccess ? FLAME_ATTN_OK : (int)e;
 }
 
+// 256-query workgroups, one wavefront per SIMD (builds without keep-mask / bias only)
+template <int D>
+int launch_fwd_wide(const FwdParams& p, hipStream_t s) {
+    using T = FwdWideTile<D>;
+    static bool attr_done = false;
+    auto kern = fwd_wide_kernel<D>;
+    if (!attr_done) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS_BYTES);
+        if (e != hipSuccess) return (int)e;
+        attr_done = true;
+    }
+    const int64_t n_qt = (p.Sq + T::BM - 1) / T::BM;
+    const int64_t grid = n_qt * p.B * p.H;
+    if (grid > 0x7fffffff) return FLAME_ATTN_ERR_UNSUPPORTED;
+    {
+        ScopedKernelTimer t(FLAME_ATTN_KERNEL_FWD, s);
+        hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), T::LDS_BYTES, s, p);
+    }
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? FLAME_ATTN_OK : (int)e;
+}
+
 size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
 // compute units of the current device (cached; 256 when the query fails)
@@ -465,8 +488,13 @@ static int attn_fwd_impl(const void* Q, const void* K, const void* V, void* O, v
     const int64_t n256 = (N_q + 255) / 256;
     const bool wide = !hm && n256 * 256 <= ((N_q + 127) / 128) * 128 && n256 * B * H >= device_cu_count() &&
                       env_int("FLAME_ATTN_WG_WAVES", 8) != 4;      // FLAME_ATTN_WG_WAVES=4 forces 128-query workgroups
-    if (D == 128) return hm ? launch_fwd<128, true, 4>(p, s) : wide ? launch_fwd<128, false, 8>(p, s) : launch_fwd<128, false, 4>(p, s);
-    return hm ? launch_fwd<64, true, 4>(p, s) : wide ? launch_fwd<64, false, 8>(p, s) : launch_fwd<64, false, 4>(p, s);
+    // ... as 4 wavefronts of 64 queries when nothing is excluded at all, else as 8 wavefronts of 32
+    const bool plain = !causal && kv_len == nullptr && N_kv % 64 == 0;
+    if (D == 128)
+        return hm ? launch_fwd<128, true, 4>(p, s)
+                  : wide ? (plain ? launch_fwd_wide<128>(p, s) : launch_fwd<128, false, 8>(p, s)) : launch_fwd<128, false, 4>(p, s);
+    return hm ? launch_fwd<64, true, 4>(p, s)
+              : wide ? (plain ? launch_fwd_wide<64>(p, s) : launch_fwd<64, false, 8>(p, s)) : launch_fwd<64, false, 4>(p, s);
 }
 
 

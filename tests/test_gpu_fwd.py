@@ -139,6 +139,22 @@ def test_cfg2_production_shape_head_subset(oracle):
     _check_fwd(oracle, w, heads=(23, 24), tag="head 23")
 
 
+@pytest.mark.parametrize("D,H,Sq,Sk", [(128, 64, 1024, 512), (64, 64, 1024, 256), (128, 3, 200, 512)])
+def test_reference_maximum_moves_during_the_walk(oracle, D, H, Sq, Sk):
+    """Later keys carry far larger logits than the first tile, so the running maximum outgrows the stale
+    reference by more than 2^8 several times and O is rescaled mid-walk; the first two shapes fill 256-query
+    workgroups on every compute unit (the one-wavefront-per-SIMD kernels), the third uses the narrow ones."""
+    seed = 4242 + D + Sq
+    B = 1
+    t = [W.normal_f32(seed, s, B * H * n * D).reshape(B, H, n, D) for s, n in enumerate((Sq, Sk, Sk))]
+    k = t[1]
+    for j, f in ((64, 4.0), (192, 12.0), (Sk - 64, 30.0)):     # logits grow in steps along the key axis
+        k[:, :, j:, :] *= f / (k[:, :, j:j + 1, :].std() + 1e-6) * k[:, :, :64, :].std()
+    bits = [W.f32_to_bf16_bits(x) for x in (t[0], k, t[2])]
+    w = W.Workload(f"maxmove_{Sq}x{Sk}_d{D}_h{H}", bits[0], bits[1], bits[2], None, 1.0 / math.sqrt(D))
+    _check_fwd(oracle, w, heads=(0, min(H, 3)))
+
+
 def test_invalid_arguments_are_rejected():
     from flame_amd import capi
     q = torch.zeros(1, 1, 8, 96, dtype=torch.bfloat16, device="cuda")
