@@ -1,6 +1,7 @@
 """Static checks of the hazards the compiler cannot see, on the library compiled to assembly.
 
-1. The dK/dV kernel emits its S / dP MFMAs by hand (accumulators pinned to the architectural VGPRs),
+1. The dK/dV kernel and the 256-query forward and dQ kernels emit their logit MFMAs by hand (accumulators
+   pinned to the architectural VGPRs),
    so the compiler's hazard recogniser does not insert the wait states an 8-pass MFMA needs before
    anything else may touch its result.  The kernels are structured so that at least two further MFMAs
    (or, off the hot paths, 11 wait states of s_nop) are issued first.
