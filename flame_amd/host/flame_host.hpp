@@ -11,6 +11,10 @@
 //   flame::autograd_v4::{SdpaConfig, SdpaSave, SdpaCtx, sdpa_forward, sdpa_backward}
 //                                                   src/autograd_v4/ops/sdpa.rs:21-96, :98-326, :826-1009
 //   flame::SageAttention                            src/sage_attention.rs:21-171
+//   flame::autograd_v4::{SdpaStats, SdpaHooks, register_sdpa_hooks}
+//                                                   src/autograd_v4/ops/sdpa.rs:56-79, :1063-1074
+//   flame::perf_telemetry::{telemetry_enabled, log_sdpa_event, log_sdpa_fallback_event}
+//                                                   src/perf_telemetry.rs:7-57, :60-190
 //
 // Only what the path needs of the tensor type is here: a reference-counted device buffer with a
 // shape, element strides, an offset and a dtype (the reference's Tensor supplies exactly these to
@@ -22,7 +26,11 @@
 #include <algorithm>
 #include <cmath>
 #include <cstdint>
+#include <cstdio>
+#include <cstdlib>
 #include <cstring>
+#include <chrono>
+#include <functional>
 #include <memory>
 #include <mutex>
 #include <optional>
@@ -480,6 +488,54 @@ struct SdpaStats {                        // :56-65
     uint32_t nan_inf_hits = 0, syncs = 0, recompute_blocks = 0;
 };
 
+// Debug hooks (:66-79, :1063-1074; the reference compiles them in under its `sdpa_debug` feature and
+// hands them default-initialised statistics).  Registered once per process; while hooks are registered
+// the forward and backward are timed with events, which costs one host synchronisation per call.
+struct SdpaHooks {
+    std::function<void(const SdpaConfig&, std::tuple<size_t, size_t, size_t, size_t>)> on_fwd_start;
+    std::function<void(const SdpaStats&)> on_fwd_end;
+    std::function<void()> on_bwd_start;
+    std::function<void(const SdpaStats&)> on_bwd_end;
+};
+namespace detail_hooks {
+inline std::unique_ptr<SdpaHooks>& slot() {
+    static std::unique_ptr<SdpaHooks> h;
+    return h;
+}
+inline std::mutex& guard() {
+    static std::mutex m;
+    return m;
+}
+}  // namespace detail_hooks
+inline bool register_sdpa_hooks(SdpaHooks hooks) {          // false when hooks are already set (OnceCell::set)
+    std::lock_guard<std::mutex> lk(detail_hooks::guard());
+    if (detail_hooks::slot()) return false;
+    detail_hooks::slot() = std::make_unique<SdpaHooks>(std::move(hooks));
+    return true;
+}
+inline const SdpaHooks* debug_hooks() {
+    std::lock_guard<std::mutex> lk(detail_hooks::guard());
+    return detail_hooks::slot().get();
+}
+// wall time of everything enqueued on `stream` between construction and stop(), in ms
+struct StreamTimer {
+    explicit StreamTimer(hipStream_t s) : stream(s) {
+        ok = hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess && hipEventRecord(e0, stream) == hipSuccess;
+    }
+    float stop() {
+        float ms = 0.f;
+        if (ok && hipEventRecord(e1, stream) == hipSuccess && hipEventSynchronize(e1) == hipSuccess) hipEventElapsedTime(&ms, e0, e1);
+        return ms;
+    }
+    ~StreamTimer() {
+        if (e0) hipEventDestroy(e0);
+        if (e1) hipEventDestroy(e1);
+    }
+    hipStream_t stream;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    bool ok = false;
+};
+
 struct SdpaCtx {                          // :80-96
     Tensor q, k, v, o;
     std::optional<Tensor> attn_mask;
@@ -579,6 +635,13 @@ inline Result<std::pair<Tensor, SdpaCtx>> sdpa_forward(const Tensor& q, const Te
                                                        const SdpaConfig& cfg) {
     if (cfg.dropout_p != 0.f) return unsupported("dropout is not built into the fused kernels");
     if (cfg.save == SdpaSave::SaveProbs) return unsupported("SaveProbs materialises [B,H,Q,K]; use SaveLSE");
+    const SdpaHooks* hooks = debug_hooks();
+    std::unique_ptr<StreamTimer> timer;
+    if (hooks && q.shape().size() == 4 && k.shape().size() == 4) {
+        if (hooks->on_fwd_start)
+            hooks->on_fwd_start(cfg, {(size_t)q.shape()[0], (size_t)q.shape()[1], (size_t)q.shape()[2], (size_t)k.shape()[2]});
+        timer = std::make_unique<StreamTimer>(nullptr);
+    }
     auto r = detail::run_forward(q, k, v, mask, cfg.causal, cfg.scale, true);
     if (!r.ok()) return r.error();
     SdpaCtx ctx;
@@ -590,6 +653,12 @@ inline Result<std::pair<Tensor, SdpaCtx>> sdpa_forward(const Tensor& q, const Te
     ctx.lse = r.value().stats;
     ctx.shapes = {(size_t)q.shape()[0], (size_t)q.shape()[1], (size_t)q.shape()[2], (size_t)k.shape()[2]};
     ctx.stats.bytes_saved = (uint64_t)ctx.o.numel() * 2 + (uint64_t)ctx.lse.numel() * 4;
+    ctx.stats.bytes_alloc = ctx.stats.bytes_saved;         // O and LSE are the only allocations of the forward
+    if (timer) {
+        ctx.stats.fwd_ms = timer->stop();
+        ctx.stats.syncs = 1;
+        if (hooks->on_fwd_end) hooks->on_fwd_end(ctx.stats);
+    }
     Tensor out = r.value().o;
     if (q.requires_grad || k.requires_grad || v.requires_grad) {     // record one Op::Sdpa node (:300-324)
         out.requires_grad = true;
@@ -612,8 +681,21 @@ inline Result<std::tuple<Tensor, Tensor, Tensor>> sdpa_backward(const SdpaCtx& c
     n.mask = ctx.attn_mask;
     n.scale = ctx.scale;
     n.causal = ctx.causal;
+    const SdpaHooks* hooks = debug_hooks();
+    std::unique_ptr<StreamTimer> timer;
+    if (hooks) {
+        if (hooks->on_bwd_start) hooks->on_bwd_start();
+        timer = std::make_unique<StreamTimer>(nullptr);
+    }
     auto g = autograd::flash_attention_backward(n, grad_out);
     if (!g.ok()) return g.error();
+    if (timer) {
+        SdpaStats st = ctx.stats;
+        st.bwd_ms = timer->stop();
+        st.syncs += 1;
+        st.recompute_blocks = (uint32_t)(((std::get<2>(ctx.shapes) + 63) / 64) * ((std::get<3>(ctx.shapes) + 63) / 64));   // P tiles rebuilt per head
+        if (hooks->on_bwd_end) hooks->on_bwd_end(st);
+    }
     return std::make_tuple(g.value().dq, g.value().dk, g.value().dv);
 }
 
@@ -654,11 +736,121 @@ inline Result<Gradients> backward_v4(const Tensor& loss) {
 // and ops::attn::streaming_attn_bf16_fp32(q, k, v, StreamingAttnCfg) (src/ops/attn.rs:7-25, :327-598):
 // the reference's host-looped / per-row streaming kernels.  Same arguments and checks; the chunk size is
 // validated and otherwise ignored, the fused kernel streams K/V tiles by itself.
+// JSONL telemetry of the streaming entry point (src/perf_telemetry.rs): one line per call appended to
+// the file named by FLAME_SDPA_TELEMETRY_PATH, same keys in the same order.  The reference's tile
+// autotuner and plan cache have no counterpart here (tile shapes are fixed per head dim and problem
+// class), so those counters are always written as 0 and plan_source as 0.
+namespace perf_telemetry {
+struct SdpaTelemetryRecord {                // :7-40
+    size_t batch = 0, heads = 0, q_len = 0, k_len = 0, dh = 0, dv = 0, chunk_requested = 0;
+    uint64_t tuned_q_chunk = 0, tuned_k_chunk = 0, plan_source = 0;
+    size_t mask_heads = 0;
+    bool has_mask = false, causal = false;
+    uint64_t workspace_bytes = 0, stream_id = 0;
+    double elapsed_ms = 0.0, tflops = 0.0;
+    float scale = 0.f;
+    uint64_t candidate_count = 0, best_time_ns = 0, autotune_env_forced = 0, autotune_clamped = 0, autotune_skipped = 0,
+             autotune_fallback = 0, autotune_errors = 0, autotune_tuned = 0, cache_hits = 0, cache_misses = 0, cache_saved = 0,
+             cache_loads = 0, cache_load_errors = 0, cache_entries = 0;
+};
+struct SdpaFallbackTelemetryRecord {        // :42-56
+    size_t batch = 0, heads = 0, q_len = 0, k_len = 0, dh = 0, dv = 0, from_chunk = 0, to_chunk = 0;
+    const char* reason = "";
+    std::optional<uint64_t> workspace_required, workspace_limit;
+    std::optional<size_t> free_mem_mb;
+    std::optional<int32_t> error_code;
+};
+inline bool telemetry_enabled() {           // :60-66 (read once)
+    static const bool on = [] {
+        const char* p = std::getenv("FLAME_SDPA_TELEMETRY_PATH");
+        return p && *p;
+    }();
+    return on;
+}
+namespace detail {
+inline std::mutex& guard() {
+    static std::mutex m;
+    return m;
+}
+inline FILE* writer() {                     // :68-101: append, parent directory is the caller's business here
+    static FILE* f = nullptr;
+    if (!f) {
+        const char* p = std::getenv("FLAME_SDPA_TELEMETRY_PATH");
+        if (p && *p) f = std::fopen(p, "a");
+    }
+    return f;
+}
+inline unsigned long long now_ns() {
+    return (unsigned long long)std::chrono::duration_cast<std::chrono::nanoseconds>(
+               std::chrono::system_clock::now().time_since_epoch()).count();
+}
+inline std::string opt_u64(const std::optional<uint64_t>& v) { return v ? std::to_string(*v) : "null"; }
+}  // namespace detail
+inline void log_sdpa_event(const SdpaTelemetryRecord& r) {          // :103-150
+    if (!telemetry_enabled()) return;
+    std::lock_guard<std::mutex> lk(detail::guard());
+    FILE* f = detail::writer();
+    if (!f) return;
+    std::fprintf(f,
+                 "{\"op\":\"sdpa_stream_bf16\",\"timestamp_ns\":%llu,\"batch\":%zu,\"heads\":%zu,\"q_len\":%zu,\"k_len\":%zu,"
+                 "\"dh\":%zu,\"dv\":%zu,\"chunk_requested\":%zu,\"tuned_q_chunk\":%llu,\"tuned_k_chunk\":%llu,\"plan_source\":%llu,"
+                 "\"mask_heads\":%zu,\"has_mask\":%d,\"causal\":%d,\"workspace_bytes\":%llu,\"stream_id\":%llu,\"elapsed_ms\":%.6f,"
+                 "\"tflops\":%.6f,\"scale\":%.6f,\"candidate_count\":%llu,\"best_time_ns\":%llu,\"autotune_env_forced\":%llu,"
+                 "\"autotune_clamped\":%llu,\"autotune_skipped\":%llu,\"autotune_fallback\":%llu,\"autotune_errors\":%llu,"
+                 "\"autotune_tuned\":%llu,\"cache_hits\":%llu,\"cache_misses\":%llu,\"cache_saved\":%llu,\"cache_loads\":%llu,"
+                 "\"cache_load_errors\":%llu,\"cache_entries\":%llu}\n",
+                 detail::now_ns(), r.batch, r.heads, r.q_len, r.k_len, r.dh, r.dv, r.chunk_requested,
+                 (unsigned long long)r.tuned_q_chunk, (unsigned long long)r.tuned_k_chunk, (unsigned long long)r.plan_source,
+                 r.mask_heads, (int)r.has_mask, (int)r.causal, (unsigned long long)r.workspace_bytes,
+                 (unsigned long long)r.stream_id, r.elapsed_ms, r.tflops, (double)r.scale,
+                 (unsigned long long)r.candidate_count, (unsigned long long)r.best_time_ns,
+                 (unsigned long long)r.autotune_env_forced, (unsigned long long)r.autotune_clamped,
+                 (unsigned long long)r.autotune_skipped, (unsigned long long)r.autotune_fallback,
+                 (unsigned long long)r.autotune_errors, (unsigned long long)r.autotune_tuned,
+                 (unsigned long long)r.cache_hits, (unsigned long long)r.cache_misses, (unsigned long long)r.cache_saved,
+                 (unsigned long long)r.cache_loads, (unsigned long long)r.cache_load_errors, (unsigned long long)r.cache_entries);
+    std::fflush(f);
+}
+inline void log_sdpa_fallback_event(const SdpaFallbackTelemetryRecord& r) {   // :152-190
+    if (!telemetry_enabled()) return;
+    std::lock_guard<std::mutex> lk(detail::guard());
+    FILE* f = detail::writer();
+    if (!f) return;
+    std::fprintf(f,
+                 "{\"op\":\"sdpa_stream_bf16_fallback\",\"timestamp_ns\":%llu,\"batch\":%zu,\"heads\":%zu,\"q_len\":%zu,"
+                 "\"k_len\":%zu,\"dh\":%zu,\"dv\":%zu,\"from_chunk\":%zu,\"to_chunk\":%zu,\"reason\":\"%s\","
+                 "\"workspace_required\":%s,\"workspace_limit\":%s,\"free_mem_mb\":%s,\"error_code\":%s}\n",
+                 detail::now_ns(), r.batch, r.heads, r.q_len, r.k_len, r.dh, r.dv, r.from_chunk, r.to_chunk, r.reason,
+                 detail::opt_u64(r.workspace_required).c_str(), detail::opt_u64(r.workspace_limit).c_str(),
+                 r.free_mem_mb ? std::to_string(*r.free_mem_mb).c_str() : "null",
+                 r.error_code ? std::to_string(*r.error_code).c_str() : "null");
+    std::fflush(f);
+}
+}  // namespace perf_telemetry
+
 namespace cuda_ops_bf16 {
 inline Result<Tensor> sdpa_stream_bf16(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor* mask, size_t chunk,
                                        bool causal, std::optional<float> scale) {
     if (chunk == 0) return invalid("sdpa_stream_bf16: chunk must be > 0");
-    return flame::sdpa::forward_v4(q, k, v, mask, causal, scale);
+    if (!perf_telemetry::telemetry_enabled()) return flame::sdpa::forward_v4(q, k, v, mask, causal, scale);
+    autograd_v4::StreamTimer timer(nullptr);
+    auto out = flame::sdpa::forward_v4(q, k, v, mask, causal, scale);
+    if (out.ok() && q.shape().size() == 4) {
+        perf_telemetry::SdpaTelemetryRecord r;
+        r.batch = (size_t)q.shape()[0]; r.heads = (size_t)q.shape()[1]; r.q_len = (size_t)q.shape()[2];
+        r.k_len = (size_t)k.shape()[2]; r.dh = (size_t)q.shape()[3]; r.dv = (size_t)v.shape()[3];
+        r.chunk_requested = chunk;
+        r.tuned_q_chunk = 256; r.tuned_k_chunk = 64;          // the largest tiles the kernels use; nothing is tuned
+        r.has_mask = mask != nullptr;
+        r.mask_heads = mask && mask->shape().size() == 4 ? (size_t)mask->shape()[1] : 0;
+        r.causal = causal;
+        r.scale = scale.value_or(1.0f / std::sqrt((float)q.shape()[3]));
+        r.elapsed_ms = timer.stop();
+        const double pairs = (double)r.batch * r.heads * r.q_len * r.k_len * (causal ? 0.5 : 1.0);
+        r.tflops = r.elapsed_ms > 0 ? 4.0 * pairs * (double)r.dh / (r.elapsed_ms * 1e-3) / 1e12 : 0.0;
+        perf_telemetry::log_sdpa_event(r);
+    }
+    return out;
 }
 }  // namespace cuda_ops_bf16
 

@@ -6,6 +6,8 @@
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
+#include <unistd.h>
+
 #include <vector>
 
 #include "../../flame_amd/host/flame_host.hpp"
@@ -122,6 +124,15 @@ static void compare(const char* name, const std::vector<float>& got, const std::
 }
 
 int main() {
+    // telemetry path is read once per process, before the first call that could log
+    {
+        char path[] = "/tmp/flame_sdpa_telemetry_XXXXXX";
+        const int fd = mkstemp(path);
+        if (fd >= 0) {
+            close(fd);
+            setenv("FLAME_SDPA_TELEMETRY_PATH", path, 1);
+        }
+    }
     int ndev = 0;
     if (hipGetDeviceCount(&ndev) != hipSuccess || ndev == 0) {
         std::printf("no GPU\n");
@@ -435,6 +446,57 @@ int main() {
         }
         Tensor plain = dev_bf16(hq, {B, H, N, D});
         CHECK(!autograd_v4::backward_v4(plain).ok(), "backward_v4 on a tensor without requires_grad must fail");
+    }
+
+    // ---- 10. debug hooks (register once, called around forward and backward with filled statistics) and the
+    //          JSONL telemetry of the streaming entry point (src/perf_telemetry.rs:103-150: same keys)
+    {
+        std::printf("[hooks and telemetry]\n");
+        static int fwd_start = 0, fwd_end = 0, bwd_start = 0, bwd_end = 0;
+        static autograd_v4::SdpaStats last_fwd, last_bwd;
+        static size_t seen_q = 0, seen_k = 0;
+        autograd_v4::SdpaHooks hooks;
+        hooks.on_fwd_start = [](const autograd_v4::SdpaConfig&, std::tuple<size_t, size_t, size_t, size_t> shp) {
+            ++fwd_start;
+            seen_q = std::get<2>(shp);
+            seen_k = std::get<3>(shp);
+        };
+        hooks.on_fwd_end = [](const autograd_v4::SdpaStats& st) { ++fwd_end; last_fwd = st; };
+        hooks.on_bwd_start = [] { ++bwd_start; };
+        hooks.on_bwd_end = [](const autograd_v4::SdpaStats& st) { ++bwd_end; last_bwd = st; };
+        CHECK(autograd_v4::register_sdpa_hooks(hooks), "first registration must succeed");
+        CHECK(!autograd_v4::register_sdpa_hooks(hooks), "second registration must be refused");
+        const int B = 1, H = 2, N = 160, D = 64;
+        auto hq = randn_bf16((size_t)B * H * N * D), hk = randn_bf16(hq.size()), hv = randn_bf16(hq.size());
+        Tensor q = dev_bf16(hq, {B, H, N, D}), k = dev_bf16(hk, {B, H, N, D}), v = dev_bf16(hv, {B, H, N, D});
+        autograd_v4::SdpaConfig cfg;
+        auto f = autograd_v4::sdpa_forward(q, k, v, nullptr, cfg);
+        CHECK(f.ok(), "sdpa_forward failed");
+        CHECK(fwd_start == 1 && fwd_end == 1 && seen_q == (size_t)N && seen_k == (size_t)N, "forward hooks");
+        CHECK(last_fwd.fwd_ms > 0.f && last_fwd.bytes_saved == (uint64_t)B * H * N * D * 2 + (uint64_t)B * H * N * 4, "forward statistics");
+        if (f.ok()) {
+            std::vector<uint16_t> ones((size_t)B * H * N * D, f2bf(1.0f));
+            Tensor g1 = dev_bf16(ones, {B, H, N, D});
+            auto g = autograd_v4::sdpa_backward(f.value().second, g1);
+            CHECK(g.ok(), "sdpa_backward failed");
+            CHECK(bwd_start == 1 && bwd_end == 1 && last_bwd.bwd_ms > 0.f && last_bwd.recompute_blocks == 9, "backward hooks");
+        }
+        // telemetry: the path was set at the top of main(); the call below appends one more line
+        CHECK(perf_telemetry::telemetry_enabled(), "telemetry must be enabled by FLAME_SDPA_TELEMETRY_PATH");
+        auto out = cuda_ops_bf16::sdpa_stream_bf16(q, k, v, nullptr, 512, true, std::nullopt);
+        CHECK(out.ok(), "sdpa_stream_bf16 failed");
+        std::string last, line;
+        if (FILE* tf = std::fopen(std::getenv("FLAME_SDPA_TELEMETRY_PATH"), "r")) {
+            char buf[4096];
+            while (std::fgets(buf, sizeof buf, tf)) last = buf;
+            std::fclose(tf);
+        }
+        CHECK(last.rfind("{\"op\":\"sdpa_stream_bf16\",\"timestamp_ns\":", 0) == 0, "telemetry line must start with op and timestamp");
+        CHECK(last.find("\"q_len\":160,\"k_len\":160,\"dh\":64,\"dv\":64,\"chunk_requested\":512,") != std::string::npos, "shape keys");
+        CHECK(last.find("\"has_mask\":0,\"causal\":1,") != std::string::npos, "flag keys");
+        CHECK(last.find("\"cache_load_errors\":0,\"cache_entries\":0}") != std::string::npos, "last keys");
+        const size_t at = last.find("\"elapsed_ms\":");
+        CHECK(at != std::string::npos && std::atof(last.c_str() + at + 13) > 0.0, "elapsed_ms must be positive");
     }
 
     if (hipDeviceSynchronize() != hipSuccess) ++g_fail;
