@@ -106,3 +106,31 @@ def test_random_case_many_heads(oracle, seed):
         for i, (name, got, S) in enumerate((("dQ", dq, Sq), ("dK", dk, Sk), ("dV", dv, Sk))):
             assert_close_bf16(oracle, f"{name}[{hb}]", sel(got, S), ref[i].reshape(B * H, S, D)[hb:hb + 1],
                               ref[i + 3].reshape(B * H, S, D)[hb:hb + 1])
+
+
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("Sk", [64, 128, 192, 320, 448])
+def test_wide_workgroups_short_key_walks(oracle, D, Sk):
+    """256-query workgroups with 1, 2, 3, 5 and 7 key tiles: every way of entering and leaving the four-step
+    pipeline of the forward and the three-stage walks of the backward, including copies clamped to the
+    last tile."""
+    from flame_amd import capi
+    B, H, Sq = 1, 64, 1024
+    print(f"[wide short walks] H={H} Sq={Sq} Sk={Sk} D={D}", flush=True)
+    q, k, v, do = (W.f32_to_bf16_bits(W.normal_f32(31000 + Sk + D, s, B * H * n * D).reshape(B, H, n, D))
+                   for s, n in enumerate((Sq, Sk, Sk, Sq)))
+    scale = 1.0 / math.sqrt(D)
+    qd, kd, vd, dod = (to_dev(t) for t in (q, k, v, do))
+    o, lse = capi.attn_fwd(qd, kd, vd, scale)
+    dq, dk, dv = capi.attn_bwd(qd, kd, vd, o, dod, lse, scale)
+    torch.cuda.synchronize()
+    for hb in (0, H - 1):
+        heads = (hb, hb + 1)
+        ro, rlse, rof = oracle.sdpa_fwd(q, k, v, scale, heads=heads, want_f32=True)
+        sel = lambda t, S: to_f32(t).reshape(B * H, S, D)[hb:hb + 1]
+        assert_close_bf16(oracle, f"O[{hb}]", sel(o, Sq), ro.reshape(B * H, Sq, D)[hb:hb + 1], rof.reshape(B * H, Sq, D)[hb:hb + 1])
+        assert np.max(np.abs(lse.cpu().numpy().reshape(B * H, Sq)[hb] - rlse.reshape(B * H, Sq)[hb])) <= TOL_LSE
+        ref = oracle.sdpa_bwd(q, k, v, ro, do, scale, heads=heads, want_f32=True)
+        for i, (name, got, S) in enumerate((("dQ", dq, Sq), ("dK", dk, Sk), ("dV", dv, Sk))):
+            assert_close_bf16(oracle, f"{name}[{hb}]", sel(got, S), ref[i].reshape(B * H, S, D)[hb:hb + 1],
+                              ref[i + 3].reshape(B * H, S, D)[hb:hb + 1])
