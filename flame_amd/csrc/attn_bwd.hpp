@@ -1,8 +1,9 @@
 // Backward of the tiled attention for gfx950: recomputes P tile by tile from Q, K and the saved
 // log-sum-exp, never materialising the Sq x Sk matrix.
 //
-//   dq       one workgroup owns 128 queries (32 per wavefront) and walks over the key tiles (64 keys),
-//            with the logits transposed (lane = query): S^T = K Q^T, dP^T = V dO^T,
+//   dq       one workgroup owns 128 queries (32 per wavefront, two wavefronts per SIMD) or, when the
+//            problem fills them, 256 queries (64 per wavefront, one wavefront per SIMD), and walks over
+//            the key tiles (64 keys), with the logits transposed (lane = query): S^T = K Q^T, dP^T = V dO^T,
 //            dS^T = P^T (dP^T - delta) and dQ^T += K^T dS^T accumulated in fp32 registers for the whole
 //            walk, dS^T going into the last MFMA straight from the accumulators.  Runs first and also
 //            leaves -delta_i = -sum_d dO_id * O_id and LSE_i * log2(e) (fp32, one value per query row)
@@ -18,8 +19,8 @@
 // clock per CU, more than the whole MFMA time of the backward; recomputing S and dP in a second,
 // query-major kernel costs 2 extra GEMMs out of 7 and no atomics, no fp32 scratch and no convert pass.
 //
-// Tiles are copied global -> LDS by asynchronous LDS-DMA loads (K / V tiles of dq double buffered,
-// Q / dO tiles of dkdv in three stages), row-major with an XOR swizzle of the 16-byte granules; their
+// Tiles are copied global -> LDS by asynchronous LDS-DMA loads (two stages where two wavefronts share a
+// SIMD, three where one wavefront runs alone and nobody would cover a drained pipeline), row-major with an XOR swizzle of the 16-byte granules; their
 // transposed MFMA operands (Q^T, dO^T) and the dS operand come from transposing LDS reads, so no tile
 // is stored twice and no access pattern has bank conflicts.  One workgroup barrier per step.
 #pragma once
@@ -634,8 +635,8 @@ struct BwdDqTile {
     static constexpr int DMA_PER_WAVE = BN / ROWS_PER_DMA / 4;
 };
 
-// NW wavefronts (4 or 8) of 32 queries each per workgroup; eight share every K/V tile among twice as
-// many queries.  Two wavefronts per SIMD either way.
+// NW wavefronts of 32 queries each per workgroup, two per SIMD (the library instantiates NW = 4; problems
+// that fill 256-query workgroups go to bwd_dq_wide_kernel below).
 template <int D, bool HASMASK, int NW>
 __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void bwd_dq_kernel(const BwdParams p) {
     using T = BwdDqTile<D>;

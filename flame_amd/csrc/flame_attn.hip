@@ -483,7 +483,7 @@ static int attn_fwd_impl(const void* Q, const void* K, const void* V, void* O, v
 
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bool hm = keep_mask != nullptr || bias != nullptr;
-    // 256-query workgroups (8 wavefronts) when they neither add padding rows nor leave compute units
+    // 256-query workgroups when they neither add padding rows nor leave compute units
     // without a workgroup
     const int64_t n256 = (N_q + 255) / 256;
     const bool wide = !hm && n256 * 256 <= ((N_q + 127) / 128) * 128 && n256 * B * H >= device_cu_count() &&
