@@ -116,6 +116,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--config", type=int, default=2, help="workload configuration (2 = the headline shape)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--keep-mask", action="store_true",
+                    help="pass an all-ones [1,1,Sq,Sk] keep-mask, which times the kernels that read an explicit mask "
+                         "(same arithmetic and flop count as the unmasked step)")
     ap.add_argument("--traffic-calibration", action="store_true",
                     help="also run one plain 256 MiB device copy, so that FETCH_SIZE / WRITE_SIZE read under "
                          "rocprofv3 --pmc can be scaled by what the same counters report for a known size")
@@ -148,9 +151,11 @@ def main():
     grads = (torch.empty_like(q), torch.empty_like(k), torch.empty_like(v))
     ws = torch.empty(capi.bwd_workspace_bytes(B, H, Sq, D), dtype=torch.uint8, device=dev)
 
+    mask = torch.ones(1, 1, Sq, Sk, dtype=torch.uint8, device=dev) if args.keep_mask else None
+
     def step():
-        _, lse = capi.attn_fwd(q, k, v, w.scale, causal=w.causal, kv_len=kvl, out=o)
-        capi.attn_bwd(q, k, v, o, do, lse, w.scale, causal=w.causal, kv_len=kvl, workspace=ws, grads=grads)
+        _, lse = capi.attn_fwd(q, k, v, w.scale, causal=w.causal, kv_len=kvl, mask=mask, out=o)
+        capi.attn_bwd(q, k, v, o, do, lse, w.scale, causal=w.causal, kv_len=kvl, mask=mask, workspace=ws, grads=grads)
 
     if args.traffic_calibration:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
@@ -191,11 +196,11 @@ def main():
         "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": w.name, "B": B, "H": H, "Sq": Sq, "Sk": Sk, "D": D, "causal": bool(w.causal),
-                   "step": "forward (O+LSE) + recompute backward (dQ,dK,dV)"},
+                   "step": "forward (O+LSE) + recompute backward (dQ,dK,dV)", "keep_mask": bool(args.keep_mask)},
         "frac_of_bf16_mfma_peak": tflops / PEAK_BF16_TFLOPS,
         "roofline": {"bound": "mfma", "kernel": "bwd_dkdv_kernel", "achieved": achieved, "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS,
-                     "traffic": DKDV_TRAFFIC_BYTES_CFG2 if args.config == 2 else None,
+                     "traffic": DKDV_TRAFFIC_BYTES_CFG2 if args.config == 2 and not args.keep_mask else None,
                      "avg_launch_ms": per_kernel[dom], "flops_per_launch": 8 * pairs_d},
         "kernels": kernels,
         "kernels_ms": per_kernel,

@@ -339,6 +339,19 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
         f32x16 sacc[2];
         bf16x8 pf[2][2], dsf[2][2];
         f32x4 l4, l4n;
+        // keep-mask bytes of this lane's key for the 64 queries of the tile, fetched up front in one batch
+        // (a load per element inside the pipelined slices would wait out a memory round trip each time)
+        uint32_t mk[2][16];
+        if (HASMASK && MASKED) {
+            const uint8_t* mkey = mbase + (int64_t)min(key, p.Sk - 1) * p.m.sk;
+#pragma unroll
+            for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int qi = q0 + 32 * qb + 8 * (r >> 2) + 4 * h + (r & 3);
+                    mk[qb][r] = mkey[(int64_t)min(qi, p.Sq - 1) * p.m.sq];
+                }
+        }
         // lse2 is read one group of four queries ahead of its use, so that waiting for it never drains
         // the fragment reads that were issued in between
         auto rows_ahead = [&](int qb, int g) { l4n = *reinterpret_cast<const f32x4*>(rows_c + 32 * qb + 8 * g + 4 * h); };
@@ -367,9 +380,7 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
                 const int qi = q0 + 32 * qb + 8 * g + 4 * h + t;
                 bool drop = key >= klimit || qi >= p.Sq;
                 if (p.m.causal) drop = drop || key > qi;
-                if (HASMASK) {
-                    if (!drop) drop = mbase[(int64_t)qi * p.m.sq + (int64_t)key * p.m.sk] == 0;
-                }
+                if (HASMASK) drop = drop || mk[qb][r] == 0;
                 pr = drop ? 0.f : pr;
             }
             sacc[qb][r] = pr;
@@ -638,7 +649,7 @@ struct BwdDqTile {
 // NW wavefronts of 32 queries each per workgroup, two per SIMD (the library instantiates NW = 4; problems
 // that fill 256-query workgroups go to bwd_dq_wide_kernel below).
 template <int D, bool HASMASK, int NW>
-__global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void bwd_dq_kernel(const BwdParams p) {
+__global__ __launch_bounds__(64 * NW, (NW == 4 && !HASMASK) ? 2 : 1) void bwd_dq_kernel(const BwdParams p) {
     using T = BwdDqTile<D>;
     constexpr int BM = 32 * NW, BN = T::BN, RS = T::RS;
     constexpr int DC = D / 16;
@@ -766,6 +777,10 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void bwd_dq_kernel(const 
         for (int r = 0; r < 16; ++r) dqacc[db][r] = 0.f;
 
     if (n_tiles > 0) issue_tile(0, 0);
+    MaskRow64 mnext;          // keep-mask bytes of this lane's query row for the next tile (vector-load layouts only)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) mnext.w[j] = u32x4{0u, 0u, 0u, 0u};
+    if (HASMASK && p.m.rows16 && n_tiles > 0 && BN <= p.Sk) mnext.load(mbase + (int64_t)min(qrow, p.Sq - 1) * p.m.sq);
     wait_vm0();
     __syncthreads();
 
@@ -810,6 +825,12 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void bwd_dq_kernel(const 
 
         f32x16 sacc[2], dpacc[2];
         bf16x8 dsf[2][2];
+        // a lane's 64 keep-mask bytes of the tile in four 16-byte loads where the layout allows it, fetched
+        // one tile ahead
+        const bool vec_mask = HASMASK && MASKED && p.m.rows16 && key0 + BN <= p.Sk;
+        const MaskRow64 mrow = mnext;
+        if (HASMASK && MASKED && p.m.rows16 && key0 + 2 * BN <= p.Sk && t + 1 < n_tiles)
+            mnext.load(mbase + (int64_t)min(qrow, p.Sq - 1) * p.m.sq + key0 + BN);
         auto p_elem = [&](int kb, int r) {          // P^T: one query per lane, so LSE is a per-lane scalar
             float pr = exp2_fast(fmaf(sacc[kb][r], c_log2, -lse2));
             if (MASKED) {
@@ -817,7 +838,8 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void bwd_dq_kernel(const 
                 bool drop = key >= klimit;
                 if (p.m.causal) drop = drop || key > qrow;
                 if (HASMASK) {
-                    if (!drop && qok) drop = mbase[(int64_t)qrow * p.m.sq + (int64_t)key * p.m.sk] == 0;
+                    if (vec_mask) drop = drop || !mrow.keep(kb, r, h);
+                    else if (!drop && qok) drop = mbase[(int64_t)qrow * p.m.sq + (int64_t)key * p.m.sk] == 0;
                 }
                 pr = drop ? 0.f : pr;
             }

@@ -291,11 +291,28 @@ struct Strides {
     int64_t b, h, n;   // element strides of a [B,H,N,D] bf16 view; the D stride is 1
 };
 
+// The 64 keep-mask bytes of one query row over a 64-key tile, as loaded by the kernels whose lanes own
+// a query: keep(kb, r) is the byte of key 32*kb + acc_row(r, h).
+struct MaskRow64 {
+    u32x4 w[4];
+    __device__ __forceinline__ void load(const uint8_t* row_tile) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) w[j] = *reinterpret_cast<const u32x4*>(row_tile + 16 * j);
+    }
+    __device__ __forceinline__ bool keep(int kb, int r, int h) const {      // kb, r compile-time; h per lane
+        const int d0 = 8 * kb + 2 * (r >> 2);                               // dword of the even half
+        const uint32_t lo = w[d0 >> 2][d0 & 3], hi = w[(d0 + 1) >> 2][(d0 + 1) & 3];
+        const uint32_t word = h ? hi : lo;
+        return (word & (0xffu << (8 * (r & 3)))) != 0;
+    }
+};
+
 struct MaskArgs {
     const int32_t* kv_len;   // [B] or null
     const uint8_t* mask;     // keep-mask (non-zero = attend) or null
     int64_t sb, sh, sq, sk;  // element strides over (b,h,q,k); 0 broadcasts
     int causal;              // key j > query i is excluded
+    int rows16 = 0;          // keep-mask rows are contiguous along keys and 16-byte aligned (vector loads allowed)
     // additive bias on the scaled logits (forward only), fp32 or bf16, or null
     const void* bias = nullptr;
     int64_t bb = 0, bh = 0, bq = 0, bk = 0;   // element strides over (b,h,q,k); 0 broadcasts

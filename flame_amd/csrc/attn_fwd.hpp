@@ -186,6 +186,11 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void fwd_kernel(const Fwd
     // exclusions of tile t: ragged tail / key length, causal, explicit keep-mask
     auto apply_mask = [&](f32x16 (&s)[2], int t) {
         const int qi = qw0 + n;
+        // a lane's 64 keep-mask bytes of the tile in four 16-byte loads where the layout allows it (each
+        // lane owns a query row, so byte loads would touch one cache line per lane and element)
+        const bool vec_mask = HASMASK && mbase && p.m.rows16 && t * BN + BN <= p.Sk;
+        MaskRow64 mrow;
+        if (vec_mask) mrow.load(mbase + (int64_t)min(qi, p.Sq - 1) * p.m.sq + t * BN);
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
@@ -195,7 +200,8 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void fwd_kernel(const Fwd
                 if (p.m.causal) drop = drop || key > qi;
                 float val = s[kb][r];
                 if (HASMASK) {
-                    if (mbase && !drop && qi < p.Sq) drop = mbase[(int64_t)qi * p.m.sq + (int64_t)key * p.m.sk] == 0;
+                    if (vec_mask) drop = drop || !mrow.keep(kb, r, h);
+                    else if (mbase && !drop && qi < p.Sq) drop = mbase[(int64_t)qi * p.m.sq + (int64_t)key * p.m.sk] == 0;
                     if (bbase) {      // scale * (s + bias / scale) = scale * s + bias
                         float bv = 0.f;
                         if (!drop && qi < p.Sq) {

@@ -318,6 +318,8 @@ int flame_attn_bwd_bf16(const void* Q, const void* K, const void* V, const void*
     p.m.sh = keep_mask ? mask_strides[1] : 0;
     p.m.sq = keep_mask ? mask_strides[2] : 0;
     p.m.sk = keep_mask ? mask_strides[3] : 0;
+    p.m.rows16 = keep_mask && p.m.sk == 1 && (reinterpret_cast<uintptr_t>(keep_mask) | (uintptr_t)p.m.sb | (uintptr_t)p.m.sh |
+                                              (uintptr_t)p.m.sq) % 16 == 0;
     p.m.causal = causal ? 1 : 0;
     p.phase_cycles = g_phase_cycles;
     hipStream_t s = static_cast<hipStream_t>(stream);
@@ -473,6 +475,8 @@ static int attn_fwd_impl(const void* Q, const void* K, const void* V, void* O, v
     p.m.sh = keep_mask ? mask_strides[1] : 0;
     p.m.sq = keep_mask ? mask_strides[2] : 0;
     p.m.sk = keep_mask ? mask_strides[3] : 0;
+    p.m.rows16 = keep_mask && p.m.sk == 1 && (reinterpret_cast<uintptr_t>(keep_mask) | (uintptr_t)p.m.sb | (uintptr_t)p.m.sh |
+                                              (uintptr_t)p.m.sq) % 16 == 0;
     p.m.causal = causal ? 1 : 0;
     p.m.bias = bias;
     if (bias) {
