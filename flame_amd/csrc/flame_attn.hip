@@ -806,9 +806,9 @@ int flame_attn_prep_rmsnorm_rope_bf16(const void* X, const void* weight, const v
     p.eps = eps;
     p.norm = apply_norm ? 1 : 0;
     p.table_f32 = table_dtype == FLAME_ATTN_DTYPE_F32;
-    const int64_t rows = (int64_t)B * H * N;
+    const int64_t items = (int64_t)B * N * ((H + kPrepHeadsPerThread - 1) / kPrepHeadsPerThread);   // (position, head group)
     const int rpb = 256 / (D / 8);
-    const int64_t grid = (rows + rpb - 1) / rpb;
+    const int64_t grid = (items + rpb - 1) / rpb;
     if (grid > 0x7fffffff) return FLAME_ATTN_ERR_UNSUPPORTED;
     hipStream_t s = static_cast<hipStream_t>(stream);
     {

@@ -10,7 +10,8 @@
 //   y[2p+1] = bf16( v[2p] * sin[n,p] + v[2p+1] * cos[n,p] )
 //
 // One row (D elements) is served by D/8 adjacent lanes, 8 elements = 4 rotation pairs per lane, so
-// loads and stores are 16 bytes per lane and the mean of squares is a butterfly over D/8 lanes.
+// loads and stores are 16 bytes per lane and the mean of squares is a butterfly over D/8 lanes; the same
+// lanes serve that position in several heads, which share its table entries.
 #pragma once
 #include "attn_common.hpp"
 
@@ -29,48 +30,30 @@ struct PrepParams {
     int table_f32;           // tables are fp32 (else bf16)
 };
 
+// Heads served by one thread: the rotation tables depend on the position only, so a thread loads its
+// four (cos, sin) pairs once and applies them to the same 8 elements of kPrepHeadsPerThread heads.
+constexpr int kPrepHeadsPerThread = 4;
+
 template <int D>
 __global__ __launch_bounds__(256) void prep_qk_kernel(const PrepParams p) {
     constexpr int LPR = D / 8;              // lanes per row
-    constexpr int RPB = 256 / LPR;          // rows per workgroup
+    constexpr int RPB = 256 / LPR;          // (position, head group) items per workgroup
+    constexpr int HPT = kPrepHeadsPerThread;
     const int tid = threadIdx.x;
     const int sub = tid % LPR;
-    const int64_t row = (int64_t)blockIdx.x * RPB + tid / LPR;      // output row index over (b, h, n)
-    const int64_t rows = (int64_t)p.B * p.H * p.N;
-    const bool ok = row < rows;
-    const int64_t r = ok ? row : rows - 1;
-    const int n = (int)(r % p.N);
-    const int64_t bh = r / p.N;
-    const int hh = (int)(bh % p.H), b = (int)(bh / p.H);
+    const int hgroups = (p.H + HPT - 1) / HPT;
+    const int64_t item = (int64_t)blockIdx.x * RPB + tid / LPR;     // index over (b, n, head group)
+    const int64_t items = (int64_t)p.B * p.N * hgroups;
+    if (item >= items) return;              // no barriers or cross-row exchanges follow (the butterfly stays inside a row's lanes,
+                                            // which leave together)
+    const int hg = (int)(item % hgroups);
+    const int64_t bn = item / hgroups;
+    const int n = (int)(bn % p.N), b = (int)(bn / p.N);
 
-    const u32x4 raw = *reinterpret_cast<const u32x4*>(p.x + b * p.xs.b + hh * p.xs.h + (int64_t)n * p.xs.n + 8 * sub);
-    float v[8];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        v[2 * i] = bf16_lo(raw[i]);
-        v[2 * i + 1] = bf16_hi(raw[i]);
-    }
-    if (p.norm) {
-        float ss = 0.f;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) ss = fmaf(v[i], v[i], ss);
-#pragma unroll
-        for (int off = LPR / 2; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
-        const float rs = rsqrtf(ss / (float)D + p.eps);
-        u32x4 wraw = {0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};      // bf16 ones
-        if (p.w) wraw = *reinterpret_cast<const u32x4*>(p.w + 8 * sub);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-#pragma clang fp contract(off)
-            // round to bf16 as the stand-alone normalisation kernel would, then carry on in fp32
-            const uint32_t packed = pack_bf16(v[2 * i] * rs * bf16_lo(wraw[i]), v[2 * i + 1] * rs * bf16_hi(wraw[i]));
-            v[2 * i] = bf16_lo(packed);
-            v[2 * i + 1] = bf16_hi(packed);
-        }
-    }
-    u32x4 out;
+    u32x4 wraw = {0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};      // bf16 ones
+    if (p.norm && p.w) wraw = *reinterpret_cast<const u32x4*>(p.w + 8 * sub);
+    float c[4], sn[4];
     if (p.cos_t) {
-        float c[4], s[4];
         const int64_t t0 = (int64_t)n * (D / 2) + 4 * sub;
         if (p.table_f32) {
             const f32x4 cv = *reinterpret_cast<const f32x4*>(static_cast<const float*>(p.cos_t) + t0);
@@ -78,7 +61,7 @@ __global__ __launch_bounds__(256) void prep_qk_kernel(const PrepParams p) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 c[i] = cv[i];
-                s[i] = sv[i];
+                sn[i] = sv[i];
             }
         } else {
             const u32x2 cv = *reinterpret_cast<const u32x2*>(static_cast<const uint16_t*>(p.cos_t) + t0);
@@ -87,24 +70,61 @@ __global__ __launch_bounds__(256) void prep_qk_kernel(const PrepParams p) {
             for (int i = 0; i < 2; ++i) {
                 c[2 * i] = bf16_lo(cv[i]);
                 c[2 * i + 1] = bf16_hi(cv[i]);
-                s[2 * i] = bf16_lo(sv[i]);
-                s[2 * i + 1] = bf16_hi(sv[i]);
+                sn[2 * i] = bf16_lo(sv[i]);
+                sn[2 * i + 1] = bf16_hi(sv[i]);
             }
         }
+    }
+
+    // all loads first, so that they are in flight together
+    u32x4 raw[HPT];
+#pragma unroll
+    for (int k = 0; k < HPT; ++k) {
+        const int hh = min(hg * HPT + k, p.H - 1);
+        raw[k] = *reinterpret_cast<const u32x4*>(p.x + b * p.xs.b + hh * p.xs.h + (int64_t)n * p.xs.n + 8 * sub);
+    }
+#pragma unroll
+    for (int k = 0; k < HPT; ++k) {
+        const int hh = hg * HPT + k;
+        float v[8];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            // plain fp32 arithmetic, every product and sum rounded on its own: no contraction into
-            // fused multiply-adds, so that the result does not depend on which product gets fused
-#pragma clang fp contract(off)
-            const float e = v[2 * i], o = v[2 * i + 1];
-            const float ec = e * c[i], os = o * s[i], es = e * s[i], oc = o * c[i];
-            out[i] = pack_bf16(ec - os, es + oc);
+            v[2 * i] = bf16_lo(raw[k][i]);
+            v[2 * i + 1] = bf16_hi(raw[k][i]);
         }
-    } else {
+        if (p.norm) {
+            float ss = 0.f;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) out[i] = pack_bf16(v[2 * i], v[2 * i + 1]);
+            for (int i = 0; i < 8; ++i) ss = fmaf(v[i], v[i], ss);
+#pragma unroll
+            for (int off = LPR / 2; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+            const float rs = rsqrtf(ss / (float)D + p.eps);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+#pragma clang fp contract(off)
+                // round to bf16 as the stand-alone normalisation kernel would, then carry on in fp32
+                const uint32_t packed = pack_bf16(v[2 * i] * rs * bf16_lo(wraw[i]), v[2 * i + 1] * rs * bf16_hi(wraw[i]));
+                v[2 * i] = bf16_lo(packed);
+                v[2 * i + 1] = bf16_hi(packed);
+            }
+        }
+        u32x4 out;
+        if (p.cos_t) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                // plain fp32 arithmetic, every product and sum rounded on its own: no contraction into
+                // fused multiply-adds, so that the result does not depend on which product gets fused
+#pragma clang fp contract(off)
+                const float e = v[2 * i], o = v[2 * i + 1];
+                const float ec = e * c[i], os = o * sn[i], es = e * sn[i], oc = o * c[i];
+                out[i] = pack_bf16(ec - os, es + oc);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) out[i] = pack_bf16(v[2 * i], v[2 * i + 1]);
+        }
+        if (hh < p.H) *reinterpret_cast<u32x4*>(p.y + b * p.ys.b + hh * p.ys.h + (int64_t)n * p.ys.n + 8 * sub) = out;
     }
-    if (ok) *reinterpret_cast<u32x4*>(p.y + b * p.ys.b + hh * p.ys.h + (int64_t)n * p.ys.n + 8 * sub) = out;
 }
 
 }  // namespace fattn
