@@ -193,6 +193,14 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
     return __builtin_bit_cast(uint32_t, b);
 }
 
+// Waits until at most N of this wavefront's LDS reads are outstanding (they return in order); the vector
+// memory and export counters are left alone.
+template <int N>
+__device__ __forceinline__ void wait_lds_reads() {
+    static_assert(N >= 0 && N < 16, "lgkmcnt is a 4-bit field");
+    __builtin_amdgcn_s_waitcnt(0xC07F | (N << 8));
+}
+
 __device__ __forceinline__ bf16x8 pack8(float a0, float a1, float a2, float a3, float a4, float a5, float a6,
                                         float a7) {
     u32x4 u = {pack_bf16(a0, a1), pack_bf16(a2, a3), pack_bf16(a4, a5), pack_bf16(a6, a7)};

@@ -628,15 +628,15 @@ __global__ __launch_bounds__(256) void fwd_wide_kernel(const FwdParams p) {
 #pragma unroll
         for (int qb = 0; qb < 2; ++qb) msc[qb] = ((m_run[qb] == -INFINITY) ? 0.f : m_run[qb]) * c_log2;
         u32x4 pw[2][4];                 // P^T operands: [query block][16-key chunk]
-        // exponentials of logits 2j, 2j + 1 (in (kb, r) order) of query block qb
-        auto exp_pair = [&](int qb, int j) {
-#pragma unroll
-            for (int e = 0; e < 2; ++e) {
-                const int idx = 2 * j + e, kb = idx >> 4, r = idx & 15;
-                cur[qb][kb][r] = exp2_fast(fmaf(cur[qb][kb][r], c_log2, -msc[qb]));
-            }
+        // exponential of logit idx (in (kb, r) order) of query block qb
+        auto exp_elem = [&](int qb, int idx) {
+            const int kb = idx >> 4, r = idx & 15;
+            cur[qb][kb][r] = exp2_fast(fmaf(cur[qb][kb][r], c_log2, -msc[qb]));
         };
-        // sums and packs a pair one slot after its exponentials, so that nothing waits on the transcendental unit
+        // Sums and packs a pair one slot after its exponentials, so that nothing waits on the transcendental
+        // unit.  (The row sum is taken over the unrounded values: summing the packed pair with one
+        // v_dot2_f32_bf16 would save an instruction per pair, but moves the logsumexp of a row that one key
+        // dominates by up to 2^-9.)
         auto pack_pair = [&](int qb, int j) {
             const int idx = 2 * j, kb = idx >> 4, r = idx & 15;
             rsum0[qb] += cur[qb][kb][r];
@@ -649,6 +649,10 @@ __global__ __launch_bounds__(256) void fwd_wide_kernel(const FwdParams p) {
             static_assert(NSL == 32 || NSL == 16, "slicing");
             // copies of K(t+3) and V(t+2); copy j goes with slot CS*j + 1
             constexpr int NCOPY = 2 * NDMA, CS = (NSL - 2) / NCOPY;
+            // exponentials per slot and query block: the first key block's in the logit phase, the second's
+            // in the first half of the other phase, whose slots have the vector unit to spare
+            constexpr int E1 = 16 / NKF, E2 = 32 / NVF;
+            static_assert(E1 >= 1 && E2 >= 2 && E2 % 2 == 0, "slicing");
             static_assert(CS >= 2, "copies do not fit the logit phase");
             auto copy_dst = [&](int g) {
                 const int j = (g - 1) / CS;
@@ -668,30 +672,37 @@ __global__ __launch_bounds__(256) void fwd_wide_kernel(const FwdParams p) {
                     constexpr int qb = decltype(qb_tag)::value;
                     constexpr int g = 2 * i + qb;
                     copy_dst(g);
+                    if (qb == 0 && !(i & 1)) {
+                        // one wait for the two fragments the ring read together; the pair read after them stays in flight
+                        constexpr int younger = (i + 2 < NKF ? 1 : 2) + (i + 3 < NKF ? 1 : 2);
+                        wait_lds_reads<younger>();
+                    }
                     mfma32_vgpr_bpinned<qb * DC + (i >> 1), (i >> 1) == 0 ? 0 : 1>(nxt[qb][i & 1], fb[i % PD], qf[qb][i >> 1], nxt[qb][i & 1]);
                     __builtin_amdgcn_sched_barrier(0);
                     copy_issue(g);
-                    // slot g: exponentials of pairs of query block qb, packing of the pairs of the slot before
-                    constexpr int PPS = 32 / NSL;        // pairs per slot and block: 1 or 2
+                    // slot g: exponentials of E1 logits of the first key block of query block qb, packing of
+                    // the pairs that were complete a slot ago
 #pragma unroll
-                    for (int e = 0; e < PPS; ++e) exp_pair(qb, PPS * i + e);
+                    for (int e = 0; e < E1; ++e) exp_elem(qb, E1 * i + e);
                     if (i > 0) {
 #pragma unroll
-                        for (int e = 0; e < PPS; ++e) pack_pair(qb, PPS * (i - 1) + e);
+                        for (int j = E1 * (i - 1) / 2; j < E1 * i / 2; ++j) pack_pair(qb, j);
                     }
-                    if (qb == 1) {
-                        if (i + PD < NKF) fb[i % PD] = k_frag(stage_t1, i + PD);
-                        else fb[i % PD] = v_frag(stage_t, i + PD - NKF);
+                    // the ring is refilled two fragments at a time, so that one wait covers both
+                    if (qb == 1 && (i & 1)) {
+#pragma unroll
+                        for (int f = i - 1; f <= i; ++f) {
+                            if (f + PD < NKF) fb[f % PD] = k_frag(stage_t1, f + PD);
+                            else fb[f % PD] = v_frag(stage_t, f + PD - NKF);
+                        }
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 });
             });
 #pragma unroll
             for (int qb = 0; qb < 2; ++qb) {
-                constexpr int PPS = 32 / NSL;
 #pragma unroll
-                for (int e = 0; e < PPS; ++e) pack_pair(qb, PPS * (NKF - 1) + e);
-                l_run[qb] += rsum0[qb] + rsum1[qb];
+                for (int j = E1 * (NKF - 1) / 2; j < 8; ++j) pack_pair(qb, j);
             }
             // ---- O^T += V(t)^T P(t)^T between the row-maximum scan of tile t+1
             float tmax[2];
@@ -702,18 +713,34 @@ __global__ __launch_bounds__(256) void fwd_wide_kernel(const FwdParams p) {
                 static_for<2>([&](auto qb_tag) {
                     constexpr int qb = decltype(qb_tag)::value;
                     constexpr int g = 2 * i + qb;
+                    if (qb == 0 && !(i & 1)) {
+                        constexpr int younger = (i + 2 < NVF ? 2 : 1) + (i + 3 < NVF ? 2 : 1);
+                        wait_lds_reads<younger>();
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
                     oacc[qb][db] = mfma32(fb[i % PD], __builtin_bit_cast(bf16x8, pw[qb][cc]), oacc[qb][db]);
                     __builtin_amdgcn_sched_barrier(0);
-                    // the logits of tile t+1 may be touched from slot 2 on
-                    if (g == 2 + qb) tmax[qb] = nxt[qb][0][0];
-                    if (g >= 2 + qb) {
-                        constexpr int MPS = (32 + (NPV - 2) / 2 - 1) / ((NPV - 2) / 2);     // logits per slot and block
-                        constexpr int k = (g - 2 - qb) / 2;
+                    if (i < NVF / 2) {
+                        // first half: the exponentials of the second key block, due at slot NVF / 2
+#pragma unroll
+                        for (int e = 0; e < E2; ++e) exp_elem(qb, 16 + E2 * i + e);
+                    }
+                    if (i >= 1 && i <= NVF / 2) {
+#pragma unroll
+                        for (int j = 8 + E2 * (i - 1) / 2; j < 8 + E2 * i / 2; ++j) pack_pair(qb, j);
+                    }
+                    if (i >= NVF / 2) {
+                        // second half: row maximum of tile t+1 (its logits may be touched from slot 2 on)
+                        constexpr int MPS = 64 / NVF;     // logits per slot and block
+                        constexpr int k = i - NVF / 2;
+                        if (k == 0) tmax[qb] = nxt[qb][0][0];
 #pragma unroll
                         for (int e = 0; e < MPS; ++e) {
-                            const int idx = 1 + MPS * k + e;
-                            if (idx < 32) tmax[qb] = fmaxf(tmax[qb], nxt[qb][idx >> 4][idx & 15]);
+                            const int idx = MPS * k + e;
+                            tmax[qb] = fmaxf(tmax[qb], nxt[qb][idx >> 4][idx & 15]);
                         }
+                        // the scan feeds nothing before the end of the step: keep this slot's part in this slot
+                        asm volatile("" : "+v"(tmax[qb]));
                     }
                     if (qb == 1) {
                         if (i == NVF - PD) {
@@ -723,12 +750,19 @@ __global__ __launch_bounds__(256) void fwd_wide_kernel(const FwdParams p) {
                             __builtin_amdgcn_s_barrier();    // ... for every wave, and every wave is past tile t-1
                             __builtin_amdgcn_sched_barrier(0);
                         }
-                        if (i + PD < NVF) fb[i % PD] = v_frag(stage_t, i + PD);
-                        else fb[i % PD] = k_frag(stage_t2, i + PD - NVF);
+                        if (i & 1) {
+#pragma unroll
+                            for (int f = i - 1; f <= i; ++f) {
+                                if (f + PD < NVF) fb[f % PD] = v_frag(stage_t, f + PD);
+                                else fb[f % PD] = k_frag(stage_t2, f + PD - NVF);
+                            }
+                        }
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 });
             });
+#pragma unroll
+            for (int qb = 0; qb < 2; ++qb) l_run[qb] += rsum0[qb] + rsum1[qb];
             // Both lanes of a query hold the same reference maximum, so each may test its own half; the
             // exchange between the halves and the rescale stay inside the rarely taken branch.
             if (__any(tmax[0] > m_run[0] + stale_ok || tmax[1] > m_run[1] + stale_ok)) {
@@ -760,23 +794,25 @@ __global__ __launch_bounds__(256) void fwd_wide_kernel(const FwdParams p) {
         using I2 = std::integral_constant<int, 2>;
         using I3 = std::integral_constant<int, 3>;
         // Tile t sits in stage t % 4 and its logits in `sa` when t is even: four step bodies.
-        const uint16_t *k3, *v2;
-        auto bases = [&](int t) {      // copies past the last tile re-read the last tile
-            k3 = kbase + (int64_t)min(t + 3, n_tiles - 1) * k_tile_stride;
-            v2 = vbase + (int64_t)min(t + 2, n_tiles - 1) * v_tile_stride;
+        // K(t+3) and V(t+2) of the step at hand; copies past the last tile re-read the last tile
+        const uint16_t* k3 = kbase + (int64_t)min(3, n_tiles - 1) * k_tile_stride;
+        const uint16_t* v2 = vbase + (int64_t)min(2, n_tiles - 1) * v_tile_stride;
+        auto advance = [&](int t) {    // from step t to step t+1
+            k3 += (t + 4 < n_tiles) ? k_tile_stride : 0;
+            v2 += (t + 3 < n_tiles) ? v_tile_stride : 0;
         };
         for (int t = 0; t < n_tiles; t += 4) {
-            bases(t);
             step(I0{}, sa, sb, k3, v2);
             if (t + 1 >= n_tiles) break;
-            bases(t + 1);
+            advance(t);
             step(I1{}, sb, sa, k3, v2);
             if (t + 2 >= n_tiles) break;
-            bases(t + 2);
+            advance(t + 1);
             step(I2{}, sa, sb, k3, v2);
             if (t + 3 >= n_tiles) break;
-            bases(t + 3);
+            advance(t + 2);
             step(I3{}, sb, sa, k3, v2);
+            advance(t + 3);
         }
         wait_vm0();          // no copy may land after the workgroup has gone
     }
