@@ -614,8 +614,10 @@ __global__ __launch_bounds__(256) void fwd_wide_kernel(const FwdParams p) {
 
     bf16x8 fb[PD];
     // One step: P(t) from the logits in `cur`, logits of tile t+1 into `nxt`, O += P(t) V(t).  MFMA slot
-    // = 2 * fragment + query block.  The exponentials of tile t are threaded between the logit MFMAs of
-    // tile t+1, the row-maximum scan of tile t+1 between the MFMAs of O += P(t) V(t).
+    // = 2 * fragment + query block.  The exponentials of the first key block of tile t are threaded between
+    // the logit MFMAs of tile t+1; those of the second key block (needed from the middle of the PV products
+    // on) between the first half of the MFMAs of O += P(t) V(t), the row-maximum scan of tile t+1 between
+    // the second half: the wavefront is bound by instruction issue, so every slot gets its share.
     // STAGE: stage of tile t (0 .. 3).  k3_base / v2_base: tiles t+3 of K and t+2 of V (clamped).
     auto step = [&](auto stage_tag, f32x16 (&cur)[2][2], f32x16 (&nxt)[2][2], const uint16_t* k3_base,
                     const uint16_t* v2_base) {
