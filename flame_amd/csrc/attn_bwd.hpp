@@ -429,7 +429,7 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
         if (COPY == 2 && have_next && !next_full) issue_q_tile(qt_next, nxt);   // partial tile: slow path, all at once
 
         // The element-wise work of a block trails the hand-emitted MFMAs that produced its S and dP by
-        // LAG MFMA slots (see mfma32_vgpr), so its last LAG slices run at the start of the phase after.
+        // LAG MFMA slots (see mfma32_vgpr_bacc), so its last LAG slices run at the start of the phase after.
         constexpr int LAG = 2;
         auto side = [&](int g) {
             const int phase = g / NS, i = g % NS;
@@ -944,7 +944,7 @@ __global__ __launch_bounds__(64 * NW, (NW == 4 && !HASMASK) ? 2 : 1) void bwd_dq
 // feeds two MFMAs (one per query block), which halves the LDS reads and waits per MFMA; the register
 // file of a lone wavefront holds dQ^T of both blocks and the Q / dO fragments in the accumulation
 // registers (Q / dO as MFMA B operands), and S^T / dP^T in architectural registers through hand-emitted
-// MFMAs (see mfma32_vgpr).  dP^T starts from -delta, so dS^T = P^T * dP'^T is one multiply.
+// MFMAs (see mfma32_vgpr_bacc).  dP^T starts from -delta, so dS^T = P^T * dP'^T is one multiply.
 // Three LDS stages of K / V tiles, one barrier per tile, one ring of fragment reads that runs on into
 // the next tile, copies split around MFMAs and spread over the tile: as in bwd_dkdv_kernel.
 // No explicit keep-mask variant: such problems use bwd_dq_kernel.

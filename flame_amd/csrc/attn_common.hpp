@@ -42,21 +42,15 @@ __device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
 // Emitted by hand, so the compiler's hazard bookkeeping does not see it.  The caller must keep at
 // least two other MFMAs between the last of these writing an accumulator and the first vector-ALU
 // instruction that touches it (the result of an 8-pass MFMA is visible 11 issue cycles after issue).
-__device__ __forceinline__ void mfma32_vgpr_first(f32x16& acc, bf16x8 a, bf16x8 b) {
-    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(acc) : "v"(a), "v"(b));
-}
-__device__ __forceinline__ void mfma32_vgpr(f32x16& acc, bf16x8 a, bf16x8 b) {
-    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
-}
-// The same two with the B operand held in the accumulation registers: operands that live for a whole
-// kernel (a workgroup's own K / V fragments) then cost no architectural VGPRs.
+// The B operand is held in the accumulation registers: operands that live for a whole kernel (a
+// workgroup's own K / V fragments) then cost no architectural VGPRs.
 __device__ __forceinline__ void mfma32_vgpr_first_bacc(f32x16& acc, bf16x8 a, bf16x8 b) {
     asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(acc) : "v"(a), "a"(b));
 }
 __device__ __forceinline__ void mfma32_vgpr_bacc(f32x16& acc, bf16x8 a, bf16x8 b) {
     asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "a"(b));
 }
-// The same three with the B operand pinned to accumulation registers a[128 + 4 SLOT : 131 + 4 SLOT], for a
+// The same with the B operand pinned to accumulation registers a[128 + 4 SLOT : 131 + 4 SLOT], for a
 // kernel whose 32 resident B fragments must stay put there (left to itself the register allocator
 // homes some of them in architectural registers and copies them over before every use).
 // MODE 0: acc = a b; 1: acc += a b; 2: acc = c + a b.

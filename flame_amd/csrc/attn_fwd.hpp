@@ -436,7 +436,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void fwd_kernel(const Fwd
 // SIMD: 4 wavefronts of 64 queries (two 32-query blocks) each, so that every K / V fragment read from
 // LDS feeds two MFMAs and the LDS reads and waits per MFMA halve.  O^T of both blocks and the Q
 // fragments live in the accumulation registers (Q as pinned MFMA B operands), the logits in
-// architectural registers through hand-emitted MFMAs (see mfma32_vgpr): nothing may touch them until
+// architectural registers through hand-emitted MFMAs (see mfma32_vgpr_bacc): nothing may touch them until
 // two further MFMAs have been issued.  Four LDS stages, K(t) and V(t) in stage t % 4: step t reads
 // K(t+1) and V(t) and issues the copies of K(t+3) and V(t+2), each into a slot whose previous tile was
 // last read two barriers ago, and each with more than a full step to land; one workgroup barrier
@@ -706,15 +706,13 @@ __global__ __launch_bounds__(256) void fwd_wide_kernel(const FwdParams p) {
 #pragma unroll
                 for (int j = E1 * (NKF - 1) / 2; j < 8; ++j) pack_pair(qb, j);
             }
-            // ---- O^T += V(t)^T P(t)^T between the row-maximum scan of tile t+1
+            // ---- O^T += V(t)^T P(t)^T, with the rest of the exponentials and the row-maximum scan of tile t+1
             float tmax[2];
-            constexpr int NPV = 2 * NVF;             // MFMA slots of this phase
             static_for<NVF>([&](auto i_tag) {
                 constexpr int i = decltype(i_tag)::value;
                 constexpr int cc = i / DB, db = i % DB;
                 static_for<2>([&](auto qb_tag) {
                     constexpr int qb = decltype(qb_tag)::value;
-                    constexpr int g = 2 * i + qb;
                     if (qb == 0 && !(i & 1)) {
                         constexpr int younger = (i + 2 < NVF ? 2 : 1) + (i + 3 < NVF ? 2 : 1);
                         wait_lds_reads<younger>();
