@@ -48,8 +48,13 @@ struct FwdTile {
     static constexpr int DMA_PER_WAVE = BN / ROWS_PER_DMA / 4;   // copies per wave and tensor
 };
 
-template <int D, bool HASMASK, int NW>
+// VECMASK (with HASMASK): the only exclusions besides key lengths and the causal flag come from a keep-mask
+// whose rows are contiguous and 16-byte aligned, Sk is a multiple of the tile and there is no bias; the
+// general exclusion code (per-element loads, bias) is then not compiled in, which frees the registers
+// that made the general masked kernel spill.
+template <int D, bool HASMASK, int NW, bool VECMASK = false>
 __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void fwd_kernel(const FwdParams p) {
+    static_assert(!VECMASK || HASMASK, "VECMASK is a special case of HASMASK");
     using T = FwdTile<D>;
     constexpr int BN = T::BN, RS = T::RS;
     constexpr int BM = 32 * NW;  // query rows per workgroup
@@ -186,6 +191,20 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void fwd_kernel(const Fwd
     // exclusions of tile t: ragged tail / key length, causal, explicit keep-mask
     auto apply_mask = [&](f32x16 (&s)[2], int t) {
         const int qi = qw0 + n;
+        if constexpr (VECMASK) {
+            MaskRow64 mrow;
+            mrow.load(mbase + (int64_t)min(qi, p.Sq - 1) * p.m.sq + t * BN);
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int key = t * BN + 32 * kb + acc_row(r, h);
+                    bool drop = key >= klimit || !mrow.keep(kb, r, h);
+                    if (p.m.causal) drop = drop || key > qi;
+                    s[kb][r] = drop ? -INFINITY : s[kb][r];
+                }
+            return;
+        }
         // a lane's 64 keep-mask bytes of the tile in four 16-byte loads where the layout allows it (each
         // lane owns a query row, so byte loads would touch one cache line per lane and element)
         const bool vec_mask = HASMASK && mbase && p.m.rows16 && t * BN + BN <= p.Sk;

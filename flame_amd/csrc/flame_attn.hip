@@ -85,12 +85,12 @@ struct ScopedKernelTimer {
     }
 };
 
-template <int D, bool HASMASK, int NW>
+template <int D, bool HASMASK, int NW, bool VECMASK = false>
 int launch_fwd(const FwdParams& p, hipStream_t s) {
     using T = FwdTile<D>;
     constexpr int BM = 32 * NW;
     static bool attr_done = false;   // idempotent, so a benign race at worst repeats the call
-    auto kern = fwd_kernel<D, HASMASK, NW>;
+    auto kern = fwd_kernel<D, HASMASK, NW, VECMASK>;
     if (!attr_done) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS_BYTES);
@@ -494,6 +494,9 @@ static int attn_fwd_impl(const void* Q, const void* K, const void* V, void* O, v
                       env_int("FLAME_ATTN_WG_WAVES", 8) != 4;      // FLAME_ATTN_WG_WAVES=4 forces 128-query workgroups
     // ... as 4 wavefronts of 64 queries when nothing is excluded at all, else as 8 wavefronts of 32
     const bool plain = !causal && kv_len == nullptr && N_kv % 64 == 0;
+    // a keep-mask with vector-loadable rows over whole tiles and no bias: the lean masked kernel
+    if (keep_mask != nullptr && bias == nullptr && p.m.rows16 && N_kv % 64 == 0)
+        return D == 128 ? launch_fwd<128, true, 4, true>(p, s) : launch_fwd<64, true, 4, true>(p, s);
     if (D == 128)
         return hm ? launch_fwd<128, true, 4>(p, s)
                   : wide ? (plain ? launch_fwd_wide<128>(p, s) : launch_fwd<128, false, 8>(p, s)) : launch_fwd<128, false, 4>(p, s);
