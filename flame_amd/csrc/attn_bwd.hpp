@@ -648,8 +648,11 @@ struct BwdDqTile {
 
 // NW wavefronts of 32 queries each per workgroup, two per SIMD (the library instantiates NW = 4; problems
 // that fill 256-query workgroups go to bwd_dq_wide_kernel below).
-template <int D, bool HASMASK, int NW>
-__global__ __launch_bounds__(64 * NW, (NW == 4 && !HASMASK) ? 2 : 1) void bwd_dq_kernel(const BwdParams p) {
+// VECMASK (with HASMASK): the keep-mask rows are contiguous and 16-byte aligned and Sk is a multiple of the
+// tile, so the per-element mask loads are not compiled in and the kernel fits two workgroups per unit again.
+template <int D, bool HASMASK, int NW, bool VECMASK = false>
+__global__ __launch_bounds__(64 * NW, (NW == 4 && (!HASMASK || VECMASK)) ? 2 : 1) void bwd_dq_kernel(const BwdParams p) {
+    static_assert(!VECMASK || HASMASK, "VECMASK is a special case of HASMASK");
     using T = BwdDqTile<D>;
     constexpr int BM = 32 * NW, BN = T::BN, RS = T::RS;
     constexpr int DC = D / 16;
@@ -780,7 +783,7 @@ __global__ __launch_bounds__(64 * NW, (NW == 4 && !HASMASK) ? 2 : 1) void bwd_dq
     MaskRow64 mnext;          // keep-mask bytes of this lane's query row for the next tile (vector-load layouts only)
 #pragma unroll
     for (int j = 0; j < 4; ++j) mnext.w[j] = u32x4{0u, 0u, 0u, 0u};
-    if (HASMASK && p.m.rows16 && n_tiles > 0 && BN <= p.Sk) mnext.load(mbase + (int64_t)min(qrow, p.Sq - 1) * p.m.sq);
+    if (HASMASK && !VECMASK && p.m.rows16 && n_tiles > 0 && BN <= p.Sk) mnext.load(mbase + (int64_t)min(qrow, p.Sq - 1) * p.m.sq);
     wait_vm0();
     __syncthreads();
 
@@ -828,16 +831,23 @@ __global__ __launch_bounds__(64 * NW, (NW == 4 && !HASMASK) ? 2 : 1) void bwd_dq
         // a lane's 64 keep-mask bytes of the tile in four 16-byte loads where the layout allows it, fetched
         // one tile ahead
         const bool vec_mask = HASMASK && MASKED && p.m.rows16 && key0 + BN <= p.Sk;
-        const MaskRow64 mrow = mnext;
-        if (HASMASK && MASKED && p.m.rows16 && key0 + 2 * BN <= p.Sk && t + 1 < n_tiles)
+        MaskRow64 mrow = mnext;
+        if constexpr (VECMASK) {
+            // two workgroups per unit: the other wavefront of the SIMD covers the load, and a second row in
+            // registers would spill
+            mrow.load(mbase + (int64_t)min(qrow, p.Sq - 1) * p.m.sq + key0);
+        } else if (HASMASK && MASKED && p.m.rows16 && key0 + 2 * BN <= p.Sk && t + 1 < n_tiles) {
             mnext.load(mbase + (int64_t)min(qrow, p.Sq - 1) * p.m.sq + key0 + BN);
+        }
         auto p_elem = [&](int kb, int r) {          // P^T: one query per lane, so LSE is a per-lane scalar
             float pr = exp2_fast(fmaf(sacc[kb][r], c_log2, -lse2));
             if (MASKED) {
                 const int key = key0 + 32 * kb + acc_row(r, h);
                 bool drop = key >= klimit;
                 if (p.m.causal) drop = drop || key > qrow;
-                if (HASMASK) {
+                if constexpr (VECMASK) {
+                    drop = drop || !mrow.keep(kb, r, h);
+                } else if (HASMASK) {
                     if (vec_mask) drop = drop || !mrow.keep(kb, r, h);
                     else if (!drop && qok) drop = mbase[(int64_t)qrow * p.m.sq + (int64_t)key * p.m.sk] == 0;
                 }

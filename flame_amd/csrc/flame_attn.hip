@@ -158,6 +158,7 @@ int launch_bwd(const BwdParams& p, hipStream_t s) {
     static bool attr_done = false;
     auto kern = bwd_dkdv_kernel<D, HASMASK, TIMING>;
     auto kern_dq = bwd_dq_kernel<D, HASMASK, 4>;
+    auto kern_dqv = bwd_dq_kernel<D, true, 4, true>;                 // keep-mask with vector-loadable rows over whole tiles
     using TW = BwdDqWideTile<D>;
     auto kern_dqw = bwd_dq_wide_kernel<D>;                           // 256-query workgroups, builds without a keep-mask only
     if (!attr_done) {
@@ -170,6 +171,11 @@ int launch_bwd(const BwdParams& p, hipStream_t s) {
         e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern_dqw),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, TW::LDS_BYTES);
         if (e != hipSuccess) return (int)e;
+        if (HASMASK) {
+            e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern_dqv),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, TQ::LDS_BYTES);
+            if (e != hipSuccess) return (int)e;
+        }
         attr_done = true;
     }
     const int64_t n_kt = (p.Sk + T::BN - 1) / T::BN;
@@ -186,6 +192,7 @@ int launch_bwd(const BwdParams& p, hipStream_t s) {
     {
         ScopedKernelTimer t(FLAME_ATTN_KERNEL_BWD_DQ, s);
         if (wide) hipLaunchKernelGGL(kern_dqw, dim3((unsigned)grid_dq), dim3(256), TW::LDS_BYTES, s, p);
+        else if (HASMASK && p.m.rows16 && p.Sk % TQ::BN == 0) hipLaunchKernelGGL(kern_dqv, dim3((unsigned)grid_dq), dim3(256), TQ::LDS_BYTES, s, p);
         else hipLaunchKernelGGL(kern_dq, dim3((unsigned)grid_dq), dim3(256), TQ::LDS_BYTES, s, p);
     }
     // The dK/dV kernel keeps one workgroup per compute unit.  When the key blocks do not fill the last
