@@ -68,6 +68,9 @@ struct BwdTile {
     static constexpr int NSTAGE = 3;
     // [3 stages of Q,dO][3 x (lse2, -delta)]
     static constexpr int LDS_BYTES = NSTAGE * STAGE_ELEMS * 2 + NSTAGE * ROW_FLOATS * 4;
+    // with a keep-mask staged through LDS: [3 x (64 queries x 128 keys) mask bytes] behind the rest
+    static constexpr int MASK_STAGE_BYTES = BM * BN;
+    static constexpr int LDS_BYTES_VECMASK = LDS_BYTES + NSTAGE * MASK_STAGE_BYTES;
     static constexpr int ROWS_PER_DMA = 1024 / (D * 2);
     static constexpr int DMA_PER_WAVE = BM / ROWS_PER_DMA / 4;    // 1 KiB copies per wave and tensor
 };
@@ -76,8 +79,14 @@ template <int D>
 __device__ __forceinline__ void dkdv_store(const BwdParams& p, const f32x16 (&dkacc)[D / 32], const f32x16 (&dvacc)[D / 32],
                                            int b, int hh, int krow, int h);
 
-template <int D, bool HASMASK, bool TIMING>
+// VECMASK (with HASMASK): the keep-mask rows are contiguous and 16-byte aligned, Sq is a multiple of 64, Sk
+// of 128, and there is no causal flag.  The 64 x 128 mask bytes of a step then travel to LDS with the step's other copies (two more
+// 1 KiB copies per wavefront) and every lane reads the bytes of its key a few elements ahead of use,
+// instead of fetching 32 bytes from global memory into 32 registers at the start of every step; with the
+// registers back, the walk runs the same straight-line steps as the unmasked one.
+template <int D, bool HASMASK, bool TIMING, bool VECMASK = false>
 __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
+    static_assert(!VECMASK || HASMASK, "VECMASK is a special case of HASMASK");
     using T = BwdTile<D>;
     constexpr int BM = T::BM, BN = T::BN, RS = T::RS;
     constexpr int DC = D / 16;     // contraction chunks over the head dim
@@ -88,6 +97,7 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
     extern __shared__ __attribute__((aligned(1024))) uint16_t lds[];
     uint16_t* stage0 = lds;                                        // [3][Q tile | dO tile]
     float* rows0 = reinterpret_cast<float*>(lds + T::NSTAGE * T::STAGE_ELEMS);   // [3][lse2 | -delta]
+    const uint8_t* mask0 = reinterpret_cast<const uint8_t*>(lds) + T::LDS_BYTES;  // [3][64 x 128] mask bytes (VECMASK)
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -206,6 +216,17 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
         return lds0 + 2u * (uint32_t)(stg * T::STAGE_ELEMS + which * T::Q_ELEMS + (wave * NDQ + i) * 512);
     };
     auto rows_dst = [&](int stg) { return rows_lds0 + 4u * (uint32_t)(stg * T::ROW_FLOATS + wave * BM); };
+    // keep-mask tile of a step: 8 copies of 8 rows x 128 bytes, two per wavefront
+    uint32_t m_lane_off[2] = {0u, 0u};
+    if (VECMASK) {
+#pragma unroll
+        for (int jm = 0; jm < 2; ++jm)
+            m_lane_off[jm] = (uint32_t)(((wave * 2 + jm) * 8 + (lane >> 3)) * (int)p.m.sq + 16 * (lane & 7));
+    }
+    auto mask_dst = [&](int stg, int jm) {
+        return lds0 + (uint32_t)(T::LDS_BYTES + stg * T::MASK_STAGE_BYTES + (wave * 2 + jm) * 1024);
+    };
+    auto mask_tile = [&](int qt) { return mbase + (int64_t)qt * BM * p.m.sq + k0; };
     auto issue_q_tile = [&](int qt, int stg) {
         const int q0 = qt * BM;
         if (q0 + BM <= p.Sq) {
@@ -217,6 +238,10 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
                 dma16u(dot_base, do_lane_off[i], q_dst(stg, 1, i));
             }
             if (wave < 2) dma4((wave == 0 ? lsebase : ndeltabase) + q0 + lane, rows_dst(stg));
+            if (VECMASK) {
+#pragma unroll
+                for (int jm = 0; jm < 2; ++jm) dma16u(mask_tile(qt), m_lane_off[jm], mask_dst(stg, jm));
+            }
         } else {   // last, partial tile: rows past the end re-read the last valid row
 #pragma unroll
             for (int i = 0; i < NDQ; ++i) {
@@ -245,6 +270,8 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
 
     const float c_log2 = p.scale * kLog2e;
     const int key = kw0 + n;
+    // VECMASK: a mask byte excludes its element when it is <= this: 0 for an attended key, 255 for one past the key length
+    const uint32_t dead_thr = key >= klimit ? 0xffu : 0u;
 
     unsigned long long ph[6] = {0, 0, 0, 0, 0, 0};
     unsigned long long tprev = TIMING ? __builtin_readcyclecounter() : 0ull;
@@ -278,7 +305,8 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
     constexpr int G = 4 * NS;       // MFMAs = operand fragments per step
     constexpr int PD = 4;           // read-ahead depth of the fragment ring
     static_assert(2 * DC == 4 * DB, "all phases must have the same number of MFMA slots");
-    static_assert(NS % PD == 0 && 4 * (2 * NDQ) + 1 < G - PD, "ring depth / copy slices do not fit");
+    constexpr int NCOPY = 2 * NDQ + 1 + (VECMASK ? 2 : 0);     // copies per wavefront and step: Q, dO, a row, mask
+    static_assert(NS % PD == 0 && 4 * (NCOPY - 1) + 1 < G - PD, "ring depth / copy slices do not fit");
     f32x16 dpacc[2];
     bf16x8 fb[PD];
     // fragment g of a step: [0, 2 NS) 16-byte row reads (block, dc, Q | dO); [2 NS, 4 NS) transposing
@@ -307,7 +335,8 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
     // stage from a run-time counter) leave the counter at 0 for the main loop, whose three unrolled
     // steps have their stages fixed at compile time.
     const int n_masked_here = max(min(n_masked, it_hi) - it_lo, 0);
-    int st = (3 - n_masked_here % 3) % 3;        // LDS stage of the step about to run
+    // (VECMASK: every step needs exclusions and the straight-line loop comes first, so it starts in stage 0)
+    int st = VECMASK ? 0 : (3 - n_masked_here % 3) % 3;        // LDS stage of the step about to run
     if (it_hi > it_lo) {
         issue_q_tile(tile_of(it_lo), st);
         wait_vm0();
@@ -342,7 +371,7 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
         // keep-mask bytes of this lane's key for the 64 queries of the tile, fetched up front in one batch
         // (a load per element inside the pipelined slices would wait out a memory round trip each time)
         uint32_t mk[2][16];
-        if (HASMASK && MASKED) {
+        if (HASMASK && !VECMASK && MASKED) {
             const uint8_t* mkey = mbase + (int64_t)min(key, p.Sk - 1) * p.m.sk;
 #pragma unroll
             for (int qb = 0; qb < 2; ++qb)
@@ -354,7 +383,17 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
         }
         // lse2 is read one group of four queries ahead of its use, so that waiting for it never drains
         // the fragment reads that were issued in between
-        auto rows_ahead = [&](int qb, int g) { l4n = *reinterpret_cast<const f32x4*>(rows_c + 32 * qb + 8 * g + 4 * h); };
+        // (VECMASK: and with it the four mask bytes of this lane's key for those queries)
+        const uint8_t* mask_c = mask0 + cur * T::MASK_STAGE_BYTES + (4 * h) * BN + 32 * wave + n;
+        const uint8_t* nm_base = VECMASK ? mask_tile(qt_next) : nullptr;
+        uint32_t m4[4], m4n[4];
+        auto rows_ahead = [&](int qb, int g) {
+            l4n = *reinterpret_cast<const f32x4*>(rows_c + 32 * qb + 8 * g + 4 * h);
+            if (VECMASK) {
+#pragma unroll
+                for (int t = 0; t < 4; ++t) m4n[t] = mask_c[(32 * qb + 8 * g + t) * BN];
+            }
+        };
 
         // element r of block qb: P = exp2(S*c - lse2), dS = P*(dP - delta); pack after 8 and 16.
         // The product for element r is issued with the exponential of element r + 1, so that no
@@ -371,6 +410,10 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
             const int g = r >> 2, t = r & 3;
             if (t == 0) {
                 l4 = l4n;
+                if (VECMASK) {
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) m4[u] = m4n[u];
+                }
                 if (g < 3) rows_ahead(qb, g + 1);
                 else if (qb == 0) rows_ahead(1, 0);
             }
@@ -378,9 +421,14 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
             if (r > 0) ds_mul(qb, r - 1);
             if (MASKED) {
                 const int qi = q0 + 32 * qb + 8 * g + 4 * h + t;
-                bool drop = key >= klimit || qi >= p.Sq;
-                if (p.m.causal) drop = drop || key > qi;
-                if (HASMASK) drop = drop || mk[qb][r] == 0;
+                bool drop;
+                if constexpr (VECMASK) {
+                    drop = m4[t] <= dead_thr;       // whole tiles, no causal flag: the mask byte decides, one compare
+                } else {
+                    // bitwise, not short-circuit: one select per element instead of a chain of branches
+                    drop = (key >= klimit) | (qi >= p.Sq) | ((p.m.causal != 0) & (key > qi));
+                    if (HASMASK) drop |= mk[qb][r] == 0;
+                }
                 pr = drop ? 0.f : pr;
             }
             sacc[qb][r] = pr;
@@ -415,13 +463,14 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
         };
         auto copy_issue = [&](int g) {
             const int j = g / 4;
-            if (COPY == 0 || g % 4 != 1 || j > 2 * NDQ) return;
+            if (COPY == 0 || g % 4 != 1 || j >= NCOPY) return;
             if (COPY == 1 && g < 2 * NS) {
                 if (j == 2 * NDQ) dma4u_issue(nrow_base, 4u * (uint32_t)lane);
                 else if (j & 1) dma16u_issue(ndo_base, do_lane_off[j >> 1]);
                 else dma16u_issue(nq_base, q_lane_off[j >> 1]);
             } else if (copying) {          // destination and copy in one piece
-                if (j == 2 * NDQ) dma4(nrow_base + lane, copy_dst_of(j));
+                if (j > 2 * NDQ) dma16u(nm_base, m_lane_off[j - 2 * NDQ - 1], mask_dst(nxt, j - 2 * NDQ - 1));
+                else if (j == 2 * NDQ) dma4(nrow_base + lane, copy_dst_of(j));
                 else if (j & 1) dma16u(ndo_base, do_lane_off[j >> 1], copy_dst_of(j));
                 else dma16u(nq_base, q_lane_off[j >> 1], copy_dst_of(j));
             }
@@ -505,7 +554,24 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
     using I2 = std::integral_constant<int, 2>;
     const int64_t q_tile_stride = (int64_t)BM * p.qs.n, do_tile_stride = (int64_t)BM * p.dos.n;
     const float* rowbase = (wave & 1) ? ndeltabase : lsebase;
-    for (int it = it_lo; it < n_masked_here + it_lo; ++it) {
+    int it_m = it_lo;
+    if constexpr (VECMASK) {
+        // Every tile needs exclusions, all are whole and consecutive: the same three straight-line steps
+        // with fixed stages as the unmasked loop below.
+        int qt = qt_begin + it_m;
+        const uint16_t* nq = qbase + (qt + 1) * q_tile_stride;
+        const uint16_t* ndo = dobase + (qt + 1) * do_tile_stride;
+        const float* nrow = rowbase + (qt + 1) * BM;
+        for (; it_m + 3 <= it_hi - 1; it_m += 3, qt += 3) {
+            step(std::true_type{}, I1{}, I0{}, 0, it_m, qt, qt + 1, nq, ndo, nrow);
+            nq += q_tile_stride, ndo += do_tile_stride, nrow += BM;
+            step(std::true_type{}, I1{}, I1{}, 1, it_m + 1, qt + 1, qt + 2, nq, ndo, nrow);
+            nq += q_tile_stride, ndo += do_tile_stride, nrow += BM;
+            step(std::true_type{}, I1{}, I2{}, 2, it_m + 2, qt + 2, qt + 3, nq, ndo, nrow);
+            nq += q_tile_stride, ndo += do_tile_stride, nrow += BM;
+        }
+    }
+    for (int it = it_m; it < n_masked_here + it_lo; ++it) {
         const int qn = it + 1 < it_hi ? tile_of(it + 1) : 0;
         step(std::true_type{}, I2{}, IM{}, st, it, tile_of(it), qn, qbase + qn * q_tile_stride, dobase + qn * do_tile_stride,
              rowbase + qn * BM);

@@ -159,6 +159,7 @@ int launch_bwd(const BwdParams& p, hipStream_t s) {
     auto kern = bwd_dkdv_kernel<D, HASMASK, TIMING>;
     auto kern_dq = bwd_dq_kernel<D, HASMASK, 4>;
     auto kern_dqv = bwd_dq_kernel<D, true, 4, true>;                 // keep-mask with vector-loadable rows over whole tiles
+    auto kern_kvv = bwd_dkdv_kernel<D, true, false, true>;           // ... whose tiles travel through LDS
     using TW = BwdDqWideTile<D>;
     auto kern_dqw = bwd_dq_wide_kernel<D>;                           // 256-query workgroups, builds without a keep-mask only
     if (!attr_done) {
@@ -174,6 +175,9 @@ int launch_bwd(const BwdParams& p, hipStream_t s) {
         if (HASMASK) {
             e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern_dqv),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, TQ::LDS_BYTES);
+            if (e != hipSuccess) return (int)e;
+            e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern_kvv),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS_BYTES_VECMASK);
             if (e != hipSuccess) return (int)e;
         }
         attr_done = true;
@@ -221,7 +225,11 @@ int launch_bwd(const BwdParams& p, hipStream_t s) {
     }
     {
         ScopedKernelTimer t(FLAME_ATTN_KERNEL_BWD_DKDV, s);
-        hipLaunchKernelGGL(kern, dim3((unsigned)grid_kv), dim3(256), T::LDS_BYTES, s, pk);
+        if (HASMASK && !TIMING && p.m.rows16 && !p.m.causal && p.Sk % T::BN == 0 && p.Sq % T::BM == 0 &&
+            (int64_t)T::BM * p.m.sq < (int64_t)1 << 31)
+            hipLaunchKernelGGL(kern_kvv, dim3((unsigned)grid_kv), dim3(256), T::LDS_BYTES_VECMASK, s, pk);
+        else
+            hipLaunchKernelGGL(kern, dim3((unsigned)grid_kv), dim3(256), T::LDS_BYTES, s, pk);
     }
     if (n_split > 0) {
         ScopedKernelTimer t(FLAME_ATTN_KERNEL_BWD_MERGE, s);
