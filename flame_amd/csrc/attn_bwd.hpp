@@ -909,10 +909,9 @@ __global__ __launch_bounds__(64 * NW, (NW == 4 && (!HASMASK || VECMASK)) ? 2 : 1
             float pr = exp2_fast(fmaf(sacc[kb][r], c_log2, -lse2));
             if (MASKED) {
                 const int key = key0 + 32 * kb + acc_row(r, h);
-                bool drop = key >= klimit;
-                if (p.m.causal) drop = drop || key > qrow;
+                bool drop = (key >= klimit) | ((p.m.causal != 0) & (key > qrow));     // bitwise: selects, not branches
                 if constexpr (VECMASK) {
-                    drop = drop || !mrow.keep(kb, r, h);
+                    drop |= !mrow.keep(kb, r, h);
                 } else if (HASMASK) {
                     if (vec_mask) drop = drop || !mrow.keep(kb, r, h);
                     else if (!drop && qok) drop = mbase[(int64_t)qrow * p.m.sq + (int64_t)key * p.m.sk] == 0;
