@@ -1212,8 +1212,7 @@ __global__ __launch_bounds__(256) void bwd_dq_wide_kernel(const BwdParams p) {
             float pr = exp2_fast(fmaf(sacc[qb][kb][r], c_log2, -lse2[qb]));
             if (MASKED) {
                 const int key = key0 + 32 * kb + acc_row(r, h);
-                bool drop = key >= klimit;
-                if (p.m.causal) drop = drop || key > qrow[qb];
+                const bool drop = (key >= klimit) | ((p.m.causal != 0) & (key > qrow[qb]));     // bitwise: selects, not branches
                 pr = drop ? 0.f : pr;
             }
             sacc[qb][kb][r] = pr;

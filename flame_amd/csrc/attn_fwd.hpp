@@ -199,8 +199,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void fwd_kernel(const Fwd
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int key = t * BN + 32 * kb + acc_row(r, h);
-                    bool drop = key >= klimit || !mrow.keep(kb, r, h);
-                    if (p.m.causal) drop = drop || key > qi;
+                    const bool drop = (key >= klimit) | !mrow.keep(kb, r, h) | ((p.m.causal != 0) & (key > qi));   // bitwise: no branches
                     s[kb][r] = drop ? -INFINITY : s[kb][r];
                 }
             return;
@@ -215,8 +214,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void fwd_kernel(const Fwd
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int key = t * BN + 32 * kb + acc_row(r, h);
-                bool drop = key >= klimit;
-                if (p.m.causal) drop = drop || key > qi;
+                bool drop = (key >= klimit) | ((p.m.causal != 0) & (key > qi));     // bitwise: selects, not branches
                 float val = s[kb][r];
                 if (HASMASK) {
                     if (vec_mask) drop = drop || !mrow.keep(kb, r, h);
