@@ -902,17 +902,21 @@ __global__ __launch_bounds__(64 * NW, (NW == 4 && (!HASMASK || VECMASK)) ? 2 : 1
             // two workgroups per unit: the other wavefront of the SIMD covers the load, and a second row in
             // registers would spill
             mrow.load(mbase + (int64_t)min(qrow, p.Sq - 1) * p.m.sq + key0);
+            // the key length and the causal diagonal cut few tiles: there they are folded into the mask bytes,
+            // so that the per-element test is the mask byte alone
+            const int lim = (p.m.causal ? min(klimit, qrow + 1) : klimit) - key0;
+            if (__any(lim < BN)) mrow.restrict_to(lim);
         } else if (HASMASK && MASKED && p.m.rows16 && key0 + 2 * BN <= p.Sk && t + 1 < n_tiles) {
             mnext.load(mbase + (int64_t)min(qrow, p.Sq - 1) * p.m.sq + key0 + BN);
         }
         auto p_elem = [&](int kb, int r) {          // P^T: one query per lane, so LSE is a per-lane scalar
             float pr = exp2_fast(fmaf(sacc[kb][r], c_log2, -lse2));
-            if (MASKED) {
+            if constexpr (VECMASK) {
+                pr = mrow.keep(kb, r, h) ? pr : 0.f;
+            } else if (MASKED) {
                 const int key = key0 + 32 * kb + acc_row(r, h);
                 bool drop = (key >= klimit) | ((p.m.causal != 0) & (key > qrow));     // bitwise: selects, not branches
-                if constexpr (VECMASK) {
-                    drop |= !mrow.keep(kb, r, h);
-                } else if (HASMASK) {
+                if (HASMASK) {
                     if (vec_mask) drop = drop || !mrow.keep(kb, r, h);
                     else if (!drop && qok) drop = mbase[(int64_t)qrow * p.m.sq + (int64_t)key * p.m.sk] == 0;
                 }

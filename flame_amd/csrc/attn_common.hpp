@@ -301,6 +301,16 @@ struct MaskRow64 {
 #pragma unroll
         for (int j = 0; j < 4; ++j) w[j] = *reinterpret_cast<const u32x4*>(row_tile + 16 * j);
     }
+    // Clears the bytes of the keys at or past `limit` (relative to the first key of the tile): key-length and
+    // causal exclusions then need no test of their own per element.  Meant for the few tiles they cut.
+    __device__ __forceinline__ void restrict_to(int limit) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int c = min(max(limit - 4 * i, 0), 4);                  // bytes of dword i that stay
+            const uint32_t m = c >= 4 ? 0xffffffffu : ((1u << (8 * c)) - 1u);
+            w[i >> 2][i & 3] &= m;
+        }
+    }
     __device__ __forceinline__ bool keep(int kb, int r, int h) const {      // kb, r compile-time; h per lane
         const int d0 = 8 * kb + 2 * (r >> 2);                               // dword of the even half
         const uint32_t lo = w[d0 >> 2][d0 & 3], hi = w[(d0 + 1) >> 2][(d0 + 1) & 3];

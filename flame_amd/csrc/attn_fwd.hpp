@@ -194,14 +194,14 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void fwd_kernel(const Fwd
         if constexpr (VECMASK) {
             MaskRow64 mrow;
             mrow.load(mbase + (int64_t)min(qi, p.Sq - 1) * p.m.sq + t * BN);
+            // the key length and the causal diagonal cut few tiles: there they are folded into the mask bytes,
+            // so that the per-element test is the mask byte alone
+            const int lim = (p.m.causal ? min(klimit, qi + 1) : klimit) - t * BN;
+            if (__any(lim < BN)) mrow.restrict_to(lim);
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int key = t * BN + 32 * kb + acc_row(r, h);
-                    const bool drop = (key >= klimit) | !mrow.keep(kb, r, h) | ((p.m.causal != 0) & (key > qi));   // bitwise: no branches
-                    s[kb][r] = drop ? -INFINITY : s[kb][r];
-                }
+                for (int r = 0; r < 16; ++r) s[kb][r] = mrow.keep(kb, r, h) ? s[kb][r] : -INFINITY;
             return;
         }
         // a lane's 64 keep-mask bytes of the tile in four 16-byte loads where the layout allows it (each

@@ -79,13 +79,14 @@ def test_general_keep_mask_and_fully_masked_rows(oracle):
     assert torch.all(dk[:, :, 149] == 0) and torch.all(dv[:, :, 149] == 0)
 
 
-@pytest.mark.parametrize("D,Sq,Sk,mshape,with_len", [
-    (128, 192, 256, "full", False),      # a mask per (batch, head, query, key)
-    (64, 128, 384, "full", True),        # ... together with per-batch key lengths
-    (128, 128, 256, "keys", False),      # key padding mask [B,1,1,Sk], broadcast over heads and queries
-    (64, 256, 128, "queries", False),    # [B,1,Sq,Sk]
+@pytest.mark.parametrize("D,Sq,Sk,mshape,with_len,causal", [
+    (128, 192, 256, "full", False, False),      # a mask per (batch, head, query, key)
+    (64, 128, 384, "full", True, False),        # ... together with per-batch key lengths
+    (128, 128, 256, "keys", False, False),      # key padding mask [B,1,1,Sk], broadcast over heads and queries
+    (64, 256, 128, "queries", False, False),    # [B,1,Sq,Sk]
+    (128, 256, 256, "full", True, True),        # mask, key lengths and the causal flag together
 ])
-def test_keep_mask_over_whole_tiles(oracle, D, Sq, Sk, mshape, with_len):
+def test_keep_mask_over_whole_tiles(oracle, D, Sq, Sk, mshape, with_len, causal):
     """Mask rows that are contiguous and 16-byte aligned, Sq a multiple of 64 and Sk of 128: the kernels that
     take the mask in 16-byte pieces (forward, dQ) and stage it through LDS (dK/dV)."""
     from flame_amd import capi
@@ -100,7 +101,8 @@ def test_keep_mask_over_whole_tiles(oracle, D, Sq, Sk, mshape, with_len):
         mask[0, 0, 5, :] = 0                           # ... one on purpose
     mask[..., Sk - 3] = 0                              # a key nobody attends to
     kv_len = np.asarray([Sk - 37, Sk], np.int32) if with_len else None
-    w = W.Workload("mask_whole_tiles_" + mshape, t[0], t[1], t[2], t[3], 1.0 / math.sqrt(D), kv_len=kv_len, mask=mask)
+    w = W.Workload("mask_whole_tiles_" + mshape, t[0], t[1], t[2], t[3], 1.0 / math.sqrt(D), causal=causal,
+                   kv_len=kv_len, mask=mask)
     dq, dk, dv = _check_bwd(oracle, w)
     if mshape != "keys":
         assert torch.all(dq[0, 0, 5] == 0)
@@ -110,8 +112,8 @@ def test_keep_mask_over_whole_tiles(oracle, D, Sq, Sk, mshape, with_len):
     # forward of the same problem
     q, k, v = (to_dev(x) for x in (w.q, w.k, w.v))
     kvl = None if kv_len is None else torch.from_numpy(kv_len).cuda()
-    o, lse = capi.attn_fwd(q, k, v, w.scale, kv_len=kvl, mask=torch.from_numpy(mask).cuda())
-    ro, rlse, rof = oracle.sdpa_fwd(w.q, w.k, w.v, w.scale, kv_len=kv_len, mask=mask, want_f32=True)
+    o, lse = capi.attn_fwd(q, k, v, w.scale, causal=causal, kv_len=kvl, mask=torch.from_numpy(mask).cuda())
+    ro, rlse, rof = oracle.sdpa_fwd(w.q, w.k, w.v, w.scale, causal=causal, kv_len=kv_len, mask=mask, want_f32=True)
     assert_close_bf16(oracle, "O", to_f32(o).reshape(B * H, Sq, D), ro.reshape(B * H, Sq, D), rof.reshape(B * H, Sq, D))
     glse = lse.cpu().numpy().reshape(B * H, Sq)
     fin = np.isfinite(rlse.reshape(B * H, Sq))
