@@ -137,11 +137,12 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
     int qt_begin = p.m.causal ? (k0 / BM) : 0;
     if (k0 >= klimit) qt_begin = n_qt;        // nothing attends to these keys: dK = dV = 0
     const int n_it = n_qt - qt_begin;
-    // The walk visits the query tiles that need per-element exclusions first (all of them when the key
-    // tile is ragged or an explicit mask is given, else the causal diagonal tiles and a partial last
-    // tile) and the fully attended ones afterwards, so that each of the two loops runs one
+    // The walk visits the query tiles that need per-element exclusions first (all of them when an explicit
+    // mask is given, else the causal diagonal tiles and a partial last tile) and the fully attended ones afterwards, so that each of the two loops runs one
     // specialised, branch-free body.  The order of the tiles does not matter to the sums.
-    const bool all_masked = HASMASK || (k0 + BN > klimit);
+    // (A key block that the key length cuts needs none: a lane owns one key, its column of dK^T / dV^T
+    // depends on no other key's P or dS, and the columns of the keys past the length are zeroed before the store.)
+    const bool all_masked = HASMASK;
     int lead_end = qt_begin;
     if (n_it > 0) {
         if (all_masked) lead_end = n_qt;
@@ -629,6 +630,15 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
                 *reinterpret_cast<f32x4*>(dst + (size_t)BN * D + ((size_t)tid * DB + db) * 16 + 4 * g) = wv;
             }
         return;
+    }
+    if (key >= klimit) {          // nothing attends to this lane's key
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                dkacc[db][r] = 0.f;
+                dvacc[db][r] = 0.f;
+            }
     }
     dkdv_store<D>(p, dkacc, dvacc, b, hh, kw0 + n, h);
 }
