@@ -77,8 +77,11 @@ def _mask_args(mask, B, H, Sq, Sk):
     return m, tuple(st), m
 
 
-def sdpa_fwd(q, k, v, scale, causal=False, kv_len=None, mask=None, heads=None, want_f32=False):
-    """Naive fp32 forward. Returns (O bf16-bits, LSE fp32[, O fp32])."""
+def sdpa_fwd(q, k, v, scale, causal=False, kv_len=None, mask=None, heads=None, want_f32=False, rows=None):
+    """Naive fp32 forward. Returns (O bf16-bits, LSE fp32[, O fp32]).
+
+    heads = (begin, end) over the flat b*H+h index and rows = (begin, end) over the query rows restrict
+    the work; the outputs keep their full shapes and only that part of them is filled."""
     B, H, Sq, D = q.shape
     Sk = k.shape[2]
     q, k, v = (np.ascontiguousarray(t, dtype=np.uint16) for t in (q, k, v))
@@ -88,9 +91,10 @@ def sdpa_fwd(q, k, v, scale, causal=False, kv_len=None, mask=None, heads=None, w
     kvl = None if kv_len is None else np.ascontiguousarray(kv_len, dtype=np.int32)
     m, st, _keep = _mask_args(mask, B, H, Sq, Sk)
     hb, he = (0, B * H) if heads is None else heads
-    rc = lib().oracle_sdpa_fwd(
+    rb, re_ = (0, Sq) if rows is None else rows
+    rc = lib().oracle_sdpa_fwd_rows(
         _p(q), _p(k), _p(v), B, H, Sq, Sk, D, ctypes.c_float(scale), int(bool(causal)),
-        _p(kvl), _p(m), *(ctypes.c_int64(s) for s in st), hb, he, _p(O), _p(LSE), _p(O32))
+        _p(kvl), _p(m), *(ctypes.c_int64(s) for s in st), hb, he, rb, re_, _p(O), _p(LSE), _p(O32))
     if rc != 0:
         raise RuntimeError(f"oracle_sdpa_fwd failed: {rc}")
     return (O, LSE, O32) if want_f32 else (O, LSE)
@@ -115,8 +119,11 @@ def sdpa_fwd_bias(q, k, v, scale, bias, want_f32=False):
     return (O, LSE, O32) if want_f32 else (O, LSE)
 
 
-def sdpa_bwd(q, k, v, o, do, scale, causal=False, kv_len=None, mask=None, heads=None, want_f32=False):
-    """Naive fp32 backward. Returns (dQ, dK, dV) bf16 bits [+ fp32 copies]."""
+def sdpa_bwd(q, k, v, o, do, scale, causal=False, kv_len=None, mask=None, heads=None, want_f32=False, rows=None):
+    """Naive fp32 backward. Returns (dQ, dK, dV) bf16 bits [+ fp32 copies].
+
+    With rows = (begin, end) only those query rows take part: dQ is filled for them, and dK / dV are
+    the sums over them (complete for every key that no query outside the band attends to)."""
     B, H, Sq, D = q.shape
     Sk = k.shape[2]
     q, k, v, o, do = (np.ascontiguousarray(t, dtype=np.uint16) for t in (q, k, v, o, do))
@@ -127,9 +134,10 @@ def sdpa_bwd(q, k, v, o, do, scale, causal=False, kv_len=None, mask=None, heads=
     kvl = None if kv_len is None else np.ascontiguousarray(kv_len, dtype=np.int32)
     m, st, _keep = _mask_args(mask, B, H, Sq, Sk)
     hb, he = (0, B * H) if heads is None else heads
-    rc = lib().oracle_sdpa_bwd(
+    rb, re_ = (0, Sq) if rows is None else rows
+    rc = lib().oracle_sdpa_bwd_rows(
         _p(q), _p(k), _p(v), _p(o), _p(do), B, H, Sq, Sk, D, ctypes.c_float(scale),
-        int(bool(causal)), _p(kvl), _p(m), *(ctypes.c_int64(s) for s in st), hb, he,
+        int(bool(causal)), _p(kvl), _p(m), *(ctypes.c_int64(s) for s in st), hb, he, rb, re_,
         _p(dQ), _p(dK), _p(dV), _p(f[0]), _p(f[1]), _p(f[2]))
     if rc != 0:
         raise RuntimeError(f"oracle_sdpa_bwd failed: {rc}")
@@ -154,7 +162,9 @@ def sage_quant(q, k, qblk=128, kblk=64, smooth_k=True):
     return out
 
 
-def sage_fwd(qi8, ki8, sq, sk, v, scale, qblk=128, kblk=64, causal=False, heads=None):
+def sage_fwd(qi8, ki8, sq, sk, v, scale, qblk=128, kblk=64, causal=False, heads=None, kv_len=None, rows=None,
+             want_f32=False):
+    """Sage forward from quantised operands. Returns (O bf16 bits, LSE[, O fp32])."""
     B, H, Sq, D = qi8.shape
     Sk = ki8.shape[2]
     qi8, ki8 = (np.ascontiguousarray(t, dtype=np.int8) for t in (qi8, ki8))
@@ -162,12 +172,16 @@ def sage_fwd(qi8, ki8, sq, sk, v, scale, qblk=128, kblk=64, causal=False, heads=
     v = np.ascontiguousarray(v, dtype=np.uint16)
     O = np.zeros((B, H, Sq, D), np.uint16)
     LSE = np.zeros((B, H, Sq), np.float32)
+    O32 = np.zeros((B, H, Sq, D), np.float32) if want_f32 else None
+    kvl = None if kv_len is None else np.ascontiguousarray(kv_len, dtype=np.int32)
     hb, he = (0, B * H) if heads is None else heads
+    rb, re_ = (0, Sq) if rows is None else rows
     rc = lib().oracle_sage_fwd(_p(qi8), _p(ki8), _p(sq), _p(sk), _p(v), B, H, Sq, Sk, D, qblk, kblk,
-                               ctypes.c_float(scale), int(bool(causal)), hb, he, _p(O), _p(LSE))
+                               ctypes.c_float(scale), int(bool(causal)), _p(kvl), hb, he, rb, re_,
+                               _p(O), _p(LSE), _p(O32))
     if rc != 0:
         raise RuntimeError(f"oracle_sage_fwd failed: {rc}")
-    return O, LSE
+    return (O, LSE, O32) if want_f32 else (O, LSE)
 
 
 # ---------------------------------------------------------------- fp64 brute force (checker of the checker)

@@ -35,9 +35,13 @@
  *                    no reference test asserts Stats values ("parity unpinned" by the reference itself)
  *   dQ, dK, dV       pinned: fp64 central finite differences, torch CPU autograd
  *   int8 quantiser   pinned: brute force in Python integers/fp64, tie and absmax unit vectors
- *   K-mean smoothing, per-block (128/64) granularity, int8-QK forward: new behaviour with no
- *                    counterpart in the reference ("parity unpinned"); pinned only by softmax
- *                    shift-invariance and cosine against the bf16 result.
+ *   K-mean smoothing pinned: fp64 column means, softmax shift invariance
+ *   int8-QK forward  (per-block 128/64 scales, causal flag, key lengths; new behaviour with no counterpart
+ *                    in the reference) pinned: a hand-worked 2x2 known answer with distinct scales per
+ *                    block; fp64 textbook attention on the dequantised operands qi8*sq[block],
+ *                    ki8*sk[block] with block magnitudes 4-8x apart and short last blocks (O and LSE
+ *                    within 2e-5), with a control that a wrong block index fails
+ *   row bands        pinned: bit-identical to the rows of the full computation
  *
  * Layout: every tensor is contiguous [B,H,S,D]; bf16 is carried as uint16_t.
  */
@@ -103,10 +107,11 @@ static inline int excluded(const mask_spec* ms, int b, int h, int i, int j) {
     return 0;
 }
 
-/* P (fp32, Sq x Sk) for one head; also row LSE.  kt = K^T in fp32 [D][Sk]. */
-static void head_probs(const float* q, const float* kt, int Sq, int Sk, int D, float scale,
+/* P (fp32, R x Sk) for the query rows [row0, row0 + R) of one head; also their LSE.
+ * q = those R rows in fp32, kt = K^T in fp32 [D][Sk]. */
+static void head_probs(const float* q, const float* kt, int row0, int R, int Sk, int D, float scale,
                        const mask_spec* ms, int b, int h, float* P, float* lse) {
-    for (int i = 0; i < Sq; ++i) {
+    for (int i = 0; i < R; ++i) {
         float* row = P + (size_t)i * Sk;
         for (int j = 0; j < Sk; ++j) row[j] = 0.f;
         for (int d = 0; d < D; ++d) {
@@ -116,8 +121,8 @@ static void head_probs(const float* q, const float* kt, int Sq, int Sk, int D, f
         }
         float m = -INFINITY;
         for (int j = 0; j < Sk; ++j) {
-            float s = excluded(ms, b, h, i, j) ? -INFINITY : row[j] * scale;
-            if (ms->bias && s != -INFINITY) s += ms->bias[b * ms->bsb + h * ms->bsh + i * ms->bsq + j * ms->bsk];
+            float s = excluded(ms, b, h, row0 + i, j) ? -INFINITY : row[j] * scale;
+            if (ms->bias && s != -INFINITY) s += ms->bias[b * ms->bsb + h * ms->bsh + (row0 + i) * ms->bsq + j * ms->bsk];
             row[j] = s;
             if (s > m) m = s;
         }
@@ -149,7 +154,8 @@ static int check_dims(int B, int H, int Sq, int Sk, int D) {
  */
 static int sdpa_fwd_impl(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
                          int B, int H, int Sq, int Sk, int D, float scale, mask_spec ms,
-                         int heads_begin, int heads_end, uint16_t* O, float* LSE, float* O32);
+                         int heads_begin, int heads_end, int row_begin, int row_end,
+                         uint16_t* O, float* LSE, float* O32);
 
 int oracle_sdpa_fwd(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
                     int B, int H, int Sq, int Sk, int D, float scale, int causal,
@@ -158,7 +164,21 @@ int oracle_sdpa_fwd(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
                     int heads_begin, int heads_end,
                     uint16_t* O, float* LSE, float* O32) {
     mask_spec ms = {causal, kv_len, mask, msb, msh, msq, msk, NULL, 0, 0, 0, 0};
-    return sdpa_fwd_impl(Q, K, V, B, H, Sq, Sk, D, scale, ms, heads_begin, heads_end, O, LSE, O32);
+    return sdpa_fwd_impl(Q, K, V, B, H, Sq, Sk, D, scale, ms, heads_begin, heads_end, 0, Sq, O, LSE, O32);
+}
+
+/* The same forward restricted to the query rows [row_begin, row_end) of the chosen heads: a band of a
+ * long sequence then costs rows x Sk instead of Sq x Sk.  Outputs keep the full [B,H,Sq,...] layout;
+ * only the rows of the band are written. */
+int oracle_sdpa_fwd_rows(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
+                         int B, int H, int Sq, int Sk, int D, float scale, int causal,
+                         const int32_t* kv_len, const uint8_t* mask,
+                         int64_t msb, int64_t msh, int64_t msq, int64_t msk,
+                         int heads_begin, int heads_end, int row_begin, int row_end,
+                         uint16_t* O, float* LSE, float* O32) {
+    mask_spec ms = {causal, kv_len, mask, msb, msh, msq, msk, NULL, 0, 0, 0, 0};
+    if (row_begin < 0 || row_end > Sq || row_begin > row_end) return -1;
+    return sdpa_fwd_impl(Q, K, V, B, H, Sq, Sk, D, scale, ms, heads_begin, heads_end, row_begin, row_end, O, LSE, O32);
 }
 
 /* Forward with an additive fp32 bias on the scaled logits (T5-style relative position bias),
@@ -168,36 +188,39 @@ int oracle_sdpa_fwd_bias(const uint16_t* Q, const uint16_t* K, const uint16_t* V
                          const float* bias, int64_t bsb, int64_t bsh, int64_t bsq, int64_t bsk,
                          uint16_t* O, float* LSE, float* O32) {
     mask_spec ms = {0, NULL, NULL, 0, 0, 0, 0, bias, bsb, bsh, bsq, bsk};
-    return sdpa_fwd_impl(Q, K, V, B, H, Sq, Sk, D, scale, ms, 0, B * H, O, LSE, O32);
+    return sdpa_fwd_impl(Q, K, V, B, H, Sq, Sk, D, scale, ms, 0, B * H, 0, Sq, O, LSE, O32);
 }
 
 static int sdpa_fwd_impl(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
                          int B, int H, int Sq, int Sk, int D, float scale, mask_spec ms,
-                         int heads_begin, int heads_end, uint16_t* O, float* LSE, float* O32) {
+                         int heads_begin, int heads_end, int row_begin, int row_end,
+                         uint16_t* O, float* LSE, float* O32) {
     if (check_dims(B, H, Sq, Sk, D)) return -1;
+    const int R = row_end - row_begin;
+    if (R <= 0) return 0;
     int fail = 0;
 #pragma omp parallel for schedule(dynamic, 1)
     for (int bh = heads_begin; bh < heads_end; ++bh) {
         const int b = bh / H, h = bh % H;
-        float* q = (float*)malloc(sizeof(float) * (size_t)Sq * D);
+        float* q = (float*)malloc(sizeof(float) * (size_t)R * D);
         float* kt = (float*)malloc(sizeof(float) * (size_t)Sk * D);
         float* v = (float*)malloc(sizeof(float) * (size_t)Sk * D);
-        float* P = (float*)malloc(sizeof(float) * (size_t)Sq * Sk);
+        float* P = (float*)malloc(sizeof(float) * (size_t)R * Sk);
         float* o = (float*)malloc(sizeof(float) * (size_t)D);
         if (!q || !kt || !v || !P || !o) {
             fail = 1;
         } else {
-            const uint16_t* Qh = Q + (size_t)bh * Sq * D;
+            const uint16_t* Qh = Q + ((size_t)bh * Sq + row_begin) * D;
             const uint16_t* Kh = K + (size_t)bh * Sk * D;
             const uint16_t* Vh = V + (size_t)bh * Sk * D;
-            for (size_t t = 0; t < (size_t)Sq * D; ++t) q[t] = bf16_to_f32(Qh[t]);
+            for (size_t t = 0; t < (size_t)R * D; ++t) q[t] = bf16_to_f32(Qh[t]);
             for (int j = 0; j < Sk; ++j)
                 for (int d = 0; d < D; ++d) {
                     kt[(size_t)d * Sk + j] = bf16_to_f32(Kh[(size_t)j * D + d]);
                     v[(size_t)j * D + d] = bf16_to_f32(Vh[(size_t)j * D + d]);
                 }
-            head_probs(q, kt, Sq, Sk, D, scale, &ms, b, h, P, LSE + (size_t)bh * Sq);
-            for (int i = 0; i < Sq; ++i) {
+            head_probs(q, kt, row_begin, R, Sk, D, scale, &ms, b, h, P, LSE + (size_t)bh * Sq + row_begin);
+            for (int i = 0; i < R; ++i) {
                 for (int d = 0; d < D; ++d) o[d] = 0.f;
                 const float* row = P + (size_t)i * Sk;
                 for (int j = 0; j < Sk; ++j) {
@@ -207,7 +230,7 @@ static int sdpa_fwd_impl(const uint16_t* Q, const uint16_t* K, const uint16_t* V
                     for (int d = 0; d < D; ++d) o[d] += p * vr[d];
                 }
                 for (int d = 0; d < D; ++d) {
-                    const size_t idx = ((size_t)bh * Sq + i) * D + d;
+                    const size_t idx = ((size_t)bh * Sq + row_begin + i) * D + d;
                     O[idx] = f32_to_bf16(o[d]);
                     if (O32) O32[idx] = o[d];
                 }
@@ -222,42 +245,49 @@ static int sdpa_fwd_impl(const uint16_t* Q, const uint16_t* K, const uint16_t* V
  * Backward.  Recomputes P from Q,K (it does not consume a saved LSE, so it is independent of the
  * forward under test).  O is the bf16-rounded forward output.  Outputs bf16 dQ [B,H,Sq,D],
  * dK,dV [B,H,Sk,D]; optional fp32 copies dQ32,dK32,dV32 (NULL to skip).
+ *
+ * Only the query rows [row_begin, row_end) of the chosen heads take part: dQ is written for those
+ * rows, and dK / dV hold the sums over those rows only (the whole gradient when the band is
+ * [0, Sq), and also for every key that no query outside the band attends to, e.g. the last keys
+ * of a causal problem when the band is the last rows).
  */
-int oracle_sdpa_bwd(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
-                    const uint16_t* O, const uint16_t* dO,
-                    int B, int H, int Sq, int Sk, int D, float scale, int causal,
-                    const int32_t* kv_len, const uint8_t* mask,
-                    int64_t msb, int64_t msh, int64_t msq, int64_t msk,
-                    int heads_begin, int heads_end,
-                    uint16_t* dQ, uint16_t* dK, uint16_t* dV,
-                    float* dQ32, float* dK32, float* dV32) {
+int oracle_sdpa_bwd_rows(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
+                         const uint16_t* O, const uint16_t* dO,
+                         int B, int H, int Sq, int Sk, int D, float scale, int causal,
+                         const int32_t* kv_len, const uint8_t* mask,
+                         int64_t msb, int64_t msh, int64_t msq, int64_t msk,
+                         int heads_begin, int heads_end, int row_begin, int row_end,
+                         uint16_t* dQ, uint16_t* dK, uint16_t* dV,
+                         float* dQ32, float* dK32, float* dV32) {
     if (check_dims(B, H, Sq, Sk, D)) return -1;
+    if (row_begin < 0 || row_end > Sq || row_begin > row_end) return -1;
+    const int R = row_end - row_begin;
     mask_spec ms = {causal, kv_len, mask, msb, msh, msq, msk, NULL, 0, 0, 0, 0};
     int fail = 0;
 #pragma omp parallel for schedule(dynamic, 1)
     for (int bh = heads_begin; bh < heads_end; ++bh) {
         const int b = bh / H, h = bh % H;
-        const size_t nq = (size_t)Sq * D, nk = (size_t)Sk * D;
-        float* q = (float*)malloc(sizeof(float) * nq);
-        float* g = (float*)malloc(sizeof(float) * nq);   /* dO */
+        const size_t nq = (size_t)Sq * D, nk = (size_t)Sk * D, nr = (size_t)R * D;
+        float* q = (float*)malloc(sizeof(float) * (nr + 1));
+        float* g = (float*)malloc(sizeof(float) * (nr + 1));   /* dO */
         float* k = (float*)malloc(sizeof(float) * nk);
         float* kt = (float*)malloc(sizeof(float) * nk);
         float* vt = (float*)malloc(sizeof(float) * nk);
-        float* P = (float*)malloc(sizeof(float) * (size_t)Sq * Sk);
+        float* P = (float*)malloc(sizeof(float) * ((size_t)R * Sk + 1));
         float* dp = (float*)malloc(sizeof(float) * (size_t)Sk);
-        float* lse = (float*)malloc(sizeof(float) * (size_t)Sq);
-        float* dq = (float*)calloc(nq, sizeof(float));
+        float* lse = (float*)malloc(sizeof(float) * (size_t)(R + 1));
+        float* dq = (float*)calloc(nr + 1, sizeof(float));
         float* dk = (float*)calloc(nk, sizeof(float));
         float* dv = (float*)calloc(nk, sizeof(float));
         if (!q || !g || !k || !kt || !vt || !P || !dp || !lse || !dq || !dk || !dv) {
             fail = 1;
         } else {
-            const uint16_t* Qh = Q + (size_t)bh * nq;
-            const uint16_t* Gh = dO + (size_t)bh * nq;
-            const uint16_t* Oh = O + (size_t)bh * nq;
+            const uint16_t* Qh = Q + (size_t)bh * nq + (size_t)row_begin * D;
+            const uint16_t* Gh = dO + (size_t)bh * nq + (size_t)row_begin * D;
+            const uint16_t* Oh = O + (size_t)bh * nq + (size_t)row_begin * D;
             const uint16_t* Kh = K + (size_t)bh * nk;
             const uint16_t* Vh = V + (size_t)bh * nk;
-            for (size_t t = 0; t < nq; ++t) { q[t] = bf16_to_f32(Qh[t]); g[t] = bf16_to_f32(Gh[t]); }
+            for (size_t t = 0; t < nr; ++t) { q[t] = bf16_to_f32(Qh[t]); g[t] = bf16_to_f32(Gh[t]); }
             for (int j = 0; j < Sk; ++j)
                 for (int d = 0; d < D; ++d) {
                     const float kv = bf16_to_f32(Kh[(size_t)j * D + d]);
@@ -265,8 +295,8 @@ int oracle_sdpa_bwd(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
                     kt[(size_t)d * Sk + j] = kv;
                     vt[(size_t)d * Sk + j] = bf16_to_f32(Vh[(size_t)j * D + d]);
                 }
-            head_probs(q, kt, Sq, Sk, D, scale, &ms, b, h, P, lse);
-            for (int i = 0; i < Sq; ++i) {
+            head_probs(q, kt, row_begin, R, Sk, D, scale, &ms, b, h, P, lse);
+            for (int i = 0; i < R; ++i) {
                 const float* gi = g + (size_t)i * D;
                 const float* qi = q + (size_t)i * D;
                 float* row = P + (size_t)i * Sk;
@@ -293,10 +323,11 @@ int oracle_sdpa_bwd(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
                     }
                 }
             }
-            for (size_t t = 0; t < nq; ++t) {
+            for (size_t t = 0; t < nr; ++t) {
                 const float x = dq[t] * scale;
-                dQ[(size_t)bh * nq + t] = f32_to_bf16(x);
-                if (dQ32) dQ32[(size_t)bh * nq + t] = x;
+                const size_t idx = (size_t)bh * nq + (size_t)row_begin * D + t;
+                dQ[idx] = f32_to_bf16(x);
+                if (dQ32) dQ32[idx] = x;
             }
             for (size_t t = 0; t < nk; ++t) {
                 const float x = dk[t] * scale;
@@ -310,6 +341,18 @@ int oracle_sdpa_bwd(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
         free(dq); free(dk); free(dv);
     }
     return fail ? -2 : 0;
+}
+
+int oracle_sdpa_bwd(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
+                    const uint16_t* O, const uint16_t* dO,
+                    int B, int H, int Sq, int Sk, int D, float scale, int causal,
+                    const int32_t* kv_len, const uint8_t* mask,
+                    int64_t msb, int64_t msh, int64_t msq, int64_t msk,
+                    int heads_begin, int heads_end,
+                    uint16_t* dQ, uint16_t* dK, uint16_t* dV,
+                    float* dQ32, float* dK32, float* dV32) {
+    return oracle_sdpa_bwd_rows(Q, K, V, O, dO, B, H, Sq, Sk, D, scale, causal, kv_len, mask, msb, msh, msq, msk,
+                                heads_begin, heads_end, 0, Sq, dQ, dK, dV, dQ32, dK32, dV32);
 }
 
 /* ------------------------------------------------------------------------------------------
@@ -392,18 +435,24 @@ int oracle_sage_quant(const uint16_t* Q, const uint16_t* K,
 
 /*
  * Sage forward from quantised operands:
- *   S_ij = (float)(int32 sum_d Qi8_id Ki8_jd) * sq[i/qblk] * sk[j/kblk] * scale
- *   P = softmax(S) in fp32 (naive, materialised); O = P V -> bf16.
+ *   S_ij = (float)(int32 sum_d Qi8_id Ki8_jd) * (sq[i/qblk] * sk[j/kblk] * scale)
+ *   key j is excluded when causal and j > i, or when j >= kv_len[b]
+ *   P = softmax(S) in fp32 (naive, materialised); O = P V -> bf16 (O32: the same before rounding).
+ *   A row with every key excluded gives O = 0 and LSE = -inf.
+ * Only the query rows [row_begin, row_end) of the chosen heads are computed.
  */
 int oracle_sage_fwd(const int8_t* Qi8, const int8_t* Ki8, const float* sq, const float* sk,
                     const uint16_t* V, int B, int H, int Sq, int Sk, int D, int qblk, int kblk,
-                    float scale, int causal, int heads_begin, int heads_end,
-                    uint16_t* O, float* LSE) {
+                    float scale, int causal, const int32_t* kv_len,
+                    int heads_begin, int heads_end, int row_begin, int row_end,
+                    uint16_t* O, float* LSE, float* O32) {
     if (check_dims(B, H, Sq, Sk, D) || qblk <= 0 || kblk <= 0) return -1;
+    if (row_begin < 0 || row_end > Sq || row_begin > row_end) return -1;
     const int nqb = (Sq + qblk - 1) / qblk, nkb = (Sk + kblk - 1) / kblk;
     int fail = 0;
 #pragma omp parallel for schedule(dynamic, 1)
     for (int bh = heads_begin; bh < heads_end; ++bh) {
+        const int b = bh / H;
         float* v = (float*)malloc(sizeof(float) * (size_t)Sk * D);
         float* row = (float*)malloc(sizeof(float) * (size_t)Sk);
         float* o = (float*)malloc(sizeof(float) * (size_t)D);
@@ -413,8 +462,9 @@ int oracle_sage_fwd(const int8_t* Qi8, const int8_t* Ki8, const float* sq, const
             const int8_t* Qh = Qi8 + (size_t)bh * Sq * D;
             const int8_t* Kh = Ki8 + (size_t)bh * Sk * D;
             const uint16_t* Vh = V + (size_t)bh * Sk * D;
+            const int klim = kv_len ? (kv_len[b] < Sk ? (kv_len[b] < 0 ? 0 : kv_len[b]) : Sk) : Sk;
             for (size_t t = 0; t < (size_t)Sk * D; ++t) v[t] = bf16_to_f32(Vh[t]);
-            for (int i = 0; i < Sq; ++i) {
+            for (int i = row_begin; i < row_end; ++i) {
                 const float sqi = sq[(size_t)bh * nqb + i / qblk];
                 float m = -INFINITY;
                 for (int j = 0; j < Sk; ++j) {
@@ -422,19 +472,28 @@ int oracle_sage_fwd(const int8_t* Qi8, const int8_t* Ki8, const float* sq, const
                     for (int d = 0; d < D; ++d)
                         acc += (int32_t)Qh[(size_t)i * D + d] * (int32_t)Kh[(size_t)j * D + d];
                     float s = (float)acc * (sqi * sk[(size_t)bh * nkb + j / kblk] * scale);
-                    if (causal && j > i) s = -INFINITY;
+                    if ((causal && j > i) || j >= klim) s = -INFINITY;
                     row[j] = s;
                     if (s > m) m = s;
                 }
-                float l = 0.f;
-                for (int j = 0; j < Sk; ++j) { row[j] = expf(row[j] - m); l += row[j]; }
                 for (int d = 0; d < D; ++d) o[d] = 0.f;
-                for (int j = 0; j < Sk; ++j) {
-                    const float p = row[j] / l;
-                    for (int d = 0; d < D; ++d) o[d] += p * v[(size_t)j * D + d];
+                float lse = -INFINITY;
+                if (m != -INFINITY) {
+                    float l = 0.f;
+                    for (int j = 0; j < Sk; ++j) { row[j] = expf(row[j] - m); l += row[j]; }
+                    for (int j = 0; j < Sk; ++j) {
+                        const float p = row[j] / l;
+                        if (p == 0.f) continue;
+                        for (int d = 0; d < D; ++d) o[d] += p * v[(size_t)j * D + d];
+                    }
+                    lse = m + logf(l);
                 }
-                for (int d = 0; d < D; ++d) O[((size_t)bh * Sq + i) * D + d] = f32_to_bf16(o[d]);
-                if (LSE) LSE[(size_t)bh * Sq + i] = m + logf(l);
+                for (int d = 0; d < D; ++d) {
+                    const size_t idx = ((size_t)bh * Sq + i) * D + d;
+                    O[idx] = f32_to_bf16(o[d]);
+                    if (O32) O32[idx] = o[d];
+                }
+                if (LSE) LSE[(size_t)bh * Sq + i] = lse;
             }
         }
         free(v); free(row); free(o);

@@ -80,6 +80,93 @@ def test_k_smoothing_mean_and_shift_invariance(oracle):
     assert oracle.cosine(oracle.bf16_to_f32(o_sage), oracle.bf16_to_f32(o_ref)) > 0.999
 
 
+def test_sage_forward_literal_known_answer(oracle):
+    """2 queries x 2 keys x head dim 1 with one block per row, worked by hand:
+    S = qi8 * ki8 * sq[i] * sk[j] = [[2*1*0.5*1, 2*(-1)*0.5*2], [3*1*1*1, 3*(-1)*1*2]] = [[1, -2], [3, -6]];
+    V = [1, 0], so O_i is the weight of key 0: 1/(1+e^-3), 1/(1+e^-9); LSE = 1 + ln(1+e^-3), 3 + ln(1+e^-9).
+    Swapping sq and sk, or indexing either by the other's block, gives different logits."""
+    qi8 = np.array([2, 3], np.int8).reshape(1, 1, 2, 1)
+    ki8 = np.array([1, -1], np.int8).reshape(1, 1, 2, 1)
+    sq = np.array([0.5, 1.0], np.float32).reshape(1, 1, 2)
+    sk = np.array([1.0, 2.0], np.float32).reshape(1, 1, 2)
+    v = _bits(np.array([1.0, 0.0], np.float32).reshape(1, 1, 2, 1))
+    _, lse, o = oracle.sage_fwd(qi8, ki8, sq, sk, v, 1.0, qblk=1, kblk=1, want_f32=True)
+    assert np.allclose(o.ravel(), [0.9525741268224334, 0.9998766054240137], rtol=0, atol=2e-7)
+    assert np.allclose(lse.ravel(), [1.048587351573742, 3.000123402189723], rtol=0, atol=5e-7)
+    # causal: key 1 is excluded for query 0 (j > i), not for query 1
+    _, lse, o = oracle.sage_fwd(qi8, ki8, sq, sk, v, 1.0, qblk=1, kblk=1, causal=True, want_f32=True)
+    assert np.allclose(o.ravel(), [1.0, 0.9998766054240137], rtol=0, atol=2e-7)
+    assert np.allclose(lse.ravel(), [1.0, 3.000123402189723], rtol=0, atol=5e-7)
+    # key length 1: key 1 is excluded for both; key length 0: nothing is attended
+    _, lse, o = oracle.sage_fwd(qi8, ki8, sq, sk, v, 1.0, qblk=1, kblk=1, kv_len=[1], want_f32=True)
+    assert np.allclose(o.ravel(), [1.0, 1.0], rtol=0, atol=2e-7) and np.allclose(lse.ravel(), [1.0, 3.0], atol=5e-7)
+    ob, lse = oracle.sage_fwd(qi8, ki8, sq, sk, v, 1.0, qblk=1, kblk=1, kv_len=[0])
+    assert np.all(ob == 0) and np.all(lse == -np.inf)
+
+
+def _sage_case(oracle, B, H, Sq, Sk, D, seed):
+    """Quantised operands whose blocks have deliberately different magnitudes, short last blocks."""
+    qf = W.normal_f32(seed, 0, B * H * Sq * D).reshape(B, H, Sq, D)
+    kf = W.normal_f32(seed, 1, B * H * Sk * D).reshape(B, H, Sk, D)
+    for ib, mul in enumerate((1.0, 6.0, 0.5)):
+        qf[:, :, 128 * ib:128 * (ib + 1)] *= np.float32(mul)
+    for jb, mul in enumerate((1.0, 4.0, 0.25, 2.0, 8.0)):
+        kf[:, :, 64 * jb:64 * (jb + 1)] *= np.float32(mul)
+    v = _bits(W.normal_f32(seed, 2, B * H * Sk * D).reshape(B, H, Sk, D))
+    z = oracle.sage_quant(_bits(qf), _bits(kf), qblk=128, kblk=64, smooth_k=False)
+    # per-block scales differ by the factors above, so a wrong block index cannot go unnoticed
+    assert z["sq"].max() / z["sq"].min() > 4 and z["sk"].max() / z["sk"].min() > 8
+    return z, v
+
+
+def _dequantised(z, Sq, Sk):
+    qd = z["qi8"].astype(np.float64) * np.repeat(z["sq"].astype(np.float64), 128, axis=-1)[..., :Sq, None]
+    kd = z["ki8"].astype(np.float64) * np.repeat(z["sk"].astype(np.float64), 64, axis=-1)[..., :Sk, None]
+    return qd, kd
+
+
+def test_sage_forward_against_fp64_brute_force_on_dequantised_operands(oracle):
+    """oracle_sage_fwd must equal textbook attention on Q~ = qi8 * sq[block], K~ = ki8 * sk[block]:
+    O (before rounding) and LSE within 2e-5, with and without the causal flag and key lengths,
+    Sq != Sk, short last blocks (200 = 128 + 72 queries, 150 = 64 + 64 + 22 keys)."""
+    B, H, Sq, Sk, D = 2, 2, 200, 150, 16
+    z, v = _sage_case(oracle, B, H, Sq, Sk, D, seed=31)
+    qd, kd = _dequantised(z, Sq, Sk)
+    vf = W.bf16_bits_to_f32(v).astype(np.float64)
+    scale = 0.03            # logits of a few units: fp32 rounding of the logits stays far below 2e-5
+    i = np.arange(Sq)[:, None]
+    j = np.arange(Sk)[None, :]
+    kv_len = np.array([150, 97], np.int32)
+    cases = {
+        "plain": (False, None, None),
+        "causal": (True, None, np.broadcast_to(j <= i, (B, H, Sq, Sk))),
+        "kv_len": (False, kv_len, np.broadcast_to((j < kv_len[:, None, None, None]), (B, H, Sq, Sk))),
+        "causal+kv_len": (True, kv_len, np.broadcast_to((j <= i) & (j < kv_len[:, None, None, None]), (B, H, Sq, Sk))),
+    }
+    for name, (causal, kvl, keep) in cases.items():
+        want_o, want_lse, _ = oracle.brute_sdpa_f64(qd, kd, vf, scale, keep=keep)
+        assert np.abs(want_lse).max() < 30 and np.abs(want_lse).max() > 1, name
+        _, lse, o32 = oracle.sage_fwd(z["qi8"], z["ki8"], z["sq"], z["sk"], v, scale, causal=causal, kv_len=kvl,
+                                      want_f32=True)
+        assert oracle.max_abs(o32, want_o) <= 2e-5, (name, oracle.max_abs(o32, want_o))
+        assert oracle.max_abs(lse, want_lse) <= 2e-5, (name, oracle.max_abs(lse, want_lse))
+    # the check has teeth: block scales indexed by the other operand's block size change the result
+    bad_sq = np.repeat(z["sq"], 2, axis=-1)[..., :z["sq"].shape[-1]]     # as if Q blocks were 64 rows
+    _, _, o_bad = oracle.sage_fwd(z["qi8"], z["ki8"], bad_sq, z["sk"], v, scale, want_f32=True)
+    want_o, _, _ = oracle.brute_sdpa_f64(qd, kd, vf, scale)
+    assert oracle.max_abs(o_bad, want_o) > 1e-2
+
+
+def test_sage_forward_row_and_head_ranges(oracle):
+    B, H, Sq, Sk, D = 1, 3, 200, 150, 16
+    z, v = _sage_case(oracle, B, H, Sq, Sk, D, seed=32)
+    full_o, full_lse = oracle.sage_fwd(z["qi8"], z["ki8"], z["sq"], z["sk"], v, 0.03, causal=True)
+    o, lse = oracle.sage_fwd(z["qi8"], z["ki8"], z["sq"], z["sk"], v, 0.03, causal=True, heads=(1, 2), rows=(120, 140))
+    assert np.array_equal(o[0, 1, 120:140], full_o[0, 1, 120:140]) and np.array_equal(lse[0, 1, 120:140], full_lse[0, 1, 120:140])
+    o[0, 1, 120:140] = 0
+    assert not o.any()
+
+
 def test_generator_is_a_pure_function_and_gaussian():
     a = W.normal_f32(123, 4, 200000)
     b = W.normal_f32(123, 4, 200000, chunk=777)

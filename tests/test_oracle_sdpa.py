@@ -232,3 +232,29 @@ def test_additive_bias_forward_against_torch_and_invariants(oracle):
     o_m, _ = oracle.sdpa_fwd(q, k, v, scale, mask=keep)
     o_b, _ = oracle.sdpa_fwd_bias(q, k, v, scale, ((1.0 - keep) * -1e9).astype(np.float32))
     assert np.array_equal(o_m, o_b)
+
+
+def test_row_bands_equal_the_full_computation(oracle):
+    """A band of query rows gives the rows of the full result bit for bit; under the causal flag the
+    last band alone already holds the whole dK / dV of the keys that only it attends to."""
+    B, H, S, D = 1, 3, 96, 8
+    q, k, v, do = (W.f32_to_bf16_bits(W.normal_f32(41, s, B * H * S * D).reshape(B, H, S, D)) for s in range(4))
+    scale = 0.3
+    o, lse, o32 = oracle.sdpa_fwd(q, k, v, scale, causal=True, want_f32=True)
+    dq, dk, dv, dq32, dk32, dv32 = oracle.sdpa_bwd(q, k, v, o, do, scale, causal=True, want_f32=True)
+    for r0, r1 in ((0, 16), (40, 56), (80, 96)):
+        bo, blse, bo32 = oracle.sdpa_fwd(q, k, v, scale, causal=True, heads=(1, 3), rows=(r0, r1), want_f32=True)
+        assert np.array_equal(bo[0, 1:, r0:r1], o[0, 1:, r0:r1]) and np.array_equal(blse[0, 1:, r0:r1], lse[0, 1:, r0:r1])
+        assert np.array_equal(bo32[0, 1:, r0:r1], o32[0, 1:, r0:r1])
+        bo[0, 1:, r0:r1] = 0
+        assert not bo.any()                      # nothing outside the band and the chosen heads is touched
+        bdq, bdk, bdv, bdq32, _, bdv32 = oracle.sdpa_bwd(q, k, v, o, do, scale, causal=True, heads=(1, 3),
+                                                         rows=(r0, r1), want_f32=True)
+        assert np.array_equal(bdq[0, 1:, r0:r1], dq[0, 1:, r0:r1]) and np.array_equal(bdq32[0, 1:, r0:r1], dq32[0, 1:, r0:r1])
+        if r1 == S:      # keys >= r0 are attended by queries >= r0 only
+            assert np.array_equal(bdk[0, 1:, r0:], dk[0, 1:, r0:]) and np.array_equal(bdv[0, 1:, r0:], dv[0, 1:, r0:])
+            assert not np.array_equal(bdv32[0, 1:, :r0], dv32[0, 1:, :r0])
+    # the bands of a non-causal problem add up to the whole dK / dV
+    _, _, _, _, dk32, dv32 = oracle.sdpa_bwd(q, k, v, o, do, scale, want_f32=True)
+    parts = [oracle.sdpa_bwd(q, k, v, o, do, scale, rows=r, want_f32=True) for r in ((0, 50), (50, 96))]
+    assert np.allclose(parts[0][4] + parts[1][4], dk32, atol=1e-5) and np.allclose(parts[0][5] + parts[1][5], dv32, atol=1e-5)
