@@ -133,9 +133,8 @@ def test_strided_views_match_contiguous(oracle):
 
     grads = tuple(bnhd(torch.empty_like(t)) for t in (q, k, v))
     got = capi.attn_bwd(bnhd(q), bnhd(k), bnhd(v), bnhd(o), bnhd(do), lse, w.scale, grads=grads)
-    for a, b_ in zip(got[1:], ref[1:]):
-        assert torch.equal(a, b_)            # dK, dV: no atomics, bit-identical
-    assert oracle.max_abs(to_f32(got[0]), to_f32(ref[0])) < 1e-2   # dQ: fp32 atomic order may differ
+    for a, b_ in zip(got, ref):
+        assert torch.equal(a, b_)            # the layout changes no arithmetic: dQ, dK, dV bit-identical
     _check_bwd(oracle, w)
 
 
