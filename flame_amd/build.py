@@ -21,10 +21,19 @@ FLAGS = [
 ]
 
 
+def hipcc_version() -> str:
+    """The compiler's own version line ("HIP version: ..." plus the clang version), one token string."""
+    out = subprocess.run([HIPCC, "--version"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True).stdout
+    hip = next((l.split(":", 1)[1].strip() for l in out.splitlines() if l.startswith("HIP version")), "?")
+    clang = next((l.strip() for l in out.splitlines() if "clang version" in l), "?")
+    clang = clang.split("clang version", 1)[1].split()[0] if "clang version" in clang else "?"
+    return f"{hip} clang-{clang}"
+
+
 def build_lib(verbose: bool = False, extra=()) -> str:
     os.makedirs(LIB_DIR, exist_ok=True)
     src = os.path.join(CSRC, "flame_attn.hip")
-    cmd = [HIPCC, *FLAGS, *extra, src, "-o", LIB_PATH]
+    cmd = [HIPCC, *FLAGS, f'-DFLAME_ATTN_HIPCC_VERSION="{hipcc_version()}"', *extra, src, "-o", LIB_PATH]
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)

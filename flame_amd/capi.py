@@ -133,6 +133,24 @@ def attn_bwd(q, k, v, o, do, lse, scale, causal=False, kv_len=None, mask=None, w
     return dq, dk, dv
 
 
+def cudnn_sdpa_bwd(q, k, v, o, do, stats, scale, grads=None):
+    """flame_cudnn_sdpa_bwd_bf16(...): the reference-named backward (no workspace argument)."""
+    B, H, Sq, D = q.shape
+    Sk = k.shape[2]
+    if grads is None:
+        grads = (torch.empty_like(q), torch.empty_like(k), torch.empty_like(v))
+    dq, dk, dv = grads
+    rc = lib().flame_cudnn_sdpa_bwd_bf16(
+        _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(do), _ptr(stats), _ptr(dq), _ptr(dk), _ptr(dv),
+        B, H, Sq, Sk, D, ctypes.c_float(scale),
+        _i64x4(q.stride()), _i64x4(k.stride()), _i64x4(v.stride()), _i64x4(o.stride()),
+        _i64x4(do.stride()), _i64x4(dq.stride()), _i64x4(dk.stride()), _i64x4(dv.stride()),
+        *(ctypes.c_int64(0) for _ in range(9)), _stream())
+    if rc != 0:
+        raise FlameAttnError("flame_cudnn_sdpa_bwd_bf16", rc)
+    return dq, dk, dv
+
+
 KERNEL_KINDS = ("fwd", "unused1", "bwd_dkdv", "bwd_dq", "sage_kmean", "sage_quant", "sage_fwd", "input_prep",
                 "bwd_merge", "reserved9", "reserved10", "reserved11")
 

@@ -1,6 +1,8 @@
 // C ABI of the gfx950 attention library: argument validation and kernel launches.
-// No allocation, no host synchronisation, no global state: every call only enqueues kernels on the
-// caller's stream, so calls may be captured into a HIP graph.
+// The primary entry points only enqueue kernels on the caller's stream (no allocation, no host
+// synchronisation), so they may be captured into a HIP graph.  Process-wide state kept here: the
+// optional per-kernel event profiler, the cached compute-unit count and workgroup-width override, the
+// and the per-stream scratch buffers of the reference-named backward shim (which has no workspace argument).
 #include "../../include/flame_attn.h"
 
 #include <algorithm>
@@ -37,9 +39,13 @@ int check_view(const void* base, const int64_t* st, int64_t off) {
 
 Strides mk(const int64_t* st) { return Strides{st[0], st[1], st[2]}; }
 
-int env_int(const char* name, int dflt) {
-    const char* v = getenv(name);
-    return v ? atoi(v) : dflt;
+// FLAME_ATTN_WG_WAVES=4 forces 128-query workgroups in the forward and dQ kernels (read once per process)
+int wg_waves_override() {
+    static const int value = [] {
+        const char* v = getenv("FLAME_ATTN_WG_WAVES");
+        return v ? atoi(v) : 8;
+    }();
+    return value;
 }
 
 
@@ -69,7 +75,9 @@ struct Profiler {
     }
 };
 Profiler g_prof;
+#ifdef FLAME_ATTN_PHASE_TIMING
 unsigned long long* g_phase_cycles = nullptr;   // device buffer set by flame_attn_debug_set_phase_buffer
+#endif
 
 struct ScopedKernelTimer {
     hipEvent_t stop_ev = nullptr;
@@ -187,7 +195,7 @@ int launch_bwd(const BwdParams& p, hipStream_t s) {
     // 256-query workgroups (4 wavefronts of 64 queries) when they neither add padding rows nor leave compute units idle
     const int64_t n256 = (p.Sq + 255) / 256;
     const bool wide = !HASMASK && n256 * 256 <= ((int64_t)(p.Sq + 127) / 128) * 128 && n256 * p.B * p.H >= device_cu_count() &&
-                      env_int("FLAME_ATTN_WG_WAVES", 8) != 4;
+                      wg_waves_override() != 4;
     const int64_t n_qt = wide ? n256 : (p.Sq + TQ::BM - 1) / TQ::BM;
     const int64_t grid_dq = n_qt * p.B * p.H;
     if (grid > 0x7fffffff || grid_dq > 0x7fffffff) return FLAME_ATTN_ERR_UNSUPPORTED;
@@ -243,10 +251,14 @@ int launch_bwd(const BwdParams& p, hipStream_t s) {
 
 extern "C" {
 
+#ifdef FLAME_ATTN_PHASE_TIMING
+// Development builds only: device buffer of 6 uint64 per workgroup that the timing build of the dK/dV
+// kernel fills with per-phase cycle counts (null switches it off again).
 int flame_attn_debug_set_phase_buffer(void* device_buffer) {
     g_phase_cycles = static_cast<unsigned long long*>(device_buffer);
     return FLAME_ATTN_OK;
 }
+#endif
 
 int flame_attn_profiling_enable(int on) {
     std::lock_guard<std::mutex> g(g_prof.mu);
@@ -336,9 +348,12 @@ int flame_attn_bwd_bf16(const void* Q, const void* K, const void* V, const void*
     p.m.rows16 = keep_mask && p.m.sk == 1 && (reinterpret_cast<uintptr_t>(keep_mask) | (uintptr_t)p.m.sb | (uintptr_t)p.m.sh |
                                               (uintptr_t)p.m.sq) % 16 == 0;
     p.m.causal = causal ? 1 : 0;
-    p.phase_cycles = g_phase_cycles;
+    p.phase_cycles = nullptr;
     hipStream_t s = static_cast<hipStream_t>(stream);
+#ifdef FLAME_ATTN_PHASE_TIMING
+    p.phase_cycles = g_phase_cycles;
     if (D == 128 && !keep_mask && g_phase_cycles) return launch_bwd<128, false, true>(p, s);   // phase-timing build
+#endif
     if (D == 128) return keep_mask ? launch_bwd<128, true>(p, s) : launch_bwd<128, false>(p, s);
     return keep_mask ? launch_bwd<64, true>(p, s) : launch_bwd<64, false>(p, s);
 }
@@ -506,7 +521,7 @@ static int attn_fwd_impl(const void* Q, const void* K, const void* V, void* O, v
     // without a workgroup
     const int64_t n256 = (N_q + 255) / 256;
     const bool wide = !hm && n256 * 256 <= ((N_q + 127) / 128) * 128 && n256 * B * H >= device_cu_count() &&
-                      env_int("FLAME_ATTN_WG_WAVES", 8) != 4;      // FLAME_ATTN_WG_WAVES=4 forces 128-query workgroups
+                      wg_waves_override() != 4;
     // ... as 4 wavefronts of 64 queries when nothing is excluded at all, else as 8 wavefronts of 32
     const bool plain = !causal && kv_len == nullptr && N_kv % 64 == 0;
     // a keep-mask with vector-loadable rows over whole tiles and no bias: the lean masked kernel
@@ -581,34 +596,46 @@ int flame_cudnn_sdpa_bf16_train_fwd(const void* Q, const void* K, const void* V,
 
 namespace {
 // Scratch for the reference-signature backward, which has no workspace argument: one lazily grown
-// buffer per device (the reference's shim likewise keeps a workspace it allocated once per shape).
-// Calls that overlap on one device share it and therefore race; callers that need concurrency or
-// graph capture from the first call use flame_attn_bwd_bf16 with their own workspace.
+// buffer per (device, stream), as the reference's shim keeps a workspace it allocated once per shape.
+// Calls on one stream are ordered, so they may share a buffer; calls on different streams get
+// different buffers and cannot race.  A buffer that has to grow is replaced by a new allocation and
+// kept until the process ends: a kernel still running on it keeps valid memory (a hipFree would
+// synchronise the device and, in a capture, fail).  hipMalloc happens on first use or growth only, so
+// the first call with a given stream and size class cannot be captured into a graph.
+struct BwdScratchSlot {
+    int dev;
+    hipStream_t stream;
+    void* ptr;
+    size_t bytes;
+};
 struct BwdScratch {
     std::mutex mu;
-    void* ptr[64] = {};
-    size_t bytes[64] = {};
+    std::vector<BwdScratchSlot> slots;
+    std::vector<void*> retired;
 };
 BwdScratch g_bwd_scratch;
 
-int bwd_scratch_get(size_t need, void** out) {
+int bwd_scratch_get(size_t need, hipStream_t stream, void** out) {
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return (int)e;
-    if (dev < 0 || dev >= 64) return FLAME_ATTN_ERR_UNSUPPORTED;
     std::lock_guard<std::mutex> g(g_bwd_scratch.mu);
-    if (g_bwd_scratch.bytes[dev] < need) {
-        if (g_bwd_scratch.ptr[dev]) {
-            e = hipFree(g_bwd_scratch.ptr[dev]);      // synchronises: earlier users are done
-            if (e != hipSuccess) return (int)e;
-            g_bwd_scratch.ptr[dev] = nullptr;
-            g_bwd_scratch.bytes[dev] = 0;
-        }
-        e = hipMalloc(&g_bwd_scratch.ptr[dev], need);
-        if (e != hipSuccess) return (int)e;
-        g_bwd_scratch.bytes[dev] = need;
+    BwdScratchSlot* slot = nullptr;
+    for (auto& sl : g_bwd_scratch.slots)
+        if (sl.dev == dev && sl.stream == stream) slot = &sl;
+    if (!slot) {
+        g_bwd_scratch.slots.push_back(BwdScratchSlot{dev, stream, nullptr, 0});
+        slot = &g_bwd_scratch.slots.back();
     }
-    *out = g_bwd_scratch.ptr[dev];
+    if (slot->bytes < need) {
+        void* fresh = nullptr;
+        e = hipMalloc(&fresh, need);
+        if (e != hipSuccess) return (int)e;
+        if (slot->ptr) g_bwd_scratch.retired.push_back(slot->ptr);
+        slot->ptr = fresh;
+        slot->bytes = need;
+    }
+    *out = slot->ptr;
     return FLAME_ATTN_OK;
 }
 
@@ -660,7 +687,7 @@ int flame_cudnn_sdpa_bwd_bf16(const void* Q, const void* K, const void* V, const
     const size_t need = flame_attn_bwd_workspace_bytes(B, H, N_q, D);
     if (need == 0) return FLAME_ATTN_ERR_INVALID;
     void* ws = nullptr;
-    int rc = bwd_scratch_get(need, &ws);
+    int rc = bwd_scratch_get(need, static_cast<hipStream_t>(stream), &ws);
     if (rc) return rc;
     return flame_attn_bwd_bf16(Q, K, V, O, dO, Stats, dQ, dK, dV, B, H, N_q, N_kv, D, scale, q_strides, k_strides,
                                v_strides, o_strides, do_strides, dq_strides, dk_strides, dv_strides, q_offset_elems,
@@ -838,6 +865,11 @@ int flame_attn_prep_rmsnorm_rope_bf16(const void* X, const void* weight, const v
     return e == hipSuccess ? FLAME_ATTN_OK : (int)e;
 }
 
-const char* flame_attn_version(void) { return "flame-attn-gfx950 0.1"; }
+#ifndef FLAME_ATTN_HIPCC_VERSION
+#define FLAME_ATTN_HIPCC_VERSION "unknown"
+#endif
+// names the compiler that built this library: the static checks of the hand-emitted instructions are
+// only meaningful for the assembly that this very compiler generates
+const char* flame_attn_version(void) { return "flame-attn-gfx950 0.2 (hipcc " FLAME_ATTN_HIPCC_VERSION ")"; }
 
 }  // extern "C"

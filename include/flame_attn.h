@@ -154,10 +154,11 @@ int flame_cudnn_sdpa_bf16_train_fwd(const void* Q, const void* K, const void* V,
                                     int64_t o_offset_elems, int64_t stats_offset_elems, void* stream);
 
 /* src/cuda/ffi.rs:682-716 (src/cuda/cudnn_sdpa_bwd.cpp:265-361).  The reference signature has no
- * workspace argument: this shim keeps one lazily grown scratch buffer per device (hipMalloc on first
- * use or growth, as the reference's shim does at src/cuda/cudnn_sdpa.cpp:204-212), so overlapping
- * calls on one device race and the first call cannot be captured into a graph.  Use
- * flame_attn_bwd_bf16 when either matters. */
+ * workspace argument: this shim keeps one lazily grown scratch buffer per (device, stream), as the
+ * reference's shim keeps a workspace per shape (src/cuda/cudnn_sdpa.cpp:204-212).  Calls on different
+ * streams use different buffers and may overlap; a buffer that must grow is replaced, never freed, so
+ * work in flight keeps valid memory.  hipMalloc happens on the first call of a stream and on growth
+ * only: such a call cannot be captured into a graph (use flame_attn_bwd_bf16 there). */
 int flame_cudnn_sdpa_bwd_bf16(const void* Q, const void* K, const void* V, const void* O, const void* dO,
                               const void* Stats, void* dQ, void* dK, void* dV,
                               int B, int H, int N_q, int N_kv, int D, float scale,
@@ -216,9 +217,6 @@ typedef struct {
 int flame_attn_profiling_enable(int on);
 /* Waits for the recorded events and returns per-kernel sums since the last read. */
 int flame_attn_profiling_read(FlameAttnKernelTimes* out);
-/* Device buffer of 6 uint64 per workgroup that the dK/dV kernel fills with per-phase cycle counts
- * (null switches the timing build of the kernel off again). */
-int flame_attn_debug_set_phase_buffer(void* device_buffer);
 
 /* ------------------------------------------------------------------------------------------------
  * Small conversions the host layer needs at the boundary.
@@ -257,6 +255,7 @@ int flame_attn_prep_rmsnorm_rope_bf16(const void* X, const void* weight, const v
                                       int apply_norm, const int64_t* x_strides, const int64_t* y_strides,
                                       int64_t x_off, int64_t y_off, void* stream);
 
+/* "flame-attn-gfx950 <version> (hipcc <version of the compiler that built the library>)" */
 const char* flame_attn_version(void);
 
 #ifdef __cplusplus

@@ -156,3 +156,39 @@ def test_stream_symbol_reports_reason_when_unsupported(oracle):
     ok = lib.sdpa_stream_bf16_launch(_p(q), _p(k), _p(v), _p(o), B, H, Q, K, D, ctypes.c_float(0.125), None,
                                      *_z(4), 12, 128, 96, _stream(), reason, 256)
     assert not ok and b"q_tile" in reason.value
+
+
+def test_cudnn_named_backward_on_two_streams_at_once():
+    """flame_cudnn_sdpa_bwd_bf16 keeps its scratch per stream: calls of different shapes enqueued on two
+    streams back to back, and a growing shape on a stream whose earlier call may still be running, give
+    the results of the same calls made one at a time (same kernels and schedule: bit-identical)."""
+    from flame_amd import capi
+
+    def problem(seed, B, H, S, D):
+        t = [to_dev(W.f32_to_bf16_bits(W.normal_f32(seed, s, B * H * S * D).reshape(B, H, S, D))) for s in range(4)]
+        o, lse = capi.attn_fwd(t[0], t[1], t[2], 1.0 / math.sqrt(D))
+        return (*t[:3], o, t[3], lse, 1.0 / math.sqrt(D))
+
+    pa = problem(71, 1, 12, 3456, 128)     # splits its last dK/dV round: uses the partial-sum part of the scratch
+    pb = problem(72, 2, 6, 1024, 64)
+    pc = problem(73, 1, 16, 4096, 128)     # larger than pa: the scratch of pa's stream has to grow
+    torch.cuda.synchronize()
+    want = [capi.cudnn_sdpa_bwd(*p) for p in (pa, pb, pc)]
+    torch.cuda.synchronize()
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    got = [None, None, None]
+    for _ in range(3):
+        with torch.cuda.stream(s1):
+            got[0] = capi.cudnn_sdpa_bwd(*pa)
+        with torch.cuda.stream(s2):
+            got[1] = capi.cudnn_sdpa_bwd(*pb)
+        with torch.cuda.stream(s1):
+            got[2] = capi.cudnn_sdpa_bwd(*pc)        # grows while pa may still be running on s1
+        with torch.cuda.stream(s2):
+            again = capi.cudnn_sdpa_bwd(*pb)
+        torch.cuda.synchronize()
+        for w_, g_ in zip(want, got):
+            for a, b in zip(w_, g_):
+                assert torch.equal(a, b)
+        for a, b in zip(want[1], again):
+            assert torch.equal(a, b)

@@ -35,10 +35,25 @@ def text():
         pytest.skip("hipcc not available")
     with tempfile.TemporaryDirectory() as tmp:
         out = os.path.join(tmp, "flame_attn.s")
-        flags = [f for f in fb.FLAGS if f not in ("-shared", "-fPIC")]
+        flags = [f for f in fb.FLAGS if f not in ("-shared", "-fPIC")]     # the flags the library is built with
         subprocess.run([fb.HIPCC, *flags, "-S", "--cuda-device-only", SRC, "-o", out], check=True,
                        stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
         return open(out).read()
+
+
+def test_checks_run_on_the_compiler_that_built_the_library():
+    """The assembly inspected here comes from this machine's hipcc; the shipped library records the hipcc
+    that built it.  The checks say nothing about the library unless the two are the same compiler."""
+    import ctypes
+    lib_path = fb.LIB_PATH
+    if not os.path.exists(lib_path):
+        pytest.skip("library not built")
+    if shutil.which(fb.HIPCC) is None and not os.path.exists(fb.HIPCC):
+        pytest.skip("hipcc not available")
+    lib = ctypes.CDLL(lib_path)
+    lib.flame_attn_version.restype = ctypes.c_char_p
+    built_with = lib.flame_attn_version().decode()
+    assert f"(hipcc {fb.hipcc_version()})" in built_with, (built_with, fb.hipcc_version())
 
 
 def test_hand_emitted_mfma_results_are_not_touched_too_early(text):
