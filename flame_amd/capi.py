@@ -15,13 +15,14 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("FLAME_ATTN_LIB") or os.path.join(_HERE, "lib", "libflame_attn_hip.so")
 _lib = None
 
-OK, ERR_INVALID, ERR_UNSUPPORTED = 0, -1, -2
+OK, ERR_INVALID, ERR_UNSUPPORTED, ERR_TOO_LARGE = 0, -1, -2, -3
 
 
 class FlameAttnError(RuntimeError):
     def __init__(self, fn: str, code: int):
         self.code = code
-        kind = {ERR_INVALID: "invalid argument", ERR_UNSUPPORTED: "unsupported"}.get(code, "HIP error")
+        kind = {ERR_INVALID: "invalid argument", ERR_UNSUPPORTED: "unsupported",
+                ERR_TOO_LARGE: "too many query rows for the fixed scratch"}.get(code, "HIP error")
         super().__init__(f"{fn} failed: {kind} ({code})")
 
 
@@ -130,6 +131,25 @@ def attn_bwd(q, k, v, o, do, lse, scale, causal=False, kv_len=None, mask=None, w
         _ptr(workspace), ctypes.c_size_t(workspace.numel()), _stream())
     if rc != 0:
         raise FlameAttnError("flame_attn_bwd_bf16", rc)
+    return dq, dk, dv
+
+
+def attn_bwd_noalloc(q, k, v, o, do, lse, scale, grads, causal=False, kv_len=None, mask=None):
+    """flame_attn_bwd_bf16_noalloc(...): the backward on the library's fixed device scratch.  The caller
+    passes the gradient tensors; nothing is allocated on the way."""
+    B, H, Sq, D = q.shape
+    Sk = k.shape[2]
+    dq, dk, dv = grads
+    ms = _mask_strides(mask, B, H, Sq, Sk)
+    rc = lib().flame_attn_bwd_bf16_noalloc(
+        _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(do), _ptr(lse), _ptr(dq), _ptr(dk), _ptr(dv),
+        B, H, Sq, Sk, D, ctypes.c_float(scale),
+        _i64x4(q.stride()), _i64x4(k.stride()), _i64x4(v.stride()), _i64x4(o.stride()),
+        _i64x4(do.stride()), _i64x4(dq.stride()), _i64x4(dk.stride()), _i64x4(dv.stride()),
+        *(ctypes.c_int64(0) for _ in range(9)),
+        int(bool(causal)), _ptr(kv_len), _ptr(mask), ms, _stream())
+    if rc != 0:
+        raise FlameAttnError("flame_attn_bwd_bf16_noalloc", rc)
     return dq, dk, dv
 
 

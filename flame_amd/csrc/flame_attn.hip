@@ -2,7 +2,8 @@
 // The primary entry points only enqueue kernels on the caller's stream (no allocation, no host
 // synchronisation), so they may be captured into a HIP graph.  Process-wide state kept here: the
 // optional per-kernel event profiler, the cached compute-unit count and workgroup-width override, the
-// and the per-stream scratch buffers of the reference-named backward shim (which has no workspace argument).
+// per-stream scratch buffers of the reference-named backward shim (which has no workspace argument),
+// and the per-device address of the static scratch of the allocation-free backward.
 #include "../../include/flame_attn.h"
 
 #include <algorithm>
@@ -639,6 +640,38 @@ int bwd_scratch_get(size_t need, hipStream_t stream, void** out) {
     return FLAME_ATTN_OK;
 }
 
+// Scratch of the allocation-free backward: a fixed array in device memory that every GPU the library
+// runs on holds until the process ends.  Layout as the caller workspace of flame_attn_bwd_bf16: two fp32
+// rows per query (at most FLAME_ATTN_NOALLOC_MAX_ROWS queries over all batches and heads), then the fp32
+// dK/dV partial sums of the split key blocks.  The name below is a host-side stand-in: the address the
+// kernels are given comes from hipGetSymbolAddress, once per device.
+constexpr size_t kNoallocRowsBytes = 2 * (size_t)FLAME_ATTN_NOALLOC_MAX_ROWS * sizeof(float);
+constexpr size_t kNoallocSplitBytes = (size_t)32 << 20;
+static __device__ __align__(256) unsigned char scratch[kNoallocRowsBytes + kNoallocSplitBytes];
+
+struct NoallocScratch {
+    std::mutex mu;
+    void* ptr[64] = {};
+};
+NoallocScratch g_noalloc;
+
+int noalloc_scratch_get(void** out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= 64) return FLAME_ATTN_ERR_UNSUPPORTED;
+    std::lock_guard<std::mutex> g(g_noalloc.mu);
+    if (!g_noalloc.ptr[dev]) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (!ptr) return FLAME_ATTN_ERR_UNSUPPORTED;
+        g_noalloc.ptr[dev] = ptr;
+    }
+    *out = g_noalloc.ptr[dev];
+    return FLAME_ATTN_OK;
+}
+
 // bf16 keep-mask (>= 0.5 attends) -> uint8 keep-mask, contiguous
 __global__ void mask_bf16_to_u8_kernel(const uint16_t* src, uint8_t* dst, int64_t n, int invert) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -694,6 +727,32 @@ int flame_cudnn_sdpa_bwd_bf16(const void* Q, const void* K, const void* V, const
                                k_offset_elems, v_offset_elems, o_offset_elems, do_offset_elems, stats_offset_elems,
                                dq_offset_elems, dk_offset_elems, dv_offset_elems, 0, nullptr, nullptr, nullptr, ws,
                                need, stream);
+}
+
+int flame_attn_bwd_noalloc_max_rows(void) { return FLAME_ATTN_NOALLOC_MAX_ROWS; }
+
+int flame_attn_bwd_bf16_noalloc(const void* Q, const void* K, const void* V, const void* O, const void* dO,
+                                const void* LSE, void* dQ, void* dK, void* dV,
+                                int B, int H, int N_q, int N_kv, int D, float scale,
+                                const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                                const int64_t* o_strides, const int64_t* do_strides, const int64_t* dq_strides,
+                                const int64_t* dk_strides, const int64_t* dv_strides,
+                                int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off, int64_t do_off,
+                                int64_t lse_off, int64_t dq_off, int64_t dk_off, int64_t dv_off,
+                                int causal, const int32_t* kv_len,
+                                const uint8_t* keep_mask, const int64_t* mask_strides, void* stream) {
+    if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0) return FLAME_ATTN_ERR_INVALID;
+    if ((int64_t)B * H * N_q > FLAME_ATTN_NOALLOC_MAX_ROWS) return FLAME_ATTN_ERR_TOO_LARGE;
+    void* ws = nullptr;
+    int rc = noalloc_scratch_get(&ws);
+    if (rc) return rc;
+    // The row part is sized for this call, so the partial sums start where flame_attn_bwd_bf16 expects
+    // them; every byte the kernels read from the scratch was written earlier in the same call.
+    const size_t bytes = bwd_rows_bytes(B, H, N_q) + kNoallocSplitBytes;
+    return flame_attn_bwd_bf16(Q, K, V, O, dO, LSE, dQ, dK, dV, B, H, N_q, N_kv, D, scale, q_strides, k_strides,
+                               v_strides, o_strides, do_strides, dq_strides, dk_strides, dv_strides, q_off, k_off,
+                               v_off, o_off, do_off, lse_off, dq_off, dk_off, dv_off, causal, kv_len, keep_mask,
+                               mask_strides, ws, bytes, stream);
 }
 
 int flame_flash_attention_bf16(const void* Q, const void* K, const void* V, void* O, float* LSE,

@@ -43,6 +43,7 @@ extern "C" {
 #define FLAME_ATTN_OK 0
 #define FLAME_ATTN_ERR_INVALID (-1)
 #define FLAME_ATTN_ERR_UNSUPPORTED (-2)
+#define FLAME_ATTN_ERR_TOO_LARGE (-3)   /* flame_attn_bwd_bf16_noalloc only: more query rows than its fixed scratch holds */
 
 /* Status enum of the reference's flame_* / fc_* family (cuda/include/flame_cuda_status.h:7-12). */
 typedef enum {
@@ -109,6 +110,29 @@ int flame_attn_bwd_bf16(const void* Q, const void* K, const void* V, const void*
                         const uint8_t* keep_mask, const int64_t* mask_strides,
                         void* workspace, size_t workspace_bytes, void* stream);
 
+/* The same backward for callers that cannot allocate device memory and have no workspace to hand over:
+ * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart
+ * in the reference.  The scratch is a fixed array in device memory that every GPU the library runs on
+ * holds until the process ends (40 MiB: two fp32 rows for up to FLAME_ATTN_NOALLOC_MAX_ROWS query rows,
+ * 32 MiB of fp32 dK/dV partial sums); the call allocates and frees nothing.
+ * B * H * N_q above FLAME_ATTN_NOALLOC_MAX_ROWS returns FLAME_ATTN_ERR_TOO_LARGE and launches nothing.
+ * All calls on one GPU share that array: calls that overlap on one GPU (different streams, or host
+ * threads on different streams) race; calls on one stream are ordered and safe.  Nothing in the array
+ * has to start at zero and nothing is kept between calls.  Results are bit-identical to
+ * flame_attn_bwd_bf16 with a workspace of flame_attn_bwd_workspace_bytes(...) bytes. */
+#define FLAME_ATTN_NOALLOC_MAX_ROWS (1 << 20)
+int flame_attn_bwd_noalloc_max_rows(void);
+int flame_attn_bwd_bf16_noalloc(const void* Q, const void* K, const void* V, const void* O, const void* dO,
+                                const void* LSE, void* dQ, void* dK, void* dV,
+                                int B, int H, int N_q, int N_kv, int D, float scale,
+                                const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                                const int64_t* o_strides, const int64_t* do_strides, const int64_t* dq_strides,
+                                const int64_t* dk_strides, const int64_t* dv_strides,
+                                int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off, int64_t do_off,
+                                int64_t lse_off, int64_t dq_off, int64_t dk_off, int64_t dv_off,
+                                int causal, const int32_t* kv_len,
+                                const uint8_t* keep_mask, const int64_t* mask_strides, void* stream);
+
 /* ------------------------------------------------------------------------------------------------
  * SageAttention int8-QK inference variant (API shape: src/sage_attention.rs:21-65; quantiser closed
  * form: src/sage_attention.rs:524-541; block granularity, K mean smoothing and int8 MFMA are new).
@@ -158,7 +182,8 @@ int flame_cudnn_sdpa_bf16_train_fwd(const void* Q, const void* K, const void* V,
  * reference's shim keeps a workspace per shape (src/cuda/cudnn_sdpa.cpp:204-212).  Calls on different
  * streams use different buffers and may overlap; a buffer that must grow is replaced, never freed, so
  * work in flight keeps valid memory.  hipMalloc happens on the first call of a stream and on growth
- * only: such a call cannot be captured into a graph (use flame_attn_bwd_bf16 there). */
+ * only: such a call cannot be captured into a graph (use flame_attn_bwd_bf16 or
+ * flame_attn_bwd_bf16_noalloc there). */
 int flame_cudnn_sdpa_bwd_bf16(const void* Q, const void* K, const void* V, const void* O, const void* dO,
                               const void* Stats, void* dQ, void* dK, void* dV,
                               int B, int H, int N_q, int N_kv, int D, float scale,
