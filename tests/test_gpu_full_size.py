@@ -70,10 +70,10 @@ def test_cfg4_long_causal_full_size(oracle):
     _, lse = capi.attn_fwd(q, k, v, w.scale, causal=True, out=o)
     capi.attn_bwd(q, k, v, o, do, lse, w.scale, causal=True, workspace=ws, grads=(dq, dk, dv))
     torch.cuda.synchronize()
-    tensors = 9 * q.numel() * 2 + lse.numel() * 4
+    tensors = 8 * q.numel() * 2 + lse.numel() * 4      # Q, K, V, dO, O, dQ, dK, dV
     peak = torch.cuda.max_memory_allocated() - base
     extra = peak - tensors
-    print(f"      device memory: peak {peak / 2**20:.1f} MiB = 9 tensors + LSE {tensors / 2**20:.1f} MiB + {extra / 2**20:.1f} MiB "
+    print(f"      device memory: peak {peak / 2**20:.1f} MiB = 8 tensors + LSE {tensors / 2**20:.1f} MiB + {extra / 2**20:.1f} MiB "
           f"(declared workspace {ws_bytes / 2**20:.1f} MiB; a materialised bf16 P would be {H * S * S * 2 / 2**30:.0f} GiB)", flush=True)
     assert extra <= ws_bytes + (1 << 20)            # allocator rounding only; never O(S^2)
     assert ws_bytes <= 64 << 20
@@ -103,12 +103,12 @@ def test_cfg4_long_causal_full_size(oracle):
     rel = float((sum_dv - sum_do).norm() / sum_do.norm())
     worst = float(((sum_dv - sum_do).norm(dim=-1) / sum_do.norm(dim=-1)).max())
     print(f"      sum_j dV_j vs sum_i dO_i: rel-L2 {rel:.3e}, worst head {worst:.3e}", flush=True)
-    assert worst <= 5e-3
+    assert worst <= 1e-3
     sum_dk = dk.double().sum(dim=2).abs()
     abs_dk = dk.double().abs().sum(dim=2)
     ratio = float((sum_dk / abs_dk).max())
     print(f"      |sum_j dK_j| / sum_j |dK_j|: worst (head, channel) {ratio:.3e}", flush=True)
-    assert ratio <= 2e-3
+    assert ratio <= 1e-3
     assert bool(torch.isfinite(dq.float()).all()) and bool(torch.isfinite(dk.float()).all())
     # the first key of every head is attended by every query: its dV is the P-weighted sum of all dO rows,
     # and the last key by the last query alone, with weight P = exp(s - LSE) of that one pair
