@@ -110,8 +110,8 @@ def test_cfg4_long_causal_full_size(oracle):
     print(f"      |sum_j dK_j| / sum_j |dK_j|: worst (head, channel) {ratio:.3e}", flush=True)
     assert ratio <= 1e-3
     assert bool(torch.isfinite(dq.float()).all()) and bool(torch.isfinite(dk.float()).all())
-    # the first key of every head is attended by every query: its dV is the P-weighted sum of all dO rows,
-    # and the last key by the last query alone, with weight P = exp(s - LSE) of that one pair
+    # the last key of every head is attended by the last query alone: dV there is P * dO of that one pair,
+    # with P = exp(s - LSE)
     last = S - 1
     s_last = (q[0, :, last].float() * k[0, :, last].float()).sum(-1) * w.scale
     p_last = torch.exp(s_last - lse.view(B, H, S)[0, :, last])
