@@ -131,7 +131,7 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
 
     int klimit = p.Sk;
     if (p.m.kv_len) klimit = min(klimit, max(p.m.kv_len[b], 0));
-    const uint8_t* mbase = HASMASK ? p.m.mask + b * p.m.sb + hh * p.m.sh : nullptr;
+    const uint8_t* mbase = HASMASK ? mask_head_base(p.m, b, hh) : nullptr;
 
     const int n_qt = (p.Sq + BM - 1) / BM;
     int qt_begin = p.m.causal ? (k0 / BM) : 0;
@@ -373,13 +373,13 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
         // (a load per element inside the pipelined slices would wait out a memory round trip each time)
         uint32_t mk[2][16];
         if (HASMASK && !VECMASK && MASKED) {
-            const uint8_t* mkey = mbase + (int64_t)min(key, p.Sk - 1) * p.m.sk;
+            const int64_t mkey = (int64_t)min(key, p.Sk - 1) * p.m.sk;
 #pragma unroll
             for (int qb = 0; qb < 2; ++qb)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int qi = q0 + 32 * qb + 8 * (r >> 2) + 4 * h + (r & 3);
-                    mk[qb][r] = mkey[(int64_t)min(qi, p.Sq - 1) * p.m.sq];
+                    mk[qb][r] = mask_attends(p.m, mbase, mkey + (int64_t)min(qi, p.Sq - 1) * p.m.sq) ? 1u : 0u;
                 }
         }
         // lse2 is read one group of four queries ahead of its use, so that waiting for it never drains
@@ -760,7 +760,7 @@ __global__ __launch_bounds__(64 * NW, (NW == 4 && (!HASMASK || VECMASK)) ? 2 : 1
     int kend = klimit;
     if (p.m.causal) kend = min(kend, q0 + BM);
     const int n_tiles = (kend + BN - 1) / BN;
-    const uint8_t* mbase = HASMASK ? p.m.mask + b * p.m.sb + hh * p.m.sh : nullptr;
+    const uint8_t* mbase = HASMASK ? mask_head_base(p.m, b, hh) : nullptr;
 
     // ---- Q and dO fragments (B operands: column = query, 8 consecutive d), per-query scalars
     const int qrow = qw0 + n;
@@ -928,7 +928,7 @@ __global__ __launch_bounds__(64 * NW, (NW == 4 && (!HASMASK || VECMASK)) ? 2 : 1
                 bool drop = (key >= klimit) | ((p.m.causal != 0) & (key > qrow));     // bitwise: selects, not branches
                 if (HASMASK) {
                     if (vec_mask) drop = drop || !mrow.keep(kb, r, h);
-                    else if (!drop && qok) drop = mbase[(int64_t)qrow * p.m.sq + (int64_t)key * p.m.sk] == 0;
+                    else if (!drop && qok) drop = !mask_attends(p.m, mbase, (int64_t)qrow * p.m.sq + (int64_t)key * p.m.sk);
                 }
                 pr = drop ? 0.f : pr;
             }

@@ -319,17 +319,35 @@ struct MaskRow64 {
     }
 };
 
+enum MaskMode : int {
+    kMaskU8 = 0,             // uint8, non-zero attends
+    kMaskBf16Keep = 1,       // bf16, a value below 0.5 excludes (the public keep-mask convention of the reference)
+    kMaskBf16Drop = 2,       // bf16, a value above 0.5 excludes (the convention of the reference's streaming entry point)
+};
+
 struct MaskArgs {
     const int32_t* kv_len;   // [B] or null
-    const uint8_t* mask;     // keep-mask (non-zero = attend) or null
+    const uint8_t* mask;     // explicit mask or null; element type and meaning per mask_mode
     int64_t sb, sh, sq, sk;  // element strides over (b,h,q,k); 0 broadcasts
     int causal;              // key j > query i is excluded
-    int rows16 = 0;          // keep-mask rows are contiguous along keys and 16-byte aligned (vector loads allowed)
+    int rows16 = 0;          // uint8 keep-mask rows are contiguous along keys and 16-byte aligned (vector loads allowed)
+    int mask_mode = kMaskU8;
     // additive bias on the scaled logits (forward only), fp32 or bf16, or null
     const void* bias = nullptr;
     int64_t bb = 0, bh = 0, bq = 0, bk = 0;   // element strides over (b,h,q,k); 0 broadcasts
     int bias_f32 = 1;
     float inv_scale = 1.f;   // 1 / softmax scale: the bias is folded into the raw scores as bias / scale
 };
+
+// one element of an explicit mask, addressed in elements from the (batch, head) base: does it attend?
+__device__ __forceinline__ bool mask_attends(const MaskArgs& m, const uint8_t* base, int64_t elem) {
+    if (m.mask_mode == kMaskU8) return base[elem] != 0;
+    const float v = __builtin_bit_cast(float, (uint32_t)reinterpret_cast<const uint16_t*>(base)[elem] << 16);
+    return m.mask_mode == kMaskBf16Keep ? !(v < 0.5f) : !(v > 0.5f);
+}
+// (batch, head) base of an explicit mask
+__device__ __forceinline__ const uint8_t* mask_head_base(const MaskArgs& m, int b, int hh) {
+    return m.mask + (b * m.sb + hh * m.sh) * (m.mask_mode == kMaskU8 ? 1 : 2);
+}
 
 }  // namespace fattn

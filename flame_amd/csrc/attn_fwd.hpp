@@ -95,7 +95,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void fwd_kernel(const Fwd
     int kend = klimit;
     if (p.m.causal) kend = min(kend, q0 + BM);
     const int n_tiles = (kend + BN - 1) / BN;
-    const uint8_t* mbase = (HASMASK && p.m.mask) ? p.m.mask + b * p.m.sb + hh * p.m.sh : nullptr;
+    const uint8_t* mbase = (HASMASK && p.m.mask) ? mask_head_base(p.m, b, hh) : nullptr;
     const char* bbase = (HASMASK && p.m.bias)
                             ? static_cast<const char*>(p.m.bias) + (b * p.m.bb + hh * p.m.bh) * (p.m.bias_f32 ? 4 : 2)
                             : nullptr;
@@ -218,7 +218,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void fwd_kernel(const Fwd
                 float val = s[kb][r];
                 if (HASMASK) {
                     if (vec_mask) drop = drop || !mrow.keep(kb, r, h);
-                    else if (mbase && !drop && qi < p.Sq) drop = mbase[(int64_t)qi * p.m.sq + (int64_t)key * p.m.sk] == 0;
+                    else if (mbase && !drop && qi < p.Sq) drop = !mask_attends(p.m, mbase, (int64_t)qi * p.m.sq + (int64_t)key * p.m.sk);
                     if (bbase) {      // scale * (s + bias / scale) = scale * s + bias
                         float bv = 0.f;
                         if (!drop && qi < p.Sq) {

@@ -478,7 +478,7 @@ static int attn_fwd_impl(const void* Q, const void* K, const void* V, void* O, v
                         int causal, const int32_t* kv_len,
                         const uint8_t* keep_mask, const int64_t* mask_strides,
                         const void* bias, int bias_dtype, const int64_t* bias_strides,
-                        void* stream) {
+                        void* stream, int mask_mode = kMaskU8) {
     if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0) return FLAME_ATTN_ERR_INVALID;
     if (!(scale > 0.f) || !isfinite(scale)) return FLAME_ATTN_ERR_INVALID;
     if (D != 64 && D != 128) return FLAME_ATTN_ERR_UNSUPPORTED;
@@ -506,8 +506,9 @@ static int attn_fwd_impl(const void* Q, const void* K, const void* V, void* O, v
     p.m.sh = keep_mask ? mask_strides[1] : 0;
     p.m.sq = keep_mask ? mask_strides[2] : 0;
     p.m.sk = keep_mask ? mask_strides[3] : 0;
-    p.m.rows16 = keep_mask && p.m.sk == 1 && (reinterpret_cast<uintptr_t>(keep_mask) | (uintptr_t)p.m.sb | (uintptr_t)p.m.sh |
-                                              (uintptr_t)p.m.sq) % 16 == 0;
+    p.m.mask_mode = mask_mode;
+    p.m.rows16 = keep_mask && mask_mode == kMaskU8 && p.m.sk == 1 &&
+                 (reinterpret_cast<uintptr_t>(keep_mask) | (uintptr_t)p.m.sb | (uintptr_t)p.m.sh | (uintptr_t)p.m.sq) % 16 == 0;
     p.m.causal = causal ? 1 : 0;
     p.m.bias = bias;
     if (bias) {
@@ -673,11 +674,9 @@ int noalloc_scratch_get(void** out) {
 }
 
 // bf16 keep-mask (>= 0.5 attends) -> uint8 keep-mask, contiguous
-__global__ void mask_bf16_to_u8_kernel(const uint16_t* src, uint8_t* dst, int64_t n, int invert) {
+__global__ void mask_bf16_to_u8_kernel(const uint16_t* src, uint8_t* dst, int64_t n) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= n) return;
-    const bool ge_half = __builtin_bit_cast(float, (uint32_t)src[i] << 16) >= 0.5f;
-    dst[i] = (ge_half != (invert != 0)) ? 1 : 0;
+    if (i < n) dst[i] = __builtin_bit_cast(float, (uint32_t)src[i] << 16) >= 0.5f ? 1 : 0;
 }
 __global__ void mask_f32_to_u8_kernel(const float* src, uint8_t* dst, int64_t n) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -783,23 +782,20 @@ FlameAttnStatus flame_sdpa_chunked_bf16(const void* q, const void* k, const void
     if (Dv != Dh) return FLAME_ATTN_STATUS_ERR_UNSUPPORTED;
     const int64_t qs[4] = {(int64_t)H * Q * Dh, (int64_t)Q * Dh, Dh, 1};
     const int64_t ks[4] = {(int64_t)H * K * Dh, (int64_t)K * Dh, Dh, 1};
-    const uint8_t* m8 = nullptr;
+    // bf16 keep-mask [B, mask_heads, Q, K], a value below 0.5 excludes: read in place by the masked kernel, so
+    // the workspace (which the reference sizes for its own score chunks) is not needed at all
+    (void)workspace; (void)workspace_bytes;
     int64_t ms[4] = {0, 0, 0, 0};
     if (mask) {
         if (mask_heads != 1 && mask_heads != H) return FLAME_ATTN_STATUS_ERR_INVALID;
-        const int64_t n = (int64_t)B * mask_heads * Q * K;
-        if (!workspace || workspace_bytes < (uint64_t)n) return FLAME_ATTN_STATUS_ERR_UNSUPPORTED;
-        hipLaunchKernelGGL(mask_bf16_to_u8_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
-                           static_cast<hipStream_t>(stream), static_cast<const uint16_t*>(mask),
-                           static_cast<uint8_t*>(workspace), n, 0);
-        m8 = static_cast<const uint8_t*>(workspace);
         ms[0] = (int64_t)mask_heads * Q * K;
         ms[1] = mask_heads == 1 ? 0 : (int64_t)Q * K;
         ms[2] = K;
         ms[3] = 1;
     }
-    return to_status(flame_attn_fwd_bf16(q, k, v, out, nullptr, B, H, Q, K, Dh, scale, qs, ks, ks, qs, 0, 0, 0, 0, 0,
-                                         causal, nullptr, m8, m8 ? ms : nullptr, stream));
+    return to_status(attn_fwd_impl(q, k, v, out, nullptr, B, H, Q, K, Dh, scale, qs, ks, ks, qs, 0, 0, 0, 0, 0, causal,
+                                   nullptr, static_cast<const uint8_t*>(mask), mask ? ms : nullptr, nullptr,
+                                   FLAME_ATTN_DTYPE_F32, nullptr, stream, kMaskBf16Keep));
 }
 
 int streaming_attn_bf16_fp32_launch(const void* Q, const void* K, const void* V, int B, int H, int S, int Dh, int Dv,
@@ -823,14 +819,16 @@ bool sdpa_stream_bf16_launch(const void* dQ, const void* dK, const void* dV, voi
         if (unsupported_reason && reason_buflen > 0) snprintf(unsupported_reason, (size_t)reason_buflen, "%s", why);
         return false;
     };
-    (void)mask_stride_ek; (void)mask_stride_eq; (void)mask_stride_eh; (void)mask_stride_eb; (void)head_tile;
+    (void)head_tile;
     if (q_tile > max_q_tile) return fail("q_tile exceeds max_q_tile");
-    if (attn_mask) return fail("bf16 masks are not taken here: pass a uint8 keep-mask to flame_attn_fwd_bf16");
     if (d != 64 && d != 128) return fail("head dim must be 64 or 128");
     const int64_t qs[4] = {(int64_t)H * Q_len * d, (int64_t)Q_len * d, d, 1};
     const int64_t ks[4] = {(int64_t)H * K_len * d, (int64_t)K_len * d, d, 1};
-    const int rc = flame_attn_fwd_bf16(dQ, dK, dV, dO, nullptr, B, H, Q_len, K_len, d, scale, qs, ks, ks, qs, 0, 0, 0,
-                                       0, 0, 0, nullptr, nullptr, nullptr, stream);
+    // bf16 mask addressed by the caller's four element strides; in this entry point a value above 0.5 EXCLUDES
+    const int64_t ms[4] = {mask_stride_eb, mask_stride_eh, mask_stride_eq, mask_stride_ek};
+    const int rc = attn_fwd_impl(dQ, dK, dV, dO, nullptr, B, H, Q_len, K_len, d, scale, qs, ks, ks, qs, 0, 0, 0, 0, 0, 0,
+                                 nullptr, static_cast<const uint8_t*>(attn_mask), attn_mask ? ms : nullptr, nullptr,
+                                 FLAME_ATTN_DTYPE_F32, nullptr, stream, kMaskBf16Drop);
     if (rc != FLAME_ATTN_OK) return fail(rc == FLAME_ATTN_ERR_INVALID ? "invalid argument" : "unsupported shape or HIP error");
     if (unsupported_reason && reason_buflen > 0) unsupported_reason[0] = 0;
     return true;
@@ -843,7 +841,7 @@ int flame_attn_convert_keep_mask(const void* src, int src_dtype, void* dst_u8, i
     if (n > (int64_t)0x7fffffff * 256) return FLAME_ATTN_ERR_UNSUPPORTED;
     if (src_dtype == FLAME_ATTN_DTYPE_BF16)
         hipLaunchKernelGGL(mask_bf16_to_u8_kernel, dim3(grid), dim3(256), 0, s, static_cast<const uint16_t*>(src),
-                           static_cast<uint8_t*>(dst_u8), n, 0);
+                           static_cast<uint8_t*>(dst_u8), n);
     else if (src_dtype == FLAME_ATTN_DTYPE_F32)
         hipLaunchKernelGGL(mask_f32_to_u8_kernel, dim3(grid), dim3(256), 0, s, static_cast<const float*>(src),
                            static_cast<uint8_t*>(dst_u8), n);

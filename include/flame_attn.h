@@ -201,8 +201,9 @@ int flame_flash_attention_bf16(const void* Q, const void* K, const void* V, void
                                int batch_heads, int seq_len_q, int seq_len_kv, int head_dim, void* stream);
 
 /* src/ffi/cuda_ffi.h:98-115 (cuda/src/flame_sdpa_stub.cu:869-1379): contiguous tensors, optional bf16
- * keep-mask [B, mask_heads, Q, K] (< 0.5 excluded, flame_sdpa_stub.cu:793-802) which is converted to
- * uint8 inside `workspace` (needs B*mask_heads*Q*K bytes there); Dv must equal Dh. */
+ * keep-mask [B, mask_heads, Q, K] (< 0.5 excluded, flame_sdpa_stub.cu:793-802), read in place by the
+ * kernel.  `workspace` is accepted and not used (the reference keeps its score chunks there,
+ * flame_sdpa_stub.cu:973-976), so any size, including none, works.  Dv must equal Dh. */
 FlameAttnStatus flame_sdpa_chunked_bf16(const void* q, const void* k, const void* v, int B, int H, int Q, int K,
                                         int Dh, int Dv, float scale, int chunk, int causal, int mask_heads,
                                         const void* mask, void* out, void* workspace, uint64_t workspace_bytes,
@@ -216,10 +217,12 @@ int streaming_attn_bf16_fp32_launch(const void* Q, const void* K, const void* V,
                                     float scale, int chunk_size, int causal, const uint8_t* k_pad_mask,
                                     void* stream);
 
-/* src/cuda_ops_ffi.rs:199-221 (cuda/sdpa_stream_bf16.cu:180-413): contiguous, d in {64,128}.  A bf16
- * mask (where >= 0.5 means EXCLUDED in that one entry point, cuda/include/sdpa_stream_bf16.h:30-33)
- * is reported as unsupported with a reason, which is the documented way for the caller to take its
- * other path (src/cuda_ops_bf16.rs:1955-2059). */
+/* src/cuda_ops_ffi.rs:199-221 (cuda/sdpa_stream_bf16.cu:180-413): contiguous Q, K, V, O.  attn_mask
+ * (may be null) is bf16, addressed by the four element strides, 0 broadcasting heads or batches
+ * (src/cuda_ops_bf16.rs:1848-1873); in this one entry point a value above 0.5 EXCLUDES the position
+ * (cuda/sdpa_stream_bf16.cu:79-81, cuda/include/sdpa_stream_bf16.h:30-33).  What is not built is
+ * reported as unsupported with a reason, which is the documented way for the caller to take its other
+ * path (src/cuda_ops_bf16.rs:1955-2059). */
 bool sdpa_stream_bf16_launch(const void* dQ, const void* dK, const void* dV, void* dO, int B, int H, int Q_len,
                              int K_len, int d, float scale, const void* attn_mask, int64_t mask_stride_ek,
                              int64_t mask_stride_eq, int64_t mask_stride_eh, int64_t mask_stride_eb, int head_tile,

@@ -90,13 +90,27 @@ def test_chunked_symbol_with_bf16_keep_mask_and_causal(oracle):
     keep[..., 0] = 1
     mask_bf16 = torch.from_numpy(keep.astype(np.float32)).to(torch.bfloat16).cuda()
     out = torch.empty_like(q)
-    ws = torch.empty(B * Q * K, dtype=torch.uint8, device="cuda")
-    rc = lib.flame_sdpa_chunked_bf16(_p(q), _p(k), _p(v), B, H, Q, K, D, D, ctypes.c_float(0.125), 64, 0, 1,
+    # workspace sized the way the reference's caller sizes it: 4 * (chunk * K + chunk * (Dv + 2)) bytes
+    # (cuda/src/flame_sdpa_stub.cu:973-976), far less than one byte per mask element times B*H
+    chunk = 8
+    ws = torch.empty(4 * (chunk * K + chunk * (D + 2)), dtype=torch.uint8, device="cuda")
+    rc = lib.flame_sdpa_chunked_bf16(_p(q), _p(k), _p(v), B, H, Q, K, D, D, ctypes.c_float(0.125), chunk, 0, 1,
                                      _p(mask_bf16), _p(out), _p(ws), ctypes.c_uint64(ws.numel()), _stream())
     assert rc == 0
     torch.cuda.synchronize()
     ro, _, ro32 = oracle.sdpa_fwd(t[0], t[1], t[2], 0.125, mask=keep, want_f32=True)
     assert_close_bf16(oracle, "O", to_f32(out), ro, ro32)
+    # ... and with no workspace at all; a mask per head; mask together with the causal flag
+    keep_h = (W.normal_f32(323, 0, B * H * Q * K).reshape(B, H, Q, K) > 0.1).astype(np.uint8)
+    keep_h[..., 0] = 1
+    mask_h = torch.from_numpy(keep_h.astype(np.float32)).to(torch.bfloat16).cuda()
+    for causal in (0, 1):
+        rc = lib.flame_sdpa_chunked_bf16(_p(q), _p(k), _p(v), B, H, Q, K, D, D, ctypes.c_float(0.125), 64, causal, H,
+                                         _p(mask_h), _p(out), None, ctypes.c_uint64(0), _stream())
+        assert rc == 0
+        torch.cuda.synchronize()
+        ro, _, ro32 = oracle.sdpa_fwd(t[0], t[1], t[2], 0.125, causal=bool(causal), mask=keep_h, want_f32=True)
+        assert_close_bf16(oracle, f"O per-head mask causal={causal}", to_f32(out), ro, ro32)
     # causal, no mask
     rc = lib.flame_sdpa_chunked_bf16(_p(q), _p(k), _p(v), B, H, Q, K, D, D, ctypes.c_float(0.125), 64, 1, 1,
                                      None, _p(out), None, ctypes.c_uint64(0), _stream())
@@ -135,6 +149,33 @@ def test_streaming_symbol_causal_and_key_padding(oracle):
                                                ctypes.c_float(0.125), 0, 0, None, _stream()) != 0
 
 
+def test_stream_symbol_takes_a_bf16_mask_where_one_means_excluded(oracle):
+    """sdpa_stream_bf16_launch reads a bf16 mask through the caller's four element strides, and in this one
+    entry point a value above 0.5 EXCLUDES (cuda/sdpa_stream_bf16.cu:79-81); the strides are those the
+    reference's wrapper computes (src/cuda_ops_bf16.rs:1848-1873), 0 broadcasting heads or batches."""
+    from flame_amd import capi
+    lib = capi.lib()
+    lib.sdpa_stream_bf16_launch.restype = ctypes.c_bool
+    reason = ctypes.create_string_buffer(256)
+    for D, (B, H, Q, K) in ((64, (2, 3, 96, 200)), (128, (1, 2, 130, 257))):
+        t = [W.f32_to_bf16_bits(W.normal_f32(778 + D, s, B * H * n * D).reshape(B, H, n, D)) for s, n in enumerate((Q, K, K))]
+        q, k, v = (to_dev(x) for x in t)
+        o = torch.empty_like(q)
+        for mh, mb in ((H, B), (1, B), (1, 1)):
+            excl = (W.normal_f32(779, mh + 10 * mb, mb * mh * Q * K).reshape(mb, mh, Q, K) > 0.4).astype(np.uint8)
+            excl[..., 0] = 0                       # the first key is never excluded
+            excl[0, 0, 3, :] = 1                   # ... except for one row that loses every key
+            m = torch.from_numpy(excl.astype(np.float32)).to(torch.bfloat16).cuda()
+            strides = [1, K, 0 if mh == 1 else Q * K, 0 if mb == 1 else mh * Q * K]      # ek, eq, eh, eb
+            ok = lib.sdpa_stream_bf16_launch(_p(q), _p(k), _p(v), _p(o), B, H, Q, K, D, ctypes.c_float(0.11), _p(m),
+                                             *[ctypes.c_int64(x) for x in strides], 12, 96, 96, _stream(), reason, 256)
+            assert ok and reason.value == b"", reason.value
+            torch.cuda.synchronize()
+            ro, _, ro32 = oracle.sdpa_fwd(t[0], t[1], t[2], 0.11, mask=(1 - excl).astype(np.uint8), want_f32=True)
+            assert_close_bf16(oracle, f"O D={D} mask heads={mh} batches={mb}", to_f32(o), ro, ro32)
+            assert torch.all(o[0, 0, 3] == 0)
+
+
 def test_stream_symbol_reports_reason_when_unsupported(oracle):
     from flame_amd import capi
     lib = capi.lib()
@@ -150,9 +191,6 @@ def test_stream_symbol_reports_reason_when_unsupported(oracle):
     torch.cuda.synchronize()
     ro, _, ro32 = oracle.sdpa_fwd(t[0], t[1], t[2], 0.125, want_f32=True)
     assert_close_bf16(oracle, "O", to_f32(o), ro, ro32)
-    ok = lib.sdpa_stream_bf16_launch(_p(q), _p(k), _p(v), _p(o), B, H, Q, K, D, ctypes.c_float(0.125), _p(q),
-                                     *_z(4), 12, 96, 96, _stream(), reason, 256)
-    assert not ok and b"mask" in reason.value
     ok = lib.sdpa_stream_bf16_launch(_p(q), _p(k), _p(v), _p(o), B, H, Q, K, D, ctypes.c_float(0.125), None,
                                      *_z(4), 12, 128, 96, _stream(), reason, 256)
     assert not ok and b"q_tile" in reason.value
