@@ -51,6 +51,7 @@ struct BwdParams {
     float* lse2;          // workspace, [B*H, Sq]: LSE * log2(e), +inf where LSE = -inf
     Strides qs, ks, vs, os, dos, dqs, dks, dvs;
     int B, H, Sq, Sk;
+    int d;                // real head dim: a multiple of 8, at most the compiled D
     float scale;
     MaskArgs m;
     unsigned long long* phase_cycles;   // profiling aid: per-phase cycle sums of wave 0 of every workgroup, or null
@@ -189,12 +190,24 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
             const int ji = wave * NDMA + i;
             const int row = ji * RPD + dma_row_in;
             const int key = max(min(k0 + row, klimit - 1), 0);   // rows past the attended range re-read a valid row
-            const int c = dma_gran ^ swz<D>(row);
+            const int c = src_granule(dma_gran ^ swz<D>(row), p.d);
             dma16(kbase + (int64_t)key * p.ks.n + c * 8, lds0 + 2u * (T::STAGE_ELEMS + ji * 512));
             dma16(vbase + (int64_t)key * p.vs.n + c * 8, lds0 + 2u * (ji * 512));
         }
         wait_vm0();
         __syncthreads();
+        if (p.d < D) {      // padded head dim: S and dP must not see the copies' filler, so it is zeroed in LDS
+            const u32x4 z = {0u, 0u, 0u, 0u};
+            for (int idx = tid; idx < BN * GPR; idx += 256) {
+                const int row = idx / GPR, gl = idx % GPR;
+                if (gl * 8 >= p.d) {
+                    const int off = row * RS + ((gl ^ swz<D>(row)) << 3);
+                    *reinterpret_cast<u32x4*>(stage0 + off) = z;
+                    *reinterpret_cast<u32x4*>(stage0 + T::STAGE_ELEMS + off) = z;
+                }
+            }
+            __syncthreads();
+        }
 #pragma unroll
         for (int dc = 0; dc < DC; ++dc) {
             kf[dc] = *reinterpret_cast<const bf16x8*>(stage0 + T::STAGE_ELEMS + roff[dc] + 32 * wave * RS);
@@ -209,7 +222,7 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
 #pragma unroll
     for (int i = 0; i < NDQ; ++i) {
         const int row = (wave * NDQ + i) * RPD + dma_row_in;
-        const int c = dma_gran ^ swz<D>(row);
+        const int c = src_granule(dma_gran ^ swz<D>(row), p.d);
         q_lane_off[i] = 2u * (uint32_t)(row * (int)p.qs.n + c * 8);
         do_lane_off[i] = 2u * (uint32_t)(row * (int)p.dos.n + c * 8);
     }
@@ -249,7 +262,7 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
                 const int ji = wave * NDQ + i;
                 const int row = ji * RPD + dma_row_in;
                 const int qi = min(q0 + row, p.Sq - 1);
-                const int c = dma_gran ^ swz<D>(row);
+                const int c = src_granule(dma_gran ^ swz<D>(row), p.d);
                 dma16(qbase + (int64_t)qi * p.qs.n + c * 8, q_dst(stg, 0, i));
                 dma16(dobase + (int64_t)qi * p.dos.n + c * 8, q_dst(stg, 1, i));
             }
@@ -660,8 +673,8 @@ __device__ __forceinline__ void dkdv_store(const BwdParams& p, const f32x16 (&dk
                 const f32x16& c = dvacc[db];
                 u32x2 wk = {pack_bf16(a[4 * g] * s, a[4 * g + 1] * s), pack_bf16(a[4 * g + 2] * s, a[4 * g + 3] * s)};
                 u32x2 wv = {pack_bf16(c[4 * g], c[4 * g + 1]), pack_bf16(c[4 * g + 2], c[4 * g + 3])};
-                *reinterpret_cast<u32x2*>(dkrow + 32 * db + 8 * g + 4 * h) = wk;
-                *reinterpret_cast<u32x2*>(dvrow + 32 * db + 8 * g + 4 * h) = wv;
+                if (32 * db + 8 * g + 4 * h < p.d) *reinterpret_cast<u32x2*>(dkrow + 32 * db + 8 * g + 4 * h) = wk;
+                if (32 * db + 8 * g + 4 * h < p.d) *reinterpret_cast<u32x2*>(dvrow + 32 * db + 8 * g + 4 * h) = wv;
             }
     }
 }
@@ -703,8 +716,8 @@ __global__ __launch_bounds__(256) void bwd_dkdv_merge_kernel(const BwdParams p) 
         for (int g = 0; g < 4; ++g) {
             u32x2 wk = {pack_bf16(ak[g][0] * s, ak[g][1] * s), pack_bf16(ak[g][2] * s, ak[g][3] * s)};
             u32x2 wv = {pack_bf16(av[g][0], av[g][1]), pack_bf16(av[g][2], av[g][3])};
-            *reinterpret_cast<u32x2*>(dkrow + 32 * db + 8 * g + 4 * h) = wk;
-            *reinterpret_cast<u32x2*>(dvrow + 32 * db + 8 * g + 4 * h) = wv;
+            if (32 * db + 8 * g + 4 * h < p.d) *reinterpret_cast<u32x2*>(dkrow + 32 * db + 8 * g + 4 * h) = wk;
+            if (32 * db + 8 * g + 4 * h < p.d) *reinterpret_cast<u32x2*>(dvrow + 32 * db + 8 * g + 4 * h) = wv;
         }
     }
 }
@@ -771,8 +784,9 @@ __global__ __launch_bounds__(64 * NW, (NW == 4 && (!HASMASK || VECMASK)) ? 2 : 1
         const uint16_t* rd = dobase + (int64_t)qrow * p.dos.n + 8 * h;
 #pragma unroll
         for (int dc = 0; dc < DC; ++dc) {
-            qf[dc] = __builtin_bit_cast(bf16x8, ldg16(rq + 16 * dc, qok));
-            dof[dc] = __builtin_bit_cast(bf16x8, ldg16(rd + 16 * dc, qok));
+            const bool in_d = qok && 16 * dc + 8 * h < p.d;
+            qf[dc] = __builtin_bit_cast(bf16x8, ldg16(rq + 16 * dc, in_d));
+            dof[dc] = __builtin_bit_cast(bf16x8, ldg16(rd + 16 * dc, in_d));
         }
     }
     // Per-query scalars, formed here and also left in the workspace for the dK/dV kernel that runs next:
@@ -784,7 +798,7 @@ __global__ __launch_bounds__(64 * NW, (NW == 4 && (!HASMASK || VECMASK)) ? 2 : 1
         float part = 0.f;
 #pragma unroll
         for (int dc = 0; dc < DC; ++dc) {
-            const u32x4 ov = ldg16(ro + 16 * dc, qok);
+            const u32x4 ov = ldg16(ro + 16 * dc, qok && 16 * dc + 8 * h < p.d);
             const u32x4 dv = __builtin_bit_cast(u32x4, dof[dc]);
 #pragma unroll
             for (int i = 0; i < 4; ++i) part += bf16_lo(dv[i]) * bf16_lo(ov[i]) + bf16_hi(dv[i]) * bf16_hi(ov[i]);
@@ -808,7 +822,7 @@ __global__ __launch_bounds__(64 * NW, (NW == 4 && (!HASMASK || VECMASK)) ? 2 : 1
 #pragma unroll
     for (int i = 0; i < NDMA; ++i) {
         const int row = (wave * NDMA + i) * T::ROWS_PER_DMA + dma_row_in;
-        const int c = dma_gran ^ swz<D>(row);
+        const int c = src_granule(dma_gran ^ swz<D>(row), p.d);
         k_lane_off[i] = 2u * (uint32_t)(row * (int)p.ks.n + c * 8);
         v_lane_off[i] = 2u * (uint32_t)(row * (int)p.vs.n + c * 8);
     }
@@ -820,7 +834,7 @@ __global__ __launch_bounds__(64 * NW, (NW == 4 && (!HASMASK || VECMASK)) ? 2 : 1
         for (int i = 0; i < NDMA; ++i) {
             const int row = (wave * NDMA + i) * T::ROWS_PER_DMA + dma_row_in;
             const int key = min(t * BN + row, klimit - 1);   // tail rows re-read the last attended key
-            const int c = dma_gran ^ swz<D>(row);
+            const int c = src_granule(dma_gran ^ swz<D>(row), p.d);
             dma16(kbase + (int64_t)key * p.ks.n + c * 8, dst_of(buf, 0, i));
             dma16(vbase + (int64_t)key * p.vs.n + c * 8, dst_of(buf, 1, i));
         }
@@ -1022,7 +1036,7 @@ __global__ __launch_bounds__(64 * NW, (NW == 4 && (!HASMASK || VECMASK)) ? 2 : 1
             for (int g = 0; g < 4; ++g) {
                 const f32x16& a = dqacc[db];
                 u32x2 w = {pack_bf16(a[4 * g] * s, a[4 * g + 1] * s), pack_bf16(a[4 * g + 2] * s, a[4 * g + 3] * s)};
-                *reinterpret_cast<u32x2*>(dqrow + 32 * db + 8 * g + 4 * h) = w;
+                if (32 * db + 8 * g + 4 * h < p.d) *reinterpret_cast<u32x2*>(dqrow + 32 * db + 8 * g + 4 * h) = w;
             }
     }
 }
@@ -1101,10 +1115,11 @@ __global__ __launch_bounds__(256) void bwd_dq_wide_kernel(const BwdParams p) {
         float part = 0.f;
         static_for<DC>([&](auto dc_tag) {
             constexpr int dc = decltype(dc_tag)::value;
-            qf[qb][dc] = pin_b_fragment<qb * DC + dc>(ldg16(rq + 16 * dc, qok));
-            const u32x4 dv = ldg16(rd + 16 * dc, qok);
+            const bool in_d = qok && 16 * dc + 8 * h < p.d;
+            qf[qb][dc] = pin_b_fragment<qb * DC + dc>(ldg16(rq + 16 * dc, in_d));
+            const u32x4 dv = ldg16(rd + 16 * dc, in_d);
             dof[qb][dc] = pin_b_fragment<16 + qb * DC + dc>(dv);
-            const u32x4 ov = ldg16(ro + 16 * dc, qok);
+            const u32x4 ov = ldg16(ro + 16 * dc, in_d);
 #pragma unroll
             for (int i = 0; i < 4; ++i) part += bf16_lo(dv[i]) * bf16_lo(ov[i]) + bf16_hi(dv[i]) * bf16_hi(ov[i]);
         });
@@ -1131,7 +1146,7 @@ __global__ __launch_bounds__(256) void bwd_dq_wide_kernel(const BwdParams p) {
 #pragma unroll
     for (int i = 0; i < NDMA; ++i) {
         const int row = (wave * NDMA + i) * T::ROWS_PER_DMA + dma_row_in;
-        const int c = dma_gran ^ swz<D>(row);
+        const int c = src_granule(dma_gran ^ swz<D>(row), p.d);
         k_lane_off[i] = 2u * (uint32_t)(row * (int)p.ks.n + c * 8);
         v_lane_off[i] = 2u * (uint32_t)(row * (int)p.vs.n + c * 8);
     }
@@ -1143,7 +1158,7 @@ __global__ __launch_bounds__(256) void bwd_dq_wide_kernel(const BwdParams p) {
         for (int i = 0; i < NDMA; ++i) {
             const int row = (wave * NDMA + i) * T::ROWS_PER_DMA + dma_row_in;
             const int key = max(min(t * BN + row, klimit - 1), 0);
-            const int c = dma_gran ^ swz<D>(row);
+            const int c = src_granule(dma_gran ^ swz<D>(row), p.d);
             dma16(kbase + (int64_t)key * p.ks.n + c * 8, dst_of(stg, 0, i));
             dma16(vbase + (int64_t)key * p.vs.n + c * 8, dst_of(stg, 1, i));
         }
@@ -1386,7 +1401,7 @@ __global__ __launch_bounds__(256) void bwd_dq_wide_kernel(const BwdParams p) {
                 for (int g = 0; g < 4; ++g) {
                     const f32x16& a = dqacc[qb][db];
                     u32x2 w = {pack_bf16(a[4 * g] * s, a[4 * g + 1] * s), pack_bf16(a[4 * g + 2] * s, a[4 * g + 3] * s)};
-                    *reinterpret_cast<u32x2*>(dqrow + 32 * db + 8 * g + 4 * h) = w;
+                    if (32 * db + 8 * g + 4 * h < p.d) *reinterpret_cast<u32x2*>(dqrow + 32 * db + 8 * g + 4 * h) = w;
                 }
         }
 }

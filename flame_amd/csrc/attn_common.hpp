@@ -293,6 +293,12 @@ struct Strides {
     int64_t b, h, n;   // element strides of a [B,H,N,D] bf16 view; the D stride is 1
 };
 
+// Head dims below the compiled one (any multiple of 8, e.g. 96 on the 128-wide kernels) run zero-padded:
+// fragments loaded straight from global memory are zero past the real head dim, tile copies re-read
+// granule 0 of their row there (finite values that only ever meet those zero operands, or land in
+// output rows past the real head dim, which are not stored), and stores skip those rows.
+__device__ __forceinline__ int src_granule(int c, int d_real) { return c * 8 < d_real ? c : 0; }
+
 // The 64 keep-mask bytes of one query row over a 64-key tile, as loaded by the kernels whose lanes own
 // a query: keep(kb, r) is the byte of key 32*kb + acc_row(r, h).
 struct MaskRow64 {

@@ -33,6 +33,7 @@ struct FwdParams {
     float* lse;          // contiguous [B*H, Sq] or null
     Strides qs, ks, vs, os;
     int B, H, Sq, Sk;
+    int d;               // real head dim: a multiple of 8, at most the compiled D
     float scale;
     MaskArgs m;
 };
@@ -107,7 +108,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void fwd_kernel(const Fwd
         const bool ok = row < p.Sq;
         const uint16_t* rp = qbase + (int64_t)row * p.qs.n + 8 * h;
 #pragma unroll
-        for (int dc = 0; dc < DC; ++dc) qf[dc] = __builtin_bit_cast(bf16x8, ldg16(rp + 16 * dc, ok));
+        for (int dc = 0; dc < DC; ++dc) qf[dc] = __builtin_bit_cast(bf16x8, ldg16(rp + 16 * dc, ok && 16 * dc + 8 * h < p.d));
     }
 
     // ---- asynchronous tile copies.  K(t) and V(t) live in stage t&1.  Full tiles: uniform tile base
@@ -120,7 +121,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void fwd_kernel(const Fwd
 #pragma unroll
     for (int i = 0; i < NDMA; ++i) {
         const int row = (wave * NDMA + i) * T::ROWS_PER_DMA + dma_row_in;
-        const int c = dma_gran ^ swz<D>(row);
+        const int c = src_granule(dma_gran ^ swz<D>(row), p.d);
         k_lane_off[i] = 2u * (uint32_t)(row * (int)p.ks.n + c * 8);
         v_lane_off[i] = 2u * (uint32_t)(row * (int)p.vs.n + c * 8);
     }
@@ -132,7 +133,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void fwd_kernel(const Fwd
         for (int i = 0; i < NDMA; ++i) {
             const int row = (wave * NDMA + i) * T::ROWS_PER_DMA + dma_row_in;
             const int key = min(t * BN + row, klimit - 1);   // tail rows re-read the last attended key
-            const int c = dma_gran ^ swz<D>(row);
+            const int c = src_granule(dma_gran ^ swz<D>(row), p.d);
             dma16(base + (int64_t)key * row_stride + c * 8, dst_of(t, which, i));
         }
     };
@@ -438,7 +439,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void fwd_kernel(const Fwd
                     const f32x16& a = oacc[db];
                     u32x2 w = {pack_bf16(a[4 * g] * inv, a[4 * g + 1] * inv),
                                pack_bf16(a[4 * g + 2] * inv, a[4 * g + 3] * inv)};
-                    *reinterpret_cast<u32x2*>(orow + 32 * db + 8 * g + 4 * h) = w;
+                    if (32 * db + 8 * g + 4 * h < p.d) *reinterpret_cast<u32x2*>(orow + 32 * db + 8 * g + 4 * h) = w;
                 }
             if (p.lse && h == 0) {
                 const float v = l > 0.f ? (m_run * c_log2 + log2_fast(l)) * kLn2 : -INFINITY;
@@ -521,7 +522,7 @@ __global__ __launch_bounds__(256) void fwd_wide_kernel(const FwdParams p) {
         const uint16_t* rp = qbase + (int64_t)qrow[qb] * p.qs.n + 8 * h;
         static_for<DC>([&](auto dc_tag) {
             constexpr int dc = decltype(dc_tag)::value;
-            qf[qb][dc] = pin_b_fragment<qb * DC + dc>(ldg16(rp + 16 * dc, ok));
+            qf[qb][dc] = pin_b_fragment<qb * DC + dc>(ldg16(rp + 16 * dc, ok && 16 * dc + 8 * h < p.d));
         });
     });
 
@@ -532,7 +533,7 @@ __global__ __launch_bounds__(256) void fwd_wide_kernel(const FwdParams p) {
 #pragma unroll
     for (int i = 0; i < NDMA; ++i) {
         const int row = (wave * NDMA + i) * T::ROWS_PER_DMA + dma_row_in;
-        const int c = dma_gran ^ swz<D>(row);
+        const int c = src_granule(dma_gran ^ swz<D>(row), p.d);
         k_lane_off[i] = 2u * (uint32_t)(row * (int)p.ks.n + c * 8);
         v_lane_off[i] = 2u * (uint32_t)(row * (int)p.vs.n + c * 8);
     }
@@ -849,7 +850,7 @@ __global__ __launch_bounds__(256) void fwd_wide_kernel(const FwdParams p) {
                     const f32x16& a = oacc[qb][db];
                     u32x2 w = {pack_bf16(a[4 * g] * inv, a[4 * g + 1] * inv),
                                pack_bf16(a[4 * g + 2] * inv, a[4 * g + 3] * inv)};
-                    *reinterpret_cast<u32x2*>(orow + 32 * db + 8 * g + 4 * h) = w;
+                    if (32 * db + 8 * g + 4 * h < p.d) *reinterpret_cast<u32x2*>(orow + 32 * db + 8 * g + 4 * h) = w;
                 }
             if (p.lse && h == 0) {
                 const float v = l > 0.f ? (m_run[qb] * c_log2 + log2_fast(l)) * kLn2 : -INFINITY;

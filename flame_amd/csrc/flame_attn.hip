@@ -142,6 +142,11 @@ int launch_fwd_wide(const FwdParams& p, hipStream_t s) {
 
 size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
+// Head dims: the kernels are compiled for 64 and 128; any other multiple of 8 up to 128 (96 among them) runs
+// zero-padded on the next compiled size.
+bool head_dim_ok(int D) { return D > 0 && D <= 128 && D % 8 == 0; }
+int padded_head_dim(int D) { return D <= 64 ? 64 : 128; }
+
 // compute units of the current device (cached; 256 when the query fails)
 int device_cu_count() {
     static int cus = 0;
@@ -290,7 +295,7 @@ int flame_attn_profiling_read(FlameAttnKernelTimes* out) {
 
 size_t flame_attn_bwd_workspace_bytes(int B, int H, int N_q, int D) {
     if (B <= 0 || H <= 0 || N_q <= 0 || D <= 0) return 0;
-    return bwd_rows_bytes(B, H, N_q) + (size_t)device_cu_count() * bwd_split_slot_bytes(D);
+    return bwd_rows_bytes(B, H, N_q) + (size_t)device_cu_count() * bwd_split_slot_bytes(padded_head_dim(D));
 }
 
 int flame_attn_bwd_bf16(const void* Q, const void* K, const void* V, const void* O, const void* dO,
@@ -307,7 +312,7 @@ int flame_attn_bwd_bf16(const void* Q, const void* K, const void* V, const void*
     if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0) return FLAME_ATTN_ERR_INVALID;
     if (!(scale > 0.f) || !isfinite(scale)) return FLAME_ATTN_ERR_INVALID;
     if (!LSE || !workspace) return FLAME_ATTN_ERR_INVALID;
-    if (D != 64 && D != 128) return FLAME_ATTN_ERR_UNSUPPORTED;
+    if (!head_dim_ok(D)) return FLAME_ATTN_ERR_UNSUPPORTED;
     if (workspace_bytes < bwd_rows_bytes(B, H, N_q)) return FLAME_ATTN_ERR_INVALID;
     if (!aligned16(workspace)) return FLAME_ATTN_ERR_UNSUPPORTED;
     int rc;
@@ -339,6 +344,7 @@ int flame_attn_bwd_bf16(const void* Q, const void* K, const void* V, const void*
     p.qs = mk(q_strides); p.ks = mk(k_strides); p.vs = mk(v_strides); p.os = mk(o_strides);
     p.dos = mk(do_strides); p.dqs = mk(dq_strides); p.dks = mk(dk_strides); p.dvs = mk(dv_strides);
     p.B = B; p.H = H; p.Sq = N_q; p.Sk = N_kv;
+    p.d = D;
     p.scale = scale;
     p.m.kv_len = kv_len;
     p.m.mask = keep_mask;
@@ -355,7 +361,7 @@ int flame_attn_bwd_bf16(const void* Q, const void* K, const void* V, const void*
     p.phase_cycles = g_phase_cycles;
     if (D == 128 && !keep_mask && g_phase_cycles) return launch_bwd<128, false, true>(p, s);   // phase-timing build
 #endif
-    if (D == 128) return keep_mask ? launch_bwd<128, true>(p, s) : launch_bwd<128, false>(p, s);
+    if (padded_head_dim(D) == 128) return keep_mask ? launch_bwd<128, true>(p, s) : launch_bwd<128, false>(p, s);
     return keep_mask ? launch_bwd<64, true>(p, s) : launch_bwd<64, false>(p, s);
 }
 
@@ -481,7 +487,7 @@ static int attn_fwd_impl(const void* Q, const void* K, const void* V, void* O, v
                         void* stream, int mask_mode = kMaskU8) {
     if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0) return FLAME_ATTN_ERR_INVALID;
     if (!(scale > 0.f) || !isfinite(scale)) return FLAME_ATTN_ERR_INVALID;
-    if (D != 64 && D != 128) return FLAME_ATTN_ERR_UNSUPPORTED;
+    if (!head_dim_ok(D)) return FLAME_ATTN_ERR_UNSUPPORTED;
     int rc;
     if ((rc = check_view(Q, q_strides, q_off))) return rc;
     if ((rc = check_view(K, k_strides, k_off))) return rc;
@@ -499,6 +505,7 @@ static int attn_fwd_impl(const void* Q, const void* K, const void* V, void* O, v
     p.lse = LSE ? static_cast<float*>(LSE) + lse_off : nullptr;
     p.qs = mk(q_strides); p.ks = mk(k_strides); p.vs = mk(v_strides); p.os = mk(o_strides);
     p.B = B; p.H = H; p.Sq = N_q; p.Sk = N_kv;
+    p.d = D;
     p.scale = scale;
     p.m.kv_len = kv_len;
     p.m.mask = keep_mask;
@@ -527,9 +534,10 @@ static int attn_fwd_impl(const void* Q, const void* K, const void* V, void* O, v
     // ... as 4 wavefronts of 64 queries when nothing is excluded at all, else as 8 wavefronts of 32
     const bool plain = !causal && kv_len == nullptr && N_kv % 64 == 0;
     // a keep-mask with vector-loadable rows over whole tiles and no bias: the lean masked kernel
+    const int DP = padded_head_dim(D);
     if (keep_mask != nullptr && bias == nullptr && p.m.rows16 && N_kv % 64 == 0)
-        return D == 128 ? launch_fwd<128, true, 4, true>(p, s) : launch_fwd<64, true, 4, true>(p, s);
-    if (D == 128)
+        return DP == 128 ? launch_fwd<128, true, 4, true>(p, s) : launch_fwd<64, true, 4, true>(p, s);
+    if (DP == 128)
         return hm ? launch_fwd<128, true, 4>(p, s)
                   : wide ? (plain ? launch_fwd_wide<128>(p, s) : launch_fwd<128, false, 8>(p, s)) : launch_fwd<128, false, 4>(p, s);
     return hm ? launch_fwd<64, true, 4>(p, s)
@@ -821,7 +829,7 @@ bool sdpa_stream_bf16_launch(const void* dQ, const void* dK, const void* dV, voi
     };
     (void)head_tile;
     if (q_tile > max_q_tile) return fail("q_tile exceeds max_q_tile");
-    if (d != 64 && d != 128) return fail("head dim must be 64 or 128");
+    if (!head_dim_ok(d)) return fail("head dim must be a multiple of 8, at most 128");
     const int64_t qs[4] = {(int64_t)H * Q_len * d, (int64_t)Q_len * d, d, 1};
     const int64_t ks[4] = {(int64_t)H * K_len * d, (int64_t)K_len * d, d, 1};
     // bf16 mask addressed by the caller's four element strides; in this entry point a value above 0.5 EXCLUDES

@@ -13,7 +13,11 @@
  *     be 1, the other strides and the offsets multiples of 8 (16-byte rows), N strides below 2^24.
  *     This admits the DiT view reshape([B,N,H,D]).permute(0,2,1,3) without a copy
  *     (reference: src/sdpa.rs:607-621, :646-651).
- *   - D is 64 or 128; anything else returns FLAME_ATTN_ERR_UNSUPPORTED.
+ *   - D (head dim) is any multiple of 8 up to 128.  The kernels are compiled for 64 and 128 (the
+ *     reference's production sizes, with 96: src/sdpa.rs:149, src/cuda/flash_attention_fwd.cu:307-324);
+ *     other sizes, 96 included, run zero-padded to the next compiled size inside the tile loads and
+ *     stores, at that size's cost.  Anything else returns FLAME_ATTN_ERR_UNSUPPORTED.  The Sage and
+ *     input-preparation entry points take 64 or 128 only.
  *   - LSE / Stats: fp32, contiguous [B*H, N_q] (== [B,H,N_q,1] with strides [H*N_q, N_q, 1, 1]),
  *     value = max_j s_ij + ln(sum_j exp(s_ij - max)), s = scale * Q K^T, natural log
  *     (reference: src/cuda/cudnn_sdpa.cpp:271-279, src/sdpa.rs:715-722).  A row with no attended

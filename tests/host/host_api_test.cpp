@@ -171,7 +171,8 @@ int main() {
         Tensor dd = Tensor::empty({1, 2, 8, 128}, DType::BF16).value();
         Tensor ln = Tensor::empty({1, 2, 16, 64}, DType::BF16).value();
         Tensor f32 = Tensor::empty({1, 2, 8, 64}, DType::F32).value();
-        Tensor d96 = Tensor::empty({1, 2, 8, 96}, DType::BF16).value();
+        Tensor d100 = Tensor::empty({1, 2, 8, 104}, DType::BF16).value();
+        Tensor d256 = Tensor::empty({1, 2, 8, 256}, DType::BF16).value();
         Tensor badm = Tensor::empty({1, 2, 8, 9}, DType::U8).value();
         auto kind = [](const Result<Tensor>& r) { return r.ok() ? -1 : (int)r.error().kind; };
         CHECK(kind(sdpa::forward(r3, r3, r3)) == Error::InvalidInput, "rank 3");
@@ -180,12 +181,13 @@ int main() {
         CHECK(kind(sdpa::forward(a, a, ln)) == Error::InvalidInput, "k_len != v_len");
         CHECK(kind(sdpa::forward(a, a, a, &badm)) == Error::InvalidInput, "mask not broadcastable");
         CHECK(kind(sdpa::forward(f32, f32, f32)) == Error::InvalidInput, "non-bf16");
-        CHECK(kind(sdpa::forward(d96, d96, d96)) == Error::Unsupported, "head dim 96");
+        CHECK(sdpa::forward(d100, d100, d100).ok(), "head dim 104 runs (padded to 128)");
+        CHECK(kind(sdpa::forward(d256, d256, d256)) == Error::Unsupported, "head dim 256");
     }
 
     // ---- 3. forward == forward_train, taped backward vs the naive recompute; shapes of
     //         tests/cudnn_sdpa_bwd_parity.rs:311-320
-    for (int D : {64, 128}) {
+    for (int D : {64, 96, 128}) {
         const int B = 1, H = 4, N = D == 64 ? 128 : 256;
         std::printf("[train fwd/bwd  B=%d H=%d N=%d D=%d]\n", B, H, N, D);
         auto hq = randn_bf16((size_t)B * H * N * D), hk = randn_bf16(hq.size()), hv = randn_bf16(hq.size()), hdo = randn_bf16(hq.size());
