@@ -1,15 +1,26 @@
 #!/usr/bin/env python3
 """Benchmark of the attention hot path on one MI355X.
 
-One "step" = one forward (O + log-sum-exp) followed by one tile-recompute backward (dQ, dK, dV) of
-the DiT joint-attention configuration B=1 H=24 S=4608 (512 text + 4096 image tokens) D=128 bf16,
-inputs resident in HBM.  Prints ONE JSON line; see --help for the knobs.
+One "step" = one forward (O + log-sum-exp) followed by one tile-recompute backward (dQ, dK, dV), inputs
+resident in HBM.  The default workload is the DiT joint-attention configuration B=1 H=24 S=4608 (512 text
++ 4096 image tokens) D=128 bf16; `--config 1..5` selects the other configurations (5 is the inference-only
+int8-QK forward, whose step is quantisation + forward).  Prints ONE JSON line.
+
+Three timed loops after the warm-up, all with the same inputs:
+  1. `--steps` steps bracketed by a device synchronisation on both sides, nothing else running on the
+     host side: `ms_per_step` and `value` come from this one;
+  2. the same steps with a HIP event before the forward, between forward and backward, and after the
+     backward (events on the stream the kernels are launched on): medians in `timing`;
+  3. at most 50 steps with the library's own event pair around every kernel launch: `kernels_ms`, and from
+     them the roofline of the dominant kernel.
 """
 from __future__ import annotations
 
 import argparse
 import json
 import os
+import re
+import statistics
 import sys
 import time
 
@@ -17,34 +28,76 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0      # MI355X dense bf16 MFMA, published
-# HBM bytes per launch of the dominant kernel (bwd_dkdv_kernel) at the headline configuration, from two
-# rocprofv3 --pmc passes (FETCH_SIZE, WRITE_SIZE; KiB per dispatch), each scaled by what the same
-# counter reads for a plain 256 MiB device copy (FETCH_SIZE under-reads by 2.0, WRITE_SIZE is exact):
-# 95 271 KiB x 2.0 fetched + 76 025 KiB written (25 MB of that each way are the fp32 partial sums of the
-# split key blocks).  Counters cannot be read from inside this script.
-DKDV_TRAFFIC_BYTES_CFG2 = int((95271 * 2.0 + 76025 * 1.0) * 1024)
+PEAK_INT8_TOPS = 5000.0        # MI355X dense int8 MFMA, published
 METRIC = "fwd+bwd attn TFLOP/s & % MFMA peak, S=4608 D=128 bf16; saved-activation bytes"
 
 
-def cpu_baseline(w, max_seconds_hint=30.0):
-    """Naive materialised fp32 SDPA forward+backward (the parity checker) timed on the host cores."""
+def profile_path(workload_name: str) -> str:
+    return os.path.join(ROOT, "profiles", f"attention_kernels_{workload_name}.md")
+
+
+def recorded_traffic(workload_name: str, kernel: str):
+    """HBM bytes per launch of `kernel` as recorded in this workload's rocprofv3 summary under profiles/
+    (FETCH_SIZE and WRITE_SIZE passes, already scaled by the copy-kernel calibration that the summary
+    states next to the commands).  Counters cannot be read from inside this script; None when the
+    summary or the row is missing."""
+    try:
+        text = open(profile_path(workload_name)).read()
+    except OSError:
+        return None
+    sec = text.split("## HBM traffic", 1)
+    if len(sec) < 2:
+        return None
+    for line in sec[1].splitlines():
+        m = re.match(r"\|\s*`fattn::%s[<`][^|]*\|\s*[\d.]+\s*\|\s*([\d.]+)\s*\|\s*[\d.]+\s*\|\s*([\d.]+)\s*\|" % re.escape(kernel), line)
+        if m:
+            return int((float(m.group(1)) + float(m.group(2))) * 1e6)
+    return None
+
+
+def cpu_baseline(w):
+    """Naive materialised fp32 SDPA forward+backward (the parity checker) timed on the host cores, on a
+    bounded sample of the same workload: whole passes while they are short, else one band of query
+    rows of every head (a band costs rows x Sk)."""
     from oracle import oracle as O
     O.lib()
     B, H, Sq, Sk, D = w.shape
     cores = O.num_threads()
     heads = B * H
+    rows = (0, Sq)
+    sample_pairs = w.valid_pairs()
+    what = f"all {heads} (batch,head) slices"
+    if w.flops() > 4e12:                                     # long causal: the last 1024 query rows of every head
+        rows = (Sq - 1024, Sq)
+        sample_pairs = heads * sum(min(i + 1, Sk) if w.causal else Sk for i in range(*rows))
+        what = f"query rows {rows[0]}..{rows[1]} of all {heads} (batch,head) slices"
     passes, dt = 0, 0.0
     t0 = time.perf_counter()
-    while dt < 10.0 and passes < 8:              # whole workload, repeated to about 10 s of CPU work
-        o, _ = O.sdpa_fwd(w.q, w.k, w.v, w.scale, causal=w.causal, kv_len=w.kv_len, heads=(0, heads))
-        O.sdpa_bwd(w.q, w.k, w.v, o, w.do, w.scale, causal=w.causal, kv_len=w.kv_len, heads=(0, heads))
+    while dt < 10.0 and passes < 8:              # repeated to about 10 s of CPU work
+        o, _ = O.sdpa_fwd(w.q, w.k, w.v, w.scale, causal=w.causal, kv_len=w.kv_len, heads=(0, heads), rows=rows)
+        O.sdpa_bwd(w.q, w.k, w.v, o, w.do, w.scale, causal=w.causal, kv_len=w.kv_len, heads=(0, heads), rows=rows)
         passes += 1
         dt = time.perf_counter() - t0
-    flops = w.flops() * passes
+    flops = 14.0 * sample_pairs * D * passes
     return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
-            "sample": f"{passes} passes over all {heads} (batch,head) slices of the same workload, "
-                      f"naive fp32 fwd+bwd, {dt:.1f} s wall",
+            "sample": f"{passes} passes over {what} of the same workload, naive fp32 fwd+bwd, {dt:.1f} s wall",
             "seconds": dt}
+
+
+def cpu_baseline_sage(w):
+    """The oracle's quantiser + int8-QK forward on a bounded sample: all heads, the first 512 query rows."""
+    from oracle import oracle as O
+    O.lib()
+    B, H, Sq, Sk, D = w.shape
+    rows = (0, min(512, Sq))
+    t0 = time.perf_counter()
+    z = O.sage_quant(w.q, w.k)
+    O.sage_fwd(z["qi8"], z["ki8"], z["sq"], z["sk"], w.v, w.scale, rows=rows)
+    dt = time.perf_counter() - t0
+    ops = 4.0 * B * H * (rows[1] - rows[0]) * Sk * D
+    return {"value": ops / dt / 1e12, "unit": "TOP/s", "cores": O.num_threads(), "kind": "port",
+            "sample": f"quantisation of the whole workload + int8-QK forward of query rows {rows[0]}..{rows[1]} "
+                      f"of all {B * H} (batch,head) slices, {dt:.1f} s wall", "seconds": dt}
 
 
 def input_prep_rate(capi, W, torch, B, H, N, D, dev, iters=20):
@@ -71,42 +124,94 @@ def input_prep_rate(capi, W, torch, B, H, N, D, dev, iters=20):
             "GB_per_s": nbytes / (ms * 1e-3) / 1e9, "frac_of_hbm_peak": nbytes / (ms * 1e-3) / 8e12}
 
 
+def timed_loops(torch, capi, first, second, steps, warmup):
+    """The three loops of the module docstring.  `first` / `second`: the two halves of a step (forward and
+    backward; quantisation and forward).  Returns (wall ms per step, event medians, per-kernel averages)."""
+    for _ in range(warmup):
+        first()
+        second()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        first()
+        second()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+    for e in ev:
+        e[0].record()
+        first()
+        e[1].record()
+        second()
+        e[2].record()
+    torch.cuda.synchronize()
+    a = [e[0].elapsed_time(e[1]) for e in ev]
+    b = [e[1].elapsed_time(e[2]) for e in ev]
+    j = [e[0].elapsed_time(e[2]) for e in ev]
+    medians = {"first_ms_median": statistics.median(a), "second_ms_median": statistics.median(b),
+               "step_ms_median": statistics.median(j), "step_ms_min": min(j), "step_ms_max": max(j), "samples": steps}
+
+    capi.profiling_enable(True)          # an event pair around every kernel, on the launch stream
+    for _ in range(min(steps, 50)):
+        first()
+        second()
+    torch.cuda.synchronize()
+    times = capi.profiling_read()
+    capi.profiling_enable(False)
+    per_kernel = {kname: tot / n for kname, (tot, n) in times.items() if n}
+    return wall_ms, medians, per_kernel
+
+
 def sage_line(args, capi, torch, w, dev):
     """Inference-only configuration: one step = quantise Q and K to int8 + the int8-QK forward."""
     import numpy as np
     B, H, Sq, Sk, D = w.shape
     q, k, v = (torch.from_numpy(np.ascontiguousarray(t).view(np.int16)).view(torch.bfloat16).to(dev) for t in (w.q, w.k, w.v))
+    o = torch.empty_like(q)
+    state = {}
 
-    def step():
-        return capi.sage_fwd(capi.sage_quant(q, k), v, w.scale)
+    def quant():
+        state["qz"] = capi.sage_quant(q, k)
 
-    for _ in range(args.warmup):
-        step()
+    def fwd():
+        capi.sage_fwd(state["qz"], v, w.scale, out=o)
+
+    torch.cuda.reset_peak_memory_stats()
+    ms, med, per_kernel = timed_loops(torch, capi, quant, fwd, args.steps, args.warmup)
+    # the bf16 forward on the same inputs, for the comparison the int8 path has to win
+    for _ in range(5):
+        capi.attn_fwd(q, k, v, w.scale, want_lse=False, out=o)
+    e = [torch.cuda.Event(enable_timing=True) for _ in range(21)]
+    for i in range(20):
+        e[i].record()
+        capi.attn_fwd(q, k, v, w.scale, want_lse=False, out=o)
+    e[20].record()
     torch.cuda.synchronize()
-    capi.profiling_enable(True)
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
-    times = capi.profiling_read()
-    capi.profiling_enable(False)
-    ms = dt * 1e3 / args.steps
-    per_kernel = {kname: tot / n for kname, (tot, n) in times.items() if n}
+    bf16_fwd_ms = statistics.median(e[i].elapsed_time(e[i + 1]) for i in range(20))
     ops = 4.0 * w.valid_pairs() * D            # 2*pairs*D int8 (QK^T) + 2*pairs*D bf16 (PV)
     t_fwd = per_kernel["sage_fwd"] * 1e-3
     # time-weighted blend of the two peaks: the int8 half is priced at 5.0 POP/s, the bf16 half at 2.5 PFLOP/s
-    ideal = 0.5 * ops / 5.0e15 + 0.5 * ops / 2.5e15
-    print(json.dumps({
+    ideal = 0.5 * ops / (PEAK_INT8_TOPS * 1e12) + 0.5 * ops / (PEAK_BF16_TFLOPS * 1e12)
+    out = {
         "metric": "int8-QK attention forward incl. quantisation, T(FL)OP/s", "value": ops / (ms * 1e-3) / 1e12,
         "unit": "TOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8+bf16", "data": "synthetic",
         "config": {"workload": w.name, "B": B, "H": H, "Sq": Sq, "Sk": Sk, "D": D, "causal": bool(w.causal),
                    "step": "quantise Q,K (per-block int8, mean-smoothed K) + int8-QK forward"},
+        "timing": {"quantise_ms_median": med["first_ms_median"], "forward_ms_median": med["second_ms_median"],
+                   "step_ms_median": med["step_ms_median"], "samples": med["samples"], "clock": "HIP events on the launch stream",
+                   "bf16_forward_same_inputs_ms_median": bf16_fwd_ms},
         "roofline": {"bound": "mfma", "kernel": "sage_fwd_kernel", "achieved": ops / t_fwd / 1e12,
-                     "peak": ops / ideal / 1e12, "unit": "TOP/s", "frac": ideal / t_fwd, "traffic": None,
-                     "avg_launch_ms": per_kernel["sage_fwd"], "note": "peak = time-weighted blend of 5.0 POP/s int8 and 2.5 PFLOP/s bf16"},
-        "kernels_ms": per_kernel}))
+                     "peak": ops / ideal / 1e12, "unit": "TOP/s", "frac": ideal / t_fwd,
+                     "traffic": recorded_traffic(w.name, "sage_fwd_kernel"),
+                     "avg_launch_ms": per_kernel["sage_fwd"], "ops_per_launch": ops,
+                     "note": "peak = time-weighted blend of 5.0 POP/s int8 and 2.5 PFLOP/s bf16"},
+        "kernels_ms": per_kernel,
+        "peak_device_MiB": torch.cuda.max_memory_allocated() / 2 ** 20}
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline_sage(w)
+    print(json.dumps(out))
 
 
 def main():
@@ -138,44 +243,37 @@ def main():
     w = W.CONFIGS[args.config]()
     B, H, Sq, Sk, D = w.shape
     dev = torch.device("cuda:0")
-    if w.do is None:            # inference-only workload (int8-QK forward): a parity-test case, timed on request
+    if args.traffic_calibration:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+        torch.empty_like(src).copy_(src)          # one elementwise copy kernel: reads 256 MiB, writes 256 MiB
+        del src
+    if w.do is None:            # inference-only workload (int8-QK forward)
         return sage_line(args, capi, torch, w, dev)
 
     def dev_t(bits):
         import numpy as np
         return torch.from_numpy(np.ascontiguousarray(bits).view(np.int16)).view(torch.bfloat16).to(dev)
 
+    torch.cuda.reset_peak_memory_stats()
     q, k, v, do = (dev_t(t) for t in (w.q, w.k, w.v, w.do))
     kvl = None if w.kv_len is None else torch.from_numpy(w.kv_len).to(dev)
     o = torch.empty_like(q)
     grads = (torch.empty_like(q), torch.empty_like(k), torch.empty_like(v))
     ws = torch.empty(capi.bwd_workspace_bytes(B, H, Sq, D), dtype=torch.uint8, device=dev)
-
     mask = torch.ones(1, 1, Sq, Sk, dtype=torch.uint8, device=dev) if args.keep_mask else None
+    state = {}
 
-    def step():
-        _, lse = capi.attn_fwd(q, k, v, w.scale, causal=w.causal, kv_len=kvl, mask=mask, out=o)
-        capi.attn_bwd(q, k, v, o, do, lse, w.scale, causal=w.causal, kv_len=kvl, mask=mask, workspace=ws, grads=grads)
+    def fwd():
+        _, state["lse"] = capi.attn_fwd(q, k, v, w.scale, causal=w.causal, kv_len=kvl, mask=mask, out=o)
 
-    if args.traffic_calibration:
-        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
-        torch.empty_like(src).copy_(src)          # one elementwise copy kernel: reads 256 MiB, writes 256 MiB
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    capi.profiling_enable(True)          # HIP events around every kernel, on the launch stream
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
-    times = capi.profiling_read()
-    capi.profiling_enable(False)
+    def bwd():
+        capi.attn_bwd(q, k, v, o, do, state["lse"], w.scale, causal=w.causal, kv_len=kvl, mask=mask, workspace=ws, grads=grads)
 
-    ms = dt * 1e3 / args.steps
+    ms, med, per_kernel = timed_loops(torch, capi, fwd, bwd, args.steps, args.warmup)
+    peak_mib = torch.cuda.max_memory_allocated() / 2 ** 20
+
     flops_fwd, flops_bwd = w.flops(True, False), w.flops(False, True)
     tflops = (flops_fwd + flops_bwd) / (ms * 1e-3) / 1e12
-    per_kernel = {kname: tot / n for kname, (tot, n) in times.items() if n}
     # Dominant kernel: bwd_dkdv_kernel.  Per launch it carries four of the five backward GEMMs over
     # every attended (query, key) pair: S recompute, dP, dV, dK = 8 * pairs * D flops.  The fifth
     # (dQ) runs in bwd_dq_kernel, which recomputes S and dP (6 * pairs * D executed, 2 * pairs * D
@@ -198,12 +296,19 @@ def main():
         "config": {"workload": w.name, "B": B, "H": H, "Sq": Sq, "Sk": Sk, "D": D, "causal": bool(w.causal),
                    "step": "forward (O+LSE) + recompute backward (dQ,dK,dV)", "keep_mask": bool(args.keep_mask)},
         "frac_of_bf16_mfma_peak": tflops / PEAK_BF16_TFLOPS,
+        "timing": {"forward_ms_median": med["first_ms_median"], "backward_ms_median": med["second_ms_median"],
+                   "step_ms_median": med["step_ms_median"], "step_ms_min": med["step_ms_min"], "step_ms_max": med["step_ms_max"],
+                   "samples": med["samples"], "clock": "HIP events on the launch stream",
+                   "forward_tflops": flops_fwd / (med["first_ms_median"] * 1e-3) / 1e12,
+                   "backward_tflops": flops_bwd / (med["second_ms_median"] * 1e-3) / 1e12,
+                   "step_tflops": (flops_fwd + flops_bwd) / (med["step_ms_median"] * 1e-3) / 1e12},
         "roofline": {"bound": "mfma", "kernel": "bwd_dkdv_kernel", "achieved": achieved, "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS,
-                     "traffic": DKDV_TRAFFIC_BYTES_CFG2 if args.config == 2 and not args.keep_mask else None,
+                     "traffic": None if args.keep_mask else recorded_traffic(w.name, "bwd_dkdv_kernel"),
                      "avg_launch_ms": per_kernel[dom], "flops_per_launch": 8 * pairs_d},
         "kernels": kernels,
         "kernels_ms": per_kernel,
+        "peak_device_MiB": peak_mib,
         "saved_activations": w.saved_activation_bytes(),
     }
     if args.config == 2:

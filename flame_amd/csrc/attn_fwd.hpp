@@ -33,7 +33,8 @@ struct FwdParams {
     float* lse;          // contiguous [B*H, Sq] or null
     Strides qs, ks, vs, os;
     int B, H, Sq, Sk;
-    int d;               // real head dim: a multiple of 8, at most the compiled D
+    int d;               // real head dim of Q and K: a multiple of 8, at most the compiled D
+    int dv;              // real head dim of V and O, likewise
     float scale;
     MaskArgs m;
 };
@@ -121,9 +122,9 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void fwd_kernel(const Fwd
 #pragma unroll
     for (int i = 0; i < NDMA; ++i) {
         const int row = (wave * NDMA + i) * T::ROWS_PER_DMA + dma_row_in;
-        const int c = src_granule(dma_gran ^ swz<D>(row), p.d);
-        k_lane_off[i] = 2u * (uint32_t)(row * (int)p.ks.n + c * 8);
-        v_lane_off[i] = 2u * (uint32_t)(row * (int)p.vs.n + c * 8);
+        const int c = dma_gran ^ swz<D>(row);
+        k_lane_off[i] = 2u * (uint32_t)(row * (int)p.ks.n + src_granule(c, p.d) * 8);
+        v_lane_off[i] = 2u * (uint32_t)(row * (int)p.vs.n + src_granule(c, p.dv) * 8);
     }
     auto dst_of = [&](int t, int which, int i) {             // LDS byte address of copy i of this wave
         return lds0 + 2u * (uint32_t)((t & (NSTAGE - 1)) * T::STAGE_ELEMS + which * T::TILE_ELEMS + (wave * NDMA + i) * 512);
@@ -133,7 +134,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void fwd_kernel(const Fwd
         for (int i = 0; i < NDMA; ++i) {
             const int row = (wave * NDMA + i) * T::ROWS_PER_DMA + dma_row_in;
             const int key = min(t * BN + row, klimit - 1);   // tail rows re-read the last attended key
-            const int c = src_granule(dma_gran ^ swz<D>(row), p.d);
+            const int c = src_granule(dma_gran ^ swz<D>(row), which ? p.dv : p.d);
             dma16(base + (int64_t)key * row_stride + c * 8, dst_of(t, which, i));
         }
     };
@@ -439,7 +440,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void fwd_kernel(const Fwd
                     const f32x16& a = oacc[db];
                     u32x2 w = {pack_bf16(a[4 * g] * inv, a[4 * g + 1] * inv),
                                pack_bf16(a[4 * g + 2] * inv, a[4 * g + 3] * inv)};
-                    if (32 * db + 8 * g + 4 * h < p.d) *reinterpret_cast<u32x2*>(orow + 32 * db + 8 * g + 4 * h) = w;
+                    if (32 * db + 8 * g + 4 * h < p.dv) *reinterpret_cast<u32x2*>(orow + 32 * db + 8 * g + 4 * h) = w;
                 }
             if (p.lse && h == 0) {
                 const float v = l > 0.f ? (m_run * c_log2 + log2_fast(l)) * kLn2 : -INFINITY;
@@ -533,9 +534,9 @@ __global__ __launch_bounds__(256) void fwd_wide_kernel(const FwdParams p) {
 #pragma unroll
     for (int i = 0; i < NDMA; ++i) {
         const int row = (wave * NDMA + i) * T::ROWS_PER_DMA + dma_row_in;
-        const int c = src_granule(dma_gran ^ swz<D>(row), p.d);
-        k_lane_off[i] = 2u * (uint32_t)(row * (int)p.ks.n + c * 8);
-        v_lane_off[i] = 2u * (uint32_t)(row * (int)p.vs.n + c * 8);
+        const int c = dma_gran ^ swz<D>(row);
+        k_lane_off[i] = 2u * (uint32_t)(row * (int)p.ks.n + src_granule(c, p.d) * 8);
+        v_lane_off[i] = 2u * (uint32_t)(row * (int)p.vs.n + src_granule(c, p.dv) * 8);
     }
     auto dst_of = [&](int stg, int which, int i) {
         return lds0 + 2u * (uint32_t)(stg * T::STAGE_ELEMS + which * T::TILE_ELEMS + (wave * NDMA + i) * 512);
@@ -850,7 +851,7 @@ __global__ __launch_bounds__(256) void fwd_wide_kernel(const FwdParams p) {
                     const f32x16& a = oacc[qb][db];
                     u32x2 w = {pack_bf16(a[4 * g] * inv, a[4 * g + 1] * inv),
                                pack_bf16(a[4 * g + 2] * inv, a[4 * g + 3] * inv)};
-                    if (32 * db + 8 * g + 4 * h < p.d) *reinterpret_cast<u32x2*>(orow + 32 * db + 8 * g + 4 * h) = w;
+                    if (32 * db + 8 * g + 4 * h < p.dv) *reinterpret_cast<u32x2*>(orow + 32 * db + 8 * g + 4 * h) = w;
                 }
             if (p.lse && h == 0) {
                 const float v = l > 0.f ? (m_run[qb] * c_log2 + log2_fast(l)) * kLn2 : -INFINITY;

@@ -484,10 +484,11 @@ static int attn_fwd_impl(const void* Q, const void* K, const void* V, void* O, v
                         int causal, const int32_t* kv_len,
                         const uint8_t* keep_mask, const int64_t* mask_strides,
                         const void* bias, int bias_dtype, const int64_t* bias_strides,
-                        void* stream, int mask_mode = kMaskU8) {
-    if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0) return FLAME_ATTN_ERR_INVALID;
+                        void* stream, int mask_mode = kMaskU8, int Dv = 0) {
+    if (Dv == 0) Dv = D;           // V and O may have a head dim of their own (forward only)
+    if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0 || Dv < 0) return FLAME_ATTN_ERR_INVALID;
     if (!(scale > 0.f) || !isfinite(scale)) return FLAME_ATTN_ERR_INVALID;
-    if (!head_dim_ok(D)) return FLAME_ATTN_ERR_UNSUPPORTED;
+    if (!head_dim_ok(D) || !head_dim_ok(Dv)) return FLAME_ATTN_ERR_UNSUPPORTED;
     int rc;
     if ((rc = check_view(Q, q_strides, q_off))) return rc;
     if ((rc = check_view(K, k_strides, k_off))) return rc;
@@ -506,6 +507,7 @@ static int attn_fwd_impl(const void* Q, const void* K, const void* V, void* O, v
     p.qs = mk(q_strides); p.ks = mk(k_strides); p.vs = mk(v_strides); p.os = mk(o_strides);
     p.B = B; p.H = H; p.Sq = N_q; p.Sk = N_kv;
     p.d = D;
+    p.dv = Dv;
     p.scale = scale;
     p.m.kv_len = kv_len;
     p.m.mask = keep_mask;
@@ -534,7 +536,7 @@ static int attn_fwd_impl(const void* Q, const void* K, const void* V, void* O, v
     // ... as 4 wavefronts of 64 queries when nothing is excluded at all, else as 8 wavefronts of 32
     const bool plain = !causal && kv_len == nullptr && N_kv % 64 == 0;
     // a keep-mask with vector-loadable rows over whole tiles and no bias: the lean masked kernel
-    const int DP = padded_head_dim(D);
+    const int DP = std::max(padded_head_dim(D), padded_head_dim(Dv));
     if (keep_mask != nullptr && bias == nullptr && p.m.rows16 && N_kv % 64 == 0)
         return DP == 128 ? launch_fwd<128, true, 4, true>(p, s) : launch_fwd<64, true, 4, true>(p, s);
     if (DP == 128)
@@ -787,9 +789,10 @@ FlameAttnStatus flame_sdpa_chunked_bf16(const void* q, const void* k, const void
     if (B <= 0 || H <= 0 || Q < 0 || K < 0 || Dh <= 0 || Dv <= 0) return FLAME_ATTN_STATUS_ERR_INVALID;
     if (Q == 0 || K == 0) return FLAME_ATTN_STATUS_OK;
     if (chunk <= 0) return FLAME_ATTN_STATUS_ERR_INVALID;
-    if (Dv != Dh) return FLAME_ATTN_STATUS_ERR_UNSUPPORTED;
     const int64_t qs[4] = {(int64_t)H * Q * Dh, (int64_t)Q * Dh, Dh, 1};
     const int64_t ks[4] = {(int64_t)H * K * Dh, (int64_t)K * Dh, Dh, 1};
+    const int64_t vs[4] = {(int64_t)H * K * Dv, (int64_t)K * Dv, Dv, 1};     // V [B,H,K,Dv], out [B,H,Q,Dv]
+    const int64_t os[4] = {(int64_t)H * Q * Dv, (int64_t)Q * Dv, Dv, 1};
     // bf16 keep-mask [B, mask_heads, Q, K], a value below 0.5 excludes: read in place by the masked kernel, so
     // the workspace (which the reference sizes for its own score chunks) is not needed at all
     (void)workspace; (void)workspace_bytes;
@@ -801,9 +804,9 @@ FlameAttnStatus flame_sdpa_chunked_bf16(const void* q, const void* k, const void
         ms[2] = K;
         ms[3] = 1;
     }
-    return to_status(attn_fwd_impl(q, k, v, out, nullptr, B, H, Q, K, Dh, scale, qs, ks, ks, qs, 0, 0, 0, 0, 0, causal,
+    return to_status(attn_fwd_impl(q, k, v, out, nullptr, B, H, Q, K, Dh, scale, qs, ks, vs, os, 0, 0, 0, 0, 0, causal,
                                    nullptr, static_cast<const uint8_t*>(mask), mask ? ms : nullptr, nullptr,
-                                   FLAME_ATTN_DTYPE_F32, nullptr, stream, kMaskBf16Keep));
+                                   FLAME_ATTN_DTYPE_F32, nullptr, stream, kMaskBf16Keep, Dv));
 }
 
 int streaming_attn_bf16_fp32_launch(const void* Q, const void* K, const void* V, int B, int H, int S, int Dh, int Dv,
@@ -812,11 +815,10 @@ int streaming_attn_bf16_fp32_launch(const void* Q, const void* K, const void* V,
                                     float scale, int chunk_size, int causal, const uint8_t* k_pad_mask,
                                     void* stream) {
     if (chunk_size <= 0) return FLAME_ATTN_ERR_INVALID;
-    if (Dv != Dh) return FLAME_ATTN_ERR_UNSUPPORTED;
     const int64_t qs[4] = {qB, qH, qS, qD}, ks[4] = {kB, kH, kS, kD}, vs[4] = {vB, vH, vS, vD}, os[4] = {oB, oH, oS, oD};
     const int64_t ms[4] = {(int64_t)H * S, S, 0, 1};     // [B,H,S] key-padding mask, 0 = excluded
-    return flame_attn_fwd_bf16(Q, K, V, O, nullptr, B, H, S, S, Dh, scale, qs, ks, vs, os, 0, 0, 0, 0, 0, causal,
-                               nullptr, k_pad_mask, k_pad_mask ? ms : nullptr, stream);
+    return attn_fwd_impl(Q, K, V, O, nullptr, B, H, S, S, Dh, scale, qs, ks, vs, os, 0, 0, 0, 0, 0, causal, nullptr,
+                         k_pad_mask, k_pad_mask ? ms : nullptr, nullptr, FLAME_ATTN_DTYPE_F32, nullptr, stream, kMaskU8, Dv);
 }
 
 bool sdpa_stream_bf16_launch(const void* dQ, const void* dK, const void* dV, void* dO, int B, int H, int Q_len,

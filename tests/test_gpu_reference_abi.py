@@ -118,11 +118,57 @@ def test_chunked_symbol_with_bf16_keep_mask_and_causal(oracle):
     torch.cuda.synchronize()
     ro, _, ro32 = oracle.sdpa_fwd(t[0], t[1], t[2], 0.125, causal=True, want_f32=True)
     assert_close_bf16(oracle, "O", to_f32(out), ro, ro32)
-    # Dv != Dh -> unsupported (2), bad chunk -> invalid (1): status enum of cuda/include/flame_cuda_status.h
-    assert lib.flame_sdpa_chunked_bf16(_p(q), _p(k), _p(v), B, H, Q, K, D, 32, ctypes.c_float(0.125), 64, 0, 1,
+    # a head dim above 128 -> unsupported (2), bad chunk -> invalid (1): status enum of cuda/include/flame_cuda_status.h
+    assert lib.flame_sdpa_chunked_bf16(_p(q), _p(k), _p(v), B, H, Q, K, D, 256, ctypes.c_float(0.125), 64, 0, 1,
                                        None, _p(out), None, ctypes.c_uint64(0), _stream()) == 2
     assert lib.flame_sdpa_chunked_bf16(_p(q), _p(k), _p(v), B, H, Q, K, D, D, ctypes.c_float(0.125), 0, 0, 1,
                                        None, _p(out), None, ctypes.c_uint64(0), _stream()) == 1
+
+
+@pytest.mark.parametrize("Dh,Dv", [(64, 32), (64, 128), (96, 64), (40, 104)])
+def test_value_head_dim_differs_from_query_head_dim(oracle, Dh, Dv):
+    """V and O may have a head dim of their own in the chunked and streaming entry points
+    (cuda/src/flame_sdpa_stub.cu:973-982, cuda/streaming_attn_bf16.h:7-17).  The oracle takes one head dim, so it
+    is given both sides zero-padded to the larger one: zero channels change neither the logits nor the other
+    channels of O."""
+    from flame_amd import capi
+    lib = capi.lib()
+    lib.flame_sdpa_chunked_bf16.restype = ctypes.c_int
+    B, H, Q, K = 2, 3, 150, 210
+    q, k = (W.f32_to_bf16_bits(W.normal_f32(650 + Dh, s, B * H * n * Dh).reshape(B, H, n, Dh)) for s, n in ((0, Q), (1, K)))
+    v = W.f32_to_bf16_bits(W.normal_f32(650 + Dv, 2, B * H * K * Dv).reshape(B, H, K, Dv))
+    Dm = max(Dh, Dv)
+
+    def pad(x):
+        out = np.zeros(x.shape[:3] + (Dm,), np.uint16)
+        out[..., :x.shape[3]] = x
+        return out
+
+    scale = 1.0 / math.sqrt(Dh)
+    qd, kd, vd = to_dev(q), to_dev(k), to_dev(v)
+    out = torch.full((B, H, Q, Dv), float("nan"), dtype=torch.bfloat16, device="cuda")
+    for causal in (0, 1):
+        rc = lib.flame_sdpa_chunked_bf16(_p(qd), _p(kd), _p(vd), B, H, Q, K, Dh, Dv, ctypes.c_float(scale), 64, causal, 1,
+                                         None, _p(out), None, ctypes.c_uint64(0), _stream())
+        assert rc == 0
+        torch.cuda.synchronize()
+        ro, _, ro32 = oracle.sdpa_fwd(pad(q), pad(k), pad(v), scale, causal=bool(causal), want_f32=True)
+        assert_close_bf16(oracle, f"O chunked Dh={Dh} Dv={Dv} causal={causal}", to_f32(out), ro[..., :Dv], ro32[..., :Dv])
+    # the streaming entry point (self-attention: one sequence length), strided
+    S = K
+    q2 = W.f32_to_bf16_bits(W.normal_f32(651 + Dh, 0, B * H * S * Dh).reshape(B, H, S, Dh))
+    q2d = to_dev(q2)
+    o2 = torch.full((B, H, S, Dv), float("nan"), dtype=torch.bfloat16, device="cuda")
+    sq = [ctypes.c_long(x) for x in q2d.stride()]
+    sk = [ctypes.c_long(x) for x in kd.stride()]
+    sv = [ctypes.c_long(x) for x in vd.stride()]
+    so = [ctypes.c_long(x) for x in o2.stride()]
+    rc = lib.streaming_attn_bf16_fp32_launch(_p(q2d), _p(kd), _p(vd), B, H, S, Dh, Dv, *sq, *sk, *sv, _p(o2), *so,
+                                             ctypes.c_float(scale), 128, 1, None, _stream())
+    assert rc == 0
+    torch.cuda.synchronize()
+    ro, _, ro32 = oracle.sdpa_fwd(pad(q2), pad(k), pad(v), scale, causal=True, want_f32=True)
+    assert_close_bf16(oracle, f"O streaming Dh={Dh} Dv={Dv}", to_f32(o2), ro[..., :Dv], ro32[..., :Dv])
 
 
 def test_streaming_symbol_causal_and_key_padding(oracle):
