@@ -108,7 +108,7 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
     const int n_kt = (p.Sk + BN - 1) / BN;
     int wg, part = 0, nparts = 1;
     if (p.n_whole < 0) {
-        wg = xcd_remap(blockIdx.x, gridDim.x);
+        wg = p.m.kv_len ? xcd_remap_heads(blockIdx.x, gridDim.x, n_kt) : xcd_remap(blockIdx.x, gridDim.x);
     } else if ((int)blockIdx.x < p.n_whole) {
         wg = xcd_remap(blockIdx.x, p.n_whole);
     } else {          // the split key blocks come last in dispatch order and fill the final, partial round
@@ -136,7 +136,18 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
 
     const int n_qt = (p.Sq + BM - 1) / BM;
     int qt_begin = p.m.causal ? (k0 / BM) : 0;
-    if (k0 >= klimit) qt_begin = n_qt;        // nothing attends to these keys: dK = dV = 0
+    if (k0 >= klimit || (p.m.causal && k0 >= p.Sq)) {
+        // Nothing attends to these keys (past the key length, or past the last query under the causal flag):
+        // dK = dV = 0, written at once.  Padded batches launch many such workgroups; they must not cost a
+        // prologue each.
+        f32x16 zero[D / 32];
+#pragma unroll
+        for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) zero[db][r] = 0.f;
+        dkdv_store<D>(p, zero, zero, b, hh, kw0 + n, h);
+        return;
+    }
     const int n_it = n_qt - qt_begin;
     // The walk visits the query tiles that need per-element exclusions first (all of them when an explicit
     // mask is given, else the causal diagonal tiles and a partial last tile) and the fully attended ones afterwards, so that each of the two loops runs one
@@ -756,7 +767,7 @@ __global__ __launch_bounds__(64 * NW, (NW == 4 && (!HASMASK || VECMASK)) ? 2 : 1
     const int n = lane & 31, h = lane >> 5;
 
     const int n_qt = (p.Sq + BM - 1) / BM;
-    const int wg = xcd_remap(blockIdx.x, gridDim.x);
+    const int wg = p.m.kv_len ? xcd_remap_heads(blockIdx.x, gridDim.x, n_qt) : xcd_remap(blockIdx.x, gridDim.x);
     const int qt = wg % n_qt;
     const int bh = wg / n_qt;
     const int b = bh / p.H, hh = bh % p.H;
@@ -1081,7 +1092,7 @@ __global__ __launch_bounds__(256) void bwd_dq_wide_kernel(const BwdParams p) {
     const int n = lane & 31, h = lane >> 5;
 
     const int n_qt = (p.Sq + BM - 1) / BM;
-    const int wg = xcd_remap(blockIdx.x, gridDim.x);
+    const int wg = p.m.kv_len ? xcd_remap_heads(blockIdx.x, gridDim.x, n_qt) : xcd_remap(blockIdx.x, gridDim.x);
     const int qt = wg % n_qt;
     const int bh = wg / n_qt;
     const int b = bh / p.H, hh = bh % p.H;

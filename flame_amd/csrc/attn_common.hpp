@@ -288,6 +288,17 @@ __device__ __forceinline__ int xcd_remap(int linear, int total) {
     constexpr int kXcd = 8;
     return (total % kXcd == 0) ? (linear % kXcd) * (total / kXcd) + linear / kXcd : linear;
 }
+// The same for batches whose sequences differ in length (per-batch key lengths): contiguous ranges would hand
+// whole batches, the long ones and the short ones, to different XCDs.  Here XCD x takes the (batch, head)
+// slices x, x + 8, x + 16, ...: every slice still stays in one L2, and the heads of one batch are spread
+// over all XCDs.  `per_head`: tiles per (batch, head) slice; the id runs slice-major.
+__device__ __forceinline__ int xcd_remap_heads(int linear, int total, int per_head) {
+    constexpr int kXcd = 8;
+    const int n_heads = total / per_head;
+    if (n_heads % kXcd != 0) return xcd_remap(linear, total);
+    const int x = linear % kXcd, j = linear / kXcd;
+    return ((j / per_head) * kXcd + x) * per_head + j % per_head;
+}
 
 struct Strides {
     int64_t b, h, n;   // element strides of a [B,H,N,D] bf16 view; the D stride is 1

@@ -80,7 +80,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void fwd_kernel(const Fwd
     const int n = lane & 31, h = lane >> 5;
 
     const int n_qt = (p.Sq + BM - 1) / BM;
-    const int wg = xcd_remap(blockIdx.x, gridDim.x);
+    const int wg = p.m.kv_len ? xcd_remap_heads(blockIdx.x, gridDim.x, n_qt) : xcd_remap(blockIdx.x, gridDim.x);
     const int qt = wg % n_qt;
     const int bh = wg / n_qt;
     const int b = bh / p.H, hh = bh % p.H;

@@ -200,8 +200,10 @@ int launch_bwd(const BwdParams& p, hipStream_t s) {
     const int64_t grid = n_kt * p.B * p.H;
     // 256-query workgroups (4 wavefronts of 64 queries) when they neither add padding rows nor leave compute units idle
     const int64_t n256 = (p.Sq + 255) / 256;
+    // (with key lengths the walks differ in length and the longest ones set the time: unless the units fill two
+    // rounds, twice as many workgroups of half the size finish sooner)
     const bool wide = !HASMASK && n256 * 256 <= ((int64_t)(p.Sq + 127) / 128) * 128 && n256 * p.B * p.H >= device_cu_count() &&
-                      wg_waves_override() != 4;
+                      !(p.m.kv_len && n256 * p.B * p.H < 2 * device_cu_count()) && wg_waves_override() != 4;
     const int64_t n_qt = wide ? n256 : (p.Sq + TQ::BM - 1) / TQ::BM;
     const int64_t grid_dq = n_qt * p.B * p.H;
     if (grid > 0x7fffffff || grid_dq > 0x7fffffff) return FLAME_ATTN_ERR_UNSUPPORTED;
@@ -532,7 +534,7 @@ static int attn_fwd_impl(const void* Q, const void* K, const void* V, void* O, v
     // without a workgroup
     const int64_t n256 = (N_q + 255) / 256;
     const bool wide = !hm && n256 * 256 <= ((N_q + 127) / 128) * 128 && n256 * B * H >= device_cu_count() &&
-                      wg_waves_override() != 4;
+                      !(kv_len && n256 * B * H < 2 * device_cu_count()) && wg_waves_override() != 4;
     // ... as 4 wavefronts of 64 queries when nothing is excluded at all, else as 8 wavefronts of 32
     const bool plain = !causal && kv_len == nullptr && N_kv % 64 == 0;
     // a keep-mask with vector-loadable rows over whole tiles and no bias: the lean masked kernel
