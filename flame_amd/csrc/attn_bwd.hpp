@@ -768,8 +768,8 @@ __global__ __launch_bounds__(64 * NW, (NW == 4 && (!HASMASK || VECMASK)) ? 2 : 1
 
     const int n_qt = (p.Sq + BM - 1) / BM;
     const int wg = p.m.kv_len ? xcd_remap_heads(blockIdx.x, gridDim.x, n_qt) : xcd_remap(blockIdx.x, gridDim.x);
-    const int qt = wg % n_qt;
-    const int bh = wg / n_qt;
+    int qt = wg % n_qt, bh = wg / n_qt;
+    if (p.m.causal && !p.m.kv_len) causal_longest_first(wg, n_qt, gridDim.x, qt, bh);
     const int b = bh / p.H, hh = bh % p.H;
     const int q0 = qt * BM;
     const int qw0 = q0 + wave * 32;
@@ -1093,8 +1093,8 @@ __global__ __launch_bounds__(256) void bwd_dq_wide_kernel(const BwdParams p) {
 
     const int n_qt = (p.Sq + BM - 1) / BM;
     const int wg = p.m.kv_len ? xcd_remap_heads(blockIdx.x, gridDim.x, n_qt) : xcd_remap(blockIdx.x, gridDim.x);
-    const int qt = wg % n_qt;
-    const int bh = wg / n_qt;
+    int qt = wg % n_qt, bh = wg / n_qt;
+    if (p.m.causal && !p.m.kv_len) causal_longest_first(wg, n_qt, gridDim.x, qt, bh);
     const int b = bh / p.H, hh = bh % p.H;
     const int q0 = qt * BM;
     const int qw0 = q0 + wave * 64;

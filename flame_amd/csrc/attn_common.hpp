@@ -300,6 +300,23 @@ __device__ __forceinline__ int xcd_remap_heads(int linear, int total, int per_he
     return ((j / per_head) * kXcd + x) * per_head + j % per_head;
 }
 
+// Causal problems: the key walk of query unit qt grows with qt, and workgroups start in id order, so the longest
+// walks must come first or they finish alone at the end.  Within the contiguous range of units that one XCD
+// works through (whole heads where the counts allow), the order becomes: last unit of every head, then the
+// units before them, and so on.  `wg`: unit id after xcd_remap, head-major; returns (qt, head) through refs.
+__device__ __forceinline__ void causal_longest_first(int wg, int n_qt, int total, int& qt, int& bh) {
+    const int per_xcd = (total % 8 == 0) ? total / 8 : total;
+    if (per_xcd % n_qt == 0) {
+        const int heads = per_xcd / n_qt;
+        const int base = wg / per_xcd * per_xcd, j = wg - base;
+        qt = n_qt - 1 - j / heads;
+        bh = base / n_qt + j % heads;
+    } else {
+        qt = n_qt - 1 - wg % n_qt;
+        bh = wg / n_qt;
+    }
+}
+
 struct Strides {
     int64_t b, h, n;   // element strides of a [B,H,N,D] bf16 view; the D stride is 1
 };
