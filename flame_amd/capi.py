@@ -195,10 +195,11 @@ def profiling_read() -> dict:
     return {name: (kt.total_ms[i], kt.launches[i]) for i, name in enumerate(KERNEL_KINDS)}
 
 
-def sage_quant(q, k, smooth_k=True):
+def sage_quant(q, k, smooth_k=True, want_ks=False):
     """Per-block int8 quantisation of Q (128 rows) and mean-smoothed K (64 rows).
 
-    Returns dict(qi8, ki8, sq, sk, kmean): int8 [B,H,S,D], fp32 [B,H,nblk], fp32 [B,H,D]."""
+    Returns dict(qi8, ki8, sq, sk, kmean[, ks]): int8 [B,H,S,D], fp32 [B,H,nblk], fp32 [B,H,D]; with
+    want_ks also the smoothed bf16 K that was quantised."""
     B, H, Sq, D = q.shape
     Sk = k.shape[2]
     dev = q.device
@@ -208,27 +209,40 @@ def sage_quant(q, k, smooth_k=True):
         sq=torch.empty((B, H, -(-Sq // 128)), dtype=torch.float32, device=dev),
         sk=torch.empty((B, H, -(-Sk // 64)), dtype=torch.float32, device=dev),
         kmean=torch.empty((B, H, D), dtype=torch.float32, device=dev))
-    rc = lib().flame_sage_quant_qk_int8(
+    if want_ks:
+        out["ks"] = torch.empty((B, H, Sk, D), dtype=torch.bfloat16, device=dev)
+    rc = lib().flame_sage_quant_qk_int8_ks(
         _ptr(q), _ptr(k), B, H, Sq, Sk, D, _i64x4(q.stride()), _i64x4(k.stride()),
         ctypes.c_int64(0), ctypes.c_int64(0), int(bool(smooth_k)),
-        _ptr(out["qi8"]), _ptr(out["ki8"]), _ptr(out["sq"]), _ptr(out["sk"]), _ptr(out["kmean"]), _stream())
+        _ptr(out["qi8"]), _ptr(out["ki8"]), _ptr(out["sq"]), _ptr(out["sk"]), _ptr(out["kmean"]),
+        _ptr(out.get("ks")), _stream())
     if rc != 0:
-        raise FlameAttnError("flame_sage_quant_qk_int8", rc)
+        raise FlameAttnError("flame_sage_quant_qk_int8_ks", rc)
     return out
 
 
-def sage_fwd(qz, v, scale, causal=False, kv_len=None, want_lse=False, out=None):
-    """O (and LSE) from quantised operands `qz` (the dict returned by sage_quant) and bf16 V."""
+def sage_fwd(qz, v, scale, causal=False, kv_len=None, want_lse=False, out=None, bias=None):
+    """O (and LSE) from quantised operands `qz` (the dict returned by sage_quant) and bf16 V.
+    bias: additive fp32 or bf16 [B|1, H|1, Sq, Sk] on the scaled logits (-inf excludes), or None."""
     B, H, Sq, D = qz["qi8"].shape
     Sk = qz["ki8"].shape[2]
     o = torch.empty((B, H, Sq, D), dtype=torch.bfloat16, device=v.device) if out is None else out
     lse = torch.empty((B * H, Sq), dtype=torch.float32, device=v.device) if want_lse else None
-    rc = lib().flame_sage_attn_fwd_int8(
+    bst, bdt = None, 1
+    if bias is not None:
+        assert bias.dim() == 4 and bias.dtype in (torch.float32, torch.bfloat16)
+        full = (B, H, Sq, Sk)
+        st = []
+        for ax in range(4):
+            assert bias.shape[ax] in (1, full[ax]), "bias is not broadcastable to [B,H,Sq,Sk]"
+            st.append(0 if (bias.shape[ax] == 1 and full[ax] != 1) else bias.stride(ax))
+        bst, bdt = _i64x4(st), (1 if bias.dtype == torch.float32 else 0)
+    rc = lib().flame_sage_attn_fwd_bias_int8(
         _ptr(qz["qi8"]), _ptr(qz["ki8"]), _ptr(qz["sq"]), _ptr(qz["sk"]), _ptr(v), _ptr(o), _ptr(lse),
         B, H, Sq, Sk, D, ctypes.c_float(scale), _i64x4(v.stride()), _i64x4(o.stride()),
-        ctypes.c_int64(0), ctypes.c_int64(0), int(bool(causal)), _ptr(kv_len), _stream())
+        ctypes.c_int64(0), ctypes.c_int64(0), int(bool(causal)), _ptr(kv_len), _ptr(bias), bdt, bst, _stream())
     if rc != 0:
-        raise FlameAttnError("flame_sage_attn_fwd_int8", rc)
+        raise FlameAttnError("flame_sage_attn_fwd_bias_int8", rc)
     return (o, lse) if want_lse else o
 
 

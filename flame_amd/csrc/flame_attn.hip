@@ -371,7 +371,16 @@ int flame_sage_quant_qk_int8(const void* Q, const void* K, int B, int H, int N_q
                              const int64_t* q_strides, const int64_t* k_strides, int64_t q_off, int64_t k_off,
                              int smooth_k, void* Qi8, void* Ki8, void* q_scales, void* k_scales, void* k_mean,
                              void* stream) {
+    return flame_sage_quant_qk_int8_ks(Q, K, B, H, N_q, N_kv, D, q_strides, k_strides, q_off, k_off, smooth_k, Qi8, Ki8,
+                                       q_scales, k_scales, k_mean, nullptr, stream);
+}
+
+int flame_sage_quant_qk_int8_ks(const void* Q, const void* K, int B, int H, int N_q, int N_kv, int D,
+                                const int64_t* q_strides, const int64_t* k_strides, int64_t q_off, int64_t k_off,
+                                int smooth_k, void* Qi8, void* Ki8, void* q_scales, void* k_scales, void* k_mean,
+                                void* K_smoothed, void* stream) {
     if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0) return FLAME_ATTN_ERR_INVALID;
+    if (K_smoothed && !aligned16(K_smoothed)) return FLAME_ATTN_ERR_UNSUPPORTED;
     if (!Qi8 || !Ki8 || !q_scales || !k_scales || !k_mean) return FLAME_ATTN_ERR_INVALID;
     if (D != 64 && D != 128) return FLAME_ATTN_ERR_UNSUPPORTED;
     int rc;
@@ -389,6 +398,7 @@ int flame_sage_quant_qk_int8(const void* Q, const void* K, int B, int H, int N_q
     p.ki8 = static_cast<int8_t*>(Ki8);
     p.sq = static_cast<float*>(q_scales);
     p.sk = static_cast<float*>(k_scales);
+    p.ks_out = static_cast<uint16_t*>(K_smoothed);
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int64_t bh = (int64_t)B * H;
     const int64_t nblk = (N_q + kSageQBlk - 1) / kSageQBlk + (N_kv + kSageKBlk - 1) / kSageKBlk;
@@ -449,7 +459,19 @@ int flame_sage_attn_fwd_int8(const void* Qi8, const void* Ki8, const void* q_sca
                              const void* V, void* O, void* LSE, int B, int H, int N_q, int N_kv, int D,
                              float scale, const int64_t* v_strides, const int64_t* o_strides,
                              int64_t v_off, int64_t o_off, int causal, const int32_t* kv_len, void* stream) {
+    return flame_sage_attn_fwd_bias_int8(Qi8, Ki8, q_scales, k_scales, V, O, LSE, B, H, N_q, N_kv, D, scale, v_strides,
+                                         o_strides, v_off, o_off, causal, kv_len, nullptr, FLAME_ATTN_DTYPE_F32, nullptr,
+                                         stream);
+}
+
+int flame_sage_attn_fwd_bias_int8(const void* Qi8, const void* Ki8, const void* q_scales, const void* k_scales,
+                                  const void* V, void* O, void* LSE, int B, int H, int N_q, int N_kv, int D,
+                                  float scale, const int64_t* v_strides, const int64_t* o_strides,
+                                  int64_t v_off, int64_t o_off, int causal, const int32_t* kv_len,
+                                  const void* bias, int bias_dtype, const int64_t* bias_strides, void* stream) {
     if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0) return FLAME_ATTN_ERR_INVALID;
+    if (bias && !bias_strides) return FLAME_ATTN_ERR_INVALID;
+    if (bias && bias_dtype != FLAME_ATTN_DTYPE_BF16 && bias_dtype != FLAME_ATTN_DTYPE_F32) return FLAME_ATTN_ERR_INVALID;
     if (!(scale > 0.f) || !isfinite(scale)) return FLAME_ATTN_ERR_INVALID;
     if (!Qi8 || !Ki8 || !q_scales || !k_scales) return FLAME_ATTN_ERR_INVALID;
     if (D != 64 && D != 128) return FLAME_ATTN_ERR_UNSUPPORTED;
@@ -470,6 +492,11 @@ int flame_sage_attn_fwd_int8(const void* Qi8, const void* Ki8, const void* q_sca
     p.scale = scale;
     p.kv_len = kv_len;
     p.causal = causal ? 1 : 0;
+    p.bias = bias;
+    if (bias) {
+        p.bb = bias_strides[0]; p.bhs = bias_strides[1]; p.bq = bias_strides[2]; p.bk = bias_strides[3];
+        p.bias_f32 = bias_dtype == FLAME_ATTN_DTYPE_F32;
+    }
     hipStream_t s = static_cast<hipStream_t>(stream);
     // 4 wavefronts per workgroup: with the small int8 K tile, 8-wavefront workgroups measured 7 % slower
     if (D == 128) return launch_sage_fwd<128, 4>(p, s);

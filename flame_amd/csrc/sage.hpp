@@ -33,6 +33,7 @@ struct SageQuantParams {
     int8_t* ki8;     // [B*H, Sk, D]
     float* sq;       // [B*H, ceil(Sq/128)]
     float* sk;       // [B*H, ceil(Sk/64)]
+    uint16_t* ks_out = nullptr;   // [B*H, Sk, D] bf16 or null: the smoothed K that was quantised, for a backward pass
 };
 
 // Channel mean of K, short sequences: one workgroup of 512 threads per (batch, head)
@@ -190,11 +191,17 @@ __global__ __launch_bounds__(256) void sage_quant_kernel(const SageQuantParams p
         else p.sk[(int64_t)bh * nkb + (blk - nqb)] = s;
     }
     int8_t* dst = (is_q ? p.qi8 : p.ki8) + (int64_t)bh * S * D;
+    uint16_t* ks_dst = (!is_q && p.ks_out) ? p.ks_out + (int64_t)bh * S * D : nullptr;
 #pragma unroll
     for (int i = 0; i < MAXC; ++i) {
         const int row = r0 + rsub + RPP * i;
         const bool ok = (rsub + RPP * i) < rows_blk && row < S;
         if (!ok) continue;
+        if (ks_dst) {       // the values are bf16 already: packing them again is exact
+            const u32x4 kw = {pack_bf16(x[i][0], x[i][1]), pack_bf16(x[i][2], x[i][3]), pack_bf16(x[i][4], x[i][5]),
+                              pack_bf16(x[i][6], x[i][7])};
+            *reinterpret_cast<u32x4*>(ks_dst + (int64_t)row * D + chunk * 8) = kw;
+        }
         uint32_t w0 = 0, w1 = 0;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -220,6 +227,10 @@ struct SageFwdParams {
     float scale;
     const int32_t* kv_len;
     int causal;
+    // additive bias on the scaled, dequantised logits (natural-log units; -inf excludes), fp32 or bf16, or null
+    const void* bias = nullptr;
+    int64_t bb = 0, bhs = 0, bq = 0, bk = 0;   // element strides over (b,h,q,k); 0 broadcasts
+    int bias_f32 = 1;
 };
 
 template <int D>
@@ -400,6 +411,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sage_fwd_kernel(cons
             for (int r = 0; r < 16; ++r) s[kb][r] = 0;
     };
     // int32 accumulators -> dequantised, scaled, masked logits (log2 units), in place; returns their maximum
+    const char* bbase = p.bias ? static_cast<const char*>(p.bias) + (b * p.bb + hh * p.bhs) * (p.bias_f32 ? 4 : 2) : nullptr;
     auto finish_masked = [&](i32x16 (&s)[2], int t) {
         const float f = qfac * skb[t];
         const int qi = qw0 + n;
@@ -409,8 +421,15 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sage_fwd_kernel(cons
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int key = t * BN + 32 * kb + acc_row(r, h);
-                const bool drop = key >= klimit || (p.causal && key > qi);
-                const float v = drop ? -INFINITY : (float)s[kb][r] * f;
+                const bool drop = (key >= klimit) | ((p.causal != 0) & (key > qi));
+                float v = (float)s[kb][r] * f;
+                if (bbase && !drop && qi < p.Sq) {      // the logits are in log2 units here
+                    const int64_t e = (int64_t)qi * p.bq + (int64_t)key * p.bk;
+                    const float bv = p.bias_f32 ? reinterpret_cast<const float*>(bbase)[e]
+                                                : __uint_as_float((uint32_t)reinterpret_cast<const uint16_t*>(bbase)[e] << 16);
+                    v = fmaf(bv, kLog2e, v);
+                }
+                v = drop ? -INFINITY : v;
                 tmax = fmaxf(tmax, v);
                 s[kb][r] = __float_as_int(v);
             }
@@ -549,7 +568,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sage_fwd_kernel(cons
     };
 
     // tiles [0, n_full) need no exclusions for any query of the workgroup
-    int n_full = klimit / BN;
+    int n_full = p.bias ? 0 : klimit / BN;       // a bias touches every logit
     if (p.causal) n_full = min(n_full, (q0 + 1) / BN);
     n_full = min(n_full, n_tiles);
 

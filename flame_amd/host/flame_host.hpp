@@ -642,18 +642,22 @@ inline Result<std::pair<Tensor, SdpaCtx>> sdpa_forward(const Tensor& q, const Te
             hooks->on_fwd_start(cfg, {(size_t)q.shape()[0], (size_t)q.shape()[1], (size_t)q.shape()[2], (size_t)k.shape()[2]});
         timer = std::make_unique<StreamTimer>(nullptr);
     }
-    auto r = detail::run_forward(q, k, v, mask, cfg.causal, cfg.scale, true);
+    // SaveLSE keeps O and the log-sum-exp for the backward; Recompute (:21-47) keeps neither and the backward
+    // runs the forward once more to get them back (the outputs are deterministic, so it sees the same O).
+    const bool keep = cfg.save != SdpaSave::Recompute;
+    auto r = detail::run_forward(q, k, v, mask, cfg.causal, cfg.scale, keep);
     if (!r.ok()) return r.error();
     SdpaCtx ctx;
-    ctx.q = q; ctx.k = k; ctx.v = v; ctx.o = r.value().o;
+    ctx.q = q; ctx.k = k; ctx.v = v;
+    if (keep) ctx.o = r.value().o;
     if (mask) ctx.attn_mask = *mask;
     ctx.scale = cfg.scale.value_or(1.0f / std::sqrt((float)q.shape()[3]));
     ctx.save = cfg.save;
     ctx.causal = cfg.causal;
-    ctx.lse = r.value().stats;
+    if (keep) ctx.lse = r.value().stats;
     ctx.shapes = {(size_t)q.shape()[0], (size_t)q.shape()[1], (size_t)q.shape()[2], (size_t)k.shape()[2]};
-    ctx.stats.bytes_saved = (uint64_t)ctx.o.numel() * 2 + (uint64_t)ctx.lse.numel() * 4;
-    ctx.stats.bytes_alloc = ctx.stats.bytes_saved;         // O and LSE are the only allocations of the forward
+    ctx.stats.bytes_saved = keep ? (uint64_t)ctx.o.numel() * 2 + (uint64_t)ctx.lse.numel() * 4 : 0;
+    ctx.stats.bytes_alloc = (uint64_t)r.value().o.numel() * 2 + (keep ? (uint64_t)ctx.lse.numel() * 4 : 0);   // what the forward allocated
     if (timer) {
         ctx.stats.fwd_ms = timer->stop();
         ctx.stats.syncs = 1;
@@ -681,6 +685,12 @@ inline Result<std::tuple<Tensor, Tensor, Tensor>> sdpa_backward(const SdpaCtx& c
     n.mask = ctx.attn_mask;
     n.scale = ctx.scale;
     n.causal = ctx.causal;
+    if (ctx.save == SdpaSave::Recompute) {          // nothing was kept: O and the log-sum-exp come from one more forward
+        auto f = detail::run_forward(ctx.q, ctx.k, ctx.v, ctx.attn_mask ? &*ctx.attn_mask : nullptr, ctx.causal, ctx.scale, true);
+        if (!f.ok()) return f.error();
+        n.output = f.value().o;
+        n.stats = f.value().stats;
+    }
     const SdpaHooks* hooks = debug_hooks();
     std::unique_ptr<StreamTimer> timer;
     if (hooks) {
@@ -936,7 +946,19 @@ inline Result<Tensor> prep_qk(const Tensor& x_bnhd, const Tensor* weight, const 
 // ------------------------------------------------------------------------------------ SageAttention
 // Builder-style API of the reference (src/sage_attention.rs:21-65).  `scale` is the softmax scale
 // (default 1/sqrt(D)); the reference's field of the same name is a divisor defaulting to sqrt(D)
-// (:108, :588), i.e. the same default arithmetic.  Inference only: int8 Q/K per block, mean-smoothed K.
+// (:108, :588), i.e. the same default arithmetic.  int8 Q/K per block, mean-smoothed K.
+//
+// forward(q, k, v, attention_mask): attention_mask is ADDED to the scores before the softmax, as the
+// reference does (:126-131): F32 or BF16, [B|1, H|1, Sq, Sk], -inf excludes a position.
+// forward_saving(...) also returns what the reference records for its backward (:134-150): the query, the
+// smoothed key and the value.  The materialised attention weights it saves as well are not produced here;
+// sage_attention_backward recomputes them tile by tile.
+struct SageSaved {
+    Tensor output, query, key_smoothed, value;
+    float scale = 0.f;
+    bool causal = false;
+};
+
 class SageAttention {
    public:
     SageAttention() = default;
@@ -945,12 +967,31 @@ class SageAttention {
     SageAttention with_smoothing(bool on) const { auto s = *this; s.smooth_k_ = on; return s; }
 
     Result<Tensor> forward(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor* attention_mask = nullptr) const {
-        if (attention_mask) return unsupported("SageAttention: explicit masks are not built (causal and key lengths are)");
+        auto r = run(q, k, v, attention_mask, false);
+        if (!r.ok()) return r.error();
+        return r.value().output;
+    }
+    Result<SageSaved> forward_saving(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor* attention_mask = nullptr) const {
+        return run(q, k, v, attention_mask, true);
+    }
+
+   private:
+    Result<SageSaved> run(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor* bias, bool save) const {
         auto dv = detail::validate(q, k, v, nullptr);
         if (!dv.ok()) return dv.error();
         const detail::Dims d = dv.value();
         for (const Tensor* t : {&q, &k, &v})
             if (!detail::abi_friendly(*t)) return unsupported("tensor view needs D stride 1 and 16-byte aligned rows");
+        std::vector<int64_t> bst(4, 0);
+        if (bias) {
+            const auto& bs = bias->shape();
+            if (bs.size() != 4) return invalid("attention_mask must be 4D [B|1, H|1, Q, K]");
+            if (!(bs[0] == d.B || bs[0] == 1) || !(bs[1] == d.H || bs[1] == 1) || bs[2] != d.Sq || bs[3] != d.Sk)
+                return invalid("attention_mask dims not broadcastable to [B,H,Q,K]");
+            if (bias->dtype() != DType::F32 && bias->dtype() != DType::BF16) return invalid("attention_mask must be F32 or BF16 (it is added to the scores)");
+            const int64_t full[4] = {d.B, d.H, d.Sq, d.Sk};
+            for (int i = 0; i < 4; ++i) bst[i] = (bs[i] == 1 && full[i] != 1) ? 0 : bias->strides()[i];
+        }
         const int64_t nqb = (d.Sq + 127) / 128, nkb = (d.Sk + 63) / 64;
         auto qi8 = Tensor::empty({d.B, d.H, d.Sq, d.D}, DType::I8);
         auto ki8 = Tensor::empty({d.B, d.H, d.Sk, d.D}, DType::I8);
@@ -959,23 +1000,53 @@ class SageAttention {
         auto km = Tensor::empty({d.B, d.H, d.D}, DType::F32);
         auto o = Tensor::empty({d.B, d.H, d.Sq, d.D}, DType::BF16);
         if (!qi8.ok() || !ki8.ok() || !sq.ok() || !sk.ok() || !km.ok() || !o.ok()) return cuda_error("hipMalloc", -1);
-        int rc = flame_sage_quant_qk_int8(q.base(), k.base(), d.B, d.H, d.Sq, d.Sk, d.D, q.strides().data(), k.strides().data(),
-                                          q.offset(), k.offset(), smooth_k_ ? 1 : 0, qi8.value().data(), ki8.value().data(),
-                                          sq.value().data(), sk.value().data(), km.value().data(), nullptr);
+        Tensor ks;
+        if (save) {
+            auto t = Tensor::empty({d.B, d.H, d.Sk, d.D}, DType::BF16);
+            if (!t.ok()) return t.error();
+            ks = t.value();
+        }
+        int rc = flame_sage_quant_qk_int8_ks(q.base(), k.base(), d.B, d.H, d.Sq, d.Sk, d.D, q.strides().data(), k.strides().data(),
+                                             q.offset(), k.offset(), smooth_k_ ? 1 : 0, qi8.value().data(), ki8.value().data(),
+                                             sq.value().data(), sk.value().data(), km.value().data(), save ? ks.data() : nullptr,
+                                             nullptr);
         if (rc == FLAME_ATTN_ERR_UNSUPPORTED) return unsupported("flame_sage_quant_qk_int8: head dim or layout not built");
         if (rc != 0) return cuda_error("flame_sage_quant_qk_int8", rc);
         const float sc = scale_.value_or(1.0f / std::sqrt((float)d.D));
-        rc = flame_sage_attn_fwd_int8(qi8.value().data(), ki8.value().data(), sq.value().data(), sk.value().data(), v.base(),
-                                      o.value().base(), nullptr, d.B, d.H, d.Sq, d.Sk, d.D, sc, v.strides().data(),
-                                      o.value().strides().data(), v.offset(), 0, causal_ ? 1 : 0, nullptr, nullptr);
+        rc = flame_sage_attn_fwd_bias_int8(qi8.value().data(), ki8.value().data(), sq.value().data(), sk.value().data(), v.base(),
+                                           o.value().base(), nullptr, d.B, d.H, d.Sq, d.Sk, d.D, sc, v.strides().data(),
+                                           o.value().strides().data(), v.offset(), 0, causal_ ? 1 : 0, nullptr,
+                                           bias ? bias->data() : nullptr,
+                                           bias && bias->dtype() == DType::BF16 ? FLAME_ATTN_DTYPE_BF16 : FLAME_ATTN_DTYPE_F32,
+                                           bias ? bst.data() : nullptr, nullptr);
         if (rc != 0) return cuda_error("flame_sage_attn_fwd_int8", rc);
-        return o.value();
+        return SageSaved{o.value(), q, ks, v, sc, causal_};
     }
 
-   private:
     std::optional<float> scale_;
     bool causal_ = false;
     bool smooth_k_ = true;
 };
+
+// sage_attention_backward (src/sage_attention.rs:470-505): the reference's backward of its Sage operator is
+// "standard attention backward" on (query, key_smoothed, value), ignoring the quantisation, from the
+// materialised attention weights it saved.  The same gradients here without that [B,H,Sq,Sk] tensor: one bf16
+// forward recomputes O and the log-sum-exp of (query, key_smoothed, value), then the tile-recompute backward
+// runs.  `scale` is the softmax scale (a multiplier; the reference passes its divisor).  As in the reference
+// the key gradient is the one with respect to the smoothed key.
+inline Result<autograd::AttentionGrads> sage_attention_backward(const Tensor& grad_output, const Tensor& query,
+                                                                const Tensor& key_smoothed, const Tensor& value, float scale,
+                                                                bool causal) {
+    auto f = detail::run_forward(query, key_smoothed, value, nullptr, causal, scale, true);
+    if (!f.ok()) return f.error();
+    autograd::FlashAttentionNode n;
+    n.query = query; n.key = key_smoothed; n.value = value;
+    n.output = f.value().o; n.stats = f.value().stats;
+    n.scale = scale; n.causal = causal;
+    return autograd::flash_attention_backward(n, grad_output);
+}
+inline Result<autograd::AttentionGrads> sage_attention_backward(const SageSaved& s, const Tensor& grad_output) {
+    return sage_attention_backward(grad_output, s.query, s.key_smoothed, s.value, s.scale, s.causal);
+}
 
 }  // namespace flame

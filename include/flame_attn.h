@@ -152,12 +152,30 @@ int flame_sage_quant_qk_int8(const void* Q, const void* K, int B, int H, int N_q
                              int smooth_k, void* Qi8, void* Ki8, void* q_scales, void* k_scales, void* k_mean,
                              void* stream);
 
+/* The same, and also writes the smoothed K that was quantised, Ks = bf16(float(K) - k_mean), contiguous bf16
+ * [B,H,N_kv,D] (K_smoothed may be null).  The reference saves this tensor for the backward of its Sage
+ * operator (src/sage_attention.rs:138-144, key_smoothed); see flame_host.hpp sage_attention_backward. */
+int flame_sage_quant_qk_int8_ks(const void* Q, const void* K, int B, int H, int N_q, int N_kv, int D,
+                                const int64_t* q_strides, const int64_t* k_strides, int64_t q_off, int64_t k_off,
+                                int smooth_k, void* Qi8, void* Ki8, void* q_scales, void* k_scales, void* k_mean,
+                                void* K_smoothed, void* stream);
+
 /* S = float(int32 Q^ K^^T) * sq * sk * scale on int8 MFMA, online softmax fp32, P bf16, O = P V
  * on bf16 MFMA.  LSE may be null. */
 int flame_sage_attn_fwd_int8(const void* Qi8, const void* Ki8, const void* q_scales, const void* k_scales,
                              const void* V, void* O, void* LSE, int B, int H, int N_q, int N_kv, int D,
                              float scale, const int64_t* v_strides, const int64_t* o_strides,
                              int64_t v_off, int64_t o_off, int causal, const int32_t* kv_len, void* stream);
+
+/* The same with an additive bias on the dequantised, scaled logits (fp32 or bf16, four element strides
+ * over (B,H,N_q,N_kv), 0 = broadcast; -inf excludes a position): the attention_mask argument of the
+ * reference's SageAttention::forward, which it adds to the scores before the softmax
+ * (src/sage_attention.rs:126-131). */
+int flame_sage_attn_fwd_bias_int8(const void* Qi8, const void* Ki8, const void* q_scales, const void* k_scales,
+                                  const void* V, void* O, void* LSE, int B, int H, int N_q, int N_kv, int D,
+                                  float scale, const int64_t* v_strides, const int64_t* o_strides,
+                                  int64_t v_off, int64_t o_off, int causal, const int32_t* kv_len,
+                                  const void* bias, int bias_dtype, const int64_t* bias_strides, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
  * Entry points with the reference's own names and argument lists: drop-in symbols for the

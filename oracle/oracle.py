@@ -163,7 +163,7 @@ def sage_quant(q, k, qblk=128, kblk=64, smooth_k=True):
 
 
 def sage_fwd(qi8, ki8, sq, sk, v, scale, qblk=128, kblk=64, causal=False, heads=None, kv_len=None, rows=None,
-             want_f32=False):
+             want_f32=False, bias=None):
     """Sage forward from quantised operands. Returns (O bf16 bits, LSE[, O fp32])."""
     B, H, Sq, D = qi8.shape
     Sk = ki8.shape[2]
@@ -176,8 +176,14 @@ def sage_fwd(qi8, ki8, sq, sk, v, scale, qblk=128, kblk=64, causal=False, heads=
     kvl = None if kv_len is None else np.ascontiguousarray(kv_len, dtype=np.int32)
     hb, he = (0, B * H) if heads is None else heads
     rb, re_ = (0, Sq) if rows is None else rows
+    bst = (0, 0, 0, 0)
+    if bias is not None:
+        bias = np.ascontiguousarray(bias, dtype=np.float32)
+        assert bias.ndim == 4 and bias.shape[2:] == (Sq, Sk) and bias.shape[0] in (1, B) and bias.shape[1] in (1, H)
+        bst = tuple(0 if bias.shape[i] == 1 and i < 2 else bias.strides[i] // 4 for i in range(4))
     rc = lib().oracle_sage_fwd(_p(qi8), _p(ki8), _p(sq), _p(sk), _p(v), B, H, Sq, Sk, D, qblk, kblk,
-                               ctypes.c_float(scale), int(bool(causal)), _p(kvl), hb, he, rb, re_,
+                               ctypes.c_float(scale), int(bool(causal)), _p(kvl),
+                               _p(bias), *(ctypes.c_int64(x) for x in bst), hb, he, rb, re_,
                                _p(O), _p(LSE), _p(O32))
     if rc != 0:
         raise RuntimeError(f"oracle_sage_fwd failed: {rc}")
@@ -185,13 +191,16 @@ def sage_fwd(qi8, ki8, sq, sk, v, scale, qblk=128, kblk=64, causal=False, heads=
 
 
 # ---------------------------------------------------------------- fp64 brute force (checker of the checker)
-def brute_sdpa_f64(q, k, v, scale, keep=None):
-    """Pure numpy fp64 attention on float arrays [.., Sq, D]; keep: bool [.., Sq, Sk] or None.
+def brute_sdpa_f64(q, k, v, scale, keep=None, bias=None):
+    """Pure numpy fp64 attention on float arrays [.., Sq, D]; keep: bool [.., Sq, Sk] or None; bias: additive,
+    broadcastable to [.., Sq, Sk], or None.
 
     Returns (O, LSE, P), all fp64.  Written from the textbook definition, not from the C file.
     """
     q, k, v = (np.asarray(t, np.float64) for t in (q, k, v))
     s = np.einsum("...id,...jd->...ij", q, k) * float(scale)
+    if bias is not None:
+        s = s + np.asarray(bias, np.float64)
     if keep is not None:
         s = np.where(keep, s, -np.inf)
     m = s.max(axis=-1, keepdims=True)

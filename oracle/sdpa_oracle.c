@@ -436,7 +436,8 @@ int oracle_sage_quant(const uint16_t* Q, const uint16_t* K,
 /*
  * Sage forward from quantised operands:
  *   S_ij = (float)(int32 sum_d Qi8_id Ki8_jd) * (sq[i/qblk] * sk[j/kblk] * scale)
- *   key j is excluded when causal and j > i, or when j >= kv_len[b]
+ *   an optional additive fp32 bias [B|1,H|1,Sq,Sk] (element strides, 0 = broadcast) is added to S
+ *   (src/sage_attention.rs:126-131); key j is excluded when causal and j > i, or when j >= kv_len[b]
  *   P = softmax(S) in fp32 (naive, materialised); O = P V -> bf16 (O32: the same before rounding).
  *   A row with every key excluded gives O = 0 and LSE = -inf.
  * Only the query rows [row_begin, row_end) of the chosen heads are computed.
@@ -444,6 +445,7 @@ int oracle_sage_quant(const uint16_t* Q, const uint16_t* K,
 int oracle_sage_fwd(const int8_t* Qi8, const int8_t* Ki8, const float* sq, const float* sk,
                     const uint16_t* V, int B, int H, int Sq, int Sk, int D, int qblk, int kblk,
                     float scale, int causal, const int32_t* kv_len,
+                    const float* bias, int64_t bsb, int64_t bsh, int64_t bsq, int64_t bsk,
                     int heads_begin, int heads_end, int row_begin, int row_end,
                     uint16_t* O, float* LSE, float* O32) {
     if (check_dims(B, H, Sq, Sk, D) || qblk <= 0 || kblk <= 0) return -1;
@@ -452,7 +454,7 @@ int oracle_sage_fwd(const int8_t* Qi8, const int8_t* Ki8, const float* sq, const
     int fail = 0;
 #pragma omp parallel for schedule(dynamic, 1)
     for (int bh = heads_begin; bh < heads_end; ++bh) {
-        const int b = bh / H;
+        const int b = bh / H, hh = bh % H;
         float* v = (float*)malloc(sizeof(float) * (size_t)Sk * D);
         float* row = (float*)malloc(sizeof(float) * (size_t)Sk);
         float* o = (float*)malloc(sizeof(float) * (size_t)D);
@@ -472,6 +474,7 @@ int oracle_sage_fwd(const int8_t* Qi8, const int8_t* Ki8, const float* sq, const
                     for (int d = 0; d < D; ++d)
                         acc += (int32_t)Qh[(size_t)i * D + d] * (int32_t)Kh[(size_t)j * D + d];
                     float s = (float)acc * (sqi * sk[(size_t)bh * nkb + j / kblk] * scale);
+                    if (bias) s += bias[b * bsb + hh * bsh + i * bsq + j * bsk];     /* the reference adds its mask to the scores */
                     if ((causal && j > i) || j >= klim) s = -INFINITY;
                     row[j] = s;
                     if (s > m) m = s;

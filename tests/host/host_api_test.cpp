@@ -54,6 +54,11 @@ static std::vector<uint16_t> randn_bf16(size_t n) {
 static Tensor dev_bf16(const std::vector<uint16_t>& h, std::vector<int64_t> shape) {
     return Tensor::from_host(h.data(), std::move(shape), DType::BF16).value();
 }
+static std::vector<uint16_t> host_bits_of_bf16(const Tensor& t) {
+    std::vector<uint16_t> h((size_t)t.numel());
+    t.to_host(h.data());
+    return h;
+}
 static std::vector<float> host_f32_of_bf16(const Tensor& t) {
     std::vector<uint16_t> h((size_t)t.numel());
     t.to_host(h.data());
@@ -288,6 +293,25 @@ int main() {
                 compare("dV causal", host_f32_of_bf16(std::get<2>(g.value())), rdv);
             }
         }
+        // SdpaSave::Recompute keeps neither O nor the log-sum-exp; its backward recomputes them and gives the same bits
+        if (f.ok()) {
+            autograd_v4::SdpaConfig rc = cfg;
+            rc.save = autograd_v4::SdpaSave::Recompute;
+            auto fr = autograd_v4::sdpa_forward(q, k, v, nullptr, rc);
+            CHECK(fr.ok(), "sdpa_forward (Recompute) failed");
+            if (fr.ok()) {
+                CHECK(fr.value().second.stats.bytes_saved == 0, "Recompute must save nothing besides Q, K, V");
+                CHECK(host_bits_of_bf16(fr.value().first) == host_bits_of_bf16(f.value().first), "Recompute forward output differs");
+                auto g1 = autograd_v4::sdpa_backward(f.value().second, d_o);
+                auto g2 = autograd_v4::sdpa_backward(fr.value().second, d_o);
+                CHECK(g1.ok() && g2.ok(), "sdpa_backward (Recompute) failed");
+                if (g1.ok() && g2.ok())
+                    CHECK(host_bits_of_bf16(std::get<0>(g1.value())) == host_bits_of_bf16(std::get<0>(g2.value())) &&
+                              host_bits_of_bf16(std::get<1>(g1.value())) == host_bits_of_bf16(std::get<1>(g2.value())) &&
+                              host_bits_of_bf16(std::get<2>(g1.value())) == host_bits_of_bf16(std::get<2>(g2.value())),
+                          "Recompute gradients differ from SaveLSE gradients");
+            }
+        }
         cfg.dropout_p = 0.1f;
         CHECK(!autograd_v4::sdpa_forward(q, k, v, nullptr, cfg).ok(), "dropout must be refused");
         cfg.dropout_p = 0.f;
@@ -313,8 +337,52 @@ int main() {
             std::printf("  cosine sage vs bf16 = %.6f\n", c);
             CHECK(c >= 0.999, "sage cosine %.6f", c);
         }
-        Tensor m = Tensor::empty({1, 1, N, N}, DType::U8).value();
-        CHECK(!SageAttention().forward(q, k, v, &m).ok(), "sage + mask must be refused");
+        // attention_mask is added to the scores (src/sage_attention.rs:126-131): a 0 / -inf causal bias must
+        // reproduce the causal flag; a U8 mask is not something that can be added and is refused
+        {
+            std::vector<float> hb((size_t)N * N);
+            for (int i = 0; i < N; ++i)
+                for (int j = 0; j < N; ++j) hb[(size_t)i * N + j] = j > i ? -INFINITY : 0.f;
+            Tensor bias = Tensor::from_host(hb.data(), {1, 1, N, N}, DType::F32).value();
+            auto ob = SageAttention().forward(q, k, v, &bias);
+            auto oc = SageAttention().with_causal(true).forward(q, k, v);
+            CHECK(ob.ok() && oc.ok(), "sage bias / causal forward failed");
+            if (ob.ok() && oc.ok()) {
+                auto x = host_f32_of_bf16(ob.value()), y = host_f32_of_bf16(oc.value());
+                double worst = 0;
+                for (size_t i = 0; i < x.size(); ++i) worst = std::max(worst, (double)std::fabs(x[i] - y[i]));
+                std::printf("  sage additive causal bias vs causal flag: max abs diff %.3e\n", worst);
+                CHECK(worst <= 2e-2, "sage bias differs from the causal flag by %.3e", worst);
+            }
+            Tensor m = Tensor::empty({1, 1, N, N}, DType::U8).value();
+            CHECK(!SageAttention().forward(q, k, v, &m).ok(), "a U8 attention_mask cannot be added to the scores");
+        }
+        // backward of the Sage operator: standard attention backward on (query, smoothed key, value), against the
+        // naive recompute on the same three tensors
+        {
+            auto hdo = randn_bf16(hq.size());
+            Tensor d_o = dev_bf16(hdo, {B, H, N, D});
+            auto sv = SageAttention().forward_saving(q, k, v);
+            CHECK(sv.ok(), "sage forward_saving failed");
+            if (sv.ok()) {
+                auto g = sage_attention_backward(sv.value(), d_o);
+                CHECK(g.ok(), "sage_attention_backward failed");
+                auto hks = host_bits_of_bf16(sv.value().key_smoothed);
+                if (g.ok()) {
+                    std::vector<float> rdq, rdk, rdv;
+                    for (int bh = 0; bh < B * H; ++bh) {
+                        const size_t off = (size_t)bh * N * D;
+                        Naive nv = naive_head(&hq[off], &hks[off], &hv[off], &hdo[off], N, N, D, 1.0f / std::sqrt((float)D), false, nullptr);
+                        rdq.insert(rdq.end(), nv.dq.begin(), nv.dq.end());
+                        rdk.insert(rdk.end(), nv.dk.begin(), nv.dk.end());
+                        rdv.insert(rdv.end(), nv.dv.begin(), nv.dv.end());
+                    }
+                    compare("sage dQ", host_f32_of_bf16(g.value().dq), rdq);
+                    compare("sage dK", host_f32_of_bf16(g.value().dk), rdk);
+                    compare("sage dV", host_f32_of_bf16(g.value().dv), rdv);
+                }
+            }
+        }
     }
 
     // ---- 7. input preparation: fused RMS-norm + RoPE + [B,N,H,D]->[B,H,N,D] equals the three separate calls,

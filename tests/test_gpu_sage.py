@@ -126,6 +126,39 @@ def test_sage_blocks_of_different_magnitude(oracle):
     _check_sage_fwd(oracle, w, qz, ref, v, o_bf16c, causal=True)
 
 
+def test_sage_additive_bias_and_smoothed_k_output(oracle):
+    """The attention_mask of the reference's Sage operator is added to the scores (src/sage_attention.rs:126-131):
+    fp32 and bf16 biases, per head and broadcast, with excluded positions and a row that loses every key; and the
+    smoothed K that the quantiser can hand back for a backward pass, bit-exact."""
+    from flame_amd import capi
+    B, H, Sq, Sk, D = 2, 3, 200, 328, 128
+    w = W.config5(B=B, H=H, S=Sk, D=D)
+    qbits = w.q[:, :, :Sq].copy()
+    q, k, v = to_dev(qbits), to_dev(w.k), to_dev(w.v)
+    qz = capi.sage_quant(q, k, want_ks=True)
+    ref = oracle.sage_quant(qbits, w.k)
+    assert np.array_equal(qz["ks"].cpu().view(torch.int16).numpy().view(np.uint16), ref["ks"]), "smoothed K bits"
+    assert np.array_equal(qz["ki8"].cpu().numpy(), ref["ki8"])
+    rng = np.random.default_rng(11)
+    for shape, dt in (((B, H, Sq, Sk), torch.float32), ((1, H, Sq, Sk), torch.bfloat16), ((B, 1, Sq, Sk), torch.float32)):
+        bias = (rng.normal(size=shape) * 2).astype(np.float32)
+        bias[..., 5::9] = -np.inf
+        bias[0, 0, 7, :] = -np.inf
+        bt = torch.from_numpy(bias).cuda().to(dt)
+        bias_seen = bt.float().cpu().numpy()             # what the kernel reads (bf16-rounded in the second case)
+        for causal in (False, True):
+            o, lse = capi.sage_fwd(qz, v, w.scale, causal=causal, bias=bt, want_lse=True)
+            torch.cuda.synchronize()
+            ro, rlse, ro32 = oracle.sage_fwd(ref["qi8"], ref["ki8"], ref["sq"], ref["sk"], w.v, w.scale, causal=causal,
+                                             bias=bias_seen, want_f32=True)
+            assert_close_bf16(oracle, f"O_sage bias {shape} {dt} causal={causal}", to_f32(o), ro, ro32)
+            glse = lse.cpu().numpy().reshape(rlse.shape)
+            fin = np.isfinite(rlse)
+            assert np.array_equal(np.isfinite(glse), fin) and np.all(glse[~fin] == -np.inf)
+            assert oracle.max_abs(glse[fin], rlse[fin]) <= TOL_LSE
+            assert torch.all(o[0, 0, 7] == 0)
+
+
 def test_cfg5_production_shape(oracle):
     """B=2 H=24 S=4608 D=128: every int8 code and scale bit-exact; O cosine vs the bf16 kernel."""
     from flame_amd import capi

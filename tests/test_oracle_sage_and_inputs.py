@@ -150,6 +150,17 @@ def test_sage_forward_against_fp64_brute_force_on_dequantised_operands(oracle):
                                       want_f32=True)
         assert oracle.max_abs(o32, want_o) <= 2e-5, (name, oracle.max_abs(o32, want_o))
         assert oracle.max_abs(lse, want_lse) <= 2e-5, (name, oracle.max_abs(lse, want_lse))
+    # additive bias (the reference's attention_mask), per head and broadcast over heads, with excluded positions
+    rng = np.random.default_rng(5)
+    for shape in ((B, H, Sq, Sk), (B, 1, Sq, Sk), (1, 1, Sq, Sk)):
+        bias = rng.normal(size=shape).astype(np.float32) * 2
+        bias[..., 3::7] = -np.inf
+        bias[0, 0, 5, :] = -np.inf                       # a row that loses every key
+        want_o, want_lse, _ = oracle.brute_sdpa_f64(qd, kd, vf, scale, bias=np.broadcast_to(bias, (B, H, Sq, Sk)))
+        _, lse, o32 = oracle.sage_fwd(z["qi8"], z["ki8"], z["sq"], z["sk"], v, scale, bias=bias, want_f32=True)
+        fin = np.isfinite(want_lse)
+        assert not fin[0, 0, 5] and np.array_equal(np.isfinite(lse), fin)
+        assert oracle.max_abs(o32, want_o) <= 2e-5 and oracle.max_abs(lse[fin], want_lse[fin]) <= 2e-5, shape
     # the check has teeth: block scales indexed by the other operand's block size change the result
     bad_sq = np.repeat(z["sq"], 2, axis=-1)[..., :z["sq"].shape[-1]]     # as if Q blocks were 64 rows
     _, _, o_bad = oracle.sage_fwd(z["qi8"], z["ki8"], bad_sq, z["sk"], v, scale, want_f32=True)
