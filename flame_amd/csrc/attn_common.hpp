@@ -98,6 +98,53 @@ __device__ __forceinline__ void mfma32_vgpr_bpinned(f32x16& acc, bf16x8 a, bf16x
 #undef FATTN_PIN
 }
 
+// The int8 counterpart (v_mfma_i32_32x32x32_i8: D[32x32] += A[32x32] * B[32x32], 16 consecutive int8 of the
+// contraction per lane and operand, int32 accumulators in architectural VGPRs), same pinned B slots; the B
+// value is the 128-bit carrier that pin_b_fragment returned.
+template <int SLOT, int MODE>
+__device__ __forceinline__ void mfma32i8_vgpr_bpinned(i32x16& acc, u32x4 a, bf16x8 b, const i32x16& c) {
+    static_assert(SLOT >= 0 && SLOT < 32, "32 pinned fragments");
+#define FATTN_PIN(I, R)                                                                                                  \
+    if constexpr (SLOT == I) {                                                                                           \
+        if constexpr (MODE == 0) asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, 0" : "=&v"(acc) : "v"(a), R(b));     \
+        if constexpr (MODE == 1) asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0" : "+v"(acc) : "v"(a), R(b));     \
+        if constexpr (MODE == 2) asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %3" : "=&v"(acc) : "v"(a), R(b), "v"(c)); \
+    }
+    FATTN_PIN(0, "{a[128:131]}")
+    FATTN_PIN(1, "{a[132:135]}")
+    FATTN_PIN(2, "{a[136:139]}")
+    FATTN_PIN(3, "{a[140:143]}")
+    FATTN_PIN(4, "{a[144:147]}")
+    FATTN_PIN(5, "{a[148:151]}")
+    FATTN_PIN(6, "{a[152:155]}")
+    FATTN_PIN(7, "{a[156:159]}")
+    FATTN_PIN(8, "{a[160:163]}")
+    FATTN_PIN(9, "{a[164:167]}")
+    FATTN_PIN(10, "{a[168:171]}")
+    FATTN_PIN(11, "{a[172:175]}")
+    FATTN_PIN(12, "{a[176:179]}")
+    FATTN_PIN(13, "{a[180:183]}")
+    FATTN_PIN(14, "{a[184:187]}")
+    FATTN_PIN(15, "{a[188:191]}")
+    FATTN_PIN(16, "{a[192:195]}")
+    FATTN_PIN(17, "{a[196:199]}")
+    FATTN_PIN(18, "{a[200:203]}")
+    FATTN_PIN(19, "{a[204:207]}")
+    FATTN_PIN(20, "{a[208:211]}")
+    FATTN_PIN(21, "{a[212:215]}")
+    FATTN_PIN(22, "{a[216:219]}")
+    FATTN_PIN(23, "{a[220:223]}")
+    FATTN_PIN(24, "{a[224:227]}")
+    FATTN_PIN(25, "{a[228:231]}")
+    FATTN_PIN(26, "{a[232:235]}")
+    FATTN_PIN(27, "{a[236:239]}")
+    FATTN_PIN(28, "{a[240:243]}")
+    FATTN_PIN(29, "{a[244:247]}")
+    FATTN_PIN(30, "{a[248:251]}")
+    FATTN_PIN(31, "{a[252:255]}")
+#undef FATTN_PIN
+}
+
 // Moves a fragment into its pinned accumulation registers (the value the MFMAs above are given).
 template <int SLOT>
 __device__ __forceinline__ bf16x8 pin_b_fragment(u32x4 w) {

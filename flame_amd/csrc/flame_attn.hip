@@ -431,8 +431,9 @@ int flame_sage_quant_qk_int8_ks(const void* Q, const void* K, int B, int H, int 
 
 }  // extern "C"
 
+// wg_count workgroups starting at workgroup p.wg_base of the problem (0: all of them)
 template <int D, int NW>
-static int launch_sage_fwd(const SageFwdParams& p, hipStream_t s) {
+static int launch_sage_fwd(const SageFwdParams& p, hipStream_t s, int64_t wg_count = 0) {
     using T = SageTile<D>;
     static bool attr_done = false;
     auto kern = sage_fwd_kernel<D, NW>;
@@ -443,12 +444,27 @@ static int launch_sage_fwd(const SageFwdParams& p, hipStream_t s) {
         attr_done = true;
     }
     constexpr int BM = 32 * NW;
-    const int64_t grid = (int64_t)((p.Sq + BM - 1) / BM) * p.B * p.H;
+    const int64_t grid = wg_count ? wg_count : (int64_t)((p.Sq + BM - 1) / BM) * p.B * p.H;
     if (grid > 0x7fffffff) return FLAME_ATTN_ERR_UNSUPPORTED;
-    {
-        ScopedKernelTimer t(FLAME_ATTN_KERNEL_SAGE_FWD, s);
-        hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(64 * NW), T::LDS_BYTES, s, p);
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(64 * NW), T::LDS_BYTES, s, p);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? FLAME_ATTN_OK : (int)e;
+}
+
+// the first wg_count 256-query workgroups of the problem
+template <int D>
+static int launch_sage_fwd_wide(const SageFwdParams& p, hipStream_t s, int64_t wg_count) {
+    using T = SageWideTile<D>;
+    static bool attr_done = false;
+    auto kern = sage_fwd_wide_kernel<D>;
+    if (!attr_done) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS_BYTES);
+        if (e != hipSuccess) return (int)e;
+        attr_done = true;
     }
+    if (wg_count > 0x7fffffff) return FLAME_ATTN_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(kern, dim3((unsigned)wg_count), dim3(256), T::LDS_BYTES, s, p);
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? FLAME_ATTN_OK : (int)e;
 }
@@ -498,7 +514,25 @@ int flame_sage_attn_fwd_bias_int8(const void* Qi8, const void* Ki8, const void* 
         p.bias_f32 = bias_dtype == FLAME_ATTN_DTYPE_F32;
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
-    // 4 wavefronts per workgroup: with the small int8 K tile, 8-wavefront workgroups measured 7 % slower
+    ScopedKernelTimer timer(FLAME_ATTN_KERNEL_SAGE_FWD, s);
+    // 256-query workgroups of four 64-query wavefronts (one per SIMD) when they neither add padding rows nor leave
+    // compute units without a workgroup, and nothing is excluded; else 128-query workgroups of four 32-query
+    // wavefronts.  A last round that would occupy at most half of the compute units with 256-query workgroups is
+    // cut into 128-query workgroups in a launch of its own: alone on its compute unit, such a workgroup takes little
+    // more than half the time of a 256-query one.
+    const int cus = device_cu_count();
+    const int64_t n256 = (N_q + 255) / 256, total256 = n256 * B * H;
+    const bool wide = n256 * 256 <= ((N_q + 127) / 128) * 128 && total256 >= cus && !causal && !kv_len && !bias &&
+                      N_kv % 64 == 0 && wg_waves_override() != 4;
+    if (wide) {
+        const int64_t rest = total256 % cus;
+        const int64_t wide_count = rest <= cus / 2 ? total256 - rest : total256;
+        if (2 * total256 > 0x7fffffff) return FLAME_ATTN_ERR_UNSUPPORTED;
+        rc = D == 128 ? launch_sage_fwd_wide<128>(p, s, wide_count) : launch_sage_fwd_wide<64>(p, s, wide_count);
+        if (rc != FLAME_ATTN_OK || wide_count == total256) return rc;
+        p.wg_base = (int)(2 * wide_count);
+        return D == 128 ? launch_sage_fwd<128, 4>(p, s, 2 * rest) : launch_sage_fwd<64, 4>(p, s, 2 * rest);
+    }
     if (D == 128) return launch_sage_fwd<128, 4>(p, s);
     return launch_sage_fwd<64, 4>(p, s);
 }

@@ -126,6 +126,30 @@ def test_sage_blocks_of_different_magnitude(oracle):
     _check_sage_fwd(oracle, w, qz, ref, v, o_bf16c, causal=True)
 
 
+@pytest.mark.parametrize("B,H,Sq,Sk,D", [(2, 16, 2048, 256, 64),      # 256 workgroups of 256 queries: whole rounds only
+                                          (1, 36, 2048, 192, 64),      # 288: the last 32 are cut into 64 of 128 queries
+                                          (1, 33, 2048, 320, 128),     # 264: the last 8 are cut into 16
+                                          (1, 50, 1280, 576, 128)])    # 250 < compute units: 128-query workgroups only
+def test_sage_large_problems_take_256_query_workgroups(oracle, B, H, Sq, Sk, D):
+    """Problems without exclusions that fill the chip run 256-query workgroups, with a short last round cut into
+    128-query workgroups: every head against the oracle, with Q blocks (128 rows) and K blocks (64 keys) scaled
+    apart so that a scale taken from a neighbouring block, or a query tile mapped to the wrong rows, shows."""
+    from flame_amd import capi
+    qf = W.normal_f32(67, 0, B * H * Sq * D).reshape(B, H, Sq, D)
+    kf = W.normal_f32(67, 1, B * H * Sk * D).reshape(B, H, Sk, D)
+    for ib in range(Sq // 128):
+        qf[:, :, 128 * ib:128 * (ib + 1)] *= np.float32((1.0, 3.0, 0.5, 2.0, 0.25)[ib % 5])
+    for jb in range(Sk // 64):
+        kf[:, :, 64 * jb:64 * (jb + 1)] *= np.float32((1.0, 2.0, 0.25, 1.5, 0.5, 2.0, 0.125)[jb % 7])
+    w = W.Workload("sage_wide", W.f32_to_bf16_bits(qf), W.f32_to_bf16_bits(kf),
+                   W.f32_to_bf16_bits(W.normal_f32(67, 2, B * H * Sk * D).reshape(B, H, Sk, D)), None, 0.5 / np.sqrt(D))
+    print(f"[sage] {B}x{H} Sq={Sq} Sk={Sk} D={D}", flush=True)
+    q, k, v = (to_dev(t) for t in (w.q, w.k, w.v))
+    qz, ref = _check_quant(oracle, w, smooth=True)
+    o_bf16, _ = capi.attn_fwd(q, k, v, w.scale)
+    _check_sage_fwd(oracle, w, qz, ref, v, o_bf16)
+
+
 def test_sage_additive_bias_and_smoothed_k_output(oracle):
     """The attention_mask of the reference's Sage operator is added to the scores (src/sage_attention.rs:126-131):
     fp32 and bf16 biases, per head and broadcast, with excluded positions and a row that loses every key; and the
