@@ -129,6 +129,57 @@ def input_prep_rate(capi, W, torch, B, H, N, D, dev, iters=20):
             "GB_per_s": nbytes / (ms * 1e-3) / 1e9, "frac_of_hbm_peak": nbytes / (ms * 1e-3) / 8e12}
 
 
+def tile_ops_line(args, capi, torch, dev):
+    """The element-wise tile primitives on one tile of the headline shape (all 24 heads, 1024 query rows, 4608
+    keys): median HIP-event time per call and the algorithmic bytes each moves, against 8 TB/s."""
+    BH, q_t, k_t = 24, 1024, 4608
+    n = BH * q_t * k_t
+    g = torch.Generator(device=dev).manual_seed(7)
+    logits = torch.randn((BH, q_t, k_t), device=dev, generator=g)
+    scores = logits.view(1, BH, q_t, k_t)
+    keep = (torch.rand((1, BH, q_t, k_t), device=dev, generator=g) < 0.9).to(torch.uint8)
+    keep_pad = torch.ones((1, BH, q_t, k_t), device=dev, dtype=torch.uint8)
+    keep_pad[..., k_t - k_t // 10:] = 0
+    add = torch.randn((BH, k_t), device=dev, generator=g)
+    lse = torch.logsumexp(logits, -1)
+    lse_other = lse.clone()
+    probs = torch.rand((BH, q_t, k_t), device=dev, generator=g).to(torch.bfloat16)
+    n_future = int((torch.arange(k_t, device=dev)[None, :] > torch.arange(q_t, device=dev)[:, None]).sum()) * BH
+    n_dropped = int((keep == 0).sum())
+    cases = [
+        ("flame_apply_causal_mask_fp32", lambda: capi.tile_causal_mask(scores), 4 * n_future),
+        ("flame_apply_attn_mask_fp32 (last tenth of the keys excluded)", lambda: capi.tile_attn_mask(scores, keep_pad),
+         n + 4 * int((keep_pad == 0).sum())),
+        ("flame_apply_attn_mask_fp32 (a random tenth excluded: scattered 4-byte stores)", lambda: capi.tile_attn_mask(scores, keep),
+         n + 4 * n_dropped),
+        ("flame_sdpa_add_mask_tile_fp32", lambda: capi.tile_add_mask(logits, keep.view(BH, q_t, k_t), add, bool_rank=3,
+                                                                      add_rank=2, k_total=k_t, causal=True), 9 * n + 4 * BH * k_t),
+        ("flame_sdpa_lse_from_logits_tile", lambda: capi.tile_lse_from_logits(logits), 4 * n + 4 * BH * q_t),
+        ("flame_sdpa_softmax_from_lse_tile", lambda: capi.tile_softmax_from_lse(logits, lse, out=probs), 6 * n + 4 * BH * q_t),
+        ("flame_sdpa_lse_merge_rows", lambda: capi.tile_lse_merge(lse, lse_other), 12 * BH * q_t),
+        ("flame_sdpa_dropout_bf16_inplace", lambda: capi.tile_dropout(probs, 0.1, 2024), 4 * n),
+    ]
+    out = {}
+    for name, fn, nbytes in cases:
+        for _ in range(3):
+            fn()
+        times = []
+        for _ in range(20):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            fn()
+            e1.record()
+            e1.synchronize()
+            times.append(e0.elapsed_time(e1))
+        ms = sorted(times)[len(times) // 2]
+        out[name] = {"ms_median": ms, "algorithmic_bytes": nbytes, "GB_per_s": nbytes / (ms * 1e-3) / 1e9,
+                     "frac_of_hbm_peak": nbytes / (ms * 1e-3) / 8e12}
+    print(json.dumps({"metric": "element-wise tile primitives, GB/s of algorithmic bytes", "unit": "GB/s", "n_gpus": 1,
+                      "dtype": "f32/bf16/u8", "data": "synthetic",
+                      "config": {"workload": "score tile [24, 1024, 4608]"}, "primitives": out}))
+    return 0
+
+
 def timed_loops(torch, capi, first, second, steps, warmup):
     """The three loops of the module docstring.  `first` / `second`: the two halves of a step (forward and
     backward; quantisation and forward).  Returns (wall ms per step, event medians, per-kernel averages)."""
@@ -232,6 +283,8 @@ def main():
     ap.add_argument("--traffic-calibration", action="store_true",
                     help="also run one plain 256 MiB device copy, so that FETCH_SIZE / WRITE_SIZE read under "
                          "rocprofv3 --pmc can be scaled by what the same counters report for a known size")
+    ap.add_argument("--tile-ops", action="store_true",
+                    help="time the element-wise tile primitives instead of an attention workload (a line of its own)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (heads shard without communication; "
@@ -245,9 +298,11 @@ def main():
         sys.exit(3)
     capi.lib()      # fails loudly when the HIP library is missing
 
+    dev = torch.device("cuda:0")
+    if args.tile_ops:
+        return tile_ops_line(args, capi, torch, dev)
     w = W.CONFIGS[args.config]()
     B, H, Sq, Sk, D = w.shape
-    dev = torch.device("cuda:0")
     if args.traffic_calibration:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
         torch.empty_like(src).copy_(src)          # one elementwise copy kernel: reads 256 MiB, writes 256 MiB

@@ -270,3 +270,76 @@ def prep_rmsnorm_rope(x_bnhd, weight=None, cos=None, sin=None, eps=1e-6, apply_n
     if rc != 0:
         raise FlameAttnError("flame_attn_prep_rmsnorm_rope_bf16", rc)
     return out
+
+
+# ---------------------------------------------------------------- element-wise primitives on score tiles
+# (the reference's symbols of src/cuda/ffi.rs:349-422; 0 = launched, 1 = not)
+def _tile_rc(fn: str, rc: int) -> None:
+    if rc != 0:
+        raise FlameAttnError(fn, rc)
+
+
+def tile_causal_mask(scores, q_offset=0, k_offset=0):
+    B, H, Q, K = scores.shape
+    assert scores.dtype == torch.float32 and scores.is_contiguous()
+    _tile_rc("flame_apply_causal_mask_fp32",
+             lib().flame_apply_causal_mask_fp32(_ptr(scores), B, H, Q, K, int(q_offset), int(k_offset), _stream()))
+    return scores
+
+
+def tile_attn_mask(scores, mask):
+    B, H, Q, K = scores.shape
+    assert scores.dtype == torch.float32 and mask.dtype == torch.uint8 and mask.shape == scores.shape
+    assert scores.is_contiguous() and mask.is_contiguous()
+    _tile_rc("flame_apply_attn_mask_fp32", lib().flame_apply_attn_mask_fp32(_ptr(scores), _ptr(mask), B, H, Q, K, _stream()))
+    return scores
+
+
+def tile_add_mask(logits, user_bool=None, user_add=None, q_abs_start=0, k_abs_start=0, bool_rank=0, add_rank=0, k_total=0,
+                  zero_is_mask=True, causal=False):
+    BH, q_t, k_t = logits.shape
+    assert logits.dtype == torch.float32 and logits.is_contiguous()
+    assert user_bool is None or (user_bool.dtype == torch.uint8 and user_bool.is_contiguous())
+    assert user_add is None or (user_add.dtype == torch.float32 and user_add.is_contiguous())
+    _tile_rc("flame_sdpa_add_mask_tile_fp32",
+             lib().flame_sdpa_add_mask_tile_fp32(_ptr(logits), _ptr(user_bool), _ptr(user_add), BH, q_t, k_t, int(q_abs_start),
+                                                 int(k_abs_start), int(bool_rank), int(add_rank), int(k_total),
+                                                 int(bool(zero_is_mask)), int(bool(causal)), _stream()))
+    return logits
+
+
+def tile_softmax_from_lse(logits, lse_row, out=None):
+    BH, q_t, k_t = logits.shape
+    assert logits.dtype == torch.float32 and lse_row.dtype == torch.float32 and tuple(lse_row.shape) == (BH, q_t)
+    assert logits.is_contiguous() and lse_row.is_contiguous()
+    if out is None:
+        out = torch.empty(logits.shape, dtype=torch.bfloat16, device=logits.device)
+    _tile_rc("flame_sdpa_softmax_from_lse_tile",
+             lib().flame_sdpa_softmax_from_lse_tile(_ptr(logits), _ptr(lse_row), _ptr(out), BH, q_t, k_t, _stream()))
+    return out
+
+
+def tile_lse_from_logits(logits):
+    BH, q_t, k_t = logits.shape
+    assert logits.dtype == torch.float32 and logits.is_contiguous()
+    out = torch.empty((BH, q_t), dtype=torch.float32, device=logits.device)
+    _tile_rc("flame_sdpa_lse_from_logits_tile",
+             lib().flame_sdpa_lse_from_logits_tile(_ptr(logits), _ptr(out), BH, q_t, k_t, _stream()))
+    return out
+
+
+def tile_lse_merge(lse_row, tile_lse_row):
+    BH, q_t = lse_row.shape
+    assert lse_row.dtype == torch.float32 and tile_lse_row.dtype == torch.float32 and lse_row.shape == tile_lse_row.shape
+    assert lse_row.is_contiguous() and tile_lse_row.is_contiguous()
+    _tile_rc("flame_sdpa_lse_merge_rows", lib().flame_sdpa_lse_merge_rows(_ptr(lse_row), _ptr(tile_lse_row), BH, q_t, _stream()))
+    return lse_row
+
+
+def tile_dropout(probs, p, seed):
+    BH, q_t, k_t = probs.shape
+    assert probs.dtype == torch.bfloat16 and probs.is_contiguous()
+    _tile_rc("flame_sdpa_dropout_bf16_inplace",
+             lib().flame_sdpa_dropout_bf16_inplace(_ptr(probs), ctypes.c_float(p), ctypes.c_uint64(seed & (2 ** 64 - 1)),
+                                                   BH, q_t, k_t, _stream()))
+    return probs

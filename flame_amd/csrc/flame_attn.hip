@@ -20,6 +20,7 @@
 #include "attn_fwd.hpp"
 #include "prep.hpp"
 #include "sage.hpp"
+#include "tile_ops.hpp"
 
 using namespace fattn;
 
@@ -993,6 +994,134 @@ int flame_attn_prep_rmsnorm_rope_bf16(const void* X, const void* weight, const v
     }
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? FLAME_ATTN_OK : (int)e;
+}
+
+// ---- element-wise primitives on score tiles, under the reference's names; 0 = launched, 1 = not (the
+// reference's convention for these symbols: src/kernels/sdpa_kernels.cu:232-403)
+
+static int tile_launched() { return hipGetLastError() == hipSuccess ? 0 : 1; }
+static bool tile_grid(int64_t n_threads, unsigned* grid) {
+    const int64_t g = (n_threads + 255) / 256;
+    if (g > 0x7fffffff) return false;
+    *grid = (unsigned)g;
+    return true;
+}
+
+int flame_apply_causal_mask_fp32(float* scores, int B, int H, int Q, int K, int q_offset, int k_offset, void* stream) {
+    if (B < 0 || H < 0 || Q < 0 || K < 0) return 1;
+    const int64_t total = (int64_t)B * H * Q * K;
+    if (total == 0) return 0;
+    if (!scores) return 1;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    unsigned grid;
+    if (K % 4 == 0 && aligned16(scores)) {
+        if (!tile_grid(total / 4, &grid)) return 1;
+        hipLaunchKernelGGL(tile_causal_mask_kernel<4>, dim3(grid), dim3(256), 0, s, scores, total / 4, Q, K, q_offset, k_offset);
+    } else {
+        if (!tile_grid(total, &grid)) return 1;
+        hipLaunchKernelGGL(tile_causal_mask_kernel<1>, dim3(grid), dim3(256), 0, s, scores, total, Q, K, q_offset, k_offset);
+    }
+    return tile_launched();
+}
+
+int flame_apply_attn_mask_fp32(float* scores, const uint8_t* mask, int B, int H, int Q, int K, void* stream) {
+    if (B < 0 || H < 0 || Q < 0 || K < 0) return 1;
+    const int64_t total = (int64_t)B * H * Q * K;
+    if (total == 0) return 0;
+    if (!scores || !mask) return 1;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    unsigned grid;
+    if (total % 4 == 0 && aligned16(scores) && (reinterpret_cast<uintptr_t>(mask) & 3) == 0) {
+        if (!tile_grid(total / 4, &grid)) return 1;
+        hipLaunchKernelGGL(tile_attn_mask_kernel<4>, dim3(grid), dim3(256), 0, s, scores, mask, total / 4);
+    } else {
+        if (!tile_grid(total, &grid)) return 1;
+        hipLaunchKernelGGL(tile_attn_mask_kernel<1>, dim3(grid), dim3(256), 0, s, scores, mask, total);
+    }
+    return tile_launched();
+}
+
+int flame_sdpa_add_mask_tile_fp32(float* logits, const uint8_t* user_bool, const float* user_add, int BH, int q_t, int k_t,
+                                  int q_abs_start, int k_abs_start, int user_bool_rank, int user_add_rank, int k_total,
+                                  int bool_zero_is_mask, int causal_flag, void* stream) {
+    if (BH < 0 || q_t < 0 || k_t < 0) return 1;
+    const int64_t total = (int64_t)BH * q_t * k_t;
+    if (total == 0) return 0;
+    if (!logits) return 1;
+    TileMaskParams p{logits, user_bool, user_add, q_t, k_t, q_abs_start, k_abs_start, user_bool_rank, user_add_rank, k_total,
+                     bool_zero_is_mask != 0, causal_flag != 0};
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    unsigned grid;
+    if (k_t % 4 == 0 && aligned16(logits)) {
+        if (!tile_grid(total / 4, &grid)) return 1;
+        hipLaunchKernelGGL(tile_add_mask_kernel<4>, dim3(grid), dim3(256), 0, s, p, total / 4);
+    } else {
+        if (!tile_grid(total, &grid)) return 1;
+        hipLaunchKernelGGL(tile_add_mask_kernel<1>, dim3(grid), dim3(256), 0, s, p, total);
+    }
+    return tile_launched();
+}
+
+int flame_sdpa_softmax_from_lse_tile(const float* logits, const float* lse_row, void* probs_bf16, int BH, int q_t, int k_t,
+                                     void* stream) {
+    if (BH < 0 || q_t < 0 || k_t < 0) return 1;
+    const int64_t total = (int64_t)BH * q_t * k_t;
+    if (total == 0) return 0;
+    if (!logits || !lse_row || !probs_bf16) return 1;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    uint16_t* probs = static_cast<uint16_t*>(probs_bf16);
+    unsigned grid;
+    if (k_t % 8 == 0 && aligned16(logits) && aligned16(probs_bf16)) {
+        if (!tile_grid(total / 8, &grid)) return 1;
+        hipLaunchKernelGGL(tile_softmax_from_lse_kernel<8>, dim3(grid), dim3(256), 0, s, logits, lse_row, probs, total / 8, k_t);
+    } else {
+        if (!tile_grid(total, &grid)) return 1;
+        hipLaunchKernelGGL(tile_softmax_from_lse_kernel<1>, dim3(grid), dim3(256), 0, s, logits, lse_row, probs, total, k_t);
+    }
+    return tile_launched();
+}
+
+int flame_sdpa_lse_from_logits_tile(const float* logits, float* out_lse_row, int BH, int q_t, int k_t, void* stream) {
+    if (BH < 0 || q_t < 0 || k_t < 0) return 1;
+    const int64_t rows = (int64_t)BH * q_t;
+    if (rows == 0) return 0;
+    if (!out_lse_row || (!logits && k_t > 0)) return 1;
+    unsigned grid;
+    if (!tile_grid(rows * 64, &grid)) return 1;
+    hipLaunchKernelGGL(tile_lse_from_logits_kernel, dim3(grid), dim3(256), 0, static_cast<hipStream_t>(stream), logits,
+                       out_lse_row, rows, k_t);
+    return tile_launched();
+}
+
+int flame_sdpa_lse_merge_rows(float* lse_row, const float* tile_lse_row, int BH, int q_t, void* stream) {
+    if (BH < 0 || q_t < 0) return 1;
+    const int64_t n = (int64_t)BH * q_t;
+    if (n == 0) return 0;
+    if (!lse_row || !tile_lse_row) return 1;
+    unsigned grid;
+    if (!tile_grid(n, &grid)) return 1;
+    hipLaunchKernelGGL(tile_lse_merge_kernel, dim3(grid), dim3(256), 0, static_cast<hipStream_t>(stream), lse_row, tile_lse_row, n);
+    return tile_launched();
+}
+
+int flame_sdpa_dropout_bf16_inplace(void* probs_bf16, float p, uint64_t seed, int BH, int q_t, int k_t, void* stream) {
+    if (BH < 0 || q_t < 0 || k_t < 0) return 1;
+    const int64_t total = (int64_t)BH * q_t * k_t;
+    if (total == 0) return 0;
+    if (!probs_bf16) return 1;
+    const float keep = 1.0f - p;
+    const float scale = keep > 0.0f ? 1.0f / keep : 0.0f;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    uint16_t* probs = static_cast<uint16_t*>(probs_bf16);
+    unsigned grid;
+    if (k_t % 8 == 0 && aligned16(probs_bf16)) {
+        if (!tile_grid(total / 8, &grid)) return 1;
+        hipLaunchKernelGGL(tile_dropout_kernel<8>, dim3(grid), dim3(256), 0, s, probs, p, scale, seed, total / 8, q_t, k_t);
+    } else {
+        if (!tile_grid(total, &grid)) return 1;
+        hipLaunchKernelGGL(tile_dropout_kernel<1>, dim3(grid), dim3(256), 0, s, probs, p, scale, seed, total, q_t, k_t);
+    }
+    return tile_launched();
 }
 
 #ifndef FLAME_ATTN_HIPCC_VERSION

@@ -252,6 +252,36 @@ bool sdpa_stream_bf16_launch(const void* dQ, const void* dK, const void* dV, voi
                              int64_t mask_stride_eq, int64_t mask_stride_eh, int64_t mask_stride_eb, int head_tile,
                              int q_tile, int max_q_tile, void* stream, char* unsupported_reason, int reason_buflen);
 
+/* ---- Element-wise primitives on score tiles, under the reference's names (src/cuda/ffi.rs:349-422, kernels in
+ * src/kernels/sdpa_kernels.cu:34-403): what the reference's chunked host loops call between their GEMMs.  The
+ * fused kernels above need none of them; they are for host code that keeps such a loop (the dropout path).
+ * Tiles are contiguous [BH, q_t, k_t] (scores: [B, H, Q, K]).  Return 0 when the kernel was launched, 1 otherwise
+ * (the reference's convention for these symbols); empty tiles return 0 without a launch. */
+
+/* src/cuda/ffi.rs:349-358: scores[b,h,q,k] = -1e9 where k_offset + k > q_offset + q. */
+int flame_apply_causal_mask_fp32(float* scores, int B, int H, int Q, int K, int q_offset, int k_offset, void* stream);
+/* src/cuda/ffi.rs:360-368: scores = -1e9 where the uint8 mask of the same shape is 0. */
+int flame_apply_attn_mask_fp32(float* scores, const uint8_t* mask, int B, int H, int Q, int K, void* stream);
+/* src/cuda/ffi.rs:370-385: logits += user_add (+ -1e30 where user_bool excludes) (+ -1e30 where the absolute key
+ * is past the absolute query), summed in that order.  Rank 3 operands have the tile's shape; rank 2 operands are
+ * [BH, k_total] rows indexed by k_abs_start + kj; any other rank ignores the operand.  bool_zero_is_mask picks
+ * which byte value excludes. */
+int flame_sdpa_add_mask_tile_fp32(float* logits, const uint8_t* user_bool, const float* user_add, int BH, int q_t, int k_t,
+                                  int q_abs_start, int k_abs_start, int user_bool_rank, int user_add_rank, int k_total,
+                                  int bool_zero_is_mask, int causal_flag, void* stream);
+/* src/cuda/ffi.rs:387-395: probs = bf16(exp(logits - lse_row[bh, qi])). */
+int flame_sdpa_softmax_from_lse_tile(const float* logits, const float* lse_row, void* probs_bf16, int BH, int q_t, int k_t,
+                                     void* stream);
+/* src/cuda/ffi.rs:397-404: out_lse_row[bh, qi] = log sum_k exp(logits[bh, qi, k]); an empty row gives -inf. */
+int flame_sdpa_lse_from_logits_tile(const float* logits, float* out_lse_row, int BH, int q_t, int k_t, void* stream);
+/* src/cuda/ffi.rs:406-412: lse_row = log(exp(lse_row) + exp(tile_lse_row)), element-wise over BH * q_t rows.  Two
+ * -inf give -inf (the reference's expression gives NaN there; its callers pass the finite -1e30). */
+int flame_sdpa_lse_merge_rows(float* lse_row, const float* tile_lse_row, int BH, int q_t, void* stream);
+/* src/cuda/ffi.rs:414-422: in place, probs = u < p ? 0 : bf16(float(probs) / (1 - p)), with the reference's
+ * counter-based uniform u(seed, bh, qi, kj) of the coordinates inside the tile (sdpa_kernels.cu:18-33), so the
+ * kept set is bit-identical to the reference's for the same seed and tile shape. */
+int flame_sdpa_dropout_bf16_inplace(void* probs_bf16, float p, uint64_t seed, int BH, int q_t, int k_t, void* stream);
+
 /* ------------------------------------------------------------------------------------------------
  * Profiling aids (the counterpart of the reference's SdpaStats / SdpaHooks timing fields,
  * src/autograd_v4/ops/sdpa.rs:55-79).  No counterpart in the FFI of the reference.

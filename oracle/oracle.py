@@ -263,3 +263,72 @@ def prep_rmsnorm_rope(x_bnhd, weight=None, cos=None, sin=None, eps=1e-6, apply_n
         y[..., 1::2] = (e * s_).astype(np.float32) + (o * c).astype(np.float32)
         x = y
     return f32_to_bf16(x)
+
+
+# ---------------------------------------------------------------- element-wise primitives on score tiles
+# (tile_ops_oracle.c; reference: src/kernels/sdpa_kernels.cu).  Arrays are modified in place where the
+# reference's kernels work in place; the result is returned as well.
+def tile_causal_mask(scores: np.ndarray, q_offset: int, k_offset: int) -> np.ndarray:
+    B, H, Q, K = scores.shape
+    assert scores.dtype == np.float32 and scores.flags.c_contiguous
+    lib().oracle_tile_causal_mask(_p(scores), B, H, Q, K, int(q_offset), int(k_offset))
+    return scores
+
+
+def tile_attn_mask(scores: np.ndarray, mask: np.ndarray) -> np.ndarray:
+    assert scores.dtype == np.float32 and mask.dtype == np.uint8 and scores.shape == mask.shape
+    assert scores.flags.c_contiguous and mask.flags.c_contiguous
+    lib().oracle_tile_attn_mask(_p(scores), _p(mask), ctypes.c_int64(scores.size))
+    return scores
+
+
+def tile_add_mask(logits: np.ndarray, user_bool=None, user_add=None, q_abs_start=0, k_abs_start=0, bool_rank=0,
+                  add_rank=0, k_total=0, zero_is_mask=True, causal=False) -> np.ndarray:
+    BH, q_t, k_t = logits.shape
+    assert logits.dtype == np.float32 and logits.flags.c_contiguous
+    if user_bool is not None:
+        assert user_bool.dtype == np.uint8 and user_bool.flags.c_contiguous
+    if user_add is not None:
+        assert user_add.dtype == np.float32 and user_add.flags.c_contiguous
+    lib().oracle_tile_add_mask(_p(logits), _p(user_bool), _p(user_add), BH, q_t, k_t, int(q_abs_start), int(k_abs_start),
+                               int(bool_rank), int(add_rank), int(k_total), int(bool(zero_is_mask)), int(bool(causal)))
+    return logits
+
+
+def tile_softmax_from_lse(logits: np.ndarray, lse_row: np.ndarray):
+    """Returns (bf16 bit patterns, the fp32 values before rounding)."""
+    BH, q_t, k_t = logits.shape
+    assert logits.dtype == np.float32 and lse_row.dtype == np.float32 and lse_row.shape == (BH, q_t)
+    probs = np.empty(logits.shape, np.uint16)
+    p32 = np.empty(logits.shape, np.float32)
+    lib().oracle_tile_softmax_from_lse(_p(np.ascontiguousarray(logits)), _p(np.ascontiguousarray(lse_row)), _p(probs), _p(p32),
+                                       BH, q_t, k_t)
+    return probs, p32
+
+
+def tile_lse_from_logits(logits: np.ndarray) -> np.ndarray:
+    BH, q_t, k_t = logits.shape
+    assert logits.dtype == np.float32
+    out = np.empty((BH, q_t), np.float32)
+    lib().oracle_tile_lse_from_logits(_p(np.ascontiguousarray(logits)), _p(out), BH, q_t, k_t)
+    return out
+
+
+def tile_lse_merge(lse_row: np.ndarray, tile_lse_row: np.ndarray) -> np.ndarray:
+    assert lse_row.dtype == np.float32 and tile_lse_row.dtype == np.float32 and lse_row.shape == tile_lse_row.shape
+    assert lse_row.flags.c_contiguous and tile_lse_row.flags.c_contiguous
+    lib().oracle_tile_lse_merge(_p(lse_row), _p(tile_lse_row), ctypes.c_int64(lse_row.size))
+    return lse_row
+
+
+def tile_uniform01(seed: int, b: int, qi: int, kj: int) -> float:
+    f = lib().oracle_tile_uniform01
+    f.restype = ctypes.c_float
+    return float(f(ctypes.c_uint64(seed & (2 ** 64 - 1)), int(b), int(qi), int(kj)))
+
+
+def tile_dropout(probs: np.ndarray, p: float, seed: int) -> np.ndarray:
+    BH, q_t, k_t = probs.shape
+    assert probs.dtype == np.uint16 and probs.flags.c_contiguous
+    lib().oracle_tile_dropout(_p(probs), ctypes.c_float(p), ctypes.c_uint64(seed & (2 ** 64 - 1)), BH, q_t, k_t)
+    return probs
