@@ -20,6 +20,7 @@
 #include "attn_fwd.hpp"
 #include "prep.hpp"
 #include "sage.hpp"
+#include "plan_cache.hpp"
 #include "tile_ops.hpp"
 
 using namespace fattn;
@@ -540,6 +541,13 @@ int flame_sage_attn_fwd_bias_int8(const void* Qi8, const void* Ki8, const void* 
 
 }  // extern "C"
 
+// the rule for the forward's query tile: 256 rows per workgroup (true) or 128
+static bool fwd_rule_wide(int B, int H, int N_q, bool has_mask_or_bias, bool has_kv_len) {
+    const int64_t n256 = (N_q + 255) / 256;
+    return !has_mask_or_bias && n256 * 256 <= ((int64_t)(N_q + 127) / 128) * 128 && n256 * B * H >= device_cu_count() &&
+           !(has_kv_len && n256 * B * H < 2 * device_cu_count()) && wg_waves_override() != 4;
+}
+
 static int attn_fwd_impl(const void* Q, const void* K, const void* V, void* O, void* LSE,
                         int B, int H, int N_q, int N_kv, int D, float scale,
                         const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
@@ -548,7 +556,7 @@ static int attn_fwd_impl(const void* Q, const void* K, const void* V, void* O, v
                         int causal, const int32_t* kv_len,
                         const uint8_t* keep_mask, const int64_t* mask_strides,
                         const void* bias, int bias_dtype, const int64_t* bias_strides,
-                        void* stream, int mask_mode = kMaskU8, int Dv = 0) {
+                        void* stream, int mask_mode = kMaskU8, int Dv = 0, int q_tile_plan = 0) {
     if (Dv == 0) Dv = D;           // V and O may have a head dim of their own (forward only)
     if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0 || Dv < 0) return FLAME_ATTN_ERR_INVALID;
     if (!(scale > 0.f) || !isfinite(scale)) return FLAME_ATTN_ERR_INVALID;
@@ -594,9 +602,10 @@ static int attn_fwd_impl(const void* Q, const void* K, const void* V, void* O, v
     const bool hm = keep_mask != nullptr || bias != nullptr;
     // 256-query workgroups when they neither add padding rows nor leave compute units
     // without a workgroup
-    const int64_t n256 = (N_q + 255) / 256;
-    const bool wide = !hm && n256 * 256 <= ((N_q + 127) / 128) * 128 && n256 * B * H >= device_cu_count() &&
-                      !(kv_len && n256 * B * H < 2 * device_cu_count()) && wg_waves_override() != 4;
+    bool wide = fwd_rule_wide(B, H, N_q, hm, kv_len != nullptr);
+    // a plan (128 or 256 query rows per workgroup) overrides the rule where the kernels leave the choice open
+    if (q_tile_plan == 128) wide = false;
+    else if (q_tile_plan == 256 && !hm) wide = true;
     // ... as 4 wavefronts of 64 queries when nothing is excluded at all, else as 8 wavefronts of 32
     const bool plain = !causal && kv_len == nullptr && N_kv % 64 == 0;
     // a keep-mask with vector-loadable rows over whole tiles and no bias: the lean masked kernel
@@ -868,9 +877,111 @@ FlameAttnStatus flame_sdpa_chunked_bf16(const void* q, const void* k, const void
         ms[2] = K;
         ms[3] = 1;
     }
-    return to_status(attn_fwd_impl(q, k, v, out, nullptr, B, H, Q, K, Dh, scale, qs, ks, vs, os, 0, 0, 0, 0, 0, causal,
-                                   nullptr, static_cast<const uint8_t*>(mask), mask ? ms : nullptr, nullptr,
-                                   FLAME_ATTN_DTYPE_F32, nullptr, stream, kMaskBf16Keep, Dv));
+    auto run = [&](int q_tile) {
+        return attn_fwd_impl(q, k, v, out, nullptr, B, H, Q, K, Dh, scale, qs, ks, vs, os, 0, 0, 0, 0, 0, causal, nullptr,
+                             static_cast<const uint8_t*>(mask), mask ? ms : nullptr, nullptr, FLAME_ATTN_DTYPE_F32, nullptr,
+                             stream, kMaskBf16Keep, Dv, q_tile);
+    };
+    // ---- the launch plan: the query tile of a workgroup (see plan_cache.hpp)
+    PlanCache& pc = PlanCache::instance();
+    const PlanConfig& cfg = pc.config();
+    const bool one_tile = mask != nullptr;                 // the masked kernels come with 128-row workgroups only
+    const int rule_q = fwd_rule_wide(B, H, Q, one_tile, false) ? 256 : 128;
+    const PlanKey key{B, H, Q, K, Dh, Dv, mask ? mask_heads : 0, causal ? 1 : 0};
+    int q_tile = rule_q;
+    uint64_t source = kPlanRule, candidates = 1, best_ns = 0;
+    if (cfg.q_override > 0) {
+        q_tile = (cfg.q_override <= 128 || one_tile) ? 128 : 256;
+        source = kPlanForced;
+        pc.with_stats([&](FlameSdpaAutotuneStats& st) {
+            st.env_forced += 1;
+            if (q_tile != cfg.q_override) st.clamped += 1;
+        });
+    } else if (cfg.enabled) {
+        Plan plan;
+        const bool hit = pc.lookup(key, &plan) && (plan.q_tile == 128 || (plan.q_tile == 256 && !one_tile)) && plan.k_tile == 64;
+        pc.with_stats([&](FlameSdpaAutotuneStats& st) { (hit ? st.cache_hits : st.cache_misses) += 1; });
+        if (hit) {
+            q_tile = plan.q_tile;
+            source = kPlanCacheHit;
+        } else {
+            hipStream_t hs = static_cast<hipStream_t>(stream);
+            hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+            if (hipStreamIsCapturing(hs, &capturing) != hipSuccess) (void)hipGetLastError();
+            if (one_tile || capturing != hipStreamCaptureStatusNone) {
+                pc.with_stats([&](FlameSdpaAutotuneStats& st) { st.skipped += 1; });
+            } else {
+                // both tiles on the caller's own problem: the forward only reads its inputs, so running it several
+                // times leaves the same output
+                double ms_of[2] = {0, 0};
+                bool ok = true;
+                hipEvent_t e0 = nullptr, e1 = nullptr;
+                ok = hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess;
+                for (int c = 0; c < 2 && ok; ++c) {
+                    const int cand = c == 0 ? 128 : 256;
+                    for (int i = 0; i < cfg.warmups && ok; ++i) ok = run(cand) == FLAME_ATTN_OK;
+                    ok = ok && hipEventRecord(e0, hs) == hipSuccess;
+                    for (int i = 0; i < cfg.repeats && ok; ++i) ok = run(cand) == FLAME_ATTN_OK;
+                    float ms_f = 0.f;
+                    ok = ok && hipEventRecord(e1, hs) == hipSuccess && hipEventSynchronize(e1) == hipSuccess &&
+                         hipEventElapsedTime(&ms_f, e0, e1) == hipSuccess;
+                    ms_of[c] = ms_f / cfg.repeats;
+                }
+                if (e0) (void)hipEventDestroy(e0);
+                if (e1) (void)hipEventDestroy(e1);
+                if (ok) {
+                    // within the tie margin the rule's tile stays
+                    const int fastest = ms_of[0] <= ms_of[1] ? 128 : 256;
+                    const double t_fast = std::min(ms_of[0], ms_of[1]), t_rule = ms_of[rule_q == 128 ? 0 : 1];
+                    q_tile = (t_rule <= t_fast * (1.0 + cfg.tie_eps)) ? rule_q : fastest;
+                    source = kPlanTuned;
+                    candidates = 2;
+                    best_ns = (uint64_t)(ms_of[q_tile == 128 ? 0 : 1] * 1e6);
+                    pc.with_stats([&](FlameSdpaAutotuneStats& st) { st.tuned += 1; });
+                } else {
+                    (void)hipGetLastError();
+                    pc.with_stats([&](FlameSdpaAutotuneStats& st) {
+                        st.errors += 1;
+                        st.fallback += 1;
+                    });
+                }
+            }
+            pc.store(key, q_tile, 64);
+        }
+    }
+    const int rc = run(q_tile);
+    pc.with_stats([&](FlameSdpaAutotuneStats& st) {
+        if (rc != FLAME_ATTN_OK) {
+            st.errors += 1;
+            return;
+        }
+        st.last_q_chunk = (uint64_t)q_tile;
+        st.last_k_chunk = 64;
+        st.last_candidate_count = candidates;
+        st.last_best_time_ns = best_ns;
+        st.last_plan_source = source;
+        st.last_shape_b = (uint64_t)B; st.last_shape_h = (uint64_t)H; st.last_shape_q = (uint64_t)Q; st.last_shape_k = (uint64_t)K;
+        st.last_shape_dh = (uint64_t)Dh; st.last_shape_dv = (uint64_t)Dv;
+        st.last_shape_mask_heads = (uint64_t)(mask ? mask_heads : 0);
+        st.last_shape_causal = causal ? 1 : 0;
+    });
+    return to_status(rc);
+}
+
+int flame_sdpa_autotune_get_stats(FlameSdpaAutotuneStats* out) {
+    if (!out) return FLAME_ATTN_ERR_INVALID;
+    PlanCache::instance().get_stats(out);
+    return FLAME_ATTN_OK;
+}
+
+int flame_sdpa_autotune_reset_stats(void) {
+    PlanCache::instance().reset_stats();
+    return FLAME_ATTN_OK;
+}
+
+int flame_sdpa_autotune_flush_cache(void) {
+    PlanCache::instance().flush();
+    return FLAME_ATTN_OK;
 }
 
 int streaming_attn_bf16_fp32_launch(const void* Q, const void* K, const void* V, int B, int H, int S, int Dh, int Dv,

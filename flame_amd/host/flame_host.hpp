@@ -747,9 +747,32 @@ inline Result<Gradients> backward_v4(const Tensor& loss) {
 // the reference's host-looped / per-row streaming kernels.  Same arguments and checks; the chunk size is
 // validated and otherwise ignored, the fused kernel streams K/V tiles by itself.
 // JSONL telemetry of the streaming entry point (src/perf_telemetry.rs): one line per call appended to
-// the file named by FLAME_SDPA_TELEMETRY_PATH, same keys in the same order.  The reference's tile
-// autotuner and plan cache have no counterpart here (tile shapes are fixed per head dim and problem
-// class), so those counters are always written as 0 and plan_source as 0.
+// the file named by FLAME_SDPA_TELEMETRY_PATH, same keys in the same order.  The plan and autotune fields
+// come from the library's launch-plan cache when the call went through flame_sdpa_chunked_bf16
+// (contiguous tensors, no mask or a contiguous bf16 mask), as in src/cuda_ops_bf16.rs:2081-2127.
+
+// staging::{SdpaAutotuneStats, sdpa_autotune_stats, reset_sdpa_autotune_stats, flush_sdpa_autotune_cache}
+// (src/staging.rs:582-672): the counters of the launch-plan cache, same field names.
+namespace staging {
+using SdpaAutotuneStats = FlameSdpaAutotuneStats;
+inline Result<SdpaAutotuneStats> sdpa_autotune_stats() {
+    SdpaAutotuneStats raw{};
+    const int rc = flame_sdpa_autotune_get_stats(&raw);
+    if (rc != 0) return cuda_error("flame_sdpa_autotune_get_stats", rc);
+    return raw;
+}
+inline Result<bool> reset_sdpa_autotune_stats() {
+    const int rc = flame_sdpa_autotune_reset_stats();
+    if (rc != 0) return cuda_error("flame_sdpa_autotune_reset_stats", rc);
+    return true;
+}
+inline Result<bool> flush_sdpa_autotune_cache() {
+    const int rc = flame_sdpa_autotune_flush_cache();
+    if (rc != 0) return cuda_error("flame_sdpa_autotune_flush_cache", rc);
+    return true;
+}
+}  // namespace staging
+
 namespace perf_telemetry {
 struct SdpaTelemetryRecord {                // :7-40
     size_t batch = 0, heads = 0, q_len = 0, k_len = 0, dh = 0, dv = 0, chunk_requested = 0;
@@ -842,15 +865,63 @@ namespace cuda_ops_bf16 {
 inline Result<Tensor> sdpa_stream_bf16(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor* mask, size_t chunk,
                                        bool causal, std::optional<float> scale) {
     if (chunk == 0) return invalid("sdpa_stream_bf16: chunk must be > 0");
-    if (!perf_telemetry::telemetry_enabled()) return flame::sdpa::forward_v4(q, k, v, mask, causal, scale);
+    // Contiguous BF16 tensors with no mask, or a contiguous BF16 mask [B, 1|H, Q, K], go through the chunked entry
+    // point, which consults the launch-plan cache; every other layout takes the general forward.
+    auto through_chunked = [&]() -> std::optional<Result<Tensor>> {
+        if (q.shape().size() != 4 || k.shape().size() != 4 || v.shape().size() != 4) return std::nullopt;
+        for (const Tensor* t : {&q, &k, &v})
+            if (t->dtype() != DType::BF16 || !t->is_contiguous() || t->offset() != 0) return std::nullopt;
+        const auto& qs = q.shape();
+        const int64_t B = qs[0], H = qs[1], Q = qs[2], D = qs[3], K = k.shape()[2], Dv = v.shape()[3];
+        if (k.shape()[0] != B || k.shape()[1] != H || k.shape()[3] != D || v.shape()[0] != B || v.shape()[1] != H ||
+            v.shape()[2] != K)
+            return std::nullopt;
+        int mask_heads = 1;
+        if (mask) {
+            const auto& ms = mask->shape();
+            if (mask->dtype() != DType::BF16 || !mask->is_contiguous() || mask->offset() != 0 || ms.size() != 4 || ms[0] != B ||
+                (ms[1] != 1 && ms[1] != H) || ms[2] != Q || ms[3] != K)
+                return std::nullopt;
+            mask_heads = (int)ms[1];
+        }
+        auto o = Tensor::empty({B, H, Q, Dv}, DType::BF16);
+        if (!o.ok()) return Result<Tensor>(o.error());
+        const float sc = scale.value_or(1.0f / std::sqrt((float)D));
+        const FlameAttnStatus st = flame_sdpa_chunked_bf16(q.base(), k.base(), v.base(), (int)B, (int)H, (int)Q, (int)K, (int)D, (int)Dv,
+                                                           sc, (int)std::min<size_t>(chunk, 1u << 30), causal ? 1 : 0, mask_heads,
+                                                           mask ? mask->base() : nullptr, o.value().base(), nullptr, 0, nullptr);
+        if (st == FLAME_ATTN_STATUS_ERR_UNSUPPORTED) return std::nullopt;       // e.g. a head dim the kernels lack: general path reports it
+        if (st != FLAME_ATTN_STATUS_OK) return Result<Tensor>(cuda_error("flame_sdpa_chunked_bf16", (int)st));
+        return Result<Tensor>(o.value());
+    };
+    bool used_plan = false;
+    auto run = [&]() -> Result<Tensor> {
+        if (auto r = through_chunked()) {
+            used_plan = true;
+            return *r;
+        }
+        return flame::sdpa::forward_v4(q, k, v, mask, causal, scale);
+    };
+    if (!perf_telemetry::telemetry_enabled()) return run();
     autograd_v4::StreamTimer timer(nullptr);
-    auto out = flame::sdpa::forward_v4(q, k, v, mask, causal, scale);
+    auto out = run();
     if (out.ok() && q.shape().size() == 4) {
         perf_telemetry::SdpaTelemetryRecord r;
         r.batch = (size_t)q.shape()[0]; r.heads = (size_t)q.shape()[1]; r.q_len = (size_t)q.shape()[2];
         r.k_len = (size_t)k.shape()[2]; r.dh = (size_t)q.shape()[3]; r.dv = (size_t)v.shape()[3];
         r.chunk_requested = chunk;
-        r.tuned_q_chunk = 256; r.tuned_k_chunk = 64;          // the largest tiles the kernels use; nothing is tuned
+        r.tuned_q_chunk = 256; r.tuned_k_chunk = 64;          // the general forward: the largest tiles the kernels use
+        if (used_plan) {
+            if (auto st = staging::sdpa_autotune_stats(); st.ok()) {
+                const auto& a = st.value();
+                r.tuned_q_chunk = a.last_q_chunk; r.tuned_k_chunk = a.last_k_chunk; r.plan_source = a.last_plan_source;
+                r.candidate_count = a.last_candidate_count; r.best_time_ns = a.last_best_time_ns;
+                r.autotune_env_forced = a.env_forced; r.autotune_clamped = a.clamped; r.autotune_skipped = a.skipped;
+                r.autotune_fallback = a.fallback; r.autotune_errors = a.errors; r.autotune_tuned = a.tuned;
+                r.cache_hits = a.cache_hits; r.cache_misses = a.cache_misses; r.cache_saved = a.cache_saved;
+                r.cache_loads = a.cache_loads; r.cache_load_errors = a.cache_load_errors; r.cache_entries = a.cache_entries;
+            }
+        }
         r.has_mask = mask != nullptr;
         r.mask_heads = mask && mask->shape().size() == 4 ? (size_t)mask->shape()[1] : 0;
         r.causal = causal;

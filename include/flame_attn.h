@@ -252,6 +252,23 @@ bool sdpa_stream_bf16_launch(const void* dQ, const void* dK, const void* dV, voi
                              int64_t mask_stride_eq, int64_t mask_stride_eh, int64_t mask_stride_eb, int head_tile,
                              int q_tile, int max_q_tile, void* stream, char* unsupported_reason, int reason_buflen);
 
+/* ---- Launch-plan cache of flame_sdpa_chunked_bf16 (src/ffi/cuda_ffi.h:119-121, src/cuda_ops_ffi.rs:60-85 and
+ * :308-310; implementation in the reference: cuda/src/flame_sdpa_stub.cu:38-650, :1080-1442).  The counters keep the
+ * reference's names and order; "q chunk" is the query tile of a workgroup here (128 or 256 rows), "k chunk" the
+ * key tile (64).  last_plan_source: 1 cache hit, 2 measured on this call, 3 taken from the rule, 4 forced by
+ * FLAME_SDPA_QCHUNK.  Environment variables as in the reference (cuda/src/flame_sdpa_stub.cu:617-650). */
+typedef struct FlameSdpaAutotuneStats {
+    uint64_t env_forced, clamped, skipped, fallback, errors, cache_hits, cache_misses, tuned, last_q_chunk, last_k_chunk,
+        cache_saved, cache_loads, cache_load_errors, cache_entries, last_candidate_count, last_best_time_ns,
+        last_plan_source, last_shape_b, last_shape_h, last_shape_q, last_shape_k, last_shape_dh, last_shape_dv,
+        last_shape_mask_heads, last_shape_causal;
+} FlameSdpaAutotuneStats;
+/* 0 on success, -1 for a null pointer. */
+int flame_sdpa_autotune_get_stats(FlameSdpaAutotuneStats* out);
+int flame_sdpa_autotune_reset_stats(void);
+/* Writes the cache file now if persistence is on (FLAME_SDPA_AUTOTUNE_PERSIST=1) and the cache changed. */
+int flame_sdpa_autotune_flush_cache(void);
+
 /* ---- Element-wise primitives on score tiles, under the reference's names (src/cuda/ffi.rs:349-422, kernels in
  * src/kernels/sdpa_kernels.cu:34-403): what the reference's chunked host loops call between their GEMMs.  The
  * fused kernels above need none of them; they are for host code that keeps such a loop (the dropout path).

@@ -564,7 +564,30 @@ int main() {
         CHECK(last.rfind("{\"op\":\"sdpa_stream_bf16\",\"timestamp_ns\":", 0) == 0, "telemetry line must start with op and timestamp");
         CHECK(last.find("\"q_len\":160,\"k_len\":160,\"dh\":64,\"dv\":64,\"chunk_requested\":512,") != std::string::npos, "shape keys");
         CHECK(last.find("\"has_mask\":0,\"causal\":1,") != std::string::npos, "flag keys");
-        CHECK(last.find("\"cache_load_errors\":0,\"cache_entries\":0}") != std::string::npos, "last keys");
+        // contiguous tensors without a mask went through the chunked entry point: its launch plan is in the line
+        // and in the counters (first call of this shape: a miss that measured both query tiles)
+        CHECK(last.find("\"plan_source\":2,") != std::string::npos, "plan measured on the first call of a shape");
+        CHECK(last.find("\"tuned_q_chunk\":128,\"tuned_k_chunk\":64,") != std::string::npos ||
+              last.find("\"tuned_q_chunk\":256,\"tuned_k_chunk\":64,") != std::string::npos, "plan tiles");
+        CHECK(last.find("\"candidate_count\":2,") != std::string::npos, "two candidates");
+        CHECK(last.find("\"cache_load_errors\":0,\"cache_entries\":") != std::string::npos && last.back() == '\n', "last keys");
+        {
+            auto st = staging::sdpa_autotune_stats();
+            CHECK(st.ok() && st.value().cache_misses >= 1 && st.value().tuned >= 1 && st.value().last_shape_q == 160 &&
+                      st.value().last_shape_causal == 1,
+                  "plan cache counters after the first call");
+            const uint64_t hits = st.ok() ? st.value().cache_hits : 0;
+            auto again = cuda_ops_bf16::sdpa_stream_bf16(q, k, v, nullptr, 512, true, std::nullopt);
+            auto st2 = staging::sdpa_autotune_stats();
+            CHECK(again.ok() && st2.ok() && st2.value().cache_hits == hits + 1 && st2.value().last_plan_source == 1,
+                  "second call of the shape is a cache hit");
+            if (again.ok() && out.ok()) {
+                CHECK(host_bits_of_bf16(again.value()) == host_bits_of_bf16(out.value()), "same output on the cached plan");
+            }
+            CHECK(staging::reset_sdpa_autotune_stats().ok() && staging::sdpa_autotune_stats().value().cache_hits == 0,
+                  "reset clears the counters");
+            CHECK(staging::flush_sdpa_autotune_cache().ok(), "flush without persistence is a no-op");
+        }
         const size_t at = last.find("\"elapsed_ms\":");
         CHECK(at != std::string::npos && std::atof(last.c_str() + at + 13) > 0.0, "elapsed_ms must be positive");
     }
