@@ -180,6 +180,62 @@ def tile_ops_line(args, capi, torch, dev):
     return 0
 
 
+def materialised_comparator(capi, torch, q, k, v, do, scale, o_fused, grads_fused, iters=5):
+    """The structure this path replaces, run on the same GPU for comparison: scores = Q K^T as one library GEMM
+    per head, softmax through this library's tile primitives, P kept in bf16 for the backward, PV / dV / dP / dQ /
+    dK as library GEMMs (the reference's materialised path: src/sdpa.rs:788-961, backward
+    src/autograd.rs:3918-3969).  Reports its time, its peak device memory next to the fused path's, and how far its
+    results are from the fused kernels'.  Unmasked problems only."""
+    B, H, Sq, D = q.shape
+    Sk = k.shape[2]
+    BH = B * H
+    q3, k3, v3, do3 = (t.reshape(BH, -1, D) for t in (q, k, v, do))
+
+    def fwd():
+        s = torch.bmm(q3, k3.transpose(1, 2)).float()            # bf16 GEMM, fp32 scores
+        s *= scale
+        lse = capi.tile_lse_from_logits(s)
+        p = capi.tile_softmax_from_lse(s, lse)                    # bf16 [BH, Sq, Sk]: what is saved for the backward
+        return p, torch.bmm(p, v3)
+
+    def bwd(p):
+        dv = torch.bmm(p.transpose(1, 2), do3)
+        dp = torch.bmm(do3, v3.transpose(1, 2)).float()
+        pf = p.float()
+        ds = (pf * (dp - (dp * pf).sum(-1, keepdim=True)) * scale).to(torch.bfloat16)
+        return torch.bmm(ds, k3), torch.bmm(ds.transpose(1, 2), q3), dv
+
+    p, o = fwd()
+    dq, dk, dv = bwd(p)
+    torch.cuda.synchronize()
+
+    def rel(a, b):
+        return float((a.float() - b.reshape(a.shape).float()).norm() / b.float().norm())
+
+    diffs = {"O": rel(o, o_fused), "dQ": rel(dq, grads_fused[0]), "dK": rel(dk, grads_fused[1]), "dV": rel(dv, grads_fused[2])}
+    del p, o, dq, dk, dv
+    torch.cuda.empty_cache()
+    base = torch.cuda.memory_allocated()
+    torch.cuda.reset_peak_memory_stats()
+    tf, tb = [], []
+    for _ in range(iters):
+        e = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+        e[0].record()
+        p, o = fwd()
+        e[1].record()
+        g = bwd(p)
+        e[2].record()
+        e[2].synchronize()
+        tf.append(e[0].elapsed_time(e[1]))
+        tb.append(e[1].elapsed_time(e[2]))
+        del p, o, g
+    peak = torch.cuda.max_memory_allocated() - base
+    return {"what": "QK^T / PV / backward products as library GEMMs, softmax by the tile primitives, bf16 P saved",
+            "forward_ms_median": sorted(tf)[len(tf) // 2], "backward_ms_median": sorted(tb)[len(tb) // 2],
+            "saved_between_forward_and_backward_bytes": BH * Sq * Sk * 2 + BH * Sq * D * 2,
+            "peak_device_MiB_beyond_inputs": peak / 2 ** 20, "rel_l2_vs_fused": diffs}
+
+
 def timed_loops(torch, capi, first, second, steps, warmup):
     """The three loops of the module docstring.  `first` / `second`: the two halves of a step (forward and
     backward; quantisation and forward).  Returns (wall ms per step, event medians, per-kernel averages)."""
@@ -373,6 +429,9 @@ def main():
     }
     if args.config == 2:
         out["input_prep"] = input_prep_rate(capi, W, torch, B, H, Sq, D, dev)
+        if not args.keep_mask:
+            del ws
+            out["materialised_comparator"] = materialised_comparator(capi, torch, q, k, v, do, w.scale, o, grads)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(w)
     print(json.dumps(out))
