@@ -129,6 +129,8 @@ def test_sage_blocks_of_different_magnitude(oracle):
 @pytest.mark.parametrize("B,H,Sq,Sk,D", [(2, 16, 2048, 256, 64),      # 256 workgroups of 256 queries: whole rounds only
                                           (1, 36, 2048, 192, 64),      # 288: the last 32 are cut into 64 of 128 queries
                                           (1, 33, 2048, 320, 128),     # 264: the last 8 are cut into 16
+                                          (2, 16, 2048, 64, 64),       # one key tile: prologue and a single step
+                                          (2, 16, 1948, 128, 128),     # two key tiles; the last query tile is partly empty
                                           (1, 50, 1280, 576, 128)])    # 250 < compute units: 128-query workgroups only
 def test_sage_large_problems_take_256_query_workgroups(oracle, B, H, Sq, Sk, D):
     """Problems without exclusions that fill the chip run 256-query workgroups, with a short last round cut into
@@ -137,7 +139,7 @@ def test_sage_large_problems_take_256_query_workgroups(oracle, B, H, Sq, Sk, D):
     from flame_amd import capi
     qf = W.normal_f32(67, 0, B * H * Sq * D).reshape(B, H, Sq, D)
     kf = W.normal_f32(67, 1, B * H * Sk * D).reshape(B, H, Sk, D)
-    for ib in range(Sq // 128):
+    for ib in range((Sq + 127) // 128):
         qf[:, :, 128 * ib:128 * (ib + 1)] *= np.float32((1.0, 3.0, 0.5, 2.0, 0.25)[ib % 5])
     for jb in range(Sk // 64):
         kf[:, :, 64 * jb:64 * (jb + 1)] *= np.float32((1.0, 2.0, 0.25, 1.5, 0.5, 2.0, 0.125)[jb % 7])
