@@ -403,7 +403,8 @@ int flame_sage_quant_qk_int8_ks(const void* Q, const void* K, int B, int H, int 
     p.ks_out = static_cast<uint16_t*>(K_smoothed);
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int64_t bh = (int64_t)B * H;
-    const int64_t nblk = (N_q + kSageQBlk - 1) / kSageQBlk + (N_kv + kSageKBlk - 1) / kSageKBlk;
+    // workgroups per (batch, head): one per Q block, one per pair of K blocks
+    const int64_t nblk = (N_q + kSageQBlk - 1) / kSageQBlk + ((N_kv + kSageKBlk - 1) / kSageKBlk + 1) / 2;
     if (bh * nblk > 0x7fffffff) return FLAME_ATTN_ERR_UNSUPPORTED;
     {
         ScopedKernelTimer t(FLAME_ATTN_KERNEL_SAGE_KMEAN, s);

@@ -119,31 +119,42 @@ __global__ __launch_bounds__(D) void sage_kmean_final_kernel(const SageQuantPara
     p.kmean[(int64_t)bh * D + tid] = m;
 }
 
-__device__ __forceinline__ int quant_code(float x, float s) {
-    if (s == 0.f) return 0;
-    float r = __builtin_rintf(x / s);      // IEEE division, round half to even
-    r = fminf(fmaxf(r, -128.f), 127.f);
-    return (int)r;
+// The low byte of the int8 code clamp(rint(x / s), -128, 127) with the IEEE quotient, round half to even, for
+// |x| <= 127 s (the block maximum defines s, so the clamp never acts); inv = 1 / s (0 when s is 0).
+// x * inv lies within 4e-5 of the correctly rounded quotient (both factors rounded once), so unless it falls within
+// 1e-4 of a rounding boundary k + 1/2 the two round to the same integer; only those rare elements (about one in
+// 5000) pay for the division itself.  Adding 1.5 * 2^23 rounds to the nearest even integer and leaves the code in
+// two's complement in the low mantissa bits.
+__device__ __forceinline__ uint32_t quant_code_byte(float x, float s, float inv) {
+    constexpr float kMagic = 12582912.0f;
+    const float t = x * inv;
+    float biased = t + kMagic;
+    const float r = biased - kMagic;
+    // written so that an infinite or NaN product (a subnormal scale) takes the division as well
+    if (__builtin_expect(!(0.5f - fabsf(t - r) >= 1.0e-4f) && s != 0.f, 0)) biased = x / s + kMagic;
+    return __float_as_uint(biased) & 0xffu;
 }
 
-// grid = B*H*(nqb + nkb); one workgroup quantises one block
+// grid = B*H*(nqb + ceil(nkb / 2)); one workgroup quantises 128 rows: one Q block, or two neighbouring K blocks
+// (rows 0..63 and 64..127 of its range, each with a scale of its own)
 template <int D>
 __global__ __launch_bounds__(256) void sage_quant_kernel(const SageQuantParams p) {
     constexpr int CPR = D / 8;
     constexpr int RPP = 256 / CPR;            // rows per pass
-    constexpr int MAXC = kSageQBlk / RPP;     // chunks per thread for a 128-row block
-    __shared__ float red[4];
+    constexpr int MAXC = kSageQBlk / RPP;     // chunks per thread for 128 rows; the first half of them are rows 0..63
+    static_assert(kSageQBlk == 2 * kSageKBlk && MAXC % 2 == 0, "a workgroup's 128 rows are one Q block or two K blocks");
+    __shared__ float red[4][2];
     const int tid = threadIdx.x;
     const int nqb = (p.Sq + kSageQBlk - 1) / kSageQBlk;
     const int nkb = (p.Sk + kSageKBlk - 1) / kSageKBlk;
-    const int per_bh = nqb + nkb;
+    const int nkp = (nkb + 1) / 2;
+    const int per_bh = nqb + nkp;
     const int bh = blockIdx.x / per_bh;
     const int blk = blockIdx.x % per_bh;
     const bool is_q = blk < nqb;
     const int b = bh / p.H, hh = bh % p.H;
-    const int rows_blk = is_q ? kSageQBlk : kSageKBlk;
     const int S = is_q ? p.Sq : p.Sk;
-    const int r0 = (is_q ? blk : blk - nqb) * rows_blk;
+    const int r0 = (is_q ? blk : blk - nqb) * kSageQBlk;
     const Strides st = is_q ? p.qs : p.ks;
     const uint16_t* src = (is_q ? p.q : p.k) + b * st.b + hh * st.h;
     const int chunk = tid % CPR;
@@ -160,53 +171,71 @@ __global__ __launch_bounds__(256) void sage_quant_kernel(const SageQuantParams p
     }
 
     float x[MAXC][8];
-    float amax = 0.f;
+    float amax[2] = {0.f, 0.f};               // rows 0..63 / 64..127
+    u32x4 raw[MAXC];
+#pragma unroll
+    for (int i = 0; i < MAXC; ++i) {          // all loads first
+        const int row = r0 + rsub + RPP * i;
+        raw[i] = ldg16(src + (int64_t)row * st.n + chunk * 8, row < S);
+    }
 #pragma unroll
     for (int i = 0; i < MAXC; ++i) {
-        const int row = r0 + rsub + RPP * i;
-        const bool ok = (rsub + RPP * i) < rows_blk && row < S;
-        const u32x4 w = ldg16(src + (int64_t)row * st.n + chunk * 8, ok);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            float lo = bf16_lo(w[j]), hi = bf16_hi(w[j]);
+            float lo = bf16_lo(raw[i][j]), hi = bf16_hi(raw[i][j]);
             if (!is_q) {   // smoothed K, rounded to bf16 exactly as the checker does
                 const uint32_t pk = pack_bf16(lo - mu[2 * j], hi - mu[2 * j + 1]);
                 lo = bf16_lo(pk);
                 hi = bf16_hi(pk);
             }
-            if (!ok) { lo = 0.f; hi = 0.f; }
+            if (r0 + rsub + RPP * i >= S) { lo = 0.f; hi = 0.f; }
             x[i][2 * j] = lo;
             x[i][2 * j + 1] = hi;
-            amax = fmaxf(amax, fmaxf(fabsf(lo), fabsf(hi)));
+            amax[i >= MAXC / 2] = fmaxf(amax[i >= MAXC / 2], fmaxf(fabsf(lo), fabsf(hi)));
         }
     }
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
-    if ((tid & 63) == 0) red[tid >> 6] = amax;
+    for (int hf = 0; hf < 2; ++hf) {
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) amax[hf] = fmaxf(amax[hf], __shfl_xor(amax[hf], off, 64));
+        if ((tid & 63) == 0) red[tid >> 6][hf] = amax[hf];
+    }
     __syncthreads();
-    amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-    const float s = amax / 127.0f;
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf) amax[hf] = fmaxf(fmaxf(red[0][hf], red[1][hf]), fmaxf(red[2][hf], red[3][hf]));
+    if (is_q) amax[0] = amax[1] = fmaxf(amax[0], amax[1]);
+    float s[2], inv[2];
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf) {
+        s[hf] = amax[hf] / 127.0f;
+        inv[hf] = s[hf] == 0.f ? 0.f : 1.0f / s[hf];
+    }
     if (tid == 0) {
-        if (is_q) p.sq[(int64_t)bh * nqb + blk] = s;
-        else p.sk[(int64_t)bh * nkb + (blk - nqb)] = s;
+        if (is_q) {
+            p.sq[(int64_t)bh * nqb + blk] = s[0];
+        } else {
+            const int kb = 2 * (blk - nqb);
+            p.sk[(int64_t)bh * nkb + kb] = s[0];
+            if (kb + 1 < nkb) p.sk[(int64_t)bh * nkb + kb + 1] = s[1];
+        }
     }
     int8_t* dst = (is_q ? p.qi8 : p.ki8) + (int64_t)bh * S * D;
     uint16_t* ks_dst = (!is_q && p.ks_out) ? p.ks_out + (int64_t)bh * S * D : nullptr;
 #pragma unroll
     for (int i = 0; i < MAXC; ++i) {
         const int row = r0 + rsub + RPP * i;
-        const bool ok = (rsub + RPP * i) < rows_blk && row < S;
-        if (!ok) continue;
+        if (row >= S) continue;
         if (ks_dst) {       // the values are bf16 already: packing them again is exact
             const u32x4 kw = {pack_bf16(x[i][0], x[i][1]), pack_bf16(x[i][2], x[i][3]), pack_bf16(x[i][4], x[i][5]),
                               pack_bf16(x[i][6], x[i][7])};
             *reinterpret_cast<u32x4*>(ks_dst + (int64_t)row * D + chunk * 8) = kw;
         }
+        const float sc = s[i >= MAXC / 2], iv = inv[i >= MAXC / 2];
         uint32_t w0 = 0, w1 = 0;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            w0 |= (uint32_t)(quant_code(x[i][j], s) & 0xff) << (8 * j);
-            w1 |= (uint32_t)(quant_code(x[i][4 + j], s) & 0xff) << (8 * j);
+            w0 |= quant_code_byte(x[i][j], sc, iv) << (8 * j);
+            w1 |= quant_code_byte(x[i][4 + j], sc, iv) << (8 * j);
         }
         u32x2 w = {w0, w1};
         *reinterpret_cast<u32x2*>(dst + (int64_t)row * D + chunk * 8) = w;

@@ -49,6 +49,29 @@ def test_quantisation_ties_and_zero_block(oracle):
     assert float(got["sk"][0, 0, 1]) == 0.0 and torch.all(got["ki8"][0, 0, 64:] == 0)
 
 
+def test_quantisation_rounding_boundaries_and_tiny_scales(oracle):
+    """The quantiser multiplies by 1/scale and falls back to the division only near a rounding boundary: blocks
+    whose quotients sit on and next to k + 1/2 for scales that are not powers of two, and blocks so small that the
+    scale is subnormal and its reciprocal overflows, must still give the codes of the IEEE quotient bit for bit."""
+    D = 64
+    rng = np.random.default_rng(17)
+    q = np.zeros((1, 2, 512, D), np.float32)
+    for blk, amax in enumerate((1.0, 3.0, 0.7109375, 254.0)):          # bf16-representable block maxima
+        s = np.float32(amax) / np.float32(127.0)
+        k = rng.integers(-126, 127, size=(128, D)).astype(np.float32)
+        x = (k + np.float32(0.5)) * s                                   # on a boundary before the bf16 rounding ...
+        x = W.bf16_bits_to_f32(W.f32_to_bf16_bits(x))                   # ... which moves it to either side, or not
+        x[0, 0] = amax
+        q[0, 0, 128 * blk:128 * (blk + 1)] = x
+    tiny = np.float32(2.0 ** -120)
+    q[0, 1, :128] = rng.integers(-64, 65, size=(128, D)).astype(np.float32) * tiny / 64
+    q[0, 1, 128:256] = rng.integers(-3, 4, size=(128, D)).astype(np.float32) * np.float32(2.0 ** -126)
+    kk = rng.normal(size=(1, 2, 128, D)).astype(np.float32) * np.float32(2.0 ** -118)
+    w = W.Workload("boundaries", W.f32_to_bf16_bits(q), W.f32_to_bf16_bits(kk), W.f32_to_bf16_bits(kk), None, 1.0)
+    _check_quant(oracle, w, smooth=True)
+    _check_quant(oracle, w, smooth=False)
+
+
 @pytest.mark.parametrize("D", [64, 128])
 def test_sage_forward_small_against_oracle_and_bf16_path(oracle, D):
     from flame_amd import capi
