@@ -332,3 +332,57 @@ def tile_dropout(probs: np.ndarray, p: float, seed: int) -> np.ndarray:
     assert probs.dtype == np.uint16 and probs.flags.c_contiguous
     lib().oracle_tile_dropout(_p(probs), ctypes.c_float(p), ctypes.c_uint64(seed & (2 ** 64 - 1)), BH, q_t, k_t)
     return probs
+
+
+# ---------------------------------------------------------------- dropout of the probabilities
+# (the reference's autograd_v4 operator, unchunked: src/autograd_v4/ops/sdpa.rs:229-231, :600-649; src/rng/mod.rs:14-24)
+def dropout_keep(seed: int, flat_index: int, p: float) -> bool:
+    return bool(lib().oracle_dropout_keep(ctypes.c_uint64(seed & (2 ** 64 - 1)), ctypes.c_uint64(flat_index), ctypes.c_float(p)))
+
+
+def dropout_uniforms(B, H, Sq, Sk, seed) -> np.ndarray:
+    """fp32 [B,H,Sq,Sk]: the uniform each probability is compared with, written from the recurrence in numpy (not
+    through the C file)."""
+    idx = (np.arange(B * H * Sq * Sk, dtype=np.uint64) & np.uint64(0xFFFFFFFF)).astype(np.uint32)
+    s = idx ^ np.uint32(seed & 0xFFFFFFFF)
+    s ^= s << np.uint32(13)
+    s ^= s >> np.uint32(17)
+    s ^= s << np.uint32(5)
+    return ((s >> np.uint32(8)).astype(np.float32) * np.float32(1.0 / 16777216.0)).reshape(B, H, Sq, Sk)
+
+
+def dropout_keep_mask(B, H, Sq, Sk, p, seed) -> np.ndarray:
+    """bool [B,H,Sq,Sk]: kept where the uniform is >= p."""
+    return dropout_uniforms(B, H, Sq, Sk, seed) >= np.float32(p)
+
+
+def sdpa_fwd_dropout(q, k, v, scale, p, seed, causal=False, kv_len=None, want_f32=False):
+    B, H, Sq, D = q.shape
+    Sk = k.shape[2]
+    q, k, v = (np.ascontiguousarray(t, dtype=np.uint16) for t in (q, k, v))
+    O = np.zeros((B, H, Sq, D), np.uint16)
+    LSE = np.zeros((B, H, Sq), np.float32)
+    O32 = np.zeros((B, H, Sq, D), np.float32) if want_f32 else None
+    kvl = None if kv_len is None else np.ascontiguousarray(kv_len, dtype=np.int32)
+    rc = lib().oracle_sdpa_fwd_dropout(_p(q), _p(k), _p(v), B, H, Sq, Sk, D, ctypes.c_float(scale), int(bool(causal)), _p(kvl),
+                                       ctypes.c_float(p), ctypes.c_uint64(seed & (2 ** 64 - 1)), _p(O), _p(LSE), _p(O32))
+    if rc != 0:
+        raise RuntimeError(f"oracle_sdpa_fwd_dropout failed: {rc}")
+    return (O, LSE, O32) if want_f32 else (O, LSE)
+
+
+def sdpa_bwd_dropout(q, k, v, o, do, scale, p, seed, causal=False, kv_len=None, want_f32=False):
+    B, H, Sq, D = q.shape
+    Sk = k.shape[2]
+    q, k, v, o, do = (np.ascontiguousarray(t, dtype=np.uint16) for t in (q, k, v, o, do))
+    dQ = np.zeros((B, H, Sq, D), np.uint16)
+    dK = np.zeros((B, H, Sk, D), np.uint16)
+    dV = np.zeros((B, H, Sk, D), np.uint16)
+    f = [np.zeros(t.shape, np.float32) for t in (dQ, dK, dV)] if want_f32 else [None] * 3
+    kvl = None if kv_len is None else np.ascontiguousarray(kv_len, dtype=np.int32)
+    rc = lib().oracle_sdpa_bwd_dropout(_p(q), _p(k), _p(v), _p(o), _p(do), B, H, Sq, Sk, D, ctypes.c_float(scale),
+                                       int(bool(causal)), _p(kvl), ctypes.c_float(p), ctypes.c_uint64(seed & (2 ** 64 - 1)),
+                                       _p(dQ), _p(dK), _p(dV), _p(f[0]), _p(f[1]), _p(f[2]))
+    if rc != 0:
+        raise RuntimeError(f"oracle_sdpa_bwd_dropout failed: {rc}")
+    return (dQ, dK, dV, *f) if want_f32 else (dQ, dK, dV)

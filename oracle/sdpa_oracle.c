@@ -98,7 +98,34 @@ typedef struct {
     int64_t msb, msh, msq, msk; /* element strides of mask over (b,h,q,k); 0 = broadcast */
     const float* bias;       /* additive fp32 bias on the scaled logits or NULL (src/sdpa.rs:288-305) */
     int64_t bsb, bsh, bsq, bsk; /* its element strides over (b,h,q,k); 0 = broadcast     */
+    float drop_p;            /* dropout probability, 0 = none                          */
+    uint64_t drop_seed;
 } mask_spec;
+
+/* Dropout of the attention probabilities as the reference's autograd_v4 operator draws it when it is not
+ * chunked (src/autograd_v4/ops/sdpa.rs:229-231, :600-649 with q_offset = k_offset = 0): one uniform per element of
+ * the [B*H, Sq, Sk] probability tensor, u = (xorshift32(seed32 ^ index32) >> 8) / 2^24 with index the flat element
+ * index and seed32 / index32 their low 32 bits (src/rng/mod.rs:14-24); an element is kept when u >= p, and kept
+ * elements are multiplied by 1 / (1 - p), both in fp32.  The probabilities themselves, and the log-sum-exp, are
+ * those of the undropped softmax. */
+static inline uint32_t drop_xorshift32(uint32_t x) {
+    x ^= x << 13;
+    x ^= x >> 17;
+    x ^= x << 5;
+    return x;
+}
+int oracle_dropout_keep(uint64_t seed, uint64_t flat_index, float p) {
+    const uint32_t s = drop_xorshift32((uint32_t)seed ^ (uint32_t)flat_index);
+    const float u = (float)(s >> 8) * (1.0f / 16777216.0f);
+    return u >= p;
+}
+/* factor applied to P[bh, i, j]: 0 or 1 / (1 - p); 1 without dropout */
+static inline float drop_factor(const mask_spec* ms, int bh, int i, int j, int Sq, int Sk) {
+    if (!(ms->drop_p > 0.f)) return 1.0f;
+    const uint64_t idx = ((uint64_t)bh * (uint64_t)Sq + (uint64_t)i) * (uint64_t)Sk + (uint64_t)j;
+    const float keep = 1.0f - ms->drop_p;
+    return oracle_dropout_keep(ms->drop_seed, idx, ms->drop_p) ? 1.0f / keep : 0.f;
+}
 
 static inline int excluded(const mask_spec* ms, int b, int h, int i, int j) {
     if (ms->causal && j > i) return 1;
@@ -163,7 +190,7 @@ int oracle_sdpa_fwd(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
                     int64_t msb, int64_t msh, int64_t msq, int64_t msk,
                     int heads_begin, int heads_end,
                     uint16_t* O, float* LSE, float* O32) {
-    mask_spec ms = {causal, kv_len, mask, msb, msh, msq, msk, NULL, 0, 0, 0, 0};
+    mask_spec ms = {causal, kv_len, mask, msb, msh, msq, msk, NULL, 0, 0, 0, 0, 0.f, 0};
     return sdpa_fwd_impl(Q, K, V, B, H, Sq, Sk, D, scale, ms, heads_begin, heads_end, 0, Sq, O, LSE, O32);
 }
 
@@ -176,7 +203,7 @@ int oracle_sdpa_fwd_rows(const uint16_t* Q, const uint16_t* K, const uint16_t* V
                          int64_t msb, int64_t msh, int64_t msq, int64_t msk,
                          int heads_begin, int heads_end, int row_begin, int row_end,
                          uint16_t* O, float* LSE, float* O32) {
-    mask_spec ms = {causal, kv_len, mask, msb, msh, msq, msk, NULL, 0, 0, 0, 0};
+    mask_spec ms = {causal, kv_len, mask, msb, msh, msq, msk, NULL, 0, 0, 0, 0, 0.f, 0};
     if (row_begin < 0 || row_end > Sq || row_begin > row_end) return -1;
     return sdpa_fwd_impl(Q, K, V, B, H, Sq, Sk, D, scale, ms, heads_begin, heads_end, row_begin, row_end, O, LSE, O32);
 }
@@ -187,7 +214,7 @@ int oracle_sdpa_fwd_bias(const uint16_t* Q, const uint16_t* K, const uint16_t* V
                          int B, int H, int Sq, int Sk, int D, float scale,
                          const float* bias, int64_t bsb, int64_t bsh, int64_t bsq, int64_t bsk,
                          uint16_t* O, float* LSE, float* O32) {
-    mask_spec ms = {0, NULL, NULL, 0, 0, 0, 0, bias, bsb, bsh, bsq, bsk};
+    mask_spec ms = {0, NULL, NULL, 0, 0, 0, 0, bias, bsb, bsh, bsq, bsk, 0.f, 0};
     return sdpa_fwd_impl(Q, K, V, B, H, Sq, Sk, D, scale, ms, 0, B * H, 0, Sq, O, LSE, O32);
 }
 
@@ -224,7 +251,7 @@ static int sdpa_fwd_impl(const uint16_t* Q, const uint16_t* K, const uint16_t* V
                 for (int d = 0; d < D; ++d) o[d] = 0.f;
                 const float* row = P + (size_t)i * Sk;
                 for (int j = 0; j < Sk; ++j) {
-                    const float p = row[j];
+                    const float p = row[j] * drop_factor(&ms, bh, row_begin + i, j, Sq, Sk);
                     if (p == 0.f) continue;
                     const float* vr = v + (size_t)j * D;
                     for (int d = 0; d < D; ++d) o[d] += p * vr[d];
@@ -251,18 +278,15 @@ static int sdpa_fwd_impl(const uint16_t* Q, const uint16_t* K, const uint16_t* V
  * [0, Sq), and also for every key that no query outside the band attends to, e.g. the last keys
  * of a causal problem when the band is the last rows).
  */
-int oracle_sdpa_bwd_rows(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
+static int sdpa_bwd_impl(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
                          const uint16_t* O, const uint16_t* dO,
-                         int B, int H, int Sq, int Sk, int D, float scale, int causal,
-                         const int32_t* kv_len, const uint8_t* mask,
-                         int64_t msb, int64_t msh, int64_t msq, int64_t msk,
+                         int B, int H, int Sq, int Sk, int D, float scale, mask_spec ms,
                          int heads_begin, int heads_end, int row_begin, int row_end,
                          uint16_t* dQ, uint16_t* dK, uint16_t* dV,
                          float* dQ32, float* dK32, float* dV32) {
     if (check_dims(B, H, Sq, Sk, D)) return -1;
     if (row_begin < 0 || row_end > Sq || row_begin > row_end) return -1;
     const int R = row_end - row_begin;
-    mask_spec ms = {causal, kv_len, mask, msb, msh, msq, msk, NULL, 0, 0, 0, 0};
     int fail = 0;
 #pragma omp parallel for schedule(dynamic, 1)
     for (int bh = heads_begin; bh < heads_end; ++bh) {
@@ -312,12 +336,16 @@ int oracle_sdpa_bwd_rows(const uint16_t* Q, const uint16_t* K, const uint16_t* V
                 for (int j = 0; j < Sk; ++j) {
                     const float p = row[j];
                     if (p == 0.f) continue;
-                    const float ds = p * (dp[j] - delta);
+                    /* with dropout O = (P * f) V, f = 0 or 1 / (1 - p): dV takes P * f, dP = f * (dO V^T), and
+                     * rowsum(dP * P) = rowsum(dO * O) = delta as without it */
+                    const float f = drop_factor(&ms, bh, row_begin + i, j, Sq, Sk);
+                    const float ds = p * (f * dp[j] - delta);
+                    const float pd = p * f;
                     float* dvj = dv + (size_t)j * D;
                     float* dkj = dk + (size_t)j * D;
                     const float* kj = k + (size_t)j * D;
                     for (int d = 0; d < D; ++d) {
-                        dvj[d] += p * gi[d];
+                        dvj[d] += pd * gi[d];
                         dqi[d] += ds * kj[d];
                         dkj[d] += ds * qi[d];
                     }
@@ -341,6 +369,37 @@ int oracle_sdpa_bwd_rows(const uint16_t* Q, const uint16_t* K, const uint16_t* V
         free(dq); free(dk); free(dv);
     }
     return fail ? -2 : 0;
+}
+
+int oracle_sdpa_bwd_rows(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
+                         const uint16_t* O, const uint16_t* dO,
+                         int B, int H, int Sq, int Sk, int D, float scale, int causal,
+                         const int32_t* kv_len, const uint8_t* mask,
+                         int64_t msb, int64_t msh, int64_t msq, int64_t msk,
+                         int heads_begin, int heads_end, int row_begin, int row_end,
+                         uint16_t* dQ, uint16_t* dK, uint16_t* dV,
+                         float* dQ32, float* dK32, float* dV32) {
+    mask_spec ms = {causal, kv_len, mask, msb, msh, msq, msk, NULL, 0, 0, 0, 0, 0.f, 0};
+    return sdpa_bwd_impl(Q, K, V, O, dO, B, H, Sq, Sk, D, scale, ms, heads_begin, heads_end, row_begin, row_end,
+                         dQ, dK, dV, dQ32, dK32, dV32);
+}
+
+/* Forward and backward with dropout of the probabilities (see drop_factor); causal flag and key lengths as the
+ * only exclusions. */
+int oracle_sdpa_fwd_dropout(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
+                            int B, int H, int Sq, int Sk, int D, float scale, int causal, const int32_t* kv_len,
+                            float drop_p, uint64_t drop_seed, uint16_t* O, float* LSE, float* O32) {
+    mask_spec ms = {causal, kv_len, NULL, 0, 0, 0, 0, NULL, 0, 0, 0, 0, drop_p, drop_seed};
+    return sdpa_fwd_impl(Q, K, V, B, H, Sq, Sk, D, scale, ms, 0, B * H, 0, Sq, O, LSE, O32);
+}
+
+int oracle_sdpa_bwd_dropout(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
+                            const uint16_t* O, const uint16_t* dO,
+                            int B, int H, int Sq, int Sk, int D, float scale, int causal, const int32_t* kv_len,
+                            float drop_p, uint64_t drop_seed,
+                            uint16_t* dQ, uint16_t* dK, uint16_t* dV, float* dQ32, float* dK32, float* dV32) {
+    mask_spec ms = {causal, kv_len, NULL, 0, 0, 0, 0, NULL, 0, 0, 0, 0, drop_p, drop_seed};
+    return sdpa_bwd_impl(Q, K, V, O, dO, B, H, Sq, Sk, D, scale, ms, 0, B * H, 0, Sq, dQ, dK, dV, dQ32, dK32, dV32);
 }
 
 int oracle_sdpa_bwd(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
