@@ -85,7 +85,9 @@ __device__ __forceinline__ void dkdv_store(const BwdParams& p, const f32x16 (&dk
 // 1 KiB copies per wavefront) and every lane reads the bytes of its key a few elements ahead of use,
 // instead of fetching 32 bytes from global memory into 32 registers at the start of every step; with the
 // registers back, the walk runs the same straight-line steps as the unmasked one.
-template <int D, bool HASMASK, bool TIMING, bool VECMASK = false>
+// DROPOUT: dV takes the dropped and rescaled probabilities, dP = f (dO V^T) with the same factor f (drop_factor), and
+// -delta is added per element instead of seeding the dP accumulators.
+template <int D, bool HASMASK, bool TIMING, bool VECMASK = false, bool DROPOUT = false>
 __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
     static_assert(!VECMASK || HASMASK, "VECMASK is a special case of HASMASK");
     using T = BwdTile<D>;
@@ -350,7 +352,7 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
     auto ndelta_rows = [&](const float* rows, int qb, int g4) {
         const f32x4 v = *reinterpret_cast<const f32x4*>(rows + BM + 32 * qb + 8 * g4 + 4 * h);
 #pragma unroll
-        for (int t = 0; t < 4; ++t) dpacc[qb][4 * g4 + t] = v[t];
+        for (int t = 0; t < 4; ++t) dpacc[qb][4 * g4 + t] = DROPOUT ? 0.f : v[t];
     };
 
     // this workgroup's slice [it_lo, it_hi) of the walk
@@ -412,8 +414,10 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
         const uint8_t* mask_c = mask0 + cur * T::MASK_STAGE_BYTES + (4 * h) * BN + 32 * wave + n;
         const uint8_t* nm_base = VECMASK ? mask_tile(qt_next) : nullptr;
         uint32_t m4[4], m4n[4];
+        f32x4 nd4, nd4n;                 // DROPOUT: -delta of the same four queries
         auto rows_ahead = [&](int qb, int g) {
             l4n = *reinterpret_cast<const f32x4*>(rows_c + 32 * qb + 8 * g + 4 * h);
+            if (DROPOUT) nd4n = *reinterpret_cast<const f32x4*>(rows_c + BM + 32 * qb + 8 * g + 4 * h);
             if (VECMASK) {
 #pragma unroll
                 for (int t = 0; t < 4; ++t) m4n[t] = mask_c[(32 * qb + 8 * g + t) * BN];
@@ -424,7 +428,7 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
         // The product for element r is issued with the exponential of element r + 1, so that no
         // instruction waits on the transcendental unit.
         auto ds_mul = [&](int qb, int r) {
-            dpacc[qb][r] = sacc[qb][r] * dpacc[qb][r];
+            if (!DROPOUT) dpacc[qb][r] = sacc[qb][r] * dpacc[qb][r];       // DROPOUT: elem() has formed dS already
             if ((r & 7) == 7) {
                 const int c = r >> 3, o8 = 8 * c;
                 const f32x16& d = dpacc[qb];
@@ -435,6 +439,7 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
             const int g = r >> 2, t = r & 3;
             if (t == 0) {
                 l4 = l4n;
+                if (DROPOUT) nd4 = nd4n;
                 if (VECMASK) {
 #pragma unroll
                     for (int u = 0; u < 4; ++u) m4[u] = m4n[u];
@@ -455,6 +460,12 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
                     if (HASMASK) drop |= mk[qb][r] == 0;
                 }
                 pr = drop ? 0.f : pr;
+            }
+            if constexpr (DROPOUT) {
+                const uint32_t qi = (uint32_t)(q0 + 32 * qb + 8 * g + 4 * h + t);
+                const float f = drop_factor(p.m, ((uint32_t)bh * (uint32_t)p.Sq + qi) * (uint32_t)p.Sk + (uint32_t)key);
+                dpacc[qb][r] = pr * fmaf(f, dpacc[qb][r], nd4[t]);       // dS = P (f dP - delta)
+                pr *= f;                                                  // what multiplied V in the forward
             }
             sacc[qb][r] = pr;
             if ((r & 7) == 7) {
@@ -750,7 +761,7 @@ struct BwdDqTile {
 // that fill 256-query workgroups go to bwd_dq_wide_kernel below).
 // VECMASK (with HASMASK): the keep-mask rows are contiguous and 16-byte aligned and Sk is a multiple of the
 // tile, so the per-element mask loads are not compiled in and the kernel fits two workgroups per unit again.
-template <int D, bool HASMASK, int NW, bool VECMASK = false>
+template <int D, bool HASMASK, int NW, bool VECMASK = false, bool DROPOUT = false>
 __global__ __launch_bounds__(64 * NW, (NW == 4 && (!HASMASK || VECMASK)) ? 2 : 1) void bwd_dq_kernel(const BwdParams p) {
     static_assert(!VECMASK || HASMASK, "VECMASK is a special case of HASMASK");
     using T = BwdDqTile<D>;
@@ -960,7 +971,14 @@ __global__ __launch_bounds__(64 * NW, (NW == 4 && (!HASMASK || VECMASK)) ? 2 : 1
             sacc[kb][r] = pr;
         };
         auto ds_elem = [&](int kb, int r) {         // dS^T = P^T (dP^T - delta), packed after 8 and 16
-            dpacc[kb][r] = sacc[kb][r] * (dpacc[kb][r] - delta);
+            if constexpr (DROPOUT) {
+                // O = (P f) V with f = 0 or 1 / (1 - p): dP = f (dO V^T), and rowsum(dP P) is still rowsum(dO O)
+                const uint32_t key = (uint32_t)(key0 + 32 * kb + acc_row(r, h));
+                const uint32_t row = ((uint32_t)bh * (uint32_t)p.Sq + (uint32_t)qrow) * (uint32_t)p.Sk;
+                dpacc[kb][r] = sacc[kb][r] * fmaf(drop_factor(p.m, row + key), dpacc[kb][r], -delta);
+            } else {
+                dpacc[kb][r] = sacc[kb][r] * (dpacc[kb][r] - delta);
+            }
             if ((r & 7) == 7) {
                 const int o8 = r - 7;
                 const f32x16& d = dpacc[kb];

@@ -418,7 +418,23 @@ struct MaskArgs {
     int64_t bb = 0, bh = 0, bq = 0, bk = 0;   // element strides over (b,h,q,k); 0 broadcasts
     int bias_f32 = 1;
     float inv_scale = 1.f;   // 1 / softmax scale: the bias is folded into the raw scores as bias / scale
+    // dropout of the probabilities (kernels instantiated with DROPOUT only): see drop_factor
+    uint32_t drop_seed = 0;  // low 32 bits of the seed
+    uint32_t drop_thr = 0;   // ceil(p * 2^24): an element is kept when its 24-bit uniform is >= this
+    float drop_scale = 1.f;  // 1 / (1 - p)
 };
+
+// Factor that dropout applies to the probability of flat element index idx of the [B*H, Sq, Sk] probability tensor
+// (low 32 bits): 0 or 1 / (1 - p).  The uniform is the reference's (src/rng/mod.rs:14-24, drawn over the whole
+// tensor by src/autograd_v4/ops/sdpa.rs:229-231, :604-649): u = (xorshift32(seed ^ idx) >> 8) / 2^24, kept when
+// u >= p, which in integers is (xorshift32(seed ^ idx) >> 8) >= ceil(p * 2^24).
+__device__ __forceinline__ float drop_factor(const MaskArgs& m, uint32_t idx) {
+    uint32_t s = m.drop_seed ^ idx;
+    s ^= s << 13;
+    s ^= s >> 17;
+    s ^= s << 5;
+    return (s >> 8) >= m.drop_thr ? m.drop_scale : 0.f;
+}
 
 // one element of an explicit mask, addressed in elements from the (batch, head) base: does it attend?
 __device__ __forceinline__ bool mask_attends(const MaskArgs& m, const uint8_t* base, int64_t elem) {

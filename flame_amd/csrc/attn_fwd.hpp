@@ -54,7 +54,9 @@ struct FwdTile {
 // whose rows are contiguous and 16-byte aligned, Sk is a multiple of the tile and there is no bias; the
 // general exclusion code (per-element loads, bias) is then not compiled in, which frees the registers
 // that made the general masked kernel spill.
-template <int D, bool HASMASK, int NW, bool VECMASK = false>
+// DROPOUT: the probabilities that multiply V are dropped and rescaled element by element (drop_factor); the row sums,
+// and with them the log-sum-exp, stay those of the undropped softmax.
+template <int D, bool HASMASK, int NW, bool VECMASK = false, bool DROPOUT = false>
 __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void fwd_kernel(const FwdParams p) {
     static_assert(!VECMASK || HASMASK, "VECMASK is a special case of HASMASK");
     using T = FwdTile<D>;
@@ -190,6 +192,9 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void fwd_kernel(const Fwd
     constexpr int NP = 4 * DB;     // PV MFMAs per tile
     constexpr int EPS = 32 / NS;   // logits handled per softmax slice
 
+    // flat index (mod 2^32) of this lane's query row in the [B*H, Sq, Sk] probability tensor
+    const uint32_t drop_row = ((uint32_t)bh * (uint32_t)p.Sq + (uint32_t)(qw0 + n)) * (uint32_t)p.Sk;
+    (void)drop_row;
     // exclusions of tile t: ragged tail / key length, causal, explicit keep-mask
     auto apply_mask = [&](f32x16 (&s)[2], int t) {
         const int qi = qw0 + n;
@@ -283,9 +288,14 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void fwd_kernel(const Fwd
             for (int e = 0; e < EPS; ++e) {
                 const int idx = EPS * j + e, kb = idx >> 4, r = idx & 15;
                 const float v = exp2_fast(fmaf(cur[kb][r], c_log2, -msc));
-                cur[kb][r] = v;
                 if (e & 1) rsum1 += v;
                 else rsum0 += v;
+                if constexpr (DROPOUT) {
+                    const uint32_t key = (uint32_t)(t * BN + 32 * kb + acc_row(r, h));
+                    cur[kb][r] = v * drop_factor(p.m, drop_row + key);
+                } else {
+                    cur[kb][r] = v;
+                }
                 if ((idx & 7) == 7) {
                     const int o8 = r - 7;
                     const f32x16& s = cur[kb];

@@ -257,6 +257,70 @@ int launch_bwd(const BwdParams& p, hipStream_t s) {
     return e == hipSuccess ? FLAME_ATTN_OK : (int)e;
 }
 
+// Dropout of the probabilities: the 128-query forward and dQ kernels and the dK/dV kernel in their DROPOUT
+// instantiations, without the split of the last round.  No explicit mask or bias.
+template <int D>
+int launch_fwd_dropout(const FwdParams& p, hipStream_t s) {
+    using T = FwdTile<D>;
+    static bool attr_done = false;
+    auto kern = fwd_kernel<D, false, 4, false, true>;
+    if (!attr_done) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS_BYTES);
+        if (e != hipSuccess) return (int)e;
+        attr_done = true;
+    }
+    const int64_t grid = (int64_t)((p.Sq + 127) / 128) * p.B * p.H;
+    if (grid > 0x7fffffff) return FLAME_ATTN_ERR_UNSUPPORTED;
+    {
+        ScopedKernelTimer t(FLAME_ATTN_KERNEL_FWD, s);
+        hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), T::LDS_BYTES, s, p);
+    }
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? FLAME_ATTN_OK : (int)e;
+}
+
+template <int D>
+int launch_bwd_dropout(const BwdParams& p, hipStream_t s) {
+    using T = BwdTile<D>;
+    using TQ = BwdDqTile<D>;
+    static bool attr_done = false;
+    auto kern = bwd_dkdv_kernel<D, false, false, false, true>;
+    auto kern_dq = bwd_dq_kernel<D, false, 4, false, true>;
+    if (!attr_done) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS_BYTES);
+        if (e != hipSuccess) return (int)e;
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern_dq),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, TQ::LDS_BYTES);
+        if (e != hipSuccess) return (int)e;
+        attr_done = true;
+    }
+    const int64_t grid = (int64_t)((p.Sk + T::BN - 1) / T::BN) * p.B * p.H;
+    const int64_t grid_dq = (int64_t)((p.Sq + TQ::BM - 1) / TQ::BM) * p.B * p.H;
+    if (grid > 0x7fffffff || grid_dq > 0x7fffffff) return FLAME_ATTN_ERR_UNSUPPORTED;
+    {
+        ScopedKernelTimer t(FLAME_ATTN_KERNEL_BWD_DQ, s);        // first: it leaves -delta and the rescaled LSE rows
+        hipLaunchKernelGGL(kern_dq, dim3((unsigned)grid_dq), dim3(256), TQ::LDS_BYTES, s, p);
+    }
+    {
+        ScopedKernelTimer t(FLAME_ATTN_KERNEL_BWD_DKDV, s);
+        hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), T::LDS_BYTES, s, p);
+    }
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? FLAME_ATTN_OK : (int)e;
+}
+
+// 0 <= p < 1 (src/autograd_v4/ops/sdpa.rs:110-116); fills the kernel-side description of the draw
+bool set_dropout(MaskArgs& m, float dropout_p, uint64_t dropout_seed) {
+    if (!(dropout_p >= 0.f) || !(dropout_p < 1.f)) return false;
+    m.drop_seed = (uint32_t)dropout_seed;
+    m.drop_thr = (uint32_t)ceil((double)dropout_p * 16777216.0);      // u >= p  <=>  24-bit integer >= ceil(p * 2^24)
+    const float keep = 1.0f - dropout_p;
+    m.drop_scale = 1.0f / keep;
+    return true;
+}
+
 }  // namespace
 
 extern "C" {
@@ -302,7 +366,7 @@ size_t flame_attn_bwd_workspace_bytes(int B, int H, int N_q, int D) {
     return bwd_rows_bytes(B, H, N_q) + (size_t)device_cu_count() * bwd_split_slot_bytes(padded_head_dim(D));
 }
 
-int flame_attn_bwd_bf16(const void* Q, const void* K, const void* V, const void* O, const void* dO,
+static int attn_bwd_impl(const void* Q, const void* K, const void* V, const void* O, const void* dO,
                         const void* LSE, void* dQ, void* dK, void* dV,
                         int B, int H, int N_q, int N_kv, int D, float scale,
                         const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
@@ -312,7 +376,7 @@ int flame_attn_bwd_bf16(const void* Q, const void* K, const void* V, const void*
                         int64_t lse_off, int64_t dq_off, int64_t dk_off, int64_t dv_off,
                         int causal, const int32_t* kv_len,
                         const uint8_t* keep_mask, const int64_t* mask_strides,
-                        void* workspace, size_t workspace_bytes, void* stream) {
+                        void* workspace, size_t workspace_bytes, void* stream, float dropout_p, uint64_t dropout_seed) {
     if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0) return FLAME_ATTN_ERR_INVALID;
     if (!(scale > 0.f) || !isfinite(scale)) return FLAME_ATTN_ERR_INVALID;
     if (!LSE || !workspace) return FLAME_ATTN_ERR_INVALID;
@@ -365,8 +429,45 @@ int flame_attn_bwd_bf16(const void* Q, const void* K, const void* V, const void*
     p.phase_cycles = g_phase_cycles;
     if (D == 128 && !keep_mask && g_phase_cycles) return launch_bwd<128, false, true>(p, s);   // phase-timing build
 #endif
+    if (dropout_p != 0.f) {
+        if (!set_dropout(p.m, dropout_p, dropout_seed)) return FLAME_ATTN_ERR_INVALID;
+        if (keep_mask) return FLAME_ATTN_ERR_UNSUPPORTED;
+        return padded_head_dim(D) == 128 ? launch_bwd_dropout<128>(p, s) : launch_bwd_dropout<64>(p, s);
+    }
     if (padded_head_dim(D) == 128) return keep_mask ? launch_bwd<128, true>(p, s) : launch_bwd<128, false>(p, s);
     return keep_mask ? launch_bwd<64, true>(p, s) : launch_bwd<64, false>(p, s);
+}
+
+int flame_attn_bwd_bf16(const void* Q, const void* K, const void* V, const void* O, const void* dO,
+                        const void* LSE, void* dQ, void* dK, void* dV,
+                        int B, int H, int N_q, int N_kv, int D, float scale,
+                        const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                        const int64_t* o_strides, const int64_t* do_strides, const int64_t* dq_strides,
+                        const int64_t* dk_strides, const int64_t* dv_strides,
+                        int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off, int64_t do_off,
+                        int64_t lse_off, int64_t dq_off, int64_t dk_off, int64_t dv_off,
+                        int causal, const int32_t* kv_len,
+                        const uint8_t* keep_mask, const int64_t* mask_strides,
+                        void* workspace, size_t workspace_bytes, void* stream) {
+    return attn_bwd_impl(Q, K, V, O, dO, LSE, dQ, dK, dV, B, H, N_q, N_kv, D, scale, q_strides, k_strides, v_strides, o_strides,
+                         do_strides, dq_strides, dk_strides, dv_strides, q_off, k_off, v_off, o_off, do_off, lse_off, dq_off,
+                         dk_off, dv_off, causal, kv_len, keep_mask, mask_strides, workspace, workspace_bytes, stream, 0.f, 0);
+}
+
+int flame_attn_bwd_dropout_bf16(const void* Q, const void* K, const void* V, const void* O, const void* dO,
+                                const void* LSE, void* dQ, void* dK, void* dV,
+                                int B, int H, int N_q, int N_kv, int D, float scale,
+                                const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                                const int64_t* o_strides, const int64_t* do_strides, const int64_t* dq_strides,
+                                const int64_t* dk_strides, const int64_t* dv_strides,
+                                int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off, int64_t do_off,
+                                int64_t lse_off, int64_t dq_off, int64_t dk_off, int64_t dv_off,
+                                int causal, const int32_t* kv_len, float dropout_p, uint64_t dropout_seed,
+                                void* workspace, size_t workspace_bytes, void* stream) {
+    return attn_bwd_impl(Q, K, V, O, dO, LSE, dQ, dK, dV, B, H, N_q, N_kv, D, scale, q_strides, k_strides, v_strides, o_strides,
+                         do_strides, dq_strides, dk_strides, dv_strides, q_off, k_off, v_off, o_off, do_off, lse_off, dq_off,
+                         dk_off, dv_off, causal, kv_len, nullptr, nullptr, workspace, workspace_bytes, stream, dropout_p,
+                         dropout_seed);
 }
 
 int flame_sage_quant_qk_int8(const void* Q, const void* K, int B, int H, int N_q, int N_kv, int D,
@@ -557,7 +658,8 @@ static int attn_fwd_impl(const void* Q, const void* K, const void* V, void* O, v
                         int causal, const int32_t* kv_len,
                         const uint8_t* keep_mask, const int64_t* mask_strides,
                         const void* bias, int bias_dtype, const int64_t* bias_strides,
-                        void* stream, int mask_mode = kMaskU8, int Dv = 0, int q_tile_plan = 0) {
+                        void* stream, int mask_mode = kMaskU8, int Dv = 0, int q_tile_plan = 0, float dropout_p = 0.f,
+                        uint64_t dropout_seed = 0) {
     if (Dv == 0) Dv = D;           // V and O may have a head dim of their own (forward only)
     if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0 || Dv < 0) return FLAME_ATTN_ERR_INVALID;
     if (!(scale > 0.f) || !isfinite(scale)) return FLAME_ATTN_ERR_INVALID;
@@ -601,6 +703,11 @@ static int attn_fwd_impl(const void* Q, const void* K, const void* V, void* O, v
 
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bool hm = keep_mask != nullptr || bias != nullptr;
+    if (dropout_p != 0.f) {
+        if (!set_dropout(p.m, dropout_p, dropout_seed)) return FLAME_ATTN_ERR_INVALID;
+        if (hm) return FLAME_ATTN_ERR_UNSUPPORTED;
+        return std::max(padded_head_dim(D), padded_head_dim(Dv)) == 128 ? launch_fwd_dropout<128>(p, s) : launch_fwd_dropout<64>(p, s);
+    }
     // 256-query workgroups when they neither add padding rows nor leave compute units
     // without a workgroup
     bool wide = fwd_rule_wide(B, H, N_q, hm, kv_len != nullptr);
@@ -634,6 +741,17 @@ int flame_attn_fwd_bf16(const void* Q, const void* K, const void* V, void* O, vo
     return attn_fwd_impl(Q, K, V, O, LSE, B, H, N_q, N_kv, D, scale, q_strides, k_strides, v_strides, o_strides,
                          q_off, k_off, v_off, o_off, lse_off, causal, kv_len, keep_mask, mask_strides,
                          nullptr, FLAME_ATTN_DTYPE_F32, nullptr, stream);
+}
+
+int flame_attn_fwd_dropout_bf16(const void* Q, const void* K, const void* V, void* O, void* LSE,
+                                int B, int H, int N_q, int N_kv, int D, float scale,
+                                const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                                const int64_t* o_strides,
+                                int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off, int64_t lse_off,
+                                int causal, const int32_t* kv_len, float dropout_p, uint64_t dropout_seed, void* stream) {
+    return attn_fwd_impl(Q, K, V, O, LSE, B, H, N_q, N_kv, D, scale, q_strides, k_strides, v_strides, o_strides,
+                         q_off, k_off, v_off, o_off, lse_off, causal, kv_len, nullptr, nullptr,
+                         nullptr, FLAME_ATTN_DTYPE_F32, nullptr, stream, kMaskU8, 0, 0, dropout_p, dropout_seed);
 }
 
 int flame_attn_fwd_bias_bf16(const void* Q, const void* K, const void* V, void* O, void* LSE,

@@ -217,7 +217,7 @@ struct FwdOut {
 };
 
 inline Result<FwdOut> run_forward(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor* mask, bool causal,
-                                  std::optional<float> scale, bool want_stats) {
+                                  std::optional<float> scale, bool want_stats, float dropout_p = 0.f, uint64_t dropout_seed = 0) {
     auto dv = validate(q, k, v, mask);
     if (!dv.ok()) return dv.error();
     const Dims d = dv.value();
@@ -240,6 +240,16 @@ inline Result<FwdOut> run_forward(const Tensor& q, const Tensor& k, const Tensor
         mst = pm.value().second;
     }
     const float sc = scale.value_or(1.0f / std::sqrt((float)d.D));
+    if (dropout_p != 0.f) {
+        if (mask) return unsupported("dropout together with a mask is not built");
+        const int rc = flame_attn_fwd_dropout_bf16(q.base(), k.base(), v.base(), o.value().base(), want_stats ? stats.base() : nullptr,
+                                                   d.B, d.H, d.Sq, d.Sk, d.D, sc, q.strides().data(), k.strides().data(),
+                                                   v.strides().data(), o.value().strides().data(), q.offset(), k.offset(),
+                                                   v.offset(), 0, 0, causal ? 1 : 0, nullptr, dropout_p, dropout_seed, nullptr);
+        if (rc == FLAME_ATTN_ERR_UNSUPPORTED) return unsupported("flame_attn_fwd_dropout_bf16: head dim or layout not built");
+        if (rc != 0) return cuda_error("flame_attn_fwd_dropout_bf16", rc);
+        return FwdOut{o.value(), stats};
+    }
     const int rc = flame_attn_fwd_bf16(q.base(), k.base(), v.base(), o.value().base(), want_stats ? stats.base() : nullptr,
                                        d.B, d.H, d.Sq, d.Sk, d.D, sc, q.strides().data(), k.strides().data(),
                                        v.strides().data(), o.value().strides().data(), q.offset(), k.offset(), v.offset(), 0, 0,
@@ -262,6 +272,8 @@ struct FlashAttentionNode {
     std::optional<Tensor> mask;
     float scale = 0.f;
     bool causal = false;
+    float dropout_p = 0.f;            // set by the v4 operator only (autograd_v4::SdpaCtx)
+    uint64_t dropout_seed = 0;
 };
 
 class AutogradContext {
@@ -337,6 +349,19 @@ inline Result<AttentionGrads> flash_attention_backward(const FlashAttentionNode&
         if (!pm.ok()) return pm.error();
         m8 = pm.value().first;
         mst = pm.value().second;
+    }
+    if (n.dropout_p != 0.f) {
+        if (n.mask) return unsupported("dropout together with a mask is not built");
+        const int rc = flame_attn_bwd_dropout_bf16(
+            n.query.base(), n.key.base(), n.value.base(), n.output.base(), g.base(), n.stats.base(), dq.value().base(),
+            dk.value().base(), dv.value().base(), B, H, Sq, Sk, D, n.scale, n.query.strides().data(), n.key.strides().data(),
+            n.value.strides().data(), n.output.strides().data(), g.strides().data(), dq.value().strides().data(),
+            dk.value().strides().data(), dv.value().strides().data(), n.query.offset(), n.key.offset(), n.value.offset(),
+            n.output.offset(), g.offset(), 0, 0, 0, 0, n.causal ? 1 : 0, nullptr, n.dropout_p, n.dropout_seed, ws.value().data(),
+            wsb, nullptr);
+        if (rc == FLAME_ATTN_ERR_UNSUPPORTED) return unsupported("flame_attn_bwd_dropout_bf16: head dim or layout not built");
+        if (rc != 0) return cuda_error("flame_attn_bwd_dropout_bf16", rc);
+        return AttentionGrads{dq.value(), dk.value(), dv.value()};
     }
     const int rc = flame_attn_bwd_bf16(
         n.query.base(), n.key.base(), n.value.base(), n.output.base(), g.base(), n.stats.base(), dq.value().base(),
@@ -545,6 +570,8 @@ struct SdpaCtx {                          // :80-96
     Tensor lse;                           // fp32 [B*H, Q]
     std::tuple<size_t, size_t, size_t, size_t> shapes;   // (B,H,Q,K)
     SdpaStats stats;
+    float dropout_p = 0.f;                // :94-95
+    std::optional<uint64_t> dropout_seed;
 };
 
 // ---- tape of the v4 engine (src/autograd_v4/graph.rs:12-94): nodes keyed by the output tensor's id,
@@ -629,11 +656,48 @@ class Gradients {
     std::unordered_map<uint64_t, std::string> names_;
 };
 
+// Seeds for calls that give none (the reference draws them from its global generator, src/rng/mod.rs:60-70 and
+// src/autograd_v4/ops/sdpa.rs:120-124; deterministic after set_seed, though not the same stream as Rust's StdRng).
+namespace rng {
+inline std::mutex& guard() {
+    static std::mutex m;
+    return m;
+}
+inline uint64_t& state() {
+    static uint64_t s = 0;
+    return s;
+}
+inline void set_seed(uint64_t seed) {
+    std::lock_guard<std::mutex> g(guard());
+    state() = seed;
+}
+inline uint64_t next_u64() {          // SplitMix64
+    std::lock_guard<std::mutex> g(guard());
+    uint64_t z = (state() += 0x9E3779B97F4A7C15ull);
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+}
+}  // namespace rng
+
 // sdpa_forward(q,k,v,mask,&cfg) -> (output, ctx) (:98-326).  SaveProbs would materialise the
-// [B,H,Q,K] matrix and dropout is not built: both are refused rather than emulated.
+// [B,H,Q,K] matrix and is refused rather than emulated.  Dropout (:110-124, :229-231) runs inside the fused
+// kernels with the kept set the reference draws for the same seed when it does not chunk; a chunked draw
+// (chunk_q / chunk_kv smaller than the lengths) re-seeds per chunk (:600-602) and is not built, nor is dropout
+// together with a mask.
 inline Result<std::pair<Tensor, SdpaCtx>> sdpa_forward(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor* mask,
                                                        const SdpaConfig& cfg) {
-    if (cfg.dropout_p != 0.f) return unsupported("dropout is not built into the fused kernels");
+    if (cfg.dropout_p < 0.f || cfg.dropout_p >= 1.f || cfg.dropout_p != cfg.dropout_p)
+        return invalid("sdpa_forward: dropout_p=" + std::to_string(cfg.dropout_p) + " is out of range [0, 1)");
+    std::optional<uint64_t> dropout_seed;
+    if (cfg.dropout_p > 0.f) {
+        if (q.shape().size() == 4 && k.shape().size() == 4 &&
+            ((cfg.chunk_q && *cfg.chunk_q > 0 && (int64_t)*cfg.chunk_q < q.shape()[2]) ||
+             (cfg.chunk_kv && *cfg.chunk_kv > 0 && (int64_t)*cfg.chunk_kv < k.shape()[2])))
+            return unsupported("dropout with a chunked draw is not built: leave chunk_q / chunk_kv unset");
+        if (cfg.save == SdpaSave::Recompute) return unsupported("dropout with SdpaSave::Recompute is not built");
+        dropout_seed = cfg.dropout_seed ? *cfg.dropout_seed : rng::next_u64();
+    }
     if (cfg.save == SdpaSave::SaveProbs) return unsupported("SaveProbs materialises [B,H,Q,K]; use SaveLSE");
     const SdpaHooks* hooks = debug_hooks();
     std::unique_ptr<StreamTimer> timer;
@@ -645,9 +709,11 @@ inline Result<std::pair<Tensor, SdpaCtx>> sdpa_forward(const Tensor& q, const Te
     // SaveLSE keeps O and the log-sum-exp for the backward; Recompute (:21-47) keeps neither and the backward
     // runs the forward once more to get them back (the outputs are deterministic, so it sees the same O).
     const bool keep = cfg.save != SdpaSave::Recompute;
-    auto r = detail::run_forward(q, k, v, mask, cfg.causal, cfg.scale, keep);
+    auto r = detail::run_forward(q, k, v, mask, cfg.causal, cfg.scale, keep, cfg.dropout_p, dropout_seed.value_or(0));
     if (!r.ok()) return r.error();
     SdpaCtx ctx;
+    ctx.dropout_p = cfg.dropout_p;
+    ctx.dropout_seed = dropout_seed;
     ctx.q = q; ctx.k = k; ctx.v = v;
     if (keep) ctx.o = r.value().o;
     if (mask) ctx.attn_mask = *mask;
@@ -685,6 +751,9 @@ inline Result<std::tuple<Tensor, Tensor, Tensor>> sdpa_backward(const SdpaCtx& c
     n.mask = ctx.attn_mask;
     n.scale = ctx.scale;
     n.causal = ctx.causal;
+    n.dropout_p = ctx.dropout_p;
+    n.dropout_seed = ctx.dropout_seed.value_or(0);
+    if (ctx.dropout_p > 0.f && !ctx.dropout_seed) return Error{Error::InvalidInput, "dropout seed required when dropout_p > 0"};
     if (ctx.save == SdpaSave::Recompute) {          // nothing was kept: O and the log-sum-exp come from one more forward
         auto f = detail::run_forward(ctx.q, ctx.k, ctx.v, ctx.attn_mask ? &*ctx.attn_mask : nullptr, ctx.causal, ctx.scale, true);
         if (!f.ok()) return f.error();

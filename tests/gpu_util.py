@@ -28,8 +28,9 @@ def bf16_ulp(x: np.ndarray) -> np.ndarray:
     return 2.0 ** (np.floor(np.log2(ax)) - 7)
 
 
-def assert_close_bf16(oracle, name, got_f32, ref_bits, ref_f32):
-    """The parity bar for a bf16 output tensor.
+def assert_close_bf16(oracle, name, got_f32, ref_bits, ref_f32, max_abs=TOL_MAX_ABS):
+    """The parity bar for a bf16 output tensor (max_abs: the flat bound, the north-star 2e-2 unless a test states why
+    its quantities are scaled).
 
     * relative L2 <= 1e-2 against the oracle's un-rounded fp32 values;
     * max-abs <= 2e-2 against both the un-rounded fp32 values and the oracle's bf16-rounded values,
@@ -44,12 +45,12 @@ def assert_close_bf16(oracle, name, got_f32, ref_bits, ref_f32):
     ma_b = float(diff_b.max()) if diff_b.size else 0.0
     diff_f = np.abs(got_f32.astype(np.float64) - ref_f.astype(np.float64))
     # elements that pass only through the one-ulp allowance (their error exceeds the flat 2e-2)
-    n_ulp = int(np.count_nonzero((diff_f > TOL_MAX_ABS) | (diff_b > TOL_MAX_ABS)))
+    n_ulp = int(np.count_nonzero((diff_f > max_abs) | (diff_b > max_abs)))
     print(f"      {name}: vs fp32 oracle max_abs={ma_f:.3e} rel_l2={rl_f:.3e}; vs bf16 oracle max_abs={ma_b:.3e} "
           f"(|ref|max={np.abs(ref_f).max():.2f}; {n_ulp} of {diff_f.size} elements needed the one-ulp allowance "
           f"for |x| >= 4)", flush=True)
     assert np.all(np.isfinite(got_f32)), name
     assert rl_f <= TOL_REL_L2, name
-    assert np.all(diff_f <= np.maximum(TOL_MAX_ABS, bf16_ulp(ref_f))), name
-    assert np.all(diff_b <= np.maximum(TOL_MAX_ABS, bf16_ulp(ref_b))), name
+    assert np.all(diff_f <= np.maximum(max_abs, bf16_ulp(ref_f))), name
+    assert np.all(diff_b <= np.maximum(max_abs, bf16_ulp(ref_b))), name
     return ma_f, rl_f

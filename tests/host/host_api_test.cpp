@@ -312,9 +312,53 @@ int main() {
                           "Recompute gradients differ from SaveLSE gradients");
             }
         }
-        cfg.dropout_p = 0.1f;
-        CHECK(!autograd_v4::sdpa_forward(q, k, v, nullptr, cfg).ok(), "dropout must be refused");
-        cfg.dropout_p = 0.f;
+        // dropout: range check as the reference's (:110-116); the same seed gives the same bits, forward and backward;
+        // without a seed one is drawn from the global generator and kept in the context; a chunked draw is refused
+        {
+            autograd_v4::SdpaConfig dc = cfg;
+            dc.chunk_q.reset();
+            dc.chunk_kv.reset();
+            dc.dropout_p = 1.0f;
+            auto bad = autograd_v4::sdpa_forward(q, k, v, nullptr, dc);
+            CHECK(!bad.ok() && bad.error().kind == Error::InvalidInput, "dropout_p = 1 must be InvalidInput");
+            dc.dropout_p = -0.5f;
+            CHECK(!autograd_v4::sdpa_forward(q, k, v, nullptr, dc).ok(), "negative dropout_p must be refused");
+            dc.dropout_p = 0.25f;
+            dc.dropout_seed = 0x2545F4914F6CDD1Dull;
+            auto d1 = autograd_v4::sdpa_forward(q, k, v, nullptr, dc);
+            auto d2 = autograd_v4::sdpa_forward(q, k, v, nullptr, dc);
+            CHECK(d1.ok() && d2.ok(), "sdpa_forward with dropout failed");
+            if (d1.ok() && d2.ok() && f.ok()) {
+                CHECK(host_bits_of_bf16(d1.value().first) == host_bits_of_bf16(d2.value().first), "same seed, different output");
+                CHECK(host_bits_of_bf16(d1.value().first) != host_bits_of_bf16(f.value().first), "dropout changed nothing");
+                CHECK(d1.value().second.dropout_p == 0.25f && d1.value().second.dropout_seed == dc.dropout_seed, "context keeps p and seed");
+                std::vector<float> l1((size_t)d1.value().second.lse.numel()), l0(l1.size());
+                d1.value().second.lse.to_host(l1.data());
+                f.value().second.lse.to_host(l0.data());
+                CHECK(l1 == l0, "the log-sum-exp is that of the undropped softmax");
+                auto g1 = autograd_v4::sdpa_backward(d1.value().second, d_o);
+                auto g2 = autograd_v4::sdpa_backward(d2.value().second, d_o);
+                auto g0 = autograd_v4::sdpa_backward(f.value().second, d_o);
+                CHECK(g1.ok() && g2.ok() && g0.ok(), "sdpa_backward with dropout failed");
+                if (g1.ok() && g2.ok() && g0.ok()) {
+                    CHECK(host_bits_of_bf16(std::get<2>(g1.value())) == host_bits_of_bf16(std::get<2>(g2.value())), "same seed, different dV");
+                    CHECK(host_bits_of_bf16(std::get<2>(g1.value())) != host_bits_of_bf16(std::get<2>(g0.value())), "dropout left dV unchanged");
+                    for (float x : host_f32_of_bf16(std::get<0>(g1.value()))) if (!std::isfinite(x)) { CHECK(false, "dQ with dropout not finite"); break; }
+                }
+            }
+            dc.dropout_seed.reset();
+            autograd_v4::rng::set_seed(5);
+            auto r1 = autograd_v4::sdpa_forward(q, k, v, nullptr, dc);
+            autograd_v4::rng::set_seed(5);
+            auto r2 = autograd_v4::sdpa_forward(q, k, v, nullptr, dc);
+            CHECK(r1.ok() && r2.ok() && r1.value().second.dropout_seed.has_value() &&
+                      r1.value().second.dropout_seed == r2.value().second.dropout_seed &&
+                      host_bits_of_bf16(r1.value().first) == host_bits_of_bf16(r2.value().first),
+                  "a drawn seed is deterministic after set_seed and kept in the context");
+            dc.chunk_q = 64;
+            auto ch = autograd_v4::sdpa_forward(q, k, v, nullptr, dc);
+            CHECK(!ch.ok() && ch.error().kind == Error::Unsupported, "chunked dropout draw must be Unsupported");
+        }
         cfg.save = autograd_v4::SdpaSave::SaveProbs;
         CHECK(!autograd_v4::sdpa_forward(q, k, v, nullptr, cfg).ok(), "SaveProbs must be refused");
     }

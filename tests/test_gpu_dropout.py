@@ -1,0 +1,92 @@
+"""Dropout of the attention probabilities inside the fused kernels, through the C ABI, against the CPU oracle: the
+kept set is the reference's (one xorshift round of seed ^ flat element index, src/rng/mod.rs:14-24 drawn over the whole
+[B*H, Sq, Sk] tensor by src/autograd_v4/ops/sdpa.rs:229-231), so O, dQ, dK and dV match the oracle to the usual bar,
+and the log-sum-exp is that of the undropped softmax, bit for bit."""
+import numpy as np
+import pytest
+import torch
+
+from flame_amd import workloads as W
+from tests.gpu_util import TOL_LSE, TOL_MAX_ABS, assert_close_bf16, to_dev, to_f32
+
+pytestmark = pytest.mark.gpu
+
+SEED = 0x2545F4914F6CDD1D
+
+
+def _inputs(tag, B, H, Sq, Sk, D):
+    shapes = [(B, H, Sq, D), (B, H, Sk, D), (B, H, Sk, D), (B, H, Sq, D)]
+    return [W.f32_to_bf16_bits(W.normal_f32(tag, i, int(np.prod(s))).reshape(s)) for i, s in enumerate(shapes)]
+
+
+@pytest.mark.parametrize("B,H,Sq,Sk,D,causal,kv_len,p", [
+    (2, 3, 200, 328, 64, False, None, 0.1),
+    (2, 2, 256, 256, 128, True, None, 0.3),
+    (2, 2, 130, 77, 128, False, [77, 40], 0.5),
+    (1, 3, 192, 320, 96, True, None, 0.2),          # head dim padded inside the kernels
+    (1, 2, 1024, 1024, 128, False, None, 0.1),      # several query and key tiles per workgroup
+])
+def test_dropout_forward_and_backward_against_oracle(oracle, B, H, Sq, Sk, D, causal, kv_len, p):
+    from flame_amd import capi
+    print(f"[dropout] {B}x{H} Sq={Sq} Sk={Sk} D={D} causal={causal} kv_len={kv_len} p={p}", flush=True)
+    q, k, v, do = _inputs(950 + D + Sq, B, H, Sq, Sk, D)
+    scale = 1.0 / np.sqrt(D)
+    # One xorshift round gives neighbouring indices nearly the same uniform, so on small tensors a fixed p keeps
+    # nearly all or nearly nothing: p is placed at the quantile of this tensor's own uniforms instead, which drops
+    # that fraction of the elements whatever the seed.
+    p = float(np.quantile(oracle.dropout_uniforms(B, H, Sq, Sk, SEED), p))
+    kept = float(oracle.dropout_keep_mask(B, H, Sq, Sk, p, SEED).mean())
+    print(f"      p = {p:.6f}, kept fraction {kept:.3f}", flush=True)
+    assert 0.3 < kept < 0.95
+    kvl_np = None if kv_len is None else np.array(kv_len, np.int32)
+    kvl = None if kv_len is None else torch.tensor(kv_len, dtype=torch.int32, device="cuda")
+    dq_, dk_, dv_, ddo = (to_dev(t) for t in (q, k, v, do))
+    o, lse = capi.attn_fwd_dropout(dq_, dk_, dv_, scale, p, SEED, causal=causal, kv_len=kvl)
+    o_plain, lse_plain = capi.attn_fwd(dq_, dk_, dv_, scale, causal=causal, kv_len=kvl)
+    torch.cuda.synchronize()
+    ro, rlse, ro32 = oracle.sdpa_fwd_dropout(q, k, v, scale, p, SEED, causal=causal, kv_len=kvl_np, want_f32=True)
+    # The kept probabilities, and with them O, dP and the gradients, are 1 / (1 - p) times what they are without
+    # dropout, and so are the bf16 rounding errors of the MFMA operands: the flat bound scales with them.
+    tol = TOL_MAX_ABS / (1.0 - p)
+    assert_close_bf16(oracle, "O", to_f32(o), ro, ro32, max_abs=tol)
+    assert oracle.max_abs(lse.cpu().numpy().reshape(rlse.shape), rlse) <= TOL_LSE
+    assert torch.equal(lse, lse_plain) or float((lse - lse_plain).abs().max()) <= 1e-6      # the undropped softmax's
+    assert not torch.equal(o, o_plain)
+    g = capi.attn_bwd_dropout(dq_, dk_, dv_, o, ddo, lse, scale, p, SEED, causal=causal, kv_len=kvl)
+    torch.cuda.synchronize()
+    ref = oracle.sdpa_bwd_dropout(q, k, v, ro, do, scale, p, SEED, causal=causal, kv_len=kvl_np, want_f32=True)
+    for i, (name, got) in enumerate((("dQ", g[0]), ("dK", g[1]), ("dV", g[2]))):
+        assert_close_bf16(oracle, name, to_f32(got), ref[i], ref[i + 3], max_abs=tol)
+    # teeth: the plain forward, rescaled or not, is far from this oracle
+    assert oracle.rel_l2(to_f32(o_plain), ro32) > 0.05 and oracle.rel_l2(to_f32(o_plain) / (1 - p), ro32) > 0.05
+
+
+def test_dropout_kept_set_bit_exact_through_a_one_hot_value_matrix(oracle):
+    """V = identity over the keys (Sk = D = 128) turns O into the dropped probabilities themselves: zero exactly
+    where the reference's generator drops, non-zero elsewhere."""
+    from flame_amd import capi
+    B, H, Sq, Sk, D, p = 1, 2, 256, 128, 128, 0.4
+    q, k, _, _ = _inputs(990, B, H, Sq, Sk, D)
+    v = np.zeros((B, H, Sk, D), np.float32)
+    v[..., np.arange(Sk), np.arange(D)] = 1.0
+    vb = W.f32_to_bf16_bits(v)
+    p = float(np.quantile(oracle.dropout_uniforms(B, H, Sq, Sk, SEED), p))
+    o, _ = capi.attn_fwd_dropout(to_dev(q), to_dev(k), to_dev(vb), 0.05, p, SEED)
+    torch.cuda.synchronize()
+    keep = oracle.dropout_keep_mask(B, H, Sq, Sk, p, SEED)
+    got = to_f32(o)
+    assert np.array_equal(got != 0, keep)
+    assert 0.05 < keep.mean() < 0.95
+
+
+def test_dropout_argument_checks():
+    from flame_amd import capi
+    q = torch.zeros((1, 1, 64, 64), dtype=torch.bfloat16, device="cuda")
+    for bad in (-0.1, 1.0, 1.5, float("nan")):
+        with pytest.raises(capi.FlameAttnError) as e:
+            capi.attn_fwd_dropout(q, q, q, 0.125, bad, 1)
+        assert e.value.code == capi.ERR_INVALID
+    o, lse = capi.attn_fwd_dropout(q, q, q, 0.125, 0.0, 1)         # p = 0: the plain forward
+    o2, lse2 = capi.attn_fwd(q, q, q, 0.125)
+    torch.cuda.synchronize()
+    assert torch.equal(o, o2) and torch.equal(lse, lse2)
