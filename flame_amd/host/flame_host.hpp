@@ -695,7 +695,6 @@ inline Result<std::pair<Tensor, SdpaCtx>> sdpa_forward(const Tensor& q, const Te
             ((cfg.chunk_q && *cfg.chunk_q > 0 && (int64_t)*cfg.chunk_q < q.shape()[2]) ||
              (cfg.chunk_kv && *cfg.chunk_kv > 0 && (int64_t)*cfg.chunk_kv < k.shape()[2])))
             return unsupported("dropout with a chunked draw is not built: leave chunk_q / chunk_kv unset");
-        if (cfg.save == SdpaSave::Recompute) return unsupported("dropout with SdpaSave::Recompute is not built");
         dropout_seed = cfg.dropout_seed ? *cfg.dropout_seed : rng::next_u64();
     }
     if (cfg.save == SdpaSave::SaveProbs) return unsupported("SaveProbs materialises [B,H,Q,K]; use SaveLSE");
@@ -755,7 +754,8 @@ inline Result<std::tuple<Tensor, Tensor, Tensor>> sdpa_backward(const SdpaCtx& c
     n.dropout_seed = ctx.dropout_seed.value_or(0);
     if (ctx.dropout_p > 0.f && !ctx.dropout_seed) return Error{Error::InvalidInput, "dropout seed required when dropout_p > 0"};
     if (ctx.save == SdpaSave::Recompute) {          // nothing was kept: O and the log-sum-exp come from one more forward
-        auto f = detail::run_forward(ctx.q, ctx.k, ctx.v, ctx.attn_mask ? &*ctx.attn_mask : nullptr, ctx.causal, ctx.scale, true);
+        auto f = detail::run_forward(ctx.q, ctx.k, ctx.v, ctx.attn_mask ? &*ctx.attn_mask : nullptr, ctx.causal, ctx.scale, true,
+                                     ctx.dropout_p, ctx.dropout_seed.value_or(0));     // the same seed: the same kept set
         if (!f.ok()) return f.error();
         n.output = f.value().o;
         n.stats = f.value().stats;

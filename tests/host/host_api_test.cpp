@@ -346,6 +346,19 @@ int main() {
                     for (float x : host_f32_of_bf16(std::get<0>(g1.value()))) if (!std::isfinite(x)) { CHECK(false, "dQ with dropout not finite"); break; }
                 }
             }
+            {   // Recompute with dropout: the backward reruns the forward with the kept seed and gives the same gradients
+                autograd_v4::SdpaConfig rc2 = dc;
+                rc2.save = autograd_v4::SdpaSave::Recompute;
+                auto fr = autograd_v4::sdpa_forward(q, k, v, nullptr, rc2);
+                CHECK(fr.ok() && d1.ok(), "sdpa_forward (dropout, Recompute) failed");
+                if (fr.ok() && d1.ok()) {
+                    auto ga = autograd_v4::sdpa_backward(d1.value().second, d_o);
+                    auto gb = autograd_v4::sdpa_backward(fr.value().second, d_o);
+                    CHECK(ga.ok() && gb.ok() && host_bits_of_bf16(std::get<0>(ga.value())) == host_bits_of_bf16(std::get<0>(gb.value())) &&
+                              host_bits_of_bf16(std::get<1>(ga.value())) == host_bits_of_bf16(std::get<1>(gb.value())),
+                          "dropout: Recompute gradients differ from SaveLSE gradients");
+                }
+            }
             dc.dropout_seed.reset();
             autograd_v4::rng::set_seed(5);
             auto r1 = autograd_v4::sdpa_forward(q, k, v, nullptr, dc);
