@@ -346,7 +346,7 @@ def tile_dropout(probs, p, seed):
 
 
 # ---------------------------------------------------------------- dropout of the probabilities
-def attn_fwd_dropout(q, k, v, scale, dropout_p, dropout_seed, causal=False, kv_len=None, out=None):
+def attn_fwd_dropout(q, k, v, scale, dropout_p, dropout_seed, causal=False, kv_len=None, mask=None, out=None):
     """O, LSE = flame_attn_fwd_dropout_bf16(...): the kept set of the reference's autograd_v4 operator for this seed."""
     B, H, Sq, D = q.shape
     Sk = k.shape[2]
@@ -356,13 +356,14 @@ def attn_fwd_dropout(q, k, v, scale, dropout_p, dropout_seed, causal=False, kv_l
         _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), B, H, Sq, Sk, D, ctypes.c_float(scale),
         _i64x4(q.stride()), _i64x4(k.stride()), _i64x4(v.stride()), _i64x4(o.stride()),
         *(ctypes.c_int64(0) for _ in range(5)),
-        int(bool(causal)), _ptr(kv_len), ctypes.c_float(dropout_p), ctypes.c_uint64(dropout_seed & (2 ** 64 - 1)), _stream())
+        int(bool(causal)), _ptr(kv_len), _ptr(mask), _mask_strides(mask, B, H, Sq, Sk),
+        ctypes.c_float(dropout_p), ctypes.c_uint64(dropout_seed & (2 ** 64 - 1)), _stream())
     if rc != 0:
         raise FlameAttnError("flame_attn_fwd_dropout_bf16", rc)
     return o, lse
 
 
-def attn_bwd_dropout(q, k, v, o, do, lse, scale, dropout_p, dropout_seed, causal=False, kv_len=None, workspace=None):
+def attn_bwd_dropout(q, k, v, o, do, lse, scale, dropout_p, dropout_seed, causal=False, kv_len=None, mask=None, workspace=None):
     B, H, Sq, D = q.shape
     Sk = k.shape[2]
     if workspace is None:
@@ -376,7 +377,8 @@ def attn_bwd_dropout(q, k, v, o, do, lse, scale, dropout_p, dropout_seed, causal
         _i64x4(q.stride()), _i64x4(k.stride()), _i64x4(v.stride()), _i64x4(o.stride()),
         _i64x4(do.stride()), _i64x4(dq.stride()), _i64x4(dk.stride()), _i64x4(dv.stride()),
         *(ctypes.c_int64(0) for _ in range(9)),
-        int(bool(causal)), _ptr(kv_len), ctypes.c_float(dropout_p), ctypes.c_uint64(dropout_seed & (2 ** 64 - 1)),
+        int(bool(causal)), _ptr(kv_len), _ptr(mask), _mask_strides(mask, B, H, Sq, Sk),
+        ctypes.c_float(dropout_p), ctypes.c_uint64(dropout_seed & (2 ** 64 - 1)),
         _ptr(workspace), ctypes.c_size_t(workspace.numel()), _stream())
     if rc != 0:
         raise FlameAttnError("flame_attn_bwd_dropout_bf16", rc)

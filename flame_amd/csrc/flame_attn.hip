@@ -258,12 +258,12 @@ int launch_bwd(const BwdParams& p, hipStream_t s) {
 }
 
 // Dropout of the probabilities: the 128-query forward and dQ kernels and the dK/dV kernel in their DROPOUT
-// instantiations, without the split of the last round.  No explicit mask or bias.
-template <int D>
+// instantiations, without the split of the last round; HASMASK: the general kernels for an explicit mask or bias.
+template <int D, bool HASMASK>
 int launch_fwd_dropout(const FwdParams& p, hipStream_t s) {
     using T = FwdTile<D>;
     static bool attr_done = false;
-    auto kern = fwd_kernel<D, false, 4, false, true>;
+    auto kern = fwd_kernel<D, HASMASK, 4, false, true>;
     if (!attr_done) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS_BYTES);
@@ -280,13 +280,13 @@ int launch_fwd_dropout(const FwdParams& p, hipStream_t s) {
     return e == hipSuccess ? FLAME_ATTN_OK : (int)e;
 }
 
-template <int D>
+template <int D, bool HASMASK>
 int launch_bwd_dropout(const BwdParams& p, hipStream_t s) {
     using T = BwdTile<D>;
     using TQ = BwdDqTile<D>;
     static bool attr_done = false;
-    auto kern = bwd_dkdv_kernel<D, false, false, false, true>;
-    auto kern_dq = bwd_dq_kernel<D, false, 4, false, true>;
+    auto kern = bwd_dkdv_kernel<D, HASMASK, false, false, true>;
+    auto kern_dq = bwd_dq_kernel<D, HASMASK, 4, false, true>;
     if (!attr_done) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS_BYTES);
@@ -431,8 +431,8 @@ static int attn_bwd_impl(const void* Q, const void* K, const void* V, const void
 #endif
     if (dropout_p != 0.f) {
         if (!set_dropout(p.m, dropout_p, dropout_seed)) return FLAME_ATTN_ERR_INVALID;
-        if (keep_mask) return FLAME_ATTN_ERR_UNSUPPORTED;
-        return padded_head_dim(D) == 128 ? launch_bwd_dropout<128>(p, s) : launch_bwd_dropout<64>(p, s);
+        if (padded_head_dim(D) == 128) return keep_mask ? launch_bwd_dropout<128, true>(p, s) : launch_bwd_dropout<128, false>(p, s);
+        return keep_mask ? launch_bwd_dropout<64, true>(p, s) : launch_bwd_dropout<64, false>(p, s);
     }
     if (padded_head_dim(D) == 128) return keep_mask ? launch_bwd<128, true>(p, s) : launch_bwd<128, false>(p, s);
     return keep_mask ? launch_bwd<64, true>(p, s) : launch_bwd<64, false>(p, s);
@@ -462,11 +462,12 @@ int flame_attn_bwd_dropout_bf16(const void* Q, const void* K, const void* V, con
                                 const int64_t* dk_strides, const int64_t* dv_strides,
                                 int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off, int64_t do_off,
                                 int64_t lse_off, int64_t dq_off, int64_t dk_off, int64_t dv_off,
-                                int causal, const int32_t* kv_len, float dropout_p, uint64_t dropout_seed,
+                                int causal, const int32_t* kv_len, const uint8_t* keep_mask, const int64_t* mask_strides,
+                                float dropout_p, uint64_t dropout_seed,
                                 void* workspace, size_t workspace_bytes, void* stream) {
     return attn_bwd_impl(Q, K, V, O, dO, LSE, dQ, dK, dV, B, H, N_q, N_kv, D, scale, q_strides, k_strides, v_strides, o_strides,
                          do_strides, dq_strides, dk_strides, dv_strides, q_off, k_off, v_off, o_off, do_off, lse_off, dq_off,
-                         dk_off, dv_off, causal, kv_len, nullptr, nullptr, workspace, workspace_bytes, stream, dropout_p,
+                         dk_off, dv_off, causal, kv_len, keep_mask, mask_strides, workspace, workspace_bytes, stream, dropout_p,
                          dropout_seed);
 }
 
@@ -705,8 +706,9 @@ static int attn_fwd_impl(const void* Q, const void* K, const void* V, void* O, v
     const bool hm = keep_mask != nullptr || bias != nullptr;
     if (dropout_p != 0.f) {
         if (!set_dropout(p.m, dropout_p, dropout_seed)) return FLAME_ATTN_ERR_INVALID;
-        if (hm) return FLAME_ATTN_ERR_UNSUPPORTED;
-        return std::max(padded_head_dim(D), padded_head_dim(Dv)) == 128 ? launch_fwd_dropout<128>(p, s) : launch_fwd_dropout<64>(p, s);
+        if (std::max(padded_head_dim(D), padded_head_dim(Dv)) == 128)
+            return hm ? launch_fwd_dropout<128, true>(p, s) : launch_fwd_dropout<128, false>(p, s);
+        return hm ? launch_fwd_dropout<64, true>(p, s) : launch_fwd_dropout<64, false>(p, s);
     }
     // 256-query workgroups when they neither add padding rows nor leave compute units
     // without a workgroup
@@ -748,9 +750,10 @@ int flame_attn_fwd_dropout_bf16(const void* Q, const void* K, const void* V, voi
                                 const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
                                 const int64_t* o_strides,
                                 int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off, int64_t lse_off,
-                                int causal, const int32_t* kv_len, float dropout_p, uint64_t dropout_seed, void* stream) {
+                                int causal, const int32_t* kv_len, const uint8_t* keep_mask, const int64_t* mask_strides,
+                                float dropout_p, uint64_t dropout_seed, void* stream) {
     return attn_fwd_impl(Q, K, V, O, LSE, B, H, N_q, N_kv, D, scale, q_strides, k_strides, v_strides, o_strides,
-                         q_off, k_off, v_off, o_off, lse_off, causal, kv_len, nullptr, nullptr,
+                         q_off, k_off, v_off, o_off, lse_off, causal, kv_len, keep_mask, mask_strides,
                          nullptr, FLAME_ATTN_DTYPE_F32, nullptr, stream, kMaskU8, 0, 0, dropout_p, dropout_seed);
 }
 

@@ -241,11 +241,12 @@ inline Result<FwdOut> run_forward(const Tensor& q, const Tensor& k, const Tensor
     }
     const float sc = scale.value_or(1.0f / std::sqrt((float)d.D));
     if (dropout_p != 0.f) {
-        if (mask) return unsupported("dropout together with a mask is not built");
         const int rc = flame_attn_fwd_dropout_bf16(q.base(), k.base(), v.base(), o.value().base(), want_stats ? stats.base() : nullptr,
                                                    d.B, d.H, d.Sq, d.Sk, d.D, sc, q.strides().data(), k.strides().data(),
                                                    v.strides().data(), o.value().strides().data(), q.offset(), k.offset(),
-                                                   v.offset(), 0, 0, causal ? 1 : 0, nullptr, dropout_p, dropout_seed, nullptr);
+                                                   v.offset(), 0, 0, causal ? 1 : 0, nullptr,
+                                                   mask ? static_cast<const uint8_t*>(m8.data()) : nullptr, mask ? mst.data() : nullptr,
+                                                   dropout_p, dropout_seed, nullptr);
         if (rc == FLAME_ATTN_ERR_UNSUPPORTED) return unsupported("flame_attn_fwd_dropout_bf16: head dim or layout not built");
         if (rc != 0) return cuda_error("flame_attn_fwd_dropout_bf16", rc);
         return FwdOut{o.value(), stats};
@@ -351,14 +352,14 @@ inline Result<AttentionGrads> flash_attention_backward(const FlashAttentionNode&
         mst = pm.value().second;
     }
     if (n.dropout_p != 0.f) {
-        if (n.mask) return unsupported("dropout together with a mask is not built");
         const int rc = flame_attn_bwd_dropout_bf16(
             n.query.base(), n.key.base(), n.value.base(), n.output.base(), g.base(), n.stats.base(), dq.value().base(),
             dk.value().base(), dv.value().base(), B, H, Sq, Sk, D, n.scale, n.query.strides().data(), n.key.strides().data(),
             n.value.strides().data(), n.output.strides().data(), g.strides().data(), dq.value().strides().data(),
             dk.value().strides().data(), dv.value().strides().data(), n.query.offset(), n.key.offset(), n.value.offset(),
-            n.output.offset(), g.offset(), 0, 0, 0, 0, n.causal ? 1 : 0, nullptr, n.dropout_p, n.dropout_seed, ws.value().data(),
-            wsb, nullptr);
+            n.output.offset(), g.offset(), 0, 0, 0, 0, n.causal ? 1 : 0, nullptr,
+            n.mask ? static_cast<const uint8_t*>(m8.data()) : nullptr, n.mask ? mst.data() : nullptr, n.dropout_p, n.dropout_seed,
+            ws.value().data(), wsb, nullptr);
         if (rc == FLAME_ATTN_ERR_UNSUPPORTED) return unsupported("flame_attn_bwd_dropout_bf16: head dim or layout not built");
         if (rc != 0) return cuda_error("flame_attn_bwd_dropout_bf16", rc);
         return AttentionGrads{dq.value(), dk.value(), dv.value()};
@@ -683,8 +684,7 @@ inline uint64_t next_u64() {          // SplitMix64
 // sdpa_forward(q,k,v,mask,&cfg) -> (output, ctx) (:98-326).  SaveProbs would materialise the
 // [B,H,Q,K] matrix and is refused rather than emulated.  Dropout (:110-124, :229-231) runs inside the fused
 // kernels with the kept set the reference draws for the same seed when it does not chunk; a chunked draw
-// (chunk_q / chunk_kv smaller than the lengths) re-seeds per chunk (:600-602) and is not built, nor is dropout
-// together with a mask.
+// (chunk_q / chunk_kv smaller than the lengths) re-seeds per chunk (:600-602) and is not built.
 inline Result<std::pair<Tensor, SdpaCtx>> sdpa_forward(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor* mask,
                                                        const SdpaConfig& cfg) {
     if (cfg.dropout_p < 0.f || cfg.dropout_p >= 1.f || cfg.dropout_p != cfg.dropout_p)

@@ -95,7 +95,7 @@ int flame_attn_fwd_bias_bf16(const void* Q, const void* K, const void* V, void* 
  * src/rng/mod.rs:14-24): every element of the [B*H, N_q, N_kv] probability tensor with flat index i is kept when
  * (xorshift32(seed ^ i) >> 8) / 2^24 >= dropout_p (seed and i in their low 32 bits) and then multiplied by
  * 1 / (1 - dropout_p); the kept set is bit-identical to the reference's for the same seed.  O = (P * factor) V; LSE is
- * that of the undropped softmax, as the reference saves it.  0 <= dropout_p < 1 (else -1); no keep-mask or bias.
+ * that of the undropped softmax, as the reference saves it.  0 <= dropout_p < 1 (else -1).
  * Arguments otherwise as flame_attn_fwd_bf16.  No counterpart in the reference's FFI: there the operator is a chain of
  * tensor operations. */
 int flame_attn_fwd_dropout_bf16(const void* Q, const void* K, const void* V, void* O, void* LSE,
@@ -103,7 +103,8 @@ int flame_attn_fwd_dropout_bf16(const void* Q, const void* K, const void* V, voi
                                 const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
                                 const int64_t* o_strides,
                                 int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off, int64_t lse_off,
-                                int causal, const int32_t* kv_len, float dropout_p, uint64_t dropout_seed, void* stream);
+                                int causal, const int32_t* kv_len, const uint8_t* keep_mask, const int64_t* mask_strides,
+                                float dropout_p, uint64_t dropout_seed, void* stream);
 /* Its backward: dV = (P * factor)^T dO, dS = P * (factor * (dO V^T) - rowsum(dO * O)), dQ = scale dS K,
  * dK = scale dS^T Q with the same kept set, i.e. the derivative of the forward above (the reference's own backward,
  * src/autograd_v4/ops/sdpa.rs:756-772, forms dS without the factor P and is not reproduced).  O is the output of
@@ -116,7 +117,8 @@ int flame_attn_bwd_dropout_bf16(const void* Q, const void* K, const void* V, con
                                 const int64_t* dk_strides, const int64_t* dv_strides,
                                 int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off, int64_t do_off,
                                 int64_t lse_off, int64_t dq_off, int64_t dk_off, int64_t dv_off,
-                                int causal, const int32_t* kv_len, float dropout_p, uint64_t dropout_seed,
+                                int causal, const int32_t* kv_len, const uint8_t* keep_mask, const int64_t* mask_strides,
+                                float dropout_p, uint64_t dropout_seed,
                                 void* workspace, size_t workspace_bytes, void* stream);
 
 /* Recommended bytes of device scratch for the backward: two fp32 values per query row (required),

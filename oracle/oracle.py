@@ -356,7 +356,7 @@ def dropout_keep_mask(B, H, Sq, Sk, p, seed) -> np.ndarray:
     return dropout_uniforms(B, H, Sq, Sk, seed) >= np.float32(p)
 
 
-def sdpa_fwd_dropout(q, k, v, scale, p, seed, causal=False, kv_len=None, want_f32=False):
+def sdpa_fwd_dropout(q, k, v, scale, p, seed, causal=False, kv_len=None, mask=None, want_f32=False):
     B, H, Sq, D = q.shape
     Sk = k.shape[2]
     q, k, v = (np.ascontiguousarray(t, dtype=np.uint16) for t in (q, k, v))
@@ -364,14 +364,15 @@ def sdpa_fwd_dropout(q, k, v, scale, p, seed, causal=False, kv_len=None, want_f3
     LSE = np.zeros((B, H, Sq), np.float32)
     O32 = np.zeros((B, H, Sq, D), np.float32) if want_f32 else None
     kvl = None if kv_len is None else np.ascontiguousarray(kv_len, dtype=np.int32)
+    m, st, _keep = _mask_args(mask, B, H, Sq, Sk)
     rc = lib().oracle_sdpa_fwd_dropout(_p(q), _p(k), _p(v), B, H, Sq, Sk, D, ctypes.c_float(scale), int(bool(causal)), _p(kvl),
-                                       ctypes.c_float(p), ctypes.c_uint64(seed & (2 ** 64 - 1)), _p(O), _p(LSE), _p(O32))
+                                       _p(m), *(ctypes.c_int64(x) for x in st), ctypes.c_float(p), ctypes.c_uint64(seed & (2 ** 64 - 1)), _p(O), _p(LSE), _p(O32))
     if rc != 0:
         raise RuntimeError(f"oracle_sdpa_fwd_dropout failed: {rc}")
     return (O, LSE, O32) if want_f32 else (O, LSE)
 
 
-def sdpa_bwd_dropout(q, k, v, o, do, scale, p, seed, causal=False, kv_len=None, want_f32=False):
+def sdpa_bwd_dropout(q, k, v, o, do, scale, p, seed, causal=False, kv_len=None, mask=None, want_f32=False):
     B, H, Sq, D = q.shape
     Sk = k.shape[2]
     q, k, v, o, do = (np.ascontiguousarray(t, dtype=np.uint16) for t in (q, k, v, o, do))
@@ -380,8 +381,9 @@ def sdpa_bwd_dropout(q, k, v, o, do, scale, p, seed, causal=False, kv_len=None, 
     dV = np.zeros((B, H, Sk, D), np.uint16)
     f = [np.zeros(t.shape, np.float32) for t in (dQ, dK, dV)] if want_f32 else [None] * 3
     kvl = None if kv_len is None else np.ascontiguousarray(kv_len, dtype=np.int32)
+    m, st, _keep = _mask_args(mask, B, H, Sq, Sk)
     rc = lib().oracle_sdpa_bwd_dropout(_p(q), _p(k), _p(v), _p(o), _p(do), B, H, Sq, Sk, D, ctypes.c_float(scale),
-                                       int(bool(causal)), _p(kvl), ctypes.c_float(p), ctypes.c_uint64(seed & (2 ** 64 - 1)),
+                                       int(bool(causal)), _p(kvl), _p(m), *(ctypes.c_int64(x) for x in st), ctypes.c_float(p), ctypes.c_uint64(seed & (2 ** 64 - 1)),
                                        _p(dQ), _p(dK), _p(dV), _p(f[0]), _p(f[1]), _p(f[2]))
     if rc != 0:
         raise RuntimeError(f"oracle_sdpa_bwd_dropout failed: {rc}")

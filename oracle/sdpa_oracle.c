@@ -384,21 +384,22 @@ int oracle_sdpa_bwd_rows(const uint16_t* Q, const uint16_t* K, const uint16_t* V
                          dQ, dK, dV, dQ32, dK32, dV32);
 }
 
-/* Forward and backward with dropout of the probabilities (see drop_factor); causal flag and key lengths as the
- * only exclusions. */
+/* Forward and backward with dropout of the probabilities (see drop_factor). */
 int oracle_sdpa_fwd_dropout(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
                             int B, int H, int Sq, int Sk, int D, float scale, int causal, const int32_t* kv_len,
+                            const uint8_t* mask, int64_t msb, int64_t msh, int64_t msq, int64_t msk,
                             float drop_p, uint64_t drop_seed, uint16_t* O, float* LSE, float* O32) {
-    mask_spec ms = {causal, kv_len, NULL, 0, 0, 0, 0, NULL, 0, 0, 0, 0, drop_p, drop_seed};
+    mask_spec ms = {causal, kv_len, mask, msb, msh, msq, msk, NULL, 0, 0, 0, 0, drop_p, drop_seed};
     return sdpa_fwd_impl(Q, K, V, B, H, Sq, Sk, D, scale, ms, 0, B * H, 0, Sq, O, LSE, O32);
 }
 
 int oracle_sdpa_bwd_dropout(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
                             const uint16_t* O, const uint16_t* dO,
                             int B, int H, int Sq, int Sk, int D, float scale, int causal, const int32_t* kv_len,
+                            const uint8_t* mask, int64_t msb, int64_t msh, int64_t msq, int64_t msk,
                             float drop_p, uint64_t drop_seed,
                             uint16_t* dQ, uint16_t* dK, uint16_t* dV, float* dQ32, float* dK32, float* dV32) {
-    mask_spec ms = {causal, kv_len, NULL, 0, 0, 0, 0, NULL, 0, 0, 0, 0, drop_p, drop_seed};
+    mask_spec ms = {causal, kv_len, mask, msb, msh, msq, msk, NULL, 0, 0, 0, 0, drop_p, drop_seed};
     return sdpa_bwd_impl(Q, K, V, O, dO, B, H, Sq, Sk, D, scale, ms, 0, B * H, 0, Sq, dQ, dK, dV, dQ32, dK32, dV32);
 }
 
