@@ -50,6 +50,15 @@ __device__ __forceinline__ void mfma32_vgpr_first_bacc(f32x16& acc, bf16x8 a, bf
 __device__ __forceinline__ void mfma32_vgpr_bacc(f32x16& acc, bf16x8 a, bf16x8 b) {
     asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "a"(b));
 }
+// Both operands in architectural registers (a kernel whose B fragments are too many for the accumulation file's
+// free part).  After the last MFMA of a chain, mfma32_vgpr_settle spends the 11 wait states before its result may be
+// read, for kernels that have no other MFMAs to put there.
+__device__ __forceinline__ void mfma32_vgpr(f32x16& acc, bf16x8 a, bf16x8 b) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void mfma32_vgpr_settle(f32x16& acc) {
+    asm volatile("s_nop 11" : "+v"(acc));
+}
 // The same with the B operand pinned to accumulation registers a[128 + 4 SLOT : 131 + 4 SLOT], for a
 // kernel whose 32 resident B fragments must stay put there (left to itself the register allocator
 // homes some of them in architectural registers and copies them over before every use).
@@ -213,6 +222,50 @@ __device__ __forceinline__ void rescale_pinned(f32x16& acc, float alpha) {
         asm volatile("v_accvgpr_read_b32 %1, a96\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a96, %1\n\tv_accvgpr_read_b32 %1, a97\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a97, %1\n\tv_accvgpr_read_b32 %1, a98\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a98, %1\n\tv_accvgpr_read_b32 %1, a99\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a99, %1\n\tv_accvgpr_read_b32 %1, a100\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a100, %1\n\tv_accvgpr_read_b32 %1, a101\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a101, %1\n\tv_accvgpr_read_b32 %1, a102\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a102, %1\n\tv_accvgpr_read_b32 %1, a103\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a103, %1\n\tv_accvgpr_read_b32 %1, a104\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a104, %1\n\tv_accvgpr_read_b32 %1, a105\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a105, %1\n\tv_accvgpr_read_b32 %1, a106\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a106, %1\n\tv_accvgpr_read_b32 %1, a107\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a107, %1\n\tv_accvgpr_read_b32 %1, a108\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a108, %1\n\tv_accvgpr_read_b32 %1, a109\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a109, %1\n\tv_accvgpr_read_b32 %1, a110\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a110, %1\n\tv_accvgpr_read_b32 %1, a111\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a111, %1" : "+{a[96:111]}"(acc), "=&v"(tmp) : "v"(alpha));
     if constexpr (IDX == 7)
         asm volatile("v_accvgpr_read_b32 %1, a112\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a112, %1\n\tv_accvgpr_read_b32 %1, a113\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a113, %1\n\tv_accvgpr_read_b32 %1, a114\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a114, %1\n\tv_accvgpr_read_b32 %1, a115\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a115, %1\n\tv_accvgpr_read_b32 %1, a116\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a116, %1\n\tv_accvgpr_read_b32 %1, a117\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a117, %1\n\tv_accvgpr_read_b32 %1, a118\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a118, %1\n\tv_accvgpr_read_b32 %1, a119\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a119, %1\n\tv_accvgpr_read_b32 %1, a120\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a120, %1\n\tv_accvgpr_read_b32 %1, a121\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a121, %1\n\tv_accvgpr_read_b32 %1, a122\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a122, %1\n\tv_accvgpr_read_b32 %1, a123\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a123, %1\n\tv_accvgpr_read_b32 %1, a124\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a124, %1\n\tv_accvgpr_read_b32 %1, a125\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a125, %1\n\tv_accvgpr_read_b32 %1, a126\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a126, %1\n\tv_accvgpr_read_b32 %1, a127\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a127, %1" : "+{a[112:127]}"(acc), "=&v"(tmp) : "v"(alpha));
+}
+
+// acc += a b with the accumulator pinned to a[16 IDX : 16 IDX + 15] (the tuples rescale_pinned works on) and both
+// operands in architectural registers, emitted by hand: given the same fixed registers at every use, the accumulator
+// never moves (left to the compiler's MFMA form, accumulators that a conditional rescale also touches travelled
+// through architectural registers once per key tile).  FRESH_B: the B operand was just written by the vector ALU, which
+// needs two wait states before an MFMA reads it.  mfma32_apinned_settle<IDX, WAIT> is the fence before the
+// accumulators are read after the last tile: the one with WAIT spends the 11 wait states, and since volatile
+// statements keep their order, fencing every accumulator after it orders all their reads behind that wait.
+template <int IDX, bool FRESH_B>
+__device__ __forceinline__ void mfma32_apinned(f32x16& acc, bf16x8 a, bf16x8 b) {
+    static_assert(IDX >= 0 && IDX < 8, "eight pinned accumulator tuples");
+#define FATTN_PIN(I, R)                                                                                        \
+    if constexpr (IDX == I) {                                                                                  \
+        if constexpr (FRESH_B) asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : R(acc) : "v"(a), "v"(b)); \
+        else asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : R(acc) : "v"(a), "v"(b));                \
+    }
+    FATTN_PIN(0, "+{a[0:15]}")
+    FATTN_PIN(1, "+{a[16:31]}")
+    FATTN_PIN(2, "+{a[32:47]}")
+    FATTN_PIN(3, "+{a[48:63]}")
+    FATTN_PIN(4, "+{a[64:79]}")
+    FATTN_PIN(5, "+{a[80:95]}")
+    FATTN_PIN(6, "+{a[96:111]}")
+    FATTN_PIN(7, "+{a[112:127]}")
+#undef FATTN_PIN
+}
+template <int IDX, bool WAIT>
+__device__ __forceinline__ void mfma32_apinned_settle(f32x16& acc) {
+    static_assert(IDX >= 0 && IDX < 8, "eight pinned accumulator tuples");
+#define FATTN_PIN(I, R)                                                                                        \
+    if constexpr (IDX == I) {                                                                                  \
+        if constexpr (WAIT) asm volatile("s_nop 11" : R(acc));                                                 \
+        else asm volatile("" : R(acc));                                                                        \
+    }
+    FATTN_PIN(0, "+{a[0:15]}")
+    FATTN_PIN(1, "+{a[16:31]}")
+    FATTN_PIN(2, "+{a[32:47]}")
+    FATTN_PIN(3, "+{a[48:63]}")
+    FATTN_PIN(4, "+{a[64:79]}")
+    FATTN_PIN(5, "+{a[80:95]}")
+    FATTN_PIN(6, "+{a[96:111]}")
+    FATTN_PIN(7, "+{a[112:127]}")
+#undef FATTN_PIN
 }
 
 // compile-time loop: f(std::integral_constant<int, 0>{}) ... f(std::integral_constant<int, N - 1>{})

@@ -18,6 +18,7 @@
 
 #include "attn_bwd.hpp"
 #include "attn_fwd.hpp"
+#include "attn_fwd_bigd.hpp"
 #include "prep.hpp"
 #include "sage.hpp"
 #include "plan_cache.hpp"
@@ -147,6 +148,8 @@ size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 // Head dims: the kernels are compiled for 64 and 128; any other multiple of 8 up to 128 (96 among them) runs
 // zero-padded on the next compiled size.
 bool head_dim_ok(int D) { return D > 0 && D <= 128 && D % 8 == 0; }
+// head dims served by the forward alone, in chunks of 128 (attn_fwd_bigd.hpp)
+bool big_head_dim_ok(int D) { return D > 128 && D <= 512 && D % 8 == 0; }
 int padded_head_dim(int D) { return D <= 64 ? 64 : 128; }
 
 // compute units of the current device (cached; 256 when the query fails)
@@ -252,6 +255,28 @@ int launch_bwd(const BwdParams& p, hipStream_t s) {
     if (n_split > 0) {
         ScopedKernelTimer t(FLAME_ATTN_KERNEL_BWD_MERGE, s);
         hipLaunchKernelGGL(bwd_dkdv_merge_kernel<D>, dim3((unsigned)(n_split * (D / 32))), dim3(256), 0, s, pk);
+    }
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? FLAME_ATTN_OK : (int)e;
+}
+
+template <int NC>
+int launch_fwd_bigd(const FwdParams& p, hipStream_t s) {
+    constexpr bool SPLIT = NC > 2;
+    using T = FwdBigDTile<NC, SPLIT>;
+    static bool attr_done = false;
+    auto kern = fwd_bigd_kernel<NC, SPLIT>;
+    if (!attr_done) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS_BYTES);
+        if (e != hipSuccess) return (int)e;
+        attr_done = true;
+    }
+    const int64_t grid = (int64_t)((p.Sq + T::BM - 1) / T::BM) * p.B * p.H;
+    if (grid > 0x7fffffff) return FLAME_ATTN_ERR_UNSUPPORTED;
+    {
+        ScopedKernelTimer t(FLAME_ATTN_KERNEL_FWD, s);
+        hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), T::LDS_BYTES, s, p);
     }
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? FLAME_ATTN_OK : (int)e;
@@ -664,7 +689,9 @@ static int attn_fwd_impl(const void* Q, const void* K, const void* V, void* O, v
     if (Dv == 0) Dv = D;           // V and O may have a head dim of their own (forward only)
     if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0 || Dv < 0) return FLAME_ATTN_ERR_INVALID;
     if (!(scale > 0.f) || !isfinite(scale)) return FLAME_ATTN_ERR_INVALID;
-    if (!head_dim_ok(D) || !head_dim_ok(Dv)) return FLAME_ATTN_ERR_UNSUPPORTED;
+    // head dims above 128: the forward in chunks of 128, without explicit mask, bias or dropout and with Dv = D
+    const bool big = big_head_dim_ok(D) && Dv == D && !keep_mask && !bias && dropout_p == 0.f;
+    if (!big && (!head_dim_ok(D) || !head_dim_ok(Dv))) return FLAME_ATTN_ERR_UNSUPPORTED;
     int rc;
     if ((rc = check_view(Q, q_strides, q_off))) return rc;
     if ((rc = check_view(K, k_strides, k_off))) return rc;
@@ -703,6 +730,7 @@ static int attn_fwd_impl(const void* Q, const void* K, const void* V, void* O, v
     }
 
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (big) return D <= 256 ? launch_fwd_bigd<2>(p, s) : D <= 384 ? launch_fwd_bigd<3>(p, s) : launch_fwd_bigd<4>(p, s);
     const bool hm = keep_mask != nullptr || bias != nullptr;
     if (dropout_p != 0.f) {
         if (!set_dropout(p.m, dropout_p, dropout_seed)) return FLAME_ATTN_ERR_INVALID;
@@ -1128,7 +1156,8 @@ bool sdpa_stream_bf16_launch(const void* dQ, const void* dK, const void* dV, voi
     };
     (void)head_tile;
     if (q_tile > max_q_tile) return fail("q_tile exceeds max_q_tile");
-    if (!head_dim_ok(d)) return fail("head dim must be a multiple of 8, at most 128");
+    if (!head_dim_ok(d) && !(big_head_dim_ok(d) && !attn_mask))
+        return fail("head dim must be a multiple of 8, at most 128 (at most 512 without a mask)");
     const int64_t qs[4] = {(int64_t)H * Q_len * d, (int64_t)Q_len * d, d, 1};
     const int64_t ks[4] = {(int64_t)H * K_len * d, (int64_t)K_len * d, d, 1};
     // bf16 mask addressed by the caller's four element strides; in this entry point a value above 0.5 EXCLUDES

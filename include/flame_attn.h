@@ -16,7 +16,11 @@
  *   - D (head dim) is any multiple of 8 up to 128.  The kernels are compiled for 64 and 128 (the
  *     reference's production sizes, with 96: src/sdpa.rs:149, src/cuda/flash_attention_fwd.cu:307-324);
  *     other sizes, 96 included, run zero-padded to the next compiled size inside the tile loads and
- *     stores, at that size's cost.  Anything else returns FLAME_ATTN_ERR_UNSUPPORTED.  The Sage and
+ *     stores, at that size's cost.  The forward entry points also take multiples of 8 above 128, up
+ *     to 512 (the reference serves those through its materialised path, src/sdpa.rs:483-587; e.g. the
+ *     one-head D = 512 attention of a VAE mid block), in chunks of 128, when there is no keep-mask,
+ *     bias or dropout and V has the head dim of Q; the backward does not (recompute through a
+ *     materialised path there).  Anything else returns FLAME_ATTN_ERR_UNSUPPORTED.  The Sage and
  *     input-preparation entry points take 64 or 128 only.
  *   - LSE / Stats: fp32, contiguous [B*H, N_q] (== [B,H,N_q,1] with strides [H*N_q, N_q, 1, 1]),
  *     value = max_j s_ij + ln(sum_j exp(s_ij - max)), s = scale * Q K^T, natural log

@@ -178,6 +178,7 @@ int main() {
         Tensor f32 = Tensor::empty({1, 2, 8, 64}, DType::F32).value();
         Tensor d100 = Tensor::empty({1, 2, 8, 104}, DType::BF16).value();
         Tensor d256 = Tensor::empty({1, 2, 8, 256}, DType::BF16).value();
+        Tensor d520 = Tensor::empty({1, 2, 8, 520}, DType::BF16).value();
         Tensor badm = Tensor::empty({1, 2, 8, 9}, DType::U8).value();
         auto kind = [](const Result<Tensor>& r) { return r.ok() ? -1 : (int)r.error().kind; };
         CHECK(kind(sdpa::forward(r3, r3, r3)) == Error::InvalidInput, "rank 3");
@@ -187,7 +188,8 @@ int main() {
         CHECK(kind(sdpa::forward(a, a, a, &badm)) == Error::InvalidInput, "mask not broadcastable");
         CHECK(kind(sdpa::forward(f32, f32, f32)) == Error::InvalidInput, "non-bf16");
         CHECK(sdpa::forward(d100, d100, d100).ok(), "head dim 104 runs (padded to 128)");
-        CHECK(kind(sdpa::forward(d256, d256, d256)) == Error::Unsupported, "head dim 256");
+        CHECK(sdpa::forward(d256, d256, d256).ok(), "head dim 256 runs (forward only, two chunks of 128)");
+        CHECK(kind(sdpa::forward(d520, d520, d520)) == Error::Unsupported, "head dim 520");
     }
 
     // ---- 3. forward == forward_train, taped backward vs the naive recompute; shapes of

@@ -58,8 +58,8 @@ def test_argument_validation_without_a_device():
                                    *(ctypes.c_int64(0),) * 5, 0, null, null, null, null) == -1
     assert lib.flame_attn_fwd_bf16(null, one, one, one, null, 1, 1, 64, 64, 64, ctypes.c_float(0.1), st, st, st, st,
                                    *(ctypes.c_int64(0),) * 5, 0, null, null, null, null) == -1
-    # head dims that are not a multiple of 8 or exceed 128, and a D stride of 2, are not built -> -2
-    for bad_d in (100, 136, 256):
+    # head dims that are not a multiple of 8 or exceed 512, and a D stride of 2, are not built -> -2
+    for bad_d in (100, 132, 520, 1024):
         assert lib.flame_attn_fwd_bf16(one, one, one, one, null, 1, 1, 64, 64, bad_d, ctypes.c_float(0.1), st, st, st, st,
                                        *(ctypes.c_int64(0),) * 5, 0, null, null, null, null) == -2
     bad = (ctypes.c_int64 * 4)(64 * 64, 64 * 64, 64, 2)
