@@ -144,6 +144,8 @@ def tile_ops_line(args, capi, torch, dev):
     lse = torch.logsumexp(logits, -1)
     lse_other = lse.clone()
     probs = torch.rand((BH, q_t, k_t), device=dev, generator=g).to(torch.bfloat16)
+    saved = torch.randn((4, 24, 4608, 128), device=dev, generator=g).to(torch.bfloat16)
+    saved_fp8 = torch.empty(saved.shape, device=dev, dtype=torch.uint8)
     n_future = int((torch.arange(k_t, device=dev)[None, :] > torch.arange(q_t, device=dev)[:, None]).sum()) * BH
     n_dropped = int((keep == 0).sum())
     cases = [
@@ -158,6 +160,9 @@ def tile_ops_line(args, capi, torch, dev):
         ("flame_sdpa_softmax_from_lse_tile", lambda: capi.tile_softmax_from_lse(logits, lse, out=probs), 6 * n + 4 * BH * q_t),
         ("flame_sdpa_lse_merge_rows", lambda: capi.tile_lse_merge(lse, lse_other), 12 * BH * q_t),
         ("flame_sdpa_dropout_bf16_inplace", lambda: capi.tile_dropout(probs, 0.1, 2024), 4 * n),
+        # the saved set of the headline shape on its way to the offload pool: Q, K, V, O = 4 x [1, 24, 4608, 128] bf16
+        ("flame_bf16_to_fp8 (saved Q,K,V,O of cfg 2)", lambda: capi.bf16_to_fp8(saved, 56.0, out=saved_fp8), 3 * saved.numel()),
+        ("flame_fp8_to_bf16 (saved Q,K,V,O of cfg 2)", lambda: capi.fp8_to_bf16(saved_fp8, 1.0 / 56.0, out=saved), 3 * saved.numel()),
     ]
     out = {}
     for name, fn, nbytes in cases:
@@ -176,7 +181,7 @@ def tile_ops_line(args, capi, torch, dev):
                      "frac_of_hbm_peak": nbytes / (ms * 1e-3) / 8e12}
     print(json.dumps({"metric": "element-wise tile primitives, GB/s of algorithmic bytes", "unit": "GB/s", "n_gpus": 1,
                       "dtype": "f32/bf16/u8", "data": "synthetic",
-                      "config": {"workload": "score tile [24, 1024, 4608]"}, "primitives": out}))
+                      "config": {"workload": "score tile [24, 1024, 4608]; FP8 pair on 4 x [1, 24, 4608, 128] bf16"}, "primitives": out}))
     return 0
 
 

@@ -345,6 +345,29 @@ def tile_dropout(probs, p, seed):
     return probs
 
 
+# ---------------------------------------------------------------- FP8 form of offloaded activations
+def bf16_to_fp8(x, inv_scale, out=None):
+    """out[i] = fp8_e4m3(float(x[i]) * inv_scale) (uint8), flame_bf16_to_fp8; x is any contiguous bf16 tensor."""
+    assert x.dtype == torch.bfloat16 and x.is_contiguous()
+    out = torch.empty(x.shape, dtype=torch.uint8, device=x.device) if out is None else out
+    assert out.dtype == torch.uint8 and out.is_contiguous() and out.numel() == x.numel()
+    rc = lib().flame_bf16_to_fp8(_ptr(x), _ptr(out), ctypes.c_float(inv_scale), ctypes.c_size_t(x.numel()), _stream())
+    if rc != 0:
+        raise FlameAttnError("flame_bf16_to_fp8", rc)
+    return out
+
+
+def fp8_to_bf16(codes, scale, out=None):
+    """out[i] = bf16(float(fp8(codes[i])) * scale), flame_fp8_to_bf16."""
+    assert codes.dtype == torch.uint8 and codes.is_contiguous()
+    out = torch.empty(codes.shape, dtype=torch.bfloat16, device=codes.device) if out is None else out
+    assert out.dtype == torch.bfloat16 and out.is_contiguous() and out.numel() == codes.numel()
+    rc = lib().flame_fp8_to_bf16(_ptr(codes), _ptr(out), ctypes.c_float(scale), ctypes.c_size_t(codes.numel()), _stream())
+    if rc != 0:
+        raise FlameAttnError("flame_fp8_to_bf16", rc)
+    return out
+
+
 # ---------------------------------------------------------------- dropout of the probabilities
 def attn_fwd_dropout(q, k, v, scale, dropout_p, dropout_seed, causal=False, kv_len=None, mask=None, out=None):
     """O, LSE = flame_attn_fwd_dropout_bf16(...): the kept set of the reference's autograd_v4 operator for this seed."""

@@ -23,6 +23,7 @@
 #include "sage.hpp"
 #include "plan_cache.hpp"
 #include "tile_ops.hpp"
+#include "fp8_offload.hpp"
 
 using namespace fattn;
 
@@ -1384,6 +1385,37 @@ int flame_sdpa_dropout_bf16_inplace(void* probs_bf16, float p, uint64_t seed, in
         hipLaunchKernelGGL(tile_dropout_kernel<1>, dim3(grid), dim3(256), 0, s, probs, p, scale, seed, total, q_t, k_t);
     }
     return tile_launched();
+}
+
+// ---- FP8 E4M3 form of saved activations for the offload pool (src/cuda/fp8_quant.cu:74-92, fp8_dequant.cu:42-58)
+static float fp8_flushed(float s) { return fabsf(s) < 1.17549435e-38f ? copysignf(0.f, s) : s; }   // the reference's multiply flushes denormal operands
+static unsigned fp8_grid(size_t n, bool vec) {
+    const size_t work = vec ? (n / 16 > n % 16 ? n / 16 : n % 16) : n;      // lanes that have something to do
+    const size_t g = (work + 255) / 256;
+    const size_t cap = (size_t)device_cu_count() * 8;                               // grid-stride beyond 8 workgroups per CU
+    return (unsigned)(g < 1 ? 1 : g > cap ? cap : g);
+}
+
+int flame_bf16_to_fp8(const void* input, void* output, float inv_scale, size_t n_elements, void* stream) {
+    if (n_elements == 0) return 0;
+    if (!input || !output) return (int)hipErrorInvalidValue;
+    const bool vec = aligned16(input) && aligned16(output) && n_elements >= 16;
+    const Fp8Params p{input, output, fp8_flushed(inv_scale), n_elements};
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (vec) hipLaunchKernelGGL(bf16_to_fp8_kernel<true>, dim3(fp8_grid(n_elements, true)), dim3(256), 0, s, p);
+    else hipLaunchKernelGGL(bf16_to_fp8_kernel<false>, dim3(fp8_grid(n_elements, false)), dim3(256), 0, s, p);
+    return (int)hipGetLastError();
+}
+
+int flame_fp8_to_bf16(const void* input, void* output, float scale, size_t n_elements, void* stream) {
+    if (n_elements == 0) return 0;
+    if (!input || !output) return (int)hipErrorInvalidValue;
+    const bool vec = aligned16(input) && aligned16(output) && n_elements >= 16;
+    const Fp8Params p{input, output, fp8_flushed(scale), n_elements};
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (vec) hipLaunchKernelGGL(fp8_to_bf16_kernel<true>, dim3(fp8_grid(n_elements, true)), dim3(256), 0, s, p);
+    else hipLaunchKernelGGL(fp8_to_bf16_kernel<false>, dim3(fp8_grid(n_elements, false)), dim3(256), 0, s, p);
+    return (int)hipGetLastError();
 }
 
 #ifndef FLAME_ATTN_HIPCC_VERSION

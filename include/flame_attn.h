@@ -335,6 +335,23 @@ int flame_sdpa_lse_merge_rows(float* lse_row, const float* tile_lse_row, int BH,
 int flame_sdpa_dropout_bf16_inplace(void* probs_bf16, float p, uint64_t seed, int BH, int q_t, int k_t, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
+ * FP8 E4M3 form of saved activations (O, or Q / K / V) on their way to and from pinned host memory: the pair the
+ * reference's activation offload pool runs on its transfer stream around the copies
+ * (src/cuda/ffi.rs:545-562; src/cuda/fp8_quant.cu:74-92, src/cuda/fp8_dequant.cu:42-58; used by
+ * src/activation_offload.rs:536-586, :678-700 with scale = 8 / 448).  Contiguous tensors of n_elements; any
+ * alignment (16-byte aligned pointers take the vector path).  Return 0 or the HIP error code, like the reference.
+ *   flame_bf16_to_fp8:  output[i] = fp8_e4m3(float(input[i]) * inv_scale)   (1 byte per element)
+ *   flame_fp8_to_bf16:  output[i] = bf16(float(fp8(input[i])) * scale)
+ * The codes are the reference's bit for bit, including its deviations from OCP E4M3: the mantissa is rounded half
+ * up in magnitude; products of 256 and above all become 0x7F, which the decoder reads as 480 (no NaN code);
+ * a product that would round up to the smallest normal stays at the largest subnormal; operands and products below
+ * 2^-126 count as zero (the reference is built with flush-to-zero).  With the pool's fixed scale every |x| >= 32/7
+ * therefore comes back as 60/7 = 8.57: callers whose activations reach that range should pass a larger scale.
+ * ---------------------------------------------------------------------------------------------- */
+int flame_bf16_to_fp8(const void* input, void* output, float inv_scale, size_t n_elements, void* stream);
+int flame_fp8_to_bf16(const void* input, void* output, float scale, size_t n_elements, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
  * Profiling aids (the counterpart of the reference's SdpaStats / SdpaHooks timing fields,
  * src/autograd_v4/ops/sdpa.rs:55-79).  No counterpart in the FFI of the reference.
  * ---------------------------------------------------------------------------------------------- */

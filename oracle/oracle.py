@@ -388,3 +388,27 @@ def sdpa_bwd_dropout(q, k, v, o, do, scale, p, seed, causal=False, kv_len=None, 
     if rc != 0:
         raise RuntimeError(f"oracle_sdpa_bwd_dropout failed: {rc}")
     return (dQ, dK, dV, *f) if want_f32 else (dQ, dK, dV)
+
+
+# --------------------------------------------------------------------------- FP8 form of offloaded activations
+def f32_to_fp8_e4m3(val: float) -> int:
+    """The reference's scalar encoder (src/cuda/fp8_quant.cu:19-57) on one fp32 product."""
+    f = lib().oracle_f32_to_fp8_e4m3
+    f.restype = ctypes.c_uint8
+    return int(f(ctypes.c_float(val)))
+
+
+def bf16_to_fp8(x_bits: np.ndarray, inv_scale: float) -> np.ndarray:
+    """out[i] = fp8(bf16(x[i]) * inv_scale), src/cuda/fp8_quant.cu:59-72."""
+    x = np.ascontiguousarray(x_bits, dtype=np.uint16)
+    out = np.empty(x.shape, np.uint8)
+    lib().oracle_bf16_to_fp8(_p(x), _p(out), ctypes.c_float(inv_scale), ctypes.c_size_t(x.size))
+    return out
+
+
+def fp8_to_bf16(codes: np.ndarray, scale: float) -> np.ndarray:
+    """out[i] = bf16(fp8(codes[i]) * scale), src/cuda/fp8_dequant.cu:10-39."""
+    c = np.ascontiguousarray(codes, dtype=np.uint8)
+    out = np.empty(c.shape, np.uint16)
+    lib().oracle_fp8_to_bf16(_p(c), _p(out), ctypes.c_float(scale), ctypes.c_size_t(c.size))
+    return out

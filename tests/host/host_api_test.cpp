@@ -651,6 +651,159 @@ int main() {
         CHECK(at != std::string::npos && std::atof(last.c_str() + at + 13) > 0.0, "elapsed_ms must be positive");
     }
 
+    // ---- 11. activation offload pool: the reference's own four tests (src/activation_offload.rs:843-978), FP8
+    //          compression, and the saved set of an attention call through the pool and back into the backward
+    {
+        using namespace activation_offload;
+        {   // push_pull_round_trip_bf16
+            auto pr = ActivationOffloadPool::create(2, 1024, OffloadCompression::None);
+            CHECK(pr.ok(), "pool");
+            if (pr.ok()) {
+                auto& pool = *pr.value();
+                CHECK(pool.num_slots() == 2 && pool.slot_bytes() == 1024 && pool.host_bytes() == 2048, "pool sizes");
+                std::vector<uint16_t> src(32);
+                for (int i = 0; i < 32; ++i) src[i] = f2bf((float)i * 0.125f - 1.0f);
+                Tensor t = dev_bf16(src, {4, 8});
+                auto h = pool.push(t);
+                CHECK(h.ok() && pool.in_flight() == 1, "push");
+                if (h.ok()) {
+                    auto back = pool.pull(h.value());
+                    CHECK(back.ok() && pool.in_flight() == 0, "pull");
+                    if (back.ok()) {
+                        CHECK(back.value().dtype() == DType::BF16 && back.value().shape() == std::vector<int64_t>({4, 8}), "pulled dtype/shape");
+                        CHECK(host_bits_of_bf16(back.value()) == src, "round trip is bit-exact without compression");
+                    }
+                    CHECK(!pool.pull(h.value()).ok(), "double pull must fail");
+                }
+            }
+        }
+        {   // push_pull_lifo_two_slots_bf16
+            auto pr = ActivationOffloadPool::create(2, 2048, OffloadCompression::None);
+            if (pr.ok()) {
+                auto& pool = *pr.value();
+                std::vector<uint16_t> a = {f2bf(1), f2bf(2), f2bf(3), f2bf(4)}, b = {f2bf(-1), f2bf(-2), f2bf(-3), f2bf(-4)};
+                Tensor ta = dev_bf16(a, {4}), tb = dev_bf16(b, {4});
+                auto ha = pool.push(ta), hb = pool.push(tb);
+                CHECK(ha.ok() && hb.ok() && ha.value().slot() != hb.value().slot() && pool.in_flight() == 2, "two pushes, two slots");
+                if (ha.ok() && hb.ok()) {
+                    auto pb = pool.pull(hb.value()), pa = pool.pull(ha.value());
+                    CHECK(pa.ok() && pb.ok() && pool.in_flight() == 0, "LIFO pulls");
+                    if (pa.ok() && pb.ok())
+                        CHECK(host_bits_of_bf16(pa.value()) == a && host_bits_of_bf16(pb.value()) == b, "LIFO contents");
+                }
+            }
+        }
+        {   // push_when_full_errors, clear_invalidates_handles, argument checks
+            auto pr = ActivationOffloadPool::create(1, 512, OffloadCompression::None);
+            if (pr.ok()) {
+                auto& pool = *pr.value();
+                Tensor a = dev_bf16(std::vector<uint16_t>(8, f2bf(1.f)), {8}), b = dev_bf16(std::vector<uint16_t>(8, f2bf(2.f)), {8});
+                auto ha = pool.push(a);
+                auto hb = pool.push(b);
+                CHECK(ha.ok() && !hb.ok() && hb.error().kind == Error::InvalidOperation, "second push into a 1-slot pool must fail");
+                pool.clear();
+                CHECK(pool.in_flight() == 0, "clear frees the slots");
+                CHECK(ha.ok() && !pool.pull(ha.value()).ok(), "pull after clear must fail");
+                Tensor big = Tensor::empty({512}, DType::BF16).value();
+                auto hbig = pool.push(big);
+                CHECK(!hbig.ok() && hbig.error().kind == Error::InvalidInput, "tensor larger than a slot");
+                Tensor u8 = Tensor::empty({16}, DType::U8).value();
+                auto hu = pool.push(u8);
+                CHECK(!hu.ok() && hu.error().kind == Error::Unsupported, "dtype other than BF16/F32");
+                std::vector<float> f = {1.5f, -2.25f, 3.0f};
+                Tensor tf = Tensor::from_host(f.data(), {3}, DType::F32).value();
+                auto hf = pool.push(tf);
+                CHECK(hf.ok(), "F32 is taken without compression");
+                if (hf.ok()) {
+                    auto bf = pool.pull(hf.value());
+                    std::vector<float> g(3);
+                    CHECK(bf.ok() && bf.value().to_host(g.data()).ok() && g == f, "F32 round trip");
+                }
+            }
+            CHECK(!ActivationOffloadPool::create(0, 16, OffloadCompression::None).ok() &&
+                      !ActivationOffloadPool::create(1, 0, OffloadCompression::None).ok(), "empty pools are refused");
+        }
+        {   // FP8: half the host bytes, values on the E4M3 grid of scale 8/448 round-trip exactly, others within 2^-4
+            auto pr = ActivationOffloadPool::create(2, 4096, OffloadCompression::FP8);
+            CHECK(pr.ok(), "FP8 pool");
+            if (pr.ok()) {
+                auto& pool = *pr.value();
+                CHECK(pool.host_bytes() == 4096, "FP8 pool holds half the bytes");
+                // powers of two times 56 are 1.75 2^k: on the E4M3 grid, so they come back exactly
+                std::vector<uint16_t> grid;
+                for (float x : {0.0f, 1.0f, -0.5f, 0.25f, 2.0f, -4.0f, 0.03125f, -0.0009765625f}) grid.push_back(f2bf(x));
+                {
+                    Tensor tg = dev_bf16(grid, {8});
+                    auto hg = pool.push(tg);
+                    CHECK(hg.ok(), "FP8 push of grid values");
+                    if (hg.ok()) {
+                        auto bg = pool.pull(hg.value());
+                        CHECK(bg.ok() && host_bits_of_bf16(bg.value()) == grid, "values on the FP8 grid must round-trip exactly");
+                    }
+                }
+                std::vector<uint16_t> src = randn_bf16(2048);
+                Tensor t = dev_bf16(src, {16, 128});
+                auto h = pool.push(t);
+                CHECK(h.ok(), "FP8 push");
+                if (h.ok()) {
+                    auto back = pool.pull(h.value());
+                    CHECK(back.ok(), "FP8 pull");
+                    if (back.ok()) {
+                        auto got = host_f32_of_bf16(back.value());
+                        double worst = 0;
+                        for (size_t i = 0; i < src.size(); ++i) {
+                            const float x = bf2f(src[i]);
+                            if (std::fabs(x) >= 4.5f) continue;            // beyond 32/7 the reference's encoder saturates
+                            worst = std::fmax(worst, std::fabs(got[i] - x) - std::fabs(x) / 16.0);
+                        }
+                        CHECK(worst <= 3.6e-5, "FP8 round trip error beyond 2^-4 relative + one subnormal step: %.3e", worst);
+                    }
+                }
+                std::vector<float> f = {1.f, 2.f};
+                Tensor tf = Tensor::from_host(f.data(), {2}, DType::F32).value();
+                auto hf = pool.push(tf);
+                CHECK(!hf.ok() && hf.error().kind == Error::Unsupported && pool.in_flight() == 0, "FP8 pool takes BF16 only");
+            }
+        }
+        {   // the saved set of an attention call leaves the device and comes back for the backward
+            const int B = 1, H = 2, S = 192, D = 64;
+            Tensor q = dev_bf16(randn_bf16((size_t)B * H * S * D), {B, H, S, D});
+            Tensor k = dev_bf16(randn_bf16((size_t)B * H * S * D), {B, H, S, D});
+            Tensor v = dev_bf16(randn_bf16((size_t)B * H * S * D), {B, H, S, D});
+            Tensor go = dev_bf16(randn_bf16((size_t)B * H * S * D), {B, H, S, D});
+            autograd_v4::SdpaConfig cfg;
+            cfg.causal = true;
+            auto f = autograd_v4::sdpa_forward(q, k, v, nullptr, cfg);
+            CHECK(f.ok(), "forward for the offload test");
+            if (f.ok()) {
+                auto g0 = autograd_v4::sdpa_backward(f.value().second, go);
+                auto pr = ActivationOffloadPool::create(4, (size_t)B * H * S * D * 2, OffloadCompression::None);
+                CHECK(pr.ok() && g0.ok(), "pool for the saved set");
+                if (pr.ok() && g0.ok()) {
+                    auto off = autograd_v4::offload_saved(f.value().second, *pr.value());
+                    CHECK(off.ok() && pr.value()->in_flight() == 4 && !off.value().rest.q.defined() && off.value().rest.lse.defined(),
+                          "Q, K, V, O offloaded, LSE resident");
+                    if (off.ok()) {
+                        auto ctx = autograd_v4::restore_saved(off.value(), *pr.value());
+                        CHECK(ctx.ok() && pr.value()->in_flight() == 0, "restore");
+                        if (ctx.ok()) {
+                            auto g1 = autograd_v4::sdpa_backward(ctx.value(), go);
+                            CHECK(g1.ok() && host_bits_of_bf16(std::get<0>(g1.value())) == host_bits_of_bf16(std::get<0>(g0.value())) &&
+                                      host_bits_of_bf16(std::get<1>(g1.value())) == host_bits_of_bf16(std::get<1>(g0.value())) &&
+                                      host_bits_of_bf16(std::get<2>(g1.value())) == host_bits_of_bf16(std::get<2>(g0.value())),
+                                  "gradients from the restored saved set differ");
+                        }
+                    }
+                    auto small = ActivationOffloadPool::create(2, (size_t)B * H * S * D * 2, OffloadCompression::None);
+                    if (small.ok()) {
+                        auto off2 = autograd_v4::offload_saved(f.value().second, *small.value());
+                        CHECK(!off2.ok() && small.value()->in_flight() == 0, "a pool with too few slots refuses and gives its slots back");
+                    }
+                }
+            }
+        }
+    }
+
     if (hipDeviceSynchronize() != hipSuccess) ++g_fail;
     std::printf(g_fail ? "HOST API TEST: %d FAILURES\n" : "HOST API TEST: all checks passed\n", g_fail);
     return g_fail ? 1 : 0;
