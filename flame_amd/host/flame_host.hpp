@@ -1004,21 +1004,145 @@ inline Result<Tensor> sdpa_stream_bf16(const Tensor& q, const Tensor& k, const T
     }
     return out;
 }
+
+// src/cuda_ops_bf16.rs:49-52, :1686-1695: the reference lets the caller bring the device scratch of its host-looped
+// kernels (fp32 logits of one chunk and running rows).  The fused forward keeps those in registers and LDS: a
+// workspace is accepted, checked for consistency and left untouched.
+struct SdpaWorkspace {
+    void* ptr = nullptr;
+    uint64_t bytes = 0;
+};
+inline Result<Tensor> sdpa_stream_bf16_with_workspace(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor* mask, size_t chunk,
+                                                      bool causal, std::optional<float> scale, std::optional<SdpaWorkspace> workspace) {
+    if (workspace && workspace->bytes > 0 && !workspace->ptr) return invalid("sdpa_stream_bf16: workspace pointer is null");
+    return sdpa_stream_bf16(q, k, v, mask, chunk, causal, scale);
+}
 }  // namespace cuda_ops_bf16
 
 namespace ops {
 namespace attn {
-struct StreamingAttnCfg {
+// src/ops/attn.rs.  The reference plans a query chunk whose fp32 scratch (chunk x K logits + chunk x (Dv + 2) rows,
+// :72-84) fits a budget taken from free device memory, and steps down a list of candidate chunks when the planner or
+// an allocation refuses one, recording every step.  The planner, its candidates, its budget rules and its records are
+// mirrored; the scratch the kernels here need is zero bytes, so the requested chunk (clamped as there) is always the
+// chosen one and the list of fallbacks stays empty unless the launch itself fails.
+struct StreamingAttnCfg {                                     // :8-25
     float scale = 1.0f;
     size_t chunk_size = 2048;
     bool causal = false;
     const Tensor* mask = nullptr;
 };
+
+constexpr size_t STREAM_ATTENTION_MIN_CHUNK = 32, STREAM_ATTENTION_MAX_CHUNK = 2048;                  // :113-119
+constexpr uint64_t STREAM_ATTENTION_MIN_BUDGET_BYTES = 64ull << 20, STREAM_ATTENTION_DEFAULT_BUDGET_BYTES = 512ull << 20,
+                   STREAM_ATTENTION_HARD_CAP_BYTES = 2ull << 30;
+
+// what the reference's kernels would need for this chunk (:72-84); nullopt on overflow
+inline std::optional<uint64_t> reference_streaming_workspace_bytes(size_t chunk_rows, size_t k_len, size_t dv) {
+    if (chunk_rows == 0 || k_len == 0) return 0;
+    unsigned __int128 total = (unsigned __int128)chunk_rows * k_len + (unsigned __int128)chunk_rows * ((unsigned __int128)dv + 2);
+    total *= 4;
+    if (total > UINT64_MAX) return std::nullopt;
+    return (uint64_t)total;
+}
+// scratch of the kernels behind this header
+inline uint64_t streaming_workspace_bytes(size_t, size_t, size_t) { return 0; }
+
+inline std::vector<size_t> streaming_chunk_candidates(size_t q_len) {                                   // :128-155
+    static const size_t preferred[13] = {2048, 1536, 1024, 768, 512, 384, 256, 192, 128, 96, 64, 48, 32};
+    std::vector<size_t> c;
+    if (q_len == 0) return c;
+    for (size_t p : preferred) {
+        const size_t cand = std::min(p, q_len);
+        if (cand < STREAM_ATTENTION_MIN_CHUNK && q_len >= STREAM_ATTENTION_MIN_CHUNK) continue;
+        if (std::find(c.begin(), c.end(), cand) == c.end()) c.push_back(cand);
+    }
+    if (c.empty()) c.push_back(std::max<size_t>(q_len, 1));
+    std::sort(c.begin(), c.end(), std::greater<size_t>());
+    return c;
+}
+
+struct StreamingTilePlan {                                    // :121-126
+    size_t chunk = 1;
+    uint64_t workspace_bytes = 0, budget_bytes = 0;
+};
+inline Result<StreamingTilePlan> plan_streaming_chunk(size_t q_len, size_t k_len, size_t dv) {           // :157-209
+    if (q_len == 0 || k_len == 0 || dv == 0) return StreamingTilePlan{std::max<size_t>(q_len, 1), 0, 0};
+    uint64_t budget;
+    const char* forced = std::getenv("FLAME_SDPA_PLANNER_BUDGET_BYTES");
+    char* end = nullptr;
+    const unsigned long long forced_v = forced ? std::strtoull(forced, &end, 10) : 0;
+    if (forced && end != forced && *end == 0) {
+        budget = forced_v;
+    } else {
+        size_t free_b = 0, total_b = 0;
+        if (hipMemGetInfo(&free_b, &total_b) != hipSuccess) free_b = 0;
+        budget = free_b > 0 ? (uint64_t)((double)free_b * 0.75) : STREAM_ATTENTION_DEFAULT_BUDGET_BYTES;
+        budget = std::max(budget, STREAM_ATTENTION_MIN_BUDGET_BYTES);
+    }
+    budget = std::min(budget, STREAM_ATTENTION_HARD_CAP_BYTES);
+    for (size_t chunk : streaming_chunk_candidates(q_len)) {
+        const uint64_t required = streaming_workspace_bytes(std::min(chunk, q_len), k_len, dv);
+        if (required <= budget) return StreamingTilePlan{chunk, required, budget};
+    }
+    return Error{Error::Cuda, "streaming attention planner: no chunk fits the budget (OOM)"};
+}
+
+struct StreamingFallbackReason {                              // :211-223
+    enum Kind { Oom, WorkspaceBudget } kind = Oom;
+    int error_code = -1;
+    std::optional<uint64_t> required_bytes, budget_bytes;
+};
+struct StreamingFallbackEvent {                               // :225-230
+    size_t from_chunk = 0, to_chunk = 0;
+    StreamingFallbackReason reason;
+};
+struct StreamingAttnLaunchInfo {                              // :232-239
+    size_t requested_chunk = 0;
+    std::optional<size_t> chosen_chunk;
+    size_t retries = 0;
+    std::vector<StreamingFallbackEvent> fallbacks;
+    std::optional<int> last_error;
+};
+namespace detail_launch {
+inline std::mutex& guard() {
+    static std::mutex m;
+    return m;
+}
+inline StreamingAttnLaunchInfo& last() {
+    static StreamingAttnLaunchInfo info;
+    return info;
+}
+inline void record(const StreamingAttnLaunchInfo& info) {
+    std::lock_guard<std::mutex> lk(guard());
+    last() = info;
+}
+}  // namespace detail_launch
+inline StreamingAttnLaunchInfo streaming_attn_last_launch_info() {                                       // :318-323
+    std::lock_guard<std::mutex> lk(detail_launch::guard());
+    return detail_launch::last();
+}
+
+// :326-600.  Beyond the reference: a keep-mask is taken (the reference refuses one, :366-370), and the three
+// tensors may be strided views and have key lengths of their own.
 inline Result<Tensor> streaming_attn_bf16_fp32(const Tensor& q, const Tensor& k, const Tensor& v, const StreamingAttnCfg& cfg) {
     if (cfg.chunk_size == 0) return invalid("streaming attention chunk_size must be > 0");
     if (q.dtype() != DType::BF16 || k.dtype() != DType::BF16 || v.dtype() != DType::BF16)
         return invalid("streaming attention expects BF16 tensors");
-    return flame::sdpa::forward_v4(q, k, v, cfg.mask, cfg.causal, cfg.scale);
+    if (q.shape().size() != 4 || k.shape().size() != 4 || v.shape().size() != 4) return invalid("expected 4D tensors");
+    if (q.shape()[3] != k.shape()[3]) return invalid("head dimensions for Q and K differ");
+    const size_t s = (size_t)q.shape()[2], s_k = (size_t)k.shape()[2], dv = (size_t)v.shape()[3];
+    auto plan = plan_streaming_chunk(s, s_k, dv);
+    if (!plan.ok()) return plan.error();
+    const size_t requested = std::min(std::min(std::max<size_t>(cfg.chunk_size, 1), std::max<size_t>(s, 1)), STREAM_ATTENTION_MAX_CHUNK);
+    if (streaming_workspace_bytes(std::min(requested, s), s_k, dv) <= plan.value().budget_bytes) plan.value().chunk = requested;
+    StreamingAttnLaunchInfo info;
+    info.requested_chunk = std::max<size_t>(requested, 1);
+    auto out = cuda_ops_bf16::sdpa_stream_bf16_with_workspace(q, k, v, cfg.mask, plan.value().chunk, cfg.causal, cfg.scale, std::nullopt);
+    info.chosen_chunk = plan.value().chunk;
+    if (!out.ok()) info.last_error = out.error().kind == Error::Cuda ? 2 : 1;        // FC_ERR_LAUNCH / FC_ERR_INVALID_ARGUMENT
+    detail_launch::record(info);
+    return out;
 }
 }  // namespace attn
 }  // namespace ops

@@ -529,6 +529,40 @@ int main() {
         auto so2 = cuda_ops_bf16::sdpa_stream_bf16(q, k, v, nullptr, 1024, true, 0.125f);
         CHECK(so.ok() && so2.ok(), "streaming wrappers failed");
         if (so.ok() && so2.ok()) CHECK(host_f32_of_bf16(so.value()) == host_f32_of_bf16(so2.value()), "streaming wrappers disagree");
+        {   // launch record, planner and candidates (src/ops/attn.rs:128-209, :232-239, :318-323)
+            auto info = ops::attn::streaming_attn_last_launch_info();
+            CHECK(info.requested_chunk == std::min<size_t>(2048, (size_t)Sq) && info.chosen_chunk && *info.chosen_chunk == info.requested_chunk &&
+                      info.retries == 0 && info.fallbacks.empty() && !info.last_error,
+                  "launch info after a plain call");
+            cfg.chunk_size = 48;
+            CHECK(ops::attn::streaming_attn_bf16_fp32(q, k, v, cfg).ok(), "small chunk");
+            info = ops::attn::streaming_attn_last_launch_info();
+            CHECK(info.requested_chunk == std::min<size_t>(48, (size_t)Sq) && info.chosen_chunk && *info.chosen_chunk == info.requested_chunk,
+                  "the requested chunk is the chosen one: the kernels need no scratch");
+            using ops::attn::streaming_chunk_candidates;
+            CHECK(streaming_chunk_candidates(0).empty(), "no candidates for an empty sequence");
+            CHECK(streaming_chunk_candidates(20) == std::vector<size_t>({20}), "short sequences: the sequence itself");
+            CHECK(streaming_chunk_candidates(100) == std::vector<size_t>({100, 96, 64, 48, 32}), "candidates below 100");
+            CHECK(streaming_chunk_candidates(5000).size() == 13 && streaming_chunk_candidates(5000).front() == 2048 &&
+                      streaming_chunk_candidates(5000).back() == 32, "all thirteen preferred chunks");
+            auto plan = ops::attn::plan_streaming_chunk(4608, 4608, 128);
+            CHECK(plan.ok() && plan.value().chunk == 2048 && plan.value().workspace_bytes == 0 &&
+                      plan.value().budget_bytes >= (64ull << 20) && plan.value().budget_bytes <= (2ull << 30),
+                  "planner: largest candidate, budget between the reference's floor and cap");
+            setenv("FLAME_SDPA_PLANNER_BUDGET_BYTES", "12345", 1);
+            auto forced = ops::attn::plan_streaming_chunk(4608, 4608, 128);
+            unsetenv("FLAME_SDPA_PLANNER_BUDGET_BYTES");
+            CHECK(forced.ok() && forced.value().budget_bytes == 12345, "forced planner budget");
+            CHECK(ops::attn::reference_streaming_workspace_bytes(2048, 4608, 128).value_or(0) == (2048ull * 4608 + 2048ull * 130) * 4,
+                  "the reference's scratch formula");
+            cuda_ops_bf16::SdpaWorkspace ws;
+            ws.bytes = 16;
+            CHECK(!cuda_ops_bf16::sdpa_stream_bf16_with_workspace(q, k, v, nullptr, 64, true, 0.125f, ws).ok(), "null workspace with bytes");
+            ws.ptr = q.data();
+            auto so3 = cuda_ops_bf16::sdpa_stream_bf16_with_workspace(q, k, v, nullptr, 64, true, 0.125f, ws);
+            CHECK(so3.ok() && so2.ok() && host_bits_of_bf16(so3.value()) == host_bits_of_bf16(so2.value()), "workspace variant");
+            CHECK(host_bits_of_bf16(q) == hq, "workspace memory is left untouched");
+        }
         cfg.chunk_size = 0;
         CHECK(!ops::attn::streaming_attn_bf16_fp32(q, k, v, cfg).ok(), "chunk_size 0 must be refused");
     }
