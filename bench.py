@@ -360,14 +360,14 @@ def main():
     capi.lib()      # fails loudly when the HIP library is missing
 
     dev = torch.device("cuda:0")
-    if args.tile_ops:
-        return tile_ops_line(args, capi, torch, dev)
-    w = W.CONFIGS[args.config]()
-    B, H, Sq, Sk, D = w.shape
     if args.traffic_calibration:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
         torch.empty_like(src).copy_(src)          # one elementwise copy kernel: reads 256 MiB, writes 256 MiB
         del src
+    if args.tile_ops:
+        return tile_ops_line(args, capi, torch, dev)
+    w = W.CONFIGS[args.config]()
+    B, H, Sq, Sk, D = w.shape
     if w.do is None:            # inference-only workload (int8-QK forward)
         return sage_line(args, capi, torch, w, dev)
 
