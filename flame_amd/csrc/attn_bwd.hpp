@@ -545,12 +545,14 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
                 const int g = PHASE * NS + i;
                 if constexpr (PHASE < 2) {      // S = Q K^T and dP = dO V^T - delta, rows = queries of block qb, columns = this wave's keys
                     const int qb = PHASE, dc = i >> 1;
-                    mfma32_vgpr_bacc(dpacc[qb], fb[(g + 1) % PD], vf[dc]);
+                    // the dropout builds: the allocator splits the accumulators around the longer element arithmetic
+                    // and moves parts of them back right before these statements
+                    mfma32_vgpr_bacc<DROPOUT>(dpacc[qb], fb[(g + 1) % PD], vf[dc]);
                     side(g);
                     __builtin_amdgcn_sched_barrier(0);
                     copy_dst(g + 1);
-                    if (i == 0) mfma32_vgpr_first_bacc(sacc[qb], fb[g % PD], kf[dc]);
-                    else mfma32_vgpr_bacc(sacc[qb], fb[g % PD], kf[dc]);
+                    if (i == 0) mfma32_vgpr_first_bacc<DROPOUT>(sacc[qb], fb[g % PD], kf[dc]);
+                    else mfma32_vgpr_bacc<DROPOUT>(sacc[qb], fb[g % PD], kf[dc]);
                     side(g + 1);
                 } else {              // dV^T += dO^T P, dK^T += Q^T dS: rows = d, columns = keys, contraction over queries
                     const int qb = PHASE - 2, c = i / (2 * DB), db = (i >> 1) % DB;

@@ -44,17 +44,27 @@ __device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
 // instruction that touches it (the result of an 8-pass MFMA is visible 11 issue cycles after issue).
 // The B operand is held in the accumulation registers: operands that live for a whole kernel (a
 // workgroup's own K / V fragments) then cost no architectural VGPRs.
+// GUARD: two wait states in front, for kernel variants in which the register allocator moves an operand (part of an
+// accumulator it has split, a fragment) into place right before the statement: an MFMA may read a register the vector
+// ALU wrote two wait states later at the earliest, and the compiler keeps that distance only for its own MFMAs.
+template <bool GUARD = false>
 __device__ __forceinline__ void mfma32_vgpr_first_bacc(f32x16& acc, bf16x8 a, bf16x8 b) {
-    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(acc) : "v"(a), "a"(b));
+    if constexpr (GUARD) asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(acc) : "v"(a), "a"(b));
+    else asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(acc) : "v"(a), "a"(b));
 }
+template <bool GUARD = false>
 __device__ __forceinline__ void mfma32_vgpr_bacc(f32x16& acc, bf16x8 a, bf16x8 b) {
-    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "a"(b));
+    if constexpr (GUARD) asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "a"(b));
+    else asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "a"(b));
 }
 // Both operands in architectural registers (a kernel whose B fragments are too many for the accumulation file's
 // free part).  After the last MFMA of a chain, mfma32_vgpr_settle spends the 11 wait states before its result may be
 // read, for kernels that have no other MFMAs to put there.
+// The two wait states in front: an operand the register allocator moved into place just before the statement was
+// written by the vector ALU, and an MFMA may read such a register two wait states later at the earliest (the compiler
+// keeps that distance for its own MFMAs, not for these).
 __device__ __forceinline__ void mfma32_vgpr(f32x16& acc, bf16x8 a, bf16x8 b) {
-    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
+    asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
 }
 __device__ __forceinline__ void mfma32_vgpr_settle(f32x16& acc) {
     asm volatile("s_nop 11" : "+v"(acc));
@@ -227,17 +237,16 @@ __device__ __forceinline__ void rescale_pinned(f32x16& acc, float alpha) {
 // acc += a b with the accumulator pinned to a[16 IDX : 16 IDX + 15] (the tuples rescale_pinned works on) and both
 // operands in architectural registers, emitted by hand: given the same fixed registers at every use, the accumulator
 // never moves (left to the compiler's MFMA form, accumulators that a conditional rescale also touches travelled
-// through architectural registers once per key tile).  FRESH_B: the B operand was just written by the vector ALU, which
-// needs two wait states before an MFMA reads it.  mfma32_apinned_settle<IDX, WAIT> is the fence before the
+// through architectural registers once per key tile).  Two wait states in front, as in mfma32_vgpr: the B operand may
+// have been written, or moved into place, by the vector ALU just before.  mfma32_apinned_settle<IDX, WAIT> is the fence before the
 // accumulators are read after the last tile: the one with WAIT spends the 11 wait states, and since volatile
 // statements keep their order, fencing every accumulator after it orders all their reads behind that wait.
-template <int IDX, bool FRESH_B>
+template <int IDX>
 __device__ __forceinline__ void mfma32_apinned(f32x16& acc, bf16x8 a, bf16x8 b) {
     static_assert(IDX >= 0 && IDX < 8, "eight pinned accumulator tuples");
 #define FATTN_PIN(I, R)                                                                                        \
     if constexpr (IDX == I) {                                                                                  \
-        if constexpr (FRESH_B) asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : R(acc) : "v"(a), "v"(b)); \
-        else asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : R(acc) : "v"(a), "v"(b));                \
+        asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : R(acc) : "v"(a), "v"(b));          \
     }
     FATTN_PIN(0, "+{a[0:15]}")
     FATTN_PIN(1, "+{a[16:31]}")

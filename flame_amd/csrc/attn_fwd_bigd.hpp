@@ -9,12 +9,20 @@
 //     so two wavefronts share 32 queries: both form the same S^T and P^T, and each accumulates one half of the
 //     output head dim (two of the four 32-wide column blocks of every chunk): 64 queries per workgroup, 1.5x the
 //     MFMA work of the unsplit form instead of register spills in the inner loop;
-//   * 32-key tiles (K and V: 8 KiB per chunk each), two LDS stages, the copies of tile t+1 in flight while tile t
-//     is computed, one workgroup barrier per tile; inside a tile the LDS fragments are read one chunk ahead of the
-//     MFMAs that use them;
+//     NW = wavefronts per workgroup; the library launches NW = 4 only: a wavefront's time does not depend on how
+//     many share its K/V tiles, so smaller workgroups make nothing faster (measured: a single D = 512 head of 4096
+//     positions 0.234 ms with NW = 4, 0.273 ms with NW = 2, which issues twice the copies per wavefront);
+//   * 32-key tiles (K and V: 8 KiB per chunk each), two LDS stages of K and two of V, one workgroup barrier per tile;
+//   * a software pipeline one tile deep: step t = [S^T of tile t+1, with the copies of V(t+1) and K(t+2) issued
+//     between its MFMAs] [PV of tile t, with the softmax of tile t+1 (maximum, exponentials, bf16 packing) threaded
+//     between its MFMAs] [the rare rescale of O^T].  LDS fragments are read one chunk ahead of the MFMAs that use
+//     them (one wavefront per SIMD: nothing else hides the latency);
 //   * S^T accumulates in architectural registers and O^T in accumulation registers pinned to a[0:127], both emitted
 //     by hand: a kernel whose accumulators a conditional rescale also touches otherwise moves them through
-//     architectural registers every tile.
+//     architectural registers every tile.  The Q fragments of the first two chunks are pinned to a[128:191]: left
+//     unpinned, the register allocator moved them into place before each use, and a hand-emitted MFMA directly
+//     behind such a move read the old contents (the compiler spaces its own MFMAs two wait states from a vector-ALU
+//     write of their operands; the hand-emitted forms used here carry those wait states themselves).
 // Exclusions: causal flag, key lengths, ragged last tile.  Head dims that are not a multiple of 128 are zero-padded
 // on the way in (as in the other kernels) and not stored on the way out.
 #pragma once
@@ -22,19 +30,20 @@
 
 namespace fattn {
 
-template <int NC, bool SPLIT>
+template <int NC, bool SPLIT, int NW>
 struct FwdBigDTile {
-    static constexpr int BM = SPLIT ? 64 : 128, BN = 32;
+    static_assert(NW == 4 || NW == 2 || (NW == 1 && !SPLIT), "wavefronts per workgroup (the library launches 4)");
+    static constexpr int BM = (SPLIT ? 16 : 32) * NW, BN = 32;
     static constexpr int NDB = SPLIT ? 2 : 4;                  // 32-wide output column blocks per chunk and wavefront
     static constexpr int SUB_ELEMS = BN * 128;                 // one chunk of one tensor: 32 rows x 128
-    static constexpr int STAGE_ELEMS = 2 * NC * SUB_ELEMS;     // K chunks, then V chunks
-    static constexpr int LDS_BYTES = 2 * STAGE_ELEMS * 2;
-    static constexpr int COPIES_PER_WAVE = NC * 8 / 4;         // 1 KiB copies (4 rows of one chunk) per tensor and wave
+    static constexpr int TENSOR_STAGE_ELEMS = NC * SUB_ELEMS;  // one tile of K or of V
+    static constexpr int LDS_BYTES = 4 * TENSOR_STAGE_ELEMS * 2; // two stages of K, two of V
+    static constexpr int COPIES_PER_WAVE = NC * 8 / NW;        // 1 KiB copies (4 rows of one chunk) per tensor and wave
 };
 
-template <int NC, bool SPLIT>
-__global__ __launch_bounds__(256) void fwd_bigd_kernel(const FwdParams p) {
-    using T = FwdBigDTile<NC, SPLIT>;
+template <int NC, bool SPLIT, int NW>
+__global__ __launch_bounds__(64 * NW) void fwd_bigd_kernel(const FwdParams p) {
+    using T = FwdBigDTile<NC, SPLIT, NW>;
     constexpr int BN = T::BN, BM = T::BM, NDB = T::NDB;
     constexpr int NCP = T::COPIES_PER_WAVE;
 
@@ -71,41 +80,46 @@ __global__ __launch_bounds__(256) void fwd_bigd_kernel(const FwdParams p) {
     {
         const bool ok = qi < p.Sq;
         const uint16_t* rp = qbase + (int64_t)qi * p.qs.n + 8 * h;
-#pragma unroll
-        for (int c = 0; c < NC; ++c)
-#pragma unroll
-            for (int dc = 0; dc < 8; ++dc)
-                qf[c][dc] = __builtin_bit_cast(bf16x8, ldg16(rp + 128 * c + 16 * dc, ok && 128 * c + 16 * dc + 8 * h < p.d));
+        // the fragments of the first two chunks are pinned to accumulation registers a[128:191] (beside O^T in
+        // a[0:127]); left to the register allocator they are moved into place before every use, and a hand-emitted
+        // MFMA right behind such a move reads the old contents
+        static_for<NC * 8>([&](auto i_tag) {
+            constexpr int i = decltype(i_tag)::value;
+            constexpr int c = i / 8, dc = i % 8;
+            const u32x4 w = ldg16(rp + 128 * c + 16 * dc, ok && 128 * c + 16 * dc + 8 * h < p.d);
+            if constexpr (c < 2) qf[c][dc] = pin_b_fragment<i>(w);
+            else qf[c][dc] = __builtin_bit_cast(bf16x8, w);
+        });
     }
 
     // ---- tile copies: copy j of a wavefront moves 4 rows of one chunk (1 KiB); lane = (row in copy, physical granule).
     //      Source = wave-uniform address of the tile + a 32-bit per-lane byte offset (rows past the attended range
     //      re-read the last attended key; row strides are below 2^24 elements, so 31 rows fit).  The offsets are formed
-    //      again for every tile from two lane constants: kept per copy across the loop they would take 4 NC registers
-    //      that the Q fragments and O^T need (a spill reload in the loop waits on vmcnt, that is, on the copies).
+    //      again for every copy from two lane constants: kept per copy across the loop they would take 4 NC registers
+    //      that the Q fragments and O^T need (a spill reload in the loop waits on vmcnt, that is, on the copies), and
+    //      made opaque per copy they stay where they are written: between the MFMAs of the logit phase.
+    //      LDS: K stages 0 and 1, then V stages 0 and 1 (tile t in stage t & 1 of its tensor).
     const uint32_t lds0 = lds_addr(lds);
     const int cp_row_in = lane >> 4;
     const int cp_gl = (lane & 15) ^ (cp_row_in << 2);            // physical granule ^ the lane's part of the swizzle
-    auto issue_tile = [&](int t) {
-        const uint32_t stage = lds0 + 2u * (uint32_t)((t & 1) * T::STAGE_ELEMS);
-        const uint16_t* kt = kbase + (int64_t)t * BN * p.ks.n;
-        const uint16_t* vt = vbase + (int64_t)t * BN * p.vs.n;
-        const int rmax = klimit - 1 - t * BN;                    // >= 0 for every tile of the loop
+    auto issue_copy = [&](auto which_tag, int t, int j) {        // which: 0 = K, 1 = V
+        constexpr int which = decltype(which_tag)::value;
+        const int64_t row_stride = which ? p.vs.n : p.ks.n;
+        const uint16_t* tb = (which ? vbase : kbase) + (int64_t)t * BN * row_stride;
+        const int rmax = klimit - 1 - t * BN;                    // >= 0 for every tile that is copied
         int row_in = cp_row_in, gl = cp_gl;
-        asm volatile("" : "+v"(row_in), "+v"(gl));               // opaque: nothing below is hoisted out of the key loop
-#pragma unroll
-        for (int j = 0; j < NCP; ++j) {
-            const int cj = wave * NCP + j;                       // 0 .. 8 NC - 1, wave-uniform
-            const int chunk = cj >> 3;
-            const int row = min(4 * (cj & 7) + row_in, rmax);
-            const int g = gl ^ (cj & 3);                         // logical granule: swz<128>(row) = (row & 3) << 2 | (row >> 2) & 3
-            int dk = 128 * chunk + 8 * g;
-            dk = dk < p.d ? dk : 0;                              // p.dv == p.d in this kernel
-            const uint32_t dst = stage + 2u * (uint32_t)(chunk * T::SUB_ELEMS + (cj & 7) * 512);
-            dma16u(kt, 2u * (uint32_t)(row * (int)p.ks.n + dk), dst);
-            dma16u(vt, 2u * (uint32_t)(row * (int)p.vs.n + dk), dst + 2u * (uint32_t)(NC * T::SUB_ELEMS));
-        }
+        asm volatile("" : "+v"(row_in), "+v"(gl));
+        const int cj = wave * NCP + j;                           // 0 .. 8 NC - 1, wave-uniform
+        const int chunk = cj >> 3;
+        const int row = min(4 * (cj & 7) + row_in, rmax);
+        const int g = gl ^ (cj & 3);                             // logical granule: swz<128>(row) = (row & 3) << 2 | (row >> 2) & 3
+        int dk = 128 * chunk + 8 * g;
+        dk = dk < p.d ? dk : 0;                                  // p.dv == p.d in this kernel
+        const uint32_t dst = lds0 + 2u * (uint32_t)((2 * which + (t & 1)) * T::TENSOR_STAGE_ELEMS + chunk * T::SUB_ELEMS + (cj & 7) * 512);
+        dma16u(tb, 2u * (uint32_t)(row * (int)row_stride + dk), dst);
     };
+    using KTag = std::integral_constant<int, 0>;
+    using VTag = std::integral_constant<int, 1>;
 
     // ---- per-lane LDS read offsets inside a chunk (elements), as in the 128-wide kernels
     int koff[8];
@@ -132,109 +146,170 @@ __global__ __launch_bounds__(256) void fwd_bigd_kernel(const FwdParams p) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) oacc[c][db][r] = 0.f;
 
-    if (n_tiles > 0) {
-        issue_tile(0);
-        wait_vm0();
-        __syncthreads();
-    }
-    for (int t = 0; t < n_tiles; ++t) {
-        if (t + 1 < n_tiles) issue_tile(t + 1);
-        const uint16_t* ks = lds + (t & 1) * T::STAGE_ELEMS;
-        const uint16_t* vs = ks + NC * T::SUB_ELEMS;
-        // ---- S^T (32 keys x 32 queries) over all chunks
-        //      (emitted by hand with the accumulator in architectural registers: O^T below is pinned to the
-        //      accumulation registers).  The K fragments of chunk c + 1 are read while the MFMAs of chunk c run:
-        //      with one wavefront per SIMD nothing else hides the LDS latency.
-        f32x16 s;
-        {
-            bf16x8 kf[2][8];
-            auto read_k = [&](int c, bf16x8 (&dst)[8]) {
+    // ---- the phases of a tile
+    // S^T (32 keys x 32 queries) of tile t1 over all chunks, emitted by hand with the accumulator in architectural
+    // registers (O^T is pinned to the accumulation registers).  The K fragments of chunk c + 1 are read while the MFMAs
+    // of chunk c run: with one wavefront per SIMD nothing else hides the LDS latency.  COPIES: the copies of V tile t1
+    // and of K tile t1 + 1 are issued between the MFMAs, one (NW = 1: two) per MFMA from the first on.
+    constexpr int CPS = (2 * NCP + 8 * NC - 1) / (8 * NC);       // copies per MFMA slot
+    auto logits = [&](auto copies_tag, int t1, f32x16& s) {
+        constexpr bool COPIES = decltype(copies_tag)::value;
+        const uint16_t* ks = lds + (t1 & 1) * T::TENSOR_STAGE_ELEMS;
+        const bool more_k = t1 + 1 < n_tiles;
+        bf16x8 kf[2][8];
+        auto read_k = [&](int c, bf16x8 (&dst)[8]) {
 #pragma unroll
-                for (int dc = 0; dc < 8; ++dc) dst[dc] = *reinterpret_cast<const bf16x8*>(ks + c * T::SUB_ELEMS + koff[dc]);
-            };
-            read_k(0, kf[0]);
-            static_for<NC>([&](auto c_tag) {
-                constexpr int c = decltype(c_tag)::value;
-                if constexpr (c + 1 < NC) read_k(c + 1, kf[(c + 1) & 1]);
-                __builtin_amdgcn_sched_barrier(0);
+            for (int dc = 0; dc < 8; ++dc) dst[dc] = *reinterpret_cast<const bf16x8*>(ks + c * T::SUB_ELEMS + koff[dc]);
+        };
+        read_k(0, kf[0]);
+        static_for<NC>([&](auto c_tag) {
+            constexpr int c = decltype(c_tag)::value;
+            if constexpr (c + 1 < NC) read_k(c + 1, kf[(c + 1) & 1]);
+            __builtin_amdgcn_sched_barrier(0);
+            static_for<8>([&](auto dc_tag) {
+                constexpr int dc = decltype(dc_tag)::value;
+                // Q fragments of the first two chunks live in the accumulation registers beside O^T (at most
+                // 128 + 64), those of the others in architectural registers
+                if constexpr (c < 2) mfma32_vgpr_bpinned<c * 8 + dc, (c == 0 && dc == 0) ? 0 : 1>(s, kf[c & 1][dc], qf[c][dc], s);
+                else mfma32_vgpr(s, kf[c & 1][dc], qf[c][dc]);
+                if constexpr (COPIES) {
 #pragma unroll
-                for (int dc = 0; dc < 8; ++dc) {
-                    // Q fragments of the first two chunks live in the accumulation registers beside O^T (at most
-                    // 128 + 64), those of the others in architectural registers
-                    if (c == 0 && dc == 0) mfma32_vgpr_first_bacc(s, kf[c & 1][dc], qf[c][dc]);
-                    else if (c < 2) mfma32_vgpr_bacc(s, kf[c & 1][dc], qf[c][dc]);
-                    else mfma32_vgpr(s, kf[c & 1][dc], qf[c][dc]);
+                    for (int u = 0; u < CPS; ++u) {
+                        constexpr int slot = c * 8 + dc;
+                        const int idx = slot * CPS + u;
+                        if (idx < NCP) issue_copy(VTag{}, t1, idx);
+                        else if (idx < 2 * NCP && more_k) issue_copy(KTag{}, t1 + 1, idx - NCP);
+                    }
                 }
-                __builtin_amdgcn_sched_barrier(0);
             });
+            __builtin_amdgcn_sched_barrier(0);
+        });
+    };
+    // Exclusions and the running maximum of tile t1; returns each lane's factor for the accumulated O^T and sets
+    // `rescale` (wave-uniform) when some lane's is not 1: the reference maximum may lag the true one by 2^8.
+    auto fold_max = [&](int t1, f32x16& s, bool& rescale) -> float {
+        const bool edge = (t1 + 1) * BN > klimit || (p.m.causal && (t1 + 1) * BN > qw0 + 1);
+        if (edge) {
+            const int key_limit = p.m.causal ? min(klimit, qi + 1) : klimit;      // keys below it are attended
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s[r] = t1 * BN + acc_row(r, h) >= key_limit ? -INFINITY : s[r];
         }
-        mfma32_vgpr_settle(s);
-        // ---- exclusions and the tile maximum
-        const bool edge = (t + 1) * BN > klimit || (p.m.causal && (t + 1) * BN > qw0 + 1);
         float tmax = -INFINITY;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            if (edge) {
-                const int key = t * BN + acc_row(r, h);
-                const bool drop = (key >= klimit) | ((p.m.causal != 0) & (key > qi));
-                s[r] = drop ? -INFINITY : s[r];
-            }
-            tmax = fmaxf(tmax, s[r]);
-        }
+        for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, s[r]);
+        asm volatile("" : "+v"(tmax));       // the scan stays in its slot
         tmax = fmaxf(tmax, xhalf(tmax));
-        if (__any(tmax > m_run + stale_ok)) {
+        float alpha = 1.0f;
+        rescale = __any(tmax > m_run + stale_ok);
+        if (rescale) {
             const float m_new = fmaxf(m_run, tmax);
             const float m_to = (m_new == -INFINITY) ? 0.f : m_new;
-            const float alpha = exp2_fast((m_run - m_to) * c_log2);
+            alpha = exp2_fast((m_run - m_to) * c_log2);
             m_run = m_new;
             l_run *= alpha;
-            static_for<NC * NDB>([&](auto i_tag) {
-                constexpr int i = decltype(i_tag)::value;
-                rescale_pinned<i>(oacc[i / NDB][i % NDB], alpha);
-            });
         }
-        // ---- P^T in the B-operand layout of the second product
-        const float msc = ((m_run == -INFINITY) ? 0.f : m_run) * c_log2;
-        float rsum = 0.f;
+        return alpha;
+    };
+    auto exps = [&](f32x16& s, int lo, int hi, float msc) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            s[r] = exp2_fast(fmaf(s[r], c_log2, -msc));
-            rsum += s[r];
+        for (int r = lo; r < hi; ++r) {
+            float e = exp2_fast(fmaf(s[r], c_log2, -msc));
+            asm volatile("" : "+v"(e));      // computed here, between the MFMAs, not where the compiler would sink it
+            s[r] = e;
+            l_run += e;
         }
-        l_run += rsum;
-        const bf16x8 pf[2] = {pack8(s[0], s[1], s[2], s[3], s[4], s[5], s[6], s[7]),
-                              pack8(s[8], s[9], s[10], s[11], s[12], s[13], s[14], s[15])};
-        // ---- O^T += V^T P^T (accumulators pinned: see mfma32_apinned), V^T fragments read one chunk ahead
-        {
-            bf16x8 vf[2][2 * NDB];
-            auto read_v = [&](int c, bf16x8 (&dst)[2 * NDB]) {
+    };
+    auto rescale_all = [&](float alpha) {
+        static_for<NC * NDB>([&](auto i_tag) {
+            constexpr int i = decltype(i_tag)::value;
+            mfma32_apinned_settle<i, i == 0>(oacc[i / NDB][i % NDB]);
+        });
+        static_for<NC * NDB>([&](auto i_tag) {
+            constexpr int i = decltype(i_tag)::value;
+            rescale_pinned<i>(oacc[i / NDB][i % NDB], alpha);
+        });
+    };
+    // O^T += V^T P^T of tile t (accumulators pinned: see mfma32_apinned), V^T fragments read one chunk ahead.  SOFTMAX:
+    // the softmax of the next tile's logits s is threaded between the MFMAs: nothing for the first two (the logits
+    // were written by hand-emitted MFMAs just before), the maximum after the third, the exponentials after the others,
+    // and the bf16 P^T operands of the next tile come out in pn.
+    constexpr int NM = 2 * NC * NDB;                             // PV MFMAs per tile
+    constexpr int NE = NM - 3;                                   // of which carry exponentials
+    auto pv = [&](auto softmax_tag, int t, const bf16x8 (&pf)[2], f32x16& s, bf16x8 (&pn)[2], float& alpha, bool& rescale) {
+        constexpr bool SOFTMAX = decltype(softmax_tag)::value;
+        const uint16_t* vs = lds + (2 + (t & 1)) * T::TENSOR_STAGE_ELEMS;
+        bf16x8 vf[2][2 * NDB];
+        auto read_v = [&](int c, bf16x8 (&dst)[2 * NDB]) {
 #pragma unroll
-                for (int db = 0; db < NDB; ++db)
+            for (int cc = 0; cc < 2; ++cc)
 #pragma unroll
-                    for (int cc = 0; cc < 2; ++cc) {
-                        const uint16_t* vsub = vs + c * T::SUB_ELEMS + 16 * cc * 128;
-                        const u32x2 lo = lds_read_tr16(vsub + voff[0][db]);
-                        const u32x2 hi = lds_read_tr16(vsub + voff[1][db]);
-                        const u32x4 u = {lo[0], lo[1], hi[0], hi[1]};
-                        dst[2 * db + cc] = __builtin_bit_cast(bf16x8, u);
+                for (int db = 0; db < NDB; ++db) {
+                    const uint16_t* vsub = vs + c * T::SUB_ELEMS + 16 * cc * 128;
+                    const u32x2 lo = lds_read_tr16(vsub + voff[0][db]);
+                    const u32x2 hi = lds_read_tr16(vsub + voff[1][db]);
+                    const u32x4 u = {lo[0], lo[1], hi[0], hi[1]};
+                    dst[cc * NDB + db] = __builtin_bit_cast(bf16x8, u);
+                }
+        };
+        float msc = 0.f;
+        read_v(0, vf[0]);
+        static_for<NC>([&](auto c_tag) {
+            constexpr int c = decltype(c_tag)::value;
+            if constexpr (c + 1 < NC) read_v(c + 1, vf[(c + 1) & 1]);
+            __builtin_amdgcn_sched_barrier(0);
+            static_for<2 * NDB>([&](auto f_tag) {                // 16 keys cc, then column block db: neighbours are independent
+                constexpr int f = decltype(f_tag)::value;
+                constexpr int cc = f / NDB, db = f % NDB, i = c * NDB + db, m = c * 2 * NDB + f;
+                mfma32_apinned<i>(oacc[c][db], vf[c & 1][f], pf[cc]);
+                if constexpr (SOFTMAX) {
+                    if constexpr (m == 2) {
+                        alpha = fold_max(t + 1, s, rescale);
+                        msc = ((m_run == -INFINITY) ? 0.f : m_run) * c_log2;
                     }
-            };
-            read_v(0, vf[0]);
-            static_for<NC>([&](auto c_tag) {
-                constexpr int c = decltype(c_tag)::value;
-                if constexpr (c + 1 < NC) read_v(c + 1, vf[(c + 1) & 1]);
-                __builtin_amdgcn_sched_barrier(0);
-                static_for<NDB>([&](auto db_tag) {
-                    constexpr int db = decltype(db_tag)::value;
-                    constexpr int i = c * NDB + db;
-                    mfma32_apinned<i, i == 0>(oacc[c][db], vf[c & 1][2 * db], pf[0]);
-                    mfma32_apinned<i, i == 0>(oacc[c][db], vf[c & 1][2 * db + 1], pf[1]);
-                });
-                __builtin_amdgcn_sched_barrier(0);
+                    if constexpr (m >= 3) exps(s, ((m - 3) * 16) / NE, ((m - 2) * 16) / NE, msc);
+                    if constexpr (m == NM - 1) {
+                        pn[0] = pack8(s[0], s[1], s[2], s[3], s[4], s[5], s[6], s[7]);
+                        pn[1] = pack8(s[8], s[9], s[10], s[11], s[12], s[13], s[14], s[15]);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             });
+            __builtin_amdgcn_sched_barrier(0);
+        });
+    };
+    using Yes = std::integral_constant<bool, true>;
+    using No = std::integral_constant<bool, false>;
+
+    // ---- the walk over the key tiles.  Tile t's logits and softmax run one step ahead of its PV products: step t is
+    //      [S^T of tile t+1 with the copies of V(t+1) and K(t+2) between its MFMAs] [PV of tile t with the softmax of
+    //      tile t+1 between its MFMAs] [the rare rescale of O^T] [all copies landed, one workgroup barrier].
+    if (n_tiles > 0) {
+        f32x16 s;
+        bf16x8 pf[2], pn[2];
+        float alpha = 1.0f;
+        bool rescale = false;
+        for (int j = 0; j < NCP; ++j) issue_copy(KTag{}, 0, j);
+        for (int j = 0; j < NCP; ++j) issue_copy(VTag{}, 0, j);
+        if (n_tiles > 1)
+            for (int j = 0; j < NCP; ++j) issue_copy(KTag{}, 1, j);
+        wait_vm0();
+        __syncthreads();
+        logits(No{}, 0, s);
+        mfma32_vgpr_settle(s);
+        (void)fold_max(0, s, rescale);                           // nothing accumulated yet: no rescale
+        exps(s, 0, 16, ((m_run == -INFINITY) ? 0.f : m_run) * c_log2);
+        pf[0] = pack8(s[0], s[1], s[2], s[3], s[4], s[5], s[6], s[7]);
+        pf[1] = pack8(s[8], s[9], s[10], s[11], s[12], s[13], s[14], s[15]);
+        for (int t = 0; t + 1 < n_tiles; ++t) {
+            logits(Yes{}, t + 1, s);
+            pv(Yes{}, t, pf, s, pn, alpha, rescale);
+            if (rescale) rescale_all(alpha);
+            pf[0] = pn[0];
+            pf[1] = pn[1];
+            wait_vm0();            // the copies issued in this step have landed ...
+            __syncthreads();       // ... everyone's, and everyone is done with the stages they go to next
         }
-        wait_vm0();            // the copies of tile t+1 have landed ...
-        __syncthreads();       // ... everyone's, and everyone is done reading tile t
+        pv(No{}, n_tiles - 1, pf, s, pn, alpha, rescale);
     }
 
     // ---- epilogue

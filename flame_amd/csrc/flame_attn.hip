@@ -261,12 +261,12 @@ int launch_bwd(const BwdParams& p, hipStream_t s) {
     return e == hipSuccess ? FLAME_ATTN_OK : (int)e;
 }
 
-template <int NC>
-int launch_fwd_bigd(const FwdParams& p, hipStream_t s) {
+template <int NC, int NW>
+int launch_fwd_bigd_nw(const FwdParams& p, hipStream_t s) {
     constexpr bool SPLIT = NC > 2;
-    using T = FwdBigDTile<NC, SPLIT>;
+    using T = FwdBigDTile<NC, SPLIT, NW>;
     static bool attr_done = false;
-    auto kern = fwd_bigd_kernel<NC, SPLIT>;
+    auto kern = fwd_bigd_kernel<NC, SPLIT, NW>;
     if (!attr_done) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS_BYTES);
@@ -277,11 +277,13 @@ int launch_fwd_bigd(const FwdParams& p, hipStream_t s) {
     if (grid > 0x7fffffff) return FLAME_ATTN_ERR_UNSUPPORTED;
     {
         ScopedKernelTimer t(FLAME_ATTN_KERNEL_FWD, s);
-        hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), T::LDS_BYTES, s, p);
+        hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(64 * NW), T::LDS_BYTES, s, p);
     }
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? FLAME_ATTN_OK : (int)e;
 }
+template <int NC>
+int launch_fwd_bigd(const FwdParams& p, hipStream_t s) { return launch_fwd_bigd_nw<NC, 4>(p, s); }
 
 // Dropout of the probabilities: the 128-query forward and dQ kernels and the dK/dV kernel in their DROPOUT
 // instantiations, without the split of the last round; HASMASK: the general kernels for an explicit mask or bias.

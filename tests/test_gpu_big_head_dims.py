@@ -60,6 +60,14 @@ def test_big_head_dims_tile_edges(oracle, D, Sq, Sk):
         _check(oracle, t, 1.0 / math.sqrt(D), causal=True)
 
 
+@pytest.mark.parametrize("B,H,S,D", [(2, 8, 2048, 256), (1, 8, 2048, 384), (1, 8, 2048, 512)])
+def test_more_query_blocks_than_compute_units(oracle, B, H, S, D):
+    """At least 256 workgroups (128 queries each up to D = 256, 64 above), 64 key tiles per walk, causal: every
+    compute unit walks, and the walks differ in length."""
+    t = _case(5150 + D, B, H, S, S, D)
+    _check(oracle, t, 1.0 / math.sqrt(D), causal=True)
+
+
 def test_vae_mid_block_shape(oracle):
     """One head of D = 512 over a 48 x 48 latent (2304 positions), batch 2: more workgroups than the chip has CUs
     for one batch element is not needed for parity; large logits (Q and K of standard deviation 2: logits of

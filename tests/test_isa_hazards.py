@@ -107,6 +107,46 @@ def test_hand_emitted_mfma_results_are_not_touched_too_early(text):
     assert checked >= 4 * 96
 
 
+def test_operands_of_hand_emitted_mfmas_are_not_written_just_before(text):
+    """An MFMA may read a register the vector ALU wrote two wait states later at the earliest.  The compiler keeps
+    that distance for its own MFMAs; for the hand-emitted ones (architectural accumulator, or the big-head-dim
+    forward's pinned accumulation tuples) it must come from the statement itself (an s_nop in front) or from where
+    the operands live (pinned registers that nothing moves).  Checked: no vector-ALU instruction within the two
+    wait states in front of such an MFMA writes one of its source registers."""
+    kernels = re.findall(r"^(_ZN5fattn(?:15bwd_dkdv_kernel|18bwd_dq_wide_kernel|15fwd_wide_kernel|20sage_fwd_wide_kernel|15fwd_bigd_kernel)\w+):.*?\.end_amdhsa_kernel", text, re.S | re.M)
+    checked = 0
+    for name in kernels:
+        body = re.search(r"^%s:.*?\.end_amdhsa_kernel" % re.escape(name), text, re.S | re.M).group(0)
+        ins = [l.strip() for l in body.split("\n") if re.match(r"^\s+[a-z]", l)]
+        for idx, l in enumerate(ins):
+            if not l.startswith("v_mfma"):
+                continue
+            ops = [t.strip() for t in l.split(None, 1)[1].split(",")]
+            by_hand = ops[0].startswith("v[") or ("fwd_bigd_kernel" in name and ops[0].startswith("a["))
+            if not by_hand:
+                continue
+            checked += 1
+            src_v, src_a = set(), set()
+            for t in ops[1:4]:
+                src_v |= _regs(t, "v")
+                src_a |= _regs(t, "a")
+            states = 0
+            for l2 in reversed(ins[max(0, idx - 4):idx]):
+                m = re.match(r"s_nop\s+(\d+)", l2)
+                if m:
+                    states += int(m.group(1)) + 1
+                elif l2.startswith("v_") and not l2.startswith("v_mfma"):
+                    dst = l2.split(None, 1)[1].split(",")[0].strip()
+                    wrote = (_regs(dst, "v") & src_v) | (_regs(dst, "a") & src_a)
+                    assert not wrote, f"{name}: `{l2}` writes an operand of `{l}` {states} wait states before it"
+                    states += 1
+                else:
+                    states += 1
+                if states >= 2:
+                    break
+    assert checked >= 4 * 96
+
+
 def test_every_lds_dma_finds_its_destination_in_m0(text):
     kernels = re.findall(r"^(_ZN5fattn\w+):.*?\.end_amdhsa_kernel", text, re.S | re.M)
     assert kernels
