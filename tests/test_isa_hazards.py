@@ -111,9 +111,9 @@ def test_operands_of_hand_emitted_mfmas_are_not_written_just_before(text):
     """An MFMA may read a register the vector ALU wrote two wait states later at the earliest.  The compiler keeps
     that distance for its own MFMAs; for the hand-emitted ones (architectural accumulator, or the big-head-dim
     forward's pinned accumulation tuples) it must come from the statement itself (an s_nop in front) or from where
-    the operands live (pinned registers that nothing moves).  Checked: no vector-ALU instruction within the two
-    wait states in front of such an MFMA writes one of its source registers."""
-    kernels = re.findall(r"^(_ZN5fattn(?:15bwd_dkdv_kernel|18bwd_dq_wide_kernel|15fwd_wide_kernel|20sage_fwd_wide_kernel|15fwd_bigd_kernel)\w+):.*?\.end_amdhsa_kernel", text, re.S | re.M)
+    the operands live (pinned registers that nothing moves).  Checked on every MFMA of every kernel: no vector-ALU
+    instruction within the two wait states in front of it writes one of its source registers."""
+    kernels = re.findall(r"^(_ZN5fattn\w+):.*?\.end_amdhsa_kernel", text, re.S | re.M)      # every kernel of the library
     checked = 0
     for name in kernels:
         body = re.search(r"^%s:.*?\.end_amdhsa_kernel" % re.escape(name), text, re.S | re.M).group(0)
@@ -121,10 +121,7 @@ def test_operands_of_hand_emitted_mfmas_are_not_written_just_before(text):
         for idx, l in enumerate(ins):
             if not l.startswith("v_mfma"):
                 continue
-            ops = [t.strip() for t in l.split(None, 1)[1].split(",")]
-            by_hand = ops[0].startswith("v[") or ("fwd_bigd_kernel" in name and ops[0].startswith("a["))
-            if not by_hand:
-                continue
+            ops = [t.strip() for t in l.split(None, 1)[1].split(",")]      # the compiler's own MFMAs pass by construction
             checked += 1
             src_v, src_a = set(), set()
             for t in ops[1:4]:
