@@ -185,6 +185,42 @@ def tile_ops_line(args, capi, torch, dev):
     return 0
 
 
+def big_head_dims_line(args, capi, torch, dev):
+    """The forward for head dims above 128 on four shapes (one with a single head of one image, the case of a VAE mid
+    block), next to torch's materialised bf16 matmul - fp32 softmax - matmul on the same GPU: median HIP-event
+    times, useful TFLOP/s (4 B H S^2 D)."""
+    import math
+    out = {}
+    g = torch.Generator(device=dev).manual_seed(11)
+    for (B, H, S, D) in [(16, 1, 4096, 512), (1, 1, 4096, 512), (2, 8, 4096, 384), (2, 8, 4096, 256)]:
+        q, k, v = (torch.randn((B, H, S, D), device=dev, generator=g).to(torch.bfloat16) for _ in range(3))
+        sc = 1.0 / math.sqrt(D)
+
+        def materialised():
+            p = torch.softmax(torch.matmul(q, k.transpose(-1, -2)).float() * sc, -1).to(torch.bfloat16)
+            return torch.matmul(p, v)
+
+        res = {}
+        for name, fn, iters in (("fused", lambda: capi.attn_fwd(q, k, v, sc), 20), ("materialised_torch", materialised, 8)):
+            for _ in range(3):
+                fn()
+            times = []
+            for _ in range(iters):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                fn()
+                e1.record()
+                e1.synchronize()
+                times.append(e0.elapsed_time(e1))
+            res[name + "_ms_median"] = sorted(times)[len(times) // 2]
+        res["fused_useful_TFLOPs"] = 4.0 * B * H * S * S * D / (res["fused_ms_median"] * 1e-3) / 1e12
+        out[f"B={B} H={H} S={S} D={D}"] = res
+    print(json.dumps({"metric": "forward for head dims above 128, ms", "unit": "ms", "n_gpus": 1, "dtype": "bf16",
+                      "data": "synthetic", "higher_is_better": False,
+                      "config": {"workload": "forward only, non-causal, head dims 256 / 384 / 512"}, "shapes": out}))
+    return 0
+
+
 def materialised_comparator(capi, torch, q, k, v, do, scale, o_fused, grads_fused, iters=5):
     """The structure this path replaces, run on the same GPU for comparison: scores = Q K^T as one library GEMM
     per head, softmax through this library's tile primitives, P kept in bf16 for the backward, PV / dV / dP / dQ /
@@ -344,6 +380,8 @@ def main():
     ap.add_argument("--traffic-calibration", action="store_true",
                     help="also run one plain 256 MiB device copy, so that FETCH_SIZE / WRITE_SIZE read under "
                          "rocprofv3 --pmc can be scaled by what the same counters report for a known size")
+    ap.add_argument("--big-head-dims", action="store_true",
+                    help="time the forward for head dims above 128 next to a materialised comparator (a line of its own)")
     ap.add_argument("--tile-ops", action="store_true",
                     help="time the element-wise tile primitives instead of an attention workload (a line of its own)")
     args = ap.parse_args()
@@ -366,6 +404,8 @@ def main():
         del src
     if args.tile_ops:
         return tile_ops_line(args, capi, torch, dev)
+    if args.big_head_dims:
+        return big_head_dims_line(args, capi, torch, dev)
     w = W.CONFIGS[args.config]()
     B, H, Sq, Sk, D = w.shape
     if w.do is None:            # inference-only workload (int8-QK forward)
