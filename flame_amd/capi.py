@@ -369,24 +369,27 @@ def fp8_to_bf16(codes, scale, out=None):
 
 
 # ---------------------------------------------------------------- dropout of the probabilities
-def attn_fwd_dropout(q, k, v, scale, dropout_p, dropout_seed, causal=False, kv_len=None, mask=None, out=None):
-    """O, LSE = flame_attn_fwd_dropout_bf16(...): the kept set of the reference's autograd_v4 operator for this seed."""
+def attn_fwd_dropout(q, k, v, scale, dropout_p, dropout_seed, causal=False, kv_len=None, mask=None, out=None,
+                     draw_chunk_q=0, draw_chunk_kv=0):
+    """O, LSE = flame_attn_fwd_dropout_tiled_bf16(...): the kept set of the reference's autograd_v4 operator for this
+    seed; draw_chunk_q / draw_chunk_kv: the tiles it draws over when it is chunked (0 = the whole axis)."""
     B, H, Sq, D = q.shape
     Sk = k.shape[2]
     o = torch.empty((B, H, Sq, D), dtype=torch.bfloat16, device=q.device) if out is None else out
     lse = torch.empty((B * H, Sq), dtype=torch.float32, device=q.device)
-    rc = lib().flame_attn_fwd_dropout_bf16(
+    rc = lib().flame_attn_fwd_dropout_tiled_bf16(
         _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), B, H, Sq, Sk, D, ctypes.c_float(scale),
         _i64x4(q.stride()), _i64x4(k.stride()), _i64x4(v.stride()), _i64x4(o.stride()),
         *(ctypes.c_int64(0) for _ in range(5)),
         int(bool(causal)), _ptr(kv_len), _ptr(mask), _mask_strides(mask, B, H, Sq, Sk),
-        ctypes.c_float(dropout_p), ctypes.c_uint64(dropout_seed & (2 ** 64 - 1)), _stream())
+        ctypes.c_float(dropout_p), ctypes.c_uint64(dropout_seed & (2 ** 64 - 1)), int(draw_chunk_q), int(draw_chunk_kv), _stream())
     if rc != 0:
-        raise FlameAttnError("flame_attn_fwd_dropout_bf16", rc)
+        raise FlameAttnError("flame_attn_fwd_dropout_tiled_bf16", rc)
     return o, lse
 
 
-def attn_bwd_dropout(q, k, v, o, do, lse, scale, dropout_p, dropout_seed, causal=False, kv_len=None, mask=None, workspace=None):
+def attn_bwd_dropout(q, k, v, o, do, lse, scale, dropout_p, dropout_seed, causal=False, kv_len=None, mask=None, workspace=None,
+                     draw_chunk_q=0, draw_chunk_kv=0):
     B, H, Sq, D = q.shape
     Sk = k.shape[2]
     if workspace is None:
@@ -394,15 +397,15 @@ def attn_bwd_dropout(q, k, v, o, do, lse, scale, dropout_p, dropout_seed, causal
     dq = torch.empty((B, H, Sq, D), dtype=torch.bfloat16, device=q.device)
     dk = torch.empty((B, H, Sk, D), dtype=torch.bfloat16, device=q.device)
     dv = torch.empty((B, H, Sk, D), dtype=torch.bfloat16, device=q.device)
-    rc = lib().flame_attn_bwd_dropout_bf16(
+    rc = lib().flame_attn_bwd_dropout_tiled_bf16(
         _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(do), _ptr(lse), _ptr(dq), _ptr(dk), _ptr(dv),
         B, H, Sq, Sk, D, ctypes.c_float(scale),
         _i64x4(q.stride()), _i64x4(k.stride()), _i64x4(v.stride()), _i64x4(o.stride()),
         _i64x4(do.stride()), _i64x4(dq.stride()), _i64x4(dk.stride()), _i64x4(dv.stride()),
         *(ctypes.c_int64(0) for _ in range(9)),
         int(bool(causal)), _ptr(kv_len), _ptr(mask), _mask_strides(mask, B, H, Sq, Sk),
-        ctypes.c_float(dropout_p), ctypes.c_uint64(dropout_seed & (2 ** 64 - 1)),
+        ctypes.c_float(dropout_p), ctypes.c_uint64(dropout_seed & (2 ** 64 - 1)), int(draw_chunk_q), int(draw_chunk_kv),
         _ptr(workspace), ctypes.c_size_t(workspace.numel()), _stream())
     if rc != 0:
-        raise FlameAttnError("flame_attn_bwd_dropout_bf16", rc)
+        raise FlameAttnError("flame_attn_bwd_dropout_tiled_bf16", rc)
     return dq, dk, dv

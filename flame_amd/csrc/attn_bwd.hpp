@@ -463,7 +463,7 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
             }
             if constexpr (DROPOUT) {
                 const uint32_t qi = (uint32_t)(q0 + 32 * qb + 8 * g + 4 * h + t);
-                const float f = drop_factor(p.m, ((uint32_t)bh * (uint32_t)p.Sq + qi) * (uint32_t)p.Sk + (uint32_t)key);
+                const float f = drop_factor_at(p.m, (uint32_t)bh, qi, (uint32_t)key, (uint32_t)p.Sq, (uint32_t)p.Sk);
                 dpacc[qb][r] = pr * fmaf(f, dpacc[qb][r], nd4[t]);       // dS = P (f dP - delta)
                 pr *= f;                                                  // what multiplied V in the forward
             }
@@ -976,8 +976,8 @@ __global__ __launch_bounds__(64 * NW, (NW == 4 && (!HASMASK || VECMASK)) ? 2 : 1
             if constexpr (DROPOUT) {
                 // O = (P f) V with f = 0 or 1 / (1 - p): dP = f (dO V^T), and rowsum(dP P) is still rowsum(dO O)
                 const uint32_t key = (uint32_t)(key0 + 32 * kb + acc_row(r, h));
-                const uint32_t row = ((uint32_t)bh * (uint32_t)p.Sq + (uint32_t)qrow) * (uint32_t)p.Sk;
-                dpacc[kb][r] = sacc[kb][r] * fmaf(drop_factor(p.m, row + key), dpacc[kb][r], -delta);
+                const float f = drop_factor_at(p.m, (uint32_t)bh, (uint32_t)qrow, key, (uint32_t)p.Sq, (uint32_t)p.Sk);
+                dpacc[kb][r] = sacc[kb][r] * fmaf(f, dpacc[kb][r], -delta);
             } else {
                 dpacc[kb][r] = sacc[kb][r] * (dpacc[kb][r] - delta);
             }

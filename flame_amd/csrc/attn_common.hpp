@@ -484,6 +484,7 @@ struct MaskArgs {
     uint32_t drop_seed = 0;  // low 32 bits of the seed
     uint32_t drop_thr = 0;   // ceil(p * 2^24): an element is kept when its 24-bit uniform is >= this
     float drop_scale = 1.f;  // 1 / (1 - p)
+    uint32_t drop_cq = 0, drop_ck = 0;   // tiles of a chunked draw along queries and keys; drop_cq = 0: one draw over the tensor
 };
 
 // Factor that dropout applies to the probability of flat element index idx of the [B*H, Sq, Sk] probability tensor
@@ -492,6 +493,21 @@ struct MaskArgs {
 // u >= p, which in integers is (xorshift32(seed ^ idx) >> 8) >= ceil(p * 2^24).
 __device__ __forceinline__ float drop_factor(const MaskArgs& m, uint32_t idx) {
     uint32_t s = m.drop_seed ^ idx;
+    s ^= s << 13;
+    s ^= s >> 17;
+    s ^= s << 5;
+    return (s >> 8) >= m.drop_thr ? m.drop_scale : 0.f;
+}
+
+// The same for element (bh, qi, key) when the reference's operator is chunked (src/autograd_v4/ops/sdpa.rs:180-199,
+// :444): it draws per tile of drop_cq x drop_ck (the last ones shorter) over the tile's own [B*H, q_t, k_t] tensor,
+// under the seed derive_tile_seed gives (:600-602), whose low word is seed + k_offset (the query offset is shifted
+// out of it).  drop_cq = 0 is the draw over the whole tensor.
+__device__ __forceinline__ float drop_factor_at(const MaskArgs& m, uint32_t bh, uint32_t qi, uint32_t key, uint32_t Sq, uint32_t Sk) {
+    if (m.drop_cq == 0) return drop_factor(m, (bh * Sq + qi) * Sk + key);
+    const uint32_t qo = qi / m.drop_cq * m.drop_cq, ko = key / m.drop_ck * m.drop_ck;
+    const uint32_t qt = min(m.drop_cq, Sq - qo), kt = min(m.drop_ck, Sk - ko);
+    uint32_t s = (m.drop_seed + ko) ^ ((bh * qt + (qi - qo)) * kt + (key - ko));
     s ^= s << 13;
     s ^= s >> 17;
     s ^= s << 5;

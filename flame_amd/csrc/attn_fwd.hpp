@@ -193,8 +193,8 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void fwd_kernel(const Fwd
     constexpr int EPS = 32 / NS;   // logits handled per softmax slice
 
     // flat index (mod 2^32) of this lane's query row in the [B*H, Sq, Sk] probability tensor
-    const uint32_t drop_row = ((uint32_t)bh * (uint32_t)p.Sq + (uint32_t)(qw0 + n)) * (uint32_t)p.Sk;
-    (void)drop_row;
+    const uint32_t drop_qi = (uint32_t)(qw0 + n);
+    (void)drop_qi;
     // exclusions of tile t: ragged tail / key length, causal, explicit keep-mask
     auto apply_mask = [&](f32x16 (&s)[2], int t) {
         const int qi = qw0 + n;
@@ -292,7 +292,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void fwd_kernel(const Fwd
                 else rsum0 += v;
                 if constexpr (DROPOUT) {
                     const uint32_t key = (uint32_t)(t * BN + 32 * kb + acc_row(r, h));
-                    cur[kb][r] = v * drop_factor(p.m, drop_row + key);
+                    cur[kb][r] = v * drop_factor_at(p.m, (uint32_t)bh, drop_qi, key, (uint32_t)p.Sq, (uint32_t)p.Sk);
                 } else {
                     cur[kb][r] = v;
                 }

@@ -340,8 +340,12 @@ int launch_bwd_dropout(const BwdParams& p, hipStream_t s) {
 }
 
 // 0 <= p < 1 (src/autograd_v4/ops/sdpa.rs:110-116); fills the kernel-side description of the draw
-bool set_dropout(MaskArgs& m, float dropout_p, uint64_t dropout_seed) {
-    if (!(dropout_p >= 0.f) || !(dropout_p < 1.f)) return false;
+// draw_cq / draw_ck: the tiles of the reference's chunked draw (0, or at least the sequence: the whole axis)
+bool set_dropout(MaskArgs& m, float dropout_p, uint64_t dropout_seed, int draw_cq, int draw_ck, int Sq, int Sk) {
+    if (!(dropout_p >= 0.f) || !(dropout_p < 1.f) || draw_cq < 0 || draw_ck < 0) return false;
+    const int cq = (draw_cq == 0 || draw_cq > Sq) ? Sq : draw_cq, ck = (draw_ck == 0 || draw_ck > Sk) ? Sk : draw_ck;
+    m.drop_cq = (cq == Sq && ck == Sk) ? 0u : (uint32_t)cq;
+    m.drop_ck = (uint32_t)ck;
     m.drop_seed = (uint32_t)dropout_seed;
     m.drop_thr = (uint32_t)ceil((double)dropout_p * 16777216.0);      // u >= p  <=>  24-bit integer >= ceil(p * 2^24)
     const float keep = 1.0f - dropout_p;
@@ -404,7 +408,8 @@ static int attn_bwd_impl(const void* Q, const void* K, const void* V, const void
                         int64_t lse_off, int64_t dq_off, int64_t dk_off, int64_t dv_off,
                         int causal, const int32_t* kv_len,
                         const uint8_t* keep_mask, const int64_t* mask_strides,
-                        void* workspace, size_t workspace_bytes, void* stream, float dropout_p, uint64_t dropout_seed) {
+                        void* workspace, size_t workspace_bytes, void* stream, float dropout_p, uint64_t dropout_seed,
+                        int draw_cq = 0, int draw_ck = 0) {
     if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0) return FLAME_ATTN_ERR_INVALID;
     if (!(scale > 0.f) || !isfinite(scale)) return FLAME_ATTN_ERR_INVALID;
     if (!LSE || !workspace) return FLAME_ATTN_ERR_INVALID;
@@ -458,7 +463,7 @@ static int attn_bwd_impl(const void* Q, const void* K, const void* V, const void
     if (D == 128 && !keep_mask && g_phase_cycles) return launch_bwd<128, false, true>(p, s);   // phase-timing build
 #endif
     if (dropout_p != 0.f) {
-        if (!set_dropout(p.m, dropout_p, dropout_seed)) return FLAME_ATTN_ERR_INVALID;
+        if (!set_dropout(p.m, dropout_p, dropout_seed, draw_cq, draw_ck, N_q, N_kv)) return FLAME_ATTN_ERR_INVALID;
         if (padded_head_dim(D) == 128) return keep_mask ? launch_bwd_dropout<128, true>(p, s) : launch_bwd_dropout<128, false>(p, s);
         return keep_mask ? launch_bwd_dropout<64, true>(p, s) : launch_bwd_dropout<64, false>(p, s);
     }
@@ -497,6 +502,23 @@ int flame_attn_bwd_dropout_bf16(const void* Q, const void* K, const void* V, con
                          do_strides, dq_strides, dk_strides, dv_strides, q_off, k_off, v_off, o_off, do_off, lse_off, dq_off,
                          dk_off, dv_off, causal, kv_len, keep_mask, mask_strides, workspace, workspace_bytes, stream, dropout_p,
                          dropout_seed);
+}
+
+int flame_attn_bwd_dropout_tiled_bf16(const void* Q, const void* K, const void* V, const void* O, const void* dO,
+                                      const void* LSE, void* dQ, void* dK, void* dV,
+                                      int B, int H, int N_q, int N_kv, int D, float scale,
+                                      const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                                      const int64_t* o_strides, const int64_t* do_strides, const int64_t* dq_strides,
+                                      const int64_t* dk_strides, const int64_t* dv_strides,
+                                      int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off, int64_t do_off,
+                                      int64_t lse_off, int64_t dq_off, int64_t dk_off, int64_t dv_off,
+                                      int causal, const int32_t* kv_len, const uint8_t* keep_mask, const int64_t* mask_strides,
+                                      float dropout_p, uint64_t dropout_seed, int draw_chunk_q, int draw_chunk_kv,
+                                      void* workspace, size_t workspace_bytes, void* stream) {
+    return attn_bwd_impl(Q, K, V, O, dO, LSE, dQ, dK, dV, B, H, N_q, N_kv, D, scale, q_strides, k_strides, v_strides, o_strides,
+                         do_strides, dq_strides, dk_strides, dv_strides, q_off, k_off, v_off, o_off, do_off, lse_off, dq_off,
+                         dk_off, dv_off, causal, kv_len, keep_mask, mask_strides, workspace, workspace_bytes, stream, dropout_p,
+                         dropout_seed, draw_chunk_q, draw_chunk_kv);
 }
 
 int flame_sage_quant_qk_int8(const void* Q, const void* K, int B, int H, int N_q, int N_kv, int D,
@@ -688,7 +710,7 @@ static int attn_fwd_impl(const void* Q, const void* K, const void* V, void* O, v
                         const uint8_t* keep_mask, const int64_t* mask_strides,
                         const void* bias, int bias_dtype, const int64_t* bias_strides,
                         void* stream, int mask_mode = kMaskU8, int Dv = 0, int q_tile_plan = 0, float dropout_p = 0.f,
-                        uint64_t dropout_seed = 0) {
+                        uint64_t dropout_seed = 0, int draw_cq = 0, int draw_ck = 0) {
     if (Dv == 0) Dv = D;           // V and O may have a head dim of their own (forward only)
     if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0 || Dv < 0) return FLAME_ATTN_ERR_INVALID;
     if (!(scale > 0.f) || !isfinite(scale)) return FLAME_ATTN_ERR_INVALID;
@@ -736,7 +758,7 @@ static int attn_fwd_impl(const void* Q, const void* K, const void* V, void* O, v
     if (big) return D <= 256 ? launch_fwd_bigd<2>(p, s) : D <= 384 ? launch_fwd_bigd<3>(p, s) : launch_fwd_bigd<4>(p, s);
     const bool hm = keep_mask != nullptr || bias != nullptr;
     if (dropout_p != 0.f) {
-        if (!set_dropout(p.m, dropout_p, dropout_seed)) return FLAME_ATTN_ERR_INVALID;
+        if (!set_dropout(p.m, dropout_p, dropout_seed, draw_cq, draw_ck, N_q, N_kv)) return FLAME_ATTN_ERR_INVALID;
         if (std::max(padded_head_dim(D), padded_head_dim(Dv)) == 128)
             return hm ? launch_fwd_dropout<128, true>(p, s) : launch_fwd_dropout<128, false>(p, s);
         return hm ? launch_fwd_dropout<64, true>(p, s) : launch_fwd_dropout<64, false>(p, s);
@@ -786,6 +808,19 @@ int flame_attn_fwd_dropout_bf16(const void* Q, const void* K, const void* V, voi
     return attn_fwd_impl(Q, K, V, O, LSE, B, H, N_q, N_kv, D, scale, q_strides, k_strides, v_strides, o_strides,
                          q_off, k_off, v_off, o_off, lse_off, causal, kv_len, keep_mask, mask_strides,
                          nullptr, FLAME_ATTN_DTYPE_F32, nullptr, stream, kMaskU8, 0, 0, dropout_p, dropout_seed);
+}
+
+int flame_attn_fwd_dropout_tiled_bf16(const void* Q, const void* K, const void* V, void* O, void* LSE,
+                                      int B, int H, int N_q, int N_kv, int D, float scale,
+                                      const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                                      const int64_t* o_strides,
+                                      int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off, int64_t lse_off,
+                                      int causal, const int32_t* kv_len, const uint8_t* keep_mask, const int64_t* mask_strides,
+                                      float dropout_p, uint64_t dropout_seed, int draw_chunk_q, int draw_chunk_kv, void* stream) {
+    return attn_fwd_impl(Q, K, V, O, LSE, B, H, N_q, N_kv, D, scale, q_strides, k_strides, v_strides, o_strides,
+                         q_off, k_off, v_off, o_off, lse_off, causal, kv_len, keep_mask, mask_strides,
+                         nullptr, FLAME_ATTN_DTYPE_F32, nullptr, stream, kMaskU8, 0, 0, dropout_p, dropout_seed, draw_chunk_q,
+                         draw_chunk_kv);
 }
 
 int flame_attn_fwd_bias_bf16(const void* Q, const void* K, const void* V, void* O, void* LSE,

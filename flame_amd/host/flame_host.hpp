@@ -219,7 +219,8 @@ struct FwdOut {
 };
 
 inline Result<FwdOut> run_forward(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor* mask, bool causal,
-                                  std::optional<float> scale, bool want_stats, float dropout_p = 0.f, uint64_t dropout_seed = 0) {
+                                  std::optional<float> scale, bool want_stats, float dropout_p = 0.f, uint64_t dropout_seed = 0,
+                                  int draw_chunk_q = 0, int draw_chunk_kv = 0) {
     auto dv = validate(q, k, v, mask);
     if (!dv.ok()) return dv.error();
     const Dims d = dv.value();
@@ -243,14 +244,13 @@ inline Result<FwdOut> run_forward(const Tensor& q, const Tensor& k, const Tensor
     }
     const float sc = scale.value_or(1.0f / std::sqrt((float)d.D));
     if (dropout_p != 0.f) {
-        const int rc = flame_attn_fwd_dropout_bf16(q.base(), k.base(), v.base(), o.value().base(), want_stats ? stats.base() : nullptr,
-                                                   d.B, d.H, d.Sq, d.Sk, d.D, sc, q.strides().data(), k.strides().data(),
-                                                   v.strides().data(), o.value().strides().data(), q.offset(), k.offset(),
-                                                   v.offset(), 0, 0, causal ? 1 : 0, nullptr,
-                                                   mask ? static_cast<const uint8_t*>(m8.data()) : nullptr, mask ? mst.data() : nullptr,
-                                                   dropout_p, dropout_seed, nullptr);
-        if (rc == FLAME_ATTN_ERR_UNSUPPORTED) return unsupported("flame_attn_fwd_dropout_bf16: head dim or layout not built");
-        if (rc != 0) return cuda_error("flame_attn_fwd_dropout_bf16", rc);
+        const int rc = flame_attn_fwd_dropout_tiled_bf16(
+            q.base(), k.base(), v.base(), o.value().base(), want_stats ? stats.base() : nullptr, d.B, d.H, d.Sq, d.Sk, d.D, sc,
+            q.strides().data(), k.strides().data(), v.strides().data(), o.value().strides().data(), q.offset(), k.offset(),
+            v.offset(), 0, 0, causal ? 1 : 0, nullptr, mask ? static_cast<const uint8_t*>(m8.data()) : nullptr,
+            mask ? mst.data() : nullptr, dropout_p, dropout_seed, draw_chunk_q, draw_chunk_kv, nullptr);
+        if (rc == FLAME_ATTN_ERR_UNSUPPORTED) return unsupported("flame_attn_fwd_dropout_tiled_bf16: head dim or layout not built");
+        if (rc != 0) return cuda_error("flame_attn_fwd_dropout_tiled_bf16", rc);
         return FwdOut{o.value(), stats};
     }
     const int rc = flame_attn_fwd_bf16(q.base(), k.base(), v.base(), o.value().base(), want_stats ? stats.base() : nullptr,
@@ -277,6 +277,7 @@ struct FlashAttentionNode {
     bool causal = false;
     float dropout_p = 0.f;            // set by the v4 operator only (autograd_v4::SdpaCtx)
     uint64_t dropout_seed = 0;
+    int draw_chunk_q = 0, draw_chunk_kv = 0;    // tiles of a chunked draw, 0 = the whole axis
 };
 
 class AutogradContext {
@@ -354,16 +355,16 @@ inline Result<AttentionGrads> flash_attention_backward(const FlashAttentionNode&
         mst = pm.value().second;
     }
     if (n.dropout_p != 0.f) {
-        const int rc = flame_attn_bwd_dropout_bf16(
+        const int rc = flame_attn_bwd_dropout_tiled_bf16(
             n.query.base(), n.key.base(), n.value.base(), n.output.base(), g.base(), n.stats.base(), dq.value().base(),
             dk.value().base(), dv.value().base(), B, H, Sq, Sk, D, n.scale, n.query.strides().data(), n.key.strides().data(),
             n.value.strides().data(), n.output.strides().data(), g.strides().data(), dq.value().strides().data(),
             dk.value().strides().data(), dv.value().strides().data(), n.query.offset(), n.key.offset(), n.value.offset(),
             n.output.offset(), g.offset(), 0, 0, 0, 0, n.causal ? 1 : 0, nullptr,
             n.mask ? static_cast<const uint8_t*>(m8.data()) : nullptr, n.mask ? mst.data() : nullptr, n.dropout_p, n.dropout_seed,
-            ws.value().data(), wsb, nullptr);
-        if (rc == FLAME_ATTN_ERR_UNSUPPORTED) return unsupported("flame_attn_bwd_dropout_bf16: head dim or layout not built");
-        if (rc != 0) return cuda_error("flame_attn_bwd_dropout_bf16", rc);
+            n.draw_chunk_q, n.draw_chunk_kv, ws.value().data(), wsb, nullptr);
+        if (rc == FLAME_ATTN_ERR_UNSUPPORTED) return unsupported("flame_attn_bwd_dropout_tiled_bf16: head dim or layout not built");
+        if (rc != 0) return cuda_error("flame_attn_bwd_dropout_tiled_bf16", rc);
         return AttentionGrads{dq.value(), dk.value(), dv.value()};
     }
     const int rc = flame_attn_bwd_bf16(
@@ -575,6 +576,7 @@ struct SdpaCtx {                          // :80-96
     SdpaStats stats;
     float dropout_p = 0.f;                // :94-95
     std::optional<uint64_t> dropout_seed;
+    std::pair<int, int> chunk_cfg{0, 0};  // (chunk_q, chunk_kv) the forward drew its dropout tiles with; 0 = whole axis
 };
 
 // ---- tape of the v4 engine (src/autograd_v4/graph.rs:12-94): nodes keyed by the output tensor's id,
@@ -685,20 +687,20 @@ inline uint64_t next_u64() {          // SplitMix64
 
 // sdpa_forward(q,k,v,mask,&cfg) -> (output, ctx) (:98-326).  SaveProbs would materialise the
 // [B,H,Q,K] matrix and is refused rather than emulated.  Dropout (:110-124, :229-231) runs inside the fused
-// kernels with the kept set the reference draws for the same seed when it does not chunk; a chunked draw
-// (chunk_q / chunk_kv smaller than the lengths) re-seeds per chunk (:600-602) and is not built.
+// kernels with the kept set the reference draws for the same seed: over the whole tensor, or, when the operator
+// is chunked there (save = SaveLSE and chunk_q / chunk_kv smaller than the lengths, :180-199), per tile with the
+// tile's seed (:600-602).  The attention itself is never chunked here: the chunk sizes only shape the kept set.
 inline Result<std::pair<Tensor, SdpaCtx>> sdpa_forward(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor* mask,
                                                        const SdpaConfig& cfg) {
     if (cfg.dropout_p < 0.f || cfg.dropout_p >= 1.f || cfg.dropout_p != cfg.dropout_p)
         return invalid("sdpa_forward: dropout_p=" + std::to_string(cfg.dropout_p) + " is out of range [0, 1)");
     std::optional<uint64_t> dropout_seed;
     if (cfg.dropout_p > 0.f) {
-        if (q.shape().size() == 4 && k.shape().size() == 4 &&
-            ((cfg.chunk_q && *cfg.chunk_q > 0 && (int64_t)*cfg.chunk_q < q.shape()[2]) ||
-             (cfg.chunk_kv && *cfg.chunk_kv > 0 && (int64_t)*cfg.chunk_kv < k.shape()[2])))
-            return unsupported("dropout with a chunked draw is not built: leave chunk_q / chunk_kv unset");
         dropout_seed = cfg.dropout_seed ? *cfg.dropout_seed : rng::next_u64();
     }
+    // the reference chunks (and draws per tile) under SaveLSE only (:197-199)
+    const int draw_cq = cfg.save == SdpaSave::SaveLSE && cfg.chunk_q ? (int)std::min<size_t>(*cfg.chunk_q, 1u << 30) : 0;
+    const int draw_ck = cfg.save == SdpaSave::SaveLSE && cfg.chunk_kv ? (int)std::min<size_t>(*cfg.chunk_kv, 1u << 30) : 0;
     if (cfg.save == SdpaSave::SaveProbs) return unsupported("SaveProbs materialises [B,H,Q,K]; use SaveLSE");
     const SdpaHooks* hooks = debug_hooks();
     std::unique_ptr<StreamTimer> timer;
@@ -710,11 +712,12 @@ inline Result<std::pair<Tensor, SdpaCtx>> sdpa_forward(const Tensor& q, const Te
     // SaveLSE keeps O and the log-sum-exp for the backward; Recompute (:21-47) keeps neither and the backward
     // runs the forward once more to get them back (the outputs are deterministic, so it sees the same O).
     const bool keep = cfg.save != SdpaSave::Recompute;
-    auto r = detail::run_forward(q, k, v, mask, cfg.causal, cfg.scale, keep, cfg.dropout_p, dropout_seed.value_or(0));
+    auto r = detail::run_forward(q, k, v, mask, cfg.causal, cfg.scale, keep, cfg.dropout_p, dropout_seed.value_or(0), draw_cq, draw_ck);
     if (!r.ok()) return r.error();
     SdpaCtx ctx;
     ctx.dropout_p = cfg.dropout_p;
     ctx.dropout_seed = dropout_seed;
+    ctx.chunk_cfg = {draw_cq, draw_ck};
     ctx.q = q; ctx.k = k; ctx.v = v;
     if (keep) ctx.o = r.value().o;
     if (mask) ctx.attn_mask = *mask;
@@ -754,6 +757,8 @@ inline Result<std::tuple<Tensor, Tensor, Tensor>> sdpa_backward(const SdpaCtx& c
     n.causal = ctx.causal;
     n.dropout_p = ctx.dropout_p;
     n.dropout_seed = ctx.dropout_seed.value_or(0);
+    n.draw_chunk_q = ctx.chunk_cfg.first;
+    n.draw_chunk_kv = ctx.chunk_cfg.second;
     if (ctx.dropout_p > 0.f && !ctx.dropout_seed) return Error{Error::InvalidInput, "dropout seed required when dropout_p > 0"};
     if (ctx.save == SdpaSave::Recompute) {          // nothing was kept: O and the log-sum-exp come from one more forward
         auto f = detail::run_forward(ctx.q, ctx.k, ctx.v, ctx.attn_mask ? &*ctx.attn_mask : nullptr, ctx.causal, ctx.scale, true,

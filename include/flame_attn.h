@@ -124,6 +124,31 @@ int flame_attn_bwd_dropout_bf16(const void* Q, const void* K, const void* V, con
                                 int causal, const int32_t* kv_len, const uint8_t* keep_mask, const int64_t* mask_strides,
                                 float dropout_p, uint64_t dropout_seed,
                                 void* workspace, size_t workspace_bytes, void* stream);
+/* The same pair with the kept set the operator draws when it is chunked (save = SaveLSE and chunk_q < N_q or chunk_kv <
+ * N_kv, src/autograd_v4/ops/sdpa.rs:180-199, :444): one draw per tile of draw_chunk_q x draw_chunk_kv (the last tiles
+ * shorter) over the tile's own [B*H, q_t, k_t] tensor, under the seed derive_tile_seed gives (:600-602), whose low word
+ * is dropout_seed + k_offset.  0, or a chunk of at least the sequence length, means the whole axis; with both whole this
+ * is the pair above.  The attention itself is not chunked: only the kept set depends on the tiles.
+ * A seed whose low word is 0 (here: for some tile) makes the reference draw from its global generator instead
+ * (src/rng/mod.rs:187-193); no fixed kept set exists for it there, this library uses the 0. */
+int flame_attn_fwd_dropout_tiled_bf16(const void* Q, const void* K, const void* V, void* O, void* LSE,
+                                      int B, int H, int N_q, int N_kv, int D, float scale,
+                                      const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                                      const int64_t* o_strides,
+                                      int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off, int64_t lse_off,
+                                      int causal, const int32_t* kv_len, const uint8_t* keep_mask, const int64_t* mask_strides,
+                                      float dropout_p, uint64_t dropout_seed, int draw_chunk_q, int draw_chunk_kv, void* stream);
+int flame_attn_bwd_dropout_tiled_bf16(const void* Q, const void* K, const void* V, const void* O, const void* dO,
+                                      const void* LSE, void* dQ, void* dK, void* dV,
+                                      int B, int H, int N_q, int N_kv, int D, float scale,
+                                      const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                                      const int64_t* o_strides, const int64_t* do_strides, const int64_t* dq_strides,
+                                      const int64_t* dk_strides, const int64_t* dv_strides,
+                                      int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off, int64_t do_off,
+                                      int64_t lse_off, int64_t dq_off, int64_t dk_off, int64_t dv_off,
+                                      int causal, const int32_t* kv_len, const uint8_t* keep_mask, const int64_t* mask_strides,
+                                      float dropout_p, uint64_t dropout_seed, int draw_chunk_q, int draw_chunk_kv,
+                                      void* workspace, size_t workspace_bytes, void* stream);
 
 /* Recommended bytes of device scratch for the backward: two fp32 values per query row (required),
  * plus one 128-key block of fp32 dK/dV partial sums per compute unit of the current device

@@ -340,23 +340,40 @@ def dropout_keep(seed: int, flat_index: int, p: float) -> bool:
     return bool(lib().oracle_dropout_keep(ctypes.c_uint64(seed & (2 ** 64 - 1)), ctypes.c_uint64(flat_index), ctypes.c_float(p)))
 
 
-def dropout_uniforms(B, H, Sq, Sk, seed) -> np.ndarray:
-    """fp32 [B,H,Sq,Sk]: the uniform each probability is compared with, written from the recurrence in numpy (not
-    through the C file)."""
-    idx = (np.arange(B * H * Sq * Sk, dtype=np.uint64) & np.uint64(0xFFFFFFFF)).astype(np.uint32)
-    s = idx ^ np.uint32(seed & 0xFFFFFFFF)
+def dropout_keep_tiled(seed: int, bh: int, i: int, j: int, Sq: int, Sk: int, cq: int, ck: int, p: float) -> bool:
+    return bool(lib().oracle_dropout_keep_tiled(ctypes.c_uint64(seed & (2 ** 64 - 1)), bh, i, j, Sq, Sk, cq, ck, ctypes.c_float(p)))
+
+
+def _xorshift_uniform(seed32: np.ndarray, idx32: np.ndarray) -> np.ndarray:
+    s = idx32.astype(np.uint32) ^ seed32.astype(np.uint32)
     s ^= s << np.uint32(13)
     s ^= s >> np.uint32(17)
     s ^= s << np.uint32(5)
-    return ((s >> np.uint32(8)).astype(np.float32) * np.float32(1.0 / 16777216.0)).reshape(B, H, Sq, Sk)
+    return (s >> np.uint32(8)).astype(np.float32) * np.float32(1.0 / 16777216.0)
 
 
-def dropout_keep_mask(B, H, Sq, Sk, p, seed) -> np.ndarray:
+def dropout_uniforms(B, H, Sq, Sk, seed, chunk_q=0, chunk_kv=0) -> np.ndarray:
+    """fp32 [B,H,Sq,Sk]: the uniform each probability is compared with, written from the recurrence in numpy (not
+    through the C file).  chunk_q / chunk_kv: the tiles of a chunked draw (0 = the whole axis)."""
+    cq = Sq if chunk_q <= 0 or chunk_q > Sq else chunk_q
+    ck = Sk if chunk_kv <= 0 or chunk_kv > Sk else chunk_kv
+    bh = np.arange(B * H, dtype=np.uint64)[:, None, None]
+    i = np.arange(Sq, dtype=np.uint64)[None, :, None]
+    j = np.arange(Sk, dtype=np.uint64)[None, None, :]
+    q_off, k_off = (i // cq) * cq, (j // ck) * ck
+    q_t, k_t = np.minimum(cq, Sq - q_off), np.minimum(ck, Sk - k_off)
+    idx = (bh * q_t + (i - q_off)) * k_t + (j - k_off)
+    seed32 = (np.uint64(seed & 0xFFFFFFFF) + k_off) & np.uint64(0xFFFFFFFF)          # the query offset sits above bit 31
+    u = _xorshift_uniform(np.broadcast_to(seed32, idx.shape), idx & np.uint64(0xFFFFFFFF))
+    return u.reshape(B, H, Sq, Sk)
+
+
+def dropout_keep_mask(B, H, Sq, Sk, p, seed, chunk_q=0, chunk_kv=0) -> np.ndarray:
     """bool [B,H,Sq,Sk]: kept where the uniform is >= p."""
-    return dropout_uniforms(B, H, Sq, Sk, seed) >= np.float32(p)
+    return dropout_uniforms(B, H, Sq, Sk, seed, chunk_q, chunk_kv) >= np.float32(p)
 
 
-def sdpa_fwd_dropout(q, k, v, scale, p, seed, causal=False, kv_len=None, mask=None, want_f32=False):
+def sdpa_fwd_dropout(q, k, v, scale, p, seed, causal=False, kv_len=None, mask=None, want_f32=False, chunk_q=0, chunk_kv=0):
     B, H, Sq, D = q.shape
     Sk = k.shape[2]
     q, k, v = (np.ascontiguousarray(t, dtype=np.uint16) for t in (q, k, v))
@@ -366,13 +383,14 @@ def sdpa_fwd_dropout(q, k, v, scale, p, seed, causal=False, kv_len=None, mask=No
     kvl = None if kv_len is None else np.ascontiguousarray(kv_len, dtype=np.int32)
     m, st, _keep = _mask_args(mask, B, H, Sq, Sk)
     rc = lib().oracle_sdpa_fwd_dropout(_p(q), _p(k), _p(v), B, H, Sq, Sk, D, ctypes.c_float(scale), int(bool(causal)), _p(kvl),
-                                       _p(m), *(ctypes.c_int64(x) for x in st), ctypes.c_float(p), ctypes.c_uint64(seed & (2 ** 64 - 1)), _p(O), _p(LSE), _p(O32))
+                                       _p(m), *(ctypes.c_int64(x) for x in st), ctypes.c_float(p), ctypes.c_uint64(seed & (2 ** 64 - 1)), int(chunk_q), int(chunk_kv),
+                                       _p(O), _p(LSE), _p(O32))
     if rc != 0:
         raise RuntimeError(f"oracle_sdpa_fwd_dropout failed: {rc}")
     return (O, LSE, O32) if want_f32 else (O, LSE)
 
 
-def sdpa_bwd_dropout(q, k, v, o, do, scale, p, seed, causal=False, kv_len=None, mask=None, want_f32=False):
+def sdpa_bwd_dropout(q, k, v, o, do, scale, p, seed, causal=False, kv_len=None, mask=None, want_f32=False, chunk_q=0, chunk_kv=0):
     B, H, Sq, D = q.shape
     Sk = k.shape[2]
     q, k, v, o, do = (np.ascontiguousarray(t, dtype=np.uint16) for t in (q, k, v, o, do))
@@ -384,7 +402,7 @@ def sdpa_bwd_dropout(q, k, v, o, do, scale, p, seed, causal=False, kv_len=None, 
     m, st, _keep = _mask_args(mask, B, H, Sq, Sk)
     rc = lib().oracle_sdpa_bwd_dropout(_p(q), _p(k), _p(v), _p(o), _p(do), B, H, Sq, Sk, D, ctypes.c_float(scale),
                                        int(bool(causal)), _p(kvl), _p(m), *(ctypes.c_int64(x) for x in st), ctypes.c_float(p), ctypes.c_uint64(seed & (2 ** 64 - 1)),
-                                       _p(dQ), _p(dK), _p(dV), _p(f[0]), _p(f[1]), _p(f[2]))
+                                       int(chunk_q), int(chunk_kv), _p(dQ), _p(dK), _p(dV), _p(f[0]), _p(f[1]), _p(f[2]))
     if rc != 0:
         raise RuntimeError(f"oracle_sdpa_bwd_dropout failed: {rc}")
     return (dQ, dK, dV, *f) if want_f32 else (dQ, dK, dV)

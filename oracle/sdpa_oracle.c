@@ -100,6 +100,7 @@ typedef struct {
     int64_t bsb, bsh, bsq, bsk; /* its element strides over (b,h,q,k); 0 = broadcast     */
     float drop_p;            /* dropout probability, 0 = none                          */
     uint64_t drop_seed;
+    int drop_cq, drop_ck;    /* tiles of the draw along queries and keys; 0 = one draw over the whole tensor */
 } mask_spec;
 
 /* Dropout of the attention probabilities as the reference's autograd_v4 operator draws it when it is not
@@ -119,12 +120,25 @@ int oracle_dropout_keep(uint64_t seed, uint64_t flat_index, float p) {
     const float u = (float)(s >> 8) * (1.0f / 16777216.0f);
     return u >= p;
 }
+/* The same operator when it is chunked (save = SaveLSE and a query or key chunk shorter than the sequence,
+ * :180-199): it draws per tile of chunk_q x chunk_kv (the last ones shorter), over the tile's own [B*H, q_t, k_t]
+ * tensor, with the seed derive_tile_seed gives (:600-602): (seed + ((q_offset << 32) ^ k_offset)) truncated to 32
+ * bits, which is seed32 + k_offset: the query offset does not reach the low word.  Element (bh, i, j) therefore has
+ * index (bh * q_t + i - q_offset) * k_t + j - k_offset under seed32 + k_offset. */
+int oracle_dropout_keep_tiled(uint64_t seed, int bh, int i, int j, int Sq, int Sk, int cq, int ck, float p) {
+    if (cq <= 0 || cq > Sq) cq = Sq;
+    if (ck <= 0 || ck > Sk) ck = Sk;
+    const int q_off = (i / cq) * cq, k_off = (j / ck) * ck;
+    const int q_t = Sq - q_off < cq ? Sq - q_off : cq, k_t = Sk - k_off < ck ? Sk - k_off : ck;
+    const uint64_t tile_seed = seed + ((((uint64_t)q_off) << 32) ^ (uint64_t)k_off);      /* wrapping, as the reference */
+    const uint64_t idx = ((uint64_t)bh * (uint64_t)q_t + (uint64_t)(i - q_off)) * (uint64_t)k_t + (uint64_t)(j - k_off);
+    return oracle_dropout_keep(tile_seed, idx, p);
+}
 /* factor applied to P[bh, i, j]: 0 or 1 / (1 - p); 1 without dropout */
 static inline float drop_factor(const mask_spec* ms, int bh, int i, int j, int Sq, int Sk) {
     if (!(ms->drop_p > 0.f)) return 1.0f;
-    const uint64_t idx = ((uint64_t)bh * (uint64_t)Sq + (uint64_t)i) * (uint64_t)Sk + (uint64_t)j;
     const float keep = 1.0f - ms->drop_p;
-    return oracle_dropout_keep(ms->drop_seed, idx, ms->drop_p) ? 1.0f / keep : 0.f;
+    return oracle_dropout_keep_tiled(ms->drop_seed, bh, i, j, Sq, Sk, ms->drop_cq, ms->drop_ck, ms->drop_p) ? 1.0f / keep : 0.f;
 }
 
 static inline int excluded(const mask_spec* ms, int b, int h, int i, int j) {
@@ -190,7 +204,7 @@ int oracle_sdpa_fwd(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
                     int64_t msb, int64_t msh, int64_t msq, int64_t msk,
                     int heads_begin, int heads_end,
                     uint16_t* O, float* LSE, float* O32) {
-    mask_spec ms = {causal, kv_len, mask, msb, msh, msq, msk, NULL, 0, 0, 0, 0, 0.f, 0};
+    mask_spec ms = {causal, kv_len, mask, msb, msh, msq, msk, NULL, 0, 0, 0, 0, 0.f, 0, 0, 0};
     return sdpa_fwd_impl(Q, K, V, B, H, Sq, Sk, D, scale, ms, heads_begin, heads_end, 0, Sq, O, LSE, O32);
 }
 
@@ -203,7 +217,7 @@ int oracle_sdpa_fwd_rows(const uint16_t* Q, const uint16_t* K, const uint16_t* V
                          int64_t msb, int64_t msh, int64_t msq, int64_t msk,
                          int heads_begin, int heads_end, int row_begin, int row_end,
                          uint16_t* O, float* LSE, float* O32) {
-    mask_spec ms = {causal, kv_len, mask, msb, msh, msq, msk, NULL, 0, 0, 0, 0, 0.f, 0};
+    mask_spec ms = {causal, kv_len, mask, msb, msh, msq, msk, NULL, 0, 0, 0, 0, 0.f, 0, 0, 0};
     if (row_begin < 0 || row_end > Sq || row_begin > row_end) return -1;
     return sdpa_fwd_impl(Q, K, V, B, H, Sq, Sk, D, scale, ms, heads_begin, heads_end, row_begin, row_end, O, LSE, O32);
 }
@@ -214,7 +228,7 @@ int oracle_sdpa_fwd_bias(const uint16_t* Q, const uint16_t* K, const uint16_t* V
                          int B, int H, int Sq, int Sk, int D, float scale,
                          const float* bias, int64_t bsb, int64_t bsh, int64_t bsq, int64_t bsk,
                          uint16_t* O, float* LSE, float* O32) {
-    mask_spec ms = {0, NULL, NULL, 0, 0, 0, 0, bias, bsb, bsh, bsq, bsk, 0.f, 0};
+    mask_spec ms = {0, NULL, NULL, 0, 0, 0, 0, bias, bsb, bsh, bsq, bsk, 0.f, 0, 0, 0};
     return sdpa_fwd_impl(Q, K, V, B, H, Sq, Sk, D, scale, ms, 0, B * H, 0, Sq, O, LSE, O32);
 }
 
@@ -379,7 +393,7 @@ int oracle_sdpa_bwd_rows(const uint16_t* Q, const uint16_t* K, const uint16_t* V
                          int heads_begin, int heads_end, int row_begin, int row_end,
                          uint16_t* dQ, uint16_t* dK, uint16_t* dV,
                          float* dQ32, float* dK32, float* dV32) {
-    mask_spec ms = {causal, kv_len, mask, msb, msh, msq, msk, NULL, 0, 0, 0, 0, 0.f, 0};
+    mask_spec ms = {causal, kv_len, mask, msb, msh, msq, msk, NULL, 0, 0, 0, 0, 0.f, 0, 0, 0};
     return sdpa_bwd_impl(Q, K, V, O, dO, B, H, Sq, Sk, D, scale, ms, heads_begin, heads_end, row_begin, row_end,
                          dQ, dK, dV, dQ32, dK32, dV32);
 }
@@ -388,8 +402,8 @@ int oracle_sdpa_bwd_rows(const uint16_t* Q, const uint16_t* K, const uint16_t* V
 int oracle_sdpa_fwd_dropout(const uint16_t* Q, const uint16_t* K, const uint16_t* V,
                             int B, int H, int Sq, int Sk, int D, float scale, int causal, const int32_t* kv_len,
                             const uint8_t* mask, int64_t msb, int64_t msh, int64_t msq, int64_t msk,
-                            float drop_p, uint64_t drop_seed, uint16_t* O, float* LSE, float* O32) {
-    mask_spec ms = {causal, kv_len, mask, msb, msh, msq, msk, NULL, 0, 0, 0, 0, drop_p, drop_seed};
+                            float drop_p, uint64_t drop_seed, int drop_cq, int drop_ck, uint16_t* O, float* LSE, float* O32) {
+    mask_spec ms = {causal, kv_len, mask, msb, msh, msq, msk, NULL, 0, 0, 0, 0, drop_p, drop_seed, drop_cq, drop_ck};
     return sdpa_fwd_impl(Q, K, V, B, H, Sq, Sk, D, scale, ms, 0, B * H, 0, Sq, O, LSE, O32);
 }
 
@@ -397,9 +411,9 @@ int oracle_sdpa_bwd_dropout(const uint16_t* Q, const uint16_t* K, const uint16_t
                             const uint16_t* O, const uint16_t* dO,
                             int B, int H, int Sq, int Sk, int D, float scale, int causal, const int32_t* kv_len,
                             const uint8_t* mask, int64_t msb, int64_t msh, int64_t msq, int64_t msk,
-                            float drop_p, uint64_t drop_seed,
+                            float drop_p, uint64_t drop_seed, int drop_cq, int drop_ck,
                             uint16_t* dQ, uint16_t* dK, uint16_t* dV, float* dQ32, float* dK32, float* dV32) {
-    mask_spec ms = {causal, kv_len, mask, msb, msh, msq, msk, NULL, 0, 0, 0, 0, drop_p, drop_seed};
+    mask_spec ms = {causal, kv_len, mask, msb, msh, msq, msk, NULL, 0, 0, 0, 0, drop_p, drop_seed, drop_cq, drop_ck};
     return sdpa_bwd_impl(Q, K, V, O, dO, B, H, Sq, Sk, D, scale, ms, 0, B * H, 0, Sq, dQ, dK, dV, dQ32, dK32, dV32);
 }
 

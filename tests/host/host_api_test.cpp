@@ -315,7 +315,7 @@ int main() {
             }
         }
         // dropout: range check as the reference's (:110-116); the same seed gives the same bits, forward and backward;
-        // without a seed one is drawn from the global generator and kept in the context; a chunked draw is refused
+        // without a seed one is drawn from the global generator and kept in the context
         {
             autograd_v4::SdpaConfig dc = cfg;
             dc.chunk_q.reset();
@@ -370,9 +370,28 @@ int main() {
                       r1.value().second.dropout_seed == r2.value().second.dropout_seed &&
                       host_bits_of_bf16(r1.value().first) == host_bits_of_bf16(r2.value().first),
                   "a drawn seed is deterministic after set_seed and kept in the context");
+            // a chunked configuration draws per tile: another kept set, the same function otherwise; chunks that cover
+            // the sequences, and Recompute (which the reference never chunks), give the unchunked draw
+            dc.dropout_seed = 0x2545F4914F6CDD1Dull;
             dc.chunk_q = 64;
+            dc.chunk_kv = 48;
             auto ch = autograd_v4::sdpa_forward(q, k, v, nullptr, dc);
-            CHECK(!ch.ok() && ch.error().kind == Error::Unsupported, "chunked dropout draw must be Unsupported");
+            CHECK(ch.ok() && d1.ok(), "sdpa_forward with a chunked dropout draw failed");
+            if (ch.ok() && d1.ok()) {
+                CHECK(ch.value().second.chunk_cfg == std::make_pair(64, 48), "context keeps the draw tiles");
+                CHECK(host_bits_of_bf16(ch.value().first) != host_bits_of_bf16(d1.value().first), "chunked draw equals the unchunked one");
+                auto gc = autograd_v4::sdpa_backward(ch.value().second, d_o);
+                CHECK(gc.ok(), "sdpa_backward with a chunked draw failed");
+                autograd_v4::SdpaConfig big = dc;
+                big.chunk_q = 1000;
+                big.chunk_kv = 1000;
+                auto same = autograd_v4::sdpa_forward(q, k, v, nullptr, big);
+                CHECK(same.ok() && host_bits_of_bf16(same.value().first) == host_bits_of_bf16(d1.value().first), "chunks beyond the lengths");
+                autograd_v4::SdpaConfig rcp = dc;
+                rcp.save = autograd_v4::SdpaSave::Recompute;
+                auto rr = autograd_v4::sdpa_forward(q, k, v, nullptr, rcp);
+                CHECK(rr.ok() && host_bits_of_bf16(rr.value().first) == host_bits_of_bf16(d1.value().first), "Recompute never chunks the draw");
+            }
         }
         cfg.save = autograd_v4::SdpaSave::SaveProbs;
         CHECK(!autograd_v4::sdpa_forward(q, k, v, nullptr, cfg).ok(), "SaveProbs must be refused");

@@ -106,6 +106,48 @@ def test_dropout_kept_set_bit_exact_through_a_one_hot_value_matrix(oracle):
     assert 0.05 < keep.mean() < 0.95
 
 
+@pytest.mark.parametrize("cq,ck", [(48, 40), (0, 33), (100, 0), (7, 128), (256, 128)])
+def test_chunked_draw_kept_set_bit_exact(oracle, cq, ck):
+    """The kept set of the reference's chunked configuration (one draw per chunk_q x chunk_kv tile, seeded per tile),
+    read off O through a one-hot V; chunks that are not multiples of the kernels' tiles, along one axis only, and
+    covering the whole tensor (the unchunked draw)."""
+    from flame_amd import capi
+    B, H, Sq, Sk, D = 1, 3, 256, 128, 128
+    q, k, _, _ = _inputs(991, B, H, Sq, Sk, D)
+    v = np.zeros((B, H, Sk, D), np.float32)
+    v[..., np.arange(Sk), np.arange(D)] = 1.0
+    p = float(np.quantile(oracle.dropout_uniforms(B, H, Sq, Sk, SEED, cq, ck), 0.4))
+    o, _ = capi.attn_fwd_dropout(to_dev(q), to_dev(k), to_dev(W.f32_to_bf16_bits(v)), 0.05, p, SEED, draw_chunk_q=cq, draw_chunk_kv=ck)
+    torch.cuda.synchronize()
+    keep = oracle.dropout_keep_mask(B, H, Sq, Sk, p, SEED, cq, ck)
+    assert np.array_equal(to_f32(o) != 0, keep)
+    assert 0.05 < keep.mean() < 0.95
+    whole = (cq == 0 or cq >= Sq) and (ck == 0 or ck >= Sk)
+    assert np.array_equal(keep, oracle.dropout_keep_mask(B, H, Sq, Sk, p, SEED)) == whole
+
+
+@pytest.mark.parametrize("B,H,Sq,Sk,D,causal,cq,ck", [(2, 2, 200, 328, 64, False, 48, 100), (1, 2, 320, 256, 128, True, 130, 64)])
+def test_chunked_draw_forward_and_backward_against_oracle(oracle, B, H, Sq, Sk, D, causal, cq, ck):
+    from flame_amd import capi
+    print(f"[dropout tiles] {B}x{H} Sq={Sq} Sk={Sk} D={D} causal={causal} tiles {cq} x {ck}", flush=True)
+    q, k, v, do = _inputs(995 + D, B, H, Sq, Sk, D)
+    scale = 1.0 / np.sqrt(D)
+    p = float(np.quantile(oracle.dropout_uniforms(B, H, Sq, Sk, SEED, cq, ck), 0.25))
+    dq_, dk_, dv_, ddo = (to_dev(t) for t in (q, k, v, do))
+    o, lse = capi.attn_fwd_dropout(dq_, dk_, dv_, scale, p, SEED, causal=causal, draw_chunk_q=cq, draw_chunk_kv=ck)
+    g = capi.attn_bwd_dropout(dq_, dk_, dv_, o, ddo, lse, scale, p, SEED, causal=causal, draw_chunk_q=cq, draw_chunk_kv=ck)
+    torch.cuda.synchronize()
+    ro, rlse, ro32 = oracle.sdpa_fwd_dropout(q, k, v, scale, p, SEED, causal=causal, want_f32=True, chunk_q=cq, chunk_kv=ck)
+    assert_close_bf16(oracle, "O", to_f32(o), ro, ro32, max_abs=DROPOUT_MAX_ABS)
+    assert oracle.max_abs(lse.cpu().numpy().reshape(rlse.shape), rlse) <= TOL_LSE
+    ref = oracle.sdpa_bwd_dropout(q, k, v, ro, do, scale, p, SEED, causal=causal, want_f32=True, chunk_q=cq, chunk_kv=ck)
+    for i, (name, got) in enumerate((("dQ", g[0]), ("dK", g[1]), ("dV", g[2]))):
+        assert_close_bf16(oracle, name, to_f32(got), ref[i], ref[i + 3], max_abs=DROPOUT_MAX_ABS)
+    # teeth: the unchunked kept set gives another output
+    ro_flat, _ = oracle.sdpa_fwd_dropout(q, k, v, scale, p, SEED, causal=causal)
+    assert oracle.rel_l2(to_f32(o), oracle.bf16_to_f32(ro_flat)) > 0.05
+
+
 def test_dropout_argument_checks():
     from flame_amd import capi
     q = torch.zeros((1, 1, 64, 64), dtype=torch.bfloat16, device="cuda")

@@ -102,3 +102,62 @@ def test_backward_with_dropout_against_finite_differences():
     # teeth: the gradient of the undropped function is far from these
     _, _, _, dq_plain, _, dv_plain = O.sdpa_bwd(q, k, v, O.sdpa_fwd(q, k, v, scale)[0], do, scale, want_f32=True)
     assert O.rel_l2(dv_plain, grads[2]) > 0.1 and O.rel_l2(dq_plain, grads[0]) > 0.1
+
+
+# ------------------------------------------------------------------------------------------ the chunked draw
+def _tile_keep_by_hand(seed, bh, i, j, Sq, Sk, cq, ck, p):
+    """derive_tile_seed and the tile's own flat index in Python integers (src/autograd_v4/ops/sdpa.rs:600-602, :604-649):
+    the tile tensor is [B*H, q_t, k_t], its seed (seed + ((q_offset << 32) ^ k_offset)) truncated to 32 bits."""
+    q_off, k_off = (i // cq) * cq, (j // ck) * ck
+    q_t, k_t = min(cq, Sq - q_off), min(ck, Sk - k_off)
+    tile_seed = ((seed + ((q_off << 32) ^ k_off)) & (2 ** 64 - 1)) & 0xFFFFFFFF
+    return _keep_by_hand(tile_seed, (bh * q_t + (i - q_off)) * k_t + (j - k_off), p)
+
+
+def test_chunked_draw_follows_the_tile_seeds_and_indices():
+    seed, Sq, Sk, cq, ck = 0x2545F4914F6CDD1D, 10, 7, 4, 3
+    # written out once: element (bh 2, query 9, key 6) lies in the tile at offsets (8, 6) of size 2 x 1, where it has
+    # flat index (2 * 2 + 1) * 1 + 0 = 5, and the tile's seed is the low word of seed + 6 (the query offset is shifted
+    # out of it)
+    assert ((seed + ((8 << 32) ^ 6)) & 0xFFFFFFFF) == ((seed & 0xFFFFFFFF) + 6) & 0xFFFFFFFF
+    for p in (0.2, 0.5, 0.8):
+        assert O.dropout_keep_tiled(seed, 2, 9, 6, Sq, Sk, cq, ck, p) == bool(_keep_by_hand((seed & 0xFFFFFFFF) + 6, 5, p))
+    u = O.dropout_uniforms(2, 2, Sq, Sk, seed, cq, ck).reshape(4, Sq, Sk)
+    for p in (0.3, 0.6):
+        for bh in range(4):
+            for i in range(Sq):
+                for j in range(Sk):
+                    want = bool(_tile_keep_by_hand(seed, bh, i, j, Sq, Sk, cq, ck, p))
+                    assert O.dropout_keep_tiled(seed, bh, i, j, Sq, Sk, cq, ck, p) == want
+                    assert bool(u[bh, i, j] >= np.float32(p)) == want
+    # chunks that cover the whole axes are the unchunked draw; a chunk along the queries alone changes the indices only
+    assert np.array_equal(O.dropout_uniforms(2, 2, Sq, Sk, seed, Sq, Sk), O.dropout_uniforms(2, 2, Sq, Sk, seed))
+    assert np.array_equal(O.dropout_uniforms(2, 2, Sq, Sk, seed, 100, 0), O.dropout_uniforms(2, 2, Sq, Sk, seed))
+    assert not np.array_equal(O.dropout_uniforms(2, 2, Sq, Sk, seed, 4, 0), O.dropout_uniforms(2, 2, Sq, Sk, seed))
+    # a low seed word that wraps with the key offset
+    s2 = 0xFFFFFFFF_FFFFFFFE
+    assert O.dropout_keep_tiled(s2, 0, 1, 5, 4, 8, 2, 4, 0.5) == bool(_keep_by_hand((0xFFFFFFFE + 4) & 0xFFFFFFFF, (0 * 2 + 1) * 4 + 1, 0.5))
+
+
+def test_forward_and_backward_with_a_chunked_draw_against_fp64():
+    B, H, Sq, Sk, D, seed, cq, ck = 1, 2, 12, 20, 8, 0x5DEECE66D, 5, 8
+    p = float(np.median(O.dropout_uniforms(B, H, Sq, Sk, seed, cq, ck)))
+    q, k, v, do = (W.f32_to_bf16_bits(W.normal_f32(821, s, B * H * n * D).reshape(B, H, n, D)) for s, n in enumerate((Sq, Sk, Sk, Sq)))
+    f = [O.bf16_to_f32(t).astype(np.float64) for t in (q, k, v)]
+    g = O.bf16_to_f32(do).astype(np.float64)
+    m = O.dropout_keep_mask(B, H, Sq, Sk, p, seed, cq, ck)
+    assert not np.array_equal(m, O.dropout_keep_mask(B, H, Sq, Sk, p, seed)) and 0.05 < m.mean() < 0.95
+    factor = np.float64(np.float32(1.0) / (np.float32(1.0) - np.float32(p)))
+    _, lse64, p64 = O.brute_sdpa_f64(*f, 0.3)
+    pd = p64 * m * factor
+    o, lse, o32 = O.sdpa_fwd_dropout(q, k, v, 0.3, p, seed, want_f32=True, chunk_q=cq, chunk_kv=ck)
+    assert np.abs(o32 - pd @ f[2]).max() < 2e-5 and np.abs(lse - lse64).max() < 2e-5
+    # closed-form gradients of sum(g * (P m f) V) in fp64, with the oracle's D = rowsum(dO * O_bf16) convention
+    _, _, _, dq32, dk32, dv32 = O.sdpa_bwd_dropout(q, k, v, o, do, 0.3, p, seed, want_f32=True, chunk_q=cq, chunk_kv=ck)
+    dv = np.swapaxes(pd, -1, -2) @ g
+    dpd = g @ np.swapaxes(f[2], -1, -2)
+    dp = dpd * m * factor
+    delta = (g * O.bf16_to_f32(o).astype(np.float64)).sum(-1, keepdims=True)
+    ds = p64 * (dp - delta) * 0.3
+    assert O.max_abs(dv32, dv) < 1e-5
+    assert O.max_abs(dq32, ds @ f[1]) < 1e-5 and O.max_abs(dk32, np.swapaxes(ds, -1, -2) @ f[0]) < 1e-5
