@@ -30,18 +30,34 @@ def hipcc_version() -> str:
     return f"{hip} clang-{clang}"
 
 
-def build_lib(verbose: bool = False, extra=()) -> str:
-    os.makedirs(LIB_DIR, exist_ok=True)
-    src = os.path.join(CSRC, "flame_attn.hip")
-    cmd = [HIPCC, *FLAGS, f'-DFLAME_ATTN_HIPCC_VERSION="{hipcc_version()}"', *extra, src, "-o", LIB_PATH]
+STATIC_LIB_PATH = os.path.join(LIB_DIR, "libflame_attn_hip.a")
+
+
+def _run(cmd, verbose):
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     out = "\n".join(l for l in res.stdout.splitlines() if "packed-fp32-ops" not in l)
     if res.returncode != 0:
-        raise RuntimeError("hipcc failed:\n" + out)
+        raise RuntimeError(f"{os.path.basename(cmd[0])} failed:\n" + out)
     if verbose and out.strip():
         print(out)
+
+
+def build_lib(verbose: bool = False, extra=()) -> str:
+    """One compilation of flame_attn.hip to an object, from which both the shared library (what the tests, the
+    benchmark and the ctypes binding load) and the static archive (what a Rust build script links, as the reference's
+    build.rs links its own kernels) are made."""
+    os.makedirs(LIB_DIR, exist_ok=True)
+    src = os.path.join(CSRC, "flame_attn.hip")
+    obj = os.path.join(LIB_DIR, "flame_attn.o")
+    compile_flags = [f for f in FLAGS if f != "-shared"]
+    _run([HIPCC, *compile_flags, f'-DFLAME_ATTN_HIPCC_VERSION="{hipcc_version()}"', *extra, "-c", src, "-o", obj], verbose)
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", obj, "-o", LIB_PATH], verbose)
+    if os.path.exists(STATIC_LIB_PATH):
+        os.remove(STATIC_LIB_PATH)
+    _run(["ar", "rcs", STATIC_LIB_PATH, obj], verbose)
+    os.remove(obj)
     return LIB_PATH
 
 

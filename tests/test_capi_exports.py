@@ -40,6 +40,24 @@ def test_library_exports_every_declared_symbol():
     assert not missing, missing
 
 
+def test_static_archive_defines_every_declared_symbol():
+    """libflame_attn_hip.a is what a Rust build script links (the reference's build.rs links its kernels statically);
+    it is made from the same object as the shared library."""
+    import shutil
+    import subprocess
+    _lib()
+    archive = os.path.join(os.path.dirname(LIB), "libflame_attn_hip.a")
+    if not os.path.exists(archive):
+        from flame_amd import build
+        build.build_lib()
+    if shutil.which("nm") is None:
+        pytest.skip("nm not available")
+    out = subprocess.run(["nm", "--defined-only", archive], stdout=subprocess.PIPE, text=True, check=True).stdout
+    defined = {l.split()[-1] for l in out.splitlines() if len(l.split()) == 3 and l.split()[1] == "T"}
+    missing = [n for n in _declared_functions() if n not in defined]
+    assert not missing, missing
+
+
 def test_argument_validation_without_a_device():
     lib = _lib()
     lib.flame_attn_bwd_workspace_bytes.restype = ctypes.c_size_t
