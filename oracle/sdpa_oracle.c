@@ -42,6 +42,10 @@
  *                    ki8*sk[block] with block magnitudes 4-8x apart and short last blocks (O and LSE
  *                    within 2e-5), with a control that a wrong block index fails
  *   row bands        pinned: bit-identical to the rows of the full computation
+ *   dropout          (src/autograd_v4/ops/sdpa.rs:229-231, :444, :600-649; generator src/rng/mod.rs:14-24) pinned:
+ *                    the kept set of the unchunked and of the chunked draw against the xorshift recurrence, the
+ *                    tile seeds and the tiles' own flat indices in Python integers; forward against fp64 attention
+ *                    with that set; backward against fp64 central differences and closed-form fp64 gradients
  *
  * Layout: every tensor is contiguous [B,H,S,D]; bf16 is carried as uint16_t.
  */
