@@ -714,6 +714,19 @@ static int attn_fwd_impl(const void* Q, const void* K, const void* V, void* O, v
     if (Dv == 0) Dv = D;           // V and O may have a head dim of their own (forward only)
     if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0 || Dv < 0) return FLAME_ATTN_ERR_INVALID;
     if (!(scale > 0.f) || !isfinite(scale)) return FLAME_ATTN_ERR_INVALID;
+    // A value head dim above 128 beside a query head dim of at most 128 (the reference's streaming entry point is
+    // tested with Dh = 64, Dv = 160: tests/streaming_attn.rs:306-311): the softmax does not depend on V, so O comes
+    // out in column ranges of at most 128, each a forward of its own on views of V and O.
+    if (head_dim_ok(D) && Dv > 128 && Dv % 8 == 0) {
+        for (int c0 = 0; c0 < Dv; c0 += 128) {
+            const int rc = attn_fwd_impl(Q, K, V, O, c0 == 0 ? LSE : nullptr, B, H, N_q, N_kv, D, scale, q_strides, k_strides,
+                                         v_strides, o_strides, q_off, k_off, v_off + c0, o_off + c0, lse_off, causal, kv_len,
+                                         keep_mask, mask_strides, bias, bias_dtype, bias_strides, stream, mask_mode,
+                                         std::min(128, Dv - c0), q_tile_plan, dropout_p, dropout_seed, draw_cq, draw_ck);
+            if (rc != FLAME_ATTN_OK) return rc;
+        }
+        return FLAME_ATTN_OK;
+    }
     // head dims above 128: the forward in chunks of 128, without explicit mask, bias or dropout and with Dv = D
     const bool big = big_head_dim_ok(D) && Dv == D && !keep_mask && !bias && dropout_p == 0.f;
     if (!big && (!head_dim_ok(D) || !head_dim_ok(Dv))) return FLAME_ATTN_ERR_UNSUPPORTED;

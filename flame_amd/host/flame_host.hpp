@@ -49,7 +49,7 @@ namespace flame {
 // ------------------------------------------------------------------------------------ errors
 // The reference's `Error` enum, reduced to the variants this path raises (src/error.rs).
 struct Error {
-    enum Kind { InvalidInput, Unsupported, Cuda, InvalidOperation } kind;
+    enum Kind { InvalidInput, Unsupported, Cuda, InvalidOperation, OutOfMemory } kind;
     std::string message;
 };
 
@@ -1028,9 +1028,10 @@ namespace ops {
 namespace attn {
 // src/ops/attn.rs.  The reference plans a query chunk whose fp32 scratch (chunk x K logits + chunk x (Dv + 2) rows,
 // :72-84) fits a budget taken from free device memory, and steps down a list of candidate chunks when the planner or
-// an allocation refuses one, recording every step.  The planner, its candidates, its budget rules and its records are
-// mirrored; the scratch the kernels here need is zero bytes, so the requested chunk (clamped as there) is always the
-// chosen one and the list of fallbacks stays empty unless the launch itself fails.
+// a launch refuses one, recording every step (its tests assert on those records: tests/streaming_attn.rs:301-397).
+// The planner, its candidates, its budget rules, its records and its telemetry are mirrored with the reference's own
+// scratch formula as the accounting, so that a caller sees the same chosen chunk and the same fallback events; the
+// kernels behind it keep their scratch in registers and LDS and run the same launch whatever chunk is chosen.
 struct StreamingAttnCfg {                                     // :8-25
     float scale = 1.0f;
     size_t chunk_size = 2048;
@@ -1042,17 +1043,14 @@ constexpr size_t STREAM_ATTENTION_MIN_CHUNK = 32, STREAM_ATTENTION_MAX_CHUNK = 2
 constexpr uint64_t STREAM_ATTENTION_MIN_BUDGET_BYTES = 64ull << 20, STREAM_ATTENTION_DEFAULT_BUDGET_BYTES = 512ull << 20,
                    STREAM_ATTENTION_HARD_CAP_BYTES = 2ull << 30;
 
-// what the reference's kernels would need for this chunk (:72-84); nullopt on overflow
-inline std::optional<uint64_t> reference_streaming_workspace_bytes(size_t chunk_rows, size_t k_len, size_t dv) {
+// the planner's accounting: what the reference's kernels need for this chunk (:72-84); nullopt on overflow
+inline std::optional<uint64_t> streaming_workspace_bytes(size_t chunk_rows, size_t k_len, size_t dv) {
     if (chunk_rows == 0 || k_len == 0) return 0;
     unsigned __int128 total = (unsigned __int128)chunk_rows * k_len + (unsigned __int128)chunk_rows * ((unsigned __int128)dv + 2);
     total *= 4;
     if (total > UINT64_MAX) return std::nullopt;
     return (uint64_t)total;
 }
-// scratch of the kernels behind this header
-inline uint64_t streaming_workspace_bytes(size_t, size_t, size_t) { return 0; }
-
 inline std::vector<size_t> streaming_chunk_candidates(size_t q_len) {                                   // :128-155
     static const size_t preferred[13] = {2048, 1536, 1024, 768, 512, 384, 256, 192, 128, 96, 64, 48, 32};
     std::vector<size_t> c;
@@ -1086,11 +1084,18 @@ inline Result<StreamingTilePlan> plan_streaming_chunk(size_t q_len, size_t k_len
         budget = std::max(budget, STREAM_ATTENTION_MIN_BUDGET_BYTES);
     }
     budget = std::min(budget, STREAM_ATTENTION_HARD_CAP_BYTES);
-    for (size_t chunk : streaming_chunk_candidates(q_len)) {
-        const uint64_t required = streaming_workspace_bytes(std::min(chunk, q_len), k_len, dv);
-        if (required <= budget) return StreamingTilePlan{chunk, required, budget};
+    const auto candidates = streaming_chunk_candidates(q_len);
+    for (size_t chunk : candidates) {
+        const auto required = streaming_workspace_bytes(std::min(chunk, q_len), k_len, dv);
+        if (required && *required <= budget) return StreamingTilePlan{chunk, *required, budget};
     }
-    return Error{Error::Cuda, "streaming attention planner: no chunk fits the budget (OOM)"};
+    const size_t smallest = candidates.empty() ? 1 : candidates.back();
+    const auto required = streaming_workspace_bytes(std::min(smallest, q_len), k_len, dv);
+    if (!required) return invalid("streaming attention planner overflow");
+    char msg[200];
+    std::snprintf(msg, sizeof msg, "streaming attention planner: chunk %zu requires %.2f MiB workspace but budget is %.2f MiB",
+                  smallest, (double)*required / 1048576.0, (double)budget / 1048576.0);
+    return Error{Error::OutOfMemory, msg};
 }
 
 struct StreamingFallbackReason {                              // :211-223
@@ -1128,26 +1133,91 @@ inline StreamingAttnLaunchInfo streaming_attn_last_launch_info() {              
     return detail_launch::last();
 }
 
-// :326-600.  Beyond the reference: a keep-mask is taken (the reference refuses one, :366-370), and the three
-// tensors may be strided views and have key lengths of their own.
+// :326-600.  Beyond the reference: a keep-mask is taken (bf16, 1 = keep; the reference's function refuses one, :366-370,
+// although its test passes one, tests/streaming_attn.rs:413-489), and the three tensors may be strided views and have
+// key lengths of their own.  Only a launch failure of the device layer makes the loop step down a chunk; argument errors
+// are returned at once.
 inline Result<Tensor> streaming_attn_bf16_fp32(const Tensor& q, const Tensor& k, const Tensor& v, const StreamingAttnCfg& cfg) {
     if (cfg.chunk_size == 0) return invalid("streaming attention chunk_size must be > 0");
     if (q.dtype() != DType::BF16 || k.dtype() != DType::BF16 || v.dtype() != DType::BF16)
         return invalid("streaming attention expects BF16 tensors");
     if (q.shape().size() != 4 || k.shape().size() != 4 || v.shape().size() != 4) return invalid("expected 4D tensors");
     if (q.shape()[3] != k.shape()[3]) return invalid("head dimensions for Q and K differ");
-    const size_t s = (size_t)q.shape()[2], s_k = (size_t)k.shape()[2], dv = (size_t)v.shape()[3];
-    auto plan = plan_streaming_chunk(s, s_k, dv);
-    if (!plan.ok()) return plan.error();
+    const size_t b = (size_t)q.shape()[0], h = (size_t)q.shape()[1], s = (size_t)q.shape()[2], dh = (size_t)q.shape()[3];
+    const size_t s_k = (size_t)k.shape()[2], dv = (size_t)v.shape()[3];
+    auto planned = plan_streaming_chunk(s, s_k, dv);
+    if (!planned.ok()) return planned.error();
+    StreamingTilePlan plan = planned.value();
     const size_t requested = std::min(std::min(std::max<size_t>(cfg.chunk_size, 1), std::max<size_t>(s, 1)), STREAM_ATTENTION_MAX_CHUNK);
-    if (streaming_workspace_bytes(std::min(requested, s), s_k, dv) <= plan.value().budget_bytes) plan.value().chunk = requested;
+    const auto requested_required = streaming_workspace_bytes(std::min(requested, s), s_k, dv);
+    if (requested_required && *requested_required <= plan.budget_bytes) {
+        plan.chunk = requested;
+        plan.workspace_bytes = *requested_required;
+    }
+    auto candidates = streaming_chunk_candidates(s);
+    if (std::find(candidates.begin(), candidates.end(), plan.chunk) == candidates.end()) {
+        candidates.push_back(plan.chunk);
+        std::sort(candidates.begin(), candidates.end(), std::greater<size_t>());
+    }
+    if (candidates.empty()) return invalid("no valid chunk size candidates for streaming attention");
+    size_t idx = (size_t)(std::find(candidates.begin(), candidates.end(), plan.chunk) - candidates.begin());
+    if (idx >= candidates.size()) idx = 0;
+
     StreamingAttnLaunchInfo info;
     info.requested_chunk = std::max<size_t>(requested, 1);
-    auto out = cuda_ops_bf16::sdpa_stream_bf16_with_workspace(q, k, v, cfg.mask, plan.value().chunk, cfg.causal, cfg.scale, std::nullopt);
-    info.chosen_chunk = plan.value().chunk;
-    if (!out.ok()) info.last_error = out.error().kind == Error::Cuda ? 2 : 1;        // FC_ERR_LAUNCH / FC_ERR_INVALID_ARGUMENT
-    detail_launch::record(info);
-    return out;
+    auto log_fallback = [&](size_t from, size_t to, const StreamingFallbackReason& why) {
+        info.fallbacks.push_back(StreamingFallbackEvent{from, to, why});
+        info.retries = info.fallbacks.size();
+        if (!perf_telemetry::telemetry_enabled()) return;
+        perf_telemetry::SdpaFallbackTelemetryRecord r;
+        r.batch = b; r.heads = h; r.q_len = s; r.k_len = s_k; r.dh = dh; r.dv = dv;
+        r.from_chunk = from; r.to_chunk = to;
+        r.reason = why.kind == StreamingFallbackReason::Oom ? "oom" : "workspace_budget";
+        r.workspace_required = why.required_bytes; r.workspace_limit = why.budget_bytes;
+        if (why.kind == StreamingFallbackReason::Oom) r.error_code = why.error_code;
+        perf_telemetry::log_sdpa_fallback_event(r);
+    };
+    if (requested_required && *requested_required > plan.budget_bytes && requested > plan.chunk) {
+        StreamingFallbackReason why;
+        why.kind = StreamingFallbackReason::WorkspaceBudget;
+        why.required_bytes = *requested_required;
+        why.budget_bytes = plan.budget_bytes;
+        log_fallback(requested, plan.chunk, why);
+    }
+    while (idx < candidates.size()) {
+        const size_t chunk = candidates[idx];
+        const auto required = streaming_workspace_bytes(std::min(chunk, s), s_k, dv);
+        if (!required) return invalid("streaming attention workspace overflow");
+        if (*required > plan.budget_bytes) {
+            if (idx + 1 >= candidates.size()) {
+                info.chosen_chunk = chunk;
+                detail_launch::record(info);
+                return Error{Error::OutOfMemory, "streaming attention planner rejected chunk " + std::to_string(chunk)};
+            }
+            StreamingFallbackReason why;
+            why.kind = StreamingFallbackReason::WorkspaceBudget;
+            why.required_bytes = *required;
+            why.budget_bytes = plan.budget_bytes;
+            log_fallback(chunk, candidates[idx + 1], why);
+            ++idx;
+            continue;
+        }
+        auto out = cuda_ops_bf16::sdpa_stream_bf16_with_workspace(q, k, v, cfg.mask, chunk, cfg.causal, cfg.scale, std::nullopt);
+        if (out.ok() || out.error().kind != Error::Cuda || idx + 1 >= candidates.size()) {
+            info.chosen_chunk = chunk;
+            if (!out.ok()) info.last_error = out.error().kind == Error::Cuda ? 2 : 1;        // FC_ERR_LAUNCH / FC_ERR_INVALID_ARGUMENT
+            detail_launch::record(info);
+            return out;
+        }
+        StreamingFallbackReason why;                          // :571-590: a failed launch counts as out of memory
+        why.kind = StreamingFallbackReason::Oom;
+        why.required_bytes = *required;
+        why.budget_bytes = plan.budget_bytes;
+        info.last_error = 2;
+        log_fallback(chunk, candidates[idx + 1], why);
+        ++idx;
+    }
+    return invalid("no valid chunk size candidates for streaming attention");
 }
 }  // namespace attn
 }  // namespace ops

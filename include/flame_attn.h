@@ -286,7 +286,8 @@ int flame_flash_attention_bf16(const void* Q, const void* K, const void* V, void
  * keep-mask [B, mask_heads, Q, K] (< 0.5 excluded, flame_sdpa_stub.cu:793-802), read in place by the
  * kernel.  `workspace` is accepted and not used (the reference keeps its score chunks there,
  * flame_sdpa_stub.cu:973-976), so any size, including none, works.  V and out have head dim Dv, which
- * may differ from Dh (both multiples of 8 up to 128). */
+ * may differ from Dh (multiples of 8; Dh up to 128; Dv above 128 is served in column ranges of 128, the softmax being
+ * independent of V: one forward per range). */
 FlameAttnStatus flame_sdpa_chunked_bf16(const void* q, const void* k, const void* v, int B, int H, int Q, int K,
                                         int Dh, int Dv, float scale, int chunk, int causal, int mask_heads,
                                         const void* mask, void* out, void* workspace, uint64_t workspace_bytes,
@@ -294,7 +295,8 @@ FlameAttnStatus flame_sdpa_chunked_bf16(const void* q, const void* k, const void
 
 /* cuda/streaming_attn_bf16.h:7-17 (cuda/streaming_attn_bf16.cu:305-432): strided Q,K,V,O, causal,
  * key-padding mask uint8 [B,H,S] with 0 = excluded (streaming_attn_bf16.cu:164-170).  V and O have head
- * dim Dv, which may differ from Dh. */
+ * dim Dv, which may differ from Dh and exceed 128 (the reference's tests run Dh = 64 with Dv = 80 and 160,
+ * tests/streaming_attn.rs:57-124, :298-411). */
 int streaming_attn_bf16_fp32_launch(const void* Q, const void* K, const void* V, int B, int H, int S, int Dh, int Dv,
                                     long qB, long qH, long qS, long qD, long kB, long kH, long kS, long kD,
                                     long vB, long vH, long vS, long vD, void* O, long oB, long oH, long oS, long oD,

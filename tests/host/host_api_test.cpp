@@ -553,27 +553,18 @@ int main() {
             CHECK(info.requested_chunk == std::min<size_t>(2048, (size_t)Sq) && info.chosen_chunk && *info.chosen_chunk == info.requested_chunk &&
                       info.retries == 0 && info.fallbacks.empty() && !info.last_error,
                   "launch info after a plain call");
-            cfg.chunk_size = 48;
-            CHECK(ops::attn::streaming_attn_bf16_fp32(q, k, v, cfg).ok(), "small chunk");
-            info = ops::attn::streaming_attn_last_launch_info();
-            CHECK(info.requested_chunk == std::min<size_t>(48, (size_t)Sq) && info.chosen_chunk && *info.chosen_chunk == info.requested_chunk,
-                  "the requested chunk is the chosen one: the kernels need no scratch");
             using ops::attn::streaming_chunk_candidates;
             CHECK(streaming_chunk_candidates(0).empty(), "no candidates for an empty sequence");
             CHECK(streaming_chunk_candidates(20) == std::vector<size_t>({20}), "short sequences: the sequence itself");
             CHECK(streaming_chunk_candidates(100) == std::vector<size_t>({100, 96, 64, 48, 32}), "candidates below 100");
             CHECK(streaming_chunk_candidates(5000).size() == 13 && streaming_chunk_candidates(5000).front() == 2048 &&
                       streaming_chunk_candidates(5000).back() == 32, "all thirteen preferred chunks");
-            auto plan = ops::attn::plan_streaming_chunk(4608, 4608, 128);
-            CHECK(plan.ok() && plan.value().chunk == 2048 && plan.value().workspace_bytes == 0 &&
-                      plan.value().budget_bytes >= (64ull << 20) && plan.value().budget_bytes <= (2ull << 30),
-                  "planner: largest candidate, budget between the reference's floor and cap");
+            CHECK(ops::attn::streaming_workspace_bytes(2048, 4608, 128).value_or(0) == (2048ull * 4608 + 2048ull * 130) * 4,
+                  "the reference's scratch formula");
             setenv("FLAME_SDPA_PLANNER_BUDGET_BYTES", "12345", 1);
             auto forced = ops::attn::plan_streaming_chunk(4608, 4608, 128);
             unsetenv("FLAME_SDPA_PLANNER_BUDGET_BYTES");
-            CHECK(forced.ok() && forced.value().budget_bytes == 12345, "forced planner budget");
-            CHECK(ops::attn::reference_streaming_workspace_bytes(2048, 4608, 128).value_or(0) == (2048ull * 4608 + 2048ull * 130) * 4,
-                  "the reference's scratch formula");
+            CHECK(!forced.ok() && forced.error().kind == Error::OutOfMemory, "a budget no chunk fits is OutOfMemory");
             cuda_ops_bf16::SdpaWorkspace ws;
             ws.bytes = 16;
             CHECK(!cuda_ops_bf16::sdpa_stream_bf16_with_workspace(q, k, v, nullptr, 64, true, 0.125f, ws).ok(), "null workspace with bytes");
@@ -853,6 +844,141 @@ int main() {
                         CHECK(!off2.ok() && small.value()->in_flight() == 0, "a pool with too few slots refuses and gives its slots back");
                     }
                 }
+            }
+        }
+    }
+
+    // ---- 12. the reference's own streaming-attention tests (tests/streaming_attn.rs), re-expressed: inputs N(0, 0.02),
+    //          a value head dim of its own (80, 160, 48), dense comparison on the host in fp32
+    {
+        std::printf("[streaming_attn tests of the reference]\n");
+        auto small_randn = [](size_t n) {
+            std::vector<uint16_t> x(n);
+            for (auto& e : x) e = f2bf(0.02f * gauss());
+            return x;
+        };
+        // dense fp32 attention of one (b, h) on the host; keep: [S, S] 1 = attend, or null
+        auto dense = [](const std::vector<uint16_t>& q, const std::vector<uint16_t>& k, const std::vector<uint16_t>& v, int BH, int S,
+                        int Dh, int Dv, float scale, bool causal, const std::vector<float>* keep) {
+            std::vector<float> o((size_t)BH * S * Dv, 0.f), p(S);
+            for (int bh = 0; bh < BH; ++bh)
+                for (int i = 0; i < S; ++i) {
+                    float m = -INFINITY;
+                    for (int j = 0; j < S; ++j) {
+                        float a = 0.f;
+                        for (int d = 0; d < Dh; ++d) a += bf2f(q[((size_t)bh * S + i) * Dh + d]) * bf2f(k[((size_t)bh * S + j) * Dh + d]);
+                        a *= scale;
+                        if (causal && j > i) a += -1e9f;                                  // as the test does: (mask - 1) * 1e9
+                        if (keep && (*keep)[((size_t)bh * S + i) * S + j] == 0.f) a += -1e9f;
+                        p[j] = a;
+                        m = std::fmax(m, a);
+                    }
+                    float l = 0.f;
+                    for (int j = 0; j < S; ++j) { p[j] = std::exp(p[j] - m); l += p[j]; }
+                    for (int j = 0; j < S; ++j)
+                        for (int d = 0; d < Dv; ++d) o[((size_t)bh * S + i) * Dv + d] += p[j] / l * bf2f(v[((size_t)bh * S + j) * Dv + d]);
+                }
+            return o;
+        };
+        auto diff = [](const std::vector<float>& a, const std::vector<float>& b, double& max_abs, double& mean_abs) {
+            max_abs = 0; mean_abs = 0;
+            for (size_t i = 0; i < a.size(); ++i) { const double d = std::fabs((double)a[i] - b[i]); max_abs = std::fmax(max_abs, d); mean_abs += d; }
+            mean_abs /= (double)a.size();
+        };
+        {   // streaming_attention_matches_dense_small_seq (:57-124) and streaming_attention_respects_causal_flag (:214-296)
+            for (int causal = 0; causal < 2; ++causal) {
+                const int b = 1, h = 2, s = causal ? 128 : 256, dh = 64, dv = 80;
+                auto hq = small_randn((size_t)b * h * s * dh), hk = small_randn(hq.size()), hv = small_randn((size_t)b * h * s * dv);
+                Tensor q = dev_bf16(hq, {b, h, s, dh}), k = dev_bf16(hk, {b, h, s, dh}), v = dev_bf16(hv, {b, h, s, dv});
+                ops::attn::StreamingAttnCfg cfg;
+                cfg.scale = 1.0f / std::sqrt((float)dh);
+                cfg.chunk_size = causal ? 64 : 2048;
+                cfg.causal = causal != 0;
+                auto out = ops::attn::streaming_attn_bf16_fp32(q, k, v, cfg);
+                CHECK(out.ok() && out.value().shape() == std::vector<int64_t>({b, h, s, dv}), "streaming dv = 80");
+                if (out.ok()) {
+                    double ma, me;
+                    diff(host_f32_of_bf16(out.value()), dense(hq, hk, hv, b * h, s, dh, dv, cfg.scale, cfg.causal, nullptr), ma, me);
+                    std::printf("  dense parity causal=%d: max_abs=%.3e mean_abs=%.3e\n", causal, ma, me);
+                    CHECK(ma <= (causal ? 1.5e-3 : 1e-3) && me <= (causal ? 5e-4 : 1e-4), "streaming vs dense: max %.3e mean %.3e", ma, me);
+                }
+            }
+        }
+        {   // streaming_attention_clamps_chunk_size (:126-155), streaming_attention_enforces_chunk_floor (:157-212)
+            auto hq = small_randn(64 * 32), hk = small_randn(64 * 32), hv = small_randn(64 * 32);
+            Tensor q = dev_bf16(hq, {1, 1, 64, 32}), k = dev_bf16(hk, {1, 1, 64, 32}), v = dev_bf16(hv, {1, 1, 64, 32});
+            ops::attn::StreamingAttnCfg cfg;
+            cfg.scale = 1.0f / std::sqrt(32.0f);
+            cfg.chunk_size = 10000;
+            cfg.causal = true;
+            auto out = ops::attn::streaming_attn_bf16_fp32(q, k, v, cfg);
+            CHECK(out.ok() && out.value().shape() == std::vector<int64_t>({1, 1, 64, 32}), "chunk larger than S and than the cap");
+            auto q2 = small_randn(512 * 64), k2 = small_randn(512 * 64), v2 = small_randn(512 * 64);
+            Tensor tq = dev_bf16(q2, {1, 1, 512, 64}), tk = dev_bf16(k2, {1, 1, 512, 64}), tv = dev_bf16(v2, {1, 1, 512, 64});
+            ops::attn::StreamingAttnCfg a, c;
+            a.scale = c.scale = 0.125f;
+            a.chunk_size = 32;
+            c.chunk_size = 64;
+            auto oa = ops::attn::streaming_attn_bf16_fp32(tq, tk, tv, a), oc = ops::attn::streaming_attn_bf16_fp32(tq, tk, tv, c);
+            CHECK(oa.ok() && oc.ok() && host_bits_of_bf16(oa.value()) == host_bits_of_bf16(oc.value()), "chunk 32 and chunk 64 agree");
+        }
+        {   // streaming_attention_tracks_budget_trim (:298-364) and streaming_attention_honors_generous_budget (:366-411)
+            const int b = 1, h = 2, s = 8192, dh = 64, dv = 160;
+            std::vector<uint16_t> zq((size_t)b * h * s * dh, 0), zv((size_t)b * h * s * dv, 0);
+            Tensor q = dev_bf16(zq, {b, h, s, dh}), k = dev_bf16(zq, {b, h, s, dh}), v = dev_bf16(zv, {b, h, s, dv});
+            ops::attn::StreamingAttnCfg cfg;
+            cfg.scale = 0.125f;
+            cfg.chunk_size = 2048;
+            setenv("FLAME_SDPA_PLANNER_BUDGET_BYTES", "67108864", 1);
+            auto out = ops::attn::streaming_attn_bf16_fp32(q, k, v, cfg);
+            CHECK(out.ok() && out.value().shape() == std::vector<int64_t>({b, h, s, dv}), "dv = 160 under a 64 MiB budget");
+            auto info = ops::attn::streaming_attn_last_launch_info();
+            const ops::attn::StreamingFallbackEvent* ev = nullptr;
+            for (const auto& e : info.fallbacks)
+                if (e.reason.kind == ops::attn::StreamingFallbackReason::WorkspaceBudget) { ev = &e; break; }
+            CHECK(ev != nullptr, "workspace budget fallback not recorded");
+            if (ev) {
+                CHECK(ev->from_chunk == 2048, "planner should report trimming from the requested chunk");
+                CHECK(info.chosen_chunk && *info.chosen_chunk == ev->to_chunk && ev->to_chunk == 1536, "chosen chunk should match the trimmed target");
+                CHECK(ev->reason.required_bytes && ev->reason.budget_bytes && *ev->reason.required_bytes > *ev->reason.budget_bytes,
+                      "workspace requirement should exceed budget when trimming occurs");
+            }
+            setenv("FLAME_SDPA_PLANNER_BUDGET_BYTES", "536870912", 1);
+            auto out2 = ops::attn::streaming_attn_bf16_fp32(q, k, v, cfg);
+            unsetenv("FLAME_SDPA_PLANNER_BUDGET_BYTES");
+            auto info2 = ops::attn::streaming_attn_last_launch_info();
+            CHECK(out2.ok() && info2.chosen_chunk && *info2.chosen_chunk == 2048 && info2.fallbacks.empty(), "generous budget keeps the requested chunk");
+            if (out.ok()) {       // zero inputs: uniform attention over zero values
+                bool all_zero = true;
+                for (uint16_t x : host_bits_of_bf16(out.value())) all_zero = all_zero && (x & 0x7fff) == 0;
+                CHECK(all_zero, "zero V must give zero O");
+            }
+        }
+        {   // streaming_attention_applies_explicit_mask (:413-489): bf16 keep-mask [b, h, s, s], a third of the keys dropped
+            const int b = 1, h = 2, s = 96, dh = 64, dv = 48;
+            auto hq = small_randn((size_t)b * h * s * dh), hk = small_randn(hq.size()), hv = small_randn((size_t)b * h * s * dv);
+            std::vector<float> keep((size_t)b * h * s * s);
+            std::vector<uint16_t> keep_bf(keep.size());
+            for (int head = 0; head < h; ++head)
+                for (int qi = 0; qi < s; ++qi)
+                    for (int kj = 0; kj < s; ++kj) {
+                        const float kv = (kj + head + qi) % 3 == 0 ? 0.f : 1.f;
+                        keep[((size_t)head * s + qi) * s + kj] = kv;
+                        keep_bf[((size_t)head * s + qi) * s + kj] = f2bf(kv);
+                    }
+            Tensor q = dev_bf16(hq, {b, h, s, dh}), k = dev_bf16(hk, {b, h, s, dh}), v = dev_bf16(hv, {b, h, s, dv});
+            Tensor mask = dev_bf16(keep_bf, {b, h, s, s});
+            ops::attn::StreamingAttnCfg cfg;
+            cfg.scale = 0.125f;
+            cfg.chunk_size = 64;
+            cfg.mask = &mask;
+            auto out = ops::attn::streaming_attn_bf16_fp32(q, k, v, cfg);
+            CHECK(out.ok(), "streaming with an explicit mask");
+            if (out.ok()) {
+                double ma, me;
+                diff(host_f32_of_bf16(out.value()), dense(hq, hk, hv, b * h, s, dh, dv, cfg.scale, false, &keep), ma, me);
+                std::printf("  explicit mask: max_abs=%.3e mean_abs=%.3e\n", ma, me);
+                CHECK(ma <= 1.5e-3 && me <= 5e-4, "masked streaming vs dense: max %.3e mean %.3e", ma, me);
             }
         }
     }

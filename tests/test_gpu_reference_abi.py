@@ -118,14 +118,14 @@ def test_chunked_symbol_with_bf16_keep_mask_and_causal(oracle):
     torch.cuda.synchronize()
     ro, _, ro32 = oracle.sdpa_fwd(t[0], t[1], t[2], 0.125, causal=True, want_f32=True)
     assert_close_bf16(oracle, "O", to_f32(out), ro, ro32)
-    # a value head dim above 128 beside a smaller query head dim -> unsupported (2), bad chunk -> invalid (1): status enum of cuda/include/flame_cuda_status.h
-    assert lib.flame_sdpa_chunked_bf16(_p(q), _p(k), _p(v), B, H, Q, K, D, 256, ctypes.c_float(0.125), 64, 0, 1,
+    # a value head dim that is not a multiple of 8 -> unsupported (2), bad chunk -> invalid (1): status enum of cuda/include/flame_cuda_status.h
+    assert lib.flame_sdpa_chunked_bf16(_p(q), _p(k), _p(v), B, H, Q, K, D, 260, ctypes.c_float(0.125), 64, 0, 1,
                                        None, _p(out), None, ctypes.c_uint64(0), _stream()) == 2
     assert lib.flame_sdpa_chunked_bf16(_p(q), _p(k), _p(v), B, H, Q, K, D, D, ctypes.c_float(0.125), 0, 0, 1,
                                        None, _p(out), None, ctypes.c_uint64(0), _stream()) == 1
 
 
-@pytest.mark.parametrize("Dh,Dv", [(64, 32), (64, 128), (96, 64), (40, 104)])
+@pytest.mark.parametrize("Dh,Dv", [(64, 32), (64, 128), (96, 64), (40, 104), (64, 160), (64, 80), (128, 264)])
 def test_value_head_dim_differs_from_query_head_dim(oracle, Dh, Dv):
     """V and O may have a head dim of their own in the chunked and streaming entry points
     (cuda/src/flame_sdpa_stub.cu:973-982, cuda/streaming_attn_bf16.h:7-17).  The oracle takes one head dim, so it
