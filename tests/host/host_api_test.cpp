@@ -983,6 +983,55 @@ int main() {
         }
     }
 
+    // ---- 13. the reference's autograd_v4 tests (src/autograd_v4/tests.rs:14-172), re-expressed: tiny shapes, inputs
+    //          N(0, 0.01), chunked against full (plain, with a keep-mask, with dropout) within its 1e-3
+    {
+        std::printf("[autograd_v4 tests of the reference]\n");
+        auto tiny = [](size_t n) {
+            std::vector<uint16_t> x(n);
+            for (auto& e : x) e = f2bf(0.01f * gauss());
+            return x;
+        };
+        auto max_diff = [](const Tensor& a, const Tensor& b) {
+            auto x = host_f32_of_bf16(a), y = host_f32_of_bf16(b);
+            double m = 0;
+            for (size_t i = 0; i < x.size(); ++i) m = std::fmax(m, std::fabs((double)x[i] - y[i]));
+            return m;
+        };
+        {   // sdpa_v4_forward_runs, sdpa_v4_supports_causal_masks
+            Tensor q = dev_bf16(tiny(64), {1, 2, 4, 8}), k = dev_bf16(tiny(64), {1, 2, 4, 8}), v = dev_bf16(tiny(64), {1, 2, 4, 8});
+            auto out = sdpa::forward_v4(q, k, v, nullptr, false, std::nullopt, std::nullopt);
+            CHECK(out.ok() && out.value().shape() == std::vector<int64_t>({1, 2, 4, 8}), "sdpa_v4_forward_runs");
+            auto cz = sdpa::forward_v4(q, k, v, nullptr, true, std::nullopt, std::nullopt);
+            bool finite = cz.ok();
+            if (cz.ok())
+                for (float x : host_f32_of_bf16(cz.value())) finite = finite && std::isfinite(x);
+            CHECK(finite, "sdpa_v4_supports_causal_masks");
+        }
+        {   // sdpa_v4_chunked_matches_full, ..._with_mask, ..._with_dropout
+            Tensor q = dev_bf16(tiny(96), {1, 2, 6, 8}), k = dev_bf16(tiny(96), {1, 2, 6, 8}), v = dev_bf16(tiny(96), {1, 2, 6, 8});
+            auto full = sdpa::forward_v4(q, k, v, nullptr, false, std::nullopt, std::nullopt);
+            auto chunked = sdpa::forward_v4(q, k, v, nullptr, false, std::nullopt, std::make_pair<size_t, size_t>(3, 4));
+            CHECK(full.ok() && chunked.ok() && max_diff(full.value(), chunked.value()) < 1e-3, "sdpa_v4_chunked_matches_full");
+            std::vector<uint8_t> hm(2 * 6 * 6);
+            for (auto& m : hm) m = gauss() > -0.25f ? 1 : 0;
+            for (int r = 0; r < 12; ++r) hm[(size_t)r * 6] = 1;                     // no row without a key
+            Tensor mask = Tensor::from_host(hm.data(), {1, 2, 6, 6}, DType::U8).value();
+            auto fm = sdpa::forward_v4(q, k, v, &mask, false, std::nullopt, std::nullopt);
+            auto cm = sdpa::forward_v4(q, k, v, &mask, false, std::nullopt, std::make_pair<size_t, size_t>(3, 4));
+            CHECK(fm.ok() && cm.ok() && max_diff(fm.value(), cm.value()) < 1e-3, "sdpa_v4_chunked_matches_full_with_mask");
+            autograd_v4::SdpaConfig cf;
+            cf.save = autograd_v4::SdpaSave::SaveLSE;
+            cf.dropout_p = 0.1f;
+            cf.dropout_seed = 98765;
+            autograd_v4::SdpaConfig cc = cf;
+            cc.chunk_q = 3;
+            cc.chunk_kv = 4;
+            auto fd = autograd_v4::sdpa_forward(q, k, v, nullptr, cf), cd = autograd_v4::sdpa_forward(q, k, v, nullptr, cc);
+            CHECK(fd.ok() && cd.ok() && max_diff(fd.value().first, cd.value().first) < 1e-3, "sdpa_v4_chunked_matches_full_with_dropout");
+        }
+    }
+
     if (hipDeviceSynchronize() != hipSuccess) ++g_fail;
     std::printf(g_fail ? "HOST API TEST: %d FAILURES\n" : "HOST API TEST: all checks passed\n", g_fail);
     return g_fail ? 1 : 0;
