@@ -41,8 +41,17 @@ struct FwdBigDTile {
     static constexpr int COPIES_PER_WAVE = NC * 8 / NW;        // 1 KiB copies (4 rows of one chunk) per tensor and wave
 };
 
+// A problem with few query tiles leaves most compute units idle; then key_splits workgroups share a query tile, each
+// walks a contiguous slice of its key tiles and writes a normalised fp32 partial output with its log-sum-exp, and
+// fwd_bigd_merge_kernel combines them (the partial sums of flash decoding).
+struct FwdBigDParams : FwdParams {
+    int key_splits;      // 1: no split, O and LSE are written directly
+    float* part_o;       // [key_splits][B*H*Sq][dv]
+    float* part_lse;     // [key_splits][B*H*Sq], natural log, -inf for a slice without an attended key
+};
+
 template <int NC, bool SPLIT, int NW>
-__global__ __launch_bounds__(64 * NW) void fwd_bigd_kernel(const FwdParams p) {
+__global__ __launch_bounds__(64 * NW) void fwd_bigd_kernel(const FwdBigDParams p) {
     using T = FwdBigDTile<NC, SPLIT, NW>;
     constexpr int BN = T::BN, BM = T::BM, NDB = T::NDB;
     constexpr int NCP = T::COPIES_PER_WAVE;
@@ -55,7 +64,10 @@ __global__ __launch_bounds__(64 * NW) void fwd_bigd_kernel(const FwdParams p) {
     const int n = lane & 31, h = lane >> 5;
 
     const int n_qt = (p.Sq + BM - 1) / BM;
-    const int wg = xcd_remap(blockIdx.x, gridDim.x);
+    const int n_bh = p.B * p.H;
+    const int wg_all = xcd_remap(blockIdx.x, gridDim.x);
+    const int slice = wg_all / (n_qt * n_bh);         // which slice of the key tiles (0 without a split)
+    const int wg = wg_all % (n_qt * n_bh);
     const int qt = wg % n_qt, bh = wg / n_qt;
     const int b = bh / p.H, hh = bh % p.H;
     const int q0 = qt * BM;
@@ -73,7 +85,10 @@ __global__ __launch_bounds__(64 * NW) void fwd_bigd_kernel(const FwdParams p) {
     if (p.m.kv_len) klimit = min(klimit, max(p.m.kv_len[b], 0));
     int kend = klimit;
     if (p.m.causal) kend = min(kend, q0 + BM);
-    const int n_tiles = (kend + BN - 1) / BN;
+    const int n_tiles_all = (kend + BN - 1) / BN;
+    const int tiles_per_slice = (n_tiles_all + p.key_splits - 1) / p.key_splits;
+    const int t_lo = slice * tiles_per_slice;                    // this workgroup walks tiles t_lo .. n_tiles - 1
+    const int n_tiles = min(n_tiles_all, t_lo + tiles_per_slice);
 
     // ---- Q fragments of every chunk (B operand of S^T = K Q^T): column = query, 8 consecutive d
     bf16x8 qf[NC][8];
@@ -283,24 +298,24 @@ __global__ __launch_bounds__(64 * NW) void fwd_bigd_kernel(const FwdParams p) {
     // ---- the walk over the key tiles.  Tile t's logits and softmax run one step ahead of its PV products: step t is
     //      [S^T of tile t+1 with the copies of V(t+1) and K(t+2) between its MFMAs] [PV of tile t with the softmax of
     //      tile t+1 between its MFMAs] [the rare rescale of O^T] [all copies landed, one workgroup barrier].
-    if (n_tiles > 0) {
+    if (n_tiles > t_lo) {
         f32x16 s;
         bf16x8 pf[2], pn[2];
         float alpha = 1.0f;
         bool rescale = false;
-        for (int j = 0; j < NCP; ++j) issue_copy(KTag{}, 0, j);
-        for (int j = 0; j < NCP; ++j) issue_copy(VTag{}, 0, j);
-        if (n_tiles > 1)
-            for (int j = 0; j < NCP; ++j) issue_copy(KTag{}, 1, j);
+        for (int j = 0; j < NCP; ++j) issue_copy(KTag{}, t_lo, j);
+        for (int j = 0; j < NCP; ++j) issue_copy(VTag{}, t_lo, j);
+        if (n_tiles > t_lo + 1)
+            for (int j = 0; j < NCP; ++j) issue_copy(KTag{}, t_lo + 1, j);
         wait_vm0();
         __syncthreads();
-        logits(No{}, 0, s);
+        logits(No{}, t_lo, s);
         mfma32_vgpr_settle(s);
-        (void)fold_max(0, s, rescale);                           // nothing accumulated yet: no rescale
+        (void)fold_max(t_lo, s, rescale);                        // nothing accumulated yet: no rescale
         exps(s, 0, 16, ((m_run == -INFINITY) ? 0.f : m_run) * c_log2);
         pf[0] = pack8(s[0], s[1], s[2], s[3], s[4], s[5], s[6], s[7]);
         pf[1] = pack8(s[8], s[9], s[10], s[11], s[12], s[13], s[14], s[15]);
-        for (int t = 0; t + 1 < n_tiles; ++t) {
+        for (int t = t_lo; t + 1 < n_tiles; ++t) {
             logits(Yes{}, t + 1, s);
             pv(Yes{}, t, pf, s, pn, alpha, rescale);
             if (rescale) rescale_all(alpha);
@@ -319,6 +334,28 @@ __global__ __launch_bounds__(64 * NW) void fwd_bigd_kernel(const FwdParams p) {
     });
     const float l = l_run + xhalf(l_run);
     const float inv = l > 0.f ? 1.0f / l : 0.f;
+    const float lse_val = l > 0.f ? (m_run * c_log2 + log2_fast(l)) * kLn2 : -INFINITY;
+    if (p.key_splits > 1) {
+        if (qi < p.Sq) {
+            const int64_t prow_i = ((int64_t)slice * n_bh + bh) * p.Sq + qi;
+            float* prow = p.part_o + prow_i * p.dv;
+#pragma unroll
+            for (int c = 0; c < NC; ++c)
+#pragma unroll
+                for (int db = 0; db < NDB; ++db)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const int d0 = 128 * c + 32 * (db0 + db) + 8 * g + 4 * h;
+                        if (d0 < p.dv) {
+                            const f32x16& a = oacc[c][db];
+                            const f32x4 w = {a[4 * g] * inv, a[4 * g + 1] * inv, a[4 * g + 2] * inv, a[4 * g + 3] * inv};
+                            *reinterpret_cast<f32x4*>(prow + d0) = w;
+                        }
+                    }
+            if (h == 0 && db0 == 0) p.part_lse[prow_i] = lse_val;
+        }
+        return;
+    }
     if (qi < p.Sq) {
         uint16_t* orow = obase + (int64_t)qi * p.os.n;
 #pragma unroll
@@ -334,8 +371,38 @@ __global__ __launch_bounds__(64 * NW) void fwd_bigd_kernel(const FwdParams p) {
                         *reinterpret_cast<u32x2*>(orow + d0) = w;
                     }
                 }
-        if (p.lse && h == 0 && db0 == 0) p.lse[(int64_t)bh * p.Sq + qi] = l > 0.f ? (m_run * c_log2 + log2_fast(l)) * kLn2 : -INFINITY;
+        if (p.lse && h == 0 && db0 == 0) p.lse[(int64_t)bh * p.Sq + qi] = lse_val;
     }
+}
+
+// Combines the partial outputs of a key split: LSE = log sum_s exp(LSE_s), O = sum_s exp(LSE_s - LSE) O_s.  One lane
+// per query row and 4 output columns.
+__global__ __launch_bounds__(256) void fwd_bigd_merge_kernel(const FwdBigDParams p) {
+    const int groups = p.dv >> 2;
+    const int64_t rows = (int64_t)p.B * p.H * p.Sq;
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= rows * groups) return;
+    const int64_t row = idx / groups;
+    const int g = (int)(idx % groups);
+    float m = -INFINITY;
+    for (int s = 0; s < p.key_splits; ++s) m = fmaxf(m, p.part_lse[s * rows + row]);
+    float sum = 0.f;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    if (m != -INFINITY) {
+        for (int s = 0; s < p.key_splits; ++s) {
+            const float w = expf(p.part_lse[s * rows + row] - m);
+            const f32x4 v = *reinterpret_cast<const f32x4*>(p.part_o + (s * rows + row) * p.dv + 4 * g);
+            sum += w;
+            acc[0] = fmaf(w, v[0], acc[0]); acc[1] = fmaf(w, v[1], acc[1]);
+            acc[2] = fmaf(w, v[2], acc[2]); acc[3] = fmaf(w, v[3], acc[3]);
+        }
+    }
+    const float inv = sum > 0.f ? 1.0f / sum : 0.f;
+    const int64_t bh = row / p.Sq, qi = row % p.Sq;
+    uint16_t* orow = p.o + (bh / p.H) * p.os.b + (bh % p.H) * p.os.h + qi * p.os.n;
+    const u32x2 w = {pack_bf16(acc[0] * inv, acc[1] * inv), pack_bf16(acc[2] * inv, acc[3] * inv)};
+    *reinterpret_cast<u32x2*>(orow + 4 * g) = w;
+    if (p.lse && g == 0) p.lse[row] = sum > 0.f ? m + logf(sum) : -INFINITY;
 }
 
 }  // namespace fattn

@@ -261,8 +261,20 @@ int launch_bwd(const BwdParams& p, hipStream_t s) {
     return e == hipSuccess ? FLAME_ATTN_OK : (int)e;
 }
 
+int lib_scratch_get(size_t need, hipStream_t stream, void** out);
+
+// Workgroups that share one query tile of the big-head-dim forward, each over a slice of the key tiles: more than one
+// only where the query tiles alone leave at least half of the 256 compute units idle, at most 8, never above 256
+// workgroups in all, and at least 8 key tiles (256 keys) per slice.
+inline int bigd_key_splits(int64_t query_tile_wgs, int Sk) {
+    if (query_tile_wgs <= 0 || query_tile_wgs * 2 > 256) return 1;
+    int ks = (int)std::min<int64_t>(8, 256 / query_tile_wgs);
+    ks = std::min(ks, (Sk + 31) / 32 / 8);
+    return std::max(ks, 1);
+}
+
 template <int NC, int NW>
-int launch_fwd_bigd_nw(const FwdParams& p, hipStream_t s) {
+int launch_fwd_bigd_nw(const FwdParams& fp, hipStream_t s) {
     constexpr bool SPLIT = NC > 2;
     using T = FwdBigDTile<NC, SPLIT, NW>;
     static bool attr_done = false;
@@ -273,11 +285,32 @@ int launch_fwd_bigd_nw(const FwdParams& p, hipStream_t s) {
         if (e != hipSuccess) return (int)e;
         attr_done = true;
     }
-    const int64_t grid = (int64_t)((p.Sq + T::BM - 1) / T::BM) * p.B * p.H;
+    FwdBigDParams p;
+    static_cast<FwdParams&>(p) = fp;
+    const int64_t grid0 = (int64_t)((p.Sq + T::BM - 1) / T::BM) * p.B * p.H;
+    p.key_splits = bigd_key_splits(grid0, p.Sk);
+    p.part_o = nullptr;
+    p.part_lse = nullptr;
+    const int64_t rows = (int64_t)p.B * p.H * p.Sq;
+    if (p.key_splits > 1) {
+        // partial outputs: at most 256 workgroups x 128 queries x (512 + 1) floats = 67 MB, from the library's
+        // per-(device, stream) scratch (allocated on first use or growth, so not inside a graph capture)
+        void* ws = nullptr;
+        const size_t need = (size_t)p.key_splits * rows * (p.dv + 1) * sizeof(float);
+        const int rc = lib_scratch_get(need, s, &ws);
+        if (rc) return rc;
+        p.part_o = static_cast<float*>(ws);
+        p.part_lse = p.part_o + (size_t)p.key_splits * rows * p.dv;
+    }
+    const int64_t grid = grid0 * p.key_splits;
     if (grid > 0x7fffffff) return FLAME_ATTN_ERR_UNSUPPORTED;
     {
         ScopedKernelTimer t(FLAME_ATTN_KERNEL_FWD, s);
         hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(64 * NW), T::LDS_BYTES, s, p);
+        if (p.key_splits > 1) {
+            const int64_t lanes = rows * (p.dv / 4);
+            hipLaunchKernelGGL(fwd_bigd_merge_kernel, dim3((unsigned)((lanes + 255) / 256)), dim3(256), 0, s, p);
+        }
     }
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? FLAME_ATTN_OK : (int)e;
@@ -924,6 +957,9 @@ int bwd_scratch_get(size_t need, hipStream_t stream, void** out) {
     *out = slot->ptr;
     return FLAME_ATTN_OK;
 }
+// The key-split forward for head dims above 128 takes its partial outputs from the same buffers: work on one stream
+// is ordered, so a forward's partials are merged before a later backward on that stream writes there.
+int lib_scratch_get(size_t need, hipStream_t stream, void** out) { return bwd_scratch_get(need, stream, out); }
 
 // Scratch of the allocation-free backward: a fixed array in device memory that every GPU the library
 // runs on holds until the process ends.  Layout as the caller workspace of flame_attn_bwd_bf16: two fp32

@@ -20,7 +20,10 @@
  *     to 512 (the reference serves those through its materialised path, src/sdpa.rs:483-587; e.g. the
  *     one-head D = 512 attention of a VAE mid block), in chunks of 128, when there is no keep-mask,
  *     bias or dropout and V has the head dim of Q; the backward does not (recompute through a
- *     materialised path there).  Anything else returns FLAME_ATTN_ERR_UNSUPPORTED.  The Sage and
+ *     materialised path there).  On a small problem at these head dims (at most 128 query-tile workgroups, at least
+ *     512 keys) the keys are split over workgroups and the fp32 partial outputs (at most 67 MB) go to a buffer the
+ *     library keeps per (device, stream): hipMalloc on first use or growth, as stated for flame_cudnn_sdpa_bwd_bf16.
+ *     Anything else returns FLAME_ATTN_ERR_UNSUPPORTED.  The Sage and
  *     input-preparation entry points take 64 or 128 only.
  *   - LSE / Stats: fp32, contiguous [B*H, N_q] (== [B,H,N_q,1] with strides [H*N_q, N_q, 1, 1]),
  *     value = max_j s_ij + ln(sum_j exp(s_ij - max)), s = scale * Q K^T, natural log

@@ -1,8 +1,8 @@
 """Head dims above 128 (up to 512), forward only: the reference's entry points take any head dim and serve these
 through their materialised path (src/sdpa.rs:483-587, :788-961; the attention of a VAE mid block is one head of
 D = 512 over the latent positions).  O and LSE against the CPU oracle: whole and padded chunks of 128, the plain
-and the two-wavefronts-per-query-block forms (above 256), causal, key lengths, ragged tiles, strided views, the
-reference-named entry points; the cases the kernel does not serve are refused, not computed some other way."""
+and the two-wavefronts-per-query-block forms (above 256), causal, key lengths, ragged tiles, the split of the keys
+over workgroups on small grids, strided views, the reference-named entry points; the cases the kernel does not serve are refused, not computed some other way."""
 import ctypes
 import math
 
@@ -75,6 +75,23 @@ def test_vae_mid_block_shape(oracle):
     2e-2 bound on O means what it means in the other tests."""
     t = _case(5200, 2, 1, 2304, 2304, 512, mul=2.0, vmul=1.0)
     _check(oracle, t, 1.0 / math.sqrt(512))
+
+
+@pytest.mark.parametrize("D", [256, 384, 512])
+def test_key_slices_on_small_grids(oracle, D):
+    """One query tile and 66 key tiles: 8 workgroups walk 9 key tiles each (the last one 3, ending in a ragged tile) and
+    a second kernel merges their partial outputs.  With a key length of 300 most slices are empty, with 0 all of them
+    (O = 0, LSE = -inf); causal, the 100 queries see at most 4 tiles, one per slice."""
+    t = _case(5300 + D, 1, 1, 100, 2100, D, mul=1.5, vmul=1.0)
+    sc = 1.0 / math.sqrt(D)
+    _check(oracle, t, sc)
+    _check(oracle, t, sc, kv_len=[300])
+    _check(oracle, t, sc, kv_len=[0])
+    _check(oracle, t, sc, causal=True)
+    # two heads and three query tiles: slices of several (batch, head, query tile) workgroups side by side
+    t = _case(5310 + D, 1, 2, 300, 1000, D)
+    _check(oracle, t, sc)
+    _check(oracle, t, sc, causal=True, kv_len=[777])
 
 
 def test_strided_views_and_reference_named_entry_points(oracle):
