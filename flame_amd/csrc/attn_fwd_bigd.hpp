@@ -108,30 +108,38 @@ __global__ __launch_bounds__(64 * NW) void fwd_bigd_kernel(const FwdBigDParams p
     }
 
     // ---- tile copies: copy j of a wavefront moves 4 rows of one chunk (1 KiB); lane = (row in copy, physical granule).
-    //      Source = wave-uniform address of the tile + a 32-bit per-lane byte offset (rows past the attended range
-    //      re-read the last attended key; row strides are below 2^24 elements, so 31 rows fit).  The offsets are formed
-    //      again for every copy from two lane constants: kept per copy across the loop they would take 4 NC registers
-    //      that the Q fragments and O^T need (a spill reload in the loop waits on vmcnt, that is, on the copies), and
-    //      made opaque per copy they stay where they are written: between the MFMAs of the logit phase.
+    //      Source = wave-uniform address of the tile + a 32-bit per-lane byte offset (row strides are below 2^24
+    //      elements, so 31 rows fit).  For a tile that lies whole below the key limit the offsets are loop constants,
+    //      kept in 2 NCP registers (FULL); for the last, ragged tile rows past the attended range re-read the last
+    //      attended key and the offsets are formed per copy.
     //      LDS: K stages 0 and 1, then V stages 0 and 1 (tile t in stage t & 1 of its tensor).
     const uint32_t lds0 = lds_addr(lds);
     const int cp_row_in = lane >> 4;
     const int cp_gl = (lane & 15) ^ (cp_row_in << 2);            // physical granule ^ the lane's part of the swizzle
-    auto issue_copy = [&](auto which_tag, int t, int j) {        // which: 0 = K, 1 = V
+    auto copy_offset = [&](int which, int j, int rmax) -> uint32_t {
+        const int64_t row_stride = which ? p.vs.n : p.ks.n;
+        const int cj = wave * NCP + j;                           // 0 .. 8 NC - 1, wave-uniform
+        const int row = min(4 * (cj & 7) + cp_row_in, rmax);
+        const int g = cp_gl ^ (cj & 3);                          // logical granule: swz<128>(row) = (row & 3) << 2 | (row >> 2) & 3
+        int dk = 128 * (cj >> 3) + 8 * g;
+        dk = dk < p.d ? dk : 0;                                  // p.dv == p.d in this kernel
+        return 2u * (uint32_t)(row * (int)row_stride + dk);
+    };
+    uint32_t cp_off[2][NCP];
+    static_for<2 * NCP>([&](auto i_tag) {
+        constexpr int i = decltype(i_tag)::value;
+        cp_off[i / NCP][i % NCP] = copy_offset(i / NCP, i % NCP, BN - 1);
+    });
+    auto issue_copy = [&](auto which_tag, auto full_tag, int t, auto j_tag) {        // which: 0 = K, 1 = V
         constexpr int which = decltype(which_tag)::value;
+        constexpr bool FULL = decltype(full_tag)::value;
+        constexpr int j = decltype(j_tag)::value;
         const int64_t row_stride = which ? p.vs.n : p.ks.n;
         const uint16_t* tb = (which ? vbase : kbase) + (int64_t)t * BN * row_stride;
-        const int rmax = klimit - 1 - t * BN;                    // >= 0 for every tile that is copied
-        int row_in = cp_row_in, gl = cp_gl;
-        asm volatile("" : "+v"(row_in), "+v"(gl));
-        const int cj = wave * NCP + j;                           // 0 .. 8 NC - 1, wave-uniform
-        const int chunk = cj >> 3;
-        const int row = min(4 * (cj & 7) + row_in, rmax);
-        const int g = gl ^ (cj & 3);                             // logical granule: swz<128>(row) = (row & 3) << 2 | (row >> 2) & 3
-        int dk = 128 * chunk + 8 * g;
-        dk = dk < p.d ? dk : 0;                                  // p.dv == p.d in this kernel
-        const uint32_t dst = lds0 + 2u * (uint32_t)((2 * which + (t & 1)) * T::TENSOR_STAGE_ELEMS + chunk * T::SUB_ELEMS + (cj & 7) * 512);
-        dma16u(tb, 2u * (uint32_t)(row * (int)row_stride + dk), dst);
+        const int cj = wave * NCP + j;
+        const uint32_t dst = lds0 + 2u * (uint32_t)((2 * which + (t & 1)) * T::TENSOR_STAGE_ELEMS + (cj >> 3) * T::SUB_ELEMS + (cj & 7) * 512);
+        if constexpr (FULL) dma16u(tb, cp_off[which][j], dst);
+        else dma16u(tb, copy_offset(which, j, klimit - 1 - t * BN), dst);          // rmax >= 0 for every tile that is copied
     };
     using KTag = std::integral_constant<int, 0>;
     using VTag = std::integral_constant<int, 1>;
@@ -167,7 +175,7 @@ __global__ __launch_bounds__(64 * NW) void fwd_bigd_kernel(const FwdBigDParams p
     // of chunk c run: with one wavefront per SIMD nothing else hides the LDS latency.  COPIES: the copies of V tile t1
     // and of K tile t1 + 1 are issued between the MFMAs, one (NW = 1: two) per MFMA from the first on.
     constexpr int CPS = (2 * NCP + 8 * NC - 1) / (8 * NC);       // copies per MFMA slot
-    auto logits = [&](auto copies_tag, int t1, f32x16& s) {
+    auto logits = [&](auto copies_tag, auto full_tag, int t1, f32x16& s) {
         constexpr bool COPIES = decltype(copies_tag)::value;
         const uint16_t* ks = lds + (t1 & 1) * T::TENSOR_STAGE_ELEMS;
         const bool more_k = t1 + 1 < n_tiles;
@@ -188,13 +196,13 @@ __global__ __launch_bounds__(64 * NW) void fwd_bigd_kernel(const FwdBigDParams p
                 if constexpr (c < 2) mfma32_vgpr_bpinned<c * 8 + dc, (c == 0 && dc == 0) ? 0 : 1>(s, kf[c & 1][dc], qf[c][dc], s);
                 else mfma32_vgpr(s, kf[c & 1][dc], qf[c][dc]);
                 if constexpr (COPIES) {
-#pragma unroll
-                    for (int u = 0; u < CPS; ++u) {
-                        constexpr int slot = c * 8 + dc;
-                        const int idx = slot * CPS + u;
-                        if (idx < NCP) issue_copy(VTag{}, t1, idx);
-                        else if (idx < 2 * NCP && more_k) issue_copy(KTag{}, t1 + 1, idx - NCP);
-                    }
+                    static_for<CPS>([&](auto u_tag) {
+                        constexpr int idx = (c * 8 + dc) * CPS + decltype(u_tag)::value;
+                        if constexpr (idx < NCP) issue_copy(VTag{}, full_tag, t1, std::integral_constant<int, idx>{});
+                        else if constexpr (idx < 2 * NCP) {      // FULL says that K tile t1 + 1 exists, too
+                            if (decltype(full_tag)::value || more_k) issue_copy(KTag{}, full_tag, t1 + 1, std::integral_constant<int, idx - NCP>{});
+                        }
+                    });
                 }
             });
             __builtin_amdgcn_sched_barrier(0);
@@ -303,20 +311,22 @@ __global__ __launch_bounds__(64 * NW) void fwd_bigd_kernel(const FwdBigDParams p
         bf16x8 pf[2], pn[2];
         float alpha = 1.0f;
         bool rescale = false;
-        for (int j = 0; j < NCP; ++j) issue_copy(KTag{}, t_lo, j);
-        for (int j = 0; j < NCP; ++j) issue_copy(VTag{}, t_lo, j);
-        if (n_tiles > t_lo + 1)
-            for (int j = 0; j < NCP; ++j) issue_copy(KTag{}, t_lo + 1, j);
+        static_for<NCP>([&](auto j_tag) { issue_copy(KTag{}, No{}, t_lo, j_tag); });
+        static_for<NCP>([&](auto j_tag) { issue_copy(VTag{}, No{}, t_lo, j_tag); });
+        if (n_tiles > t_lo + 1) static_for<NCP>([&](auto j_tag) { issue_copy(KTag{}, No{}, t_lo + 1, j_tag); });
         wait_vm0();
         __syncthreads();
-        logits(No{}, t_lo, s);
+        logits(No{}, No{}, t_lo, s);
         mfma32_vgpr_settle(s);
         (void)fold_max(t_lo, s, rescale);                        // nothing accumulated yet: no rescale
         exps(s, 0, 16, ((m_run == -INFINITY) ? 0.f : m_run) * c_log2);
         pf[0] = pack8(s[0], s[1], s[2], s[3], s[4], s[5], s[6], s[7]);
         pf[1] = pack8(s[8], s[9], s[10], s[11], s[12], s[13], s[14], s[15]);
         for (int t = t_lo; t + 1 < n_tiles; ++t) {
-            logits(Yes{}, t + 1, s);
+            // the tiles copied in this step, V(t + 1) and K(t + 2), are both walked and lie whole below the key limit:
+            // constant copy offsets, no test per copy
+            if (t + 2 < n_tiles && (t + 3) * BN <= klimit) logits(Yes{}, Yes{}, t + 1, s);
+            else logits(Yes{}, No{}, t + 1, s);
             pv(Yes{}, t, pf, s, pn, alpha, rescale);
             if (rescale) rescale_all(alpha);
             pf[0] = pn[0];
