@@ -322,18 +322,21 @@ __global__ __launch_bounds__(64 * NW) void fwd_bigd_kernel(const FwdBigDParams p
         exps(s, 0, 16, ((m_run == -INFINITY) ? 0.f : m_run) * c_log2);
         pf[0] = pack8(s[0], s[1], s[2], s[3], s[4], s[5], s[6], s[7]);
         pf[1] = pack8(s[8], s[9], s[10], s[11], s[12], s[13], s[14], s[15]);
-        for (int t = t_lo; t + 1 < n_tiles; ++t) {
-            // the tiles copied in this step, V(t + 1) and K(t + 2), are both walked and lie whole below the key limit:
-            // constant copy offsets, no test per copy
-            if (t + 2 < n_tiles && (t + 3) * BN <= klimit) logits(Yes{}, Yes{}, t + 1, s);
-            else logits(Yes{}, No{}, t + 1, s);
+        auto step = [&](auto full_tag, int t) {
+            logits(Yes{}, full_tag, t + 1, s);
             pv(Yes{}, t, pf, s, pn, alpha, rescale);
             if (rescale) rescale_all(alpha);
             pf[0] = pn[0];
             pf[1] = pn[1];
             wait_vm0();            // the copies issued in this step have landed ...
             __syncthreads();       // ... everyone's, and everyone is done with the stages they go to next
-        }
+        };
+        // While the tiles copied in a step, V(t + 1) and K(t + 2), are both walked and lie whole below the key limit:
+        // constant copy offsets, no test per copy.  The last steps (two, or three before a ragged tile) form them.
+        int t = t_lo;
+        const int t_whole_end = min(n_tiles, klimit / BN) - 2;
+        for (; t < t_whole_end; ++t) step(Yes{}, t);
+        for (; t + 1 < n_tiles; ++t) step(No{}, t);
         pv(No{}, n_tiles - 1, pf, s, pn, alpha, rescale);
     }
 

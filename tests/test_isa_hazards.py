@@ -57,12 +57,17 @@ def test_checks_run_on_the_compiler_that_built_the_library():
 
 
 def test_hand_emitted_mfma_results_are_not_touched_too_early(text):
+    """The result of a hand-emitted MFMA (architectural accumulator, or the big-head-dim forward's pinned accumulation
+    tuples) may be touched only after two more MFMAs or 11 wait states of s_nop.  Followed along the control flow:
+    an unconditional branch to its target, a conditional one both ways."""
     kernels = re.findall(r"^(_ZN5fattn(?:15bwd_dkdv_kernel|18bwd_dq_wide_kernel|15fwd_wide_kernel|20sage_fwd_wide_kernel|15fwd_bigd_kernel)\w+):.*?\.end_amdhsa_kernel", text, re.S | re.M)
     assert len(kernels) >= 9
     checked = 0
     for name in kernels:
         body = re.search(r"^%s:.*?\.end_amdhsa_kernel" % re.escape(name), text, re.S | re.M).group(0)
-        ins = [l.strip() for l in body.split("\n") if re.match(r"^\s+[a-z]", l)]
+        # instructions and labels, in order
+        ins = [l.strip() for l in body.split("\n") if re.match(r"^\s+[a-z]", l) or re.match(r"^\.LBB\S+:", l)]
+        label_at = {re.match(r"(\.LBB\w+):", l).group(1): i for i, l in enumerate(ins) if l.startswith(".LBB")}
         for idx, l in enumerate(ins):
             if not l.startswith("v_mfma"):
                 continue
@@ -74,36 +79,50 @@ def test_hand_emitted_mfma_results_are_not_touched_too_early(text):
                 continue
             checked += 1
             dst = _regs(ops[0], "a" if by_hand_acc else "v")
-            later_mfma = 0
-            idle = 0                                # wait states spent in s_nop since the MFMA
-            for l2 in ins[idx + 1:]:
-                if l2.startswith("v_mfma"):
-                    later_mfma += 1
-                    if later_mfma >= 2:
+            todo = [(idx + 1, 0, 0)]                    # (position, MFMAs since, wait states spent in s_nop since)
+            seen = set()
+            while todo:
+                pos, later_mfma, idle = todo.pop()
+                while pos < len(ins) and pos not in seen:
+                    seen.add(pos)
+                    l2 = ins[pos]
+                    pos += 1
+                    if l2.startswith(".LBB"):
+                        continue
+                    if l2.startswith("v_mfma"):
+                        later_mfma += 1
+                        if later_mfma >= 2:
+                            break
+                        continue
+                    m = re.match(r"s_nop\s+(\d+)", l2)
+                    if m:
+                        idle += int(m.group(1)) + 1
+                        if idle >= 11:                  # an 8-pass result is visible 11 wait states after issue
+                            break
+                        continue
+                    if l2.startswith("s_endpgm"):
                         break
-                    continue
-                m = re.match(r"s_nop\s+(\d+)", l2)
-                if m:
-                    idle += int(m.group(1)) + 1
-                    if idle >= 11:                  # an 8-pass result is visible 11 wait states after issue
-                        break
-                    continue
-                if l2.startswith("s_branch") or l2.startswith("s_endpgm"):
-                    break                           # nothing falls through: what follows in the file is another path
-                if l2.startswith("s_") or l2.startswith("global_load_lds"):
-                    continue                        # scalar, or vector registers used as addresses only
-                if by_hand_acc:
-                    used = set()
-                    for t in re.findall(r"\ba\[\d+:\d+\]|\ba\d+\b", l2):
-                        used |= _regs(t, "a")
-                else:
-                    toks = re.findall(r"v\[\d+:\d+\]|v\d+", l2)
-                    if l2.startswith("ds_read"):
-                        toks = toks[:1]             # the destination; the other register is an address
-                    used = set()
-                    for t in toks:
-                        used |= _regs(t)
-                assert not (used & dst), f"{name}: `{l2}` touches the result of `{l}` before two more MFMAs"
+                    m = re.match(r"s_(c?)branch\w*\s+(\.LBB\S+)", l2)
+                    if m:
+                        if m.group(1):
+                            todo.append((label_at[m.group(2)], later_mfma, idle))     # taken; not taken goes on below
+                            continue
+                        pos = label_at[m.group(2)]
+                        continue
+                    if l2.startswith("s_") or l2.startswith("global_load_lds"):
+                        continue                        # scalar, or vector registers used as addresses only
+                    if by_hand_acc:
+                        used = set()
+                        for t in re.findall(r"\ba\[\d+:\d+\]|\ba\d+\b", l2):
+                            used |= _regs(t, "a")
+                    else:
+                        toks = re.findall(r"v\[\d+:\d+\]|v\d+", l2)
+                        if l2.startswith("ds_read"):
+                            toks = toks[:1]             # the destination; the other register is an address
+                        used = set()
+                        for t in toks:
+                            used |= _regs(t)
+                    assert not (used & dst), f"{name}: `{l2}` touches the result of `{l}` before two more MFMAs"
     assert checked >= 4 * 96
 
 
