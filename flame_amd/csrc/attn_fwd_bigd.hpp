@@ -50,6 +50,11 @@ struct FwdBigDParams : FwdParams {
     float* part_lse;     // [key_splits][B*H*Sq], natural log, -inf for a slice without an attended key
 };
 
+// the other of the two LDS stages, as a constant where the stage is one
+template <int P>
+__device__ constexpr std::integral_constant<int, 1 - P> other_stage(std::integral_constant<int, P>) { return {}; }
+__device__ inline int other_stage(int stage) { return stage ^ 1; }
+
 template <int NC, bool SPLIT, int NW>
 __global__ __launch_bounds__(64 * NW) void fwd_bigd_kernel(const FwdBigDParams p) {
     using T = FwdBigDTile<NC, SPLIT, NW>;
@@ -112,7 +117,8 @@ __global__ __launch_bounds__(64 * NW) void fwd_bigd_kernel(const FwdBigDParams p
     //      elements, so 31 rows fit).  For a tile that lies whole below the key limit the offsets are loop constants,
     //      kept in 2 NCP registers (FULL); for the last, ragged tile rows past the attended range re-read the last
     //      attended key and the offsets are formed per copy.
-    //      LDS: K stages 0 and 1, then V stages 0 and 1 (tile t in stage t & 1 of its tensor).
+    //      LDS: K stages 0 and 1, then V stages 0 and 1 (tile t in stage (t - t_lo) & 1 of its tensor;
+    //      the stage is passed along as a constant where the loop is unrolled by two, as a value elsewhere).
     const uint32_t lds0 = lds_addr(lds);
     const int cp_row_in = lane >> 4;
     const int cp_gl = (lane & 15) ^ (cp_row_in << 2);            // physical granule ^ the lane's part of the swizzle
@@ -130,14 +136,15 @@ __global__ __launch_bounds__(64 * NW) void fwd_bigd_kernel(const FwdBigDParams p
         constexpr int i = decltype(i_tag)::value;
         cp_off[i / NCP][i % NCP] = copy_offset(i / NCP, i % NCP, BN - 1);
     });
-    auto issue_copy = [&](auto which_tag, auto full_tag, int t, auto j_tag) {        // which: 0 = K, 1 = V
+    auto issue_copy = [&](auto which_tag, auto full_tag, int t, auto j_tag, auto stage_of_t) {        // which: 0 = K, 1 = V
+        const int stage = stage_of_t;
         constexpr int which = decltype(which_tag)::value;
         constexpr bool FULL = decltype(full_tag)::value;
         constexpr int j = decltype(j_tag)::value;
         const int64_t row_stride = which ? p.vs.n : p.ks.n;
         const uint16_t* tb = (which ? vbase : kbase) + (int64_t)t * BN * row_stride;
         const int cj = wave * NCP + j;
-        const uint32_t dst = lds0 + 2u * (uint32_t)((2 * which + (t & 1)) * T::TENSOR_STAGE_ELEMS + (cj >> 3) * T::SUB_ELEMS + (cj & 7) * 512);
+        const uint32_t dst = lds0 + 2u * (uint32_t)((2 * which + stage) * T::TENSOR_STAGE_ELEMS + (cj >> 3) * T::SUB_ELEMS + (cj & 7) * 512);
         if constexpr (FULL) dma16u(tb, cp_off[which][j], dst);
         else dma16u(tb, copy_offset(which, j, klimit - 1 - t * BN), dst);          // rmax >= 0 for every tile that is copied
     };
@@ -175,9 +182,10 @@ __global__ __launch_bounds__(64 * NW) void fwd_bigd_kernel(const FwdBigDParams p
     // of chunk c run: with one wavefront per SIMD nothing else hides the LDS latency.  COPIES: the copies of V tile t1
     // and of K tile t1 + 1 are issued between the MFMAs, one (NW = 1: two) per MFMA from the first on.
     constexpr int CPS = (2 * NCP + 8 * NC - 1) / (8 * NC);       // copies per MFMA slot
-    auto logits = [&](auto copies_tag, auto full_tag, int t1, f32x16& s) {
+    auto logits = [&](auto copies_tag, auto full_tag, int t1, f32x16& s, auto stage_of_t1) {
         constexpr bool COPIES = decltype(copies_tag)::value;
-        const uint16_t* ks = lds + (t1 & 1) * T::TENSOR_STAGE_ELEMS;
+        const int stage1 = stage_of_t1;
+        const uint16_t* ks = lds + stage1 * T::TENSOR_STAGE_ELEMS;
         const bool more_k = t1 + 1 < n_tiles;
         bf16x8 kf[2][8];
         auto read_k = [&](int c, bf16x8 (&dst)[8]) {
@@ -198,9 +206,9 @@ __global__ __launch_bounds__(64 * NW) void fwd_bigd_kernel(const FwdBigDParams p
                 if constexpr (COPIES) {
                     static_for<CPS>([&](auto u_tag) {
                         constexpr int idx = (c * 8 + dc) * CPS + decltype(u_tag)::value;
-                        if constexpr (idx < NCP) issue_copy(VTag{}, full_tag, t1, std::integral_constant<int, idx>{});
+                        if constexpr (idx < NCP) issue_copy(VTag{}, full_tag, t1, std::integral_constant<int, idx>{}, stage_of_t1);
                         else if constexpr (idx < 2 * NCP) {      // FULL says that K tile t1 + 1 exists, too
-                            if (decltype(full_tag)::value || more_k) issue_copy(KTag{}, full_tag, t1 + 1, std::integral_constant<int, idx - NCP>{});
+                            if (decltype(full_tag)::value || more_k) issue_copy(KTag{}, full_tag, t1 + 1, std::integral_constant<int, idx - NCP>{}, other_stage(stage_of_t1));
                         }
                     });
                 }
@@ -258,9 +266,10 @@ __global__ __launch_bounds__(64 * NW) void fwd_bigd_kernel(const FwdBigDParams p
     // and the bf16 P^T operands of the next tile come out in pn.
     constexpr int NM = 2 * NC * NDB;                             // PV MFMAs per tile
     constexpr int NE = NM - 3;                                   // of which carry exponentials
-    auto pv = [&](auto softmax_tag, int t, const bf16x8 (&pf)[2], f32x16& s, bf16x8 (&pn)[2], float& alpha, bool& rescale) {
+    auto pv = [&](auto softmax_tag, int t, const bf16x8 (&pf)[2], f32x16& s, bf16x8 (&pn)[2], float& alpha, bool& rescale, auto stage_of_t) {
         constexpr bool SOFTMAX = decltype(softmax_tag)::value;
-        const uint16_t* vs = lds + (2 + (t & 1)) * T::TENSOR_STAGE_ELEMS;
+        const int stage = stage_of_t;
+        const uint16_t* vs = lds + (2 + stage) * T::TENSOR_STAGE_ELEMS;
         bf16x8 vf[2][2 * NDB];
         auto read_v = [&](int c, bf16x8 (&dst)[2 * NDB]) {
 #pragma unroll
@@ -311,20 +320,22 @@ __global__ __launch_bounds__(64 * NW) void fwd_bigd_kernel(const FwdBigDParams p
         bf16x8 pf[2], pn[2];
         float alpha = 1.0f;
         bool rescale = false;
-        static_for<NCP>([&](auto j_tag) { issue_copy(KTag{}, No{}, t_lo, j_tag); });
-        static_for<NCP>([&](auto j_tag) { issue_copy(VTag{}, No{}, t_lo, j_tag); });
-        if (n_tiles > t_lo + 1) static_for<NCP>([&](auto j_tag) { issue_copy(KTag{}, No{}, t_lo + 1, j_tag); });
+        using S0 = std::integral_constant<int, 0>;
+        using S1 = std::integral_constant<int, 1>;
+        static_for<NCP>([&](auto j_tag) { issue_copy(KTag{}, No{}, t_lo, j_tag, S0{}); });
+        static_for<NCP>([&](auto j_tag) { issue_copy(VTag{}, No{}, t_lo, j_tag, S0{}); });
+        if (n_tiles > t_lo + 1) static_for<NCP>([&](auto j_tag) { issue_copy(KTag{}, No{}, t_lo + 1, j_tag, S1{}); });
         wait_vm0();
         __syncthreads();
-        logits(No{}, No{}, t_lo, s);
+        logits(No{}, No{}, t_lo, s, S0{});
         mfma32_vgpr_settle(s);
         (void)fold_max(t_lo, s, rescale);                        // nothing accumulated yet: no rescale
         exps(s, 0, 16, ((m_run == -INFINITY) ? 0.f : m_run) * c_log2);
         pf[0] = pack8(s[0], s[1], s[2], s[3], s[4], s[5], s[6], s[7]);
         pf[1] = pack8(s[8], s[9], s[10], s[11], s[12], s[13], s[14], s[15]);
-        auto step = [&](auto full_tag, int t) {
-            logits(Yes{}, full_tag, t + 1, s);
-            pv(Yes{}, t, pf, s, pn, alpha, rescale);
+        auto step = [&](auto full_tag, int t, auto stage_of_t) {
+            logits(Yes{}, full_tag, t + 1, s, other_stage(stage_of_t));
+            pv(Yes{}, t, pf, s, pn, alpha, rescale, stage_of_t);
             if (rescale) rescale_all(alpha);
             pf[0] = pn[0];
             pf[1] = pn[1];
@@ -332,12 +343,21 @@ __global__ __launch_bounds__(64 * NW) void fwd_bigd_kernel(const FwdBigDParams p
             __syncthreads();       // ... everyone's, and everyone is done with the stages they go to next
         };
         // While the tiles copied in a step, V(t + 1) and K(t + 2), are both walked and lie whole below the key limit:
-        // constant copy offsets, no test per copy.  The last steps (two, or three before a ragged tile) form them.
+        // constant copy offsets, no test per copy, and (up to D = 256) two steps per trip so that the LDS stages are
+        // constants, too.
+        // The last steps (two to four) form their offsets and stages.
         int t = t_lo;
         const int t_whole_end = min(n_tiles, klimit / BN) - 2;
-        for (; t < t_whole_end; ++t) step(Yes{}, t);
-        for (; t + 1 < n_tiles; ++t) step(No{}, t);
-        pv(No{}, n_tiles - 1, pf, s, pn, alpha, rescale);
+        if constexpr (NC <= 2) {
+            for (; t + 1 < t_whole_end; t += 2) {
+                step(Yes{}, t, S0{});
+                step(Yes{}, t + 1, S1{});
+            }
+        } else {           // measured: no gain with three chunks; with four the second set of LDS addresses spills
+            for (; t < t_whole_end; ++t) step(Yes{}, t, (t - t_lo) & 1);
+        }
+        for (; t + 1 < n_tiles; ++t) step(No{}, t, (t - t_lo) & 1);
+        pv(No{}, n_tiles - 1, pf, s, pn, alpha, rescale, (n_tiles - 1 - t_lo) & 1);
     }
 
     // ---- epilogue
