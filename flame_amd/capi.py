@@ -60,20 +60,33 @@ def _mask_strides(mask, B, H, Sq, Sk):
     return _i64x4(st)
 
 
-def attn_fwd(q, k, v, scale, causal=False, kv_len=None, mask=None, want_lse=True, out=None):
-    """O, LSE = flame_attn_fwd_bf16(...).  q [B,H,Sq,D], k/v [B,H,Sk,D] bf16, D stride 1."""
+def fwd_workspace_bytes(B, H, Sq, Sk, D) -> int:
+    """Bytes of workspace with which flame_attn_fwd_ws_bf16 splits the keys of a small problem at a head dim above
+    128 over workgroups (0 where it would not split)."""
+    f = lib().flame_attn_fwd_workspace_bytes
+    f.restype = ctypes.c_size_t
+    return int(f(B, H, Sq, Sk, D))
+
+
+def attn_fwd(q, k, v, scale, causal=False, kv_len=None, mask=None, want_lse=True, out=None, lse_out=None, workspace=None):
+    """O, LSE = flame_attn_fwd_bf16(...).  q [B,H,Sq,D], k/v [B,H,Sk,D] bf16, D stride 1.
+    `workspace` (uint8 device tensor): flame_attn_fwd_ws_bf16 instead, which may use it."""
     B, H, Sq, D = q.shape
     Sk = k.shape[2]
     o = torch.empty((B, H, Sq, D), dtype=torch.bfloat16, device=q.device) if out is None else out
-    lse = torch.empty((B * H, Sq), dtype=torch.float32, device=q.device) if want_lse else None
+    lse = lse_out if lse_out is not None else (torch.empty((B * H, Sq), dtype=torch.float32, device=q.device) if want_lse else None)
     ms = _mask_strides(mask, B, H, Sq, Sk)
-    rc = lib().flame_attn_fwd_bf16(
-        _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), B, H, Sq, Sk, D, ctypes.c_float(scale),
-        _i64x4(q.stride()), _i64x4(k.stride()), _i64x4(v.stride()), _i64x4(o.stride()),
-        *(ctypes.c_int64(0) for _ in range(5)),
-        int(bool(causal)), _ptr(kv_len), _ptr(mask), ms, _stream())
+    args = (_ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), B, H, Sq, Sk, D, ctypes.c_float(scale),
+            _i64x4(q.stride()), _i64x4(k.stride()), _i64x4(v.stride()), _i64x4(o.stride()),
+            *(ctypes.c_int64(0) for _ in range(5)),
+            int(bool(causal)), _ptr(kv_len), _ptr(mask), ms)
+    if workspace is None:
+        fn, rc = "flame_attn_fwd_bf16", lib().flame_attn_fwd_bf16(*args, _stream())
+    else:
+        fn, rc = "flame_attn_fwd_ws_bf16", lib().flame_attn_fwd_ws_bf16(
+            *args, _ptr(workspace), ctypes.c_size_t(workspace.numel()), _stream())
     if rc != 0:
-        raise FlameAttnError("flame_attn_fwd_bf16", rc)
+        raise FlameAttnError(fn, rc)
     return o, lse
 
 
@@ -172,7 +185,7 @@ def cudnn_sdpa_bwd(q, k, v, o, do, stats, scale, grads=None):
 
 
 KERNEL_KINDS = ("fwd", "unused1", "bwd_dkdv", "bwd_dq", "sage_kmean", "sage_quant", "sage_fwd", "input_prep",
-                "bwd_merge", "reserved9", "reserved10", "reserved11")
+                "bwd_merge", "bwd_joint", "bwd_rows", "reserved11")
 
 
 class _KernelTimes(ctypes.Structure):

@@ -36,6 +36,8 @@ struct BwdParams {
     // and leaving fp32 partial sums in split_ws for bwd_dkdv_merge_kernel.  n_whole < 0: no splitting.
     int n_whole = -1;
     int split_parts = 1;
+    int rows_ready = 0;            // -delta and lse2 are in the workspace already (bwd_rows_kernel ran): read, do not form
+    int joint_n_dq = 0;            // bwd_joint_kernel: the first joint_n_dq workgroups are dQ workgroups
     float* split_ws = nullptr;
     size_t split_ws_bytes = 0;     // host side only
     const uint16_t* q;
@@ -87,8 +89,10 @@ __device__ __forceinline__ void dkdv_store(const BwdParams& p, const f32x16 (&dk
 // registers back, the walk runs the same straight-line steps as the unmasked one.
 // DROPOUT: dV takes the dropped and rescaled probabilities, dP = f (dO V^T) with the same factor f (drop_factor), and
 // -delta is added per element instead of seeding the dP accumulators.
+// block / nblocks: this workgroup's index in the dK/dV grid and the size of that grid (the kernel's own launch, or
+// the dK/dV part of bwd_joint_kernel's).
 template <int D, bool HASMASK, bool TIMING, bool VECMASK = false, bool DROPOUT = false>
-__global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
+__device__ __forceinline__ void bwd_dkdv_body(const BwdParams& p, const int block, const int nblocks) {
     static_assert(!VECMASK || HASMASK, "VECMASK is a special case of HASMASK");
     using T = BwdTile<D>;
     constexpr int BM = T::BM, BN = T::BN, RS = T::RS;
@@ -110,11 +114,11 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
     const int n_kt = (p.Sk + BN - 1) / BN;
     int wg, part = 0, nparts = 1;
     if (p.n_whole < 0) {
-        wg = p.m.kv_len ? xcd_remap_heads(blockIdx.x, gridDim.x, n_kt) : xcd_remap(blockIdx.x, gridDim.x);
-    } else if ((int)blockIdx.x < p.n_whole) {
-        wg = xcd_remap(blockIdx.x, p.n_whole);
+        wg = p.m.kv_len ? xcd_remap_heads(block, nblocks, n_kt) : xcd_remap(block, nblocks);
+    } else if (block < p.n_whole) {
+        wg = xcd_remap(block, p.n_whole);
     } else {          // the split key blocks come last in dispatch order and fill the final, partial round
-        const int e = (int)blockIdx.x - p.n_whole;
+        const int e = block - p.n_whole;
         nparts = p.split_parts;
         wg = p.n_whole + e / nparts;
         part = e % nparts;
@@ -647,7 +651,7 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
     if (TIMING && p.phase_cycles && tid == 0) {
         ph[5] = wall_clock64() - wall0;      // 100 MHz
 #pragma unroll
-        for (int i = 0; i < 6; ++i) p.phase_cycles[(size_t)blockIdx.x * 6 + i] = ph[i];
+        for (int i = 0; i < 6; ++i) p.phase_cycles[(size_t)block * 6 + i] = ph[i];
     }
 #undef FATTN_PHASE
 
@@ -678,6 +682,11 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
             }
     }
     dkdv_store<D>(p, dkacc, dvacc, b, hh, kw0 + n, h);
+}
+
+template <int D, bool HASMASK, bool TIMING, bool VECMASK = false, bool DROPOUT = false>
+__global__ __launch_bounds__(256) void bwd_dkdv_kernel(const BwdParams p) {
+    bwd_dkdv_body<D, HASMASK, TIMING, VECMASK, DROPOUT>(p, (int)blockIdx.x, (int)gridDim.x);
 }
 
 // dK^T / dV^T accumulators (rows = d, column = this lane's key) -> bf16 rows of dK (scaled) and dV
@@ -1096,7 +1105,7 @@ struct BwdDqWideTile {
 };
 
 template <int D>
-__global__ __launch_bounds__(256) void bwd_dq_wide_kernel(const BwdParams p) {
+__device__ __forceinline__ void bwd_dq_wide_body(const BwdParams& p, const int block, const int nblocks) {
     using T = BwdDqWideTile<D>;
     constexpr int BM = T::BM, BN = T::BN, RS = T::RS;
     constexpr int DC = D / 16;
@@ -1112,9 +1121,9 @@ __global__ __launch_bounds__(256) void bwd_dq_wide_kernel(const BwdParams p) {
     const int n = lane & 31, h = lane >> 5;
 
     const int n_qt = (p.Sq + BM - 1) / BM;
-    const int wg = p.m.kv_len ? xcd_remap_heads(blockIdx.x, gridDim.x, n_qt) : xcd_remap(blockIdx.x, gridDim.x);
+    const int wg = p.m.kv_len ? xcd_remap_heads(block, nblocks, n_qt) : xcd_remap(block, nblocks);
     int qt = wg % n_qt, bh = wg / n_qt;
-    if (p.m.causal && !p.m.kv_len) causal_longest_first(wg, n_qt, gridDim.x, qt, bh);
+    if (p.m.causal && !p.m.kv_len) causal_longest_first(wg, n_qt, nblocks, qt, bh);
     const int b = bh / p.H, hh = bh % p.H;
     const int q0 = qt * BM;
     const int qw0 = q0 + wave * 64;
@@ -1150,20 +1159,29 @@ __global__ __launch_bounds__(256) void bwd_dq_wide_kernel(const BwdParams p) {
             qf[qb][dc] = pin_b_fragment<qb * DC + dc>(ldg16(rq + 16 * dc, in_d));
             const u32x4 dv = ldg16(rd + 16 * dc, in_d);
             dof[qb][dc] = pin_b_fragment<16 + qb * DC + dc>(dv);
-            const u32x4 ov = ldg16(ro + 16 * dc, in_d);
+            if (!p.rows_ready) {
+                const u32x4 ov = ldg16(ro + 16 * dc, in_d);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) part += bf16_lo(dv[i]) * bf16_lo(ov[i]) + bf16_hi(dv[i]) * bf16_hi(ov[i]);
+                for (int i = 0; i < 4; ++i) part += bf16_lo(dv[i]) * bf16_lo(ov[i]) + bf16_hi(dv[i]) * bf16_hi(ov[i]);
+            }
         });
-        part += xhalf(part);
         lse2[qb] = INFINITY;
         float nd = 0.f;
-        if (qok) {
-            const float l = p.lse[(int64_t)bh * p.Sq + qrow[qb]];
-            lse2[qb] = (l == -INFINITY) ? INFINITY : l * kLog2e;
-            nd = -part;
-            if (h == 0) {
-                p.ndelta[(int64_t)bh * p.Sq + qrow[qb]] = nd;
-                p.lse2[(int64_t)bh * p.Sq + qrow[qb]] = lse2[qb];
+        if (p.rows_ready) {       // bwd_rows_kernel has left both rows in the workspace
+            if (qok) {
+                nd = p.ndelta[(int64_t)bh * p.Sq + qrow[qb]];
+                lse2[qb] = p.lse2[(int64_t)bh * p.Sq + qrow[qb]];
+            }
+        } else {
+            part += xhalf(part);
+            if (qok) {
+                const float l = p.lse[(int64_t)bh * p.Sq + qrow[qb]];
+                lse2[qb] = (l == -INFINITY) ? INFINITY : l * kLog2e;
+                nd = -part;
+                if (h == 0) {
+                    p.ndelta[(int64_t)bh * p.Sq + qrow[qb]] = nd;
+                    p.lse2[(int64_t)bh * p.Sq + qrow[qb]] = lse2[qb];
+                }
             }
         }
 #pragma unroll
@@ -1435,6 +1453,54 @@ __global__ __launch_bounds__(256) void bwd_dq_wide_kernel(const BwdParams p) {
                     if (32 * db + 8 * g + 4 * h < p.d) *reinterpret_cast<u32x2*>(dqrow + 32 * db + 8 * g + 4 * h) = w;
                 }
         }
+}
+
+template <int D>
+__global__ __launch_bounds__(256) void bwd_dq_wide_kernel(const BwdParams p) {
+    bwd_dq_wide_body<D>(p, (int)blockIdx.x, (int)gridDim.x);
+}
+
+// ------------------------------------------------------------------------------- per-query rows
+// -delta_i = -sum_d dO_id * O_id and LSE_i * log2(e) (+inf where LSE = -inf) for every query row, as a pass of its
+// own: with both rows in the workspace beforehand (BwdParams::rows_ready) the dQ and dK/dV walks no longer depend
+// on each other and can share one grid.  D / 8 lanes per row, one 16-byte granule of O and of dO each.
+template <int D>
+__global__ __launch_bounds__(256) void bwd_rows_kernel(const BwdParams p) {
+    constexpr int LPR = D / 8;                       // lanes per row
+    constexpr int ROWS = 256 / LPR;                  // rows per workgroup
+    const int tid = threadIdx.x;
+    const int g = tid % LPR;
+    const int64_t row = (int64_t)blockIdx.x * ROWS + tid / LPR;       // over [B*H, Sq]
+    const int64_t n_rows = (int64_t)p.B * p.H * p.Sq;
+    const bool ok = row < n_rows;
+    const int64_t rr = ok ? row : 0;
+    const int bh = (int)(rr / p.Sq), qi = (int)(rr % p.Sq);
+    const int b = bh / p.H, hh = bh % p.H;
+    const bool in_d = ok && 8 * g < p.d;
+    const u32x4 ov = ldg16(p.o + b * p.os.b + hh * p.os.h + (int64_t)qi * p.os.n + 8 * g, in_d);
+    const u32x4 dv = ldg16(p.dout + b * p.dos.b + hh * p.dos.h + (int64_t)qi * p.dos.n + 8 * g, in_d);
+    float part = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) part += bf16_lo(dv[i]) * bf16_lo(ov[i]) + bf16_hi(dv[i]) * bf16_hi(ov[i]);
+#pragma unroll
+    for (int off = LPR / 2; off > 0; off >>= 1) part += __shfl_xor(part, off, 64);
+    if (ok && g == 0) {
+        const float l = p.lse[row];
+        p.ndelta[row] = -part;
+        p.lse2[row] = (l == -INFINITY) ? INFINITY : l * kLog2e;
+    }
+}
+
+// ------------------------------------------------------------------------ dQ and dK/dV in one grid
+// For problems whose walks are all equally long (no causal flag, key lengths or mask) and fill 256-query
+// workgroups: the dQ workgroups (the longer ones) come first in dispatch order, the whole dK/dV key blocks next,
+// the split ones last, so that compute units freed by one kind of workgroup go on with the next and only the
+// short split pieces make up the tail.  Needs the per-query rows beforehand (bwd_rows_kernel).
+template <int D>
+__global__ __launch_bounds__(256) void bwd_joint_kernel(const BwdParams p) {
+    const int block = (int)blockIdx.x;
+    if (block < p.joint_n_dq) bwd_dq_wide_body<D>(p, block, p.joint_n_dq);
+    else bwd_dkdv_body<D, false, false>(p, block - p.joint_n_dq, (int)gridDim.x - p.joint_n_dq);
 }
 
 }  // namespace fattn

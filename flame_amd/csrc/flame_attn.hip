@@ -12,7 +12,9 @@
 #include <math.h>
 #include <stdio.h>
 #include <stdlib.h>
+#include <string.h>
 
+#include <atomic>
 #include <mutex>
 #include <vector>
 
@@ -60,13 +62,13 @@ struct Profiler {
     static constexpr int kKinds = FLAME_ATTN_N_KERNEL_KINDS;
     static constexpr size_t kMaxPairs = 8192;
     std::mutex mu;
-    bool enabled = false;
+    std::atomic<bool> enabled{false};     // read without the lock on every launch
     std::vector<hipEvent_t> start[kKinds], stop[kKinds];
     size_t used[kKinds] = {};
 
     hipEvent_t begin(int kind, hipStream_t s, size_t* slot) {
         std::lock_guard<std::mutex> g(mu);
-        if (!enabled || used[kind] >= kMaxPairs) return nullptr;
+        if (!enabled.load(std::memory_order_relaxed) || used[kind] >= kMaxPairs) return nullptr;
         if (used[kind] == start[kind].size()) {
             hipEvent_t a, b;
             if (hipEventCreate(&a) != hipSuccess) return nullptr;
@@ -88,7 +90,7 @@ struct ScopedKernelTimer {
     hipEvent_t stop_ev = nullptr;
     hipStream_t s;
     ScopedKernelTimer(int kind, hipStream_t stream) : s(stream) {
-        if (g_prof.enabled) {
+        if (g_prof.enabled.load(std::memory_order_relaxed)) {
             size_t slot;
             stop_ev = g_prof.begin(kind, stream, &slot);
         }
@@ -145,6 +147,19 @@ int launch_fwd_wide(const FwdParams& p, hipStream_t s) {
 }
 
 size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+// FLAME_ATTN_BWD_SCHEDULE selects how the backward of a problem with equally long walks is launched (read at every
+// call, so that one process can time the variants against each other):
+//   unset / anything else  dQ kernel (which also forms the per-query rows), then dK/dV kernel     [the default]
+//   "joint"                per-query rows by a pass of their own, then dQ and dK/dV workgroups in one grid
+//   "rows"                 per-query rows by a pass of their own, then the two kernels one after the other
+// Measured at B=1 H=24 S=4608 D=128: the joint grid is 0.8 % faster than the default, within the spread between
+// machines; it stays selectable so that the comparison can be repeated.
+int bwd_schedule_override() {
+    const char* v = getenv("FLAME_ATTN_BWD_SCHEDULE");
+    if (!v) return 0;
+    return strcmp(v, "joint") == 0 ? 1 : strcmp(v, "rows") == 0 ? 2 : 0;
+}
 
 // Head dims: the kernels are compiled for 64 and 128; any other multiple of 8 up to 128 (96 among them) runs
 // zero-padded on the next compiled size.
@@ -213,6 +228,58 @@ int launch_bwd(const BwdParams& p, hipStream_t s) {
     const int64_t n_qt = wide ? n256 : (p.Sq + TQ::BM - 1) / TQ::BM;
     const int64_t grid_dq = n_qt * p.B * p.H;
     if (grid > 0x7fffffff || grid_dq > 0x7fffffff) return FLAME_ATTN_ERR_UNSUPPORTED;
+    // Equally long walks everywhere and 256-query workgroups: a pass over O and dO leaves the per-query rows in the
+    // workspace, then dQ and dK/dV workgroups share one grid (bwd_joint_kernel).
+    const int joint_mode = bwd_schedule_override();
+    if (joint_mode != 0 && wide && !HASMASK && !TIMING && !p.m.causal && !p.m.kv_len && p.split_ws) {
+        static bool joint_attr_done = false;
+        auto kern_joint = bwd_joint_kernel<D>;
+        if (!joint_attr_done) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern_joint), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                               std::max(T::LDS_BYTES, TW::LDS_BYTES));
+            if (e != hipSuccess) return (int)e;
+            joint_attr_done = true;
+        }
+        BwdParams pj = p;
+        pj.rows_ready = 1;
+        const int64_t n_rows = (int64_t)p.B * p.H * p.Sq;
+        constexpr int rows_per_wg = 256 / (D / 8);
+        {
+            ScopedKernelTimer t(FLAME_ATTN_KERNEL_BWD_ROWS, s);
+            hipLaunchKernelGGL(bwd_rows_kernel<D>, dim3((unsigned)((n_rows + rows_per_wg - 1) / rows_per_wg)), dim3(256), 0, s, pj);
+        }
+        const int cus = device_cu_count();
+        const size_t room = p.split_ws_bytes / bwd_split_slot_bytes(D);
+        // the key blocks of the last partial round are cut in two along the walk, as in the default schedule
+        int64_t n_split_j = grid % cus;
+        int parts = 2;
+        while (parts > 1 && (size_t)(n_split_j * parts) > room) --parts;
+        if (parts == 1 || (p.Sq + T::BM - 1) / T::BM < 16) n_split_j = 0;
+        if (n_split_j > 0) {
+            pj.n_whole = (int)(grid - n_split_j);
+            pj.split_parts = parts;
+        }
+        const int64_t grid_kv_j = n_split_j > 0 ? pj.n_whole + n_split_j * parts : grid;
+        if (joint_mode == 1) {
+            pj.joint_n_dq = (int)grid_dq;
+            if (grid_dq + grid_kv_j > 0x7fffffff) return FLAME_ATTN_ERR_UNSUPPORTED;
+            ScopedKernelTimer t(FLAME_ATTN_KERNEL_BWD_JOINT, s);
+            hipLaunchKernelGGL(kern_joint, dim3((unsigned)(grid_dq + grid_kv_j)), dim3(256), std::max(T::LDS_BYTES, TW::LDS_BYTES), s, pj);
+        } else {      // the same kernels one after the other, reading the rows of the pre-pass
+            {
+                ScopedKernelTimer t(FLAME_ATTN_KERNEL_BWD_DQ, s);
+                hipLaunchKernelGGL(kern_dqw, dim3((unsigned)grid_dq), dim3(256), TW::LDS_BYTES, s, pj);
+            }
+            ScopedKernelTimer t(FLAME_ATTN_KERNEL_BWD_DKDV, s);
+            hipLaunchKernelGGL(kern, dim3((unsigned)grid_kv_j), dim3(256), T::LDS_BYTES, s, pj);
+        }
+        if (n_split_j > 0) {
+            ScopedKernelTimer t(FLAME_ATTN_KERNEL_BWD_MERGE, s);
+            hipLaunchKernelGGL(bwd_dkdv_merge_kernel<D>, dim3((unsigned)(n_split_j * (D / 32))), dim3(256), 0, s, pj);
+        }
+        hipError_t e = hipGetLastError();
+        return e == hipSuccess ? FLAME_ATTN_OK : (int)e;
+    }
     // dQ first: besides dQ it leaves -delta = -rowsum(dO * O) and the rescaled LSE of every query row in the
     // workspace, which the dK/dV kernel stages per query tile.
     {
@@ -262,6 +329,14 @@ int launch_bwd(const BwdParams& p, hipStream_t s) {
 }
 
 int lib_scratch_get(size_t need, hipStream_t stream, void** out);
+std::mutex& lib_scratch_enqueue_mutex();
+
+// Where the key-split forward for head dims above 128 may put its fp32 partial outputs.
+struct FwdScratch {
+    void* ws = nullptr;          // caller workspace (device memory, 16-byte aligned), or null
+    size_t bytes = 0;
+    bool library = false;        // reference-named entry points only: the library's own per-(device, stream) buffer
+};
 
 // Workgroups that share one query tile of the big-head-dim forward, each over a slice of the key tiles: more than one
 // only where the query tiles alone leave at least half of the 256 compute units idle, at most 8, never above 256
@@ -273,8 +348,12 @@ inline int bigd_key_splits(int64_t query_tile_wgs, int Sk) {
     return std::max(ks, 1);
 }
 
+// queries per workgroup of the big-head-dim forward the library launches for head dim D
+inline int bigd_query_tile(int D) { return D <= 256 ? 128 : 64; }
+inline size_t bigd_partials_bytes(int key_splits, int64_t rows, int dv) { return (size_t)key_splits * rows * (dv + 1) * sizeof(float); }
+
 template <int NC, int NW>
-int launch_fwd_bigd_nw(const FwdParams& fp, hipStream_t s) {
+int launch_fwd_bigd_nw(const FwdParams& fp, hipStream_t s, const FwdScratch& sc) {
     constexpr bool SPLIT = NC > 2;
     using T = FwdBigDTile<NC, SPLIT, NW>;
     static bool attr_done = false;
@@ -292,15 +371,28 @@ int launch_fwd_bigd_nw(const FwdParams& fp, hipStream_t s) {
     p.part_o = nullptr;
     p.part_lse = nullptr;
     const int64_t rows = (int64_t)p.B * p.H * p.Sq;
+    static_assert(T::BM == (NC <= 2 ? 128 : 64), "bigd_query_tile must name this kernel's query tile");
+    std::unique_lock<std::mutex> enqueue(lib_scratch_enqueue_mutex(), std::defer_lock);
     if (p.key_splits > 1) {
-        // partial outputs: at most 256 workgroups x 128 queries x (512 + 1) floats = 67 MB, from the library's
-        // per-(device, stream) scratch (allocated on first use or growth, so not inside a graph capture)
+        // partial outputs (at most 256 workgroups x 128 queries x (512 + 1) floats = 67 MB): the caller's workspace,
+        // with as many slices as fit into it; without one the keys are not split (nothing is allocated here), except
+        // behind the reference-named entry points, which take the library's per-(device, stream) buffer
         void* ws = nullptr;
-        const size_t need = (size_t)p.key_splits * rows * (p.dv + 1) * sizeof(float);
-        const int rc = lib_scratch_get(need, s, &ws);
-        if (rc) return rc;
-        p.part_o = static_cast<float*>(ws);
-        p.part_lse = p.part_o + (size_t)p.key_splits * rows * p.dv;
+        if (sc.ws && aligned16(sc.ws)) {
+            while (p.key_splits > 1 && bigd_partials_bytes(p.key_splits, rows, p.dv) > sc.bytes) --p.key_splits;
+            ws = sc.ws;
+        } else if (sc.library) {
+            enqueue.lock();          // held until both kernels are enqueued
+            const int rc = lib_scratch_get(bigd_partials_bytes(p.key_splits, rows, p.dv), s, &ws);
+            if (rc == FLAME_ATTN_ERR_UNSUPPORTED) p.key_splits = 1;      // under a capture and nothing allocated yet: unsplit
+            else if (rc) return rc;
+        } else {
+            p.key_splits = 1;
+        }
+        if (p.key_splits > 1) {
+            p.part_o = static_cast<float*>(ws);
+            p.part_lse = p.part_o + (size_t)p.key_splits * rows * p.dv;
+        }
     }
     const int64_t grid = grid0 * p.key_splits;
     if (grid > 0x7fffffff) return FLAME_ATTN_ERR_UNSUPPORTED;
@@ -316,7 +408,7 @@ int launch_fwd_bigd_nw(const FwdParams& fp, hipStream_t s) {
     return e == hipSuccess ? FLAME_ATTN_OK : (int)e;
 }
 template <int NC>
-int launch_fwd_bigd(const FwdParams& p, hipStream_t s) { return launch_fwd_bigd_nw<NC, 4>(p, s); }
+int launch_fwd_bigd(const FwdParams& p, hipStream_t s, const FwdScratch& sc) { return launch_fwd_bigd_nw<NC, 4>(p, s, sc); }
 
 // Dropout of the probabilities: the 128-query forward and dQ kernels and the dK/dV kernel in their DROPOUT
 // instantiations, without the split of the last round; HASMASK: the general kernels for an explicit mask or bias.
@@ -401,7 +493,7 @@ int flame_attn_debug_set_phase_buffer(void* device_buffer) {
 
 int flame_attn_profiling_enable(int on) {
     std::lock_guard<std::mutex> g(g_prof.mu);
-    g_prof.enabled = on != 0;
+    g_prof.enabled.store(on != 0, std::memory_order_relaxed);
     for (int k = 0; k < Profiler::kKinds; ++k) g_prof.used[k] = 0;
     return FLAME_ATTN_OK;
 }
@@ -743,7 +835,7 @@ static int attn_fwd_impl(const void* Q, const void* K, const void* V, void* O, v
                         const uint8_t* keep_mask, const int64_t* mask_strides,
                         const void* bias, int bias_dtype, const int64_t* bias_strides,
                         void* stream, int mask_mode = kMaskU8, int Dv = 0, int q_tile_plan = 0, float dropout_p = 0.f,
-                        uint64_t dropout_seed = 0, int draw_cq = 0, int draw_ck = 0) {
+                        uint64_t dropout_seed = 0, int draw_cq = 0, int draw_ck = 0, FwdScratch scratch = FwdScratch{}) {
     if (Dv == 0) Dv = D;           // V and O may have a head dim of their own (forward only)
     if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0 || Dv < 0) return FLAME_ATTN_ERR_INVALID;
     if (!(scale > 0.f) || !isfinite(scale)) return FLAME_ATTN_ERR_INVALID;
@@ -755,7 +847,7 @@ static int attn_fwd_impl(const void* Q, const void* K, const void* V, void* O, v
             const int rc = attn_fwd_impl(Q, K, V, O, c0 == 0 ? LSE : nullptr, B, H, N_q, N_kv, D, scale, q_strides, k_strides,
                                          v_strides, o_strides, q_off, k_off, v_off + c0, o_off + c0, lse_off, causal, kv_len,
                                          keep_mask, mask_strides, bias, bias_dtype, bias_strides, stream, mask_mode,
-                                         std::min(128, Dv - c0), q_tile_plan, dropout_p, dropout_seed, draw_cq, draw_ck);
+                                         std::min(128, Dv - c0), q_tile_plan, dropout_p, dropout_seed, draw_cq, draw_ck, scratch);
             if (rc != FLAME_ATTN_OK) return rc;
         }
         return FLAME_ATTN_OK;
@@ -801,7 +893,7 @@ static int attn_fwd_impl(const void* Q, const void* K, const void* V, void* O, v
     }
 
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (big) return D <= 256 ? launch_fwd_bigd<2>(p, s) : D <= 384 ? launch_fwd_bigd<3>(p, s) : launch_fwd_bigd<4>(p, s);
+    if (big) return D <= 256 ? launch_fwd_bigd<2>(p, s, scratch) : D <= 384 ? launch_fwd_bigd<3>(p, s, scratch) : launch_fwd_bigd<4>(p, s, scratch);
     const bool hm = keep_mask != nullptr || bias != nullptr;
     if (dropout_p != 0.f) {
         if (!set_dropout(p.m, dropout_p, dropout_seed, draw_cq, draw_ck, N_q, N_kv)) return FLAME_ATTN_ERR_INVALID;
@@ -842,6 +934,30 @@ int flame_attn_fwd_bf16(const void* Q, const void* K, const void* V, void* O, vo
     return attn_fwd_impl(Q, K, V, O, LSE, B, H, N_q, N_kv, D, scale, q_strides, k_strides, v_strides, o_strides,
                          q_off, k_off, v_off, o_off, lse_off, causal, kv_len, keep_mask, mask_strides,
                          nullptr, FLAME_ATTN_DTYPE_F32, nullptr, stream);
+}
+
+size_t flame_attn_fwd_workspace_bytes(int B, int H, int N_q, int N_kv, int D) {
+    if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || !big_head_dim_ok(D)) return 0;
+    const int bm = bigd_query_tile(D);
+    const int ks = bigd_key_splits((int64_t)((N_q + bm - 1) / bm) * B * H, N_kv);
+    return ks > 1 ? bigd_partials_bytes(ks, (int64_t)B * H * N_q, D) : 0;
+}
+
+int flame_attn_fwd_ws_bf16(const void* Q, const void* K, const void* V, void* O, void* LSE,
+                           int B, int H, int N_q, int N_kv, int D, float scale,
+                           const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                           const int64_t* o_strides,
+                           int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off, int64_t lse_off,
+                           int causal, const int32_t* kv_len,
+                           const uint8_t* keep_mask, const int64_t* mask_strides,
+                           void* workspace, size_t workspace_bytes, void* stream) {
+    if (workspace && !aligned16(workspace)) return FLAME_ATTN_ERR_UNSUPPORTED;
+    FwdScratch sc;
+    sc.ws = workspace;
+    sc.bytes = workspace ? workspace_bytes : 0;
+    return attn_fwd_impl(Q, K, V, O, LSE, B, H, N_q, N_kv, D, scale, q_strides, k_strides, v_strides, o_strides,
+                         q_off, k_off, v_off, o_off, lse_off, causal, kv_len, keep_mask, mask_strides,
+                         nullptr, FLAME_ATTN_DTYPE_F32, nullptr, stream, kMaskU8, 0, 0, 0.f, 0, 0, 0, sc);
 }
 
 int flame_attn_fwd_dropout_bf16(const void* Q, const void* K, const void* V, void* O, void* LSE,
@@ -885,8 +1001,16 @@ int flame_attn_fwd_bias_bf16(const void* Q, const void* K, const void* V, void* 
 
 // ------------------------------------------------------------------------------------------------
 // Entry points with the names and argument lists of the reference's FFI for this path.  They are
-// thin shims onto flame_attn_fwd_bf16 / flame_attn_bwd_bf16.
+// thin shims onto the forward and backward above.  Their argument lists have no workspace, and the
+// reference's own implementations allocate behind them (a workspace per cached graph,
+// src/cuda/cudnn_sdpa.cpp:204-212; eleven buffers per call, cuda/sdpa_stream_bf16.cu:214-239): where a
+// kernel needs scratch they take the library's per-(device, stream) buffer.
 // ------------------------------------------------------------------------------------------------
+static FwdScratch library_scratch() {
+    FwdScratch sc;
+    sc.library = true;
+    return sc;
+}
 
 int flame_cudnn_sdpa_bf16(const void* Q, const void* K, const void* V, void* O,
                           int B, int H, int N_q, int N_kv, int D, float scale,
@@ -894,9 +1018,9 @@ int flame_cudnn_sdpa_bf16(const void* Q, const void* K, const void* V, void* O,
                           const int64_t* o_strides,
                           int64_t q_offset_elems, int64_t k_offset_elems, int64_t v_offset_elems,
                           int64_t o_offset_elems, void* stream) {
-    return flame_attn_fwd_bf16(Q, K, V, O, nullptr, B, H, N_q, N_kv, D, scale, q_strides, k_strides, v_strides,
-                               o_strides, q_offset_elems, k_offset_elems, v_offset_elems, o_offset_elems, 0,
-                               0, nullptr, nullptr, nullptr, stream);
+    return attn_fwd_impl(Q, K, V, O, nullptr, B, H, N_q, N_kv, D, scale, q_strides, k_strides, v_strides, o_strides,
+                         q_offset_elems, k_offset_elems, v_offset_elems, o_offset_elems, 0, 0, nullptr, nullptr, nullptr,
+                         nullptr, FLAME_ATTN_DTYPE_F32, nullptr, stream, kMaskU8, 0, 0, 0.f, 0, 0, 0, library_scratch());
 }
 
 int flame_cudnn_sdpa_bf16_train_fwd(const void* Q, const void* K, const void* V, void* O, void* Stats,
@@ -906,21 +1030,25 @@ int flame_cudnn_sdpa_bf16_train_fwd(const void* Q, const void* K, const void* V,
                                     int64_t q_offset_elems, int64_t k_offset_elems, int64_t v_offset_elems,
                                     int64_t o_offset_elems, int64_t stats_offset_elems, void* stream) {
     if (!Stats) return FLAME_ATTN_ERR_INVALID;
-    return flame_attn_fwd_bf16(Q, K, V, O, Stats, B, H, N_q, N_kv, D, scale, q_strides, k_strides, v_strides,
-                               o_strides, q_offset_elems, k_offset_elems, v_offset_elems, o_offset_elems,
-                               stats_offset_elems, 0, nullptr, nullptr, nullptr, stream);
+    return attn_fwd_impl(Q, K, V, O, Stats, B, H, N_q, N_kv, D, scale, q_strides, k_strides, v_strides, o_strides,
+                         q_offset_elems, k_offset_elems, v_offset_elems, o_offset_elems, stats_offset_elems, 0, nullptr,
+                         nullptr, nullptr, nullptr, FLAME_ATTN_DTYPE_F32, nullptr, stream, kMaskU8, 0, 0, 0.f, 0, 0, 0,
+                         library_scratch());
 }
 
 }  // extern "C"
 
 namespace {
-// Scratch for the reference-signature backward, which has no workspace argument: one lazily grown
+// Scratch for the reference-named entry points, whose argument lists have no workspace: one lazily grown
 // buffer per (device, stream), as the reference's shim keeps a workspace it allocated once per shape.
 // Calls on one stream are ordered, so they may share a buffer; calls on different streams get
-// different buffers and cannot race.  A buffer that has to grow is replaced by a new allocation and
-// kept until the process ends: a kernel still running on it keeps valid memory (a hipFree would
-// synchronise the device and, in a capture, fail).  hipMalloc happens on first use or growth only, so
-// the first call with a given stream and size class cannot be captured into a graph.
+// different buffers and cannot race; host threads that share a stream are kept apart by
+// g_lib_scratch_enqueue_mu, which an entry point holds from taking the buffer to its last launch (otherwise
+// the kernels of two calls could interleave on the stream and read each other's rows).
+// hipMalloc happens on first use or growth only; under a stream capture a call that would have to allocate
+// returns FLAME_ATTN_ERR_UNSUPPORTED instead (an allocation there would invalidate the capture).  An outgrown
+// buffer is freed at once when its stream is idle, else at a later call that finds the stream idle: a
+// kernel still running on it keeps valid memory.
 struct BwdScratchSlot {
     int dev;
     hipStream_t stream;
@@ -930,9 +1058,19 @@ struct BwdScratchSlot {
 struct BwdScratch {
     std::mutex mu;
     std::vector<BwdScratchSlot> slots;
-    std::vector<void*> retired;
+    std::vector<BwdScratchSlot> retired;      // outgrown buffers whose stream was busy when they were replaced
 };
 BwdScratch g_bwd_scratch;
+std::mutex g_lib_scratch_enqueue_mu;
+
+bool stream_is_capturing(hipStream_t stream) {
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &st) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    return st != hipStreamCaptureStatusNone;
+}
 
 int bwd_scratch_get(size_t need, hipStream_t stream, void** out) {
     int dev = 0;
@@ -946,11 +1084,37 @@ int bwd_scratch_get(size_t need, hipStream_t stream, void** out) {
         g_bwd_scratch.slots.push_back(BwdScratchSlot{dev, stream, nullptr, 0});
         slot = &g_bwd_scratch.slots.back();
     }
+    const bool capturing = stream_is_capturing(stream);
+    auto idle = [&]() {
+        if (capturing) return false;
+        if (hipStreamQuery(stream) == hipSuccess) return true;
+        (void)hipGetLastError();       // hipErrorNotReady
+        return false;
+    };
+    if (!g_bwd_scratch.retired.empty()) {
+        bool is_idle = false, asked = false;
+        for (size_t i = 0; i < g_bwd_scratch.retired.size();) {
+            BwdScratchSlot& r = g_bwd_scratch.retired[i];
+            if (r.dev == dev && r.stream == stream) {
+                if (!asked) { is_idle = idle(); asked = true; }
+                if (is_idle) {
+                    (void)hipFree(r.ptr);
+                    g_bwd_scratch.retired.erase(g_bwd_scratch.retired.begin() + (long)i);
+                    continue;
+                }
+            }
+            ++i;
+        }
+    }
     if (slot->bytes < need) {
+        if (capturing) return FLAME_ATTN_ERR_UNSUPPORTED;
         void* fresh = nullptr;
         e = hipMalloc(&fresh, need);
         if (e != hipSuccess) return (int)e;
-        if (slot->ptr) g_bwd_scratch.retired.push_back(slot->ptr);
+        if (slot->ptr) {
+            if (idle()) (void)hipFree(slot->ptr);
+            else g_bwd_scratch.retired.push_back(BwdScratchSlot{dev, stream, slot->ptr, slot->bytes});
+        }
         slot->ptr = fresh;
         slot->bytes = need;
     }
@@ -960,6 +1124,7 @@ int bwd_scratch_get(size_t need, hipStream_t stream, void** out) {
 // The key-split forward for head dims above 128 takes its partial outputs from the same buffers: work on one stream
 // is ordered, so a forward's partials are merged before a later backward on that stream writes there.
 int lib_scratch_get(size_t need, hipStream_t stream, void** out) { return bwd_scratch_get(need, stream, out); }
+std::mutex& lib_scratch_enqueue_mutex() { return g_lib_scratch_enqueue_mu; }
 
 // Scratch of the allocation-free backward: a fixed array in device memory that every GPU the library
 // runs on holds until the process ends.  Layout as the caller workspace of flame_attn_bwd_bf16: two fp32
@@ -1038,6 +1203,7 @@ int flame_cudnn_sdpa_bwd_bf16(const void* Q, const void* K, const void* V, const
                               void* stream) {
     const size_t need = flame_attn_bwd_workspace_bytes(B, H, N_q, D);
     if (need == 0) return FLAME_ATTN_ERR_INVALID;
+    std::lock_guard<std::mutex> enqueue(g_lib_scratch_enqueue_mu);      // from taking the buffer to the last launch
     void* ws = nullptr;
     int rc = bwd_scratch_get(need, static_cast<hipStream_t>(stream), &ws);
     if (rc) return rc;
@@ -1079,9 +1245,9 @@ int flame_flash_attention_bf16(const void* Q, const void* K, const void* V, void
     if (batch_heads <= 0 || seq_len_q <= 0 || seq_len_kv <= 0 || head_dim <= 0) return FLAME_ATTN_ERR_INVALID;
     const int64_t qs[4] = {(int64_t)seq_len_q * head_dim, (int64_t)seq_len_q * head_dim, head_dim, 1};
     const int64_t ks[4] = {(int64_t)seq_len_kv * head_dim, (int64_t)seq_len_kv * head_dim, head_dim, 1};
-    return flame_attn_fwd_bf16(Q, K, V, O, LSE, batch_heads, 1, seq_len_q, seq_len_kv, head_dim,
-                               1.0f / sqrtf((float)head_dim), qs, ks, ks, qs, 0, 0, 0, 0, 0, 0, nullptr, nullptr,
-                               nullptr, stream);
+    return attn_fwd_impl(Q, K, V, O, LSE, batch_heads, 1, seq_len_q, seq_len_kv, head_dim, 1.0f / sqrtf((float)head_dim),
+                         qs, ks, ks, qs, 0, 0, 0, 0, 0, 0, nullptr, nullptr, nullptr, nullptr, FLAME_ATTN_DTYPE_F32, nullptr,
+                         stream, kMaskU8, 0, 0, 0.f, 0, 0, 0, library_scratch());
 }
 
 static FlameAttnStatus to_status(int rc) {
@@ -1117,13 +1283,15 @@ FlameAttnStatus flame_sdpa_chunked_bf16(const void* q, const void* k, const void
     auto run = [&](int q_tile) {
         return attn_fwd_impl(q, k, v, out, nullptr, B, H, Q, K, Dh, scale, qs, ks, vs, os, 0, 0, 0, 0, 0, causal, nullptr,
                              static_cast<const uint8_t*>(mask), mask ? ms : nullptr, nullptr, FLAME_ATTN_DTYPE_F32, nullptr,
-                             stream, kMaskBf16Keep, Dv, q_tile);
+                             stream, kMaskBf16Keep, Dv, q_tile, 0.f, 0, 0, 0, library_scratch());
     };
     // ---- the launch plan: the query tile of a workgroup (see plan_cache.hpp)
     PlanCache& pc = PlanCache::instance();
     const PlanConfig& cfg = pc.config();
-    const bool one_tile = mask != nullptr;                 // the masked kernels come with 128-row workgroups only
-    const int rule_q = fwd_rule_wide(B, H, Q, one_tile, false) ? 256 : 128;
+    // the masked kernels come with 128-row workgroups only, and head dims above 128 have one kernel per head dim:
+    // nothing to choose, so nothing is measured
+    const bool one_tile = mask != nullptr || big_head_dim_ok(Dh);
+    const int rule_q = (!one_tile && fwd_rule_wide(B, H, Q, false, false)) ? 256 : 128;
     const PlanKey key{B, H, Q, K, Dh, Dv, mask ? mask_heads : 0, causal ? 1 : 0};
     int q_tile = rule_q;
     uint64_t source = kPlanRule, candidates = 1, best_ns = 0;
@@ -1206,7 +1374,7 @@ FlameAttnStatus flame_sdpa_chunked_bf16(const void* q, const void* k, const void
 }
 
 int flame_sdpa_autotune_get_stats(FlameSdpaAutotuneStats* out) {
-    if (!out) return FLAME_ATTN_ERR_INVALID;
+    if (!out) return FLAME_ATTN_STATUS_ERR_INVALID;     // 1, as cuda/src/flame_sdpa_stub.cu:1382-1385
     PlanCache::instance().get_stats(out);
     return FLAME_ATTN_OK;
 }
@@ -1230,7 +1398,8 @@ int streaming_attn_bf16_fp32_launch(const void* Q, const void* K, const void* V,
     const int64_t qs[4] = {qB, qH, qS, qD}, ks[4] = {kB, kH, kS, kD}, vs[4] = {vB, vH, vS, vD}, os[4] = {oB, oH, oS, oD};
     const int64_t ms[4] = {(int64_t)H * S, S, 0, 1};     // [B,H,S] key-padding mask, 0 = excluded
     return attn_fwd_impl(Q, K, V, O, nullptr, B, H, S, S, Dh, scale, qs, ks, vs, os, 0, 0, 0, 0, 0, causal, nullptr,
-                         k_pad_mask, k_pad_mask ? ms : nullptr, nullptr, FLAME_ATTN_DTYPE_F32, nullptr, stream, kMaskU8, Dv);
+                         k_pad_mask, k_pad_mask ? ms : nullptr, nullptr, FLAME_ATTN_DTYPE_F32, nullptr, stream, kMaskU8, Dv, 0, 0.f,
+                         0, 0, 0, library_scratch());
 }
 
 bool sdpa_stream_bf16_launch(const void* dQ, const void* dK, const void* dV, void* dO, int B, int H, int Q_len,
@@ -1251,7 +1420,7 @@ bool sdpa_stream_bf16_launch(const void* dQ, const void* dK, const void* dV, voi
     const int64_t ms[4] = {mask_stride_eb, mask_stride_eh, mask_stride_eq, mask_stride_ek};
     const int rc = attn_fwd_impl(dQ, dK, dV, dO, nullptr, B, H, Q_len, K_len, d, scale, qs, ks, ks, qs, 0, 0, 0, 0, 0, 0,
                                  nullptr, static_cast<const uint8_t*>(attn_mask), attn_mask ? ms : nullptr, nullptr,
-                                 FLAME_ATTN_DTYPE_F32, nullptr, stream, kMaskBf16Drop);
+                                 FLAME_ATTN_DTYPE_F32, nullptr, stream, kMaskBf16Drop, 0, 0, 0.f, 0, 0, 0, library_scratch());
     if (rc != FLAME_ATTN_OK) return fail(rc == FLAME_ATTN_ERR_INVALID ? "invalid argument" : "unsupported shape or HIP error");
     if (unsupported_reason && reason_buflen > 0) unsupported_reason[0] = 0;
     return true;

@@ -21,8 +21,10 @@
  *     one-head D = 512 attention of a VAE mid block), in chunks of 128, when there is no keep-mask,
  *     bias or dropout and V has the head dim of Q; the backward does not (recompute through a
  *     materialised path there).  On a small problem at these head dims (at most 128 query-tile workgroups, at least
- *     512 keys) the keys are split over workgroups and the fp32 partial outputs (at most 67 MB) go to a buffer the
- *     library keeps per (device, stream): hipMalloc on first use or growth, as stated for flame_cudnn_sdpa_bwd_bf16.
+ *     512 keys) the keys can be split over workgroups, which needs room for fp32 partial outputs (at most 67 MB):
+ *     flame_attn_fwd_ws_bf16 takes it from the caller (flame_attn_fwd_workspace_bytes), flame_attn_fwd_bf16 has no
+ *     such argument and does not split, the reference-named entry points use a buffer the library keeps per
+ *     (device, stream), as stated for flame_cudnn_sdpa_bwd_bf16.
  *     Anything else returns FLAME_ATTN_ERR_UNSUPPORTED.  The Sage and
  *     input-preparation entry points take 64 or 128 only.
  *   - LSE / Stats: fp32, contiguous [B*H, N_q] (== [B,H,N_q,1] with strides [H*N_q, N_q, 1, 1]),
@@ -82,6 +84,22 @@ int flame_attn_fwd_bf16(const void* Q, const void* K, const void* V, void* O, vo
                         const uint8_t* keep_mask, const int64_t* mask_strides,
                         void* stream);
 
+/* The same forward with a caller workspace (16-byte aligned device memory, used only during the call; null or too
+ * small is accepted).  Only the forward for head dims above 128 on a grid that leaves compute units idle uses it, for
+ * the fp32 partial outputs of workgroups that share a query tile and walk slices of the keys; with less room than
+ * flame_attn_fwd_workspace_bytes returns it uses fewer slices, with none it runs unsplit.  Never allocates, so a first
+ * call can be captured into a HIP graph (the reference's contract for code on the backward path:
+ * src/cuda_graph.rs:11-18).  No counterpart in the reference's FFI. */
+size_t flame_attn_fwd_workspace_bytes(int B, int H, int N_q, int N_kv, int D);
+int flame_attn_fwd_ws_bf16(const void* Q, const void* K, const void* V, void* O, void* LSE,
+                           int B, int H, int N_q, int N_kv, int D, float scale,
+                           const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                           const int64_t* o_strides,
+                           int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off, int64_t lse_off,
+                           int causal, const int32_t* kv_len,
+                           const uint8_t* keep_mask, const int64_t* mask_strides,
+                           void* workspace, size_t workspace_bytes, void* stream);
+
 /* Forward with an additive bias on the scaled logits: softmax(scale * Q K^T + bias) V, fp32 softmax.
  * bias: fp32 (FLAME_ATTN_DTYPE_F32) or bf16 device tensor read through four element strides over
  * (B,H,N_q,N_kv); a stride of 0 broadcasts that dimension ([1,H,Q,K] relative-position biases).
@@ -132,8 +150,9 @@ int flame_attn_bwd_dropout_bf16(const void* Q, const void* K, const void* V, con
  * shorter) over the tile's own [B*H, q_t, k_t] tensor, under the seed derive_tile_seed gives (:600-602), whose low word
  * is dropout_seed + k_offset.  0, or a chunk of at least the sequence length, means the whole axis; with both whole this
  * is the pair above.  The attention itself is not chunked: only the kept set depends on the tiles.
- * A seed whose low word is 0 (here: for some tile) makes the reference draw from its global generator instead
- * (src/rng/mod.rs:187-193); no fixed kept set exists for it there, this library uses the 0. */
+ * Parity unpinned for one case: a seed whose low word is 0 (in the pair above: dropout_seed itself; here: the derived
+ * seed of some tile, dropout_seed + k_offset wrapping to 0) makes the reference draw from its process-global generator
+ * instead (src/rng/mod.rs:139-143, :187-193), so no fixed kept set exists for it there; this library draws with the 0. */
 int flame_attn_fwd_dropout_tiled_bf16(const void* Q, const void* K, const void* V, void* O, void* LSE,
                                       int B, int H, int N_q, int N_kv, int D, float scale,
                                       const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
@@ -328,7 +347,7 @@ typedef struct FlameSdpaAutotuneStats {
         last_plan_source, last_shape_b, last_shape_h, last_shape_q, last_shape_k, last_shape_dh, last_shape_dv,
         last_shape_mask_heads, last_shape_causal;
 } FlameSdpaAutotuneStats;
-/* 0 on success, -1 for a null pointer. */
+/* 0 on success, 1 (FLAME_ATTN_STATUS_ERR_INVALID, the reference's FLAME_CUDA_ERR_INVALID: cuda/src/flame_sdpa_stub.cu:1382-1385) for a null pointer. */
 int flame_sdpa_autotune_get_stats(FlameSdpaAutotuneStats* out);
 int flame_sdpa_autotune_reset_stats(void);
 /* Writes the cache file now if persistence is on (FLAME_SDPA_AUTOTUNE_PERSIST=1) and the cache changed. */
@@ -388,6 +407,7 @@ int flame_fp8_to_bf16(const void* input, void* output, float scale, size_t n_ele
 enum { FLAME_ATTN_KERNEL_FWD = 0, FLAME_ATTN_KERNEL_UNUSED_1 = 1, FLAME_ATTN_KERNEL_BWD_DKDV = 2,
        FLAME_ATTN_KERNEL_BWD_DQ = 3, FLAME_ATTN_KERNEL_SAGE_KMEAN = 4, FLAME_ATTN_KERNEL_SAGE_QUANT = 5,
        FLAME_ATTN_KERNEL_SAGE_FWD = 6, FLAME_ATTN_KERNEL_INPUT_PREP = 7, FLAME_ATTN_KERNEL_BWD_MERGE = 8,
+       FLAME_ATTN_KERNEL_BWD_JOINT = 9, FLAME_ATTN_KERNEL_BWD_ROWS = 10,
        FLAME_ATTN_N_KERNEL_KINDS = 12 };
 typedef struct {
     double total_ms[FLAME_ATTN_N_KERNEL_KINDS];

@@ -29,16 +29,23 @@ def _check(oracle, t, scale, causal=False, kv_len=None, tag=""):
     print(f"[big head dim] D={D} B={B} H={H} Sq={Sq} Sk={Sk} causal={causal} kv_len={kv_len} {tag}", flush=True)
     q, k, v = (to_dev(x) for x in t)
     kvl = None if kv_len is None else torch.tensor(kv_len, dtype=torch.int32, device="cuda")
-    o = torch.full_like(q, float("nan"))       # a skipped store, or one past the head dim, shows
-    _, lse = capi.attn_fwd(q, k, v, scale, causal=causal, kv_len=kvl, out=o)
-    torch.cuda.synchronize()
     ro, rlse, ro32 = oracle.sdpa_fwd(t[0], t[1], t[2], scale, causal=causal, kv_len=kv_len, want_f32=True)
-    assert_close_bf16(oracle, "O", to_f32(o), ro, ro32)
-    assert oracle.cosine(to_f32(o), ro32) >= 0.9999
-    glse, rl = lse.cpu().numpy().reshape(rlse.shape), rlse
-    fin = np.isfinite(rl)
-    assert np.array_equal(np.isfinite(glse), fin) and oracle.max_abs(glse[fin], rl[fin]) <= TOL_LSE
-    return o, lse
+    # without a workspace (never split), then, where the library would split the keys over workgroups, with the
+    # workspace it asks for and with half of it (fewer slices)
+    need = capi.fwd_workspace_bytes(B, H, Sq, Sk, D)
+    first = None
+    for ws_bytes in (None, need, need // 2) if need else (None,):
+        ws = None if ws_bytes is None else torch.empty(ws_bytes, dtype=torch.uint8, device="cuda")
+        o = torch.full_like(q, float("nan"))       # a skipped store, or one past the head dim, shows
+        _, lse = capi.attn_fwd(q, k, v, scale, causal=causal, kv_len=kvl, out=o, workspace=ws)
+        torch.cuda.synchronize()
+        assert_close_bf16(oracle, f"O (workspace {ws_bytes})", to_f32(o), ro, ro32)
+        assert oracle.cosine(to_f32(o), ro32) >= 0.9999
+        glse, rl = lse.cpu().numpy().reshape(rlse.shape), rlse
+        fin = np.isfinite(rl)
+        assert np.array_equal(np.isfinite(glse), fin) and oracle.max_abs(glse[fin], rl[fin]) <= TOL_LSE
+        first = first or (o, lse)
+    return first
 
 
 @pytest.mark.parametrize("D", [136, 192, 256, 264, 320, 384, 392, 448, 512])
@@ -79,9 +86,13 @@ def test_vae_mid_block_shape(oracle):
 
 @pytest.mark.parametrize("D", [256, 384, 512])
 def test_key_slices_on_small_grids(oracle, D):
-    """One query tile and 66 key tiles: 8 workgroups walk 9 key tiles each (the last one 3, ending in a ragged tile) and
+    """The library asks for a workspace here (the assertion below), so _check also runs the split forms.
+    One query tile and 66 key tiles: 8 workgroups walk 9 key tiles each (the last one 3, ending in a ragged tile) and
     a second kernel merges their partial outputs.  With a key length of 300 most slices are empty, with 0 all of them
     (O = 0, LSE = -inf); causal, the 100 queries see at most 4 tiles, one per slice."""
+    from flame_amd import capi
+    assert capi.fwd_workspace_bytes(1, 1, 100, 2100, D) == 8 * 100 * (D + 1) * 4
+    assert capi.fwd_workspace_bytes(1, 1, 100, 2100, 128) == 0 and capi.fwd_workspace_bytes(4, 64, 4096, 2100, D) == 0
     t = _case(5300 + D, 1, 1, 100, 2100, D, mul=1.5, vmul=1.0)
     sc = 1.0 / math.sqrt(D)
     _check(oracle, t, sc)

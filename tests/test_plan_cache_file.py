@@ -22,7 +22,7 @@ class Stats(ctypes.Structure):
 assert ctypes.sizeof(Stats) == 200
 lib = ctypes.CDLL(%r)
 st = Stats()
-assert lib.flame_sdpa_autotune_get_stats(None) == -1
+assert lib.flame_sdpa_autotune_get_stats(None) == 1      # the reference returns FLAME_CUDA_ERR_INVALID (cuda/src/flame_sdpa_stub.cu:1382-1385)
 assert lib.flame_sdpa_autotune_get_stats(ctypes.byref(st)) == 0
 first = {f: getattr(st, f) for f in FIELDS}
 assert lib.flame_sdpa_autotune_flush_cache() == 0          # nothing changed: no file is written
