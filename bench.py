@@ -2,9 +2,11 @@
 """Benchmark of the attention hot path on one MI355X.
 
 One "step" = one forward (O + log-sum-exp) followed by one tile-recompute backward (dQ, dK, dV), inputs
-resident in HBM.  The default workload is the DiT joint-attention configuration B=1 H=24 S=4608 (512 text
-+ 4096 image tokens) D=128 bf16; `--config 1..5` selects the other configurations (5 is the inference-only
-int8-QK forward, whose step is quantisation + forward).  Prints ONE JSON line.
+resident in HBM.  The headline workload is the DiT joint-attention configuration B=1 H=24 S=4608 (512 text
++ 4096 image tokens) D=128 bf16: the line's `value`, `ms_per_step`, `roofline` and `cpu_baseline` are its.
+Without `--config` the other four configurations (1 small, 3 ragged cross attention, 4 long causal, 5 the
+inference-only int8-QK forward, whose step is quantisation + forward) are then timed the same way at up to
+20 steps each and reported as rows of `configs`; `--config 1..5` runs one configuration alone.  Prints ONE JSON line.
 
 Three timed loops after the warm-up, all with the same inputs:
   1. `--steps` steps bracketed by a device synchronisation on both sides, nothing else running on the
@@ -316,9 +318,11 @@ def timed_loops(torch, capi, first, second, steps, warmup):
     return wall_ms, medians, per_kernel
 
 
-def sage_line(args, capi, torch, w, dev):
-    """Inference-only configuration: one step = quantise Q and K to int8 + the int8-QK forward."""
+def sage_line(args, capi, torch, w, dev, steps=None, warmup=None, with_cpu_baseline=True):
+    """Inference-only configuration: one step = quantise Q and K to int8 + the int8-QK forward.  Returns the line."""
     import numpy as np
+    steps = args.steps if steps is None else steps
+    warmup = args.warmup if warmup is None else warmup
     B, H, Sq, Sk, D = w.shape
     q, k, v = (torch.from_numpy(np.ascontiguousarray(t).view(np.int16)).view(torch.bfloat16).to(dev) for t in (w.q, w.k, w.v))
     o = torch.empty_like(q)
@@ -331,7 +335,7 @@ def sage_line(args, capi, torch, w, dev):
         capi.sage_fwd(state["qz"], v, w.scale, out=o)
 
     torch.cuda.reset_peak_memory_stats()
-    ms, med, per_kernel = timed_loops(torch, capi, quant, fwd, args.steps, args.warmup)
+    ms, med, per_kernel = timed_loops(torch, capi, quant, fwd, steps, warmup)
     # the bf16 forward on the same inputs, for the comparison the int8 path has to win
     for _ in range(5):
         capi.attn_fwd(q, k, v, w.scale, want_lse=False, out=o)
@@ -348,7 +352,7 @@ def sage_line(args, capi, torch, w, dev):
     ideal = 0.5 * ops / (PEAK_INT8_TOPS * 1e12) + 0.5 * ops / (PEAK_BF16_TFLOPS * 1e12)
     out = {
         "metric": "int8-QK attention forward incl. quantisation, T(FL)OP/s", "value": ops / (ms * 1e-3) / 1e12,
-        "unit": "TOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
+        "unit": "TOP/s", "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": ms,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8+bf16", "data": "synthetic",
         "config": {"workload": w.name, "B": B, "H": H, "Sq": Sq, "Sk": Sk, "D": D, "causal": bool(w.causal),
                    "step": "quantise Q,K (per-block int8, mean-smoothed K) + int8-QK forward"},
@@ -362,54 +366,38 @@ def sage_line(args, capi, torch, w, dev):
                      "note": "peak = time-weighted blend of 5.0 POP/s int8 and 2.5 PFLOP/s bf16"},
         "kernels_ms": per_kernel,
         "peak_device_MiB": torch.cuda.max_memory_allocated() / 2 ** 20}
-    if not args.no_cpu_baseline:
+    if with_cpu_baseline and not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline_sage(w)
-    print(json.dumps(out))
+    return out
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=50)
-    ap.add_argument("--config", type=int, default=2, help="workload configuration (2 = the headline shape)")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--keep-mask", action="store_true",
-                    help="pass an all-ones [1,1,Sq,Sk] keep-mask, which times the kernels that read an explicit mask "
-                         "(same arithmetic and flop count as the unmasked step)")
-    ap.add_argument("--traffic-calibration", action="store_true",
-                    help="also run one plain 256 MiB device copy, so that FETCH_SIZE / WRITE_SIZE read under "
-                         "rocprofv3 --pmc can be scaled by what the same counters report for a known size")
-    ap.add_argument("--big-head-dims", action="store_true",
-                    help="time the forward for head dims above 128 next to a materialised comparator (a line of its own)")
-    ap.add_argument("--tile-ops", action="store_true",
-                    help="time the element-wise tile primitives instead of an attention workload (a line of its own)")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py: this build runs on one GPU only (heads shard without communication; "
-              "no multi-GPU path exists). Re-run with --gpus 1.", file=sys.stderr)
-        sys.exit(2)
+# Instructions other than MFMAs that the kernels compiled for head dim 64 issue per MFMA (vector ALU + LDS, from the
+# SQ_INSTS_* counters in profiles/attention_kernels_cfg3_ragged_cross.md): at D = 64 a 64-key tile has half the MFMAs
+# of a D = 128 tile for the same softmax / dS arithmetic.
+OTHERS_PER_MFMA_D64 = {"fwd": 12.9, "bwd_dq": 9.1, "bwd_dkdv": 7.1}
+ISSUE_CYCLES_PER_INSTRUCTION = 5.5     # measured: next to an MFMA stream a SIMD issues one other instruction every 5-6 cycles
 
-    import torch
-    from flame_amd import capi, workloads as W
-    if not torch.cuda.is_available():
-        print("bench.py: no GPU visible", file=sys.stderr)
-        sys.exit(3)
-    capi.lib()      # fails loudly when the HIP library is missing
 
-    dev = torch.device("cuda:0")
-    if args.traffic_calibration:
-        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
-        torch.empty_like(src).copy_(src)          # one elementwise copy kernel: reads 256 MiB, writes 256 MiB
-        del src
-    if args.tile_ops:
-        return tile_ops_line(args, capi, torch, dev)
-    if args.big_head_dims:
-        return big_head_dims_line(args, capi, torch, dev)
-    w = W.CONFIGS[args.config]()
+def bound_of(w, kname, launch_ms):
+    """What bounds kernel `kname` at workload `w`, and the rate that bound allows for its algorithmic flops:
+    'launch' when a launch is over before the chip fills (under 20 us), 'valu-issue' at head dim 64, where the
+    instructions between two MFMAs take longer to issue than the MFMA (32 cycles) takes to run, else 'mfma'."""
+    D = w.shape[4]
+    if launch_ms < 0.020:
+        return "launch", None, "a launch of a few microseconds: fixed launch and prologue time, not a pipe, sets the rate"
+    if D <= 64:
+        k = OTHERS_PER_MFMA_D64[kname]
+        frac = 32.0 / max(32.0, ISSUE_CYCLES_PER_INSTRUCTION * k)
+        return ("valu-issue", PEAK_BF16_TFLOPS * frac,
+                f"{k} other instructions per MFMA x {ISSUE_CYCLES_PER_INSTRUCTION} issue cycles against 32 cycles per MFMA: "
+                f"{frac:.2f} of the MFMA peak is the most this instruction mix can reach")
+    return "mfma", PEAK_BF16_TFLOPS, None
+
+
+def attention_line(args, capi, torch, W, w, dev, steps, warmup, headline):
+    """Forward + backward of one workload: the three timed loops and the line built from them.  `headline`: also
+    the input-preparation rate, the materialised comparator and the CPU baseline."""
     B, H, Sq, Sk, D = w.shape
-    if w.do is None:            # inference-only workload (int8-QK forward)
-        return sage_line(args, capi, torch, w, dev)
 
     def dev_t(bits):
         import numpy as np
@@ -423,14 +411,22 @@ def main():
     ws = torch.empty(capi.bwd_workspace_bytes(B, H, Sq, D), dtype=torch.uint8, device=dev)
     mask = torch.ones(1, 1, Sq, Sk, dtype=torch.uint8, device=dev) if args.keep_mask else None
     state = {}
+    drop = args.dropout
 
     def fwd():
-        _, state["lse"] = capi.attn_fwd(q, k, v, w.scale, causal=w.causal, kv_len=kvl, mask=mask, out=o)
+        if drop > 0.0:
+            _, state["lse"] = capi.attn_fwd_dropout(q, k, v, w.scale, drop, 2024, causal=w.causal, kv_len=kvl, mask=mask, out=o)
+        else:
+            _, state["lse"] = capi.attn_fwd(q, k, v, w.scale, causal=w.causal, kv_len=kvl, mask=mask, out=o)
 
     def bwd():
-        capi.attn_bwd(q, k, v, o, do, state["lse"], w.scale, causal=w.causal, kv_len=kvl, mask=mask, workspace=ws, grads=grads)
+        if drop > 0.0:
+            state["grads"] = capi.attn_bwd_dropout(q, k, v, o, do, state["lse"], w.scale, drop, 2024, causal=w.causal, kv_len=kvl,
+                                                   mask=mask, workspace=ws)
+        else:
+            capi.attn_bwd(q, k, v, o, do, state["lse"], w.scale, causal=w.causal, kv_len=kvl, mask=mask, workspace=ws, grads=grads)
 
-    ms, med, per_kernel = timed_loops(torch, capi, fwd, bwd, args.steps, args.warmup)
+    ms, med, per_kernel = timed_loops(torch, capi, fwd, bwd, steps, warmup)
     peak_mib = torch.cuda.max_memory_allocated() / 2 ** 20
 
     flops_fwd, flops_bwd = w.flops(True, False), w.flops(False, True)
@@ -438,24 +434,28 @@ def main():
     # Dominant kernel: bwd_dkdv_kernel.  Per launch it carries four of the five backward GEMMs over
     # every attended (query, key) pair: S recompute, dP, dV, dK = 8 * pairs * D flops.  The fifth
     # (dQ) runs in bwd_dq_kernel, which recomputes S and dP (6 * pairs * D executed, 2 * pairs * D
-    # algorithmic).  The forward kernel carries its two GEMMs (4 * pairs * D).
+    # algorithmic).  The forward kernel carries its two GEMMs (4 * pairs * D).  With the joint schedule one
+    # launch (bwd_joint_kernel) carries all five backward GEMMs: 10 * pairs * D algorithmic, 14 executed.
     pairs_d = w.valid_pairs() * D
     kern_flops = {"fwd": (4 * pairs_d, 4 * pairs_d), "bwd_dkdv": (8 * pairs_d, 8 * pairs_d),
-                  "bwd_dq": (2 * pairs_d, 6 * pairs_d)}          # (algorithmic, executed)
+                  "bwd_dq": (2 * pairs_d, 6 * pairs_d), "bwd_joint": (10 * pairs_d, 14 * pairs_d)}          # (algorithmic, executed)
     kernels = {}
     for kname, (alg, exe) in kern_flops.items():
         if kname in per_kernel:
             t = per_kernel[kname] * 1e-3
             kernels[kname] = {"avg_launch_ms": per_kernel[kname], "algorithmic_tflops": alg / t / 1e12,
                               "executed_tflops": exe / t / 1e12, "frac_of_peak_executed": exe / t / 1e12 / PEAK_BF16_TFLOPS}
-    dom = "bwd_dkdv"
+    dom = "bwd_joint" if "bwd_joint" in kernels else "bwd_dkdv"
     achieved = kernels[dom]["algorithmic_tflops"]
+    bound, bound_peak, bound_note = bound_of(w, dom, per_kernel[dom]) if dom != "bwd_joint" else ("mfma", PEAK_BF16_TFLOPS, None)
+    plain = not args.keep_mask and drop == 0.0 and args.head_dim == 0 and args.bwd_schedule == "default"
     out = {
-        "metric": METRIC, "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak",
+        "metric": METRIC, "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": steps,
+        "warmup": warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": w.name, "B": B, "H": H, "Sq": Sq, "Sk": Sk, "D": D, "causal": bool(w.causal),
-                   "step": "forward (O+LSE) + recompute backward (dQ,dK,dV)", "keep_mask": bool(args.keep_mask)},
+                   "step": "forward (O+LSE) + recompute backward (dQ,dK,dV)", "keep_mask": bool(args.keep_mask),
+                   "dropout_p": drop, "bwd_schedule": args.bwd_schedule},
         "frac_of_bf16_mfma_peak": tflops / PEAK_BF16_TFLOPS,
         "timing": {"forward_ms_median": med["first_ms_median"], "backward_ms_median": med["second_ms_median"],
                    "step_ms_median": med["step_ms_median"], "step_ms_min": med["step_ms_min"], "step_ms_max": med["step_ms_max"],
@@ -463,24 +463,193 @@ def main():
                    "forward_tflops": flops_fwd / (med["first_ms_median"] * 1e-3) / 1e12,
                    "backward_tflops": flops_bwd / (med["second_ms_median"] * 1e-3) / 1e12,
                    "step_tflops": (flops_fwd + flops_bwd) / (med["step_ms_median"] * 1e-3) / 1e12},
-        "roofline": {"bound": "mfma", "kernel": "bwd_dkdv_kernel", "achieved": achieved, "peak": PEAK_BF16_TFLOPS,
+        # `peak` is always the published MFMA peak and `frac` the fraction of it; where something else bounds the
+        # kernel, `bound` names it and `bound_peak` / `frac_of_bound` give the rate that bound allows
+        "roofline": {"bound": bound, "kernel": f"{dom}_kernel", "achieved": achieved, "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS,
-                     "traffic": None if args.keep_mask else recorded_traffic(w.name, "bwd_dkdv_kernel"),
-                     "avg_launch_ms": per_kernel[dom], "flops_per_launch": 8 * pairs_d},
+                     "traffic": recorded_traffic(w.name, f"{dom}_kernel") if plain else None,
+                     "avg_launch_ms": per_kernel[dom], "flops_per_launch": kern_flops[dom][0]},
         "kernels": kernels,
         "kernels_ms": per_kernel,
         "peak_device_MiB": peak_mib,
         "saved_activations": w.saved_activation_bytes(),
     }
-    if args.config == 2:
+    if bound != "mfma":
+        out["roofline"]["bound_note"] = bound_note
+        if bound_peak:
+            out["roofline"]["bound_peak"] = bound_peak
+            out["roofline"]["frac_of_bound"] = achieved / bound_peak
+    if headline:
         out["input_prep"] = input_prep_rate(capi, W, torch, B, H, Sq, D, dev)
-        if not args.keep_mask:
+        if plain:
             del ws
             out["materialised_comparator"] = materialised_comparator(capi, torch, q, k, v, do, w.scale, o, grads)
-    if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(w)
-    print(json.dumps(out))
+        if not args.no_cpu_baseline:
+            out["cpu_baseline"] = cpu_baseline(w)
+    return out
+
+
+def summary_of(line):
+    """The row a configuration contributes to the headline line's `configs`."""
+    r = line["roofline"]
+    row = {"workload": line["config"]["workload"], "steps": line["steps"], "ms_per_step": line["ms_per_step"],
+           "step_ms_median_hip_events": line["timing"]["step_ms_median"],
+           "value": line["value"], "unit": line["unit"], "dominant_kernel": r["kernel"], "roofline_bound": r["bound"],
+           "roofline_frac": r["frac"], "dominant_kernel_avg_launch_ms": r["avg_launch_ms"], "kernels_ms": line["kernels_ms"]}
+    if "frac_of_bf16_mfma_peak" in line:
+        row["frac_of_bf16_mfma_peak"] = line["frac_of_bf16_mfma_peak"]
+        row["forward_ms"] = line["timing"]["forward_ms_median"]
+        row["backward_ms"] = line["timing"]["backward_ms_median"]
+    else:
+        row["quantise_ms"] = line["timing"]["quantise_ms_median"]
+        row["forward_ms"] = line["timing"]["forward_ms_median"]
+        row["frac_of_int8_bf16_blend"] = r["frac"]
+    for key in ("bound_peak", "frac_of_bound", "bound_note"):
+        if key in r:
+            row["roofline_" + key] = r[key]
+    return row
+
+
+def mfma_ceiling_line(args, capi, torch, W, dev):
+    """What the matrix pipe alone allows: a loop of nothing but bf16 MFMAs on bf16 N(0,1) operands, one wavefront per
+    SIMD on every compute unit, with as many MFMAs as each attention kernel of the headline shape executes, next to
+    those kernels' own times from the same process.  Under rocprofv3 --pmc GRBM_GUI_ACTIVE the same run gives the
+    clock each of them is granted."""
+    import ctypes
+    from flame_amd import build as fb
+    probe = ctypes.CDLL(fb.PROBE_LIB_PATH)
+    probe.flame_probe_mfma_data_bytes.restype = ctypes.c_size_t
+    nbytes = probe.flame_probe_mfma_data_bytes()
+    g = torch.Generator(device=dev).manual_seed(5)
+    data = torch.randn(nbytes // 2, device=dev, generator=g).to(torch.bfloat16)
+    sink = torch.zeros(16, device=dev)
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    w = W.CONFIGS[2]()
+    B, H, Sq, Sk, D = w.shape
+    line = attention_line(args, capi, torch, W, w, dev, min(args.steps, 50), min(args.warmup, 10), headline=False)
+    pairs_d = w.valid_pairs() * D
+    executed = {"fwd": 4 * pairs_d, "bwd_dq": 6 * pairs_d, "bwd_dkdv": 8 * pairs_d}
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    ones = torch.ones_like(data)           # the same loop on constant operands: far fewer bits toggle per MFMA
+
+    def time_loop(operands, iters, waves=4):
+        def run():
+            rc = probe.flame_probe_mfma_loop(ctypes.c_void_p(operands.data_ptr()), ctypes.c_void_p(sink.data_ptr()), cus, waves, iters, stream)
+            assert rc == 0, rc
+
+        for _ in range(5):
+            run()
+        times = []
+        for _ in range(20):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            run()
+            e1.record()
+            e1.synchronize()
+            times.append(e0.elapsed_time(e1))
+        return statistics.median(times)
+
+    rows = {}
+    for kname, flops in executed.items():
+        per_wave = flops / 32768.0 / (cus * 4)                 # MFMAs (32x32x16: 32768 flops) per wavefront
+        iters = max(1, int(round(per_wave / 8)))
+        loop_flops = iters * 8 * 32768.0 * cus * 4
+        t_loop = time_loop(data, iters)
+        t_const = time_loop(ones, iters)
+        t_two = time_loop(data, max(1, iters // 2), waves=8)   # two wavefronts per SIMD, half the MFMAs each
+        t_kernel = line["kernels_ms"][kname]
+        rows[kname] = {"executed_flops": flops, "kernel_ms": t_kernel, "kernel_executed_tflops": flops / (t_kernel * 1e-3) / 1e12,
+                       "mfma_only_loop_ms_same_mfma_count": t_loop, "mfma_only_loop_tflops": loop_flops / (t_loop * 1e-3) / 1e12,
+                       "mfma_only_loop_two_wavefronts_per_simd_ms": t_two,
+                       "mfma_only_loop_constant_operands_ms": t_const,
+                       "mfma_only_loop_constant_operands_tflops": loop_flops / (t_const * 1e-3) / 1e12,
+                       "kernel_time_over_mfma_only_time": t_kernel / t_loop}
+    return {"metric": "attention kernels against an MFMA-only loop of the same MFMA count", "unit": "ms", "n_gpus": 1,
+            "dtype": "bf16", "data": "synthetic", "higher_is_better": False,
+            "config": {"workload": w.name, "probe": "v_mfma_f32_32x32x16_bf16 only, N(0,1) bf16 operands, 4 wavefronts per compute unit"},
+            "kernels": rows, "step_ms": line["ms_per_step"]}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--config", type=int, default=0,
+                    help="workload configuration 1..5 alone; default: the headline shape (2) with its extras, then 1, 3, 4, 5 "
+                         "at up to 20 steps each, reported under `configs` of the one line")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--keep-mask", action="store_true",
+                    help="pass an all-ones [1,1,Sq,Sk] keep-mask, which times the kernels that read an explicit mask "
+                         "(same arithmetic and flop count as the unmasked step)")
+    ap.add_argument("--dropout", type=float, default=0.0,
+                    help="dropout probability of the attention weights: times the DROPOUT builds of the kernels")
+    ap.add_argument("--head-dim", type=int, default=0,
+                    help="the headline shape with another head dim (e.g. 96, which runs zero-padded on the 128-wide kernels)")
+    ap.add_argument("--bwd-schedule", choices=("default", "joint", "rows"), default="default",
+                    help="how the backward of the unmasked shapes is launched (FLAME_ATTN_BWD_SCHEDULE): dQ then dK/dV kernel; "
+                         "a rows pre-pass and both in one grid; the pre-pass and the two kernels")
+    ap.add_argument("--traffic-calibration", action="store_true",
+                    help="also run one plain 256 MiB device copy, so that FETCH_SIZE / WRITE_SIZE read under "
+                         "rocprofv3 --pmc can be scaled by what the same counters report for a known size")
+    ap.add_argument("--big-head-dims", action="store_true",
+                    help="time the forward for head dims above 128 next to a materialised comparator (a line of its own)")
+    ap.add_argument("--tile-ops", action="store_true",
+                    help="time the element-wise tile primitives instead of an attention workload (a line of its own)")
+    ap.add_argument("--mfma-ceiling", action="store_true",
+                    help="time an MFMA-only loop with the MFMA count of each kernel of the headline shape (a line of its own)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (heads shard without communication; "
+              "no multi-GPU path exists). Re-run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from flame_amd import capi, workloads as W
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(3)
+    capi.lib()      # fails loudly when the HIP library is missing
+    if args.bwd_schedule != "default":
+        os.environ["FLAME_ATTN_BWD_SCHEDULE"] = args.bwd_schedule
+
+    dev = torch.device("cuda:0")
+    if args.traffic_calibration:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+        torch.empty_like(src).copy_(src)          # one elementwise copy kernel: reads 256 MiB, writes 256 MiB
+        del src
+    if args.tile_ops:
+        return tile_ops_line(args, capi, torch, dev)
+    if args.big_head_dims:
+        return big_head_dims_line(args, capi, torch, dev)
+    if args.mfma_ceiling:
+        print(json.dumps(mfma_ceiling_line(args, capi, torch, W, dev)))
+        return 0
+
+    variant = args.keep_mask or args.dropout > 0.0 or args.head_dim != 0 or args.bwd_schedule != "default"
+    all_configs = args.config == 0 and not variant
+    cfg = args.config or 2
+    w = W.config2(D=args.head_dim) if (args.head_dim and cfg == 2) else W.CONFIGS[cfg]()
+    if w.do is None:            # inference-only workload (int8-QK forward)
+        print(json.dumps(sage_line(args, capi, torch, w, dev)))
+        return 0
+    line = attention_line(args, capi, torch, W, w, dev, args.steps, args.warmup, headline=(cfg == 2 and not args.head_dim))
+    if all_configs:
+        # the other four configurations, timed the same way at up to 20 steps each (cfg 4 takes 8 ms per step), one row each
+        rows = {"cfg2": summary_of(line)}
+        del w
+        for other in (1, 3, 4, 5):
+            torch.cuda.empty_cache()
+            wo = W.CONFIGS[other]()
+            n, nw = min(args.steps, 20), min(args.warmup, 5)
+            lo = (sage_line(args, capi, torch, wo, dev, n, nw, with_cpu_baseline=False) if wo.do is None
+                  else attention_line(args, capi, torch, W, wo, dev, n, nw, headline=False))
+            rows[f"cfg{other}"] = summary_of(lo)
+            del wo, lo
+        line["configs"] = dict(sorted(rows.items()))
+    print(json.dumps(line))
+    return 0
 
 
 if __name__ == "__main__":
-    main()
+    sys.exit(main())

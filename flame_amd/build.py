@@ -63,6 +63,17 @@ def build_lib(verbose: bool = False, extra=()) -> str:
 
 
 
+PROBE_LIB_PATH = os.path.join(LIB_DIR, "libflame_mfma_probe.so")
+
+
+def build_probe(verbose: bool = False) -> str:
+    """The MFMA-only loop that bench.py --mfma-ceiling times (a measurement aid in a library of its own: nothing of
+    it is in the attention library's ABI)."""
+    os.makedirs(LIB_DIR, exist_ok=True)
+    _run([HIPCC, *FLAGS, os.path.join(CSRC, "mfma_probe.hip"), "-o", PROBE_LIB_PATH], verbose)
+    return PROBE_LIB_PATH
+
+
 def build_host_test(verbose: bool = False) -> str:
     """Compiles the C++ host-layer test driver (tests/host/host_api_test.cpp) against the library."""
     root = os.path.dirname(HERE)
@@ -81,4 +92,5 @@ def build_host_test(verbose: bool = False) -> str:
 
 if __name__ == "__main__":
     print(build_lib(verbose=True, extra=sys.argv[1:]))
+    print(build_probe(verbose=True))
     print(build_host_test(verbose=True))
