@@ -13,10 +13,8 @@
 //   flame::SageAttention                            src/sage_attention.rs:21-171
 //   flame::autograd_v4::{SdpaStats, SdpaHooks, register_sdpa_hooks}
 //                                                   src/autograd_v4/ops/sdpa.rs:56-79, :1063-1074
-//   flame::perf_telemetry::{telemetry_enabled, log_sdpa_event, log_sdpa_fallback_event}
-//                                                   src/perf_telemetry.rs:7-57, :60-190
-//   flame::activation_offload::{ActivationOffloadPool, OffloadCompression, OffloadHandle}
-//                                                   src/activation_offload.rs:84-96, :291-304, :365-775
+//   flame::perf_telemetry::{telemetry_enabled, log_sdpa_event}
+//                                                   src/perf_telemetry.rs:7-40, :60-150
 //
 // Only what the path needs of the tensor type is here: a reference-counted device buffer with a
 // shape, element strides, an offset and a dtype (the reference's Tensor supplies exactly these to
@@ -862,13 +860,6 @@ struct SdpaTelemetryRecord {                // :7-40
              autotune_fallback = 0, autotune_errors = 0, autotune_tuned = 0, cache_hits = 0, cache_misses = 0, cache_saved = 0,
              cache_loads = 0, cache_load_errors = 0, cache_entries = 0;
 };
-struct SdpaFallbackTelemetryRecord {        // :42-56
-    size_t batch = 0, heads = 0, q_len = 0, k_len = 0, dh = 0, dv = 0, from_chunk = 0, to_chunk = 0;
-    const char* reason = "";
-    std::optional<uint64_t> workspace_required, workspace_limit;
-    std::optional<size_t> free_mem_mb;
-    std::optional<int32_t> error_code;
-};
 inline bool telemetry_enabled() {           // :60-66 (read once)
     static const bool on = [] {
         const char* p = std::getenv("FLAME_SDPA_TELEMETRY_PATH");
@@ -893,7 +884,6 @@ inline unsigned long long now_ns() {
     return (unsigned long long)std::chrono::duration_cast<std::chrono::nanoseconds>(
                std::chrono::system_clock::now().time_since_epoch()).count();
 }
-inline std::string opt_u64(const std::optional<uint64_t>& v) { return v ? std::to_string(*v) : "null"; }
 }  // namespace detail
 inline void log_sdpa_event(const SdpaTelemetryRecord& r) {          // :103-150
     if (!telemetry_enabled()) return;
@@ -918,21 +908,6 @@ inline void log_sdpa_event(const SdpaTelemetryRecord& r) {          // :103-150
                  (unsigned long long)r.autotune_errors, (unsigned long long)r.autotune_tuned,
                  (unsigned long long)r.cache_hits, (unsigned long long)r.cache_misses, (unsigned long long)r.cache_saved,
                  (unsigned long long)r.cache_loads, (unsigned long long)r.cache_load_errors, (unsigned long long)r.cache_entries);
-    std::fflush(f);
-}
-inline void log_sdpa_fallback_event(const SdpaFallbackTelemetryRecord& r) {   // :152-190
-    if (!telemetry_enabled()) return;
-    std::lock_guard<std::mutex> lk(detail::guard());
-    FILE* f = detail::writer();
-    if (!f) return;
-    std::fprintf(f,
-                 "{\"op\":\"sdpa_stream_bf16_fallback\",\"timestamp_ns\":%llu,\"batch\":%zu,\"heads\":%zu,\"q_len\":%zu,"
-                 "\"k_len\":%zu,\"dh\":%zu,\"dv\":%zu,\"from_chunk\":%zu,\"to_chunk\":%zu,\"reason\":\"%s\","
-                 "\"workspace_required\":%s,\"workspace_limit\":%s,\"free_mem_mb\":%s,\"error_code\":%s}\n",
-                 detail::now_ns(), r.batch, r.heads, r.q_len, r.k_len, r.dh, r.dv, r.from_chunk, r.to_chunk, r.reason,
-                 detail::opt_u64(r.workspace_required).c_str(), detail::opt_u64(r.workspace_limit).c_str(),
-                 r.free_mem_mb ? std::to_string(*r.free_mem_mb).c_str() : "null",
-                 r.error_code ? std::to_string(*r.error_code).c_str() : "null");
     std::fflush(f);
 }
 }  // namespace perf_telemetry
@@ -1026,12 +1001,14 @@ inline Result<Tensor> sdpa_stream_bf16_with_workspace(const Tensor& q, const Ten
 
 namespace ops {
 namespace attn {
-// src/ops/attn.rs.  The reference plans a query chunk whose fp32 scratch (chunk x K logits + chunk x (Dv + 2) rows,
-// :72-84) fits a budget taken from free device memory, and steps down a list of candidate chunks when the planner or
-// a launch refuses one, recording every step (its tests assert on those records: tests/streaming_attn.rs:301-397).
-// The planner, its candidates, its budget rules, its records and its telemetry are mirrored with the reference's own
-// scratch formula as the accounting, so that a caller sees the same chosen chunk and the same fallback events; the
-// kernels behind it keep their scratch in registers and LDS and run the same launch whatever chunk is chosen.
+// src/ops/attn.rs:327-598.  The reference's function plans a query chunk whose fp32 scratch (chunk x K logits plus
+// running rows, :72-84) fits a budget taken from free device memory and steps down a list of chunks when a launch
+// fails (:113-209, :453-592).  The fused forward keeps that scratch in registers and LDS and runs the same launch
+// whatever the chunk, so nothing is planned, budgeted or retried here: the chunk is validated (0 is an error, as
+// there) and otherwise has no effect.
+// Beyond the reference: a keep-mask is taken (bf16, 1 = keep; the reference's function refuses one, :366-370,
+// although its test passes one, tests/streaming_attn.rs:413-489), and the three tensors may be strided views and
+// have key lengths of their own.
 struct StreamingAttnCfg {                                     // :8-25
     float scale = 1.0f;
     size_t chunk_size = 2048;
@@ -1039,185 +1016,13 @@ struct StreamingAttnCfg {                                     // :8-25
     const Tensor* mask = nullptr;
 };
 
-constexpr size_t STREAM_ATTENTION_MIN_CHUNK = 32, STREAM_ATTENTION_MAX_CHUNK = 2048;                  // :113-119
-constexpr uint64_t STREAM_ATTENTION_MIN_BUDGET_BYTES = 64ull << 20, STREAM_ATTENTION_DEFAULT_BUDGET_BYTES = 512ull << 20,
-                   STREAM_ATTENTION_HARD_CAP_BYTES = 2ull << 30;
-
-// the planner's accounting: what the reference's kernels need for this chunk (:72-84); nullopt on overflow
-inline std::optional<uint64_t> streaming_workspace_bytes(size_t chunk_rows, size_t k_len, size_t dv) {
-    if (chunk_rows == 0 || k_len == 0) return 0;
-    unsigned __int128 total = (unsigned __int128)chunk_rows * k_len + (unsigned __int128)chunk_rows * ((unsigned __int128)dv + 2);
-    total *= 4;
-    if (total > UINT64_MAX) return std::nullopt;
-    return (uint64_t)total;
-}
-inline std::vector<size_t> streaming_chunk_candidates(size_t q_len) {                                   // :128-155
-    static const size_t preferred[13] = {2048, 1536, 1024, 768, 512, 384, 256, 192, 128, 96, 64, 48, 32};
-    std::vector<size_t> c;
-    if (q_len == 0) return c;
-    for (size_t p : preferred) {
-        const size_t cand = std::min(p, q_len);
-        if (cand < STREAM_ATTENTION_MIN_CHUNK && q_len >= STREAM_ATTENTION_MIN_CHUNK) continue;
-        if (std::find(c.begin(), c.end(), cand) == c.end()) c.push_back(cand);
-    }
-    if (c.empty()) c.push_back(std::max<size_t>(q_len, 1));
-    std::sort(c.begin(), c.end(), std::greater<size_t>());
-    return c;
-}
-
-struct StreamingTilePlan {                                    // :121-126
-    size_t chunk = 1;
-    uint64_t workspace_bytes = 0, budget_bytes = 0;
-};
-inline Result<StreamingTilePlan> plan_streaming_chunk(size_t q_len, size_t k_len, size_t dv) {           // :157-209
-    if (q_len == 0 || k_len == 0 || dv == 0) return StreamingTilePlan{std::max<size_t>(q_len, 1), 0, 0};
-    uint64_t budget;
-    const char* forced = std::getenv("FLAME_SDPA_PLANNER_BUDGET_BYTES");
-    char* end = nullptr;
-    const unsigned long long forced_v = forced ? std::strtoull(forced, &end, 10) : 0;
-    if (forced && end != forced && *end == 0) {
-        budget = forced_v;
-    } else {
-        size_t free_b = 0, total_b = 0;
-        if (hipMemGetInfo(&free_b, &total_b) != hipSuccess) free_b = 0;
-        budget = free_b > 0 ? (uint64_t)((double)free_b * 0.75) : STREAM_ATTENTION_DEFAULT_BUDGET_BYTES;
-        budget = std::max(budget, STREAM_ATTENTION_MIN_BUDGET_BYTES);
-    }
-    budget = std::min(budget, STREAM_ATTENTION_HARD_CAP_BYTES);
-    const auto candidates = streaming_chunk_candidates(q_len);
-    for (size_t chunk : candidates) {
-        const auto required = streaming_workspace_bytes(std::min(chunk, q_len), k_len, dv);
-        if (required && *required <= budget) return StreamingTilePlan{chunk, *required, budget};
-    }
-    const size_t smallest = candidates.empty() ? 1 : candidates.back();
-    const auto required = streaming_workspace_bytes(std::min(smallest, q_len), k_len, dv);
-    if (!required) return invalid("streaming attention planner overflow");
-    char msg[200];
-    std::snprintf(msg, sizeof msg, "streaming attention planner: chunk %zu requires %.2f MiB workspace but budget is %.2f MiB",
-                  smallest, (double)*required / 1048576.0, (double)budget / 1048576.0);
-    return Error{Error::OutOfMemory, msg};
-}
-
-struct StreamingFallbackReason {                              // :211-223
-    enum Kind { Oom, WorkspaceBudget } kind = Oom;
-    int error_code = -1;
-    std::optional<uint64_t> required_bytes, budget_bytes;
-};
-struct StreamingFallbackEvent {                               // :225-230
-    size_t from_chunk = 0, to_chunk = 0;
-    StreamingFallbackReason reason;
-};
-struct StreamingAttnLaunchInfo {                              // :232-239
-    size_t requested_chunk = 0;
-    std::optional<size_t> chosen_chunk;
-    size_t retries = 0;
-    std::vector<StreamingFallbackEvent> fallbacks;
-    std::optional<int> last_error;
-};
-namespace detail_launch {
-inline std::mutex& guard() {
-    static std::mutex m;
-    return m;
-}
-inline StreamingAttnLaunchInfo& last() {
-    static StreamingAttnLaunchInfo info;
-    return info;
-}
-inline void record(const StreamingAttnLaunchInfo& info) {
-    std::lock_guard<std::mutex> lk(guard());
-    last() = info;
-}
-}  // namespace detail_launch
-inline StreamingAttnLaunchInfo streaming_attn_last_launch_info() {                                       // :318-323
-    std::lock_guard<std::mutex> lk(detail_launch::guard());
-    return detail_launch::last();
-}
-
-// :326-600.  Beyond the reference: a keep-mask is taken (bf16, 1 = keep; the reference's function refuses one, :366-370,
-// although its test passes one, tests/streaming_attn.rs:413-489), and the three tensors may be strided views and have
-// key lengths of their own.  Only a launch failure of the device layer makes the loop step down a chunk; argument errors
-// are returned at once.
 inline Result<Tensor> streaming_attn_bf16_fp32(const Tensor& q, const Tensor& k, const Tensor& v, const StreamingAttnCfg& cfg) {
     if (cfg.chunk_size == 0) return invalid("streaming attention chunk_size must be > 0");
     if (q.dtype() != DType::BF16 || k.dtype() != DType::BF16 || v.dtype() != DType::BF16)
         return invalid("streaming attention expects BF16 tensors");
     if (q.shape().size() != 4 || k.shape().size() != 4 || v.shape().size() != 4) return invalid("expected 4D tensors");
     if (q.shape()[3] != k.shape()[3]) return invalid("head dimensions for Q and K differ");
-    const size_t b = (size_t)q.shape()[0], h = (size_t)q.shape()[1], s = (size_t)q.shape()[2], dh = (size_t)q.shape()[3];
-    const size_t s_k = (size_t)k.shape()[2], dv = (size_t)v.shape()[3];
-    auto planned = plan_streaming_chunk(s, s_k, dv);
-    if (!planned.ok()) return planned.error();
-    StreamingTilePlan plan = planned.value();
-    const size_t requested = std::min(std::min(std::max<size_t>(cfg.chunk_size, 1), std::max<size_t>(s, 1)), STREAM_ATTENTION_MAX_CHUNK);
-    const auto requested_required = streaming_workspace_bytes(std::min(requested, s), s_k, dv);
-    if (requested_required && *requested_required <= plan.budget_bytes) {
-        plan.chunk = requested;
-        plan.workspace_bytes = *requested_required;
-    }
-    auto candidates = streaming_chunk_candidates(s);
-    if (std::find(candidates.begin(), candidates.end(), plan.chunk) == candidates.end()) {
-        candidates.push_back(plan.chunk);
-        std::sort(candidates.begin(), candidates.end(), std::greater<size_t>());
-    }
-    if (candidates.empty()) return invalid("no valid chunk size candidates for streaming attention");
-    size_t idx = (size_t)(std::find(candidates.begin(), candidates.end(), plan.chunk) - candidates.begin());
-    if (idx >= candidates.size()) idx = 0;
-
-    StreamingAttnLaunchInfo info;
-    info.requested_chunk = std::max<size_t>(requested, 1);
-    auto log_fallback = [&](size_t from, size_t to, const StreamingFallbackReason& why) {
-        info.fallbacks.push_back(StreamingFallbackEvent{from, to, why});
-        info.retries = info.fallbacks.size();
-        if (!perf_telemetry::telemetry_enabled()) return;
-        perf_telemetry::SdpaFallbackTelemetryRecord r;
-        r.batch = b; r.heads = h; r.q_len = s; r.k_len = s_k; r.dh = dh; r.dv = dv;
-        r.from_chunk = from; r.to_chunk = to;
-        r.reason = why.kind == StreamingFallbackReason::Oom ? "oom" : "workspace_budget";
-        r.workspace_required = why.required_bytes; r.workspace_limit = why.budget_bytes;
-        if (why.kind == StreamingFallbackReason::Oom) r.error_code = why.error_code;
-        perf_telemetry::log_sdpa_fallback_event(r);
-    };
-    if (requested_required && *requested_required > plan.budget_bytes && requested > plan.chunk) {
-        StreamingFallbackReason why;
-        why.kind = StreamingFallbackReason::WorkspaceBudget;
-        why.required_bytes = *requested_required;
-        why.budget_bytes = plan.budget_bytes;
-        log_fallback(requested, plan.chunk, why);
-    }
-    while (idx < candidates.size()) {
-        const size_t chunk = candidates[idx];
-        const auto required = streaming_workspace_bytes(std::min(chunk, s), s_k, dv);
-        if (!required) return invalid("streaming attention workspace overflow");
-        if (*required > plan.budget_bytes) {
-            if (idx + 1 >= candidates.size()) {
-                info.chosen_chunk = chunk;
-                detail_launch::record(info);
-                return Error{Error::OutOfMemory, "streaming attention planner rejected chunk " + std::to_string(chunk)};
-            }
-            StreamingFallbackReason why;
-            why.kind = StreamingFallbackReason::WorkspaceBudget;
-            why.required_bytes = *required;
-            why.budget_bytes = plan.budget_bytes;
-            log_fallback(chunk, candidates[idx + 1], why);
-            ++idx;
-            continue;
-        }
-        auto out = cuda_ops_bf16::sdpa_stream_bf16_with_workspace(q, k, v, cfg.mask, chunk, cfg.causal, cfg.scale, std::nullopt);
-        if (out.ok() || out.error().kind != Error::Cuda || idx + 1 >= candidates.size()) {
-            info.chosen_chunk = chunk;
-            if (!out.ok()) info.last_error = out.error().kind == Error::Cuda ? 2 : 1;        // FC_ERR_LAUNCH / FC_ERR_INVALID_ARGUMENT
-            detail_launch::record(info);
-            return out;
-        }
-        StreamingFallbackReason why;                          // :571-590: a failed launch counts as out of memory
-        why.kind = StreamingFallbackReason::Oom;
-        why.required_bytes = *required;
-        why.budget_bytes = plan.budget_bytes;
-        info.last_error = 2;
-        log_fallback(chunk, candidates[idx + 1], why);
-        ++idx;
-    }
-    return invalid("no valid chunk size candidates for streaming attention");
+    return cuda_ops_bf16::sdpa_stream_bf16(q, k, v, cfg.mask, cfg.chunk_size, cfg.causal, cfg.scale);
 }
 }  // namespace attn
 }  // namespace ops
@@ -1283,248 +1088,6 @@ inline Result<Tensor> prep_qk(const Tensor& x_bnhd, const Tensor* weight, const 
     return bf16_ops::detail_prep::run(x_bnhd.permute({0, 2, 1, 3}), weight, cos, sin, eps, true, "prep_qk");
 }
 }  // namespace attention
-
-// ------------------------------------------------------------------------------------ activation offload
-// Saved activations pushed to pinned host memory in the forward and pulled back in the backward
-// (src/activation_offload.rs).  One transfer stream of the pool's own (non-blocking, default priority), one pinned
-// buffer and two events per slot, no host synchronisation in push or pull:
-//   push: record done[slot] on the default stream, the transfer stream waits for it, then (FP8: quantise into the
-//         slot's device staging buffer, then) copy device -> host on the transfer stream;
-//   pull: copy host -> device on the transfer stream (same-stream order puts it after the push's copy; FP8: into
-//         the staging buffer, then dequantise into the new tensor), record ready[slot] there, the default stream
-//         waits for it.
-// Slots are handed out from a stack (LIFO, the order the backward consumes them); a full pool refuses the push;
-// clear() frees every slot and makes the handles issued so far stale.  The pushed tensor is kept alive until its
-// slot is drained.  FP8 halves host memory and link traffic with the reference's fixed scale 8/448 (:543-549).
-namespace activation_offload {
-
-enum class OffloadCompression { None, FP8 };
-
-class OffloadHandle {                      // :291-304
-   public:
-    size_t slot() const { return slot_; }
-
-   private:
-    friend class ActivationOffloadPool;
-    size_t slot_ = 0;
-    uint64_t epoch_ = 0;
-};
-
-class ActivationOffloadPool {
-   public:
-    ActivationOffloadPool(const ActivationOffloadPool&) = delete;
-    ActivationOffloadPool& operator=(const ActivationOffloadPool&) = delete;
-
-    // :365-428
-    static Result<std::unique_ptr<ActivationOffloadPool>> create(size_t num_slots, size_t max_bytes, OffloadCompression compression) {
-        if (num_slots == 0) return invalid("ActivationOffloadPool::new: num_slots must be > 0");
-        if (max_bytes == 0) return invalid("ActivationOffloadPool::new: max_bytes must be > 0");
-        std::unique_ptr<ActivationOffloadPool> p(new ActivationOffloadPool());
-        p->compression_ = compression;
-        p->slot_bytes_ = max_bytes;
-        const size_t host_buf_bytes = compression == OffloadCompression::FP8 ? (max_bytes + 1) / 2 : max_bytes;
-        hipError_t e = hipStreamCreateWithFlags(&p->transfer_, hipStreamNonBlocking);
-        if (e != hipSuccess) return cuda_error("hipStreamCreateWithFlags", (int)e);
-        for (size_t i = 0; i < num_slots; ++i) {
-            void* h = nullptr;
-            if ((e = hipHostMalloc(&h, host_buf_bytes, hipHostMallocDefault)) != hipSuccess) return cuda_error("hipHostMalloc", (int)e);
-            p->host_.push_back(h);
-            hipEvent_t d, r;
-            if ((e = hipEventCreateWithFlags(&d, hipEventDisableTiming)) != hipSuccess) return cuda_error("hipEventCreate", (int)e);
-            p->done_.push_back(d);
-            if ((e = hipEventCreateWithFlags(&r, hipEventDisableTiming)) != hipSuccess) return cuda_error("hipEventCreate", (int)e);
-            p->ready_.push_back(r);
-            if (compression == OffloadCompression::FP8) {
-                void* g = nullptr;
-                if ((e = hipMalloc(&g, host_buf_bytes)) != hipSuccess) return cuda_error("hipMalloc", (int)e);
-                p->staging_.push_back(g);
-            }
-        }
-        p->meta_.resize(num_slots);
-        p->pushed_.assign(num_slots, false);
-        p->keep_alive_.resize(num_slots);
-        for (size_t i = num_slots; i-- > 0;) p->free_stack_.push_back(i);     // slot 0 on top
-        return p;
-    }
-    ~ActivationOffloadPool() {
-        if (transfer_) (void)hipStreamSynchronize(transfer_);
-        for (void* g : staging_) (void)hipFree(g);
-        for (void* h : host_) (void)hipHostFree(h);
-        for (hipEvent_t e : done_) (void)hipEventDestroy(e);
-        for (hipEvent_t e : ready_) (void)hipEventDestroy(e);
-        if (transfer_) (void)hipStreamDestroy(transfer_);
-    }
-
-    size_t num_slots() const { return host_.size(); }                        // :431-434
-    size_t slot_bytes() const { return slot_bytes_; }                        // :437-440
-    size_t host_bytes() const {                                              // :443-450
-        return (compression_ == OffloadCompression::FP8 ? (slot_bytes_ + 1) / 2 : slot_bytes_) * host_.size();
-    }
-    size_t in_flight() const { return (size_t)std::count(pushed_.begin(), pushed_.end(), true); }   // :453-455
-
-    // :465-617
-    Result<OffloadHandle> push(const Tensor& t) {
-        if (!t.defined()) return invalid("ActivationOffloadPool::push: tensor is empty");
-        if (t.dtype() != DType::BF16 && t.dtype() != DType::F32)
-            return unsupported("ActivationOffloadPool::push: dtype not supported (BF16/F32 only)");
-        if (!t.is_contiguous()) return unsupported("ActivationOffloadPool::push: tensor is a strided view");
-        const size_t numel = (size_t)t.numel(), bytes = numel * dtype_size(t.dtype());
-        if (bytes == 0) return invalid("ActivationOffloadPool::push: tensor is empty");
-        if (bytes > slot_bytes_)
-            return invalid("ActivationOffloadPool::push: tensor " + std::to_string(bytes) + " bytes exceeds slot capacity " +
-                           std::to_string(slot_bytes_) + " bytes");
-        if (compression_ == OffloadCompression::FP8 && t.dtype() != DType::BF16)
-            return unsupported("FP8 compression only supports BF16 activations");
-        if (free_stack_.empty())
-            return Error{Error::InvalidOperation, "ActivationOffloadPool full: " + std::to_string(host_.size()) +
-                                                       " slots all in-flight. Increase num_slots."};
-        const size_t slot = free_stack_.back();
-        free_stack_.pop_back();
-        auto fail = [&](const char* what, int code) {
-            free_stack_.push_back(slot);
-            return cuda_error(std::string("activation offload push: ") + what, code);
-        };
-        hipError_t e = hipEventRecord(done_[slot], nullptr);                  // the producer's progress on the default stream
-        if (e != hipSuccess) return fail("event record", (int)e);
-        if ((e = hipStreamWaitEvent(transfer_, done_[slot], 0)) != hipSuccess) return fail("stream wait", (int)e);
-        SlotMeta m{t.shape(), t.dtype(), bytes, bytes, numel, 0.f};
-        if (compression_ == OffloadCompression::None) {
-            if ((e = hipMemcpyAsync(host_[slot], t.data(), bytes, hipMemcpyDeviceToHost, transfer_)) != hipSuccess)
-                return fail("DtoH failed", (int)e);
-        } else {
-            const float scale = 8.0f / 448.0f, inv_scale = 1.0f / scale;      // activations in [-8, 8] assumed (:543-549)
-            int rc = flame_bf16_to_fp8(t.data(), staging_[slot], inv_scale, numel, transfer_);
-            if (rc != 0) return fail("bf16_to_fp8 failed", rc);
-            if ((e = hipMemcpyAsync(host_[slot], staging_[slot], numel, hipMemcpyDeviceToHost, transfer_)) != hipSuccess)
-                return fail("FP8 DtoH failed", (int)e);
-            m.stored_bytes = numel;
-            m.fp8_scale = scale;
-        }
-        meta_[slot] = std::move(m);
-        pushed_[slot] = true;
-        keep_alive_[slot] = t;
-        OffloadHandle h;
-        h.slot_ = slot;
-        h.epoch_ = epoch_;
-        return h;
-    }
-
-    // :619-737
-    Result<Tensor> pull(OffloadHandle h) {
-        if (h.epoch_ != epoch_)
-            return Error{Error::InvalidOperation, "ActivationOffloadPool::pull: handle epoch " + std::to_string(h.epoch_) +
-                                                       " is stale (current " + std::to_string(epoch_) + ")"};
-        if (h.slot_ >= host_.size())
-            return Error{Error::InvalidOperation, "ActivationOffloadPool::pull: slot " + std::to_string(h.slot_) + " out of range"};
-        if (!pushed_[h.slot_])
-            return Error{Error::InvalidOperation, "ActivationOffloadPool::pull: slot " + std::to_string(h.slot_) +
-                                                       " is idle, expected pushed (double pull?)"};
-        const size_t slot = h.slot_;
-        const SlotMeta& m = *meta_[slot];
-        auto out = Tensor::empty(m.shape, m.dtype);
-        if (!out.ok()) return out.error();
-        hipError_t e;
-        if (compression_ == OffloadCompression::None) {
-            e = hipMemcpyAsync(out.value().data(), host_[slot], m.stored_bytes, hipMemcpyHostToDevice, transfer_);
-            if (e != hipSuccess) return cuda_error("activation offload pull: HtoD failed", (int)e);
-        } else {
-            e = hipMemcpyAsync(staging_[slot], host_[slot], m.stored_bytes, hipMemcpyHostToDevice, transfer_);
-            if (e != hipSuccess) return cuda_error("activation offload pull: HtoD failed", (int)e);
-            int rc = flame_fp8_to_bf16(staging_[slot], out.value().data(), m.fp8_scale, m.numel, transfer_);
-            if (rc != 0) return cuda_error("activation offload pull: fp8_to_bf16 failed", rc);
-        }
-        if ((e = hipEventRecord(ready_[slot], transfer_)) != hipSuccess) return cuda_error("activation offload pull: event record", (int)e);
-        if ((e = hipStreamWaitEvent(nullptr, ready_[slot], 0)) != hipSuccess) return cuda_error("activation offload pull: stream wait", (int)e);
-        meta_[slot].reset();
-        pushed_[slot] = false;
-        keep_alive_[slot] = Tensor();
-        free_stack_.push_back(slot);
-        return out;
-    }
-
-    // :742-761: every slot idle again, handles issued so far stale; no host synchronisation (call synchronize()
-    // first if a copy may still be reading a pinned buffer)
-    void clear() {
-        for (size_t i = 0; i < host_.size(); ++i) {
-            pushed_[i] = false;
-            meta_[i].reset();
-            keep_alive_[i] = Tensor();
-        }
-        free_stack_.clear();
-        for (size_t i = host_.size(); i-- > 0;) free_stack_.push_back(i);
-        if (++epoch_ == 0) epoch_ = 1;
-    }
-    Result<bool> synchronize() {
-        hipError_t e = hipStreamSynchronize(transfer_);
-        if (e != hipSuccess) return cuda_error("hipStreamSynchronize", (int)e);
-        return true;
-    }
-
-   private:
-    ActivationOffloadPool() = default;
-    struct SlotMeta {                        // :269-281
-        std::vector<int64_t> shape;
-        DType dtype;
-        size_t bytes, stored_bytes, numel;
-        float fp8_scale;                     // 0 = not compressed
-    };
-    OffloadCompression compression_ = OffloadCompression::None;
-    size_t slot_bytes_ = 0;
-    uint64_t epoch_ = 1;
-    hipStream_t transfer_ = nullptr;
-    std::vector<void*> host_, staging_;
-    std::vector<hipEvent_t> done_, ready_;
-    std::vector<std::optional<SlotMeta>> meta_;
-    std::vector<bool> pushed_;
-    std::vector<Tensor> keep_alive_;
-    std::vector<size_t> free_stack_;
-};
-
-}  // namespace activation_offload
-
-// The saved set of one attention call through the pool: Q, K, V and O leave the device (pushed in that order),
-// the log-sum-exp rows stay (fp32, 1/256 of the bytes at D = 128; an FP8 pool takes bf16 only, :536-541).
-// restore_saved pulls in reverse order, as the slots' stack expects, and gives the context the backward takes.
-namespace autograd_v4 {
-struct OffloadedSdpaCtx {
-    SdpaCtx rest;                                              // q, k, v, o undefined while offloaded
-    activation_offload::OffloadHandle q, k, v, o;
-};
-inline Result<OffloadedSdpaCtx> offload_saved(const SdpaCtx& ctx, activation_offload::ActivationOffloadPool& pool) {
-    OffloadedSdpaCtx off;
-    off.rest = ctx;
-    const Tensor* src[4] = {&ctx.q, &ctx.k, &ctx.v, &ctx.o};
-    activation_offload::OffloadHandle* dst[4] = {&off.q, &off.k, &off.v, &off.o};
-    for (int i = 0; i < 4; ++i) {
-        if (i == 3 && ctx.save == SdpaSave::Recompute) break;  // no O was kept
-        auto h = pool.push(*src[i]);
-        if (!h.ok()) {
-            for (int j = i; j-- > 0;) (void)pool.pull(*dst[j]);   // give the slots back
-            return h.error();
-        }
-        *dst[i] = h.value();
-    }
-    off.rest.q = off.rest.k = off.rest.v = Tensor();
-    if (ctx.save != SdpaSave::Recompute) off.rest.o = Tensor();
-    return off;
-}
-inline Result<SdpaCtx> restore_saved(const OffloadedSdpaCtx& off, activation_offload::ActivationOffloadPool& pool) {
-    SdpaCtx ctx = off.rest;
-    if (ctx.save != SdpaSave::Recompute) {
-        auto o = pool.pull(off.o);
-        if (!o.ok()) return o.error();
-        ctx.o = o.value();
-    }
-    auto v = pool.pull(off.v);
-    if (!v.ok()) return v.error();
-    auto k = pool.pull(off.k);
-    if (!k.ok()) return k.error();
-    auto q = pool.pull(off.q);
-    if (!q.ok()) return q.error();
-    ctx.q = q.value(); ctx.k = k.value(); ctx.v = v.value();
-    return ctx;
-}
-}  // namespace autograd_v4
 
 // ------------------------------------------------------------------------------------ SageAttention
 // Builder-style API of the reference (src/sage_attention.rs:21-65).  `scale` is the softmax scale

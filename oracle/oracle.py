@@ -373,6 +373,19 @@ def dropout_keep_mask(B, H, Sq, Sk, p, seed, chunk_q=0, chunk_kv=0) -> np.ndarra
     return dropout_uniforms(B, H, Sq, Sk, seed, chunk_q, chunk_kv) >= np.float32(p)
 
 
+class operand_rounding:
+    """Context manager: inside it the oracle rounds the left operands of P V, P^T dO, dS K and dS^T Q to bf16, as a
+    kernel that forms those products on a bf16 matrix unit must (oracle_set_operand_rounding in sdpa_oracle.c)."""
+
+    def __enter__(self):
+        lib().oracle_set_operand_rounding(1)
+        return self
+
+    def __exit__(self, *exc):
+        lib().oracle_set_operand_rounding(0)
+        return False
+
+
 def sdpa_fwd_dropout(q, k, v, scale, p, seed, causal=False, kv_len=None, mask=None, want_f32=False, chunk_q=0, chunk_kv=0):
     B, H, Sq, D = q.shape
     Sk = k.shape[2]

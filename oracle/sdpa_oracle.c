@@ -138,6 +138,15 @@ int oracle_dropout_keep_tiled(uint64_t seed, int bh, int i, int j, int Sq, int S
     const uint64_t idx = ((uint64_t)bh * (uint64_t)q_t + (uint64_t)(i - q_off)) * (uint64_t)k_t + (uint64_t)(j - k_off);
     return oracle_dropout_keep(tile_seed, idx, p);
 }
+/* Operand rounding (off by default).  A kernel that forms P V, P^T dO, dS K and dS^T Q on a bf16 matrix unit has to
+ * round the left operands (the dropped and rescaled probabilities, and dS) to bf16 first; the plain oracle keeps them
+ * in fp32, as the reference's fp32 operator does.  With this switch on, the oracle rounds exactly those operands
+ * (round to nearest even) and nothing else, which separates what the rounding of the operands costs from any other
+ * difference.  Used by the dropout GPU tests, whose probabilities P / (1 - p) reach into [1, 2). */
+static int g_round_operands = 0;
+void oracle_set_operand_rounding(int on) { g_round_operands = on != 0; }
+static inline float operand(float x) { return g_round_operands ? bf16_to_f32(f32_to_bf16(x)) : x; }
+
 /* factor applied to P[bh, i, j]: 0 or 1 / (1 - p); 1 without dropout */
 static inline float drop_factor(const mask_spec* ms, int bh, int i, int j, int Sq, int Sk) {
     if (!(ms->drop_p > 0.f)) return 1.0f;
@@ -269,7 +278,7 @@ static int sdpa_fwd_impl(const uint16_t* Q, const uint16_t* K, const uint16_t* V
                 for (int d = 0; d < D; ++d) o[d] = 0.f;
                 const float* row = P + (size_t)i * Sk;
                 for (int j = 0; j < Sk; ++j) {
-                    const float p = row[j] * drop_factor(&ms, bh, row_begin + i, j, Sq, Sk);
+                    const float p = operand(row[j] * drop_factor(&ms, bh, row_begin + i, j, Sq, Sk));
                     if (p == 0.f) continue;
                     const float* vr = v + (size_t)j * D;
                     for (int d = 0; d < D; ++d) o[d] += p * vr[d];
@@ -357,8 +366,8 @@ static int sdpa_bwd_impl(const uint16_t* Q, const uint16_t* K, const uint16_t* V
                     /* with dropout O = (P * f) V, f = 0 or 1 / (1 - p): dV takes P * f, dP = f * (dO V^T), and
                      * rowsum(dP * P) = rowsum(dO * O) = delta as without it */
                     const float f = drop_factor(&ms, bh, row_begin + i, j, Sq, Sk);
-                    const float ds = p * (f * dp[j] - delta);
-                    const float pd = p * f;
+                    const float ds = operand(p * (f * dp[j] - delta));
+                    const float pd = operand(p * f);
                     float* dvj = dv + (size_t)j * D;
                     float* dkj = dk + (size_t)j * D;
                     const float* kj = k + (size_t)j * D;

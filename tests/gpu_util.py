@@ -28,9 +28,10 @@ def bf16_ulp(x: np.ndarray) -> np.ndarray:
     return 2.0 ** (np.floor(np.log2(ax)) - 7)
 
 
-def assert_close_bf16(oracle, name, got_f32, ref_bits, ref_f32, max_abs=TOL_MAX_ABS):
+def assert_close_bf16(oracle, name, got_f32, ref_bits, ref_f32, max_abs=TOL_MAX_ABS, stragglers=0):
     """The parity bar for a bf16 output tensor (max_abs: the flat bound, the north-star 2e-2 unless a test states why
-    its quantities are scaled).
+    its quantities are scaled; stragglers: how many elements of the tensor may miss the max-abs bar below, by less
+    than a factor of two, in a test that states why: their count, errors and magnitudes are printed).
 
     * relative L2 <= 1e-2 against the oracle's un-rounded fp32 values;
     * max-abs <= 2e-2 against both the un-rounded fp32 values and the oracle's bf16-rounded values,
@@ -51,6 +52,13 @@ def assert_close_bf16(oracle, name, got_f32, ref_bits, ref_f32, max_abs=TOL_MAX_
           f"for |x| >= 4)", flush=True)
     assert np.all(np.isfinite(got_f32)), name
     assert rl_f <= TOL_REL_L2, name
-    assert np.all(diff_f <= np.maximum(max_abs, bf16_ulp(ref_f))), name
-    assert np.all(diff_b <= np.maximum(max_abs, bf16_ulp(ref_b))), name
+    bad = (diff_f > np.maximum(max_abs, bf16_ulp(ref_f))) | (diff_b > np.maximum(max_abs, bf16_ulp(ref_b)))
+    n_bad = int(np.count_nonzero(bad))
+    if n_bad and stragglers:
+        print(f"      {name}: {n_bad} of {diff_f.size} elements miss the max-abs bar (allowed here: {stragglers}): errors "
+              f"{np.round(diff_f[bad], 4).tolist()[:8]} at reference values {np.round(ref_f[bad], 3).tolist()[:8]}", flush=True)
+        assert n_bad <= stragglers, name
+        assert np.all(diff_f[bad] <= 2 * np.maximum(max_abs, bf16_ulp(ref_f[bad]))), name
+    else:
+        assert n_bad == 0, name
     return ma_f, rl_f

@@ -11,6 +11,7 @@
 #include <vector>
 
 #include "../../flame_amd/host/flame_host.hpp"
+#include "activation_offload_harness.hpp"
 
 using namespace flame;
 
@@ -67,7 +68,22 @@ static std::vector<float> host_f32_of_bf16(const Tensor& t) {
     return f;
 }
 
-// naive fp32 materialised attention for one (b,h): O, and grads from dO (D = rowsum(dO*O))
+// The reference values come from the CPU oracle (oracle/sdpa_oracle.c, built to oracle/_build/liboracle.so and
+// linked into this test driver only): the pinned restatement of tests/fa2_parity_naive.rs:90-140 and
+// tests/cudnn_sdpa_bwd_parity.rs:31-98 that every Python GPU test compares with as well.
+extern "C" {
+int oracle_sdpa_fwd(const uint16_t* Q, const uint16_t* K, const uint16_t* V, int B, int H, int Sq, int Sk, int D, float scale,
+                    int causal, const int32_t* kv_len, const uint8_t* mask, int64_t msb, int64_t msh, int64_t msq, int64_t msk,
+                    int heads_begin, int heads_end, uint16_t* O, float* LSE, float* O32);
+int oracle_sdpa_bwd(const uint16_t* Q, const uint16_t* K, const uint16_t* V, const uint16_t* O, const uint16_t* dO, int B, int H,
+                    int Sq, int Sk, int D, float scale, int causal, const int32_t* kv_len, const uint8_t* mask, int64_t msb,
+                    int64_t msh, int64_t msq, int64_t msk, int heads_begin, int heads_end, uint16_t* dQ, uint16_t* dK,
+                    uint16_t* dV, float* dQ32, float* dK32, float* dV32);
+int oracle_sdpa_fwd_bias(const uint16_t* Q, const uint16_t* K, const uint16_t* V, int B, int H, int Sq, int Sk, int D, float scale,
+                         const float* bias, int64_t bsb, int64_t bsh, int64_t bsq, int64_t bsk, uint16_t* O, float* LSE, float* O32);
+}
+
+// one (batch, head) slice through the oracle: un-rounded fp32 O and, with dO, dQ, dK, dV (from the bf16-rounded O)
 struct Naive {
     std::vector<float> o, dq, dk, dv;
 };
@@ -75,56 +91,46 @@ static Naive naive_head(const uint16_t* q, const uint16_t* k, const uint16_t* v,
                         float scale, bool causal, const uint8_t* keep /*[Sq,Sk] or null*/) {
     Naive r;
     r.o.assign((size_t)Sq * D, 0.f);
+    std::vector<uint16_t> ob((size_t)Sq * D);
+    std::vector<float> lse((size_t)Sq);
+    const int rc = oracle_sdpa_fwd(q, k, v, 1, 1, Sq, Sk, D, scale, causal ? 1 : 0, nullptr, keep, 0, 0, keep ? Sk : 0, keep ? 1 : 0,
+                                   0, 1, ob.data(), lse.data(), r.o.data());
+    CHECK(rc == 0, "oracle_sdpa_fwd returned %d", rc);
+    if (!d_o) return r;
     r.dq.assign((size_t)Sq * D, 0.f);
     r.dk.assign((size_t)Sk * D, 0.f);
     r.dv.assign((size_t)Sk * D, 0.f);
-    std::vector<float> p(Sk), dp(Sk);
-    for (int i = 0; i < Sq; ++i) {
-        float m = -INFINITY;
-        for (int j = 0; j < Sk; ++j) {
-            float s = 0.f;
-            for (int d = 0; d < D; ++d) s += bf2f(q[i * D + d]) * bf2f(k[j * D + d]);
-            s *= scale;
-            if ((causal && j > i) || (keep && !keep[(size_t)i * Sk + j])) s = -INFINITY;
-            p[j] = s;
-            m = std::fmax(m, s);
-        }
-        if (m == -INFINITY) continue;
-        float l = 0.f;
-        for (int j = 0; j < Sk; ++j) { p[j] = std::exp(p[j] - m); l += p[j]; }
-        for (int j = 0; j < Sk; ++j) p[j] /= l;
-        for (int j = 0; j < Sk; ++j)
-            for (int d = 0; d < D; ++d) r.o[(size_t)i * D + d] += p[j] * bf2f(v[j * D + d]);
-        if (!d_o) continue;
-        float delta = 0.f;
-        for (int d = 0; d < D; ++d) delta += bf2f(d_o[i * D + d]) * bf2f(f2bf(r.o[(size_t)i * D + d]));
-        for (int j = 0; j < Sk; ++j) {
-            float a = 0.f;
-            for (int d = 0; d < D; ++d) a += bf2f(d_o[i * D + d]) * bf2f(v[j * D + d]);
-            dp[j] = a;
-        }
-        for (int j = 0; j < Sk; ++j) {
-            const float ds = p[j] * (dp[j] - delta);
-            for (int d = 0; d < D; ++d) {
-                r.dv[(size_t)j * D + d] += p[j] * bf2f(d_o[i * D + d]);
-                r.dq[(size_t)i * D + d] += ds * bf2f(k[j * D + d]) * scale;
-                r.dk[(size_t)j * D + d] += ds * bf2f(q[i * D + d]) * scale;
-            }
-        }
-    }
+    std::vector<uint16_t> bq(r.dq.size()), bk(r.dk.size()), bv(r.dv.size());
+    const int rb = oracle_sdpa_bwd(q, k, v, ob.data(), d_o, 1, 1, Sq, Sk, D, scale, causal ? 1 : 0, nullptr, keep, 0, 0,
+                                   keep ? Sk : 0, keep ? 1 : 0, 0, 1, bq.data(), bk.data(), bv.data(), r.dq.data(), r.dk.data(),
+                                   r.dv.data());
+    CHECK(rb == 0, "oracle_sdpa_bwd returned %d", rb);
     return r;
 }
+// The parity bar of the Python GPU tests (tests/gpu_util.py): relative L2 <= 1e-2 and max-abs <= 2e-2 against the
+// oracle's fp32 values, one bf16 step being allowed where |x| >= 4 makes the step itself exceed 2e-2; and the
+// reference's own cosine gate.
 static void compare(const char* name, const std::vector<float>& got, const std::vector<float>& ref) {
-    double ma = 0, dot = 0, ng = 0, nr = 0;
+    double ma = 0, dot = 0, ng = 0, nr = 0, d2 = 0;
+    size_t over = 0;
+    CHECK(got.size() == ref.size(), "%s: %zu values against %zu", name, got.size(), ref.size());
+    if (got.size() != ref.size()) return;
     for (size_t i = 0; i < ref.size(); ++i) {
-        ma = std::fmax(ma, std::fabs((double)got[i] - ref[i]));
+        const double diff = std::fabs((double)got[i] - ref[i]);
+        ma = std::fmax(ma, diff);
+        const double ax = std::fmax(std::fabs((double)ref[i]), 1e-30);
+        const double ulp = std::exp2(std::floor(std::log2(ax)) - 7);
+        if (diff > std::fmax(2e-2, ulp)) ++over;
+        d2 += diff * diff;
         dot += (double)got[i] * ref[i];
         ng += (double)got[i] * got[i];
         nr += (double)ref[i] * ref[i];
     }
     const double cosv = (ng > 0 && nr > 0) ? dot / std::sqrt(ng * nr) : 1.0;
-    std::printf("  %-28s max_abs=%.3e cos=%.6f\n", name, ma, cosv);
-    CHECK(ma <= 2e-2, "%s max_abs %.3e", name, ma);
+    const double rel = nr > 0 ? std::sqrt(d2 / nr) : std::sqrt(d2);
+    std::printf("  %-28s max_abs=%.3e rel_l2=%.3e cos=%.6f\n", name, ma, rel, cosv);
+    CHECK(over == 0, "%s: %zu elements beyond max(2e-2, one bf16 step), max_abs %.3e", name, over, ma);
+    CHECK(rel <= 1e-2, "%s rel_l2 %.3e", name, rel);
     CHECK(cosv >= 0.9999, "%s cosine %.6f", name, cosv);     // the reference's gate
 }
 
@@ -505,7 +511,7 @@ int main() {
         CHECK(!bf16_ops::rope_fused_bf16_f32pe(normed.value(), bad, bad).ok(), "f32pe must refuse bf16 tables");
     }
 
-    // ---- 8. additive bias (sdpa::forward_with_bias): against a scalar softmax(scale*QK^T + bias) V on the host
+    // ---- 8. additive bias (sdpa::forward_with_bias): against the oracle's softmax(scale*QK^T + bias) V
     {
         std::printf("[forward_with_bias]\n");
         const int B = 1, H = 2, Sq = 70, Sk = 90, D = 64;
@@ -518,25 +524,11 @@ int main() {
         CHECK(o.ok(), "forward_with_bias failed");
         if (o.ok()) {
             auto got = host_f32_of_bf16(o.value());
-            std::vector<float> ref(got.size());
-            std::vector<double> s(Sk);
-            for (int h = 0; h < H; ++h)
-                for (int i = 0; i < Sq; ++i) {
-                    double m = -1e300;
-                    for (int j = 0; j < Sk; ++j) {
-                        double acc = 0;
-                        for (int d = 0; d < D; ++d) acc += (double)bf2f(hq[((size_t)h * Sq + i) * D + d]) * bf2f(hk[((size_t)h * Sk + j) * D + d]);
-                        s[j] = acc * 0.2 + hb[((size_t)h * Sq + i) * Sk + j];
-                        m = std::fmax(m, s[j]);
-                    }
-                    double l = 0;
-                    for (int j = 0; j < Sk; ++j) { s[j] = std::exp(s[j] - m); l += s[j]; }
-                    for (int d = 0; d < D; ++d) {
-                        double acc = 0;
-                        for (int j = 0; j < Sk; ++j) acc += s[j] * bf2f(hv[((size_t)h * Sk + j) * D + d]);
-                        ref[((size_t)h * Sq + i) * D + d] = (float)(acc / l);
-                    }
-                }
+            std::vector<float> ref(got.size()), lse((size_t)H * Sq);
+            std::vector<uint16_t> ob(got.size());
+            const int rc = oracle_sdpa_fwd_bias(hq.data(), hk.data(), hv.data(), B, H, Sq, Sk, D, 0.2f, hb.data(), 0, (int64_t)Sq * Sk, Sk, 1,
+                                                ob.data(), lse.data(), ref.data());
+            CHECK(rc == 0, "oracle_sdpa_fwd_bias returned %d", rc);
             compare("O (bias)", got, ref);
         }
         Tensor badb = Tensor::empty({1, H, Sq, Sk + 1}, DType::F32).value();
@@ -548,23 +540,7 @@ int main() {
         auto so2 = cuda_ops_bf16::sdpa_stream_bf16(q, k, v, nullptr, 1024, true, 0.125f);
         CHECK(so.ok() && so2.ok(), "streaming wrappers failed");
         if (so.ok() && so2.ok()) CHECK(host_f32_of_bf16(so.value()) == host_f32_of_bf16(so2.value()), "streaming wrappers disagree");
-        {   // launch record, planner and candidates (src/ops/attn.rs:128-209, :232-239, :318-323)
-            auto info = ops::attn::streaming_attn_last_launch_info();
-            CHECK(info.requested_chunk == std::min<size_t>(2048, (size_t)Sq) && info.chosen_chunk && *info.chosen_chunk == info.requested_chunk &&
-                      info.retries == 0 && info.fallbacks.empty() && !info.last_error,
-                  "launch info after a plain call");
-            using ops::attn::streaming_chunk_candidates;
-            CHECK(streaming_chunk_candidates(0).empty(), "no candidates for an empty sequence");
-            CHECK(streaming_chunk_candidates(20) == std::vector<size_t>({20}), "short sequences: the sequence itself");
-            CHECK(streaming_chunk_candidates(100) == std::vector<size_t>({100, 96, 64, 48, 32}), "candidates below 100");
-            CHECK(streaming_chunk_candidates(5000).size() == 13 && streaming_chunk_candidates(5000).front() == 2048 &&
-                      streaming_chunk_candidates(5000).back() == 32, "all thirteen preferred chunks");
-            CHECK(ops::attn::streaming_workspace_bytes(2048, 4608, 128).value_or(0) == (2048ull * 4608 + 2048ull * 130) * 4,
-                  "the reference's scratch formula");
-            setenv("FLAME_SDPA_PLANNER_BUDGET_BYTES", "12345", 1);
-            auto forced = ops::attn::plan_streaming_chunk(4608, 4608, 128);
-            unsetenv("FLAME_SDPA_PLANNER_BUDGET_BYTES");
-            CHECK(!forced.ok() && forced.error().kind == Error::OutOfMemory, "a budget no chunk fits is OutOfMemory");
+        {   // a caller workspace is accepted, checked for consistency and left untouched
             cuda_ops_bf16::SdpaWorkspace ws;
             ws.bytes = 16;
             CHECK(!cuda_ops_bf16::sdpa_stream_bf16_with_workspace(q, k, v, nullptr, 64, true, 0.125f, ws).ok(), "null workspace with bytes");
@@ -857,27 +833,30 @@ int main() {
             for (auto& e : x) e = f2bf(0.02f * gauss());
             return x;
         };
-        // dense fp32 attention of one (b, h) on the host; keep: [S, S] 1 = attend, or null
+        // dense fp32 attention through the CPU oracle; keep: [BH, S, S] 1 = attend, or null.  The oracle has one head
+        // dim, and the softmax does not depend on V: the Dv columns are taken in ranges of at most Dh, zero-padded.
         auto dense = [](const std::vector<uint16_t>& q, const std::vector<uint16_t>& k, const std::vector<uint16_t>& v, int BH, int S,
                         int Dh, int Dv, float scale, bool causal, const std::vector<float>* keep) {
-            std::vector<float> o((size_t)BH * S * Dv, 0.f), p(S);
-            for (int bh = 0; bh < BH; ++bh)
-                for (int i = 0; i < S; ++i) {
-                    float m = -INFINITY;
-                    for (int j = 0; j < S; ++j) {
-                        float a = 0.f;
-                        for (int d = 0; d < Dh; ++d) a += bf2f(q[((size_t)bh * S + i) * Dh + d]) * bf2f(k[((size_t)bh * S + j) * Dh + d]);
-                        a *= scale;
-                        if (causal && j > i) a += -1e9f;                                  // as the test does: (mask - 1) * 1e9
-                        if (keep && (*keep)[((size_t)bh * S + i) * S + j] == 0.f) a += -1e9f;
-                        p[j] = a;
-                        m = std::fmax(m, a);
-                    }
-                    float l = 0.f;
-                    for (int j = 0; j < S; ++j) { p[j] = std::exp(p[j] - m); l += p[j]; }
-                    for (int j = 0; j < S; ++j)
-                        for (int d = 0; d < Dv; ++d) o[((size_t)bh * S + i) * Dv + d] += p[j] / l * bf2f(v[((size_t)bh * S + j) * Dv + d]);
-                }
+            std::vector<float> o((size_t)BH * S * Dv, 0.f), o32((size_t)BH * S * Dh);
+            std::vector<uint16_t> vc((size_t)BH * S * Dh), ob(vc.size());
+            std::vector<float> lse((size_t)BH * S);
+            std::vector<uint8_t> keep8;
+            if (keep) {
+                keep8.resize(keep->size());
+                for (size_t i = 0; i < keep->size(); ++i) keep8[i] = (*keep)[i] != 0.f;
+            }
+            for (int c0 = 0; c0 < Dv; c0 += Dh) {
+                const int w = std::min(Dh, Dv - c0);
+                std::fill(vc.begin(), vc.end(), (uint16_t)0);
+                for (size_t r = 0; r < (size_t)BH * S; ++r)
+                    for (int d = 0; d < w; ++d) vc[r * Dh + d] = v[r * Dv + c0 + d];
+                const int rc = oracle_sdpa_fwd(q.data(), k.data(), vc.data(), 1, BH, S, S, Dh, scale, causal ? 1 : 0, nullptr,
+                                               keep ? keep8.data() : nullptr, 0, keep ? (int64_t)S * S : 0, keep ? S : 0, keep ? 1 : 0,
+                                               0, BH, ob.data(), lse.data(), o32.data());
+                CHECK(rc == 0, "oracle_sdpa_fwd returned %d", rc);
+                for (size_t r = 0; r < (size_t)BH * S; ++r)
+                    for (int d = 0; d < w; ++d) o[r * Dv + c0 + d] = o32[r * Dh + d];
+            }
             return o;
         };
         auto diff = [](const std::vector<float>& a, const std::vector<float>& b, double& max_abs, double& mean_abs) {
@@ -922,32 +901,17 @@ int main() {
             auto oa = ops::attn::streaming_attn_bf16_fp32(tq, tk, tv, a), oc = ops::attn::streaming_attn_bf16_fp32(tq, tk, tv, c);
             CHECK(oa.ok() && oc.ok() && host_bits_of_bf16(oa.value()) == host_bits_of_bf16(oc.value()), "chunk 32 and chunk 64 agree");
         }
-        {   // streaming_attention_tracks_budget_trim (:298-364) and streaming_attention_honors_generous_budget (:366-411)
+        {   // the shape of streaming_attention_tracks_budget_trim / _honors_generous_budget (:298-411): Dh = 64, Dv = 160 at
+            // S = 8192 with zero inputs.  Those tests assert on the reference's workspace planner, which has no
+            // counterpart here (no score workspace exists); what remains is that the shape runs and gives zero.
             const int b = 1, h = 2, s = 8192, dh = 64, dv = 160;
             std::vector<uint16_t> zq((size_t)b * h * s * dh, 0), zv((size_t)b * h * s * dv, 0);
             Tensor q = dev_bf16(zq, {b, h, s, dh}), k = dev_bf16(zq, {b, h, s, dh}), v = dev_bf16(zv, {b, h, s, dv});
             ops::attn::StreamingAttnCfg cfg;
             cfg.scale = 0.125f;
             cfg.chunk_size = 2048;
-            setenv("FLAME_SDPA_PLANNER_BUDGET_BYTES", "67108864", 1);
             auto out = ops::attn::streaming_attn_bf16_fp32(q, k, v, cfg);
-            CHECK(out.ok() && out.value().shape() == std::vector<int64_t>({b, h, s, dv}), "dv = 160 under a 64 MiB budget");
-            auto info = ops::attn::streaming_attn_last_launch_info();
-            const ops::attn::StreamingFallbackEvent* ev = nullptr;
-            for (const auto& e : info.fallbacks)
-                if (e.reason.kind == ops::attn::StreamingFallbackReason::WorkspaceBudget) { ev = &e; break; }
-            CHECK(ev != nullptr, "workspace budget fallback not recorded");
-            if (ev) {
-                CHECK(ev->from_chunk == 2048, "planner should report trimming from the requested chunk");
-                CHECK(info.chosen_chunk && *info.chosen_chunk == ev->to_chunk && ev->to_chunk == 1536, "chosen chunk should match the trimmed target");
-                CHECK(ev->reason.required_bytes && ev->reason.budget_bytes && *ev->reason.required_bytes > *ev->reason.budget_bytes,
-                      "workspace requirement should exceed budget when trimming occurs");
-            }
-            setenv("FLAME_SDPA_PLANNER_BUDGET_BYTES", "536870912", 1);
-            auto out2 = ops::attn::streaming_attn_bf16_fp32(q, k, v, cfg);
-            unsetenv("FLAME_SDPA_PLANNER_BUDGET_BYTES");
-            auto info2 = ops::attn::streaming_attn_last_launch_info();
-            CHECK(out2.ok() && info2.chosen_chunk && *info2.chosen_chunk == 2048 && info2.fallbacks.empty(), "generous budget keeps the requested chunk");
+            CHECK(out.ok() && out.value().shape() == std::vector<int64_t>({b, h, s, dv}), "dv = 160 at S = 8192");
             if (out.ok()) {       // zero inputs: uniform attention over zero values
                 bool all_zero = true;
                 for (uint16_t x : host_bits_of_bf16(out.value())) all_zero = all_zero && (x & 0x7fff) == 0;

@@ -12,10 +12,25 @@ from tests.gpu_util import TOL_LSE, TOL_MAX_ABS, assert_close_bf16, to_dev, to_f
 pytestmark = pytest.mark.gpu
 
 SEED = 0x2545F4914F6CDD1D
-# The kept probabilities are P / (1 - p): where P is near 1 (rows with few attended keys) they reach into [1, 2), whose
-# bf16 spacing is twice that of [0.5, 1), and the bf16 operands of the PV, dV and dS products carry twice the rounding
-# error they have without dropout.  The flat max-abs bound is doubled accordingly; the relative-L2 bound is not.
-DROPOUT_MAX_ABS = 2 * TOL_MAX_ABS
+# The bar is the one of every other test: relative L2 1e-2 and the flat max-abs 2e-2 (one bf16 step where |x| >= 4).
+# The backward is checked twice.  On the oracle's own O and log-sum-exp (identical inputs on both sides) it is held to
+# that bar without exception.  Chained behind the library's forward, its delta = rowsum(dO * O) is formed from an O
+# that differs from the oracle's by a bf16 step in places (a legitimate difference of two roundings), and with
+# dropout O is large where a row attends few keys: a step of 2^-6 in O, summed over the head dim, moves delta by
+# several hundredths and the gradients of those rows with it.  There, at most a fraction STRAGGLERS of a tensor's
+# elements may miss the max-abs bar, by less than a factor of two; their errors and magnitudes are printed.
+DROPOUT_MAX_ABS = TOL_MAX_ABS
+STRAGGLERS = 1e-4
+
+
+def _allowed(t):
+    return max(1, int(STRAGGLERS * t.numel()))
+
+
+def _check_grads(oracle, tag, g, ref, strict):
+    for i, (name, got) in enumerate((("dQ", g[0]), ("dK", g[1]), ("dV", g[2]))):
+        assert_close_bf16(oracle, f"{name} ({tag})", to_f32(got), ref[i], ref[i + 3], max_abs=DROPOUT_MAX_ABS,
+                          stragglers=0 if strict else _allowed(got))
 
 
 def _inputs(tag, B, H, Sq, Sk, D):
@@ -54,11 +69,20 @@ def test_dropout_forward_and_backward_against_oracle(oracle, B, H, Sq, Sk, D, ca
     assert oracle.max_abs(lse.cpu().numpy().reshape(rlse.shape), rlse) <= TOL_LSE
     assert torch.equal(lse, lse_plain) or float((lse - lse_plain).abs().max()) <= 1e-6      # the undropped softmax's
     assert not torch.equal(o, o_plain)
+    ref = oracle.sdpa_bwd_dropout(q, k, v, ro, do, scale, p, SEED, causal=causal, kv_len=kvl_np, want_f32=True)
+    lse_ref = torch.from_numpy(rlse.reshape(B * H, Sq)).cuda()
+    g_same = capi.attn_bwd_dropout(dq_, dk_, dv_, to_dev(ro), ddo, lse_ref, scale, p, SEED, causal=causal, kv_len=kvl)
     g = capi.attn_bwd_dropout(dq_, dk_, dv_, o, ddo, lse, scale, p, SEED, causal=causal, kv_len=kvl)
     torch.cuda.synchronize()
-    ref = oracle.sdpa_bwd_dropout(q, k, v, ro, do, scale, p, SEED, causal=causal, kv_len=kvl_np, want_f32=True)
-    for i, (name, got) in enumerate((("dQ", g[0]), ("dK", g[1]), ("dV", g[2]))):
-        assert_close_bf16(oracle, name, to_f32(got), ref[i], ref[i + 3], max_abs=tol)
+    _check_grads(oracle, "on the oracle's O and LSE", g_same, ref, strict=True)
+    _check_grads(oracle, "behind the library's forward", g, ref, strict=False)
+    # the same against the oracle that rounds P f and dS to bf16 before the four products that take them, as the
+    # kernels must
+    with oracle.operand_rounding():
+        ro_r, _, ro32_r = oracle.sdpa_fwd_dropout(q, k, v, scale, p, SEED, causal=causal, kv_len=kvl_np, want_f32=True)
+        ref_r = oracle.sdpa_bwd_dropout(q, k, v, ro, do, scale, p, SEED, causal=causal, kv_len=kvl_np, want_f32=True)
+    assert_close_bf16(oracle, "O (operands rounded)", to_f32(o), ro_r, ro32_r, max_abs=tol)
+    _check_grads(oracle, "operands rounded, on the oracle's O and LSE", g_same, ref_r, strict=True)
     # teeth: the plain forward, rescaled or not, is far from this oracle
     assert oracle.rel_l2(to_f32(o_plain), ro32) > 0.05 and oracle.rel_l2(to_f32(o_plain) / (1 - p), ro32) > 0.05
 
@@ -79,13 +103,15 @@ def test_dropout_with_a_keep_mask(oracle, B, H, Sq, Sk, D, causal, per_head):
     dq_, dk_, dv_, ddo = (to_dev(t) for t in (q, k, v, do))
     o, lse = capi.attn_fwd_dropout(dq_, dk_, dv_, scale, p, SEED, causal=causal, mask=mask)
     g = capi.attn_bwd_dropout(dq_, dk_, dv_, o, ddo, lse, scale, p, SEED, causal=causal, mask=mask)
-    torch.cuda.synchronize()
     ro, rlse, ro32 = oracle.sdpa_fwd_dropout(q, k, v, scale, p, SEED, causal=causal, mask=keep, want_f32=True)
+    lse_ref = torch.from_numpy(rlse.reshape(B * H, Sq)).cuda()
+    g_same = capi.attn_bwd_dropout(dq_, dk_, dv_, to_dev(ro), ddo, lse_ref, scale, p, SEED, causal=causal, mask=mask)
+    torch.cuda.synchronize()
     assert_close_bf16(oracle, "O", to_f32(o), ro, ro32, max_abs=tol)
     assert oracle.max_abs(lse.cpu().numpy().reshape(rlse.shape), rlse) <= TOL_LSE
     ref = oracle.sdpa_bwd_dropout(q, k, v, ro, do, scale, p, SEED, causal=causal, mask=keep, want_f32=True)
-    for i, (name, got) in enumerate((("dQ", g[0]), ("dK", g[1]), ("dV", g[2]))):
-        assert_close_bf16(oracle, name, to_f32(got), ref[i], ref[i + 3], max_abs=tol)
+    _check_grads(oracle, "on the oracle's O and LSE", g_same, ref, strict=True)
+    _check_grads(oracle, "behind the library's forward", g, ref, strict=False)
 
 
 def test_dropout_kept_set_bit_exact_through_a_one_hot_value_matrix(oracle):
@@ -141,8 +167,11 @@ def test_chunked_draw_forward_and_backward_against_oracle(oracle, B, H, Sq, Sk, 
     assert_close_bf16(oracle, "O", to_f32(o), ro, ro32, max_abs=DROPOUT_MAX_ABS)
     assert oracle.max_abs(lse.cpu().numpy().reshape(rlse.shape), rlse) <= TOL_LSE
     ref = oracle.sdpa_bwd_dropout(q, k, v, ro, do, scale, p, SEED, causal=causal, want_f32=True, chunk_q=cq, chunk_kv=ck)
-    for i, (name, got) in enumerate((("dQ", g[0]), ("dK", g[1]), ("dV", g[2]))):
-        assert_close_bf16(oracle, name, to_f32(got), ref[i], ref[i + 3], max_abs=DROPOUT_MAX_ABS)
+    lse_ref = torch.from_numpy(rlse.reshape(B * H, Sq)).cuda()
+    g_same = capi.attn_bwd_dropout(dq_, dk_, dv_, to_dev(ro), ddo, lse_ref, scale, p, SEED, causal=causal, draw_chunk_q=cq, draw_chunk_kv=ck)
+    torch.cuda.synchronize()
+    _check_grads(oracle, "on the oracle's O and LSE", g_same, ref, strict=True)
+    _check_grads(oracle, "behind the library's forward", g, ref, strict=False)
     # teeth: the unchunked kept set gives another output
     ro_flat, _ = oracle.sdpa_fwd_dropout(q, k, v, scale, p, SEED, causal=causal)
     assert oracle.rel_l2(to_f32(o), oracle.bf16_to_f32(ro_flat)) > 0.05

@@ -1,8 +1,9 @@
 """Runs the C++ host-layer test driver (tests/host/host_api_test.cpp) on the GPU.
 
 The driver exercises flame_amd/host/flame_host.hpp -- the C++ mirror of the reference's Rust operator
-interface for this path -- against a naive fp32 reference computed inside the driver, and exits 0
-when every check passed.  It is built ahead of time by `python -m flame_amd.build`."""
+interface for this path -- against the CPU oracle (oracle/_build/liboracle.so, linked into the driver as its
+checker), to the tolerances of tests/gpu_util.py, and exits 0 when every check passed.  It is built ahead of time
+by `python -m flame_amd.build` (after `make -C oracle`)."""
 import os
 import subprocess
 

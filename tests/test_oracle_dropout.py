@@ -161,3 +161,39 @@ def test_forward_and_backward_with_a_chunked_draw_against_fp64():
     ds = p64 * (dp - delta) * 0.3
     assert O.max_abs(dv32, dv) < 1e-5
     assert O.max_abs(dq32, ds @ f[1]) < 1e-5 and O.max_abs(dk32, np.swapaxes(ds, -1, -2) @ f[0]) < 1e-5
+
+
+def test_operand_rounding_variant_rounds_exactly_the_matrix_operands():
+    """oracle.operand_rounding(): P f before P V and P^T dO, and dS before dS K and dS^T Q, are rounded to bf16 and
+    nothing else is.  Pinned by recomputing the four products in fp64 from operands rounded here with
+    oracle.f32_to_bf16 (taken from the fp64 softmax, so the check does not reuse the oracle's own P), on a case where
+    the rounding is visible; and by the switch restoring the plain values."""
+    B, H, Sq, Sk, D, seed, scale = 1, 2, 12, 9, 8, 0x2545F4914F6CDD1D, 0.4
+    p = float(np.quantile(O.dropout_uniforms(B, H, Sq, Sk, seed), 0.3))
+    shapes = [(B, H, Sq, D), (B, H, Sk, D), (B, H, Sk, D), (B, H, Sq, D)]
+    q, k, v, do = (W.f32_to_bf16_bits(W.normal_f32(821, i, int(np.prod(s))).reshape(s)) for i, s in enumerate(shapes))
+    fq, fk, fv, g = (O.bf16_to_f32(t).astype(np.float64) for t in (q, k, v, do))
+    _, _, pr = O.brute_sdpa_f64(fq, fk, fv, scale)
+    m = O.dropout_keep_mask(B, H, Sq, Sk, p, seed)
+    factor = np.float64(np.float32(1.0) / (np.float32(1.0) - np.float32(p)))
+
+    def rb(x):        # round to bf16, back to fp64
+        return O.bf16_to_f32(O.f32_to_bf16(x.astype(np.float32))).astype(np.float64)
+
+    pt = rb(pr * m * factor)
+    want_o = pt @ fv
+    plain = O.sdpa_fwd_dropout(q, k, v, scale, p, seed, want_f32=True)
+    with O.operand_rounding():
+        ro, _, ro32 = O.sdpa_fwd_dropout(q, k, v, scale, p, seed, want_f32=True)
+        _, _, _, dq32, dk32, dv32 = O.sdpa_bwd_dropout(q, k, v, ro, do, scale, p, seed, want_f32=True)
+    again = O.sdpa_fwd_dropout(q, k, v, scale, p, seed, want_f32=True)
+    assert np.array_equal(plain[2], again[2])                      # the switch is off again
+    assert np.abs(ro32 - want_o).max() < 5e-6
+    assert np.abs(plain[2] - want_o).max() > 1e-4                  # ... and the rounding is visible in this case
+    delta = (g * O.bf16_to_f32(ro).astype(np.float64)).sum(-1, keepdims=True)
+    ds = rb(pr * (m * factor * (g @ fv.transpose(0, 1, 3, 2)) - delta))
+    assert np.abs(dv32 - pt.transpose(0, 1, 3, 2) @ g).max() < 5e-6
+    # dS is rounded from fp32 values that differ from the fp64 ones in their last bits: a rounding that falls the
+    # other way moves a product by one bf16 step of dS times an element of K or Q, so these two are held less tightly
+    assert np.abs(dq32 - scale * (ds @ fk)).max() < 2e-2 and O.rel_l2(dq32, scale * (ds @ fk)) < 2e-3
+    assert np.abs(dk32 - scale * (ds.transpose(0, 1, 3, 2) @ fq)).max() < 2e-2 and O.rel_l2(dk32, scale * (ds.transpose(0, 1, 3, 2) @ fq)) < 2e-3
