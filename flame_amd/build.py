@@ -74,27 +74,6 @@ def build_probe(verbose: bool = False) -> str:
     return PROBE_LIB_PATH
 
 
-def build_host_test(verbose: bool = False) -> str:
-    """Compiles the C++ host-layer test driver (tests/host/host_api_test.cpp) against the library and the CPU oracle
-    (oracle/_build/liboracle.so, which must have been built: `make -C oracle`)."""
-    root = os.path.dirname(HERE)
-    src = os.path.join(root, "tests", "host", "host_api_test.cpp")
-    out = os.path.join(root, "tests", "host", "host_api_test")
-    cmd = [HIPCC, "--offload-arch=gfx950", "-O2", "-std=c++17", "-x", "hip",
-           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", src, "-o", out,
-           "-L" + LIB_DIR, "-lflame_attn_hip", "-Wl,-rpath,$ORIGIN/../../flame_amd/lib",
-           # the CPU oracle is the checker of this test driver (and of nothing in the library)
-           "-L" + os.path.join(root, "oracle", "_build"), "-loracle", "-Wl,-rpath,$ORIGIN/../../oracle/_build"]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    if res.returncode != 0:
-        raise RuntimeError("hipcc failed:\n" + "\n".join(l for l in res.stdout.splitlines() if "packed-fp32-ops" not in l))
-    return out
-
-
 if __name__ == "__main__":
     print(build_lib(verbose=True, extra=sys.argv[1:]))
     print(build_probe(verbose=True))
-    subprocess.run(["make", "-C", os.path.join(os.path.dirname(HERE), "oracle")], check=True)     # the test driver's checker
-    print(build_host_test(verbose=True))
