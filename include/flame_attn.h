@@ -284,10 +284,12 @@ int flame_cudnn_sdpa_bf16_train_fwd(const void* Q, const void* K, const void* V,
 /* src/cuda/ffi.rs:682-716 (src/cuda/cudnn_sdpa_bwd.cpp:265-361).  The reference signature has no
  * workspace argument: this shim keeps one lazily grown scratch buffer per (device, stream), as the
  * reference's shim keeps a workspace per shape (src/cuda/cudnn_sdpa.cpp:204-212).  Calls on different
- * streams use different buffers and may overlap; a buffer that must grow is replaced, never freed, so
- * work in flight keeps valid memory.  hipMalloc happens on the first call of a stream and on growth
- * only: such a call cannot be captured into a graph (use flame_attn_bwd_bf16 or
- * flame_attn_bwd_bf16_noalloc there). */
+ * streams use different buffers and may overlap; host threads that share a stream are serialised while
+ * they enqueue.  hipMalloc happens on the first call of a stream and on growth only; an outgrown buffer
+ * is freed once its stream is idle.  Under a stream capture a call that would have to allocate returns
+ * FLAME_ATTN_ERR_UNSUPPORTED and launches nothing (call once per shape before capturing, or use
+ * flame_attn_bwd_bf16 / flame_attn_bwd_bf16_noalloc there).  The reference-named forward entry points
+ * below take their scratch (head dims above 128 on a small grid only) from the same buffer. */
 int flame_cudnn_sdpa_bwd_bf16(const void* Q, const void* K, const void* V, const void* O, const void* dO,
                               const void* Stats, void* dQ, void* dK, void* dV,
                               int B, int H, int N_q, int N_kv, int D, float scale,
