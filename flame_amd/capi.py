@@ -422,3 +422,62 @@ def attn_bwd_dropout(q, k, v, o, do, lse, scale, dropout_p, dropout_seed, causal
     if rc != 0:
         raise FlameAttnError("flame_attn_bwd_dropout_tiled_bf16", rc)
     return dq, dk, dv
+
+
+def materialised_workspace_bytes(B, H, Sq, Sk, D, Dv, backward) -> int:
+    f = lib().flame_attn_materialised_workspace_bytes
+    f.restype = ctypes.c_size_t
+    return int(f(B, H, Sq, Sk, D, Dv, int(bool(backward))))
+
+
+def _bias_strides(bias, B, H, Sq, Sk):
+    if bias is None:
+        return None
+    full = (B, H, Sq, Sk)
+    st = []
+    for ax in range(4):
+        assert bias.shape[ax] in (1, full[ax]), "bias is not broadcastable to [B,H,Sq,Sk]"
+        st.append(0 if (bias.shape[ax] == 1 and full[ax] != 1) else bias.stride(ax))
+    return _i64x4(st)
+
+
+def attn_fwd_materialised(q, k, v, scale, causal=False, kv_len=None, mask=None, bias=None, want_lse=True, out=None, workspace=None):
+    """O, LSE = flame_attn_fwd_materialised_bf16(...): any head dim, a value head dim of its own, mask and bias."""
+    B, H, Sq, D = q.shape
+    Sk, Dv = k.shape[2], v.shape[3]
+    o = torch.empty((B, H, Sq, Dv), dtype=torch.bfloat16, device=q.device) if out is None else out
+    lse = torch.empty((B * H, Sq), dtype=torch.float32, device=q.device) if want_lse else None
+    if workspace is None:
+        workspace = torch.empty(materialised_workspace_bytes(B, H, Sq, Sk, D, Dv, False), dtype=torch.uint8, device=q.device)
+    rc = lib().flame_attn_fwd_materialised_bf16(
+        _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), B, H, Sq, Sk, D, Dv, ctypes.c_float(scale),
+        _i64x4(q.stride()), _i64x4(k.stride()), _i64x4(v.stride()), _i64x4(o.stride()),
+        *(ctypes.c_int64(0) for _ in range(5)),
+        int(bool(causal)), _ptr(kv_len), _ptr(mask), _mask_strides(mask, B, H, Sq, Sk),
+        _ptr(bias), 1 if (bias is not None and bias.dtype == torch.float32) else 0, _bias_strides(bias, B, H, Sq, Sk),
+        _ptr(workspace), ctypes.c_size_t(workspace.numel()), _stream())
+    if rc != 0:
+        raise FlameAttnError("flame_attn_fwd_materialised_bf16", rc)
+    return o, lse
+
+
+def attn_bwd_materialised(q, k, v, o, do, lse, scale, causal=False, kv_len=None, mask=None, workspace=None, grads=None):
+    """dQ, dK, dV = flame_attn_bwd_materialised_bf16(...)."""
+    B, H, Sq, D = q.shape
+    Sk, Dv = k.shape[2], v.shape[3]
+    if workspace is None:
+        workspace = torch.empty(materialised_workspace_bytes(B, H, Sq, Sk, D, Dv, True), dtype=torch.uint8, device=q.device)
+    if grads is None:
+        grads = (torch.empty_like(q), torch.empty_like(k), torch.empty_like(v))
+    dq, dk, dv = grads
+    rc = lib().flame_attn_bwd_materialised_bf16(
+        _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(do), _ptr(lse), _ptr(dq), _ptr(dk), _ptr(dv),
+        B, H, Sq, Sk, D, Dv, ctypes.c_float(scale),
+        _i64x4(q.stride()), _i64x4(k.stride()), _i64x4(v.stride()), _i64x4(o.stride()),
+        _i64x4(do.stride()), _i64x4(dq.stride()), _i64x4(dk.stride()), _i64x4(dv.stride()),
+        *(ctypes.c_int64(0) for _ in range(9)),
+        int(bool(causal)), _ptr(kv_len), _ptr(mask), _mask_strides(mask, B, H, Sq, Sk),
+        _ptr(workspace), ctypes.c_size_t(workspace.numel()), _stream())
+    if rc != 0:
+        raise FlameAttnError("flame_attn_bwd_materialised_bf16", rc)
+    return dq, dk, dv

@@ -8,6 +8,7 @@
 
 #include <algorithm>
 
+#include <dlfcn.h>
 #include <hip/hip_runtime.h>
 #include <math.h>
 #include <stdio.h>
@@ -26,6 +27,7 @@
 #include "plan_cache.hpp"
 #include "tile_ops.hpp"
 #include "fp8_offload.hpp"
+#include "materialised.hpp"
 
 using namespace fattn;
 
@@ -1676,6 +1678,325 @@ int flame_fp8_to_bf16(const void* input, void* output, float scale, size_t n_ele
 #ifndef FLAME_ATTN_HIPCC_VERSION
 #define FLAME_ATTN_HIPCC_VERSION "unknown"
 #endif
+}  // extern "C"
+
+// ------------------------------------------------------------------------------------------------
+// The materialised path (materialised.hpp): rocBLAS GEMMs around the element-wise kernels.  rocBLAS is
+// loaded on first use (dlopen), so the library itself links against the HIP runtime only and nothing of
+// rocBLAS is touched unless one of these two entry points runs.
+// ------------------------------------------------------------------------------------------------
+namespace {
+
+struct RocblasApi {
+    // rocblas_status f(...): 0 is success
+    int (*create_handle)(void** handle) = nullptr;
+    int (*set_stream)(void* handle, hipStream_t stream) = nullptr;
+    int (*set_atomics_mode)(void* handle, int mode) = nullptr;
+    int (*gemm_strided_batched_ex)(void* handle, int transA, int transB, int m, int n, int k, const void* alpha, const void* a,
+                                   int a_type, int lda, int64_t stride_a, const void* b, int b_type, int ldb, int64_t stride_b,
+                                   const void* beta, const void* c, int c_type, int ldc, int64_t stride_c, void* d, int d_type,
+                                   int ldd, int64_t stride_d, int batch_count, int compute_type, int algo, int32_t solution_index,
+                                   uint32_t flags) = nullptr;
+    void* handle[64] = {};
+    bool tried = false, ok = false;
+    std::mutex mu;
+};
+RocblasApi g_rocblas;
+// values of rocblas-types.h
+constexpr int kOpN = 111, kOpT = 112, kF32 = 151, kBf16 = 168;
+
+int rocblas_for_device(void** handle_out) {
+    std::lock_guard<std::mutex> g(g_rocblas.mu);
+    if (!g_rocblas.tried) {
+        g_rocblas.tried = true;
+        void* lib = dlopen("librocblas.so.5", RTLD_NOW | RTLD_LOCAL);
+        if (!lib) lib = dlopen("librocblas.so", RTLD_NOW | RTLD_LOCAL);
+        if (lib) {
+            g_rocblas.create_handle = reinterpret_cast<decltype(g_rocblas.create_handle)>(dlsym(lib, "rocblas_create_handle"));
+            g_rocblas.set_stream = reinterpret_cast<decltype(g_rocblas.set_stream)>(dlsym(lib, "rocblas_set_stream"));
+            g_rocblas.set_atomics_mode = reinterpret_cast<decltype(g_rocblas.set_atomics_mode)>(dlsym(lib, "rocblas_set_atomics_mode"));
+            g_rocblas.gemm_strided_batched_ex =
+                reinterpret_cast<decltype(g_rocblas.gemm_strided_batched_ex)>(dlsym(lib, "rocblas_gemm_strided_batched_ex"));
+            g_rocblas.ok = g_rocblas.create_handle && g_rocblas.set_stream && g_rocblas.gemm_strided_batched_ex;
+        }
+    }
+    if (!g_rocblas.ok) return FLAME_ATTN_ERR_UNSUPPORTED;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= 64) return FLAME_ATTN_ERR_UNSUPPORTED;
+    if (!g_rocblas.handle[dev]) {
+        void* h = nullptr;
+        if (g_rocblas.create_handle(&h) != 0 || !h) return FLAME_ATTN_ERR_UNSUPPORTED;
+        if (g_rocblas.set_atomics_mode) (void)g_rocblas.set_atomics_mode(h, 0);      // no atomics: the same sums every run
+        g_rocblas.handle[dev] = h;
+    }
+    *handle_out = g_rocblas.handle[dev];
+    return FLAME_ATTN_OK;
+}
+
+// D[m x n] (column-major, leading dimension ldd) = alpha op(A) op(B) + beta D, batched over the heads of one batch element
+int mat_gemm(void* handle, int ta, int tb, int m, int n, int k, float alpha, const void* a, int lda, int64_t sa, const void* b, int ldb,
+             int64_t sb, float beta, void* d, int d_type, int ldd, int64_t sd, int batch) {
+    const int rc = g_rocblas.gemm_strided_batched_ex(handle, ta, tb, m, n, k, &alpha, a, kBf16, lda, sa, b, kBf16, ldb, sb, &beta, d,
+                                                     d_type, ldd, sd, d, d_type, ldd, sd, batch, kF32, 0, 0, 0);
+    return rc == 0 ? FLAME_ATTN_OK : FLAME_ATTN_ERR_UNSUPPORTED;
+}
+
+int check_view_any_d(const void* base, const int64_t* st) {
+    if (!base || !st) return FLAME_ATTN_ERR_INVALID;
+    if (st[3] != 1) return FLAME_ATTN_ERR_UNSUPPORTED;
+    if (st[0] < 0 || st[1] < 0 || st[2] <= 0 || st[2] > 0x7fffffff) return FLAME_ATTN_ERR_UNSUPPORTED;
+    return FLAME_ATTN_OK;
+}
+
+// bytes per query row of a band: fp32 logits + bf16 P (+ bf16 dS in the backward), over all (batch, head) slices
+size_t mat_band_row_bytes(int B, int H, int N_kv, bool backward) { return (size_t)B * H * N_kv * (backward ? 8 : 6); }
+size_t mat_fixed_bytes(int B, int H, int N_q, bool backward) { return backward ? align_up((size_t)B * H * N_q * sizeof(float), 256) : 0; }
+size_t mat_accum_bytes(int B, int H, int N_kv, int D, int Dv) { return align_up((size_t)B * H * N_kv * (size_t)(D + Dv) * sizeof(float), 256); }
+
+struct MatPlan {
+    int tq = 0;              // query rows per band
+    bool accumulate = false; // more than one band in the backward: dK / dV are summed in fp32 and stored at the end
+    char* rows = nullptr;    // delta [BH, Sq] (backward)
+    char* accum = nullptr;   // fp32 dK [BH, Sk, D] then dV [BH, Sk, Dv] (backward, several bands)
+    char* scores = nullptr;  // fp32 [BH, tq, Sk]
+    char* probs = nullptr;   // bf16 [BH, tq, Sk]
+    char* ds = nullptr;      // bf16 [BH, tq, Sk] (backward)
+};
+
+// Lays the workspace out for the largest band that fits (whole problem if it does), or fails when not even 16 rows do.
+int mat_plan(void* workspace, size_t bytes, int B, int H, int N_q, int N_kv, int D, int Dv, bool backward, MatPlan* out) {
+    if (!workspace || !aligned16(workspace)) return FLAME_ATTN_ERR_INVALID;
+    char* base = static_cast<char*>(workspace);
+    const size_t fixed = mat_fixed_bytes(B, H, N_q, backward), per_row = mat_band_row_bytes(B, H, N_kv, backward);
+    constexpr size_t kSlack = 1024;          // alignment of the three band buffers
+    if (bytes < fixed + kSlack) return FLAME_ATTN_ERR_INVALID;
+    MatPlan p;
+    p.rows = base;
+    size_t avail = bytes - fixed;
+    if (avail >= per_row * (size_t)N_q + kSlack) {
+        p.tq = N_q;
+    } else {
+        if (backward) {
+            const size_t acc = mat_accum_bytes(B, H, N_kv, D, Dv);
+            if (avail < acc + kSlack) return FLAME_ATTN_ERR_INVALID;
+            p.accumulate = true;
+            p.accum = base + fixed;
+            avail -= acc;
+        }
+        const size_t rows = (avail - kSlack) / per_row;
+        if (rows < 16) return FLAME_ATTN_ERR_INVALID;
+        p.tq = (int)std::min<size_t>(rows / 16 * 16, (size_t)N_q);
+    }
+    char* band = base + fixed + (p.accumulate ? mat_accum_bytes(B, H, N_kv, D, Dv) : 0);
+    const size_t n = (size_t)B * H * p.tq * N_kv;
+    p.scores = band;
+    p.probs = band + align_up(n * 4, 256);
+    p.ds = p.probs + align_up(n * 2, 256);
+    *out = p;
+    return FLAME_ATTN_OK;
+}
+
+void mat_fill_mask(MaskArgs& m, int causal, const int32_t* kv_len, const uint8_t* keep_mask, const int64_t* mask_strides,
+                   const void* bias, int bias_dtype, const int64_t* bias_strides) {
+    m.kv_len = kv_len;
+    m.mask = keep_mask;
+    m.sb = keep_mask ? mask_strides[0] : 0;
+    m.sh = keep_mask ? mask_strides[1] : 0;
+    m.sq = keep_mask ? mask_strides[2] : 0;
+    m.sk = keep_mask ? mask_strides[3] : 0;
+    m.causal = causal ? 1 : 0;
+    m.bias = bias;
+    if (bias) {
+        m.bb = bias_strides[0]; m.bh = bias_strides[1]; m.bq = bias_strides[2]; m.bk = bias_strides[3];
+        m.bias_f32 = bias_dtype == FLAME_ATTN_DTYPE_F32;
+    }
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t flame_attn_materialised_workspace_bytes(int B, int H, int N_q, int N_kv, int D, int Dv, int backward) {
+    if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0 || Dv <= 0) return 0;
+    const bool bw = backward != 0;
+    const size_t fixed = mat_fixed_bytes(B, H, N_q, bw), per_row = mat_band_row_bytes(B, H, N_kv, bw);
+    const size_t whole = fixed + per_row * ((size_t)N_q + 1) + 1024;
+    // bands of at least 64 rows and at most 512 MiB, with the fp32 dK / dV sums a banded backward needs
+    const size_t band_rows = std::max<size_t>(64, std::min<size_t>((size_t)N_q, ((size_t)512 << 20) / per_row / 16 * 16));
+    const size_t banded = fixed + (bw ? mat_accum_bytes(B, H, N_kv, D, Dv) : 0) + per_row * (band_rows + 1) + 1024;
+    return std::min(whole, banded);
+}
+
+int flame_attn_fwd_materialised_bf16(const void* Q, const void* K, const void* V, void* O, void* LSE,
+                                     int B, int H, int N_q, int N_kv, int D, int Dv, float scale,
+                                     const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                                     const int64_t* o_strides,
+                                     int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off, int64_t lse_off,
+                                     int causal, const int32_t* kv_len, const uint8_t* keep_mask, const int64_t* mask_strides,
+                                     const void* bias, int bias_dtype, const int64_t* bias_strides,
+                                     void* workspace, size_t workspace_bytes, void* stream) {
+    if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0 || Dv <= 0) return FLAME_ATTN_ERR_INVALID;
+    if (!(scale > 0.f) || !isfinite(scale)) return FLAME_ATTN_ERR_INVALID;
+    int rc;
+    if ((rc = check_view_any_d(Q, q_strides)) || (rc = check_view_any_d(K, k_strides)) || (rc = check_view_any_d(V, v_strides)) ||
+        (rc = check_view_any_d(O, o_strides)))
+        return rc;
+    if ((keep_mask && !mask_strides) || (bias && !bias_strides)) return FLAME_ATTN_ERR_INVALID;
+    if (bias && bias_dtype != FLAME_ATTN_DTYPE_BF16 && bias_dtype != FLAME_ATTN_DTYPE_F32) return FLAME_ATTN_ERR_INVALID;
+    if ((int64_t)B * H * N_q > 0x7fffffff) return FLAME_ATTN_ERR_UNSUPPORTED;
+    MatPlan plan;
+    if ((rc = mat_plan(workspace, workspace_bytes, B, H, N_q, N_kv, D, Dv, false, &plan))) return rc;
+    void* handle = nullptr;
+    if ((rc = rocblas_for_device(&handle))) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    std::lock_guard<std::mutex> enqueue(g_rocblas.mu);          // the handle's stream is set per call
+    if (g_rocblas.set_stream(handle, s) != 0) return FLAME_ATTN_ERR_UNSUPPORTED;
+    const uint16_t* q = static_cast<const uint16_t*>(Q) + q_off;
+    const uint16_t* k = static_cast<const uint16_t*>(K) + k_off;
+    const uint16_t* v = static_cast<const uint16_t*>(V) + v_off;
+    uint16_t* o = static_cast<uint16_t*>(O) + o_off;
+    MatRowsParams rp;
+    rp.scores = reinterpret_cast<float*>(plan.scores);
+    rp.probs = reinterpret_cast<uint16_t*>(plan.probs);
+    rp.lse = LSE ? static_cast<float*>(LSE) + lse_off : nullptr;
+    rp.H = H; rp.Sq = N_q; rp.Sk = N_kv;
+    rp.from_lse = 0;
+    mat_fill_mask(rp.m, causal, kv_len, keep_mask, mask_strides, bias, bias_dtype, bias_strides);
+    for (int q0 = 0; q0 < N_q; q0 += plan.tq) {
+        const int tq = std::min(plan.tq, N_q - q0);
+        const int64_t band = (int64_t)tq * N_kv;
+        for (int b = 0; b < B; ++b) {       // S^T [Sk x tq] = scale K Q^T, all heads of one batch element per call
+            rc = mat_gemm(handle, kOpT, kOpN, N_kv, tq, D, scale, k + b * k_strides[0], (int)k_strides[2], k_strides[1],
+                          q + b * q_strides[0] + (int64_t)q0 * q_strides[2], (int)q_strides[2], q_strides[1], 0.f,
+                          rp.scores + (int64_t)b * H * band, kF32, N_kv, band, H);
+            if (rc) return rc;
+        }
+        rp.tq = tq; rp.q0 = q0;
+        hipLaunchKernelGGL(mat_rows_kernel, dim3((unsigned)((int64_t)B * H * tq)), dim3(256), 0, s, rp);
+        for (int b = 0; b < B; ++b) {       // O^T [Dv x tq] = V^T P^T
+            rc = mat_gemm(handle, kOpN, kOpN, Dv, tq, N_kv, 1.f, v + b * v_strides[0], (int)v_strides[2], v_strides[1],
+                          rp.probs + (int64_t)b * H * band, N_kv, band, 0.f, o + b * o_strides[0] + (int64_t)q0 * o_strides[2], kBf16,
+                          (int)o_strides[2], o_strides[1], H);
+            if (rc) return rc;
+        }
+    }
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? FLAME_ATTN_OK : (int)e;
+}
+
+int flame_attn_bwd_materialised_bf16(const void* Q, const void* K, const void* V, const void* O, const void* dO,
+                                     const void* LSE, void* dQ, void* dK, void* dV,
+                                     int B, int H, int N_q, int N_kv, int D, int Dv, float scale,
+                                     const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                                     const int64_t* o_strides, const int64_t* do_strides, const int64_t* dq_strides,
+                                     const int64_t* dk_strides, const int64_t* dv_strides,
+                                     int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off, int64_t do_off,
+                                     int64_t lse_off, int64_t dq_off, int64_t dk_off, int64_t dv_off,
+                                     int causal, const int32_t* kv_len, const uint8_t* keep_mask, const int64_t* mask_strides,
+                                     void* workspace, size_t workspace_bytes, void* stream) {
+    if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0 || Dv <= 0) return FLAME_ATTN_ERR_INVALID;
+    if (!(scale > 0.f) || !isfinite(scale) || !LSE) return FLAME_ATTN_ERR_INVALID;
+    int rc;
+    if ((rc = check_view_any_d(Q, q_strides)) || (rc = check_view_any_d(K, k_strides)) || (rc = check_view_any_d(V, v_strides)) ||
+        (rc = check_view_any_d(O, o_strides)) || (rc = check_view_any_d(dO, do_strides)) || (rc = check_view_any_d(dQ, dq_strides)) ||
+        (rc = check_view_any_d(dK, dk_strides)) || (rc = check_view_any_d(dV, dv_strides)))
+        return rc;
+    if (keep_mask && !mask_strides) return FLAME_ATTN_ERR_INVALID;
+    if ((int64_t)B * H * N_q > 0x7fffffff) return FLAME_ATTN_ERR_UNSUPPORTED;
+    MatPlan plan;
+    if ((rc = mat_plan(workspace, workspace_bytes, B, H, N_q, N_kv, D, Dv, true, &plan))) return rc;
+    void* handle = nullptr;
+    if ((rc = rocblas_for_device(&handle))) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    std::lock_guard<std::mutex> enqueue(g_rocblas.mu);
+    if (g_rocblas.set_stream(handle, s) != 0) return FLAME_ATTN_ERR_UNSUPPORTED;
+    const uint16_t* q = static_cast<const uint16_t*>(Q) + q_off;
+    const uint16_t* k = static_cast<const uint16_t*>(K) + k_off;
+    const uint16_t* v = static_cast<const uint16_t*>(V) + v_off;
+    const uint16_t* d_o = static_cast<const uint16_t*>(dO) + do_off;
+    uint16_t* dq = static_cast<uint16_t*>(dQ) + dq_off;
+    uint16_t* dk = static_cast<uint16_t*>(dK) + dk_off;
+    uint16_t* dv = static_cast<uint16_t*>(dV) + dv_off;
+    float* delta = reinterpret_cast<float*>(plan.rows);
+    {
+        MatDeltaParams dp;
+        dp.o = static_cast<const uint16_t*>(O) + o_off;
+        dp.dout = d_o;
+        dp.os = mk(o_strides); dp.dos = mk(do_strides);
+        dp.delta = delta;
+        dp.B = B; dp.H = H; dp.Sq = N_q; dp.dv = Dv;
+        const int64_t rows = (int64_t)B * H * N_q;
+        hipLaunchKernelGGL(mat_delta_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, s, dp);
+    }
+    MatRowsParams rp;
+    rp.scores = reinterpret_cast<float*>(plan.scores);
+    rp.probs = reinterpret_cast<uint16_t*>(plan.probs);
+    rp.lse = const_cast<float*>(static_cast<const float*>(LSE) + lse_off);
+    rp.H = H; rp.Sq = N_q; rp.Sk = N_kv;
+    rp.from_lse = 1;
+    mat_fill_mask(rp.m, causal, kv_len, keep_mask, mask_strides, nullptr, FLAME_ATTN_DTYPE_F32, nullptr);
+    uint16_t* ds = reinterpret_cast<uint16_t*>(plan.ds);
+    float* acc_dk = reinterpret_cast<float*>(plan.accum);
+    float* acc_dv = plan.accum ? acc_dk + (size_t)B * H * N_kv * D : nullptr;
+    for (int q0 = 0; q0 < N_q; q0 += plan.tq) {
+        const int tq = std::min(plan.tq, N_q - q0);
+        const int64_t band = (int64_t)tq * N_kv;
+        const float beta = (plan.accumulate && q0 > 0) ? 1.f : 0.f;
+        for (int b = 0; b < B; ++b) {       // S^T = scale K Q^T
+            rc = mat_gemm(handle, kOpT, kOpN, N_kv, tq, D, scale, k + b * k_strides[0], (int)k_strides[2], k_strides[1],
+                          q + b * q_strides[0] + (int64_t)q0 * q_strides[2], (int)q_strides[2], q_strides[1], 0.f,
+                          rp.scores + (int64_t)b * H * band, kF32, N_kv, band, H);
+            if (rc) return rc;
+        }
+        rp.tq = tq; rp.q0 = q0;
+        hipLaunchKernelGGL(mat_rows_kernel, dim3((unsigned)((int64_t)B * H * tq)), dim3(256), 0, s, rp);      // P = exp(S - LSE)
+        for (int b = 0; b < B; ++b) {       // dP^T [Sk x tq] = V dO^T, into the logits' buffer (P has been formed)
+            rc = mat_gemm(handle, kOpT, kOpN, N_kv, tq, Dv, 1.f, v + b * v_strides[0], (int)v_strides[2], v_strides[1],
+                          d_o + b * do_strides[0] + (int64_t)q0 * do_strides[2], (int)do_strides[2], do_strides[1], 0.f,
+                          rp.scores + (int64_t)b * H * band, kF32, N_kv, band, H);
+            if (rc) return rc;
+        }
+        {
+            const int64_t n = (int64_t)B * H * band;
+            hipLaunchKernelGGL(mat_ds_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, rp.probs, rp.scores, delta, ds, n, N_kv,
+                               tq, N_q, q0);
+        }
+        for (int b = 0; b < B; ++b) {
+            const uint16_t* pb = rp.probs + (int64_t)b * H * band;
+            const uint16_t* dsb = ds + (int64_t)b * H * band;
+            // dV^T [Dv x Sk] (+)= dO^T P ; dK^T [D x Sk] (+)= scale Q^T dS ; dQ^T [D x tq] = scale K^T dS^T
+            if (plan.accumulate) {
+                rc = mat_gemm(handle, kOpN, kOpT, Dv, N_kv, tq, 1.f, d_o + b * do_strides[0] + (int64_t)q0 * do_strides[2],
+                              (int)do_strides[2], do_strides[1], pb, N_kv, band, beta, acc_dv + (size_t)b * H * N_kv * Dv, kF32, Dv,
+                              (int64_t)N_kv * Dv, H);
+                if (rc) return rc;
+                rc = mat_gemm(handle, kOpN, kOpT, D, N_kv, tq, scale, q + b * q_strides[0] + (int64_t)q0 * q_strides[2], (int)q_strides[2],
+                              q_strides[1], dsb, N_kv, band, beta, acc_dk + (size_t)b * H * N_kv * D, kF32, D, (int64_t)N_kv * D, H);
+                if (rc) return rc;
+            } else {
+                rc = mat_gemm(handle, kOpN, kOpT, Dv, N_kv, tq, 1.f, d_o + b * do_strides[0], (int)do_strides[2], do_strides[1], pb, N_kv,
+                              band, 0.f, dv + b * dv_strides[0], kBf16, (int)dv_strides[2], dv_strides[1], H);
+                if (rc) return rc;
+                rc = mat_gemm(handle, kOpN, kOpT, D, N_kv, tq, scale, q + b * q_strides[0], (int)q_strides[2], q_strides[1], dsb, N_kv,
+                              band, 0.f, dk + b * dk_strides[0], kBf16, (int)dk_strides[2], dk_strides[1], H);
+                if (rc) return rc;
+            }
+            rc = mat_gemm(handle, kOpN, kOpN, D, tq, N_kv, scale, k + b * k_strides[0], (int)k_strides[2], k_strides[1], dsb, N_kv, band, 0.f,
+                          dq + b * dq_strides[0] + (int64_t)q0 * dq_strides[2], kBf16, (int)dq_strides[2], dq_strides[1], H);
+            if (rc) return rc;
+        }
+    }
+    if (plan.accumulate) {
+        const int64_t nk = (int64_t)B * H * N_kv * D, nv = (int64_t)B * H * N_kv * Dv;
+        hipLaunchKernelGGL(mat_store_kernel, dim3((unsigned)((nk + 255) / 256)), dim3(256), 0, s, acc_dk, dk, mk(dk_strides), H, N_kv, D, nk);
+        hipLaunchKernelGGL(mat_store_kernel, dim3((unsigned)((nv + 255) / 256)), dim3(256), 0, s, acc_dv, dv, mk(dv_strides), H, N_kv, Dv, nv);
+    }
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? FLAME_ATTN_OK : (int)e;
+}
+
 // names the compiler that built this library: the static checks of the hand-emitted instructions are
 // only meaningful for the assembly that this very compiler generates
 const char* flame_attn_version(void) { return "flame-attn-gfx950 0.2 (hipcc " FLAME_ATTN_HIPCC_VERSION ")"; }

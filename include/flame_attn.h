@@ -220,6 +220,42 @@ int flame_attn_bwd_bf16_noalloc(const void* Q, const void* K, const void* V, con
                                 const uint8_t* keep_mask, const int64_t* mask_strides, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
+ * The materialised path: every shape the fused kernels refuse.  Any head dim D >= 1 (no multiple-of-8 rule, no
+ * upper limit, D stride 1 and non-negative strides as the only layout rules), a value head dim Dv of its own,
+ * causal flag, key lengths, keep-mask and (forward) additive bias as in the primary entry points, and the
+ * backward for all of them.  It is what the reference does for these shapes (materialised scores through
+ * library GEMMs: src/sdpa.rs:483-587, :788-961; backward src/autograd.rs:801-848): rocBLAS bf16 GEMMs with fp32
+ * accumulation for Q K^T, P V and the four backward products (rocBLAS is loaded with dlopen on the first call,
+ * which makes these two the only entry points that need it; FLAME_ATTN_ERR_UNSUPPORTED when it cannot be loaded),
+ * this library's element-wise kernels in between.  The scores exist for one band of query rows at a time, in the
+ * caller's workspace (8 bytes per score element of the band in the backward, 6 in the forward); what is kept
+ * between forward and backward is O and LSE, as everywhere else.  flame_attn_materialised_workspace_bytes returns
+ * the size with which the whole problem is one band or, for large problems, bands of about 512 MiB; any workspace
+ * that holds 16 query rows is accepted (more bands).  The first call creates a rocBLAS handle per device, which
+ * allocates: these entry points are not meant for graph capture.  Several times slower than the fused kernels
+ * where both apply.
+ * ---------------------------------------------------------------------------------------------- */
+size_t flame_attn_materialised_workspace_bytes(int B, int H, int N_q, int N_kv, int D, int Dv, int backward);
+int flame_attn_fwd_materialised_bf16(const void* Q, const void* K, const void* V, void* O, void* LSE,
+                                     int B, int H, int N_q, int N_kv, int D, int Dv, float scale,
+                                     const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                                     const int64_t* o_strides,
+                                     int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off, int64_t lse_off,
+                                     int causal, const int32_t* kv_len, const uint8_t* keep_mask, const int64_t* mask_strides,
+                                     const void* bias, int bias_dtype, const int64_t* bias_strides,
+                                     void* workspace, size_t workspace_bytes, void* stream);
+int flame_attn_bwd_materialised_bf16(const void* Q, const void* K, const void* V, const void* O, const void* dO,
+                                     const void* LSE, void* dQ, void* dK, void* dV,
+                                     int B, int H, int N_q, int N_kv, int D, int Dv, float scale,
+                                     const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                                     const int64_t* o_strides, const int64_t* do_strides, const int64_t* dq_strides,
+                                     const int64_t* dk_strides, const int64_t* dv_strides,
+                                     int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off, int64_t do_off,
+                                     int64_t lse_off, int64_t dq_off, int64_t dk_off, int64_t dv_off,
+                                     int causal, const int32_t* kv_len, const uint8_t* keep_mask, const int64_t* mask_strides,
+                                     void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
  * SageAttention int8-QK inference variant (API shape: src/sage_attention.rs:21-65; quantiser closed
  * form: src/sage_attention.rs:524-541; block granularity, K mean smoothing and int8 MFMA are new).
  * ---------------------------------------------------------------------------------------------- */

@@ -162,6 +162,27 @@ extern "C" {
         dq_off: i64, dk_off: i64, dv_off: i64, causal: c_int, kv_len: *const i32, keep_mask: *const u8,
         mask_strides: *const i64, stream: *mut c_void
     ) -> c_int;
+    pub fn flame_attn_materialised_workspace_bytes(
+        b: c_int, h: c_int, n_q: c_int, n_kv: c_int, d: c_int, dv: c_int, backward: c_int
+    ) -> usize;
+    pub fn flame_attn_fwd_materialised_bf16(
+        q: *const c_void, k: *const c_void, v: *const c_void, o: *mut c_void, lse: *mut c_void, b: c_int,
+        h: c_int, n_q: c_int, n_kv: c_int, d: c_int, dv: c_int, scale: f32, q_strides: *const i64,
+        k_strides: *const i64, v_strides: *const i64, o_strides: *const i64, q_off: i64, k_off: i64, v_off: i64,
+        o_off: i64, lse_off: i64, causal: c_int, kv_len: *const i32, keep_mask: *const u8,
+        mask_strides: *const i64, bias: *const c_void, bias_dtype: c_int, bias_strides: *const i64,
+        workspace: *mut c_void, workspace_bytes: usize, stream: *mut c_void
+    ) -> c_int;
+    pub fn flame_attn_bwd_materialised_bf16(
+        q: *const c_void, k: *const c_void, v: *const c_void, o: *const c_void, d_o: *const c_void,
+        lse: *const c_void, dq: *mut c_void, dk: *mut c_void, dv_out: *mut c_void, b: c_int, h: c_int, n_q: c_int,
+        n_kv: c_int, d: c_int, dv: c_int, scale: f32, q_strides: *const i64, k_strides: *const i64,
+        v_strides: *const i64, o_strides: *const i64, do_strides: *const i64, dq_strides: *const i64,
+        dk_strides: *const i64, dv_strides: *const i64, q_off: i64, k_off: i64, v_off: i64, o_off: i64,
+        do_off: i64, lse_off: i64, dq_off: i64, dk_off: i64, dv_off: i64, causal: c_int, kv_len: *const i32,
+        keep_mask: *const u8, mask_strides: *const i64, workspace: *mut c_void, workspace_bytes: usize,
+        stream: *mut c_void
+    ) -> c_int;
     pub fn flame_sage_quant_qk_int8(
         q: *const c_void, k: *const c_void, b: c_int, h: c_int, n_q: c_int, n_kv: c_int, d: c_int,
         q_strides: *const i64, k_strides: *const i64, q_off: i64, k_off: i64, smooth_k: c_int,
