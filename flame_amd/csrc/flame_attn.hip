@@ -1008,6 +1008,14 @@ int flame_attn_fwd_bias_bf16(const void* Q, const void* K, const void* V, void* 
 // src/cuda/cudnn_sdpa.cpp:204-212; eleven buffers per call, cuda/sdpa_stream_bf16.cu:214-239): where a
 // kernel needs scratch they take the library's per-(device, stream) buffer.
 // ------------------------------------------------------------------------------------------------
+static int mat_fwd_impl(const void* Q, const void* K, const void* V, void* O, void* LSE,
+                        int B, int H, int N_q, int N_kv, int D, int Dv, float scale,
+                        const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                        const int64_t* o_strides,
+                        int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off, int64_t lse_off,
+                        int causal, const int32_t* kv_len, const uint8_t* keep_mask, const int64_t* mask_strides,
+                        const void* bias, int bias_dtype, const int64_t* bias_strides,
+                        void* workspace, size_t workspace_bytes, void* stream, int mask_mode);
 static FwdScratch library_scratch() {
     FwdScratch sc;
     sc.library = true;
@@ -1283,16 +1291,27 @@ FlameAttnStatus flame_sdpa_chunked_bf16(const void* q, const void* k, const void
         ms[3] = 1;
     }
     auto run = [&](int q_tile) {
-        return attn_fwd_impl(q, k, v, out, nullptr, B, H, Q, K, Dh, scale, qs, ks, vs, os, 0, 0, 0, 0, 0, causal, nullptr,
-                             static_cast<const uint8_t*>(mask), mask ? ms : nullptr, nullptr, FLAME_ATTN_DTYPE_F32, nullptr,
-                             stream, kMaskBf16Keep, Dv, q_tile, 0.f, 0, 0, 0, library_scratch());
+        const int rc = attn_fwd_impl(q, k, v, out, nullptr, B, H, Q, K, Dh, scale, qs, ks, vs, os, 0, 0, 0, 0, 0, causal, nullptr,
+                                     static_cast<const uint8_t*>(mask), mask ? ms : nullptr, nullptr, FLAME_ATTN_DTYPE_F32, nullptr,
+                                     stream, kMaskBf16Keep, Dv, q_tile, 0.f, 0, 0, 0, library_scratch());
+        if (rc != FLAME_ATTN_ERR_UNSUPPORTED) return rc;
+        // The reference's entry point takes any head dims (its scalar kernels, cuda/src/flame_sdpa_stub.cu:696-866):
+        // what the fused kernels do not serve goes through materialised scores, in the library's own scratch.
+        const size_t need = flame_attn_materialised_workspace_bytes(B, H, Q, K, Dh, Dv, 0);
+        std::lock_guard<std::mutex> enqueue(lib_scratch_enqueue_mutex());
+        void* ws = nullptr;
+        const int rs = lib_scratch_get(need, static_cast<hipStream_t>(stream), &ws);
+        if (rs) return rs;
+        return mat_fwd_impl(q, k, v, out, nullptr, B, H, Q, K, Dh, Dv, scale, qs, ks, vs, os, 0, 0, 0, 0, 0, causal, nullptr,
+                            static_cast<const uint8_t*>(mask), mask ? ms : nullptr, nullptr, FLAME_ATTN_DTYPE_F32, nullptr, ws, need,
+                            stream, kMaskBf16Keep);
     };
     // ---- the launch plan: the query tile of a workgroup (see plan_cache.hpp)
     PlanCache& pc = PlanCache::instance();
     const PlanConfig& cfg = pc.config();
-    // the masked kernels come with 128-row workgroups only, and head dims above 128 have one kernel per head dim:
-    // nothing to choose, so nothing is measured
-    const bool one_tile = mask != nullptr || big_head_dim_ok(Dh);
+    // the masked kernels come with 128-row workgroups only, and head dims other than the multiples of 8 up to 128 have
+    // one kernel (or the materialised path): nothing to choose, so nothing is measured
+    const bool one_tile = mask != nullptr || !head_dim_ok(Dh);
     const int rule_q = (!one_tile && fwd_rule_wide(B, H, Q, false, false)) ? 256 : 128;
     const PlanKey key{B, H, Q, K, Dh, Dv, mask ? mask_heads : 0, causal ? 1 : 0};
     int q_tile = rule_q;
@@ -1799,9 +1818,10 @@ int mat_plan(void* workspace, size_t bytes, int B, int H, int N_q, int N_kv, int
 }
 
 void mat_fill_mask(MaskArgs& m, int causal, const int32_t* kv_len, const uint8_t* keep_mask, const int64_t* mask_strides,
-                   const void* bias, int bias_dtype, const int64_t* bias_strides) {
+                   const void* bias, int bias_dtype, const int64_t* bias_strides, int mask_mode = kMaskU8) {
     m.kv_len = kv_len;
     m.mask = keep_mask;
+    m.mask_mode = mask_mode;
     m.sb = keep_mask ? mask_strides[0] : 0;
     m.sh = keep_mask ? mask_strides[1] : 0;
     m.sq = keep_mask ? mask_strides[2] : 0;
@@ -1829,14 +1849,14 @@ size_t flame_attn_materialised_workspace_bytes(int B, int H, int N_q, int N_kv, 
     return std::min(whole, banded);
 }
 
-int flame_attn_fwd_materialised_bf16(const void* Q, const void* K, const void* V, void* O, void* LSE,
-                                     int B, int H, int N_q, int N_kv, int D, int Dv, float scale,
-                                     const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
-                                     const int64_t* o_strides,
-                                     int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off, int64_t lse_off,
-                                     int causal, const int32_t* kv_len, const uint8_t* keep_mask, const int64_t* mask_strides,
-                                     const void* bias, int bias_dtype, const int64_t* bias_strides,
-                                     void* workspace, size_t workspace_bytes, void* stream) {
+static int mat_fwd_impl(const void* Q, const void* K, const void* V, void* O, void* LSE,
+                        int B, int H, int N_q, int N_kv, int D, int Dv, float scale,
+                        const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                        const int64_t* o_strides,
+                        int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off, int64_t lse_off,
+                        int causal, const int32_t* kv_len, const uint8_t* keep_mask, const int64_t* mask_strides,
+                        const void* bias, int bias_dtype, const int64_t* bias_strides,
+                        void* workspace, size_t workspace_bytes, void* stream, int mask_mode) {
     if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0 || Dv <= 0) return FLAME_ATTN_ERR_INVALID;
     if (!(scale > 0.f) || !isfinite(scale)) return FLAME_ATTN_ERR_INVALID;
     int rc;
@@ -1863,7 +1883,7 @@ int flame_attn_fwd_materialised_bf16(const void* Q, const void* K, const void* V
     rp.lse = LSE ? static_cast<float*>(LSE) + lse_off : nullptr;
     rp.H = H; rp.Sq = N_q; rp.Sk = N_kv;
     rp.from_lse = 0;
-    mat_fill_mask(rp.m, causal, kv_len, keep_mask, mask_strides, bias, bias_dtype, bias_strides);
+    mat_fill_mask(rp.m, causal, kv_len, keep_mask, mask_strides, bias, bias_dtype, bias_strides, mask_mode);
     for (int q0 = 0; q0 < N_q; q0 += plan.tq) {
         const int tq = std::min(plan.tq, N_q - q0);
         const int64_t band = (int64_t)tq * N_kv;
@@ -1884,6 +1904,19 @@ int flame_attn_fwd_materialised_bf16(const void* Q, const void* K, const void* V
     }
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? FLAME_ATTN_OK : (int)e;
+}
+
+int flame_attn_fwd_materialised_bf16(const void* Q, const void* K, const void* V, void* O, void* LSE,
+                                     int B, int H, int N_q, int N_kv, int D, int Dv, float scale,
+                                     const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                                     const int64_t* o_strides,
+                                     int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off, int64_t lse_off,
+                                     int causal, const int32_t* kv_len, const uint8_t* keep_mask, const int64_t* mask_strides,
+                                     const void* bias, int bias_dtype, const int64_t* bias_strides,
+                                     void* workspace, size_t workspace_bytes, void* stream) {
+    return mat_fwd_impl(Q, K, V, O, LSE, B, H, N_q, N_kv, D, Dv, scale, q_strides, k_strides, v_strides, o_strides, q_off, k_off,
+                        v_off, o_off, lse_off, causal, kv_len, keep_mask, mask_strides, bias, bias_dtype, bias_strides, workspace,
+                        workspace_bytes, stream, kMaskU8);
 }
 
 int flame_attn_bwd_materialised_bf16(const void* Q, const void* K, const void* V, const void* O, const void* dO,

@@ -17,7 +17,16 @@ from . import capi
 class _Sdpa(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q, k, v, mask_u8, causal, scale):
-        o, lse = capi.attn_fwd(q, k, v, scale, causal=causal, mask=mask_u8)
+        # the fused kernels where they serve the shape, else the materialised path (any head dim, masks above 128),
+        # as the reference's dispatch does (src/sdpa.rs:483-587); both save O and the log-sum-exp only
+        ctx.materialised = False
+        try:
+            o, lse = capi.attn_fwd(q, k, v, scale, causal=causal, mask=mask_u8)
+        except capi.FlameAttnError as e:
+            if e.code != capi.ERR_UNSUPPORTED:
+                raise
+            o, lse = capi.attn_fwd_materialised(q, k, v, scale, causal=causal, mask=mask_u8)
+            ctx.materialised = True
         ctx.save_for_backward(q, k, v, o, lse)
         ctx.mask_u8, ctx.causal, ctx.scale = mask_u8, causal, scale
         return o
@@ -28,13 +37,21 @@ class _Sdpa(torch.autograd.Function):
         g = grad_out.to(torch.bfloat16)
         if g.stride(-1) != 1 or any(s % 8 for s in g.stride()[:-1]):
             g = g.contiguous()
-        dq, dk, dv = capi.attn_bwd(q, k, v, o, g, lse, ctx.scale, causal=ctx.causal, mask=ctx.mask_u8)
+        if not ctx.materialised:
+            try:
+                return (*capi.attn_bwd(q, k, v, o, g, lse, ctx.scale, causal=ctx.causal, mask=ctx.mask_u8), None, None, None)
+            except capi.FlameAttnError as e:         # a head dim the fused forward serves and the fused backward does not
+                if e.code != capi.ERR_UNSUPPORTED:
+                    raise
+        dq, dk, dv = capi.attn_bwd_materialised(q, k, v, o, g, lse, ctx.scale, causal=ctx.causal, mask=ctx.mask_u8)
         return dq, dk, dv, None, None, None
 
 
 def _as_bf16_view(t: torch.Tensor) -> torch.Tensor:
     t = t if t.dtype == torch.bfloat16 else t.to(torch.bfloat16)     # promote_bf16 of the reference
-    if t.stride(-1) != 1 or any(s % 8 for s in t.stride()[:-1]) or (t.storage_offset() % 8):
+    if t.shape[-1] % 8 == 0 and (t.stride(-1) != 1 or any(s % 8 for s in t.stride()[:-1]) or (t.storage_offset() % 8)):
+        t = t.contiguous()
+    elif t.stride(-1) != 1:
         t = t.contiguous()
     return t
 

@@ -223,7 +223,8 @@ inline Result<FwdOut> run_forward(const Tensor& q, const Tensor& k, const Tensor
     if (!dv.ok()) return dv.error();
     const Dims d = dv.value();
     for (const Tensor* t : {&q, &k, &v})
-        if (!abi_friendly(*t)) return unsupported("tensor view needs D stride 1 and 16-byte aligned rows; make it contiguous first");
+        if (t->strides()[3] != 1 || (d.D % 8 == 0 && !abi_friendly(*t)))
+            return unsupported("tensor view needs D stride 1 and 16-byte aligned rows; make it contiguous first");
     auto o = Tensor::empty({d.B, d.H, d.Sq, d.D}, DType::BF16);      // O = q.shape, contiguous (src/sdpa.rs:631)
     if (!o.ok()) return o.error();
     Tensor stats;
@@ -256,7 +257,22 @@ inline Result<FwdOut> run_forward(const Tensor& q, const Tensor& k, const Tensor
                                        v.strides().data(), o.value().strides().data(), q.offset(), k.offset(), v.offset(), 0, 0,
                                        causal ? 1 : 0, nullptr, mask ? static_cast<const uint8_t*>(m8.data()) : nullptr,
                                        mask ? mst.data() : nullptr, nullptr /* default stream, as the reference */);
-    if (rc == FLAME_ATTN_ERR_UNSUPPORTED) return unsupported("flame_attn_fwd_bf16: head dim or layout not built");
+    if (rc == FLAME_ATTN_ERR_UNSUPPORTED) {
+        // forward_bf16's last branch (src/sdpa.rs:543-587 -> forward_bf16_fallback, :788-961): whatever the fused
+        // kernels do not serve (a head dim that is not a multiple of 8 or lies above 512, a mask above 128) goes
+        // through materialised scores, one band of query rows at a time
+        const size_t wsb = flame_attn_materialised_workspace_bytes(d.B, d.H, d.Sq, d.Sk, d.D, d.D, 0);
+        auto ws = Tensor::empty({(int64_t)wsb}, DType::U8);
+        if (!ws.ok()) return ws.error();
+        const int rm = flame_attn_fwd_materialised_bf16(
+            q.base(), k.base(), v.base(), o.value().base(), want_stats ? stats.base() : nullptr, d.B, d.H, d.Sq, d.Sk, d.D, d.D, sc,
+            q.strides().data(), k.strides().data(), v.strides().data(), o.value().strides().data(), q.offset(), k.offset(), v.offset(),
+            0, 0, causal ? 1 : 0, nullptr, mask ? static_cast<const uint8_t*>(m8.data()) : nullptr, mask ? mst.data() : nullptr, nullptr,
+            FLAME_ATTN_DTYPE_F32, nullptr, ws.value().data(), wsb, nullptr);
+        if (rm == FLAME_ATTN_ERR_UNSUPPORTED) return unsupported("flame_attn_fwd_materialised_bf16: layout not served (or rocBLAS missing)");
+        if (rm != 0) return cuda_error("flame_attn_fwd_materialised_bf16", rm);
+        return FwdOut{o.value(), stats};
+    }
     if (rc != 0) return cuda_error("flame_attn_fwd_bf16", rc);
     return FwdOut{o.value(), stats};
 }
@@ -373,7 +389,23 @@ inline Result<AttentionGrads> flash_attention_backward(const FlashAttentionNode&
         n.output.offset(), g.offset(), 0, 0, 0, 0, n.causal ? 1 : 0, nullptr,
         n.mask ? static_cast<const uint8_t*>(m8.data()) : nullptr, n.mask ? mst.data() : nullptr, ws.value().data(), wsb,
         nullptr);
-    if (rc == FLAME_ATTN_ERR_UNSUPPORTED) return unsupported("flame_attn_bwd_bf16: head dim or layout not built");
+    if (rc == FLAME_ATTN_ERR_UNSUPPORTED) {
+        // attention_backward_recompute (src/autograd.rs:801-848): the materialising backward for what the fused one
+        // does not serve, here one band of query rows at a time
+        const size_t wsm = flame_attn_materialised_workspace_bytes(B, H, Sq, Sk, D, D, 1);
+        auto wm = Tensor::empty({(int64_t)wsm}, DType::U8);
+        if (!wm.ok()) return wm.error();
+        const int rm = flame_attn_bwd_materialised_bf16(
+            n.query.base(), n.key.base(), n.value.base(), n.output.base(), g.base(), n.stats.base(), dq.value().base(),
+            dk.value().base(), dv.value().base(), B, H, Sq, Sk, D, D, n.scale, n.query.strides().data(), n.key.strides().data(),
+            n.value.strides().data(), n.output.strides().data(), g.strides().data(), dq.value().strides().data(),
+            dk.value().strides().data(), dv.value().strides().data(), n.query.offset(), n.key.offset(), n.value.offset(),
+            n.output.offset(), g.offset(), 0, 0, 0, 0, n.causal ? 1 : 0, nullptr,
+            n.mask ? static_cast<const uint8_t*>(m8.data()) : nullptr, n.mask ? mst.data() : nullptr, wm.value().data(), wsm, nullptr);
+        if (rm == FLAME_ATTN_ERR_UNSUPPORTED) return unsupported("flame_attn_bwd_materialised_bf16: layout not served (or rocBLAS missing)");
+        if (rm != 0) return cuda_error("flame_attn_bwd_materialised_bf16", rm);
+        return AttentionGrads{dq.value(), dk.value(), dv.value()};
+    }
     if (rc != 0) return cuda_error("flame_attn_bwd_bf16", rc);
     return AttentionGrads{dq.value(), dk.value(), dv.value()};
 }

@@ -195,7 +195,7 @@ int main() {
         CHECK(kind(sdpa::forward(f32, f32, f32)) == Error::InvalidInput, "non-bf16");
         CHECK(sdpa::forward(d100, d100, d100).ok(), "head dim 104 runs (padded to 128)");
         CHECK(sdpa::forward(d256, d256, d256).ok(), "head dim 256 runs (forward only, two chunks of 128)");
-        CHECK(kind(sdpa::forward(d520, d520, d520)) == Error::Unsupported, "head dim 520");
+        CHECK(sdpa::forward(d520, d520, d520).ok(), "head dim 520 runs (materialised path, as the reference's fallback)");
     }
 
     // ---- 3. forward == forward_train, taped backward vs the naive recompute; shapes of
@@ -993,6 +993,50 @@ int main() {
             cc.chunk_kv = 4;
             auto fd = autograd_v4::sdpa_forward(q, k, v, nullptr, cf), cd = autograd_v4::sdpa_forward(q, k, v, nullptr, cc);
             CHECK(fd.ok() && cd.ok() && max_diff(fd.value().first, cd.value().first) < 1e-3, "sdpa_v4_chunked_matches_full_with_dropout");
+        }
+    }
+
+    // ---- 14. what the fused kernels refuse goes through the materialised path, as forward_bf16_fallback and
+    //          attention_backward_recompute do in the reference (src/sdpa.rs:788-961, src/autograd.rs:801-848):
+    //          a head dim that is not a multiple of 8, one above 128 with a mask and a backward, one above 512
+    {
+        std::printf("[materialised fallback behind sdpa::forward_train and the backward arm]\n");
+        for (int D : {20, 264, 520}) {
+            const int B = 1, H = 2, N = 96;
+            auto hq = randn_bf16((size_t)B * H * N * D), hk = randn_bf16(hq.size()), hv = randn_bf16(hq.size()), hdo = randn_bf16(hq.size());
+            Tensor q = dev_bf16(hq, {B, H, N, D}), k = dev_bf16(hk, {B, H, N, D}), v = dev_bf16(hv, {B, H, N, D}), d_o = dev_bf16(hdo, {B, H, N, D});
+            // keep-mask [1,1,N,N]: lower triangle (what attention_impl builds for causal = true)
+            std::vector<uint8_t> keep((size_t)N * N);
+            for (int i = 0; i < N; ++i)
+                for (int j = 0; j < N; ++j) keep[(size_t)i * N + j] = j <= i;
+            Tensor mask = Tensor::from_host(keep.data(), {1, 1, N, N}, DType::U8).value();
+            q.requires_grad = true;
+            autograd::AutogradContext::set_recording(true);
+            auto o = sdpa::forward(q, k, v, &mask);
+            autograd::AutogradContext::set_recording(false);
+            CHECK(o.ok(), "forward_train at head dim %d", D);
+            if (!o.ok()) continue;
+            auto g = autograd::backward(o.value(), d_o);
+            CHECK(g.ok(), "backward at head dim %d", D);
+            if (!g.ok()) continue;
+            std::vector<float> ro, rdq, rdk, rdv;
+            for (int bh = 0; bh < B * H; ++bh) {
+                const size_t off = (size_t)bh * N * D;
+                Naive nv = naive_head(&hq[off], &hk[off], &hv[off], &hdo[off], N, N, D, 1.0f / std::sqrt((float)D), false, keep.data());
+                ro.insert(ro.end(), nv.o.begin(), nv.o.end());
+                rdq.insert(rdq.end(), nv.dq.begin(), nv.dq.end());
+                rdk.insert(rdk.end(), nv.dk.begin(), nv.dk.end());
+                rdv.insert(rdv.end(), nv.dv.begin(), nv.dv.end());
+            }
+            char name[64];
+            std::snprintf(name, sizeof name, "O (D=%d)", D);
+            compare(name, host_f32_of_bf16(o.value()), ro);
+            std::snprintf(name, sizeof name, "dQ (D=%d)", D);
+            compare(name, host_f32_of_bf16(g.value().dq), rdq);
+            std::snprintf(name, sizeof name, "dK (D=%d)", D);
+            compare(name, host_f32_of_bf16(g.value().dk), rdk);
+            std::snprintf(name, sizeof name, "dV (D=%d)", D);
+            compare(name, host_f32_of_bf16(g.value().dv), rdv);
         }
     }
 

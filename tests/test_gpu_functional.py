@@ -25,7 +25,7 @@ def _ref(q, k, v, mask=None, causal=False, bias=None, scale=None):
 
 
 @pytest.mark.parametrize("causal", [False, True])
-@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("D", [64, 128, 20, 264])      # 20 and 264 (with its mask and its backward): the materialised path
 def test_sdpa_forward_backward_vs_torch_fp32(causal, D):
     from flame_amd import functional as F
     torch.manual_seed(3)

@@ -159,3 +159,32 @@ def test_agrees_with_the_fused_kernels_and_takes_strided_views(oracle):
     capi.attn_fwd_materialised(bnhd(q), bnhd(k), bnhd(v), sc, causal=True, out=o_s)
     torch.cuda.synchronize()
     assert oracle.rel_l2(to_f32(o_s), to_f32(o)) < 2e-3
+
+
+def test_chunked_entry_point_of_the_reference_takes_any_head_dims(oracle):
+    """flame_sdpa_chunked_bf16 (src/ffi/cuda_ffi.h:98-115) has no head-dim rule in the reference (scalar kernels,
+    cuda/src/flame_sdpa_stub.cu:696-866): Dh = 264 with its bf16 keep-mask, and Dh = 36, run through the materialised
+    path in the library's own scratch."""
+    import ctypes
+    from flame_amd import capi
+    lib = capi.lib()
+    lib.flame_sdpa_chunked_bf16.restype = ctypes.c_int
+    p = lambda x: ctypes.c_void_p(x.data_ptr())
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for D, with_mask in ((264, True), (36, False)):
+        B, H, Q, K = 2, 2, 70, 110
+        q, k, v, _ = _case(8700 + D, B, H, Q, K, D)
+        keep = None
+        mask_bf16 = None
+        if with_mask:
+            keep = (W.normal_f32(8701, 0, B * Q * K).reshape(B, 1, Q, K) > -0.3).astype(np.uint8)
+            keep[..., 0] = 1
+            mask_bf16 = torch.from_numpy(keep.astype(np.float32)).to(torch.bfloat16).cuda()
+        out = torch.full((B, H, Q, D), float("nan"), dtype=torch.bfloat16, device="cuda")
+        qd, kd, vd = to_dev(q), to_dev(k), to_dev(v)
+        rc = lib.flame_sdpa_chunked_bf16(p(qd), p(kd), p(vd), B, H, Q, K, D, D, ctypes.c_float(0.07), 64, 0, 1,
+                                         p(mask_bf16) if with_mask else None, p(out), None, ctypes.c_uint64(0), stream)
+        assert rc == 0
+        torch.cuda.synchronize()
+        ro, _, ro32 = oracle.sdpa_fwd(q, k, v, 0.07, mask=keep, want_f32=True)
+        assert_close_bf16(oracle, f"O chunked entry point Dh={D}", to_f32(out), ro, ro32)
