@@ -5,7 +5,7 @@
 //
 // Arithmetic follows the reference's two kernels run back to back, including the bf16 rounding
 // between them:
-//   v[i]    = bf16( x[i] * rsqrt(mean_i(x^2) + eps) * w[i] )            (fused_rms_norm.cu:26-86)
+//   v[i]    = bf16( x[i] * (1 / sqrt(mean_i(x^2) + eps)) * w[i] )       (fused_rms_norm.cu:26-86)
 //   y[2p]   = bf16( v[2p] * cos[n,p] - v[2p+1] * sin[n,p] )             (bf16_ops.rs:361-394)
 //   y[2p+1] = bf16( v[2p] * sin[n,p] + v[2p+1] * cos[n,p] )
 //
@@ -93,12 +93,19 @@ __global__ __launch_bounds__(256) void prep_qk_kernel(const PrepParams p) {
             v[2 * i + 1] = bf16_hi(raw[k][i]);
         }
         if (p.norm) {
-            float ss = 0.f;
+            // The sum of squares is carried in fp64: squares of bf16 values are exact there and so, for any realistic
+            // spread of magnitudes, is their sum, which makes the mean independent of the summation order and equal to
+            // a CPU restatement's; it is rounded to fp32 once.  Square root and division are the correctly rounded
+            // fp32 ones (not the hardware's approximate reciprocal square root), so every step is IEEE arithmetic.
+            double ss = 0.0;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) ss = fmaf(v[i], v[i], ss);
+            for (int i = 0; i < 8; ++i) ss += (double)v[i] * (double)v[i];
 #pragma unroll
             for (int off = LPR / 2; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
-            const float rs = rsqrtf(ss / (float)D + p.eps);
+            const float ms = (float)(ss / (double)D);
+            // __builtin_sqrtf and the division operator are the correctly rounded ones under hipcc's default
+            // -fhip-fp32-correctly-rounded-divide-sqrt (the __fsqrt_rn intrinsic is the approximate native one here)
+            const float rs = 1.0f / __builtin_sqrtf(ms + p.eps);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
 #pragma clang fp contract(off)
