@@ -208,22 +208,29 @@ def profiling_read() -> dict:
     return {name: (kt.total_ms[i], kt.launches[i]) for i, name in enumerate(KERNEL_KINDS)}
 
 
+def sage_row_elems(D) -> int:
+    """Row length of the tensors the Sage quantiser writes for head dim D (64 up to D = 64, else 128)."""
+    return 64 if D <= 64 else 128
+
+
 def sage_quant(q, k, smooth_k=True, want_ks=False):
     """Per-block int8 quantisation of Q (128 rows) and mean-smoothed K (64 rows).
 
     Returns dict(qi8, ki8, sq, sk, kmean[, ks]): int8 [B,H,S,D], fp32 [B,H,nblk], fp32 [B,H,D]; with
-    want_ks also the smoothed bf16 K that was quantised."""
+    want_ks also the smoothed bf16 K that was quantised.  For head dims other than 64 and 128 the library writes
+    rows of sage_row_elems(D) elements, zero beyond D: the tensors returned are the [..., :D] views of those."""
     B, H, Sq, D = q.shape
     Sk = k.shape[2]
     dev = q.device
+    Dp = sage_row_elems(D)
     out = dict(
-        qi8=torch.empty((B, H, Sq, D), dtype=torch.int8, device=dev),
-        ki8=torch.empty((B, H, Sk, D), dtype=torch.int8, device=dev),
+        qi8=torch.empty((B, H, Sq, Dp), dtype=torch.int8, device=dev)[..., :D],
+        ki8=torch.empty((B, H, Sk, Dp), dtype=torch.int8, device=dev)[..., :D],
         sq=torch.empty((B, H, -(-Sq // 128)), dtype=torch.float32, device=dev),
         sk=torch.empty((B, H, -(-Sk // 64)), dtype=torch.float32, device=dev),
-        kmean=torch.empty((B, H, D), dtype=torch.float32, device=dev))
+        kmean=torch.empty((B, H, Dp), dtype=torch.float32, device=dev)[..., :D])
     if want_ks:
-        out["ks"] = torch.empty((B, H, Sk, D), dtype=torch.bfloat16, device=dev)
+        out["ks"] = torch.empty((B, H, Sk, Dp), dtype=torch.bfloat16, device=dev)[..., :D]
     rc = lib().flame_sage_quant_qk_int8_ks(
         _ptr(q), _ptr(k), B, H, Sq, Sk, D, _i64x4(q.stride()), _i64x4(k.stride()),
         ctypes.c_int64(0), ctypes.c_int64(0), int(bool(smooth_k)),

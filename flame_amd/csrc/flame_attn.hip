@@ -663,12 +663,14 @@ int flame_sage_quant_qk_int8_ks(const void* Q, const void* K, int B, int H, int 
     if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0) return FLAME_ATTN_ERR_INVALID;
     if (K_smoothed && !aligned16(K_smoothed)) return FLAME_ATTN_ERR_UNSUPPORTED;
     if (!Qi8 || !Ki8 || !q_scales || !k_scales || !k_mean) return FLAME_ATTN_ERR_INVALID;
-    if (D != 64 && D != 128) return FLAME_ATTN_ERR_UNSUPPORTED;
+    if (!head_dim_ok(D)) return FLAME_ATTN_ERR_UNSUPPORTED;
+    const int Dp = padded_head_dim(D);      // row length of everything written here (flame_sage_row_elems)
     int rc;
     if ((rc = check_view(Q, q_strides, q_off))) return rc;
     if ((rc = check_view(K, k_strides, k_off))) return rc;
     if (!aligned16(Qi8) || !aligned16(Ki8) || !aligned16(k_mean)) return FLAME_ATTN_ERR_UNSUPPORTED;
     SageQuantParams p;
+    p.d = D;
     p.q = static_cast<const uint16_t*>(Q) + q_off;
     p.k = static_cast<const uint16_t*>(K) + k_off;
     p.qs = mk(q_strides); p.ks = mk(k_strides);
@@ -691,20 +693,20 @@ int flame_sage_quant_qk_int8_ks(const void* Q, const void* K, int B, int H, int 
         const int n_chunks = (int)std::max<int64_t>(1, std::min<int64_t>(32, N_kv / 256));
         const int rows_per_chunk = (N_kv + n_chunks - 1) / n_chunks;
         if (N_kv < 256) {       // short: one workgroup per head sums all rows
-            if (D == 128) hipLaunchKernelGGL(sage_kmean_kernel<128>, dim3((unsigned)bh), dim3(512), 0, s, p);
+            if (Dp == 128) hipLaunchKernelGGL(sage_kmean_kernel<128>, dim3((unsigned)bh), dim3(512), 0, s, p);
             else hipLaunchKernelGGL(sage_kmean_kernel<64>, dim3((unsigned)bh), dim3(512), 0, s, p);
         } else {
         if (smooth_k) {
-            if (D == 128) hipLaunchKernelGGL(sage_kmean_partial_kernel<128>, dim3((unsigned)(bh * n_chunks)), dim3(512), 0, s, p, n_chunks, rows_per_chunk);
+            if (Dp == 128) hipLaunchKernelGGL(sage_kmean_partial_kernel<128>, dim3((unsigned)(bh * n_chunks)), dim3(512), 0, s, p, n_chunks, rows_per_chunk);
             else hipLaunchKernelGGL(sage_kmean_partial_kernel<64>, dim3((unsigned)(bh * n_chunks)), dim3(512), 0, s, p, n_chunks, rows_per_chunk);
         }
-        if (D == 128) hipLaunchKernelGGL(sage_kmean_final_kernel<128>, dim3((unsigned)bh), dim3(128), 0, s, p, n_chunks);
+        if (Dp == 128) hipLaunchKernelGGL(sage_kmean_final_kernel<128>, dim3((unsigned)bh), dim3(128), 0, s, p, n_chunks);
         else hipLaunchKernelGGL(sage_kmean_final_kernel<64>, dim3((unsigned)bh), dim3(64), 0, s, p, n_chunks);
         }
     }
     {
         ScopedKernelTimer t(FLAME_ATTN_KERNEL_SAGE_QUANT, s);
-        if (D == 128) hipLaunchKernelGGL(sage_quant_kernel<128>, dim3((unsigned)(bh * nblk)), dim3(256), 0, s, p);
+        if (Dp == 128) hipLaunchKernelGGL(sage_quant_kernel<128>, dim3((unsigned)(bh * nblk)), dim3(256), 0, s, p);
         else hipLaunchKernelGGL(sage_quant_kernel<64>, dim3((unsigned)(bh * nblk)), dim3(256), 0, s, p);
     }
     hipError_t e = hipGetLastError();
@@ -772,12 +774,14 @@ int flame_sage_attn_fwd_bias_int8(const void* Qi8, const void* Ki8, const void* 
     if (bias && bias_dtype != FLAME_ATTN_DTYPE_BF16 && bias_dtype != FLAME_ATTN_DTYPE_F32) return FLAME_ATTN_ERR_INVALID;
     if (!(scale > 0.f) || !isfinite(scale)) return FLAME_ATTN_ERR_INVALID;
     if (!Qi8 || !Ki8 || !q_scales || !k_scales) return FLAME_ATTN_ERR_INVALID;
-    if (D != 64 && D != 128) return FLAME_ATTN_ERR_UNSUPPORTED;
+    if (!head_dim_ok(D)) return FLAME_ATTN_ERR_UNSUPPORTED;
+    const int Dp = padded_head_dim(D);
     if (!aligned16(Qi8) || !aligned16(Ki8)) return FLAME_ATTN_ERR_UNSUPPORTED;
     int rc;
     if ((rc = check_view(V, v_strides, v_off))) return rc;
     if ((rc = check_view(O, o_strides, o_off))) return rc;
     SageFwdParams p;
+    p.d = D;
     p.qi8 = static_cast<const int8_t*>(Qi8);
     p.ki8 = static_cast<const int8_t*>(Ki8);
     p.sq = static_cast<const float*>(q_scales);
@@ -810,12 +814,12 @@ int flame_sage_attn_fwd_bias_int8(const void* Qi8, const void* Ki8, const void* 
         const int64_t rest = total256 % cus;
         const int64_t wide_count = rest <= cus / 2 ? total256 - rest : total256;
         if (2 * total256 > 0x7fffffff) return FLAME_ATTN_ERR_UNSUPPORTED;
-        rc = D == 128 ? launch_sage_fwd_wide<128>(p, s, wide_count) : launch_sage_fwd_wide<64>(p, s, wide_count);
+        rc = Dp == 128 ? launch_sage_fwd_wide<128>(p, s, wide_count) : launch_sage_fwd_wide<64>(p, s, wide_count);
         if (rc != FLAME_ATTN_OK || wide_count == total256) return rc;
         p.wg_base = (int)(2 * wide_count);
-        return D == 128 ? launch_sage_fwd<128, 4>(p, s, 2 * rest) : launch_sage_fwd<64, 4>(p, s, 2 * rest);
+        return Dp == 128 ? launch_sage_fwd<128, 4>(p, s, 2 * rest) : launch_sage_fwd<64, 4>(p, s, 2 * rest);
     }
-    if (D == 128) return launch_sage_fwd<128, 4>(p, s);
+    if (Dp == 128) return launch_sage_fwd<128, 4>(p, s);
     return launch_sage_fwd<64, 4>(p, s);
 }
 

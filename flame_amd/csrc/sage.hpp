@@ -27,6 +27,8 @@ struct SageQuantParams {
     const uint16_t* k;
     Strides qs, ks;
     int B, H, Sq, Sk;
+    int d;           // real head dim: a multiple of 8, at most the compiled D; every tensor written here has rows of D
+                     // elements, zero beyond d (zero channels change neither a block's maximum nor a logit)
     int smooth_k;
     float* kmean;    // [B*H, D]
     int8_t* qi8;     // [B*H, Sq, D]
@@ -52,7 +54,7 @@ __global__ __launch_bounds__(512) void sage_kmean_kernel(const SageQuantParams p
     for (int i = 0; i < 8; ++i) acc[i] = 0.0;
     if (p.smooth_k) {
         for (int row = rg; row < p.Sk; row += RG) {
-            const u32x4 w = *reinterpret_cast<const u32x4*>(kb + (int64_t)row * p.ks.n);
+            const u32x4 w = ldg16(kb + (int64_t)row * p.ks.n, chunk * 8 < p.d);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 acc[2 * i] += (double)bf16_lo(w[i]);
@@ -89,7 +91,7 @@ __global__ __launch_bounds__(512) void sage_kmean_partial_kernel(const SageQuant
 #pragma unroll
     for (int i = 0; i < 8; ++i) acc[i] = 0.0;
     for (int row = c * rows_per_chunk + rg; row < r_end; row += RG) {
-        const u32x4 w = *reinterpret_cast<const u32x4*>(kb + (int64_t)row * p.ks.n);
+        const u32x4 w = ldg16(kb + (int64_t)row * p.ks.n, chunk * 8 < p.d);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             acc[2 * i] += (double)bf16_lo(w[i]);
@@ -176,7 +178,7 @@ __global__ __launch_bounds__(256) void sage_quant_kernel(const SageQuantParams p
 #pragma unroll
     for (int i = 0; i < MAXC; ++i) {          // all loads first
         const int row = r0 + rsub + RPP * i;
-        raw[i] = ldg16(src + (int64_t)row * st.n + chunk * 8, row < S);
+        raw[i] = ldg16(src + (int64_t)row * st.n + chunk * 8, row < S && chunk * 8 < p.d);
     }
 #pragma unroll
     for (int i = 0; i < MAXC; ++i) {
@@ -253,6 +255,7 @@ struct SageFwdParams {
     float* lse;          // [B*H, Sq] or null
     Strides vs, os;
     int B, H, Sq, Sk;
+    int d;               // real head dim of V and O (a multiple of 8, at most the compiled D)
     float scale;
     const int32_t* kv_len;
     int causal;
@@ -356,7 +359,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sage_fwd_kernel(cons
 #pragma unroll
     for (int i = 0; i < NVD; ++i) {
         const int row = (wave * NVD + i) * RPV + v_row_in;
-        v_lane_off[i] = 2u * (uint32_t)(row * (int)p.vs.n + ((v_gran ^ swz<D>(row)) << 3));
+        v_lane_off[i] = 2u * (uint32_t)(row * (int)p.vs.n + (src_granule(v_gran ^ swz<D>(row), p.d) << 3));     // columns past d: a valid filler, their O is not stored
     }
     auto k_dst = [&](int t, int i) { return lds0 + (uint32_t)((t & 1) * T::STAGE_BYTES + (wave * NKD + i) * 1024); };
     auto v_dst = [&](int t, int i) { return lds0 + (uint32_t)((t & 1) * T::STAGE_BYTES + T::K_BYTES + (wave * NVD + i) * 1024); };
@@ -373,7 +376,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sage_fwd_kernel(cons
         for (int i = 0; i < NVD; ++i) {
             const int row = (wave * NVD + i) * RPV + v_row_in;
             const int key = min(t * BN + row, klimit - 1);
-            dma16(vbase + (int64_t)key * p.vs.n + ((v_gran ^ swz<D>(row)) << 3), v_dst(t, i));
+            dma16(vbase + (int64_t)key * p.vs.n + (src_granule(v_gran ^ swz<D>(row), p.d) << 3), v_dst(t, i));
         }
     };
     auto issue_full_kv = [&](int tk, int tv) {               // K^ tile tk and V tile tv, both full
@@ -640,7 +643,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void sage_fwd_kernel(cons
             for (int g = 0; g < 4; ++g) {
                 const f32x16& a = oacc[db];
                 u32x2 w = {pack_bf16(a[4 * g] * inv, a[4 * g + 1] * inv), pack_bf16(a[4 * g + 2] * inv, a[4 * g + 3] * inv)};
-                *reinterpret_cast<u32x2*>(orow + 32 * db + 8 * g + 4 * h) = w;
+                if (32 * db + 8 * g + 4 * h < p.d) *reinterpret_cast<u32x2*>(orow + 32 * db + 8 * g + 4 * h) = w;
             }
         if (p.lse && h == 0) p.lse[(int64_t)bh * p.Sq + row] = l > 0.f ? (m_run + log2_fast(l)) * kLn2 : -INFINITY;
     }
@@ -741,7 +744,7 @@ __global__ __launch_bounds__(256) void sage_fwd_wide_kernel(const SageFwdParams 
 #pragma unroll
     for (int i = 0; i < NVD; ++i) {
         const int row = (wave * NVD + i) * RPV + v_row_in;
-        v_lane_off[i] = 2u * (uint32_t)(row * (int)p.vs.n + ((v_gran ^ swz<D>(row)) << 3));
+        v_lane_off[i] = 2u * (uint32_t)(row * (int)p.vs.n + (src_granule(v_gran ^ swz<D>(row), p.d) << 3));     // columns past d: a valid filler, their O is not stored
     }
     auto k_dst = [&](int stg, int i) { return lds0 + (uint32_t)(stg * T::STAGE_BYTES + (wave * NKD + i) * 1024); };
     auto v_dst = [&](int stg, int i) { return lds0 + (uint32_t)(stg * T::STAGE_BYTES + T::K_BYTES + (wave * NVD + i) * 1024); };
@@ -1055,7 +1058,7 @@ __global__ __launch_bounds__(256) void sage_fwd_wide_kernel(const SageFwdParams 
                     const f32x16& a = oacc[qb][db];
                     u32x2 w = {pack_bf16(a[4 * g] * inv, a[4 * g + 1] * inv),
                                pack_bf16(a[4 * g + 2] * inv, a[4 * g + 3] * inv)};
-                    *reinterpret_cast<u32x2*>(orow + 32 * db + 8 * g + 4 * h) = w;
+                    if (32 * db + 8 * g + 4 * h < p.d) *reinterpret_cast<u32x2*>(orow + 32 * db + 8 * g + 4 * h) = w;
                 }
             if (p.lse && h == 0) p.lse[(int64_t)bh * p.Sq + row] = l > 0.f ? (m_run[qb] + log2_fast(l)) * kLn2 : -INFINITY;
         }

@@ -136,6 +136,12 @@ class Tensor {
         }
         return t;
     }
+    // view of the first n elements of the last dimension (no copy)
+    Tensor narrow_last(int64_t n) const {
+        Tensor t = *this;
+        t.shape_.back() = n;
+        return t;
+    }
     Tensor reshape_contiguous(std::vector<int64_t> shape) const {
         Tensor t = *this;
         t.shape_ = std::move(shape);
@@ -1171,18 +1177,20 @@ class SageAttention {
             for (int i = 0; i < 4; ++i) bst[i] = (bs[i] == 1 && full[i] != 1) ? 0 : bias->strides()[i];
         }
         const int64_t nqb = (d.Sq + 127) / 128, nkb = (d.Sk + 63) / 64;
-        auto qi8 = Tensor::empty({d.B, d.H, d.Sq, d.D}, DType::I8);
-        auto ki8 = Tensor::empty({d.B, d.H, d.Sk, d.D}, DType::I8);
+        // the quantiser writes rows of 64 (head dims up to 64) or 128 elements, zero beyond the head dim
+        const int64_t dr = d.D <= 64 ? 64 : 128;
+        auto qi8 = Tensor::empty({d.B, d.H, d.Sq, dr}, DType::I8);
+        auto ki8 = Tensor::empty({d.B, d.H, d.Sk, dr}, DType::I8);
         auto sq = Tensor::empty({d.B, d.H, nqb}, DType::F32);
         auto sk = Tensor::empty({d.B, d.H, nkb}, DType::F32);
-        auto km = Tensor::empty({d.B, d.H, d.D}, DType::F32);
+        auto km = Tensor::empty({d.B, d.H, dr}, DType::F32);
         auto o = Tensor::empty({d.B, d.H, d.Sq, d.D}, DType::BF16);
         if (!qi8.ok() || !ki8.ok() || !sq.ok() || !sk.ok() || !km.ok() || !o.ok()) return cuda_error("hipMalloc", -1);
         Tensor ks;
         if (save) {
-            auto t = Tensor::empty({d.B, d.H, d.Sk, d.D}, DType::BF16);
+            auto t = Tensor::empty({d.B, d.H, d.Sk, dr}, DType::BF16);
             if (!t.ok()) return t.error();
-            ks = t.value();
+            ks = t.value().narrow_last(d.D);
         }
         int rc = flame_sage_quant_qk_int8_ks(q.base(), k.base(), d.B, d.H, d.Sq, d.Sk, d.D, q.strides().data(), k.strides().data(),
                                              q.offset(), k.offset(), smooth_k_ ? 1 : 0, qi8.value().data(), ki8.value().data(),

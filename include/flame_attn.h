@@ -263,15 +263,17 @@ int flame_attn_bwd_materialised_bf16(const void* Q, const void* K, const void* V
 /* k_mean[b,h,c] = float(fp64 sum_t K[b,h,t,c] / N_kv) (0 when smooth_k == 0);
  * Ks = bf16(float(K) - k_mean);  per 128-row block of Q and per 64-row block of Ks:
  * scale = absmax / 127 (IEEE fp32 division), code = clamp(rint(x / scale), -128, 127), scale 0 -> 0.
- * Outputs are contiguous: Qi8 [B,H,N_q,D], Ki8 [B,H,N_kv,D] int8; q_scales [B,H,ceil(N_q/128)],
- * k_scales [B,H,ceil(N_kv/64)], k_mean [B,H,D] fp32. */
+ * Outputs are contiguous: Qi8 [B,H,N_q,Dr], Ki8 [B,H,N_kv,Dr] int8; q_scales [B,H,ceil(N_q/128)],
+ * k_scales [B,H,ceil(N_kv/64)], k_mean [B,H,Dr] fp32.  D: any multiple of 8 up to 128.  Dr is the row length the
+ * forward below reads: 64 for D <= 64, else 128 (so Dr = D for the two compiled sizes); elements D .. Dr-1 of
+ * every row are written as zero, which changes neither a block's maximum nor a logit. */
 int flame_sage_quant_qk_int8(const void* Q, const void* K, int B, int H, int N_q, int N_kv, int D,
                              const int64_t* q_strides, const int64_t* k_strides, int64_t q_off, int64_t k_off,
                              int smooth_k, void* Qi8, void* Ki8, void* q_scales, void* k_scales, void* k_mean,
                              void* stream);
 
 /* The same, and also writes the smoothed K that was quantised, Ks = bf16(float(K) - k_mean), contiguous bf16
- * [B,H,N_kv,D] (K_smoothed may be null).  The reference saves this tensor for the backward of its Sage
+ * [B,H,N_kv,Dr] (K_smoothed may be null; a backward reads it as a [B,H,N_kv,D] view with row stride Dr).  The reference saves this tensor for the backward of its Sage
  * operator (src/sage_attention.rs:138-144, key_smoothed); see flame_host.hpp sage_attention_backward. */
 int flame_sage_quant_qk_int8_ks(const void* Q, const void* K, int B, int H, int N_q, int N_kv, int D,
                                 const int64_t* q_strides, const int64_t* k_strides, int64_t q_off, int64_t k_off,
@@ -279,7 +281,8 @@ int flame_sage_quant_qk_int8_ks(const void* Q, const void* K, int B, int H, int 
                                 void* K_smoothed, void* stream);
 
 /* S = float(int32 Q^ K^^T) * sq * sk * scale on int8 MFMA, online softmax fp32, P bf16, O = P V
- * on bf16 MFMA.  LSE may be null. */
+ * on bf16 MFMA.  LSE may be null.  Qi8 / Ki8 as the quantiser above wrote them (rows of Dr elements);
+ * V and O are bf16 views of head dim D. */
 int flame_sage_attn_fwd_int8(const void* Qi8, const void* Ki8, const void* q_scales, const void* k_scales,
                              const void* V, void* O, void* LSE, int B, int H, int N_q, int N_kv, int D,
                              float scale, const int64_t* v_strides, const int64_t* o_strides,

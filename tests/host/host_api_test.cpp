@@ -469,6 +469,48 @@ int main() {
         }
     }
 
+    // ---- 6b. SageAttention at a head dim that is not a compiled size (96: rows of 128 behind the operator, the smoothed
+    //          key a strided view of them): cosine against the bf16 path, backward against the oracle
+    {
+        std::printf("[sage, head dim 96]\n");
+        const int B = 1, H = 2, N = 200, D = 96;
+        auto hq = randn_bf16((size_t)B * H * N * D), hk = randn_bf16(hq.size()), hv = randn_bf16(hq.size()), hdo = randn_bf16(hq.size());
+        for (size_t i = 7; i < hk.size(); i += D) hk[i] = f2bf(bf2f(hk[i]) * 3.0f + 1.5f);
+        Tensor q = dev_bf16(hq, {B, H, N, D}), k = dev_bf16(hk, {B, H, N, D}), v = dev_bf16(hv, {B, H, N, D});
+        Tensor d_o = dev_bf16(hdo, {B, H, N, D});
+        auto sv = SageAttention().forward_saving(q, k, v);
+        auto o2 = sdpa::forward(q, k, v);
+        CHECK(sv.ok() && o2.ok(), "sage/bf16 forward failed at head dim 96");
+        if (sv.ok() && o2.ok()) {
+            auto a = host_f32_of_bf16(sv.value().output), b2 = host_f32_of_bf16(o2.value());
+            double dot = 0, na = 0, nb = 0;
+            for (size_t i = 0; i < a.size(); ++i) { dot += (double)a[i] * b2[i]; na += (double)a[i] * a[i]; nb += (double)b2[i] * b2[i]; }
+            const double c = dot / std::sqrt(na * nb);
+            std::printf("  cosine sage vs bf16 = %.6f\n", c);
+            CHECK(c >= 0.999, "sage cosine %.6f", c);
+            const Tensor& ks = sv.value().key_smoothed;
+            CHECK(ks.shape().back() == D && ks.strides()[2] == 128, "smoothed key is not a [.., 96] view of rows of 128");
+            std::vector<uint16_t> hks((size_t)B * H * N * D);
+            CHECK(hipMemcpy2D(hks.data(), (size_t)D * 2, ks.data(), 128 * 2, (size_t)D * 2, (size_t)B * H * N, hipMemcpyDeviceToHost) == hipSuccess,
+                  "copy of the smoothed key failed");
+            auto g = sage_attention_backward(sv.value(), d_o);
+            CHECK(g.ok(), "sage_attention_backward failed at head dim 96");
+            if (g.ok()) {
+                std::vector<float> rdq, rdk, rdv;
+                for (int bh = 0; bh < B * H; ++bh) {
+                    const size_t off = (size_t)bh * N * D;
+                    Naive nv = naive_head(&hq[off], &hks[off], &hv[off], &hdo[off], N, N, D, 1.0f / std::sqrt((float)D), false, nullptr);
+                    rdq.insert(rdq.end(), nv.dq.begin(), nv.dq.end());
+                    rdk.insert(rdk.end(), nv.dk.begin(), nv.dk.end());
+                    rdv.insert(rdv.end(), nv.dv.begin(), nv.dv.end());
+                }
+                compare("sage d96 dQ", host_f32_of_bf16(g.value().dq), rdq);
+                compare("sage d96 dK", host_f32_of_bf16(g.value().dk), rdk);
+                compare("sage d96 dV", host_f32_of_bf16(g.value().dv), rdv);
+            }
+        }
+    }
+
     // ---- 7. input preparation: fused RMS-norm + RoPE + [B,N,H,D]->[B,H,N,D] equals the three separate calls,
     //         and the rotation matches the scalar formula of the reference test (src/tests/attention_tests.rs:8-34)
     {

@@ -175,6 +175,72 @@ def test_sage_large_problems_take_256_query_workgroups(oracle, B, H, Sq, Sk, D):
     _check_sage_fwd(oracle, w, qz, ref, v, o_bf16)
 
 
+def _rows_with_padding(t, D):
+    """The [.., Dr] rows behind a [.., :D] view returned by capi.sage_quant."""
+    from flame_amd import capi
+    shape = tuple(t.shape[:-1]) + (capi.sage_row_elems(D),)
+    return torch.as_strided(t, shape, t.stride(), t.storage_offset())
+
+
+@pytest.mark.parametrize("D", [8, 40, 72, 96, 120])
+def test_sage_other_head_dims(oracle, D):
+    """Head dims that are not one of the two compiled sizes run on the next one with zero channels: codes, scales and
+    channel means bit-exact on the D real channels, zero in the padding of every row the quantiser writes, the
+    smoothed K bit-exact, and the int8 forward against the oracle on the same operands: plain, causal, with key
+    lengths, and with an additive bias."""
+    from flame_amd import capi
+    B, H, Sq, Sk = 2, 2, 200, 328
+    w = W.config5(B=B, H=H, S=Sk, D=D)
+    qbits = w.q[:, :, :Sq].copy()
+    wq = W.Workload("sage_d", qbits, w.k, w.v, None, w.scale)
+    print(f"[sage] head dim {D}", flush=True)
+    q, k, v = to_dev(qbits), to_dev(w.k), to_dev(w.v)
+    for smooth in (True, False):
+        got, ref = _check_quant(oracle, wq, smooth=smooth)
+        for name in ("qi8", "ki8", "kmean"):
+            assert torch.all(_rows_with_padding(got[name], D)[..., D:] == 0), f"{name} padding"
+    qz = capi.sage_quant(q, k, want_ks=True)
+    ref = oracle.sage_quant(qbits, w.k)
+    assert np.array_equal(qz["ks"].cpu().contiguous().view(torch.int16).numpy().view(np.uint16), ref["ks"]), "smoothed K bits"
+    assert torch.all(_rows_with_padding(qz["ks"], D)[..., D:].view(torch.int16) == 0)
+    o_bf16, _ = capi.attn_fwd(q, k, v, w.scale)
+    _check_sage_fwd(oracle, wq, qz, ref, v, o_bf16)
+    o_c, _ = capi.attn_fwd(q, k, v, w.scale, causal=True)
+    _check_sage_fwd(oracle, wq, qz, ref, v, o_c, causal=True)
+    kv_len = [Sk, 77]
+    o_l, _ = capi.attn_fwd(q, k, v, w.scale, kv_len=torch.tensor(kv_len, dtype=torch.int32, device="cuda"))
+    _check_sage_fwd(oracle, wq, qz, ref, v, o_l, kv_len=kv_len)
+    bias = (np.random.default_rng(5).normal(size=(1, H, Sq, Sk)) * 2).astype(np.float32)
+    bias[..., 3::7] = -np.inf
+    o, lse = capi.sage_fwd(qz, v, w.scale, bias=torch.from_numpy(bias).cuda(), want_lse=True)
+    torch.cuda.synchronize()
+    ro, rlse, ro32 = oracle.sage_fwd(ref["qi8"], ref["ki8"], ref["sq"], ref["sk"], w.v, w.scale, bias=bias, want_f32=True)
+    assert_close_bf16(oracle, f"O_sage bias D={D}", to_f32(o), ro, ro32)
+    assert oracle.max_abs(lse.cpu().numpy().reshape(rlse.shape), rlse) <= TOL_LSE
+
+
+def test_sage_head_dim_96_on_256_query_workgroups(oracle):
+    """D = 96 on a problem that fills the chip (264 workgroups of 256 queries, the last 8 cut into 16): every head
+    against the oracle."""
+    from flame_amd import capi
+    B, H, Sq, Sk, D = 1, 33, 2048, 320, 96
+    w = W.Workload("sage_wide_d96", W.f32_to_bf16_bits(W.normal_f32(71, 0, B * H * Sq * D).reshape(B, H, Sq, D)),
+                   W.f32_to_bf16_bits(W.normal_f32(71, 1, B * H * Sk * D).reshape(B, H, Sk, D)),
+                   W.f32_to_bf16_bits(W.normal_f32(71, 2, B * H * Sk * D).reshape(B, H, Sk, D)), None, 1.0 / np.sqrt(D))
+    q, k, v = (to_dev(t) for t in (w.q, w.k, w.v))
+    qz, ref = _check_quant(oracle, w, smooth=True)
+    o_bf16, _ = capi.attn_fwd(q, k, v, w.scale)
+    _check_sage_fwd(oracle, w, qz, ref, v, o_bf16)
+
+
+def test_sage_refuses_head_dims_it_cannot_pad():
+    from flame_amd import capi
+    for D in (136, 20):
+        q = torch.zeros((1, 1, 64, D), dtype=torch.bfloat16, device="cuda")
+        with pytest.raises(capi.FlameAttnError):
+            capi.sage_quant(q, q)
+
+
 def test_sage_additive_bias_and_smoothed_k_output(oracle):
     """The attention_mask of the reference's Sage operator is added to the scores (src/sage_attention.rs:126-131):
     fp32 and bf16 biases, per head and broadcast, with excluded positions and a row that loses every key; and the
