@@ -448,8 +448,9 @@ def _bias_strides(bias, B, H, Sq, Sk):
     return _i64x4(st)
 
 
-def attn_fwd_materialised(q, k, v, scale, causal=False, kv_len=None, mask=None, bias=None, want_lse=True, out=None, workspace=None):
-    """O, LSE = flame_attn_fwd_materialised_bf16(...): any head dim, a value head dim of its own, mask and bias."""
+def attn_fwd_materialised(q, k, v, scale, causal=False, kv_len=None, mask=None, bias=None, want_lse=True, out=None, workspace=None,
+                          dropout_p=0.0, dropout_seed=0, draw_chunk_q=0, draw_chunk_kv=0):
+    """O, LSE = flame_attn_fwd_materialised_bf16(...): any head dim, a value head dim of its own, mask, bias, dropout."""
     B, H, Sq, D = q.shape
     Sk, Dv = k.shape[2], v.shape[3]
     o = torch.empty((B, H, Sq, Dv), dtype=torch.bfloat16, device=q.device) if out is None else out
@@ -462,13 +463,15 @@ def attn_fwd_materialised(q, k, v, scale, causal=False, kv_len=None, mask=None, 
         *(ctypes.c_int64(0) for _ in range(5)),
         int(bool(causal)), _ptr(kv_len), _ptr(mask), _mask_strides(mask, B, H, Sq, Sk),
         _ptr(bias), 1 if (bias is not None and bias.dtype == torch.float32) else 0, _bias_strides(bias, B, H, Sq, Sk),
+        ctypes.c_float(dropout_p), ctypes.c_uint64(dropout_seed & (2 ** 64 - 1)), int(draw_chunk_q), int(draw_chunk_kv),
         _ptr(workspace), ctypes.c_size_t(workspace.numel()), _stream())
     if rc != 0:
         raise FlameAttnError("flame_attn_fwd_materialised_bf16", rc)
     return o, lse
 
 
-def attn_bwd_materialised(q, k, v, o, do, lse, scale, causal=False, kv_len=None, mask=None, workspace=None, grads=None):
+def attn_bwd_materialised(q, k, v, o, do, lse, scale, causal=False, kv_len=None, mask=None, workspace=None, grads=None,
+                          dropout_p=0.0, dropout_seed=0, draw_chunk_q=0, draw_chunk_kv=0):
     """dQ, dK, dV = flame_attn_bwd_materialised_bf16(...)."""
     B, H, Sq, D = q.shape
     Sk, Dv = k.shape[2], v.shape[3]
@@ -484,6 +487,7 @@ def attn_bwd_materialised(q, k, v, o, do, lse, scale, causal=False, kv_len=None,
         _i64x4(do.stride()), _i64x4(dq.stride()), _i64x4(dk.stride()), _i64x4(dv.stride()),
         *(ctypes.c_int64(0) for _ in range(9)),
         int(bool(causal)), _ptr(kv_len), _ptr(mask), _mask_strides(mask, B, H, Sq, Sk),
+        ctypes.c_float(dropout_p), ctypes.c_uint64(dropout_seed & (2 ** 64 - 1)), int(draw_chunk_q), int(draw_chunk_kv),
         _ptr(workspace), ctypes.c_size_t(workspace.numel()), _stream())
     if rc != 0:
         raise FlameAttnError("flame_attn_bwd_materialised_bf16", rc)

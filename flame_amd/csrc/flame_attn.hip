@@ -1019,7 +1019,8 @@ static int mat_fwd_impl(const void* Q, const void* K, const void* V, void* O, vo
                         int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off, int64_t lse_off,
                         int causal, const int32_t* kv_len, const uint8_t* keep_mask, const int64_t* mask_strides,
                         const void* bias, int bias_dtype, const int64_t* bias_strides,
-                        void* workspace, size_t workspace_bytes, void* stream, int mask_mode);
+                        void* workspace, size_t workspace_bytes, void* stream, int mask_mode,
+                        float dropout_p = 0.f, uint64_t dropout_seed = 0, int draw_cq = 0, int draw_ck = 0);
 static FwdScratch library_scratch() {
     FwdScratch sc;
     sc.library = true;
@@ -1860,7 +1861,8 @@ static int mat_fwd_impl(const void* Q, const void* K, const void* V, void* O, vo
                         int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off, int64_t lse_off,
                         int causal, const int32_t* kv_len, const uint8_t* keep_mask, const int64_t* mask_strides,
                         const void* bias, int bias_dtype, const int64_t* bias_strides,
-                        void* workspace, size_t workspace_bytes, void* stream, int mask_mode) {
+                        void* workspace, size_t workspace_bytes, void* stream, int mask_mode,
+                        float dropout_p, uint64_t dropout_seed, int draw_cq, int draw_ck) {
     if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0 || Dv <= 0) return FLAME_ATTN_ERR_INVALID;
     if (!(scale > 0.f) || !isfinite(scale)) return FLAME_ATTN_ERR_INVALID;
     int rc;
@@ -1888,6 +1890,10 @@ static int mat_fwd_impl(const void* Q, const void* K, const void* V, void* O, vo
     rp.H = H; rp.Sq = N_q; rp.Sk = N_kv;
     rp.from_lse = 0;
     mat_fill_mask(rp.m, causal, kv_len, keep_mask, mask_strides, bias, bias_dtype, bias_strides, mask_mode);
+    if (dropout_p != 0.f) {
+        if (!set_dropout(rp.m, dropout_p, dropout_seed, draw_cq, draw_ck, N_q, N_kv)) return FLAME_ATTN_ERR_INVALID;
+        rp.dropout = 1;
+    }
     for (int q0 = 0; q0 < N_q; q0 += plan.tq) {
         const int tq = std::min(plan.tq, N_q - q0);
         const int64_t band = (int64_t)tq * N_kv;
@@ -1917,10 +1923,11 @@ int flame_attn_fwd_materialised_bf16(const void* Q, const void* K, const void* V
                                      int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off, int64_t lse_off,
                                      int causal, const int32_t* kv_len, const uint8_t* keep_mask, const int64_t* mask_strides,
                                      const void* bias, int bias_dtype, const int64_t* bias_strides,
+                                     float dropout_p, uint64_t dropout_seed, int draw_chunk_q, int draw_chunk_kv,
                                      void* workspace, size_t workspace_bytes, void* stream) {
     return mat_fwd_impl(Q, K, V, O, LSE, B, H, N_q, N_kv, D, Dv, scale, q_strides, k_strides, v_strides, o_strides, q_off, k_off,
                         v_off, o_off, lse_off, causal, kv_len, keep_mask, mask_strides, bias, bias_dtype, bias_strides, workspace,
-                        workspace_bytes, stream, kMaskU8);
+                        workspace_bytes, stream, kMaskU8, dropout_p, dropout_seed, draw_chunk_q, draw_chunk_kv);
 }
 
 int flame_attn_bwd_materialised_bf16(const void* Q, const void* K, const void* V, const void* O, const void* dO,
@@ -1932,6 +1939,7 @@ int flame_attn_bwd_materialised_bf16(const void* Q, const void* K, const void* V
                                      int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off, int64_t do_off,
                                      int64_t lse_off, int64_t dq_off, int64_t dk_off, int64_t dv_off,
                                      int causal, const int32_t* kv_len, const uint8_t* keep_mask, const int64_t* mask_strides,
+                                     float dropout_p, uint64_t dropout_seed, int draw_chunk_q, int draw_chunk_kv,
                                      void* workspace, size_t workspace_bytes, void* stream) {
     if (B <= 0 || H <= 0 || N_q <= 0 || N_kv <= 0 || D <= 0 || Dv <= 0) return FLAME_ATTN_ERR_INVALID;
     if (!(scale > 0.f) || !isfinite(scale) || !LSE) return FLAME_ATTN_ERR_INVALID;
@@ -1974,6 +1982,8 @@ int flame_attn_bwd_materialised_bf16(const void* Q, const void* K, const void* V
     rp.H = H; rp.Sq = N_q; rp.Sk = N_kv;
     rp.from_lse = 1;
     mat_fill_mask(rp.m, causal, kv_len, keep_mask, mask_strides, nullptr, FLAME_ATTN_DTYPE_F32, nullptr);
+    MaskArgs drop = rp.m;            // drop_thr = 0: no dropout
+    if (dropout_p != 0.f && !set_dropout(drop, dropout_p, dropout_seed, draw_chunk_q, draw_chunk_kv, N_q, N_kv)) return FLAME_ATTN_ERR_INVALID;
     uint16_t* ds = reinterpret_cast<uint16_t*>(plan.ds);
     float* acc_dk = reinterpret_cast<float*>(plan.accum);
     float* acc_dv = plan.accum ? acc_dk + (size_t)B * H * N_kv * D : nullptr;
@@ -1998,7 +2008,7 @@ int flame_attn_bwd_materialised_bf16(const void* Q, const void* K, const void* V
         {
             const int64_t n = (int64_t)B * H * band;
             hipLaunchKernelGGL(mat_ds_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, rp.probs, rp.scores, delta, ds, n, N_kv,
-                               tq, N_q, q0);
+                               tq, N_q, q0, drop);
         }
         for (int b = 0; b < B; ++b) {
             const uint16_t* pb = rp.probs + (int64_t)b * H * band;

@@ -18,6 +18,7 @@ struct MatRowsParams {
     int H, Sq, Sk, tq, q0;  // the band holds query rows [q0, q0 + tq) of every (batch, head)
     MaskArgs m;
     int from_lse;           // 0: forward (row max, sum, LSE, P); 1: backward (P = exp(s - LSE) under the same exclusions)
+    int dropout = 0;        // forward only: P is stored dropped and rescaled (the backward drops it in mat_ds_kernel)
 };
 
 // s for key j of query row qi of (b, hh), or -inf when the pair is excluded
@@ -36,7 +37,8 @@ __device__ __forceinline__ float mat_logit(const MatRowsParams& p, const uint8_t
 
 // One workgroup per query row of the band.  Forward: exclusions and bias, row maximum and sum (two passes over the
 // row, which sits in L2), LSE = max + ln(sum), P = exp(s - LSE) as bf16; a row without an attended key gets
-// LSE = -inf and P = 0.  Backward: P = exp(s - LSE) from the saved LSE.
+// LSE = -inf and P = 0; with dropout P is stored as P * f, f = 0 or 1 / (1 - p) per element (drop_factor_at), the
+// LSE being that of the undropped row.  Backward: P = exp(s - LSE) from the saved LSE, undropped.
 __global__ __launch_bounds__(256) void mat_rows_kernel(const MatRowsParams p) {
     const int row = blockIdx.x;                      // over [BH, tq]
     const int bh = row / p.tq, i = row % p.tq;
@@ -77,6 +79,7 @@ __global__ __launch_bounds__(256) void mat_rows_kernel(const MatRowsParams p) {
     for (int j = tid; j < p.Sk; j += 256) {
         float pr = 0.f;
         if (lse != -INFINITY) pr = expf(mat_logit(p, mbase, bias_base, b, qi, j, klimit, s[j]) - lse);      // exp(-inf) = 0
+        if (p.dropout) pr *= drop_factor_at(p.m, (uint32_t)bh, (uint32_t)qi, (uint32_t)j, (uint32_t)p.Sq, (uint32_t)p.Sk);
         out[j] = (uint16_t)(pack_bf16(pr, 0.f) & 0xffffu);
     }
 }
@@ -105,16 +108,24 @@ __global__ __launch_bounds__(256) void mat_delta_kernel(const MatDeltaParams p) 
     if (lane == 0) p.delta[row] = acc;
 }
 
-// dS = P * (dP - delta) as bf16, element-wise over the band; delta is per query row
-__global__ __launch_bounds__(256) void mat_ds_kernel(const uint16_t* __restrict__ probs, const float* __restrict__ dp,
+// dS = P * (dP - delta) as bf16, element-wise over the band; delta is per query row.  With dropout (drop.drop_thr
+// != 0): dP is the product with the dropped V weights, dS = P * (f dP - delta), and P is overwritten by P * f, the
+// weights that multiplied V in the forward, for the dV product that follows.
+__global__ __launch_bounds__(256) void mat_ds_kernel(uint16_t* __restrict__ probs, const float* __restrict__ dp,
                                                      const float* __restrict__ delta, uint16_t* __restrict__ ds, int64_t n, int Sk,
-                                                     int tq, int Sq, int q0) {
+                                                     int tq, int Sq, int q0, const MaskArgs drop) {
     const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (e >= n) return;
     const int64_t row = e / Sk;
     const int bh = (int)(row / tq), i = (int)(row % tq);
     const float pr = __builtin_bit_cast(float, (uint32_t)probs[e] << 16);
-    const float v = pr * (dp[e] - delta[(size_t)bh * Sq + q0 + i]);
+    float g = dp[e];
+    if (drop.drop_thr != 0) {
+        const float f = drop_factor_at(drop, (uint32_t)bh, (uint32_t)(q0 + i), (uint32_t)(e % Sk), (uint32_t)Sq, (uint32_t)Sk);
+        g *= f;
+        probs[e] = (uint16_t)(pack_bf16(pr * f, 0.f) & 0xffffu);
+    }
+    const float v = pr * (g - delta[(size_t)bh * Sq + q0 + i]);
     ds[e] = (uint16_t)(pack_bf16(v, 0.f) & 0xffffu);
 }
 

@@ -248,21 +248,21 @@ inline Result<FwdOut> run_forward(const Tensor& q, const Tensor& k, const Tensor
         mst = pm.value().second;
     }
     const float sc = scale.value_or(1.0f / std::sqrt((float)d.D));
+    int rc;
     if (dropout_p != 0.f) {
-        const int rc = flame_attn_fwd_dropout_tiled_bf16(
+        rc = flame_attn_fwd_dropout_tiled_bf16(
             q.base(), k.base(), v.base(), o.value().base(), want_stats ? stats.base() : nullptr, d.B, d.H, d.Sq, d.Sk, d.D, sc,
             q.strides().data(), k.strides().data(), v.strides().data(), o.value().strides().data(), q.offset(), k.offset(),
             v.offset(), 0, 0, causal ? 1 : 0, nullptr, mask ? static_cast<const uint8_t*>(m8.data()) : nullptr,
             mask ? mst.data() : nullptr, dropout_p, dropout_seed, draw_chunk_q, draw_chunk_kv, nullptr);
-        if (rc == FLAME_ATTN_ERR_UNSUPPORTED) return unsupported("flame_attn_fwd_dropout_tiled_bf16: head dim or layout not built");
-        if (rc != 0) return cuda_error("flame_attn_fwd_dropout_tiled_bf16", rc);
-        return FwdOut{o.value(), stats};
+        if (rc != 0 && rc != FLAME_ATTN_ERR_UNSUPPORTED) return cuda_error("flame_attn_fwd_dropout_tiled_bf16", rc);
+    } else {
+        rc = flame_attn_fwd_bf16(q.base(), k.base(), v.base(), o.value().base(), want_stats ? stats.base() : nullptr,
+                                 d.B, d.H, d.Sq, d.Sk, d.D, sc, q.strides().data(), k.strides().data(),
+                                 v.strides().data(), o.value().strides().data(), q.offset(), k.offset(), v.offset(), 0, 0,
+                                 causal ? 1 : 0, nullptr, mask ? static_cast<const uint8_t*>(m8.data()) : nullptr,
+                                 mask ? mst.data() : nullptr, nullptr /* default stream, as the reference */);
     }
-    const int rc = flame_attn_fwd_bf16(q.base(), k.base(), v.base(), o.value().base(), want_stats ? stats.base() : nullptr,
-                                       d.B, d.H, d.Sq, d.Sk, d.D, sc, q.strides().data(), k.strides().data(),
-                                       v.strides().data(), o.value().strides().data(), q.offset(), k.offset(), v.offset(), 0, 0,
-                                       causal ? 1 : 0, nullptr, mask ? static_cast<const uint8_t*>(m8.data()) : nullptr,
-                                       mask ? mst.data() : nullptr, nullptr /* default stream, as the reference */);
     if (rc == FLAME_ATTN_ERR_UNSUPPORTED) {
         // forward_bf16's last branch (src/sdpa.rs:543-587 -> forward_bf16_fallback, :788-961): whatever the fused
         // kernels do not serve (a head dim that is not a multiple of 8 or lies above 512, a mask above 128) goes
@@ -274,7 +274,7 @@ inline Result<FwdOut> run_forward(const Tensor& q, const Tensor& k, const Tensor
             q.base(), k.base(), v.base(), o.value().base(), want_stats ? stats.base() : nullptr, d.B, d.H, d.Sq, d.Sk, d.D, d.D, sc,
             q.strides().data(), k.strides().data(), v.strides().data(), o.value().strides().data(), q.offset(), k.offset(), v.offset(),
             0, 0, causal ? 1 : 0, nullptr, mask ? static_cast<const uint8_t*>(m8.data()) : nullptr, mask ? mst.data() : nullptr, nullptr,
-            FLAME_ATTN_DTYPE_F32, nullptr, ws.value().data(), wsb, nullptr);
+            FLAME_ATTN_DTYPE_F32, nullptr, dropout_p, dropout_seed, draw_chunk_q, draw_chunk_kv, ws.value().data(), wsb, nullptr);
         if (rm == FLAME_ATTN_ERR_UNSUPPORTED) return unsupported("flame_attn_fwd_materialised_bf16: layout not served (or rocBLAS missing)");
         if (rm != 0) return cuda_error("flame_attn_fwd_materialised_bf16", rm);
         return FwdOut{o.value(), stats};
@@ -374,8 +374,9 @@ inline Result<AttentionGrads> flash_attention_backward(const FlashAttentionNode&
         m8 = pm.value().first;
         mst = pm.value().second;
     }
+    int rc;
     if (n.dropout_p != 0.f) {
-        const int rc = flame_attn_bwd_dropout_tiled_bf16(
+        rc = flame_attn_bwd_dropout_tiled_bf16(
             n.query.base(), n.key.base(), n.value.base(), n.output.base(), g.base(), n.stats.base(), dq.value().base(),
             dk.value().base(), dv.value().base(), B, H, Sq, Sk, D, n.scale, n.query.strides().data(), n.key.strides().data(),
             n.value.strides().data(), n.output.strides().data(), g.strides().data(), dq.value().strides().data(),
@@ -383,11 +384,9 @@ inline Result<AttentionGrads> flash_attention_backward(const FlashAttentionNode&
             n.output.offset(), g.offset(), 0, 0, 0, 0, n.causal ? 1 : 0, nullptr,
             n.mask ? static_cast<const uint8_t*>(m8.data()) : nullptr, n.mask ? mst.data() : nullptr, n.dropout_p, n.dropout_seed,
             n.draw_chunk_q, n.draw_chunk_kv, ws.value().data(), wsb, nullptr);
-        if (rc == FLAME_ATTN_ERR_UNSUPPORTED) return unsupported("flame_attn_bwd_dropout_tiled_bf16: head dim or layout not built");
-        if (rc != 0) return cuda_error("flame_attn_bwd_dropout_tiled_bf16", rc);
-        return AttentionGrads{dq.value(), dk.value(), dv.value()};
-    }
-    const int rc = flame_attn_bwd_bf16(
+        if (rc != 0 && rc != FLAME_ATTN_ERR_UNSUPPORTED) return cuda_error("flame_attn_bwd_dropout_tiled_bf16", rc);
+    } else {
+        rc = flame_attn_bwd_bf16(
         n.query.base(), n.key.base(), n.value.base(), n.output.base(), g.base(), n.stats.base(), dq.value().base(),
         dk.value().base(), dv.value().base(), B, H, Sq, Sk, D, n.scale, n.query.strides().data(), n.key.strides().data(),
         n.value.strides().data(), n.output.strides().data(), g.strides().data(), dq.value().strides().data(),
@@ -395,6 +394,7 @@ inline Result<AttentionGrads> flash_attention_backward(const FlashAttentionNode&
         n.output.offset(), g.offset(), 0, 0, 0, 0, n.causal ? 1 : 0, nullptr,
         n.mask ? static_cast<const uint8_t*>(m8.data()) : nullptr, n.mask ? mst.data() : nullptr, ws.value().data(), wsb,
         nullptr);
+    }
     if (rc == FLAME_ATTN_ERR_UNSUPPORTED) {
         // attention_backward_recompute (src/autograd.rs:801-848): the materialising backward for what the fused one
         // does not serve, here one band of query rows at a time
@@ -407,7 +407,8 @@ inline Result<AttentionGrads> flash_attention_backward(const FlashAttentionNode&
             n.value.strides().data(), n.output.strides().data(), g.strides().data(), dq.value().strides().data(),
             dk.value().strides().data(), dv.value().strides().data(), n.query.offset(), n.key.offset(), n.value.offset(),
             n.output.offset(), g.offset(), 0, 0, 0, 0, n.causal ? 1 : 0, nullptr,
-            n.mask ? static_cast<const uint8_t*>(m8.data()) : nullptr, n.mask ? mst.data() : nullptr, wm.value().data(), wsm, nullptr);
+            n.mask ? static_cast<const uint8_t*>(m8.data()) : nullptr, n.mask ? mst.data() : nullptr, n.dropout_p, n.dropout_seed,
+            n.draw_chunk_q, n.draw_chunk_kv, wm.value().data(), wsm, nullptr);
         if (rm == FLAME_ATTN_ERR_UNSUPPORTED) return unsupported("flame_attn_bwd_materialised_bf16: layout not served (or rocBLAS missing)");
         if (rm != 0) return cuda_error("flame_attn_bwd_materialised_bf16", rm);
         return AttentionGrads{dq.value(), dk.value(), dv.value()};

@@ -233,7 +233,9 @@ int flame_attn_bwd_bf16_noalloc(const void* Q, const void* K, const void* V, con
  * the size with which the whole problem is one band or, for large problems, bands of about 512 MiB; any workspace
  * that holds 16 query rows is accepted (more bands).  The first call creates a rocBLAS handle per device, which
  * allocates: these entry points are not meant for graph capture.  Several times slower than the fused kernels
- * where both apply.
+ * where both apply.  dropout_p, dropout_seed, draw_chunk_q, draw_chunk_kv: dropout of the probabilities as in
+ * flame_attn_fwd_dropout_bf16 / flame_attn_fwd_dropout_tiled_bf16 (dropout_p = 0: none; draw_chunk_* = 0: one draw
+ * over the whole tensor), the same kept set, the backward with the values the forward had.
  * ---------------------------------------------------------------------------------------------- */
 size_t flame_attn_materialised_workspace_bytes(int B, int H, int N_q, int N_kv, int D, int Dv, int backward);
 int flame_attn_fwd_materialised_bf16(const void* Q, const void* K, const void* V, void* O, void* LSE,
@@ -243,6 +245,7 @@ int flame_attn_fwd_materialised_bf16(const void* Q, const void* K, const void* V
                                      int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off, int64_t lse_off,
                                      int causal, const int32_t* kv_len, const uint8_t* keep_mask, const int64_t* mask_strides,
                                      const void* bias, int bias_dtype, const int64_t* bias_strides,
+                                     float dropout_p, uint64_t dropout_seed, int draw_chunk_q, int draw_chunk_kv,
                                      void* workspace, size_t workspace_bytes, void* stream);
 int flame_attn_bwd_materialised_bf16(const void* Q, const void* K, const void* V, const void* O, const void* dO,
                                      const void* LSE, void* dQ, void* dK, void* dV,
@@ -253,6 +256,7 @@ int flame_attn_bwd_materialised_bf16(const void* Q, const void* K, const void* V
                                      int64_t q_off, int64_t k_off, int64_t v_off, int64_t o_off, int64_t do_off,
                                      int64_t lse_off, int64_t dq_off, int64_t dk_off, int64_t dv_off,
                                      int causal, const int32_t* kv_len, const uint8_t* keep_mask, const int64_t* mask_strides,
+                                     float dropout_p, uint64_t dropout_seed, int draw_chunk_q, int draw_chunk_kv,
                                      void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------------------------------

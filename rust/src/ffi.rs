@@ -171,6 +171,7 @@ extern "C" {
         k_strides: *const i64, v_strides: *const i64, o_strides: *const i64, q_off: i64, k_off: i64, v_off: i64,
         o_off: i64, lse_off: i64, causal: c_int, kv_len: *const i32, keep_mask: *const u8,
         mask_strides: *const i64, bias: *const c_void, bias_dtype: c_int, bias_strides: *const i64,
+        dropout_p: f32, dropout_seed: u64, draw_chunk_q: c_int, draw_chunk_kv: c_int,
         workspace: *mut c_void, workspace_bytes: usize, stream: *mut c_void
     ) -> c_int;
     pub fn flame_attn_bwd_materialised_bf16(
@@ -180,8 +181,8 @@ extern "C" {
         v_strides: *const i64, o_strides: *const i64, do_strides: *const i64, dq_strides: *const i64,
         dk_strides: *const i64, dv_strides: *const i64, q_off: i64, k_off: i64, v_off: i64, o_off: i64,
         do_off: i64, lse_off: i64, dq_off: i64, dk_off: i64, dv_off: i64, causal: c_int, kv_len: *const i32,
-        keep_mask: *const u8, mask_strides: *const i64, workspace: *mut c_void, workspace_bytes: usize,
-        stream: *mut c_void
+        keep_mask: *const u8, mask_strides: *const i64, dropout_p: f32, dropout_seed: u64, draw_chunk_q: c_int,
+        draw_chunk_kv: c_int, workspace: *mut c_void, workspace_bytes: usize, stream: *mut c_void
     ) -> c_int;
     pub fn flame_sage_quant_qk_int8(
         q: *const c_void, k: *const c_void, b: c_int, h: c_int, n_q: c_int, n_kv: c_int, d: c_int,

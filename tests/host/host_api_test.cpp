@@ -1070,6 +1070,32 @@ int main() {
                 rdk.insert(rdk.end(), nv.dk.begin(), nv.dk.end());
                 rdv.insert(rdv.end(), nv.dv.begin(), nv.dv.end());
             }
+            if (D == 264) {     // the v4 operator with dropout at this head dim: same seed same bits, undropped log-sum-exp, finite gradients
+                autograd_v4::SdpaConfig dc;
+                dc.dropout_p = 0.25f;
+                dc.dropout_seed = 0x2545F4914F6CDD1Dull;
+                autograd_v4::SdpaConfig pc;
+                auto d1 = autograd_v4::sdpa_forward(q, k, v, nullptr, dc), d2 = autograd_v4::sdpa_forward(q, k, v, nullptr, dc);
+                auto f0 = autograd_v4::sdpa_forward(q, k, v, nullptr, pc);
+                CHECK(d1.ok() && d2.ok() && f0.ok(), "v4 sdpa_forward with dropout at head dim %d", D);
+                if (d1.ok() && d2.ok() && f0.ok()) {
+                    CHECK(host_bits_of_bf16(d1.value().first) == host_bits_of_bf16(d2.value().first), "same seed, different output (D=264)");
+                    CHECK(host_bits_of_bf16(d1.value().first) != host_bits_of_bf16(f0.value().first), "dropout changed nothing (D=264)");
+                    std::vector<float> l1((size_t)d1.value().second.lse.numel()), l0(l1.size());
+                    d1.value().second.lse.to_host(l1.data());
+                    f0.value().second.lse.to_host(l0.data());
+                    // (the undropped run takes the fused forward at this head dim, another summation order)
+                    double worst = 0;
+                    for (size_t i = 0; i < l1.size(); ++i) worst = std::max(worst, (double)std::fabs(l1[i] - l0[i]));
+                    CHECK(worst <= 1e-4, "the log-sum-exp is that of the undropped softmax (D=264): differs by %.3e", worst);
+                    auto g1 = autograd_v4::sdpa_backward(d1.value().second, d_o), g0 = autograd_v4::sdpa_backward(f0.value().second, d_o);
+                    CHECK(g1.ok() && g0.ok(), "v4 sdpa_backward with dropout at head dim %d", D);
+                    if (g1.ok() && g0.ok()) {
+                        CHECK(host_bits_of_bf16(std::get<2>(g1.value())) != host_bits_of_bf16(std::get<2>(g0.value())), "dropout left dV unchanged (D=264)");
+                        for (float x : host_f32_of_bf16(std::get<0>(g1.value()))) if (!std::isfinite(x)) { CHECK(false, "dQ with dropout not finite (D=264)"); break; }
+                    }
+                }
+            }
             char name[64];
             std::snprintf(name, sizeof name, "O (D=%d)", D);
             compare(name, host_f32_of_bf16(o.value()), ro);

@@ -188,3 +188,78 @@ def test_chunked_entry_point_of_the_reference_takes_any_head_dims(oracle):
         torch.cuda.synchronize()
         ro, _, ro32 = oracle.sdpa_fwd(q, k, v, 0.07, mask=keep, want_f32=True)
         assert_close_bf16(oracle, f"O chunked entry point Dh={D}", to_f32(out), ro, ro32)
+
+
+SEED = 0x2545F4914F6CDD1D
+
+
+@pytest.mark.parametrize("B,H,Sq,Sk,D,causal,kv_len,with_mask,chunks,bands", [
+    (2, 2, 200, 328, 136, False, None, False, (0, 0), False),
+    (1, 3, 192, 256, 264, True, None, False, (0, 0), True),        # several bands of query rows
+    (2, 2, 130, 77, 20, False, [77, 40], False, (0, 0), False),    # a head dim that is not a multiple of 8
+    (1, 2, 160, 200, 320, False, None, True, (0, 0), False),       # keep-mask first, the draw on what is left
+    (1, 2, 200, 328, 136, False, None, False, (64, 128), False),   # the kept set of the reference's chunked operator
+])
+def test_dropout_where_the_fused_kernels_refuse(oracle, B, H, Sq, Sk, D, causal, kv_len, with_mask, chunks, bands):
+    """Dropout of the probabilities through the materialised path (head dims the fused dropout kernels do not take):
+    the reference's kept set (src/rng/mod.rs:14-24 over the whole tensor, or tile by tile for its chunked operator),
+    O, the log-sum-exp of the undropped softmax, and the backward on the oracle's own O and LSE, to the usual bar."""
+    from flame_amd import capi
+    print(f"[materialised dropout] {B}x{H} Sq={Sq} Sk={Sk} D={D} causal={causal} kv_len={kv_len} mask={with_mask} chunks={chunks} "
+          f"bands={bands}", flush=True)
+    q, k, v, do = _case(880 + D, B, H, Sq, Sk, D)
+    scale = 1.0 / math.sqrt(D)
+    cq, ck = chunks
+    p = float(np.quantile(oracle.dropout_uniforms(B, H, Sq, Sk, SEED, cq, ck), 0.3))
+    kept = float(oracle.dropout_keep_mask(B, H, Sq, Sk, p, SEED, cq, ck).mean())
+    assert 0.3 < kept < 0.95, kept
+    keep = None
+    if with_mask:
+        keep = (W.normal_f32(881, 0, B * H * Sq * Sk).reshape(B, H, Sq, Sk) > -0.4).astype(np.uint8)
+        keep[..., 0] = 1
+    kvl = None if kv_len is None else torch.tensor(kv_len, dtype=torch.int32, device="cuda")
+    kvl_np = None if kv_len is None else np.array(kv_len, np.int32)
+    mask = None if keep is None else torch.from_numpy(keep).cuda()
+    ws_f = ws_b = None
+    if bands:          # room for 64 (forward) and 48 (backward) query rows per band, and the fp32 sums of dK and dV
+        rows_bytes = ((B * H * Sq * 4 + 255) // 256) * 256
+        accum = ((B * H * Sk * 2 * D * 4 + 255) // 256) * 256
+        ws_f = torch.empty(B * H * Sk * 6 * 64 + 1024, dtype=torch.uint8, device="cuda")
+        ws_b = torch.empty(rows_bytes + accum + B * H * Sk * 8 * 48 + 1024, dtype=torch.uint8, device="cuda")
+    dq_, dk_, dv_, ddo = (to_dev(x) for x in (q, k, v, do))
+    kw = dict(causal=causal, kv_len=kvl, mask=mask, dropout_p=p, dropout_seed=SEED, draw_chunk_q=cq, draw_chunk_kv=ck)
+    o, lse = capi.attn_fwd_materialised(dq_, dk_, dv_, scale, workspace=ws_f, **kw)
+    o_plain, lse_plain = capi.attn_fwd_materialised(dq_, dk_, dv_, scale, causal=causal, kv_len=kvl, mask=mask)
+    torch.cuda.synchronize()
+    okw = dict(causal=causal, kv_len=kvl_np, mask=keep, want_f32=True, chunk_q=cq, chunk_kv=ck)
+    ro, rlse, ro32 = oracle.sdpa_fwd_dropout(q, k, v, scale, p, SEED, **okw)
+    assert_close_bf16(oracle, "O", to_f32(o), ro, ro32)
+    glse = lse.cpu().numpy().reshape(rlse.shape)
+    fin = np.isfinite(rlse)
+    assert np.array_equal(np.isfinite(glse), fin) and oracle.max_abs(glse[fin], rlse[fin]) <= TOL_LSE
+    assert torch.equal(lse, lse_plain)                     # the undropped softmax's
+    assert oracle.rel_l2(to_f32(o_plain), ro32) > 0.05     # teeth: the plain forward is far from this oracle
+    # the kept set itself: O is zero in exactly ... cannot be read off O at these head dims; the backward, which draws
+    # again, must agree with the oracle's on identical inputs
+    ref = oracle.sdpa_bwd_dropout(q, k, v, ro, do, scale, p, SEED, **okw)
+    lse_ref = torch.from_numpy(rlse.reshape(B * H, Sq)).cuda()
+    g = capi.attn_bwd_materialised(dq_, dk_, dv_, to_dev(ro), ddo, lse_ref, scale, workspace=ws_b, **kw)
+    torch.cuda.synchronize()
+    for i, name in enumerate(("dQ", "dK", "dV")):
+        assert_close_bf16(oracle, name, to_f32(g[i]), ref[i], ref[i + 3])
+
+
+def test_dropout_kept_set_bit_exact_at_head_dim_136(oracle):
+    """V = identity over the first 136 keys (Sk = 136 = Dv, head dim 136) turns O into the dropped probabilities
+    themselves: zero exactly where the reference's generator drops, non-zero elsewhere."""
+    from flame_amd import capi
+    B, H, Sq, Sk, D = 1, 2, 64, 136, 136
+    q, k, _, _ = _case(890, B, H, Sq, Sk, D, mul=0.25)          # small logits: every probability is far from zero
+    v = np.zeros((B, H, Sk, D), np.float32)
+    v[..., np.arange(Sk), np.arange(D)] = 1.0
+    p = float(np.quantile(oracle.dropout_uniforms(B, H, Sq, Sk, SEED), 0.4))
+    o, _ = capi.attn_fwd_materialised(to_dev(q), to_dev(k), to_dev(W.f32_to_bf16_bits(v)), 1.0 / math.sqrt(D), dropout_p=p,
+                                      dropout_seed=SEED)
+    torch.cuda.synchronize()
+    kept = oracle.dropout_keep_mask(B, H, Sq, Sk, p, SEED)
+    assert np.array_equal(to_f32(o) != 0.0, kept)
