@@ -69,6 +69,66 @@ __device__ __forceinline__ void mfma32_vgpr(f32x16& acc, bf16x8 a, bf16x8 b) {
 __device__ __forceinline__ void mfma32_vgpr_settle(f32x16& acc) {
     asm volatile("s_nop 11" : "+v"(acc));
 }
+// ---------------------------------------------------------------------------------------------
+// Fixed accumulation registers.  Inline assembly can only name a physical register by a literal, so the two
+// register maps are written out once, here, and every statement below is generated from them; each row is checked
+// against the rule it follows at compile time, so a wrong number does not build.
+//   B slots:    slot s holds a 16-byte MFMA operand in a[128 + 4 s : 131 + 4 s]
+//   acc tuples: tuple t holds a 32x32 fp32 accumulator block in a[16 t : 16 t + 15]
+// ---------------------------------------------------------------------------------------------
+#define FATTN_B_SLOTS(X) \
+    X(0, 128, 129, 130, 131) \
+    X(1, 132, 133, 134, 135) \
+    X(2, 136, 137, 138, 139) \
+    X(3, 140, 141, 142, 143) \
+    X(4, 144, 145, 146, 147) \
+    X(5, 148, 149, 150, 151) \
+    X(6, 152, 153, 154, 155) \
+    X(7, 156, 157, 158, 159) \
+    X(8, 160, 161, 162, 163) \
+    X(9, 164, 165, 166, 167) \
+    X(10, 168, 169, 170, 171) \
+    X(11, 172, 173, 174, 175) \
+    X(12, 176, 177, 178, 179) \
+    X(13, 180, 181, 182, 183) \
+    X(14, 184, 185, 186, 187) \
+    X(15, 188, 189, 190, 191) \
+    X(16, 192, 193, 194, 195) \
+    X(17, 196, 197, 198, 199) \
+    X(18, 200, 201, 202, 203) \
+    X(19, 204, 205, 206, 207) \
+    X(20, 208, 209, 210, 211) \
+    X(21, 212, 213, 214, 215) \
+    X(22, 216, 217, 218, 219) \
+    X(23, 220, 221, 222, 223) \
+    X(24, 224, 225, 226, 227) \
+    X(25, 228, 229, 230, 231) \
+    X(26, 232, 233, 234, 235) \
+    X(27, 236, 237, 238, 239) \
+    X(28, 240, 241, 242, 243) \
+    X(29, 244, 245, 246, 247) \
+    X(30, 248, 249, 250, 251) \
+    X(31, 252, 253, 254, 255)
+#define FATTN_ACC_TUPLES(X) \
+    X(0, 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15) \
+    X(1, 16, 17, 18, 19, 20, 21, 22, 23, 24, 25, 26, 27, 28, 29, 30, 31) \
+    X(2, 32, 33, 34, 35, 36, 37, 38, 39, 40, 41, 42, 43, 44, 45, 46, 47) \
+    X(3, 48, 49, 50, 51, 52, 53, 54, 55, 56, 57, 58, 59, 60, 61, 62, 63) \
+    X(4, 64, 65, 66, 67, 68, 69, 70, 71, 72, 73, 74, 75, 76, 77, 78, 79) \
+    X(5, 80, 81, 82, 83, 84, 85, 86, 87, 88, 89, 90, 91, 92, 93, 94, 95) \
+    X(6, 96, 97, 98, 99, 100, 101, 102, 103, 104, 105, 106, 107, 108, 109, 110, 111) \
+    X(7, 112, 113, 114, 115, 116, 117, 118, 119, 120, 121, 122, 123, 124, 125, 126, 127)
+#define FATTN_STR_(x) #x
+#define FATTN_STR(x) FATTN_STR_(x)
+#define FATTN_AREG(r) "a" FATTN_STR(r)
+#define FATTN_ARANGE(lo, hi) "{a[" FATTN_STR(lo) ":" FATTN_STR(hi) "]}"
+#define FATTN_CHECK_B_SLOT(I, R0, R1, R2, R3) \
+    static_assert(R0 == 128 + 4 * I && R1 == R0 + 1 && R2 == R0 + 2 && R3 == R0 + 3, "row of FATTN_B_SLOTS")
+#define FATTN_CHECK_ACC_TUPLE(I, R0, R1, R2, R3, R4, R5, R6, R7, R8, R9, R10, R11, R12, R13, R14, R15)                          \
+    static_assert(R0 == 16 * I && R1 == R0 + 1 && R2 == R0 + 2 && R3 == R0 + 3 && R4 == R0 + 4 && R5 == R0 + 5 && R6 == R0 + 6 && \
+                  R7 == R0 + 7 && R8 == R0 + 8 && R9 == R0 + 9 && R10 == R0 + 10 && R11 == R0 + 11 && R12 == R0 + 12 &&           \
+                  R13 == R0 + 13 && R14 == R0 + 14 && R15 == R0 + 15, "row of FATTN_ACC_TUPLES")
+
 // The same with the B operand pinned to accumulation registers a[128 + 4 SLOT : 131 + 4 SLOT], for a
 // kernel whose 32 resident B fragments must stay put there (left to itself the register allocator
 // homes some of them in architectural registers and copies them over before every use).
@@ -76,44 +136,14 @@ __device__ __forceinline__ void mfma32_vgpr_settle(f32x16& acc) {
 template <int SLOT, int MODE>
 __device__ __forceinline__ void mfma32_vgpr_bpinned(f32x16& acc, bf16x8 a, bf16x8 b, const f32x16& c) {
     static_assert(SLOT >= 0 && SLOT < 32, "32 pinned fragments");
-#define FATTN_PIN(I, R)                                                                                                  \
-    if constexpr (SLOT == I) {                                                                                           \
-        if constexpr (MODE == 0) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(acc) : "v"(a), R(b));     \
-        if constexpr (MODE == 1) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), R(b));     \
-        if constexpr (MODE == 2) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %3" : "=&v"(acc) : "v"(a), R(b), "v"(c)); \
+#define FATTN_PIN(I, R0, R1, R2, R3)                                                                                                        \
+    FATTN_CHECK_B_SLOT(I, R0, R1, R2, R3);                                                                                                  \
+    if constexpr (SLOT == I) {                                                                                                              \
+        if constexpr (MODE == 0) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(acc) : "v"(a), FATTN_ARANGE(R0, R3)(b));     \
+        if constexpr (MODE == 1) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), FATTN_ARANGE(R0, R3)(b));     \
+        if constexpr (MODE == 2) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %3" : "=&v"(acc) : "v"(a), FATTN_ARANGE(R0, R3)(b), "v"(c)); \
     }
-    FATTN_PIN(0, "{a[128:131]}")
-    FATTN_PIN(1, "{a[132:135]}")
-    FATTN_PIN(2, "{a[136:139]}")
-    FATTN_PIN(3, "{a[140:143]}")
-    FATTN_PIN(4, "{a[144:147]}")
-    FATTN_PIN(5, "{a[148:151]}")
-    FATTN_PIN(6, "{a[152:155]}")
-    FATTN_PIN(7, "{a[156:159]}")
-    FATTN_PIN(8, "{a[160:163]}")
-    FATTN_PIN(9, "{a[164:167]}")
-    FATTN_PIN(10, "{a[168:171]}")
-    FATTN_PIN(11, "{a[172:175]}")
-    FATTN_PIN(12, "{a[176:179]}")
-    FATTN_PIN(13, "{a[180:183]}")
-    FATTN_PIN(14, "{a[184:187]}")
-    FATTN_PIN(15, "{a[188:191]}")
-    FATTN_PIN(16, "{a[192:195]}")
-    FATTN_PIN(17, "{a[196:199]}")
-    FATTN_PIN(18, "{a[200:203]}")
-    FATTN_PIN(19, "{a[204:207]}")
-    FATTN_PIN(20, "{a[208:211]}")
-    FATTN_PIN(21, "{a[212:215]}")
-    FATTN_PIN(22, "{a[216:219]}")
-    FATTN_PIN(23, "{a[220:223]}")
-    FATTN_PIN(24, "{a[224:227]}")
-    FATTN_PIN(25, "{a[228:231]}")
-    FATTN_PIN(26, "{a[232:235]}")
-    FATTN_PIN(27, "{a[236:239]}")
-    FATTN_PIN(28, "{a[240:243]}")
-    FATTN_PIN(29, "{a[244:247]}")
-    FATTN_PIN(30, "{a[248:251]}")
-    FATTN_PIN(31, "{a[252:255]}")
+    FATTN_B_SLOTS(FATTN_PIN)
 #undef FATTN_PIN
 }
 
@@ -123,44 +153,13 @@ __device__ __forceinline__ void mfma32_vgpr_bpinned(f32x16& acc, bf16x8 a, bf16x
 template <int SLOT, int MODE>
 __device__ __forceinline__ void mfma32i8_vgpr_bpinned(i32x16& acc, u32x4 a, bf16x8 b, const i32x16& c) {
     static_assert(SLOT >= 0 && SLOT < 32, "32 pinned fragments");
-#define FATTN_PIN(I, R)                                                                                                  \
-    if constexpr (SLOT == I) {                                                                                           \
-        if constexpr (MODE == 0) asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, 0" : "=&v"(acc) : "v"(a), R(b));     \
-        if constexpr (MODE == 1) asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0" : "+v"(acc) : "v"(a), R(b));     \
-        if constexpr (MODE == 2) asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %3" : "=&v"(acc) : "v"(a), R(b), "v"(c)); \
+#define FATTN_PIN(I, R0, R1, R2, R3)                                                                                                      \
+    if constexpr (SLOT == I) {                                                                                                            \
+        if constexpr (MODE == 0) asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, 0" : "=&v"(acc) : "v"(a), FATTN_ARANGE(R0, R3)(b));     \
+        if constexpr (MODE == 1) asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0" : "+v"(acc) : "v"(a), FATTN_ARANGE(R0, R3)(b));     \
+        if constexpr (MODE == 2) asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %3" : "=&v"(acc) : "v"(a), FATTN_ARANGE(R0, R3)(b), "v"(c)); \
     }
-    FATTN_PIN(0, "{a[128:131]}")
-    FATTN_PIN(1, "{a[132:135]}")
-    FATTN_PIN(2, "{a[136:139]}")
-    FATTN_PIN(3, "{a[140:143]}")
-    FATTN_PIN(4, "{a[144:147]}")
-    FATTN_PIN(5, "{a[148:151]}")
-    FATTN_PIN(6, "{a[152:155]}")
-    FATTN_PIN(7, "{a[156:159]}")
-    FATTN_PIN(8, "{a[160:163]}")
-    FATTN_PIN(9, "{a[164:167]}")
-    FATTN_PIN(10, "{a[168:171]}")
-    FATTN_PIN(11, "{a[172:175]}")
-    FATTN_PIN(12, "{a[176:179]}")
-    FATTN_PIN(13, "{a[180:183]}")
-    FATTN_PIN(14, "{a[184:187]}")
-    FATTN_PIN(15, "{a[188:191]}")
-    FATTN_PIN(16, "{a[192:195]}")
-    FATTN_PIN(17, "{a[196:199]}")
-    FATTN_PIN(18, "{a[200:203]}")
-    FATTN_PIN(19, "{a[204:207]}")
-    FATTN_PIN(20, "{a[208:211]}")
-    FATTN_PIN(21, "{a[212:215]}")
-    FATTN_PIN(22, "{a[216:219]}")
-    FATTN_PIN(23, "{a[220:223]}")
-    FATTN_PIN(24, "{a[224:227]}")
-    FATTN_PIN(25, "{a[228:231]}")
-    FATTN_PIN(26, "{a[232:235]}")
-    FATTN_PIN(27, "{a[236:239]}")
-    FATTN_PIN(28, "{a[240:243]}")
-    FATTN_PIN(29, "{a[244:247]}")
-    FATTN_PIN(30, "{a[248:251]}")
-    FATTN_PIN(31, "{a[252:255]}")
+    FATTN_B_SLOTS(FATTN_PIN)
 #undef FATTN_PIN
 }
 
@@ -168,43 +167,12 @@ __device__ __forceinline__ void mfma32i8_vgpr_bpinned(i32x16& acc, u32x4 a, bf16
 template <int SLOT>
 __device__ __forceinline__ bf16x8 pin_b_fragment(u32x4 w) {
     bf16x8 out;
-#define FATTN_PIN(I, C, R0, R1, R2, R3)                                                                        \
-    if constexpr (SLOT == I)                                                                                   \
-        asm volatile("v_accvgpr_write_b32 " R0 ", %1\n\tv_accvgpr_write_b32 " R1 ", %2\n\t"                    \
-                     "v_accvgpr_write_b32 " R2 ", %3\n\tv_accvgpr_write_b32 " R3 ", %4"                         \
-                     : C(out) : "v"(w[0]), "v"(w[1]), "v"(w[2]), "v"(w[3]));
-    FATTN_PIN(0, "={a[128:131]}", "a128", "a129", "a130", "a131")
-    FATTN_PIN(1, "={a[132:135]}", "a132", "a133", "a134", "a135")
-    FATTN_PIN(2, "={a[136:139]}", "a136", "a137", "a138", "a139")
-    FATTN_PIN(3, "={a[140:143]}", "a140", "a141", "a142", "a143")
-    FATTN_PIN(4, "={a[144:147]}", "a144", "a145", "a146", "a147")
-    FATTN_PIN(5, "={a[148:151]}", "a148", "a149", "a150", "a151")
-    FATTN_PIN(6, "={a[152:155]}", "a152", "a153", "a154", "a155")
-    FATTN_PIN(7, "={a[156:159]}", "a156", "a157", "a158", "a159")
-    FATTN_PIN(8, "={a[160:163]}", "a160", "a161", "a162", "a163")
-    FATTN_PIN(9, "={a[164:167]}", "a164", "a165", "a166", "a167")
-    FATTN_PIN(10, "={a[168:171]}", "a168", "a169", "a170", "a171")
-    FATTN_PIN(11, "={a[172:175]}", "a172", "a173", "a174", "a175")
-    FATTN_PIN(12, "={a[176:179]}", "a176", "a177", "a178", "a179")
-    FATTN_PIN(13, "={a[180:183]}", "a180", "a181", "a182", "a183")
-    FATTN_PIN(14, "={a[184:187]}", "a184", "a185", "a186", "a187")
-    FATTN_PIN(15, "={a[188:191]}", "a188", "a189", "a190", "a191")
-    FATTN_PIN(16, "={a[192:195]}", "a192", "a193", "a194", "a195")
-    FATTN_PIN(17, "={a[196:199]}", "a196", "a197", "a198", "a199")
-    FATTN_PIN(18, "={a[200:203]}", "a200", "a201", "a202", "a203")
-    FATTN_PIN(19, "={a[204:207]}", "a204", "a205", "a206", "a207")
-    FATTN_PIN(20, "={a[208:211]}", "a208", "a209", "a210", "a211")
-    FATTN_PIN(21, "={a[212:215]}", "a212", "a213", "a214", "a215")
-    FATTN_PIN(22, "={a[216:219]}", "a216", "a217", "a218", "a219")
-    FATTN_PIN(23, "={a[220:223]}", "a220", "a221", "a222", "a223")
-    FATTN_PIN(24, "={a[224:227]}", "a224", "a225", "a226", "a227")
-    FATTN_PIN(25, "={a[228:231]}", "a228", "a229", "a230", "a231")
-    FATTN_PIN(26, "={a[232:235]}", "a232", "a233", "a234", "a235")
-    FATTN_PIN(27, "={a[236:239]}", "a236", "a237", "a238", "a239")
-    FATTN_PIN(28, "={a[240:243]}", "a240", "a241", "a242", "a243")
-    FATTN_PIN(29, "={a[244:247]}", "a244", "a245", "a246", "a247")
-    FATTN_PIN(30, "={a[248:251]}", "a248", "a249", "a250", "a251")
-    FATTN_PIN(31, "={a[252:255]}", "a252", "a253", "a254", "a255")
+#define FATTN_PIN(I, R0, R1, R2, R3)                                                                                       \
+    if constexpr (SLOT == I)                                                                                               \
+        asm volatile("v_accvgpr_write_b32 " FATTN_AREG(R0) ", %1\n\tv_accvgpr_write_b32 " FATTN_AREG(R1) ", %2\n\t"        \
+                     "v_accvgpr_write_b32 " FATTN_AREG(R2) ", %3\n\tv_accvgpr_write_b32 " FATTN_AREG(R3) ", %4"             \
+                     : "=" FATTN_ARANGE(R0, R3)(out) : "v"(w[0]), "v"(w[1]), "v"(w[2]), "v"(w[3]));
+    FATTN_B_SLOTS(FATTN_PIN)
 #undef FATTN_PIN
     return out;
 }
@@ -216,22 +184,19 @@ template <int IDX>
 __device__ __forceinline__ void rescale_pinned(f32x16& acc, float alpha) {
     static_assert(IDX >= 0 && IDX < 8, "eight pinned accumulator tuples");
     float tmp;
-    if constexpr (IDX == 0)
-        asm volatile("v_accvgpr_read_b32 %1, a0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a0, %1\n\tv_accvgpr_read_b32 %1, a1\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a1, %1\n\tv_accvgpr_read_b32 %1, a2\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a2, %1\n\tv_accvgpr_read_b32 %1, a3\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a3, %1\n\tv_accvgpr_read_b32 %1, a4\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a4, %1\n\tv_accvgpr_read_b32 %1, a5\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a5, %1\n\tv_accvgpr_read_b32 %1, a6\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a6, %1\n\tv_accvgpr_read_b32 %1, a7\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a7, %1\n\tv_accvgpr_read_b32 %1, a8\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a8, %1\n\tv_accvgpr_read_b32 %1, a9\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a9, %1\n\tv_accvgpr_read_b32 %1, a10\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a10, %1\n\tv_accvgpr_read_b32 %1, a11\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a11, %1\n\tv_accvgpr_read_b32 %1, a12\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a12, %1\n\tv_accvgpr_read_b32 %1, a13\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a13, %1\n\tv_accvgpr_read_b32 %1, a14\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a14, %1\n\tv_accvgpr_read_b32 %1, a15\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a15, %1" : "+{a[0:15]}"(acc), "=&v"(tmp) : "v"(alpha));
-    if constexpr (IDX == 1)
-        asm volatile("v_accvgpr_read_b32 %1, a16\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a16, %1\n\tv_accvgpr_read_b32 %1, a17\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a17, %1\n\tv_accvgpr_read_b32 %1, a18\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a18, %1\n\tv_accvgpr_read_b32 %1, a19\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a19, %1\n\tv_accvgpr_read_b32 %1, a20\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a20, %1\n\tv_accvgpr_read_b32 %1, a21\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a21, %1\n\tv_accvgpr_read_b32 %1, a22\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a22, %1\n\tv_accvgpr_read_b32 %1, a23\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a23, %1\n\tv_accvgpr_read_b32 %1, a24\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a24, %1\n\tv_accvgpr_read_b32 %1, a25\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a25, %1\n\tv_accvgpr_read_b32 %1, a26\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a26, %1\n\tv_accvgpr_read_b32 %1, a27\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a27, %1\n\tv_accvgpr_read_b32 %1, a28\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a28, %1\n\tv_accvgpr_read_b32 %1, a29\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a29, %1\n\tv_accvgpr_read_b32 %1, a30\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a30, %1\n\tv_accvgpr_read_b32 %1, a31\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a31, %1" : "+{a[16:31]}"(acc), "=&v"(tmp) : "v"(alpha));
-    if constexpr (IDX == 2)
-        asm volatile("v_accvgpr_read_b32 %1, a32\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a32, %1\n\tv_accvgpr_read_b32 %1, a33\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a33, %1\n\tv_accvgpr_read_b32 %1, a34\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a34, %1\n\tv_accvgpr_read_b32 %1, a35\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a35, %1\n\tv_accvgpr_read_b32 %1, a36\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a36, %1\n\tv_accvgpr_read_b32 %1, a37\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a37, %1\n\tv_accvgpr_read_b32 %1, a38\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a38, %1\n\tv_accvgpr_read_b32 %1, a39\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a39, %1\n\tv_accvgpr_read_b32 %1, a40\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a40, %1\n\tv_accvgpr_read_b32 %1, a41\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a41, %1\n\tv_accvgpr_read_b32 %1, a42\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a42, %1\n\tv_accvgpr_read_b32 %1, a43\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a43, %1\n\tv_accvgpr_read_b32 %1, a44\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a44, %1\n\tv_accvgpr_read_b32 %1, a45\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a45, %1\n\tv_accvgpr_read_b32 %1, a46\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a46, %1\n\tv_accvgpr_read_b32 %1, a47\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a47, %1" : "+{a[32:47]}"(acc), "=&v"(tmp) : "v"(alpha));
-    if constexpr (IDX == 3)
-        asm volatile("v_accvgpr_read_b32 %1, a48\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a48, %1\n\tv_accvgpr_read_b32 %1, a49\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a49, %1\n\tv_accvgpr_read_b32 %1, a50\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a50, %1\n\tv_accvgpr_read_b32 %1, a51\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a51, %1\n\tv_accvgpr_read_b32 %1, a52\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a52, %1\n\tv_accvgpr_read_b32 %1, a53\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a53, %1\n\tv_accvgpr_read_b32 %1, a54\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a54, %1\n\tv_accvgpr_read_b32 %1, a55\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a55, %1\n\tv_accvgpr_read_b32 %1, a56\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a56, %1\n\tv_accvgpr_read_b32 %1, a57\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a57, %1\n\tv_accvgpr_read_b32 %1, a58\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a58, %1\n\tv_accvgpr_read_b32 %1, a59\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a59, %1\n\tv_accvgpr_read_b32 %1, a60\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a60, %1\n\tv_accvgpr_read_b32 %1, a61\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a61, %1\n\tv_accvgpr_read_b32 %1, a62\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a62, %1\n\tv_accvgpr_read_b32 %1, a63\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a63, %1" : "+{a[48:63]}"(acc), "=&v"(tmp) : "v"(alpha));
-    if constexpr (IDX == 4)
-        asm volatile("v_accvgpr_read_b32 %1, a64\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a64, %1\n\tv_accvgpr_read_b32 %1, a65\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a65, %1\n\tv_accvgpr_read_b32 %1, a66\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a66, %1\n\tv_accvgpr_read_b32 %1, a67\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a67, %1\n\tv_accvgpr_read_b32 %1, a68\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a68, %1\n\tv_accvgpr_read_b32 %1, a69\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a69, %1\n\tv_accvgpr_read_b32 %1, a70\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a70, %1\n\tv_accvgpr_read_b32 %1, a71\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a71, %1\n\tv_accvgpr_read_b32 %1, a72\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a72, %1\n\tv_accvgpr_read_b32 %1, a73\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a73, %1\n\tv_accvgpr_read_b32 %1, a74\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a74, %1\n\tv_accvgpr_read_b32 %1, a75\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a75, %1\n\tv_accvgpr_read_b32 %1, a76\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a76, %1\n\tv_accvgpr_read_b32 %1, a77\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a77, %1\n\tv_accvgpr_read_b32 %1, a78\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a78, %1\n\tv_accvgpr_read_b32 %1, a79\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a79, %1" : "+{a[64:79]}"(acc), "=&v"(tmp) : "v"(alpha));
-    if constexpr (IDX == 5)
-        asm volatile("v_accvgpr_read_b32 %1, a80\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a80, %1\n\tv_accvgpr_read_b32 %1, a81\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a81, %1\n\tv_accvgpr_read_b32 %1, a82\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a82, %1\n\tv_accvgpr_read_b32 %1, a83\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a83, %1\n\tv_accvgpr_read_b32 %1, a84\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a84, %1\n\tv_accvgpr_read_b32 %1, a85\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a85, %1\n\tv_accvgpr_read_b32 %1, a86\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a86, %1\n\tv_accvgpr_read_b32 %1, a87\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a87, %1\n\tv_accvgpr_read_b32 %1, a88\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a88, %1\n\tv_accvgpr_read_b32 %1, a89\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a89, %1\n\tv_accvgpr_read_b32 %1, a90\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a90, %1\n\tv_accvgpr_read_b32 %1, a91\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a91, %1\n\tv_accvgpr_read_b32 %1, a92\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a92, %1\n\tv_accvgpr_read_b32 %1, a93\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a93, %1\n\tv_accvgpr_read_b32 %1, a94\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a94, %1\n\tv_accvgpr_read_b32 %1, a95\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a95, %1" : "+{a[80:95]}"(acc), "=&v"(tmp) : "v"(alpha));
-    if constexpr (IDX == 6)
-        asm volatile("v_accvgpr_read_b32 %1, a96\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a96, %1\n\tv_accvgpr_read_b32 %1, a97\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a97, %1\n\tv_accvgpr_read_b32 %1, a98\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a98, %1\n\tv_accvgpr_read_b32 %1, a99\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a99, %1\n\tv_accvgpr_read_b32 %1, a100\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a100, %1\n\tv_accvgpr_read_b32 %1, a101\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a101, %1\n\tv_accvgpr_read_b32 %1, a102\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a102, %1\n\tv_accvgpr_read_b32 %1, a103\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a103, %1\n\tv_accvgpr_read_b32 %1, a104\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a104, %1\n\tv_accvgpr_read_b32 %1, a105\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a105, %1\n\tv_accvgpr_read_b32 %1, a106\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a106, %1\n\tv_accvgpr_read_b32 %1, a107\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a107, %1\n\tv_accvgpr_read_b32 %1, a108\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a108, %1\n\tv_accvgpr_read_b32 %1, a109\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a109, %1\n\tv_accvgpr_read_b32 %1, a110\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a110, %1\n\tv_accvgpr_read_b32 %1, a111\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a111, %1" : "+{a[96:111]}"(acc), "=&v"(tmp) : "v"(alpha));
-    if constexpr (IDX == 7)
-        asm volatile("v_accvgpr_read_b32 %1, a112\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a112, %1\n\tv_accvgpr_read_b32 %1, a113\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a113, %1\n\tv_accvgpr_read_b32 %1, a114\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a114, %1\n\tv_accvgpr_read_b32 %1, a115\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a115, %1\n\tv_accvgpr_read_b32 %1, a116\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a116, %1\n\tv_accvgpr_read_b32 %1, a117\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a117, %1\n\tv_accvgpr_read_b32 %1, a118\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a118, %1\n\tv_accvgpr_read_b32 %1, a119\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a119, %1\n\tv_accvgpr_read_b32 %1, a120\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a120, %1\n\tv_accvgpr_read_b32 %1, a121\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a121, %1\n\tv_accvgpr_read_b32 %1, a122\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a122, %1\n\tv_accvgpr_read_b32 %1, a123\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a123, %1\n\tv_accvgpr_read_b32 %1, a124\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a124, %1\n\tv_accvgpr_read_b32 %1, a125\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a125, %1\n\tv_accvgpr_read_b32 %1, a126\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a126, %1\n\tv_accvgpr_read_b32 %1, a127\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 a127, %1" : "+{a[112:127]}"(acc), "=&v"(tmp) : "v"(alpha));
+    // one register: read, multiply, one wait state, write back
+#define FATTN_RS(r) "v_accvgpr_read_b32 %1, " FATTN_AREG(r) "\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 " FATTN_AREG(r) ", %1"
+#define FATTN_PIN(I, R0, R1, R2, R3, R4, R5, R6, R7, R8, R9, R10, R11, R12, R13, R14, R15)                                      \
+    FATTN_CHECK_ACC_TUPLE(I, R0, R1, R2, R3, R4, R5, R6, R7, R8, R9, R10, R11, R12, R13, R14, R15);                             \
+    if constexpr (IDX == I)                                                                                                     \
+        asm volatile(FATTN_RS(R0) "\n\t" FATTN_RS(R1) "\n\t" FATTN_RS(R2) "\n\t" FATTN_RS(R3) "\n\t" FATTN_RS(R4) "\n\t"        \
+                     FATTN_RS(R5) "\n\t" FATTN_RS(R6) "\n\t" FATTN_RS(R7) "\n\t" FATTN_RS(R8) "\n\t" FATTN_RS(R9) "\n\t"        \
+                     FATTN_RS(R10) "\n\t" FATTN_RS(R11) "\n\t" FATTN_RS(R12) "\n\t" FATTN_RS(R13) "\n\t" FATTN_RS(R14) "\n\t"   \
+                     FATTN_RS(R15)                                                                                              \
+                     : "+" FATTN_ARANGE(R0, R15)(acc), "=&v"(tmp) : "v"(alpha));
+    FATTN_ACC_TUPLES(FATTN_PIN)
+#undef FATTN_PIN
+#undef FATTN_RS
 }
 
 // acc += a b with the accumulator pinned to a[16 IDX : 16 IDX + 15] (the tuples rescale_pinned works on) and both
@@ -244,36 +209,22 @@ __device__ __forceinline__ void rescale_pinned(f32x16& acc, float alpha) {
 template <int IDX>
 __device__ __forceinline__ void mfma32_apinned(f32x16& acc, bf16x8 a, bf16x8 b) {
     static_assert(IDX >= 0 && IDX < 8, "eight pinned accumulator tuples");
-#define FATTN_PIN(I, R)                                                                                        \
-    if constexpr (IDX == I) {                                                                                  \
-        asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : R(acc) : "v"(a), "v"(b));          \
+#define FATTN_PIN(I, R0, R1, R2, R3, R4, R5, R6, R7, R8, R9, R10, R11, R12, R13, R14, R15)                          \
+    if constexpr (IDX == I) {                                                                                       \
+        asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+" FATTN_ARANGE(R0, R15)(acc) : "v"(a), "v"(b)); \
     }
-    FATTN_PIN(0, "+{a[0:15]}")
-    FATTN_PIN(1, "+{a[16:31]}")
-    FATTN_PIN(2, "+{a[32:47]}")
-    FATTN_PIN(3, "+{a[48:63]}")
-    FATTN_PIN(4, "+{a[64:79]}")
-    FATTN_PIN(5, "+{a[80:95]}")
-    FATTN_PIN(6, "+{a[96:111]}")
-    FATTN_PIN(7, "+{a[112:127]}")
+    FATTN_ACC_TUPLES(FATTN_PIN)
 #undef FATTN_PIN
 }
 template <int IDX, bool WAIT>
 __device__ __forceinline__ void mfma32_apinned_settle(f32x16& acc) {
     static_assert(IDX >= 0 && IDX < 8, "eight pinned accumulator tuples");
-#define FATTN_PIN(I, R)                                                                                        \
-    if constexpr (IDX == I) {                                                                                  \
-        if constexpr (WAIT) asm volatile("s_nop 11" : R(acc));                                                 \
-        else asm volatile("" : R(acc));                                                                        \
+#define FATTN_PIN(I, R0, R1, R2, R3, R4, R5, R6, R7, R8, R9, R10, R11, R12, R13, R14, R15)     \
+    if constexpr (IDX == I) {                                                                  \
+        if constexpr (WAIT) asm volatile("s_nop 11" : "+" FATTN_ARANGE(R0, R15)(acc));         \
+        else asm volatile("" : "+" FATTN_ARANGE(R0, R15)(acc));                                \
     }
-    FATTN_PIN(0, "+{a[0:15]}")
-    FATTN_PIN(1, "+{a[16:31]}")
-    FATTN_PIN(2, "+{a[32:47]}")
-    FATTN_PIN(3, "+{a[48:63]}")
-    FATTN_PIN(4, "+{a[64:79]}")
-    FATTN_PIN(5, "+{a[80:95]}")
-    FATTN_PIN(6, "+{a[96:111]}")
-    FATTN_PIN(7, "+{a[112:127]}")
+    FATTN_ACC_TUPLES(FATTN_PIN)
 #undef FATTN_PIN
 }
 
