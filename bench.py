@@ -223,6 +223,48 @@ def big_head_dims_line(args, capi, torch, dev):
     return 0
 
 
+def materialised_path_line(args, capi, torch, dev):
+    """The library's own materialised path (flame_attn_fwd_materialised_bf16 / flame_attn_bwd_materialised_bf16: the
+    shapes the fused kernels refuse) on three shapes: median HIP-event times of forward and backward with the
+    workspace the size query recommends, useful TFLOP/s (4 / 10 B H S^2 D), and the bytes its element-wise passes move
+    over the scores (forward 4 + 4 + 4 + 2 + 2 per score element: write logits, two reads for maximum and sum, a read
+    and the bf16 P written, read by the P V product; backward 8 more for dP and dS), as a rate."""
+    import math
+    out = {}
+    g = torch.Generator(device=dev).manual_seed(13)
+    for (B, H, S, D, masked) in [(1, 8, 2048, 256, True), (2, 4, 4096, 520, False), (1, 24, 2048, 20, False)]:
+        q, k, v, do = (torch.randn((B, H, S, D), device=dev, generator=g).to(torch.bfloat16) for _ in range(4))
+        mask = torch.ones((1, 1, S, S), dtype=torch.uint8, device=dev) if masked else None
+        sc = 1.0 / math.sqrt(D)
+        ws_f = torch.empty(capi.materialised_workspace_bytes(B, H, S, S, D, D, False), dtype=torch.uint8, device=dev)
+        ws_b = torch.empty(capi.materialised_workspace_bytes(B, H, S, S, D, D, True), dtype=torch.uint8, device=dev)
+        o, lse = capi.attn_fwd_materialised(q, k, v, sc, mask=mask, workspace=ws_f)
+        grads = tuple(torch.empty_like(q) for _ in range(3))
+        res = {"workspace_MiB": {"forward": ws_f.numel() / 2 ** 20, "backward": ws_b.numel() / 2 ** 20}}
+        for name, fn in (("forward", lambda: capi.attn_fwd_materialised(q, k, v, sc, mask=mask, out=o, workspace=ws_f)),
+                         ("backward", lambda: capi.attn_bwd_materialised(q, k, v, o, do, lse, sc, mask=mask, workspace=ws_b, grads=grads))):
+            for _ in range(2):
+                fn()
+            times = []
+            for _ in range(8):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                fn()
+                e1.record()
+                e1.synchronize()
+                times.append(e0.elapsed_time(e1))
+            ms = sorted(times)[len(times) // 2]
+            flops = (4.0 if name == "forward" else 10.0) * B * H * S * S * D
+            score_bytes = (16.0 if name == "forward" else 30.0) * B * H * S * S
+            res[name] = {"ms_median": ms, "useful_TFLOPs": flops / (ms * 1e-3) / 1e12, "score_traffic_GB_per_s": score_bytes / (ms * 1e-3) / 1e9}
+        out[f"B={B} H={H} S={S} D={D}" + (" keep-mask" if masked else "")] = res
+        del q, k, v, do, o, lse, grads, ws_f, ws_b
+    print(json.dumps({"metric": "materialised path (shapes the fused kernels refuse), ms", "unit": "ms", "n_gpus": 1, "dtype": "bf16",
+                      "data": "synthetic", "higher_is_better": False,
+                      "config": {"workload": "forward and backward, head dims 256 with a keep-mask, 520 and 20"}, "shapes": out}))
+    return 0
+
+
 def materialised_comparator(capi, torch, q, k, v, do, scale, o_fused, grads_fused, iters=5):
     """The structure this path replaces, run on the same GPU for comparison: scores = Q K^T as one library GEMM
     per head, softmax through this library's tile primitives, P kept in bf16 for the backward, PV / dV / dP / dQ /
@@ -594,6 +636,9 @@ def main():
                          "rocprofv3 --pmc can be scaled by what the same counters report for a known size")
     ap.add_argument("--big-head-dims", action="store_true",
                     help="time the forward for head dims above 128 next to a materialised comparator (a line of its own)")
+    ap.add_argument("--materialised", action="store_true",
+                    help="time the materialised path (library GEMMs + element-wise kernels) on shapes the fused kernels refuse "
+                         "(a line of its own)")
     ap.add_argument("--tile-ops", action="store_true",
                     help="time the element-wise tile primitives instead of an attention workload (a line of its own)")
     ap.add_argument("--mfma-ceiling", action="store_true",
@@ -622,6 +667,8 @@ def main():
         return tile_ops_line(args, capi, torch, dev)
     if args.big_head_dims:
         return big_head_dims_line(args, capi, torch, dev)
+    if args.materialised:
+        return materialised_path_line(args, capi, torch, dev)
     if args.mfma_ceiling:
         print(json.dumps(mfma_ceiling_line(args, capi, torch, W, dev)))
         return 0
