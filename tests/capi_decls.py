@@ -1,5 +1,5 @@
 """Parsers for the two sides of the C ABI: the function declarations of include/flame_attn.h and the `extern "C"`
-blocks of Rust source (rust/src/ffi.rs, the binding examples of INTEGRATION.md).  Used by the tests that hold the two
+blocks of Rust source (rust/src/ffi.rs, the binding examples of the integration guide).  Used by the tests that hold the two
 sides together; no GPU and no compiler needed."""
 from __future__ import annotations
 

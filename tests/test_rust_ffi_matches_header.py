@@ -1,5 +1,5 @@
 """The Rust side of the boundary cannot be compiled here (no Rust toolchain), so it is held to the C header by text:
-every `extern "C"` declaration of rust/src/ffi.rs, and every one in the binding examples of INTEGRATION.md, must
+every `extern "C"` declaration of rust/src/ffi.rs, and every one in the binding examples of the integration guide, must
 name a function of include/flame_attn.h and agree with it in argument count and in every argument and return type;
 and ffi.rs must declare every function the header has.  The calls in rust/src/sdpa.rs are checked for their
 argument counts.  The same parsers then check that the shared library exports what the header declares."""
@@ -67,7 +67,7 @@ def test_binding_examples_of_the_integration_guide_match_the_header(header):
     rust = parse_rust_externs(_read("INTEGRATION.md"))
     assert {"flame_cudnn_sdpa_bf16", "flame_cudnn_sdpa_bf16_train_fwd", "flame_cudnn_sdpa_bwd_bf16", "flame_attn_fwd_bf16"} <= set(rust)
     for name, decl in rust.items():
-        assert name in header, f"INTEGRATION.md declares {name}, which the header does not have"
+        assert name in header, f"the integration guide declares {name}, which the header does not have"
         assert mismatches(header[name], decl) == [], (name, mismatches(header[name], decl))
 
 
