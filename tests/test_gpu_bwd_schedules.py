@@ -78,3 +78,57 @@ def test_schedule_switch_is_ignored_where_it_does_not_apply(oracle):
         g = _bwd(schedule, q, k, v, o, do, lse, scale, causal=True)
         for a, b in zip(g, base):
             assert torch.equal(a, b), schedule
+
+
+_FORCED_128_SCRIPT = r"""
+import sys
+sys.path.insert(0, sys.argv[1])
+import numpy as np, torch
+from flame_amd import capi, workloads as W
+B, H, S, D = 1, 32, 2048, 128
+q, k, v, do = (torch.from_numpy(W.f32_to_bf16_bits(W.normal_f32(1500, i, B * H * S * D).reshape(B, H, S, D)).view(np.int16))
+               .view(torch.bfloat16).cuda() for i in range(4))
+scale = D ** -0.5
+capi.profiling_enable(True)
+o, lse = capi.attn_fwd(q, k, v, scale)
+dq, dk, dv = capi.attn_bwd(q, k, v, o, do, lse, scale)
+torch.cuda.synchronize()
+torch.save({"o": o.cpu(), "lse": lse.cpu(), "dq": dq.cpu(), "dk": dk.cpu(), "dv": dv.cpu()}, sys.argv[2])
+print("FORCED_128_DONE")
+"""
+
+
+def test_forced_128_query_workgroups_agree_with_the_256_query_ones(oracle, tmp_path):
+    """FLAME_ATTN_WG_WAVES=4 (read once per process, hence a process of its own) makes the forward and dQ run their
+    128-query kernels on a problem that would take the 256-query ones: same results to rounding, and head 7 against
+    the oracle."""
+    import subprocess
+    import sys
+    from flame_amd import capi
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = str(tmp_path / "forced128.pt")
+    env = dict(os.environ, FLAME_ATTN_WG_WAVES="4")
+    print("[forced 128-query workgroups] 1x32 S=2048 D=128 in a process of its own", flush=True)
+    res = subprocess.run([sys.executable, "-c", _FORCED_128_SCRIPT, root, out], stdout=subprocess.PIPE, stderr=subprocess.STDOUT,
+                         text=True, timeout=110, env=env)
+    assert res.returncode == 0 and "FORCED_128_DONE" in res.stdout, res.stdout[-3000:]
+    forced = torch.load(out, weights_only=True)
+    B, H, S, D = 1, 32, 2048, 128
+    bits = [W.f32_to_bf16_bits(W.normal_f32(1500, i, B * H * S * D).reshape(B, H, S, D)) for i in range(4)]
+    q, k, v, do = (to_dev(t) for t in bits)
+    scale = D ** -0.5
+    o, lse = capi.attn_fwd(q, k, v, scale)
+    g = capi.attn_bwd(q, k, v, o, do, lse, scale)
+    torch.cuda.synchronize()
+    assert oracle.rel_l2(to_f32(forced["o"]), to_f32(o)) < 2e-3 and float((forced["lse"] - lse.cpu()).abs().max()) < 1e-4
+    for name, a in zip(("dq", "dk", "dv"), g):
+        assert oracle.rel_l2(to_f32(forced[name]), to_f32(a)) < 3e-3, name
+    # other kernels did run there: the 128-query dQ kernel sums its key tiles in another order than the 256-query one
+    assert not torch.equal(forced["dq"], g[0].cpu())
+    hd = 7
+    ro, rlse, ro32 = oracle.sdpa_fwd(bits[0], bits[1], bits[2], scale, heads=(hd, hd + 1), want_f32=True)
+    assert_close_bf16(oracle, "O (forced 128)", to_f32(forced["o"])[0, hd], ro[0, hd], ro32[0, hd])
+    ref = oracle.sdpa_bwd(bits[0], bits[1], bits[2], forced["o"].view(torch.int16).numpy().view(np.uint16), bits[3], scale,
+                          heads=(hd, hd + 1), want_f32=True)
+    for i, name in enumerate(("dq", "dk", "dv")):
+        assert_close_bf16(oracle, f"{name} (forced 128)", to_f32(forced[name])[0, hd], ref[i][0, hd], ref[i + 3][0, hd])
